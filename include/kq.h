@@ -1,0 +1,123 @@
+/*
+ * kq.h -- C ABI of libkq: GGUF K-quant / legacy / IQ / fp4 wire-byte kernels for AMD
+ * Instinct MI355X (gfx950).
+ *
+ * Conventions
+ *   - every `*_dev` pointer is DEVICE memory on the current HIP device; the caller
+ *     owns every buffer (inputs, outputs, workspace) and keeps it alive until the
+ *     stream has run the call;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); device
+ *     entry points enqueue work and return without synchronising;
+ *   - return value 0 = success, negative = error (KQ_ERR_*); the message of the last
+ *     error on the calling thread is returned by kq_last_error();
+ *   - dtype codes: KQ_F32 / KQ_F16 / KQ_BF16.  Wire bytes are the unchanged GGUF block
+ *     layout (uint8), rows packed back to back: bytes_per_row = K / weights_per_block
+ *     * bytes_per_block;
+ *   - there is no CPU fallback: a call on a machine without a usable GPU fails with
+ *     KQ_ERR_HIP.
+ */
+#ifndef KQ_H
+#define KQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KQ_NUM_CODECS 21
+
+enum { KQ_F32 = 0, KQ_F16 = 1, KQ_BF16 = 2 };
+enum { KQ_ACT_SILU = 0, KQ_ACT_GELU = 1, KQ_ACT_SILU_LIMIT = 2, KQ_ACT_SWIGLU_CLAMP = 3 };
+enum {
+  KQ_OK = 0,
+  KQ_ERR_INVALID = -1,     /* bad argument (maps to the reference's std::invalid_argument) */
+  KQ_ERR_UNSUPPORTED = -2, /* valid request this build has no kernel for (std::runtime_error) */
+  KQ_ERR_HIP = -3,         /* HIP runtime failure (std::runtime_error) */
+  KQ_ERR_WORKSPACE = -4    /* workspace missing or too small */
+};
+
+/* Replaces struct KQuantCodec, reference src/kquant_codec.h:10-19. */
+typedef struct kq_codec_info {
+  char name[16];
+  int weights_per_block;
+  int bytes_per_block;
+  int bits;
+  int has_matmul_kernel;
+  int has_encode;
+  int has_nax_kernel;
+  int requires_imatrix;
+} kq_codec_info;
+
+/* Registry, in the reference's canonical order.
+ * Replaces codec_by_name / codec_names, reference src/kquant_codec.cpp:12-57. */
+int kq_codec_count(void);
+int kq_codec_id(const char* name);               /* -1 if unknown */
+int kq_codec_get(int codec, kq_codec_info* out); /* KQ_ERR_INVALID if out of range */
+/* Replaces codec_has_moe_glu, reference src/kquant_moe_glu.cpp:792-798. */
+int kq_codec_has_moe_glu(int codec);
+
+const char* kq_last_error(void);
+const char* kq_version(void);
+
+/* out[i] = T(decode(w)[i]) for i < num_weights (num_weights a whole number of blocks).
+ * f32 results are bit-identical to the reference's scalar decoders; f16/bf16 are one
+ * round-to-nearest-even of that f32 value.
+ * Replaces kquant_dequantize_parallel<T>, reference src/kquant_cpu_decode.h:37-52 /
+ * src/kquant_cpu_decode.cpp:1189-1207 (called by KQuantDequantize::eval_cpu,
+ * src/kquant_dequantize.cpp:59-91). */
+int kq_dequantize(const void* w_dev, void* out_dev, uint64_t num_weights, int codec, int out_dtype,
+                  void* stream);
+
+/* y[M,N] = x[M,K] . W^T  (transpose != 0, W decodes to [N,K])  or  x[M,K] . W (transpose == 0,
+ * W decodes to [K,N]).  x and y have dtype `dtype` (KQ_F16 / KQ_BF16; the op layer casts f32
+ * activations to bf16 first, as the reference does); accumulation is f32 with one rounding
+ * to `dtype`.  Workspace: kq_qmm_workspace_size bytes of device memory (may be 0).
+ * Replaces kquant_qmm_cpu<T>, reference src/kquant_cpu_decode.h:54-70 /
+ * src/kquant_cpu_decode.cpp:1209-1359 (called by KQuantMatmul::eval_cpu,
+ * src/kquant_matmul.cpp:1104-1164). */
+size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int dtype);
+int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int transpose,
+           int codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
+
+/* out[b] = x[lhs[b]] . W[rhs[b]]^T for b < B; x batches are [M,K] matrices
+ * `x_batch_stride` elements apart, experts are [N, bytes_per_row] wire matrices
+ * `w_expert_stride_bytes` apart (64-bit, so strided / >2 GiB stacks work); out is
+ * [B, M, N] dense.  `rhs_sorted` != 0 promises rhs is non-decreasing.
+ * Replaces KQuantGatherQMM::eval_cpu, reference src/kquant_gather.cpp:470-746
+ * (kquant_qmm_cpu_batch, src/kquant_cpu_decode.cpp:1361-1527). */
+size_t kq_gather_qmm_workspace_size(int B, int M, int N, int K, int transpose, int codec, int dtype);
+int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_dev,
+                  const uint32_t* rhs_idx_dev, void* out_dev, int B, int M, int N, int K,
+                  int64_t x_batch_stride, int64_t w_expert_stride_bytes, int transpose, int rhs_sorted,
+                  int codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
+
+/* out[t,r,:] = T(act(x[t] . G_e^T (+gb_e), x[t] . U_e^T (+ub_e))), e = idx[t,r]; f32 throughout,
+ * one rounding.  x [T,K], gate/up stacks [E,N,bytes_per_row] dense, idx [T,R] uint32,
+ * biases f32 [E,N] or NULL, out [T,R,N].
+ * Replaces KQuantMoEGLUKQ (op moe_glu_gather_kq), reference src/kquant_moe_glu.cpp:1070-1157,
+ * dispatch :277-329, epilogue metal/mlx/backend/metal/kernels/kq_moe_glu_kq.h:34-60. */
+int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_w_dev,
+                      const uint32_t* idx_dev, const float* gate_bias_dev, const float* up_bias_dev,
+                      void* out_dev, int T, int R, int E, int N, int K, int act, float limit, float alpha,
+                      int codec, int dtype, void* stream);
+
+/* out[t,r,:] = T(x[t,r,:] . W_e^T (+ bias_e)), e = idx[t,r].  x [T,R,K], w [E,N,bytes_per_row].
+ * Replaces KQuantGatherQMVKQ (op gather_qmv_kq), reference src/kquant_moe_glu.cpp:1159-1210,
+ * dispatch :331-382, kernels kq_moe_glu_kq.h:933-999. */
+int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev, const float* bias_dev,
+                  void* out_dev, int T, int R, int E, int N, int K, int codec, int dtype, void* stream);
+
+/* HOST function: wire = encode(w[rows, K] f32) (imatrix f32 [K] or NULL), rows * bytes_per_row
+ * bytes written to wire_host.  Runs on the calling thread's CPU cores like the reference's
+ * encoder (which is CPU-only for the IQ codecs and serial).
+ * Replaces kquant_quantize_dispatch, reference src/kquant_cpu_encode.h:25-31 /
+ * src/kquant_cpu_encode.cpp:824-859 (op quantize, src/kquant_ops.cpp:550-631). */
+int kq_quantize(const float* w_host, const float* imatrix_host, uint8_t* wire_host, int64_t rows, int64_t K,
+                int codec);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KQ_H */

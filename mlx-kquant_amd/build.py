@@ -1,0 +1,68 @@
+"""Builds libkq.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+
+    python mlx-kquant_amd/build.py            # rebuild everything
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "lib", "libkq.so")
+BLOB = os.path.join(HERE, "data", "kq_iq_grids.bin")
+
+# (source, extra flags).  kq_generic.hip holds the bit-exact decoders: no FMA contraction.
+SOURCES = [
+    ("kq_api.cpp", ["-x", "hip"]),
+    ("kq_encode.cpp", ["-x", "hip"]),
+    ("kq_generic.hip", ["-ffp-contract=off"]),
+    ("kq_mfma.hip", []),
+]
+COMMON = [
+    "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
+    # packed-FP32 VALU forms are kept out of the generated code on purpose
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-I", os.path.join(ROOT, "include"), "-I", CSRC, '-DKQ_GRID_BLOB="%s"' % BLOB,
+]
+
+
+def _hipcc():
+    for c in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if c and (os.path.isabs(c) and os.path.exists(c) or not os.path.isabs(c)):
+            return c
+    raise RuntimeError("hipcc not found")
+
+
+def _compile(item):
+    src, extra = item
+    out = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    cmd = [_hipcc()] + COMMON + extra + ["-c", os.path.join(CSRC, src), "-o", out]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    log = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
+    if log.strip():
+        print(log)
+    return out
+
+
+def build_all(verbose=True):
+    os.makedirs(OBJ, exist_ok=True)
+    os.makedirs(os.path.dirname(LIB), exist_ok=True)
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        objs = list(ex.map(_compile, SOURCES))
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stdout)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

@@ -1,0 +1,218 @@
+// C ABI of libkq (declared in include/kq.h): argument validation, error reporting, per-device
+// codebook upload and routing to the HIP launchers.  Host-only code; compiled by hipcc as C++.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+#include "kq_common.h"
+
+// IQ codebook blob linked into .rodata (data file given by -DKQ_GRID_BLOB="...").
+__asm__(".section .rodata\n"
+        ".balign 16\n"
+        "kq_grid_blob_host:\n"
+        ".incbin \"" KQ_GRID_BLOB "\"\n"
+        ".previous\n");
+extern "C" const uint8_t kq_grid_blob_host[];
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+// Reference registry, src/kquant_codec.cpp:12-37.
+const kq_codec_info kCodecs[KQ_NUM_CODECS] = {
+    {"q2_k", 256, 84, 2, 1, 1, 1, 0},    {"q3_k", 256, 110, 3, 1, 1, 1, 0},
+    {"q4_k", 256, 144, 4, 1, 1, 1, 0},   {"q5_k", 256, 176, 5, 1, 1, 1, 0},
+    {"q6_k", 256, 210, 6, 1, 1, 1, 0},   {"q4_0", 32, 18, 4, 1, 1, 1, 0},
+    {"q4_1", 32, 20, 4, 1, 1, 1, 0},     {"q5_0", 32, 22, 5, 1, 1, 1, 0},
+    {"q5_1", 32, 24, 5, 1, 1, 1, 0},     {"q8_0", 32, 34, 8, 1, 1, 1, 0},
+    {"iq4_nl", 32, 18, 4, 1, 1, 1, 0},   {"iq4_xs", 256, 136, 4, 1, 1, 1, 0},
+    {"iq3_s", 256, 110, 3, 1, 1, 1, 0},  {"iq3_xxs", 256, 98, 3, 1, 1, 1, 0},
+    {"iq2_xxs", 256, 66, 2, 1, 1, 1, 1}, {"iq2_xs", 256, 74, 2, 1, 1, 1, 1},
+    {"iq2_s", 256, 82, 2, 1, 1, 1, 0},   {"iq1_s", 256, 50, 1, 1, 1, 1, 1},
+    {"iq1_m", 256, 56, 1, 1, 1, 1, 0},   {"mxfp4", 32, 17, 4, 1, 0, 0, 0},
+    {"nvfp4", 64, 36, 4, 1, 0, 0, 0},
+};
+
+constexpr int kMaxDevices = 64;
+std::mutex g_grid_mu;
+uint8_t* g_grids[kMaxDevices] = {};
+
+bool codec_ok(int c) { return c >= 0 && c < KQ_NUM_CODECS; }
+bool half_dtype(int dt) { return dt == KQ_F16 || dt == KQ_BF16; }
+
+}  // namespace
+
+int kq_set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+const uint8_t* kq_device_grids(void) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    kq_set_error(KQ_ERR_HIP, "no usable HIP device: %s", hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lk(g_grid_mu);
+  if (!g_grids[dev]) {
+    uint8_t* p = nullptr;
+    e = hipMalloc(reinterpret_cast<void**>(&p), KQ_GRID_BYTES);
+    if (e == hipSuccess) e = hipMemcpy(p, kq_grid_blob_host, KQ_GRID_BYTES, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      kq_set_error(KQ_ERR_HIP, "codebook upload failed: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    g_grids[dev] = p;  // kept for the life of the process
+  }
+  return g_grids[dev];
+}
+
+extern "C" {
+
+const char* kq_last_error(void) { return g_err; }
+const char* kq_version(void) { return "kq-mi355x 0.1 (gfx950)"; }
+int kq_codec_count(void) { return KQ_NUM_CODECS; }
+
+int kq_codec_id(const char* name) {
+  if (!name) return -1;
+  for (int i = 0; i < KQ_NUM_CODECS; i++)
+    if (std::strcmp(kCodecs[i].name, name) == 0) return i;
+  return -1;
+}
+
+int kq_codec_get(int codec, kq_codec_info* out) {
+  if (!codec_ok(codec) || !out) return kq_set_error(KQ_ERR_INVALID, "codec id %d out of range", codec);
+  *out = kCodecs[codec];
+  return KQ_OK;
+}
+
+int kq_codec_has_moe_glu(int codec) { return codec_ok(codec) ? 1 : 0; }
+
+int kq_dequantize(const void* w_dev, void* out_dev, uint64_t num_weights, int codec, int out_dtype, void* stream) {
+  if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "dequantize: unknown codec id %d", codec);
+  if (out_dtype < KQ_F32 || out_dtype > KQ_BF16)
+    return kq_set_error(KQ_ERR_INVALID, "dequantize: only real floating output dtypes are supported");
+  const int wpb = kCodecs[codec].weights_per_block;
+  if (num_weights % (uint64_t)wpb)
+    return kq_set_error(KQ_ERR_INVALID, "dequantize: num_weights (%llu) is not a whole number of %d-weight blocks",
+                        (unsigned long long)num_weights, wpb);
+  if (num_weights == 0) return KQ_OK;
+  if (!w_dev || !out_dev) return kq_set_error(KQ_ERR_INVALID, "dequantize: null buffer");
+  return kq_launch_dequantize(static_cast<const uint8_t*>(w_dev), out_dev, num_weights / wpb, codec, out_dtype,
+                              static_cast<hipStream_t>(stream));
+}
+
+size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int dtype) {
+  (void)M; (void)N; (void)K; (void)transpose; (void)codec; (void)dtype;
+  return 0;
+}
+
+int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int transpose, int codec,
+           int dtype, void* workspace_dev, size_t workspace_bytes, void* stream) {
+  (void)workspace_dev; (void)workspace_bytes;
+  if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: unknown codec id %d", codec);
+  if (!half_dtype(dtype))
+    return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: activations must be float16 or bfloat16");
+  if (M < 0 || N < 0 || K < 0) return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: negative dimension");
+  const int wpb = kCodecs[codec].weights_per_block;
+  const int inner = transpose ? K : N;
+  if (inner % wpb)
+    return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: quantized row length %d is not a multiple of %d", inner,
+                        wpb);
+  if (M == 0 || N == 0) return KQ_OK;
+  if (!x_dev || !w_dev || !y_dev) return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: null buffer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (!transpose)
+    return kq_launch_gemm_nt_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+  int rc = kq_launch_qmm_tuned(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+  if (rc != KQ_ERR_UNSUPPORTED) return rc;
+  return kq_launch_gemv_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+}
+
+size_t kq_gather_qmm_workspace_size(int B, int M, int N, int K, int transpose, int codec, int dtype) {
+  (void)B; (void)M; (void)N; (void)K; (void)transpose; (void)codec; (void)dtype;
+  return 0;
+}
+
+int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_dev, const uint32_t* rhs_idx_dev,
+                  void* out_dev, int B, int M, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride_bytes,
+                  int transpose, int rhs_sorted, int codec, int dtype, void* workspace_dev, size_t workspace_bytes,
+                  void* stream) {
+  (void)workspace_dev; (void)workspace_bytes; (void)rhs_sorted;
+  if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: unknown codec id %d", codec);
+  if (!half_dtype(dtype)) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: activations must be float16 or bfloat16");
+  if (!transpose)
+    return kq_set_error(KQ_ERR_UNSUPPORTED, "gather_qmm: transpose=false has no kernel in this build");
+  if (B < 0 || M < 0 || N < 0 || K < 0) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: negative dimension");
+  if (K % kCodecs[codec].weights_per_block)
+    return kq_set_error(KQ_ERR_INVALID, "gather_qmm: K (%d) is not a multiple of %d", K,
+                        kCodecs[codec].weights_per_block);
+  if (B == 0 || M == 0 || N == 0) return KQ_OK;
+  if (!x_dev || !w_dev || !out_dev || !lhs_idx_dev || !rhs_idx_dev)
+    return kq_set_error(KQ_ERR_INVALID, "gather_qmm: null buffer");
+  return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
+                                  nullptr, nullptr, out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0,
+                                  0, 0.f, 0.f, codec, dtype, static_cast<hipStream_t>(stream));
+}
+
+static int check_moe(const char* op, int T, int R, int E, int N, int K, int codec, int dtype) {
+  if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "%s: codec id %d has no fused MoE kernel", op, codec);
+  if (!half_dtype(dtype)) return kq_set_error(KQ_ERR_INVALID, "%s: x must be float16 or bfloat16", op);
+  if (T < 0 || R < 0 || E <= 0 || N < 0 || K < 0) return kq_set_error(KQ_ERR_INVALID, "%s: bad dimension", op);
+  if (K % kCodecs[codec].weights_per_block)
+    return kq_set_error(KQ_ERR_INVALID, "%s: weight trailing dim does not match K for '%s'", op, kCodecs[codec].name);
+  if (N % 8) return kq_set_error(KQ_ERR_INVALID, "%s: N must be a multiple of 8", op);
+  return KQ_OK;
+}
+
+int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_w_dev, const uint32_t* idx_dev,
+                      const float* gate_bias_dev, const float* up_bias_dev, void* out_dev, int T, int R, int E, int N,
+                      int K, int act, float limit, float alpha, int codec, int dtype, void* stream) {
+  const char* op = "moe_glu_gather_kq";
+  int rc = check_moe(op, T, R, E, N, K, codec, dtype);
+  if (rc) return rc;
+  if (act < KQ_ACT_SILU || act > KQ_ACT_SWIGLU_CLAMP)
+    return kq_set_error(KQ_ERR_INVALID, "%s: act must be 'silu', 'gelu', 'silu_limit' or 'swiglu_clamp'", op);
+  if (act == KQ_ACT_SILU_LIMIT && !(limit > 0.f))
+    return kq_set_error(KQ_ERR_INVALID, "%s: act 'silu_limit' requires limit > 0", op);
+  const bool biased = gate_bias_dev || up_bias_dev;
+  if (act == KQ_ACT_SWIGLU_CLAMP) {
+    if (!gate_bias_dev || !up_bias_dev || !(limit > 0.f) || !(alpha > 0.f))
+      return kq_set_error(KQ_ERR_INVALID, "%s: act 'swiglu_clamp' requires gate_bias, up_bias, limit > 0 and alpha > 0",
+                          op);
+    if (codec != KQ_MXFP4 && codec != KQ_NVFP4)
+      return kq_set_error(KQ_ERR_INVALID, "%s: biased kernels are instantiated for mxfp4/nvfp4 only", op);
+  } else if (biased) {
+    return kq_set_error(KQ_ERR_INVALID, "%s: gate_bias/up_bias require act 'swiglu_clamp'", op);
+  }
+  if (T == 0 || R == 0 || N == 0) return KQ_OK;
+  if (!x_dev || !gate_w_dev || !up_w_dev || !idx_dev || !out_dev)
+    return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
+  return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(gate_w_dev),
+                                  static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, gate_bias_dev, up_bias_dev,
+                                  out_dev, T * R, 1, N, K, R, K, estride, 1, act, limit, alpha, codec, dtype,
+                                  static_cast<hipStream_t>(stream));
+}
+
+int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev, const float* bias_dev, void* out_dev,
+                  int T, int R, int E, int N, int K, int codec, int dtype, void* stream) {
+  const char* op = "gather_qmv_kq";
+  int rc = check_moe(op, T, R, E, N, K, codec, dtype);
+  if (rc) return rc;
+  if (bias_dev && codec != KQ_MXFP4 && codec != KQ_NVFP4)
+    return kq_set_error(KQ_ERR_INVALID, "%s: biased kernels are instantiated for mxfp4/nvfp4 only", op);
+  if (T == 0 || R == 0 || N == 0) return KQ_OK;
+  if (!x_dev || !w_dev || !idx_dev || !out_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
+  return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, bias_dev,
+                                  nullptr, out_dev, T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype,
+                                  static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

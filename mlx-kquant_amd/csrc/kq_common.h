@@ -1,0 +1,66 @@
+// Shared host/device definitions: codec ids and block geometry, error plumbing, small
+// bit helpers.  Codec order follows the reference registry (src/kquant_codec.cpp:12-37).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kq.h"
+
+enum KqCodec : int {
+  KQ_Q2_K = 0, KQ_Q3_K, KQ_Q4_K, KQ_Q5_K, KQ_Q6_K, KQ_Q4_0, KQ_Q4_1, KQ_Q5_0, KQ_Q5_1, KQ_Q8_0,
+  KQ_IQ4_NL, KQ_IQ4_XS, KQ_IQ3_S, KQ_IQ3_XXS, KQ_IQ2_XXS, KQ_IQ2_XS, KQ_IQ2_S, KQ_IQ1_S, KQ_IQ1_M,
+  KQ_MXFP4, KQ_NVFP4
+};
+
+struct KqGeom {
+  int wpb;  // weights per block
+  int bpb;  // bytes per block
+};
+
+__host__ __device__ constexpr KqGeom kq_geom(int c) {
+  constexpr KqGeom g[KQ_NUM_CODECS] = {
+      {256, 84},  {256, 110}, {256, 144}, {256, 176}, {256, 210}, {32, 18},  {32, 20},
+      {32, 22},   {32, 24},   {32, 34},   {32, 18},   {256, 136}, {256, 110}, {256, 98},
+      {256, 66},  {256, 74},  {256, 82},  {256, 50},  {256, 56},  {32, 17},  {64, 36}};
+  return g[c];
+}
+
+// Offsets of the IQ codebooks inside the device copy of the grid blob
+// (iq2xxs u64[256] | iq2xs u64[512] | iq2s u64[1024] | iq1s u64[2048] | iq3xxs u32[256] |
+// iq3s u32[512]).
+#define KQ_GRID_IQ2XXS 0
+#define KQ_GRID_IQ2XS 2048
+#define KQ_GRID_IQ2S 6144
+#define KQ_GRID_IQ1S 14336
+#define KQ_GRID_IQ3XXS 30720
+#define KQ_GRID_IQ3S 31744
+#define KQ_GRID_BYTES 33792
+
+// ---- host-side plumbing (kq_api.cpp) ----
+int kq_set_error(int code, const char* fmt, ...);
+// Device copy of the IQ codebooks for the current device (uploaded once per device).
+const uint8_t* kq_device_grids(void);
+
+#define KQ_HIP_CHECK(expr)                                                              \
+  do {                                                                                  \
+    hipError_t _e = (expr);                                                             \
+    if (_e != hipSuccess)                                                               \
+      return kq_set_error(KQ_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(_e));  \
+  } while (0)
+
+// ---- per-op launchers implemented in the .hip files ----
+int kq_launch_dequantize(const uint8_t* w, void* out, uint64_t num_blocks, int codec, int out_dtype,
+                         hipStream_t s);
+int kq_launch_gemv_generic(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
+                           hipStream_t s);
+int kq_launch_gemm_nt_generic(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec,
+                              int dtype, hipStream_t s);
+int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
+                             const uint32_t* rhs, const float* bias, const float* bias2, void* out, int B, int M,
+                             int N, int K, int x_div, int64_t x_batch_stride, int64_t w_expert_stride, int glu,
+                             int act, float limit, float alpha, int codec, int dtype, hipStream_t s);
+// Tuned path: returns KQ_ERR_UNSUPPORTED (without touching the error text) when no tuned kernel
+// covers the request, so the caller can fall through to the generic kernels.
+int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
+                        hipStream_t s);

@@ -1,0 +1,255 @@
+// Device-side reference decoders: kq_decode8<CODEC>() returns weights [8g, 8g+8) of one wire
+// block as f32, with exactly the operation order of the reference's scalar decoders
+// (src/kquant_cpu_decode.cpp:49-735), so results are bit-identical as long as the including
+// translation unit is compiled with -ffp-contract=off.  These are the ground-truth device
+// decoders: the dequantize kernel and the generic matmul kernels are built on them; the tuned
+// MFMA kernels use their own integer-code paths and are tested against these.
+#pragma once
+
+#include "kq_common.h"
+
+namespace kq {
+
+__device__ __forceinline__ float h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t ld16(const uint8_t* p) { return (uint16_t)(p[0] | (p[1] << 8)); }
+__device__ __forceinline__ uint32_t ld32(const uint8_t* p) {
+  return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+__device__ __forceinline__ float ldh(const uint8_t* p) { return h2f(ld16(p)); }
+
+// src/kquant_iq_tables.h:10
+__device__ __forceinline__ float kv_iq4nl(int i) {
+  // packed as bytes to stay in registers / scalar constants
+  const uint64_t lo = 0xF6EADDCFBFAD9881ull;  // -127,-104,-83,-65,-49,-35,-22,-10
+  const uint64_t hi = 0x7159453526190D01ull;  // 1,13,25,38,53,69,89,113
+  uint64_t v = (i & 8) ? hi : lo;
+  return (float)(int8_t)(v >> (8 * (i & 7)));
+}
+// src/kquant_fp_tables.h:16 (2x OCP E2M1)
+__device__ __forceinline__ float kv_mxfp4(int i) {
+  const uint64_t mag = 0x0C08060403020100ull;  // 0,1,2,3,4,6,8,12
+  int m = (int)((mag >> (8 * (i & 7))) & 0xff);
+  return (float)((i & 8) ? -m : m);
+}
+// src/kquant_iq_tables.h:1458: 7-bit index -> 8 sign bits, bit 7 = parity
+__device__ __forceinline__ uint32_t ksigns(uint32_t i) {
+  i &= 127u;
+  return i | ((uint32_t)(__builtin_popcount(i) & 1) << 7);
+}
+// src/kquant_fp_tables.h:21-27
+__device__ __forceinline__ float e8m0_half(uint32_t e) {
+  uint32_t bits = e < 2 ? (0x00200000u << e) : ((e - 1) << 23);
+  return __builtin_bit_cast(float, bits);
+}
+// src/kquant_fp_tables.h:32-41 (all steps exact power-of-two scalings)
+__device__ __forceinline__ float ue4m3_half(uint32_t x) {
+  if (x == 0 || x == 0x7f) return 0.0f;
+  int ex = (x >> 3) & 15;
+  float man = (float)(x & 7);
+  float raw = ex == 0 ? man * 0x1p-9f : ldexpf(1.0f + man * 0.125f, ex - 7);
+  return raw * 0.5f;
+}
+__device__ __forceinline__ float sgn(uint32_t signs, int j) { return (signs >> j) & 1 ? -1.f : 1.f; }
+
+// 6-bit (scale, min) pair j of a q4_k / q5_k block (src/kquant_cpu_decode.cpp:155-174)
+__device__ __forceinline__ void q4k_scale_min(const uint8_t* s, int j, int& sc, int& mn) {
+  if (j < 4) {
+    sc = s[j] & 63;
+    mn = s[j + 4] & 63;
+  } else {
+    sc = (s[j + 4] & 15) | ((s[j - 4] >> 6) << 4);
+    mn = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+  }
+}
+
+template <int C>
+__device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, const uint8_t* __restrict__ grids,
+                                        float* __restrict__ o) {
+  if constexpr (C == KQ_Q8_0) {  // :49-63
+    float d = ldh(b);
+    for (int t = 0; t < 8; t++) o[t] = d * (float)(int8_t)b[2 + 8 * g + t];
+  } else if constexpr (C == KQ_Q4_0) {  // :65-82
+    float d = ldh(b);
+    const uint8_t* q = b + 2 + 8 * (g & 1);
+    for (int t = 0; t < 8; t++) o[t] = d * (float)((int)((g < 2) ? (q[t] & 15) : (q[t] >> 4)) - 8);
+  } else if constexpr (C == KQ_Q4_1) {  // :84-102
+    float d = ldh(b), m = ldh(b + 2);
+    const uint8_t* q = b + 4 + 8 * (g & 1);
+    for (int t = 0; t < 8; t++) o[t] = d * (float)((g < 2) ? (q[t] & 15) : (q[t] >> 4)) + m;
+  } else if constexpr (C == KQ_Q5_0) {  // :104-128
+    float d = ldh(b);
+    uint32_t qh = ld32(b + 2);
+    const uint8_t* q = b + 6 + 8 * (g & 1);
+    for (int t = 0; t < 8; t++) {
+      int hb = (qh >> (8 * g + t)) & 1;
+      int v = (int)((g < 2) ? (q[t] & 15) : (q[t] >> 4)) | (hb << 4);
+      o[t] = d * (float)(v - 16);
+    }
+  } else if constexpr (C == KQ_Q5_1) {  // :130-153
+    float d = ldh(b), m = ldh(b + 2);
+    uint32_t qh = ld32(b + 4);
+    const uint8_t* q = b + 8 + 8 * (g & 1);
+    for (int t = 0; t < 8; t++) {
+      int hb = (qh >> (8 * g + t)) & 1;
+      int v = (int)((g < 2) ? (q[t] & 15) : (q[t] >> 4)) | (hb << 4);
+      o[t] = d * (float)v + m;
+    }
+  } else if constexpr (C == KQ_Q4_K || C == KQ_Q5_K) {  // :176-235
+    float d = ldh(b), dmin = ldh(b + 2);
+    int j = g >> 2, i0 = 8 * (g & 3), isc, imn;
+    q4k_scale_min(b + 4, j, isc, imn);
+    float sc = d * (float)isc, mn = dmin * (float)imn;
+    const uint8_t* qs = b + (C == KQ_Q4_K ? 16 : 48) + 32 * (j >> 1) + i0;
+    for (int t = 0; t < 8; t++) {
+      int v = (j & 1) ? (qs[t] >> 4) : (qs[t] & 15);
+      if constexpr (C == KQ_Q5_K) v |= ((b[16 + i0 + t] >> j) & 1) << 4;
+      o[t] = sc * (float)v - mn;
+    }
+  } else if constexpr (C == KQ_Q6_K) {  // :237-280
+    float d = ldh(b + 208);
+    int w = 8 * g, h = w >> 7, r = w & 127, qd = r >> 5, l0 = r & 31;
+    const uint8_t* ql = b + 64 * h + ((qd & 1) ? 32 : 0) + l0;
+    const uint8_t* qh = b + 128 + 32 * h + l0;
+    float dsc = d * (float)(int8_t)b[192 + (w >> 4)];
+    for (int t = 0; t < 8; t++) {
+      int lo = (qd & 2) ? (ql[t] >> 4) : (ql[t] & 15);
+      int v = (lo | (((qh[t] >> (2 * qd)) & 3) << 4)) - 32;
+      o[t] = dsc * (float)v;  // (d * sc) * q, left to right
+    }
+  } else if constexpr (C == KQ_Q3_K) {  // :282-337
+    float d = ldh(b + 108);
+    int w = 8 * g, half = w >> 7, r = w & 127, si = r >> 5, l0 = r & 31, is = w >> 4;
+    const uint8_t* s = b + 96;
+    int k = is & 3, grp = is >> 2, sc;  // sc[k + 4*grp]
+    int lo4 = (grp & 1) ? s[k + 4] : s[k];
+    lo4 = (grp & 2) ? (lo4 >> 4) : (lo4 & 15);
+    sc = lo4 | (((s[8 + k] >> (2 * grp)) & 3) << 4);
+    float dl = d * (float)(sc - 32);
+    const uint8_t* q = b + 32 + 32 * half + l0;
+    const uint8_t* hm = b + l0;
+    for (int t = 0; t < 8; t++) {
+      int q2 = (q[t] >> (2 * si)) & 3;
+      int hh = ((hm[t] >> (4 * half + si)) & 1) ? 0 : 4;
+      o[t] = dl * (float)(q2 - hh);
+    }
+  } else if constexpr (C == KQ_Q2_K) {  // :339-377
+    float d = ldh(b + 80), dmin = ldh(b + 82);
+    int w = 8 * g, half = w >> 7, r = w & 127, si = r >> 5, l0 = r & 31;
+    uint8_t sb = b[w >> 4];
+    float dl = d * (float)(sb & 15), ml = dmin * (float)(sb >> 4);
+    const uint8_t* q = b + 16 + 32 * half + l0;
+    for (int t = 0; t < 8; t++) o[t] = dl * (float)((q[t] >> (2 * si)) & 3) - ml;
+  } else if constexpr (C == KQ_IQ4_NL) {  // :382-397
+    float d = ldh(b);
+    const uint8_t* q = b + 2 + 8 * (g & 1);
+    for (int t = 0; t < 8; t++) o[t] = d * kv_iq4nl((g < 2) ? (q[t] & 15) : (q[t] >> 4));
+  } else if constexpr (C == KQ_MXFP4) {  // :403-418
+    float d = e8m0_half(b[0]);
+    const uint8_t* q = b + 1 + 8 * (g & 1);
+    for (int t = 0; t < 8; t++) o[t] = d * kv_mxfp4((g < 2) ? (q[t] & 15) : (q[t] >> 4));
+  } else if constexpr (C == KQ_NVFP4) {  // :420-438
+    int grp = g >> 1;
+    float d = ue4m3_half(b[grp]);
+    const uint8_t* q = b + 4 + 8 * grp;
+    for (int t = 0; t < 8; t++) o[t] = d * kv_mxfp4((g & 1) ? (q[t] >> 4) : (q[t] & 15));
+  } else if constexpr (C == KQ_IQ4_XS) {  // :440-465
+    float d = ldh(b);
+    uint32_t sh = ld16(b + 2);
+    int ib = g >> 2, r = g & 3;
+    int ls = ((b[4 + (ib >> 1)] >> (4 * (ib & 1))) & 15) | (int)(((sh >> (2 * ib)) & 3) << 4);
+    float dl = d * (float)(ls - 32);
+    const uint8_t* q = b + 8 + 16 * ib + 8 * (r & 1);
+    for (int t = 0; t < 8; t++) o[t] = dl * kv_iq4nl((r < 2) ? (q[t] & 15) : (q[t] >> 4));
+  } else if constexpr (C == KQ_IQ3_XXS) {  // :467-500
+    float d = ldh(b);
+    int ib = g >> 2, l = g & 3;
+    uint32_t aux = ld32(b + 66 + 4 * ib);
+    float db = d * (0.5f + (float)(aux >> 28)) * 0.5f;
+    uint32_t s = ksigns(aux >> (7 * l));
+    const uint8_t* g1 = grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l];
+    const uint8_t* g2 = grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l + 1];
+    for (int j = 0; j < 4; j++) {
+      o[j] = db * (float)g1[j] * sgn(s, j);
+      o[j + 4] = db * (float)g2[j] * sgn(s, j + 4);
+    }
+  } else if constexpr (C == KQ_IQ3_S) {  // :502-551
+    float d = ldh(b);
+    int ib = g >> 2, l = g & 3;
+    int nib = (ib & 1) ? (b[106 + (ib >> 1)] >> 4) : (b[106 + (ib >> 1)] & 15);
+    float db = d * (float)(1 + 2 * nib);
+    uint32_t h = b[66 + ib];
+    uint32_t i1 = b[2 + 8 * ib + 2 * l] | ((h << (8 - 2 * l)) & 256u);
+    uint32_t i2 = b[2 + 8 * ib + 2 * l + 1] | ((h << (7 - 2 * l)) & 256u);
+    uint32_t s = b[74 + 4 * ib + l];
+    const uint8_t* g1 = grids + KQ_GRID_IQ3S + 4 * i1;
+    const uint8_t* g2 = grids + KQ_GRID_IQ3S + 4 * i2;
+    for (int j = 0; j < 4; j++) {
+      o[j] = db * (float)g1[j] * sgn(s, j);
+      o[j + 4] = db * (float)g2[j] * sgn(s, j + 4);
+    }
+  } else if constexpr (C == KQ_IQ2_XXS) {  // :556-584
+    float d = ldh(b);
+    int ib = g >> 2, l = g & 3;
+    uint32_t a1 = ld32(b + 2 + 8 * ib + 4);
+    float db = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
+    const uint8_t* gr = grids + KQ_GRID_IQ2XXS + 8 * b[2 + 8 * ib + l];
+    uint32_t s = ksigns(a1 >> (7 * l));
+    for (int j = 0; j < 8; j++) o[j] = db * (float)gr[j] * sgn(s, j);
+  } else if constexpr (C == KQ_IQ2_XS) {  // :586-617
+    float d = ldh(b);
+    int ib = g >> 2, l = g & 3;
+    uint32_t scb = b[66 + ib];
+    float dl = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
+    uint32_t q = ld16(b + 2 + 2 * (4 * ib + l));
+    const uint8_t* gr = grids + KQ_GRID_IQ2XS + 8 * (q & 511u);
+    uint32_t s = ksigns(q >> 9);
+    for (int j = 0; j < 8; j++) o[j] = dl * (float)gr[j] * sgn(s, j);
+  } else if constexpr (C == KQ_IQ2_S) {  // :619-650
+    float d = ldh(b);
+    int ib = g >> 2, l = g & 3;
+    uint32_t scb = b[74 + ib];
+    float dl = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
+    uint32_t gi = b[2 + 4 * ib + l] | (((uint32_t)b[66 + ib] << (8 - 2 * l)) & 0x300u);
+    const uint8_t* gr = grids + KQ_GRID_IQ2S + 8 * gi;
+    uint32_t s = b[34 + 4 * ib + l];
+    for (int j = 0; j < 8; j++) o[j] = dl * (float)gr[j] * sgn(s, j);
+  } else if constexpr (C == KQ_IQ1_S) {  // :658-685
+    float d = ldh(b);
+    int ib = g >> 2, l = g & 3;
+    uint32_t qh = ld16(b + 34 + 2 * ib);
+    float dl = d * (float)(2 * (int)((qh >> 12) & 7) + 1);
+    float delta = (qh & 0x8000u) ? -0.125f : 0.125f;
+    const uint8_t* gr = grids + KQ_GRID_IQ1S + 8 * (b[2 + 4 * ib + l] | (((qh >> (3 * l)) & 7) << 8));
+    for (int j = 0; j < 8; j++) o[j] = dl * ((float)(int8_t)gr[j] + delta);
+  } else if constexpr (C == KQ_IQ1_M) {  // :687-735
+    int ib = g >> 2, l = g & 3;
+    uint32_t s0 = ld16(b + 48), s1 = ld16(b + 50), s2 = ld16(b + 52), s3 = ld16(b + 54);
+    uint16_t du = (uint16_t)((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u));
+    float d = h2f(du);
+    uint32_t scw = ld16(b + 48 + 2 * (ib >> 1));
+    int sc3 = (scw >> (6 * (ib & 1) + 3 * (l >> 1))) & 7;
+    float dl = d * (float)(2 * sc3 + 1);
+    uint32_t hb = b[32 + 2 * ib + (l >> 1)];
+    uint32_t nib = (l & 1) ? (hb >> 4) : (hb & 15);
+    float delta = (nib & 8) ? -0.125f : 0.125f;
+    const uint8_t* gr = grids + KQ_GRID_IQ1S + 8 * (b[4 * ib + l] | ((nib & 7) << 8));
+    for (int j = 0; j < 8; j++) o[j] = dl * ((float)(int8_t)gr[j] + delta);
+  }
+}
+
+// f32 -> storage dtype, one round-to-nearest-even
+__device__ __forceinline__ uint16_t f2bf16(float f) {
+  uint32_t x = __builtin_bit_cast(uint32_t, f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+  x += 0x7fffu + ((x >> 16) & 1u);
+  return (uint16_t)(x >> 16);
+}
+__device__ __forceinline__ uint16_t f2f16(float f) {
+  // Keep the f32 value in a register of its own: otherwise the compiler may fold the producing
+  // multiply into a mixed-precision fma with a +0 addend, which turns -0.0 into +0.0.
+  asm volatile("" : "+v"(f));
+  return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
+__device__ __forceinline__ float bf162f(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
+
+}  // namespace kq

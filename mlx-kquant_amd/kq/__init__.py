@@ -1,0 +1,401 @@
+"""kq -- the reference's `kq.*` quantized-weight ops on PyTorch-ROCm tensors, backed by libkq
+(hand-written HIP for gfx950 behind a C ABI, include/kq.h).
+
+Mirrors the Python op boundary of the reference (bindings.cpp:94-141, 885-952, 1349-1461 and the
+validation in src/kquant_ops.cpp / src/kquant_moe_glu.cpp): same names, argument order and
+meaning, dtype rules and error types.  Wire tensors are uint8 GGUF block bytes, unchanged.
+
+There is no CPU execution path here: tensors must live on a ROCm device, and a missing or
+unloadable libkq raises at import / first call instead of falling back.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+import torch
+
+from . import codec_geometry
+from .codec_geometry import CODEC_GEOMETRY, bytes_per_row, weights_per_row
+
+# codec -> (weights_per_block, bytes_per_block)
+_GEOM = {k: (v[3], v[2]) for k, v in CODEC_GEOMETRY.items()}
+
+__all__ = [
+    "codecs", "codec_has_matmul", "codec_has_moe_glu", "dequantize", "quantized_matmul", "gather_qmm",
+    "moe_glu_gather_kq", "gather_qmv_kq", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
+    "weights_per_row", "lib_path",
+]
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libkq.so")
+_lib = None
+
+KQ_F32, KQ_F16, KQ_BF16 = 0, 1, 2
+_ACTS = {"silu": 0, "gelu": 1, "silu_limit": 2, "swiglu_clamp": 3}
+_DT = {torch.float32: KQ_F32, torch.float16: KQ_F16, torch.bfloat16: KQ_BF16}
+
+
+class _CodecInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 16), ("weights_per_block", C.c_int), ("bytes_per_block", C.c_int),
+                ("bits", C.c_int), ("has_matmul_kernel", C.c_int), ("has_encode", C.c_int),
+                ("has_nax_kernel", C.c_int), ("requires_imatrix", C.c_int)]
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def _load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise RuntimeError(
+            f"[kq] {_LIB_PATH} is missing: build it with `python mlx-kquant_amd/build.py` "
+            "(there is no fallback implementation)")
+    lib = C.CDLL(_LIB_PATH)
+    vp, i, i64, u64, f, sz = C.c_void_p, C.c_int, C.c_int64, C.c_uint64, C.c_float, C.c_size_t
+    lib.kq_last_error.restype = C.c_char_p
+    lib.kq_version.restype = C.c_char_p
+    lib.kq_codec_id.argtypes = [C.c_char_p]
+    lib.kq_codec_get.argtypes = [i, C.POINTER(_CodecInfo)]
+    lib.kq_codec_has_moe_glu.argtypes = [i]
+    lib.kq_dequantize.argtypes = [vp, vp, u64, i, i, vp]
+    lib.kq_qmm_workspace_size.restype = sz
+    lib.kq_qmm_workspace_size.argtypes = [i, i, i, i, i, i]
+    lib.kq_qmm.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
+    lib.kq_gather_qmm_workspace_size.restype = sz
+    lib.kq_gather_qmm_workspace_size.argtypes = [i, i, i, i, i, i, i]
+    lib.kq_gather_qmm.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i64, i64, i, i, i, i, vp, sz, vp]
+    lib.kq_moe_glu_gather.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, f, f, i, i, vp]
+    lib.kq_gather_qmv.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp]
+    lib.kq_quantize.argtypes = [vp, vp, vp, i64, i64, i]
+    _lib = lib
+    return lib
+
+
+def _check(rc: int):
+    if rc == 0:
+        return
+    msg = _load().kq_last_error().decode(errors="replace")
+    if rc == -1:
+        raise ValueError("[kq] " + msg)
+    raise RuntimeError("[kq] " + msg)
+
+
+def _codec(op: str, name: str):
+    cid = _load().kq_codec_id(str(name).encode())
+    if cid < 0:
+        raise ValueError(f"[kq.{op}] Unknown kquant_type: '{name}'.")
+    return cid, _GEOM[name]
+
+
+def _stream_ptr(op: str, t: torch.Tensor, stream) -> int:
+    if isinstance(stream, str) and stream == "cpu" or isinstance(stream, torch.device) and stream.type == "cpu":
+        raise RuntimeError(f"[kq.{op}] this build has no CPU execution path; tensors must be on a ROCm device")
+    if t.device.type != "cuda":
+        raise RuntimeError(f"[kq.{op}] tensors must live on a ROCm device (got {t.device}); there is no CPU path")
+    if isinstance(stream, torch.cuda.Stream):
+        return stream.cuda_stream
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _same_device(op, ref, *ts):
+    for t in ts:
+        if t is not None and t.device != ref.device:
+            raise ValueError(f"[kq.{op}] all tensors must be on the same device")
+
+
+# ------------------------------------------------------------------ introspection
+def codecs():
+    """Canonical ordered codec names (bindings.cpp:40-60)."""
+    lib = _load()
+    out, info = [], _CodecInfo()
+    for i in range(lib.kq_codec_count()):
+        lib.kq_codec_get(i, C.byref(info))
+        out.append(info.name.decode())
+    return out
+
+
+def codec_has_matmul(kquant_type: str) -> bool:
+    lib = _load()
+    cid = lib.kq_codec_id(str(kquant_type).encode())
+    if cid < 0:
+        return False
+    info = _CodecInfo()
+    lib.kq_codec_get(cid, C.byref(info))
+    return bool(info.has_matmul_kernel)
+
+
+def codec_has_moe_glu(kquant_type: str) -> bool:
+    lib = _load()
+    cid = lib.kq_codec_id(str(kquant_type).encode())
+    return cid >= 0 and bool(lib.kq_codec_has_moe_glu(cid))
+
+
+# ------------------------------------------------------------------ ops
+def dequantize(w, scales, kquant_type, dtype=None, *, stream=None):
+    """Decode wire bytes `w` (uint8 [..., bytes_per_row]) to `dtype` (default float16).
+    Mirrors dequantize, reference src/kquant_ops.cpp:55-110."""
+    op = "dequantize"
+    if w.dtype != torch.uint8:
+        raise ValueError("[kq.dequantize] w must be uint8 (raw GGUF wire bytes).")
+    if w.ndim < 1:
+        raise ValueError("[kq.dequantize] w must have at least 1 dimension.")
+    cid, (wpb, bpb) = _codec(op, kquant_type)
+    if w.shape[-1] % bpb != 0:
+        raise ValueError(f"[kq.dequantize] Last dim ({w.shape[-1]}) must be a multiple of bytes_per_block "
+                         f"({bpb}) for codec '{kquant_type}'.")
+    out_type = dtype if dtype is not None else torch.float16
+    if out_type not in _DT:
+        raise ValueError("[kq.dequantize] Only real floating output dtypes are supported.")
+    sp = _stream_ptr(op, w, stream)
+    w_c = w.contiguous()
+    out_shape = list(w.shape)
+    out_shape[-1] = w.shape[-1] // bpb * wpb
+    out = torch.empty(out_shape, dtype=out_type, device=w.device)
+    with torch.cuda.device(w.device):
+        _check(_load().kq_dequantize(w_c.data_ptr(), out.data_ptr(), out.numel(), cid, _DT[out_type], sp))
+    return out
+
+
+def _out_dtype(op, x):
+    if not x.dtype.is_floating_point or x.dtype not in _DT:
+        raise ValueError(f"[kq.{op}] Only real floating x dtypes are supported.")
+    return torch.bfloat16 if x.dtype == torch.float32 else x.dtype
+
+
+def _expand_geometry(op, x, w, kquant_type, transpose):
+    cid, (wpb, bpb) = _codec(op, kquant_type)
+    bpr = w.shape[-1]
+    if bpr % bpb != 0:
+        raise ValueError(f"[kq.{op}] KQuant weight last dim ({bpr} bytes) is not a whole number of "
+                         f"{bpb}-byte {kquant_type} blocks.")
+    wpr = bpr // bpb * wpb
+    inner = wpr if transpose else w.shape[-2]
+    outer = w.shape[-2] if transpose else wpr
+    if inner != x.shape[-1]:
+        raise ValueError(f"[kq.{op}] x last dim ({x.shape[-1]}) does not match the expanded quantized matrix inner "
+                         f"dim ({inner}) for codec '{kquant_type}' with transpose={str(bool(transpose)).lower()}.")
+    return cid, inner, outer
+
+
+def quantized_matmul(x, w, scales, kquant_type, transpose=True, *, stream=None):
+    """y = x @ W.T (transpose) or x @ W.  Output dtype = x dtype, float32 promoted to bfloat16 (the
+    activations themselves are cast first).  Mirrors quantized_matmul, src/kquant_ops.cpp:112-183."""
+    op = "quantized_matmul"
+    if w.dtype != torch.uint8:
+        raise ValueError("[kq.quantized_matmul] w must be uint8 (raw GGUF wire bytes).")
+    if x.ndim > 2 and w.ndim > 2:
+        raise ValueError("[kq.quantized_matmul] batched (>2D) weights are not supported; use gather_qmm for "
+                         "mixture-of-experts.")
+    if w.ndim != 2:
+        raise ValueError("[kq.quantized_matmul] w must be 2-D [rows, bytes_per_row].")
+    if x.ndim < 1:
+        raise ValueError("[kq.quantized_matmul] x must have at least 1 dimension.")
+    cid, K, N = _expand_geometry(op, x, w, kquant_type, transpose)
+    out_type = _out_dtype(op, x)
+    _same_device(op, x, w)
+    sp = _stream_ptr(op, x, stream)
+    x_c = x.to(out_type).contiguous()
+    w_c = w.contiguous()
+    M = x_c.numel() // K if K else 0
+    out = torch.empty(list(x.shape[:-1]) + [N], dtype=out_type, device=x.device)
+    lib = _load()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.kq_qmm_workspace_size(M, N, K, int(bool(transpose)), cid, _DT[out_type])
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+        _check(lib.kq_qmm(x_c.data_ptr(), w_c.data_ptr(), out.data_ptr(), M, N, K, int(bool(transpose)), cid,
+                          _DT[out_type], ws.data_ptr() if ws is not None else None, ws_bytes, sp))
+    return out
+
+
+def _default_indices(t):
+    shape = t.shape[:-2]
+    total = 1
+    for d in shape:
+        total *= d
+    return torch.arange(total, dtype=torch.int64, device=t.device).reshape(shape)
+
+
+def gather_qmm(x, w, scales, kquant_type, lhs_indices=None, rhs_indices=None, transpose=True,
+               sorted_indices=False, *, stream=None):
+    """out[i] = x[lhs[i]] @ W[rhs[i]].T; out shape = broadcast(lhs, rhs).shape + [M, N].
+    Mirrors gather_qmm, src/kquant_ops.cpp:293-420."""
+    op = "gather_qmm"
+    if lhs_indices is None and rhs_indices is None:
+        return quantized_matmul(x, w, scales, kquant_type, transpose, stream=stream)
+    if w.dtype != torch.uint8:
+        raise ValueError("[kq.gather_qmm] w must be uint8 (raw GGUF wire bytes).")
+    _codec(op, kquant_type)
+    if x.ndim < 2:
+        raise ValueError(f"[kq.gather_qmm] x must have at least two dimensions but got shape {tuple(x.shape)}.")
+    if w.ndim < 2:
+        raise ValueError("[kq.gather_qmm] w must have at least two dimensions.")
+    cid, K, N = _expand_geometry(op, x, w, kquant_type, transpose)
+    out_type = _out_dtype(op, x)
+    _same_device(op, x, w, lhs_indices, rhs_indices)
+    sp = _stream_ptr(op, x, stream)
+    lhs = lhs_indices if lhs_indices is not None else _default_indices(x)
+    rhs = rhs_indices if rhs_indices is not None else _default_indices(w)
+    lhs, rhs = torch.broadcast_tensors(lhs, rhs)
+    idx_shape = list(lhs.shape)
+    lhs = lhs.to(torch.int64).reshape(-1).to(torch.int32).contiguous()  # uint32 bit pattern
+    rhs = rhs.to(torch.int64).reshape(-1).to(torch.int32).contiguous()
+    M = x.shape[-2]
+    x_c = x.to(out_type).reshape(-1, M, K).contiguous()
+    # the expert (leading) dim of w may be strided; rows inside one expert must be packed
+    if w.ndim == 3 and w.stride(-1) == 1 and w.stride(-2) == w.shape[-1]:
+        w3 = w
+    else:
+        w3 = w.contiguous().reshape(-1, w.shape[-2], w.shape[-1])
+    estride = w3.stride(0) if w3.shape[0] > 1 else w3.shape[1] * w3.shape[2]
+    B = lhs.numel()
+    out = torch.empty(idx_shape + [M, N], dtype=out_type, device=x.device)
+    right_sorted = bool(sorted_indices) and lhs_indices is None
+    lib = _load()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.kq_gather_qmm_workspace_size(B, M, N, K, int(bool(transpose)), cid, _DT[out_type])
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+        _check(lib.kq_gather_qmm(x_c.data_ptr(), w3.data_ptr(), lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), B, M, N,
+                                 K, M * K, estride, int(bool(transpose)), int(right_sorted), cid, _DT[out_type],
+                                 ws.data_ptr() if ws is not None else None, ws_bytes, sp))
+    return out
+
+
+def _check_kq_expert_stack(op, w, kquant_type, K):
+    """check_kq_expert_stack, src/kquant_moe_glu.cpp:861-896."""
+    if kquant_type not in CODEC_GEOMETRY or not codec_has_moe_glu(kquant_type):
+        raise ValueError(f"[kq.{op}] codec '{kquant_type}' has no fused MoE kernel.")
+    wpb, bpb = _GEOM[kquant_type]
+    if w.ndim != 3 or w.dtype != torch.uint8:
+        raise ValueError(f"[kq.{op}] expert weights must be uint8 [E, N, bytes_per_row].")
+    if K % wpb != 0 or w.shape[2] != K // wpb * bpb:
+        raise ValueError(f"[kq.{op}] weight trailing dim does not match K for '{kquant_type}'.")
+    if w.shape[1] % 8 != 0:
+        raise ValueError(f"[kq.{op}] N must be a multiple of 8.")
+    if not w.is_contiguous():
+        raise ValueError(f"[kq.{op}] weights must be row-contiguous.")
+
+
+def _prep_idx(idx):
+    return idx.to(torch.int64).to(torch.int32).contiguous()
+
+
+def moe_glu_gather_kq(x, gate_w, up_w, kquant_type, indices, act="silu", limit=0.0, gate_bias=None, up_bias=None,
+                      alpha=0.0, *, stream=None):
+    """out[t, r] = act(x[t] @ G_e.T, x[t] @ U_e.T), e = indices[t, r]; [T, R, N] in x's dtype.
+    Mirrors moe_glu_gather_kq, src/kquant_moe_glu.cpp:1070-1157."""
+    op = "moe_glu_gather_kq"
+    if x.ndim != 2:
+        raise ValueError("[kq.moe_glu_gather_kq] x must be 2-D [T, K].")
+    if indices.ndim != 2 or indices.shape[0] != x.shape[0]:
+        raise ValueError("[kq.moe_glu_gather_kq] indices must be [T, R].")
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("[kq.moe_glu_gather_kq] x must be float16 or bfloat16.")
+    if act not in _ACTS:
+        raise ValueError("[kq.moe_glu_gather_kq] act must be 'silu', 'gelu', 'silu_limit' or 'swiglu_clamp'.")
+    if act == "silu_limit" and not (limit > 0.0):
+        raise ValueError("[kq.moe_glu_gather_kq] act 'silu_limit' requires limit > 0.")
+    biased = gate_bias is not None or up_bias is not None
+    if act == "swiglu_clamp":
+        if gate_bias is None or up_bias is None or not (limit > 0.0) or not (alpha > 0.0):
+            raise ValueError("[kq.moe_glu_gather_kq] act 'swiglu_clamp' requires gate_bias, up_bias, limit > 0 and "
+                             "alpha > 0.")
+        if kquant_type not in ("mxfp4", "nvfp4"):
+            raise ValueError("[kq.moe_glu_gather_kq] biased kernels are instantiated for mxfp4/nvfp4 only.")
+    elif biased:
+        raise ValueError("[kq.moe_glu_gather_kq] gate_bias/up_bias require act 'swiglu_clamp'.")
+    K = x.shape[1]
+    _check_kq_expert_stack(op, gate_w, kquant_type, K)
+    _check_kq_expert_stack(op, up_w, kquant_type, K)
+    if gate_w.shape[0] != up_w.shape[0] or gate_w.shape[1] != up_w.shape[1]:
+        raise ValueError("[kq.moe_glu_gather_kq] gate/up expert shapes must match.")
+    if biased:
+        for b in (gate_bias, up_bias):
+            if b.ndim != 2 or b.shape[0] != gate_w.shape[0] or b.shape[1] != gate_w.shape[1]:
+                raise ValueError("[kq.moe_glu_gather_kq] biases must be [E, N] matching the expert stacks.")
+    _same_device(op, x, gate_w, up_w, indices, gate_bias, up_bias)
+    sp = _stream_ptr(op, x, stream)
+    cid, _ = _codec(op, kquant_type)
+    x_c = x.contiguous()
+    idx = _prep_idx(indices)
+    gb = gate_bias.to(torch.float32).contiguous() if biased else None
+    ub = up_bias.to(torch.float32).contiguous() if biased else None
+    T, R = idx.shape
+    E, N = gate_w.shape[0], gate_w.shape[1]
+    out = torch.empty((T, R, N), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(_load().kq_moe_glu_gather(x_c.data_ptr(), gate_w.data_ptr(), up_w.data_ptr(), idx.data_ptr(),
+                                         gb.data_ptr() if biased else None, ub.data_ptr() if biased else None,
+                                         out.data_ptr(), T, R, E, N, K, _ACTS[act], float(limit), float(alpha), cid,
+                                         _DT[x.dtype], sp))
+    return out
+
+
+def gather_qmv_kq(x, w, kquant_type, indices, bias=None, *, stream=None):
+    """out[t, r] = x[t, r] @ W_e.T (+ bias_e), e = indices[t, r]; x [T, R, K] -> [T, R, N].
+    Mirrors gather_qmv_kq, src/kquant_moe_glu.cpp:1159-1210."""
+    op = "gather_qmv_kq"
+    if x.ndim != 3:
+        raise ValueError("[kq.gather_qmv_kq] x must be 3-D [T, R, K].")
+    if indices.ndim != 2 or indices.shape[0] != x.shape[0] or indices.shape[1] != x.shape[1]:
+        raise ValueError("[kq.gather_qmv_kq] indices must be [T, R] matching x.")
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("[kq.gather_qmv_kq] x must be float16 or bfloat16.")
+    K = x.shape[2]
+    _check_kq_expert_stack(op, w, kquant_type, K)
+    if bias is not None:
+        if kquant_type not in ("mxfp4", "nvfp4"):
+            raise ValueError("[kq.gather_qmv_kq] biased kernels are instantiated for mxfp4/nvfp4 only.")
+        if bias.ndim != 2 or bias.shape[0] != w.shape[0] or bias.shape[1] != w.shape[1]:
+            raise ValueError("[kq.gather_qmv_kq] bias must be [E, N] matching the expert stack.")
+    _same_device(op, x, w, indices, bias)
+    sp = _stream_ptr(op, x, stream)
+    cid, _ = _codec(op, kquant_type)
+    x_c = x.contiguous()
+    idx = _prep_idx(indices)
+    b = bias.to(torch.float32).contiguous() if bias is not None else None
+    T, R = idx.shape
+    E, N = w.shape[0], w.shape[1]
+    out = torch.empty((T, R, N), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(_load().kq_gather_qmv(x_c.data_ptr(), w.data_ptr(), idx.data_ptr(),
+                                     b.data_ptr() if b is not None else None, out.data_ptr(), T, R, E, N, K, cid,
+                                     _DT[x.dtype], sp))
+    return out
+
+
+def quantize(w, kquant_type, imatrix=None, *, stream=None):
+    """Encode float weights [..., K] to wire bytes; returns (wq uint8 [..., bytes_per_row], scales uint8 [1]).
+    A host (CPU) encoder, as in the reference for the IQ codecs; the result is placed on w's device.
+    Mirrors quantize, src/kquant_ops.cpp:550-631."""
+    op = "quantize"
+    cid, (wpb, bpb) = _codec(op, kquant_type)
+    if not w.dtype.is_floating_point:
+        raise ValueError("[kq.quantize] w must be a real floating tensor.")
+    if w.ndim < 1:
+        raise ValueError("[kq.quantize] w must have at least 1 dimension.")
+    K = w.shape[-1]
+    if K % wpb != 0:
+        raise ValueError(f"[kq.quantize] Last dim ({K}) must be a multiple of weights_per_block ({wpb}) for codec "
+                         f"'{kquant_type}'.")
+    info = _CodecInfo()
+    _load().kq_codec_get(cid, C.byref(info))
+    if not info.has_encode:
+        raise ValueError(f"[kq.quantize] codec '{kquant_type}' has no encoder.")
+    im = None
+    if imatrix is not None:
+        if imatrix.ndim != 1 or imatrix.shape[0] != K:
+            raise ValueError(f"[kq.quantize] imatrix must be 1-D with length {K}.")
+        im = imatrix.detach().to("cpu", torch.float32).contiguous()
+    elif info.requires_imatrix:
+        raise ValueError(f"[kq.quantize] codec '{kquant_type}' requires an importance matrix (imatrix).")
+    w_h = w.detach().to("cpu", torch.float32).contiguous()
+    rows = w_h.numel() // K if K else 0
+    wire = torch.empty(list(w.shape[:-1]) + [K // wpb * bpb], dtype=torch.uint8)
+    _check(_load().kq_quantize(w_h.data_ptr(), im.data_ptr() if im is not None else None, wire.data_ptr(), rows, K,
+                               cid))
+    return wire.to(w.device), torch.zeros(1, dtype=torch.uint8, device=w.device)

@@ -1,0 +1,89 @@
+"""GPU parity: kq.quantized_matmul (HIP) vs the CPU oracle.  Tolerance: rel-L2 <= 1e-3 on the
+rounded outputs (fp32 accumulation, one rounding to the activation dtype)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as O
+from gpu_util import bits_to_dev, dev_to_bits, make_x, rel_l2, wire_to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def kq():
+    import kq as _kq
+    return _kq
+
+
+def _wire(codec, N, K, seed):
+    wpb, bpb = O.geometry(codec)
+    return O.synth_wire(codec, N * (K // wpb), seed).reshape(N, K // wpb * bpb)
+
+
+@pytest.mark.parametrize("codec", O.ALL_CODECS)
+@pytest.mark.parametrize("M", [1, 3, 8])
+def test_qmm_all_codecs_small(kq, codec, M):
+    N, K = 96, 512
+    wire = _wire(codec, N, K, seed=31)
+    for dtype in ("bfloat16", "float16"):
+        xb, xt = make_x((M, K), dtype, seed=M)
+        got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+        want = O.qmm(xb, wire, codec, True, dtype)
+        assert tuple(got.shape) == (M, N)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, dtype)
+
+
+@pytest.mark.parametrize("codec", ["q4_k", "q6_k", "q5_k", "q8_0", "iq4_xs", "mxfp4"])
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 17, 64])
+def test_qmm_decode_and_prefill_shapes(kq, codec, M):
+    N, K = 256, 2048 if codec != "mxfp4" else 2880
+    wire = _wire(codec, N, K, seed=32)
+    xb, xt = make_x((M, K), "bfloat16", seed=100 + M)
+    got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+    want = O.qmm(xb, wire, codec, True, "bfloat16")
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, M)
+
+
+@pytest.mark.parametrize("codec", ["q4_k", "q8_0", "iq4_nl"])
+def test_qmm_no_transpose(kq, codec):
+    K, N, M = 64, 512, 5  # W decodes to [K, N]
+    wire = _wire(codec, K, N, seed=33)
+    xb, xt = make_x((M, K), "float16", seed=7)
+    got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec, transpose=False)
+    want = O.qmm(xb, wire, codec, False, "float16")
+    assert tuple(got.shape) == (M, N)
+    assert rel_l2(dev_to_bits(got), want, "float16") <= TOL
+
+
+def test_qmm_dtype_rules_and_shapes(kq):
+    N, K = 64, 256
+    wire = _wire("q4_k", N, K, seed=34)
+    w = wire_to_dev(wire)
+    x32 = torch.from_numpy(np.random.default_rng(1).standard_normal((2, 3, K)).astype(np.float32)).cuda()
+    y = kq.quantized_matmul(x32, w, None, "q4_k")
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (2, 3, N)  # f32 -> bf16, x cast first
+    xb = O.f32_to_bits(x32.cpu().numpy().reshape(6, K), "bfloat16")
+    want = O.qmm(xb, wire, "q4_k", True, "bfloat16")
+    assert rel_l2(dev_to_bits(y).reshape(6, N), want, "bfloat16") <= TOL
+    with pytest.raises(ValueError):
+        kq.quantized_matmul(x32[..., :128], w, None, "q4_k")
+    with pytest.raises(ValueError):
+        kq.quantized_matmul(x32, w.reshape(1, N, -1), None, "q4_k")
+    with pytest.raises(ValueError):
+        kq.quantized_matmul(x32.to(torch.int32), w, None, "q4_k")
+    empty = kq.quantized_matmul(x32[:0], w, None, "q4_k")
+    assert tuple(empty.shape) == (0, 3, N)
+
+
+@pytest.mark.parametrize("codec", ["q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+def test_qmm_reference_fixtures(kq, codec):
+    import os
+    gold = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    wire = np.load(os.path.join(gold, f"{codec}.npz"))["wire"]  # [256, bpr], K = 512
+    for M in (1, 64):
+        xb, xt = make_x((M, 512), "float16", seed=M)
+        got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+        want = O.qmm(xb, wire, codec, True, "float16")
+        assert rel_l2(dev_to_bits(got), want, "float16") <= TOL

@@ -1,0 +1,148 @@
+"""GPU parity: gather_qmm, moe_glu_gather_kq, gather_qmv_kq (HIP) vs the CPU oracle."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as O
+from gpu_util import bits_to_dev, dev_to_bits, make_x, rel_l2, wire_to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module")
+def kq():
+    import kq as _kq
+    return _kq
+
+
+def _stack(codec, E, N, K, seed):
+    wpb, bpb = O.geometry(codec)
+    return O.synth_wire(codec, E * N * (K // wpb), seed).reshape(E, N, K // wpb * bpb)
+
+
+def _idx_dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a).astype(np.int64)).cuda()
+
+
+@pytest.mark.parametrize("codec", ["q4_k", "q6_k", "q2_k", "iq3_s", "mxfp4", "q8_0"])
+@pytest.mark.parametrize("M", [1, 5])
+def test_gather_qmm(kq, codec, M):
+    E, N, K, B = 4, 128, 512 if codec != "mxfp4" else 288, 8
+    wire = _stack(codec, E, N, K, seed=41)
+    xb, xt = make_x((B, M, K), "float16", seed=42)
+    rng = np.random.default_rng(43)
+    rhs = rng.integers(0, E, B)
+    # arange lhs (rhs only given)
+    got = kq.gather_qmm(xt, wire_to_dev(wire), None, codec, rhs_indices=_idx_dev(rhs))
+    want = O.gather_qmm(xb, wire, codec, np.arange(B), rhs, True, "float16")
+    assert tuple(got.shape) == (B, M, N)
+    assert rel_l2(dev_to_bits(got), want, "float16") <= TOL
+    # reversed lhs with repeats, 2-D index arrays
+    lhs = np.array([7, 6, 5, 4, 3, 3, 1, 0]).reshape(2, 4)
+    got = kq.gather_qmm(xt, wire_to_dev(wire), None, codec, lhs_indices=_idx_dev(lhs),
+                        rhs_indices=_idx_dev(rhs.reshape(2, 4)))
+    want = O.gather_qmm(xb, wire, codec, lhs.reshape(-1), rhs, True, "float16")
+    assert tuple(got.shape) == (2, 4, M, N)
+    assert rel_l2(dev_to_bits(got).reshape(B, M, N), want, "float16") <= TOL
+
+
+def test_gather_qmm_reference_moe_fixture_and_strided_experts(kq):
+    wire = np.load(os.path.join(GOLD, "q4_k_moe.npz"))["wire"]  # [4, 128, 288]
+    E, N, K, B = 4, 128, 512, 64
+    xb, xt = make_x((B, 1, K), "bfloat16", seed=44)
+    rhs = np.sort(np.random.default_rng(45).integers(0, E, B))
+    got = kq.gather_qmm(xt, wire_to_dev(wire), None, "q4_k", rhs_indices=_idx_dev(rhs), sorted_indices=True)
+    want = O.gather_qmm(xb, wire, "q4_k", np.arange(B), rhs, True, "bfloat16")
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
+    # gate half of a fused gate_up stack: expert stride is twice the matrix size
+    fused = np.concatenate([wire, wire[::-1]], axis=1)  # [4, 256, 288]
+    got = kq.gather_qmm(xt, wire_to_dev(fused)[:, :128, :], None, "q4_k", rhs_indices=_idx_dev(rhs))
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
+    # duplicate (x, expert) entries give bit-identical rows
+    lhs = np.zeros(B, dtype=np.int64)
+    got = dev_to_bits(kq.gather_qmm(xt, wire_to_dev(wire), None, "q4_k", lhs_indices=_idx_dev(lhs),
+                                    rhs_indices=_idx_dev(np.zeros(B, dtype=np.int64))))
+    assert all(np.array_equal(got[0], got[i]) for i in range(B))
+
+
+def _glu_truth(codec, xb, gate, up, idx, act, limit=0.0, alpha=0.0, gb=None, ub=None, dtype="bfloat16"):
+    return O.moe_glu_gather(xb, gate, up, codec, idx, act, limit, gb, ub, alpha, dtype)
+
+
+@pytest.mark.parametrize("codec", O.ALL_CODECS)
+def test_moe_glu_all_codecs(kq, codec):
+    E, N, K, T, R = 4, 64, 512 if codec not in ("mxfp4",) else 288, 3, 2
+    gate = _stack(codec, E, N, K, seed=51)
+    up = gate[::-1].copy()
+    idx = np.random.default_rng(52).integers(0, E, (T, R))
+    for dtype in ("float16", "bfloat16"):
+        xb, xt = make_x((T, K), dtype, seed=53, scale=0.1)
+        got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx))
+        want = _glu_truth(codec, xb, gate, up, idx, "silu", dtype=dtype)
+        assert tuple(got.shape) == (T, R, N)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype)
+        hb, ht = make_x((T, R, K), dtype, seed=54, scale=0.1)
+        got = kq.gather_qmv_kq(ht, wire_to_dev(gate), codec, _idx_dev(idx))
+        want = O.gather_qmv(hb, gate, codec, idx, None, dtype)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype)
+
+
+@pytest.mark.parametrize("act,limit", [("gelu", 0.0), ("silu_limit", 0.5), ("silu", 0.0)])
+def test_moe_glu_activations(kq, act, limit):
+    codec, E, N, K, T, R = "q6_k", 4, 64, 512, 5, 3
+    gate = _stack(codec, E, N, K, seed=55)
+    up = _stack(codec, E, N, K, seed=56)
+    idx = np.random.default_rng(57).integers(0, E, (T, R))
+    xb, xt = make_x((T, K), "bfloat16", seed=58, scale=0.3)
+    got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act=act, limit=limit)
+    want = _glu_truth(codec, xb, gate, up, idx, act, limit)
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
+
+
+@pytest.mark.parametrize("codec", ["mxfp4", "nvfp4"])
+def test_moe_swiglu_clamp_bias(kq, codec):
+    E, N, K, T, R = 4, 64, 576, 4, 2
+    gate = _stack(codec, E, N, K, seed=61)
+    up = _stack(codec, E, N, K, seed=62)
+    rng = np.random.default_rng(63)
+    gb = (rng.standard_normal((E, N)) * 0.01).astype(np.float32)
+    ub = (rng.standard_normal((E, N)) * 0.01).astype(np.float32)
+    idx = rng.integers(0, E, (T, R))
+    xb, xt = make_x((T, K), "bfloat16", seed=64, scale=0.2)
+    got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act="swiglu_clamp",
+                               limit=7.0, gate_bias=torch.from_numpy(gb).cuda(), up_bias=torch.from_numpy(ub).cuda(),
+                               alpha=1.702)
+    want = _glu_truth(codec, xb, gate, up, idx, "swiglu_clamp", 7.0, 1.702, gb, ub)
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
+    hb, ht = make_x((T, R, K), "bfloat16", seed=65, scale=0.2)
+    got = kq.gather_qmv_kq(ht, wire_to_dev(gate), codec, _idx_dev(idx), bias=torch.from_numpy(gb).cuda())
+    want = O.gather_qmv(hb, gate, codec, idx, gb, "bfloat16")
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
+
+
+def test_moe_validation_errors(kq):
+    d = torch.device("cuda:0")
+    E, N, K = 2, 16, 256
+    w = torch.zeros((E, N, 144), dtype=torch.uint8, device=d)
+    x = torch.zeros((3, K), dtype=torch.float16, device=d)
+    idx = torch.zeros((3, 2), dtype=torch.int64, device=d)
+    with pytest.raises(ValueError):
+        kq.moe_glu_gather_kq(x.float(), w, w, "q4_k", idx)
+    with pytest.raises(ValueError):
+        kq.moe_glu_gather_kq(x, w, w, "q4_k", idx, act="relu")
+    with pytest.raises(ValueError):
+        kq.moe_glu_gather_kq(x, w, w, "q4_k", idx, act="silu_limit")
+    with pytest.raises(ValueError):
+        kq.moe_glu_gather_kq(x, w, w, "q4_k", idx, gate_bias=torch.zeros((E, N), device=d))
+    with pytest.raises(ValueError):
+        kq.moe_glu_gather_kq(x, w, w[:, :8], "q4_k", idx)
+    with pytest.raises(ValueError):
+        kq.moe_glu_gather_kq(x, w[:, :, :100], w[:, :, :100], "q4_k", idx)
+    with pytest.raises(ValueError):
+        kq.gather_qmv_kq(x, w, "q4_k", idx)
+    with pytest.raises(ValueError):
+        kq.gather_qmv_kq(x.reshape(3, 1, K).expand(3, 2, K), w, "q4_k", idx, bias=torch.zeros((E, N), device=d))
