@@ -19,6 +19,7 @@ SOURCES = [
     ("kq_api.cpp", ["-x", "hip"]),
     ("kq_encode.cpp", ["-x", "hip"]),
     ("kq_generic.hip", ["-ffp-contract=off"]),
+    # MFMA results are consumed by VALU code right away: keep them in VGPRs, not AGPRs
     ("kq_mfma.hip", []),
 ]
 COMMON = [
