@@ -46,6 +46,15 @@ struct StaticFor<0> {
   __device__ __forceinline__ static void run(F&&) {}
 };
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory,
+// which on this target drains every outstanding global load (s_waitcnt vmcnt(0)) and would
+// serialise the weight stream behind each barrier.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 struct Q4kRaw {
   uint4 hdr;
   uint4 q[4];
@@ -157,7 +166,6 @@ __global__ __launch_bounds__(SK_THREADS, 2) void q4k_skinny_kernel(const void* _
                                                                    void* __restrict__ y, int M, int N, int K,
                                                                    int rows_per_tile, int kch) {
   constexpr int R = MB < 4 ? MB : 4;  // accumulator registers carried per lane
-  constexpr int MAXP = 18;            // 16-byte pieces per thread per chunk (32 rows x 16 superblocks)
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // layout: wt [rows_per_tile][kch*144 + 16] | xs f16 [MB][kch*256] | xsum f32 [kch*8][MB] | red | scratch
   const int chunk_bytes = kch * 144, wstride = chunk_bytes + 16, kchunk = kch * 256;
@@ -182,56 +190,92 @@ __global__ __launch_bounds__(SK_THREADS, 2) void q4k_skinny_kernel(const void* _
 #pragma unroll
   for (int r = 0; r < R; r++) acc[r] = 0.f;
 
+  constexpr int SBC = 4;  // superblocks per sub-chunk: one per wave
+  constexpr int NCH = 4;  // sub-chunks per chunk (kch <= 16), all in flight at once
+  constexpr int PPC = 5;  // 16-byte pieces per thread per sub-chunk: ceil(32 rows * 36 / 256)
+  // activation staging slots per thread: slot t = (row t / XK, k-pass t % XK); a chunk holds at
+  // most min(512, 1024 / MB) 8-element groups per row because kch * MB <= 32
+  constexpr int XK = MB <= 2 ? 2 : 1;
+  constexpr int XG = MB * XK;
+
+  // piece map of the weight stream (see step 2): global / LDS byte offsets inside a sub-chunk
+  uint32_t goff[PPC], loff[PPC];
+  int ppc[PPC];
+  bool piece_ok[PPC];
+  {
+    int r = tid / 36, pc = tid % 36;
+    StaticFor<PPC>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      piece_ok[T] = r < nrows;
+      ppc[T] = pc;
+      goff[T] = (uint32_t)r * (uint32_t)row_bytes + 16 * pc;
+      loff[T] = (uint32_t)r * (uint32_t)wstride + 16 * pc;
+      r += SK_THREADS / 36;
+      pc += SK_THREADS % 36;
+      if (pc >= 36) {
+        pc -= 36;
+        r++;
+      }
+    });
+  }
+  uint8_t* dump = reinterpret_cast<uint8_t*>(scratch + 16) + 16 * tid;  // per-thread 16-byte dump slot
+
   for (int sb0 = 0; sb0 < nsb; sb0 += kch) {
     const int sbn = (nsb - sb0 < kch) ? (nsb - sb0) : kch;
     const int kc = sbn << 8, k0 = sb0 << 8;
-    const int cpr = sbn * 9;  // 16-byte pieces per row in this chunk
-    // ---- issue the weight loads: piece i = tid + 256 t -> (row i / cpr, 16-byte piece i % cpr),
-    // tracked incrementally; out-of-range pieces re-read piece 0 and are not stored
-    u32x4 wreg[MAXP];
-    const int step_r = SK_THREADS / cpr, step_c = SK_THREADS % cpr;
-    const int r_first = tid / cpr, c_first = tid % cpr;
-    {
-      int r = r_first, c = c_first;
-      const uint8_t* src = wtile + (size_t)sb0 * 144;
-      StaticFor<MAXP>::run([&](auto t) {
-        const bool ok = r < nrows;
-        const size_t off = ok ? (size_t)r * row_bytes + 16 * c : 0;
-        wreg[decltype(t)::value] = *reinterpret_cast<const u32x4*>(src + off);
-        r += step_r;
-        c += step_c;
-        if (c >= cpr) {
-          c -= cpr;
-          r++;
+
+    // ---- 1. activation loads first, so waiting for them does not wait for the weights
+    const int gpr = kc >> 3;         // 8-element groups per activation row in this chunk
+    u32x4 xreg[XG];
+    // (loads are unconditional and branch-free -- out-of-range slots re-read valid data -- so the
+    // compiler can count outstanding loads exactly and wait for the activations alone)
+    StaticFor<XG>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      int m = T / XK;
+      m = m < M ? m : M - 1;  // spare rows of the MB-row block mirror the last real row
+      int kgi = tid + (T % XK) * SK_THREADS;
+      kgi = kgi < gpr ? kgi : 0;
+      xreg[T] = *reinterpret_cast<const u32x4*>(x16 + (size_t)m * K + k0 + 8 * kgi);
+    });
+
+    // ---- 2. weight stream.  Sub-chunk c covers superblocks [4c, 4c+4) = 36 16-byte pieces per
+    // row; piece i = tid + 256 t maps to (row i / 36, piece i % 36), so consecutive lanes read
+    // consecutive 16-byte pieces of a row.  The map is the same for every sub-chunk (goff / loff
+    // below); pieces outside the tile or a ragged last sub-chunk re-read the tile's first bytes and
+    // land in a dump slot.  Two sub-chunks are in flight at any time (register sets c % 2); the
+    // next one is issued as soon as its register set has been parked in LDS.
+    u32x4 wreg[2 * PPC];
+    auto issue = [&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      const int sbc = sbn - SBC * c;  // superblocks left from this sub-chunk on (uniform)
+      const uint8_t* src = wtile + (size_t)(sb0 + SBC * c) * 144;
+      StaticFor<PPC>::run([&](auto t) {
+        constexpr int T = decltype(t)::value;
+        const bool ok = piece_ok[T] && ppc[T] < sbc * 9;
+        wreg[(c & 1) * PPC + T] = *reinterpret_cast<const u32x4*>(ok ? src + goff[T] : wtile);
+      });
+    };
+    issue(std::integral_constant<int, 0>{});
+    issue(std::integral_constant<int, 1>{});
+
+    // ---- 3. activations -> f16 in LDS (+ per-sub-block sums)
+    if (sb0 > 0) lds_barrier();
+    float xscale = 1.0f, inv = 1.0f;  // true x = xscale * stored f16 x
+    if constexpr (DT == KQ_BF16) {
+      float amax = 0.f;
+      StaticFor<XG>::run([&](auto t) {
+        const u32x4 v = xreg[decltype(t)::value];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] << 16)));
+          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] & 0xffff0000u)));
         }
       });
-    }
-
-    // ---- stage activations: thread handles 8 consecutive k of one row per step
-    if (sb0 > 0) __syncthreads();
-    const int ngroups = (kc >> 3) * MB;  // 8-element groups in the chunk
-    float amax = 0.f;
-    if constexpr (DT == KQ_BF16) {
-      for (int gi = tid; gi < ngroups; gi += SK_THREADS) {
-        const int m = gi / (kc >> 3), kk = (gi % (kc >> 3)) << 3;
-        if (m < M) {
-          const uint4 v = *reinterpret_cast<const uint4*>(x16 + (size_t)m * K + k0 + kk);
-          const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-          for (int t = 0; t < 4; t++) {
-            amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, u[t] << 16)));
-            amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, u[t] & 0xffff0000u)));
-          }
-        }
-      }
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
       if (lane == 0) scratch[wave] = amax;
-      __syncthreads();
+      lds_barrier();
       amax = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
-    }
-    float xscale = 1.0f, inv = 1.0f;  // true x = xscale * stored f16 x
-    if constexpr (DT == KQ_BF16) {
       // bring the largest magnitude into [2^14, 2^15): exact power-of-two scaling
       const uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff;
       if (eb != 0 && eb != 0xff) {
@@ -241,73 +285,71 @@ __global__ __launch_bounds__(SK_THREADS, 2) void q4k_skinny_kernel(const void* _
         inv = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
       }
     }
-    for (int gi = tid; gi < ngroups; gi += SK_THREADS) {
-      const int m = gi / (kc >> 3), kk = (gi % (kc >> 3)) << 3;
-      float f[8];
-      if (m < M) {
-        const uint4 v = *reinterpret_cast<const uint4*>(x16 + (size_t)m * K + k0 + kk);
-        const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+    StaticFor<XG>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      constexpr int m = T / XK;
+      const int kgi = tid + (T % XK) * SK_THREADS;
+      if (kgi < gpr) {
+        const int kk = kgi << 3;
+        const u32x4 v = xreg[T];
+        _Float16 h[8];
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
+        for (int e = 0; e < 4; e++) {
           if constexpr (DT == KQ_BF16) {
-            f[2 * t] = __builtin_bit_cast(float, u[t] << 16) * inv;
-            f[2 * t + 1] = __builtin_bit_cast(float, u[t] & 0xffff0000u) * inv;
+            h[2 * e] = (_Float16)(__builtin_bit_cast(float, v[e] << 16) * inv);
+            h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, v[e] & 0xffff0000u) * inv);
           } else {
-            f[2 * t] = kq::h2f((uint16_t)(u[t] & 0xffff));
-            f[2 * t + 1] = kq::h2f((uint16_t)(u[t] >> 16));
+            h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] & 0xffff));
+            h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
           }
         }
-      } else {
+        // MFMA fragment order inside an 8-group: k0 k2 k1 k3 k4 k6 k5 k7
+        const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+        *reinterpret_cast<f16x8*>(xs + (size_t)m * kchunk + kk) = v8;
+        float sum = 0.f;
 #pragma unroll
-        for (int t = 0; t < 8; t++) f[t] = 0.f;
+        for (int e = 0; e < 8; e++) sum += (float)h[e];
+        sum += __shfl_xor(sum, 1);  // 4 threads cover one 32-wide sub-block
+        sum += __shfl_xor(sum, 2);
+        if ((tid & 3) == 0) xsum[(kk >> 5) * MB + m] = sum;
       }
-      _Float16 h[8];
-#pragma unroll
-      for (int t = 0; t < 8; t++) h[t] = (_Float16)f[t];
-      // MFMA fragment order inside an 8-group: k0 k2 k1 k3 k4 k6 k5 k7
-      const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
-      *reinterpret_cast<f16x8*>(xs + (size_t)m * kchunk + kk) = v8;
-      float s = 0.f;
-#pragma unroll
-      for (int t = 0; t < 8; t++) s += (float)h[t];
-      s += __shfl_xor(s, 1);  // 4 threads cover one 32-wide sub-block
-      s += __shfl_xor(s, 2);
-      if ((tid & 3) == 0) xsum[(kk >> 5) * MB + m] = s;
-    }
+    });
 
-    // ---- park the weights in LDS
-    {
-      int r = r_first, c = c_first;
-      StaticFor<MAXP>::run([&](auto t) {
-        if (r < nrows) *reinterpret_cast<u32x4*>(wt + r * wstride + 16 * c) = wreg[decltype(t)::value];
-        r += step_r;
-        c += step_c;
-        if (c >= cpr) {
-          c -= cpr;
-          r++;
-        }
-      });
-    }
-    __syncthreads();
-
-    // ---- this wave's superblocks of the chunk
+    // ---- 4. sub-chunk by sub-chunk: park the arrived bytes in LDS, then one superblock per wave
+    // while the later sub-chunks are still streaming in
     const _Float16* xs_lane = xs + (size_t)(n_in & (MB - 1)) * kchunk + 16 * kg;
     const float* xsum_lane = xsum + (MB == 8 ? 4 * kg : 0);
     const uint8_t* wt_lane = wt + crow * wstride;
-    for (int s = wave; s < sbn; s += SK_WAVES) {
-      Q4kRaw raw;
-      const uint4* p = reinterpret_cast<const uint4*>(wt_lane + s * 144);
-      raw.hdr = p[0];
+    StaticFor<NCH>::run([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      const int sbc = sbn - SBC * c;
+      if (sbc > 0) {
+        StaticFor<PPC>::run([&](auto t) {
+          constexpr int T = decltype(t)::value;
+          const bool ok = piece_ok[T] && ppc[T] < sbc * 9;
+          *reinterpret_cast<u32x4*>(ok ? wt + SBC * c * 144 + loff[T] : dump) = wreg[(c & 1) * PPC + T];
+        });
+      }
+      if constexpr (c + 2 < NCH) issue(std::integral_constant<int, c + 2>{});
+      if (sbc > 0) {
+        lds_barrier();
+        const int sb = SBC * c + wave;
+        if (sb < sbn) {
+          Q4kRaw raw;
+          const uint4* p = reinterpret_cast<const uint4*>(wt_lane + sb * 144);
+          raw.hdr = p[0];
 #pragma unroll
-      for (int g = 0; g < 4; g++) raw.q[g] = p[1 + 2 * g + kg];
-      q4k_superblock<R, MB>(raw, xscale, xs_lane + 256 * s, xsum_lane + 8 * MB * s, acc);
-    }
+          for (int g = 0; g < 4; g++) raw.q[g] = p[1 + 2 * g + kg];
+          q4k_superblock<R, MB>(raw, xscale, xs_lane + 256 * sb, xsum_lane + 8 * MB * sb, acc);
+        }
+      }
+    });
   }
 
   // ---- cross-wave reduction and store
 #pragma unroll
   for (int r = 0; r < R; r++) red[(wave * R + r) * 64 + lane] = acc[r];
-  __syncthreads();
+  lds_barrier();
   for (int o = tid; o < R * 64; o += SK_THREADS) {
     const int r = o >> 6, l = o & 63;
     float v = 0.f;
@@ -334,7 +376,7 @@ int launch_q4k_skinny(const void* x, const uint8_t* w, void* y, int M, int N, in
   if (kch > 16) kch = 16;            // 18 pieces per thread at most (32 rows x 16 superblocks)
   if (kch * MB > 32) kch = 32 / MB;  // keep the f16 activations of a chunk within 16 KiB
   auto lds_bytes = [&](int kc) {
-    return (size_t)rows * (kc * 144 + 16) + (size_t)MB * kc * 512 + (size_t)kc * 8 * MB * 4 + SK_WAVES * R * 64 * 4 + 64;
+    return (size_t)rows * (kc * 144 + 16) + (size_t)MB * kc * 512 + (size_t)kc * 8 * MB * 4 + SK_WAVES * R * 64 * 4 + 64 + 16 * SK_THREADS;
   };
   while (kch > 1 && lds_bytes(kch) > 76 * 1024) kch >>= 1;  // two workgroups per CU must fit in 160 KiB
   const size_t lds = lds_bytes(kch);
