@@ -19,8 +19,8 @@ SOURCES = [
     ("kq_api.cpp", ["-x", "hip"]),
     ("kq_encode.cpp", ["-x", "hip"]),
     ("kq_generic.hip", ["-ffp-contract=off"]),
-    # MFMA results are consumed by VALU code right away: keep them in VGPRs, not AGPRs
     ("kq_mfma.hip", []),
+    ("kq_gemm.hip", []),
 ]
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",

@@ -108,13 +108,13 @@ int kq_dequantize(const void* w_dev, void* out_dev, uint64_t num_weights, int co
 }
 
 size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int dtype) {
-  (void)M; (void)N; (void)K; (void)transpose; (void)codec; (void)dtype;
+  (void)dtype;
+  if (transpose && codec_ok(codec) && kq_gemm_supported(M, N, K, codec)) return kq_gemm_workspace_bytes(M, K);
   return 0;
 }
 
 int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int transpose, int codec,
            int dtype, void* workspace_dev, size_t workspace_bytes, void* stream) {
-  (void)workspace_dev; (void)workspace_bytes;
   if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: unknown codec id %d", codec);
   if (!half_dtype(dtype))
     return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: activations must be float16 or bfloat16");
@@ -129,6 +129,14 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (!transpose)
     return kq_launch_gemm_nt_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+  if (kq_gemm_supported(M, N, K, codec)) {
+    const size_t need = kq_gemm_workspace_bytes(M, K);
+    if (!workspace_dev || workspace_bytes < need)
+      return kq_set_error(KQ_ERR_WORKSPACE, "quantized_matmul: workspace of %zu bytes required (got %zu)", need,
+                          workspace_bytes);
+    int rcg = kq_launch_gemm(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev, s);
+    if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
+  }
   int rc = kq_launch_qmm_tuned(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
   if (rc != KQ_ERR_UNSUPPORTED) return rc;
   return kq_launch_gemv_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);

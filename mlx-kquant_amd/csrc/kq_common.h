@@ -64,3 +64,8 @@ int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2,
 // covers the request, so the caller can fall through to the generic kernels.
 int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
                         hipStream_t s);
+// Prefill GEMM (q4_k / q5_k, M > 8): needs kq_gemm_workspace_bytes(M, K) bytes of device workspace.
+size_t kq_gemm_workspace_bytes(int M, int K);
+bool kq_gemm_supported(int M, int N, int K, int codec);
+int kq_launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                   hipStream_t s);

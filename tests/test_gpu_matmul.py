@@ -87,3 +87,32 @@ def test_qmm_reference_fixtures(kq, codec):
         got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
         want = O.qmm(xb, wire, codec, True, "float16")
         assert rel_l2(dev_to_bits(got), want, "float16") <= TOL
+
+
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k"])
+@pytest.mark.parametrize("M,N,K", [(9, 40, 256), (200, 200, 512), (130, 384, 2304), (512, 256, 4096)])
+def test_qmm_prefill_gemm(kq, codec, M, N, K):
+    """Prefill GEMM path (M > 8): ragged M and N tiles, several superblocks, both activation dtypes."""
+    wire = _wire(codec, N, K, seed=35)
+    for dtype in ("bfloat16", "float16"):
+        xb, xt = make_x((M, K), dtype, seed=M + K)
+        got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+        want = O.qmm(xb, wire, codec, True, dtype)
+        assert tuple(got.shape) == (M, N)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, N, K, dtype)
+
+
+def test_qmm_prefill_gemm_wide_dynamic_range(kq):
+    """bf16 activations spanning many binades and rows of very different scale: the per-row power-of-two
+    scaling of the f16 conversion must keep every row within tolerance."""
+    M, N, K = 64, 128, 1024
+    wire = _wire("q4_k", N, K, seed=36)
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((M, K)).astype(np.float32) * np.exp2(rng.integers(-12, 12, (M, K))).astype(np.float32)
+    x *= np.exp2(np.linspace(-60, 60, M)).astype(np.float32)[:, None]
+    xb = O.f32_to_bits(x, "bfloat16")
+    got = dev_to_bits(kq.quantized_matmul(bits_to_dev(xb, "bfloat16"), wire_to_dev(wire), None, "q4_k"))
+    want = O.qmm(xb, wire, "q4_k", True, "bfloat16")
+    g, w_ = O.bits_to_f32(got, "bfloat16").astype(np.float64), O.bits_to_f32(want, "bfloat16").astype(np.float64)
+    rel_rows = np.linalg.norm(g - w_, axis=1) / np.linalg.norm(w_, axis=1)
+    assert rel_rows.max() <= TOL, rel_rows.max()
