@@ -1,16 +1,17 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-weight hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--full]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-sweep] [--no-cpu]
 
 Headline (the JSON line): q4_k GEMV at M=1 on the Llama-3-8B gate/up projection
-(4096 -> 14336, bf16 activations), measured COLD: every step reads a different copy of the wire
-matrix, the copies together exceeding twice the 256 MB last-level cache, so the weight bytes come
-from HBM.  value = quantized weight bytes per step / step time.
+(4096 -> 14336, bf16 activations, weights = seeded N(0, 0.02) quantized by kq.quantize),
+measured COLD: every step reads a different copy of the wire matrix, the copies together
+exceeding twice the 256 MB last-level cache, so the weight bytes come from HBM.
+value = quantized weight bytes per step / step time (HIP events on the launching stream).
 
-Extra fields: `sweep` (the other decode projections and M in {1,2,4,8}, hot and cold), `prefill`
-(q4_k/q5_k GEMM TFLOP/s), `roofline` for the dominant kernel and `cpu_baseline` (the CPU oracle
-timed on this box's host cores on the same workload).
+Extra fields: `sweep` (the other decode projections of the q4_k_m recipe at M in {1,2,4,8}),
+`prefill` (q4_k / q5_k GEMM 8192 -> 28672 at M in {512, 2048}), `roofline` for the dominant kernel
+and `cpu_baseline` (the CPU oracle timed on this box's host cores on the headline GEMV).
 """
 import argparse
 import json
@@ -23,7 +24,7 @@ sys.path.insert(0, os.path.join(ROOT, "mlx-kquant_amd"))
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
-MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
 LLC_BYTES = 256 << 20
 
 
@@ -43,16 +44,23 @@ def synth_wire_torch(codec, rows, K, seed, device):
         wire[:, 0] = torch.randint(121, 130, (nb,), dtype=torch.uint8, device=device, generator=g)
     elif codec == "nvfp4":
         wire[:, 0:4] = torch.randint(0x08, 0x19, (nb, 4), dtype=torch.uint8, device=device, generator=g)
-    elif codec == "iq1_m":
-        pass
-    else:
+    elif codec != "iq1_m":
         for i, o in enumerate(off):
             wire[:, o:o + 2] = d[:, 2 * i:2 * i + 2]
     return wire.reshape(rows, K // wpb * bpb)
 
 
-def time_gemv(kq, torch, x, copies, codec, steps, warmup):
-    """Average per-launch time (ms) over `steps` launches rotating over `copies`."""
+def quantized_weights(kq, torch, codec, N, K, seed, device):
+    """Seeded N(0, 0.02) f32 weights [N, K] encoded by kq.quantize (host encoder), placed on the GPU."""
+    g = torch.Generator()
+    g.manual_seed(seed)
+    w = torch.randn((N, K), generator=g, dtype=torch.float32) * 0.02
+    wq, _ = kq.quantize(w, codec)
+    return wq.to(device)
+
+
+def time_matmul(kq, torch, x, copies, codec, steps, warmup):
+    """Average per-launch time (ms) over `steps` launches rotating over `copies` (events + wall)."""
     n = len(copies)
     for i in range(warmup):
         kq.quantized_matmul(x, copies[i % n], None, codec)
@@ -68,24 +76,26 @@ def time_gemv(kq, torch, x, copies, codec, steps, warmup):
     return ev0.elapsed_time(ev1) / steps, wall_ms / steps
 
 
-def cpu_baseline(codec, N, K, M, budget_s=12.0):
+def cold_copies(torch, base, wbytes):
+    ncopies = max(2, (2 * LLC_BYTES + wbytes - 1) // wbytes + 1)
+    return [base] + [base.clone() for _ in range(ncopies - 1)]
+
+
+def cpu_baseline(wire_np, codec, K, M, budget_s=12.0):
     """The CPU oracle (a port of the reference's threaded scalar eval_cpu path) on the same GEMV."""
     import numpy as np
     import oracle_lib as O
-    wpb, bpb = O.geometry(codec)
-    wire = O.synth_wire(codec, N * (K // wpb), seed=1).reshape(N, K // wpb * bpb)
     x = O.f32_to_bits(np.random.default_rng(2).standard_normal((M, K)).astype(np.float32), "bfloat16")
-    O.qmm(x, wire, codec, True, "bfloat16")
+    O.qmm(x, wire_np, codec, True, "bfloat16")
     times = []
     t_end = time.perf_counter() + budget_s
-    while time.perf_counter() < t_end or len(times) < 3:
+    while (time.perf_counter() < t_end or len(times) < 3) and len(times) < 200:
         t0 = time.perf_counter()
-        O.qmm(x, wire, codec, True, "bfloat16")
+        O.qmm(x, wire_np, codec, True, "bfloat16")
         times.append(time.perf_counter() - t0)
-        if len(times) >= 200:
-            break
     med = sorted(times)[len(times) // 2]
-    return {"value": round(wire.size / med / 1e9, 3), "unit": "GB/s", "cores": int(O.lib.kq_oracle_threads()),
+    N = wire_np.shape[0]
+    return {"value": round(wire_np.size / med / 1e9, 3), "unit": "GB/s", "cores": int(O.lib.kq_oracle_threads()),
             "kind": "port",
             "sample": f"{codec} GEMV M={M} {K}->{N}, full matrix, median of {len(times)} runs "
                       f"({med * 1e3:.2f} ms each), bf16 activations"}
@@ -96,7 +106,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--full", action="store_true", help="also run the decode sweep and the prefill GEMM")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the decode sweep and the prefill GEMM")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -109,23 +119,26 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+
+    # ---------------- headline: q4_k gate/up GEMV, M = 1, cold
     codec, N, K, M = "q4_k", 14336, 4096, 1
     wbytes = N * kq.bytes_per_row(codec, K)
-    ncopies = (2 * LLC_BYTES + wbytes - 1) // wbytes + 1
-    base = synth_wire_torch(codec, N, K, seed=1, device=dev)
-    copies = [base] + [base.clone() for _ in range(ncopies - 1)]
-    x = torch.randn((M, K), device=dev, dtype=torch.float32).to(torch.bfloat16)
-
-    ms, wall_ms = time_gemv(kq, torch, x, copies, codec, args.steps, args.warmup)
+    base = quantized_weights(kq, torch, codec, N, K, seed=2, device=dev)
+    copies = cold_copies(torch, base, wbytes)
+    gx = torch.Generator(device=dev)
+    gx.manual_seed(100)
+    x = torch.randn((M, K), device=dev, dtype=torch.float32, generator=gx).to(torch.bfloat16)
+    ms, wall_ms = time_matmul(kq, torch, x, copies, codec, args.steps, args.warmup)
     gbs = wbytes / (ms * 1e-3) / 1e9
-    hot_ms, _ = time_gemv(kq, torch, x, copies[:1], codec, args.steps, args.warmup)
+    hot_ms, _ = time_matmul(kq, torch, x, copies[:1], codec, args.steps, args.warmup)
 
     out = {
         "metric": "q4_k GEMV weight-GB/s at M=1 (cold)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic: seeded N(0,0.02) weights quantized by kq.quantize, N(0,1) bf16 activations",
         "config": {"workload": "decode GEMV, Llama-3-8B gate/up projection 4096->14336, q4_k, M=1, bf16 x, "
-                               f"cold over {ncopies} weight copies ({ncopies * wbytes >> 20} MiB)",
+                               f"cold over {len(copies)} weight copies ({len(copies) * wbytes >> 20} MiB)",
                    "codec": codec, "M": M, "N": N, "K": K},
         "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
         "hot_gbs": round(wbytes / (hot_ms * 1e-3) / 1e9, 1),
@@ -133,8 +146,44 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
     }
+    base_np = base.cpu().numpy() if not args.no_cpu else None
+    del copies
+
+    if not args.no_sweep:
+        sweep = []
+        steps, warm = max(50, args.steps // 10), max(10, args.warmup // 10)
+        shapes = [("q_proj", "q4_k", 4096, 4096, True), ("gate/up", "q4_k", 14336, 4096, True),
+                  ("down", "q6_k", 4096, 14336, True), ("lm_head", "q6_k", 128256, 4096, False)]
+        for name, c, n, k, encode in shapes:
+            wb = n * kq.bytes_per_row(c, k)
+            # the 525M-weight lm_head is filled with structurally valid random wire (encoding it on
+            # the host would dominate the run); the others are encoded from N(0, 0.02)
+            wq = base if name == "gate/up" else (quantized_weights(kq, torch, c, n, k, 3, dev) if encode
+                                                 else synth_wire_torch(c, n, k, 3, dev))
+            cps = cold_copies(torch, wq, wb)
+            for m in (1, 2, 4, 8):
+                xm = torch.randn((m, k), device=dev, dtype=torch.float32, generator=gx).to(torch.bfloat16)
+                t, _ = time_matmul(kq, torch, xm, cps, c, steps, warm)
+                sweep.append({"proj": name, "codec": c, "N": n, "K": k, "M": m, "us": round(t * 1e3, 2),
+                              "cold_gbs": round(wb / (t * 1e-3) / 1e9, 1),
+                              "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
+            del cps, wq
+        out["sweep"] = sweep
+        prefill = []
+        for c in ("q4_k", "q5_k"):
+            n, k = 28672, 8192
+            wq = quantized_weights(kq, torch, c, n, k, 5, dev)
+            for m in (512, 2048):
+                xm = torch.randn((m, k), device=dev, dtype=torch.float32, generator=gx).to(torch.bfloat16)
+                t, _ = time_matmul(kq, torch, xm, [wq], c, 20, 5)
+                tf = 2.0 * m * n * k / (t * 1e-3) / 1e12
+                prefill.append({"codec": c, "M": m, "N": n, "K": k, "ms": round(t, 4), "tflops": round(tf, 1),
+                                "pct_mfma_f16_peak": round(100 * tf / MFMA_F16_PEAK_TFLOPS, 2)})
+            del wq
+        out["prefill"] = prefill
+
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(codec, N, K, M)
+        out["cpu_baseline"] = cpu_baseline(base_np, codec, K, M)
     print(json.dumps(out))
 
 
