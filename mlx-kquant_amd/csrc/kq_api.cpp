@@ -163,6 +163,12 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
   if (B == 0 || M == 0 || N == 0) return KQ_OK;
   if (!x_dev || !w_dev || !out_dev || !lhs_idx_dev || !rhs_idx_dev)
     return kq_set_error(KQ_ERR_INVALID, "gather_qmm: null buffer");
+  {
+    const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
+                                           out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0, 0, 0.f,
+                                           codec, dtype, static_cast<hipStream_t>(stream));
+    if (rct != KQ_ERR_UNSUPPORTED) return rct;
+  }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
                                   nullptr, nullptr, out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0,
                                   0, 0.f, 0.f, codec, dtype, static_cast<hipStream_t>(stream));
@@ -202,6 +208,13 @@ int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_
   if (!x_dev || !gate_w_dev || !up_w_dev || !idx_dev || !out_dev)
     return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
   const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
+  if (!biased) {
+    const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(gate_w_dev),
+                                           static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, out_dev, T * R, 1, N,
+                                           K, R, K, estride, 1, act, limit, codec, dtype,
+                                           static_cast<hipStream_t>(stream));
+    if (rct != KQ_ERR_UNSUPPORTED) return rct;
+  }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(gate_w_dev),
                                   static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, gate_bias_dev, up_bias_dev,
                                   out_dev, T * R, 1, N, K, R, K, estride, 1, act, limit, alpha, codec, dtype,
@@ -218,6 +231,12 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
   if (T == 0 || R == 0 || N == 0) return KQ_OK;
   if (!x_dev || !w_dev || !idx_dev || !out_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
   const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
+  if (!bias_dev) {
+    const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, out_dev,
+                                           T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype,
+                                           static_cast<hipStream_t>(stream));
+    if (rct != KQ_ERR_UNSUPPORTED) return rct;
+  }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, bias_dev,
                                   nullptr, out_dev, T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype,
                                   static_cast<hipStream_t>(stream));

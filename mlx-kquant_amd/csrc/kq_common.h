@@ -64,6 +64,12 @@ int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2,
 // covers the request, so the caller can fall through to the generic kernels.
 int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
                         hipStream_t s);
+// Tuned gathered GEMV (items = (activation matrix, expert) pairs, M <= 8 rows each; with glu the
+// gate/up pair and the fused epilogue, M = 1): same fall-through contract as kq_launch_qmm_tuned.
+int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
+                           const uint32_t* rhs, void* out, int B, int M, int N, int K, int x_div,
+                           int64_t x_batch_stride, int64_t w_expert_stride, int glu, int act, float limit, int codec,
+                           int dtype, hipStream_t s);
 // Prefill GEMM (q4_k / q5_k, M > 8): needs kq_gemm_workspace_bytes(M, K) bytes of device workspace.
 size_t kq_gemm_workspace_bytes(int M, int K);
 bool kq_gemm_supported(int M, int N, int K, int codec);

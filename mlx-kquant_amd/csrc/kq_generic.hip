@@ -7,6 +7,7 @@
 #include <type_traits>
 
 #include "kq_decode.h"
+#include "kq_epilogue.h"
 
 namespace {
 
@@ -137,26 +138,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemm_nt_generic_kernel(const void*
 // One wave per (item p, output row n).  Item p reads activation matrix x[lhs[p]] (or p / x_div
 // when lhs is null) and expert rhs[p]; with GLU it also reads the `up` stack and applies the
 // fused epilogue (metal/mlx/backend/metal/kernels/kq_moe_glu_kq.h:34-60 of the reference).
-__device__ __forceinline__ float glu_epilogue(int act, float g, float u, float limit, float alpha) {
-  if (act == KQ_ACT_GELU) {
-    const float g3 = 0.044715f * g * g * g;
-    const float t = tanhf(0.7978845608028654f * (g + g3));
-    return (0.5f * g * (1.0f + t)) * u;
-  }
-  if (act == KQ_ACT_SWIGLU_CLAMP) {
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-    const float sig = 1.0f / (1.0f + expf(-alpha * g));
-    return (g * sig) * (u + 1.0f);
-  }
-  if (act == KQ_ACT_SILU_LIMIT) {
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-  }
-  const float sig = 1.0f / (1.0f + expf(-g));
-  return (g * sig) * u;
-}
-
 struct GatherArgs {
   const void* x;
   const uint8_t* w;
@@ -215,7 +196,7 @@ __global__ __launch_bounds__(GV_THREADS) void gather_generic_kernel(GatherArgs a
         if (a.bias) v += a.bias[(size_t)e * a.N + n];
         if constexpr (GLU) {
           if (a.bias2) v2 += a.bias2[(size_t)e * a.N + n];
-          v = glu_epilogue(a.act, v, v2, a.limit, a.alpha);
+          v = kq::glu_epilogue(a.act, v, v2, a.limit, a.alpha);
         }
         store_y<DT>(a.out, ((size_t)p * a.M + (m0 + m)) * a.N + n, v);
       }

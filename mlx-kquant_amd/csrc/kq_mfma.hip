@@ -1,33 +1,48 @@
 // Tuned skinny-M (decode) kernels: y[M,N] = x[M,K] . W^T for M <= 8, weights streamed once from
-// HBM, all multiply-accumulates on the matrix cores.
+// HBM, all multiply-accumulates on the matrix cores.  Codecs: q4_k and q6_k.  The same kernel
+// serves the gathered ops (one grid row per (activation matrix, expert) item) and the fused
+// gate/up GLU op, where a tile holds rows [n0, n0 + h) of the gate matrix followed by the same
+// rows of the up matrix and the epilogue combines them.
 //
-// Mapping (q4_k).  One workgroup (4 waves) owns a tile of up to 32 weight rows; its waves split
-// K by superblock.  Inside a wave the weights are the B operand of v_mfma_f32_32x32x16_f16:
-// lane l serves weight row n = l % 32 and K-half kg = l / 32, and loads, per 144-byte superblock,
-// the 16-byte header (d, dmin, 6-bit scales/mins) plus four 16-byte chunks of the nibble array:
-// every HBM byte is fetched by aligned 128-bit loads straight into registers.  Nibbles become
-// exact f16 integers with one AND-OR each (0x6400 | q = 1024 + q; high nibbles stay in place and
-// read as 1024 + 16 q), so the MFMAs over one 32-weight sub-block return
+// Mapping.  One workgroup (4 waves) owns a tile of up to 32 weight rows; its waves split K by
+// superblock.  Inside a wave the weights are the B operand of v_mfma_f32_32x32x16_f16: lane l
+// serves weight row n = l % 32 and K-half kg = l / 32.  Activations are the A operand: the
+// workgroup converts x to f16 once (scaled by a power of two so bf16 inputs cannot overflow),
+// keeps it in LDS, and every wave reads fragments back with ds_read_b128.  M is padded to the 32
+// rows of the MFMA by letting the spare rows alias real ones; only the accumulator registers of
+// real rows are carried.
+//
+// q4_k.  Nibbles become exact f16 integers with one AND-OR each (0x6400 | q = 1024 + q; high
+// nibbles stay in place and read as 1024 + 16 q), so the MFMAs over one 32-weight sub-block return
 //     P = sum_k x_k (1024 + s q_k),  s in {1, 16}
 // and the sub-block contributes  (d sc / s) P - (1024 d sc / s + dmin m) X,  X = sum_k x_k,
-// applied in f32 on the accumulator registers.  Activations are the A operand: the workgroup
-// converts x to f16 once (scaled by a power of two so bf16 inputs cannot overflow), keeps it and
-// the per-sub-block sums X in LDS, and every wave reads fragments back with ds_read_b128.  M is
-// padded to the 32 rows of the MFMA by letting the spare rows alias real ones; only the
-// accumulator registers of real rows are carried.
+// applied in f32 on the accumulator registers.
+//
+// q6_k.  sc (q - 32) with sc the int8 scale of the weight's 16-group reaches 4096 and is not always
+// an f16 number, so a weight is fed to the matrix cores as two exact f16 terms, sc ql (the low
+// nibble, <= 1920) and 16 sc (qh - 2) (the two high bits, a multiple of 16 up to 4096): the nibble
+// is masked in place as 1024 + 16 ql, the high bits as 1024 + 256 qh, and one v_pk_fma_f16 each
+// removes the 1024 and applies sc.  Two MFMAs per 16 weights share the activation fragment; one
+// accumulator collects the superblock and is folded in with a single multiply by d.
 #include <type_traits>
 
 #include "kq_decode.h"
+#include "kq_epilogue.h"
 
 namespace {
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// 16-byte global load from a 2-byte-aligned address (q6_k blocks are 210 bytes long): the
+// hardware serves unaligned vector loads, the type only stops the compiler from assuming more
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
 
 constexpr int SK_WAVES = 4;
 constexpr int SK_THREADS = SK_WAVES * 64;
 constexpr int SK_MAXM = 8;
+constexpr int SK_MAXROWS = 32;
 
 // Compile-time loop: the body sees its index as a constant from the start, so register arrays
 // indexed by it are split into scalars (a '#pragma unroll' loop is unrolled too late for that
@@ -55,22 +70,44 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// (a & mask) | magic should be ONE v_and_or_b32.  VOP3 on gfx9 takes no literal operands, so
+// with constant mask/magic the compiler emits v_and + v_or; callers therefore pass mask and magic
+// through opaque registers (see kq_opaque_*).  No instruction is written in inline asm: the
+// hazard recognizer does not see inside asm statements, and VALU writes racing an in-flight MFMA
+// destination need its wait states.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) { return (a & mask) | magic; }
+__device__ __forceinline__ uint32_t kq_opaque_vgpr(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+__device__ __forceinline__ uint32_t kq_opaque_sgpr(uint32_t v) {
+  asm volatile("" : "+s"(v));
+  return v;
+}
+
+// Per-codec geometry of the weight stream.  A superblock travels as PP 16-byte pieces (q6_k: the
+// first 208 bytes; its trailing 2-byte d goes through a side channel) and is parked in LDS LBPB
+// bytes apart, so that every block starts 16-byte aligned there.
+template <int C>
+struct SkGeom;
+template <>
+struct SkGeom<KQ_Q4_K> {
+  static constexpr int BPB = 144, LBPB = 144, PP = 9;
+  static constexpr bool SIDE_D = false, XSUM = true;
+  typedef u32x4 piece_t;
+};
+template <>
+struct SkGeom<KQ_Q6_K> {
+  static constexpr int BPB = 210, LBPB = 208, PP = 13;
+  static constexpr bool SIDE_D = true, XSUM = false;
+  typedef u32x4_a2 piece_t;
+};
+
+// ------------------------------------------------------------------ q4_k superblock
 struct Q4kRaw {
   uint4 hdr;
   uint4 q[4];
 };
-
-__device__ __forceinline__ void q4k_load(const uint8_t* __restrict__ blk, int kg, Q4kRaw& r) {
-  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-  const u32x4* p = reinterpret_cast<const u32x4*>(blk);
-  auto ld = [](const u32x4* q) {
-    const u32x4 v = __builtin_nontemporal_load(q);  // streamed once: keep it out of the caches' way
-    return make_uint4(v.x, v.y, v.z, v.w);
-  };
-  r.hdr = ld(p);
-#pragma unroll
-  for (int g = 0; g < 4; g++) r.q[g] = ld(p + 1 + 2 * g + kg);
-}
 
 // per-lane scales of one superblock: mul[j] multiplies P_j, sub[j] multiplies X_j
 __device__ __forceinline__ void q4k_scales(const uint4& hdr, float xscale, float* mul, float* sub) {
@@ -92,21 +129,6 @@ __device__ __forceinline__ void q4k_scales(const uint4& hdr, float xscale, float
   }
 }
 
-// (a & mask) | magic should be ONE v_and_or_b32.  VOP3 on gfx9 takes no literal operands, so
-// with constant mask/magic the compiler emits v_and + v_or; callers therefore pass mask and magic
-// through opaque registers (see kq_opaque_*).  No instruction is written in inline asm: the
-// hazard recognizer does not see inside asm statements, and VALU writes racing an in-flight MFMA
-// destination need its wait states.
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) { return (a & mask) | magic; }
-__device__ __forceinline__ uint32_t kq_opaque_vgpr(uint32_t v) {
-  asm volatile("" : "+v"(v));
-  return v;
-}
-__device__ __forceinline__ uint32_t kq_opaque_sgpr(uint32_t v) {
-  asm volatile("" : "+s"(v));
-  return v;
-}
-
 __device__ __forceinline__ f16x8 q4k_frag(uint32_t wa, uint32_t wa8, uint32_t wb, uint32_t wb8, uint32_t mask,
                                           uint32_t magic) {
   uint4 v;
@@ -118,11 +140,17 @@ __device__ __forceinline__ f16x8 q4k_frag(uint32_t wa, uint32_t wa8, uint32_t wb
 }
 
 // One superblock of one 32-row tile: 16 MFMAs + the f32 fix-up on R accumulator registers.
-// xs_lane: this lane's A-fragment base (f16 index) for the superblock; xsum: X_j for the
-// superblock, [8][XS] floats with XS = row stride.
+// bl: this lane's row of the superblock in LDS; xs_lane: this lane's A-fragment base (f16
+// index) for the superblock; xsum: X_j for the superblock, [8][XS] floats.
 template <int R, int XS>
-__device__ __forceinline__ void q4k_superblock(const Q4kRaw& raw, float xscale, const _Float16* __restrict__ xs_lane,
+__device__ __forceinline__ void q4k_superblock(const uint8_t* __restrict__ bl, int kg, float xscale,
+                                               const _Float16* __restrict__ xs_lane,
                                                const float* __restrict__ xsum, float* acc) {
+  Q4kRaw raw;
+  const uint4* p4 = reinterpret_cast<const uint4*>(bl);
+  raw.hdr = p4[0];
+#pragma unroll
+  for (int g = 0; g < 4; g++) raw.q[g] = p4[1 + 2 * g + kg];
   float mul[8], sub[8];
   q4k_scales(raw.hdr, xscale, mul, sub);
   const uint32_t magic = kq_opaque_vgpr(0x64006400u);
@@ -151,81 +179,174 @@ __device__ __forceinline__ void q4k_superblock(const Q4kRaw& raw, float xscale, 
   }
 }
 
-// MB = M rounded up to a power of two (1, 2, 4, 8).  Rows of the 32-row A operand beyond MB alias
-// row (r % MB); their accumulator rows are never read.
-//
-// Weight traffic: a tile (rows_per_tile rows x KCH superblocks) is fetched with fully coalesced
-// 16-byte loads -- consecutive lanes read consecutive 16-byte pieces of a row, so every wave
-// load covers 1 KiB of contiguous HBM -- and parked in LDS with a 16-byte pad per row (row
-// stride = 16 mod 256 bytes keeps the row-per-lane ds_read_b128 of the MFMA operand fetch free
-// of bank conflicts).  A row-per-lane pattern straight from global memory runs 6x slower: each
-// wave load would touch 32 different cache lines for 32 bytes apiece.
-template <int DT, int MB>
-__global__ __launch_bounds__(SK_THREADS, 2) void q4k_skinny_kernel(const void* __restrict__ x,
-                                                                   const uint8_t* __restrict__ w,
-                                                                   void* __restrict__ y, int M, int N, int K,
-                                                                   int rows_per_tile, int kch) {
-  constexpr int R = MB < 4 ? MB : 4;  // accumulator registers carried per lane
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  // layout: wt [rows_per_tile][kch*144 + 16] | xs f16 [MB][kch*256] | xsum f32 [kch*8][MB] | red | scratch
-  const int chunk_bytes = kch * 144, wstride = chunk_bytes + 16, kchunk = kch * 256;
-  uint8_t* wt = smem;
-  _Float16* xs = reinterpret_cast<_Float16*>(smem + rows_per_tile * wstride);
-  float* xsum = reinterpret_cast<float*>(smem + rows_per_tile * wstride + (size_t)MB * kchunk * 2);
-  float* red = xsum + kch * 8 * MB;
-  float* scratch = red + SK_WAVES * R * 64;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n_in = lane & 31, kg = lane >> 5;
-  const int nsb = K >> 8;
-  const size_t row_bytes = (size_t)nsb * 144;
-  const int row0 = blockIdx.x * rows_per_tile;
-  const int nrows = (N - row0 < rows_per_tile) ? (N - row0) : rows_per_tile;
-  const uint8_t* wtile = w + (size_t)row0 * row_bytes;
-  const uint16_t* x16 = static_cast<const uint16_t*>(x);
-  // compute-phase row of this lane (clamped: spare lanes re-read row 0, their results are dropped)
-  const int crow = n_in < nrows ? n_in : 0;
-
-  float acc[R];
+// ------------------------------------------------------------------ q6_k superblock
+// LDS block: ql[128] | qh[64] | int8 scales[16]; d arrives separately.  Weight 128 hf + 32 t + l
+// (hf = half, t = 0..3, l = 0..31) has its low nibble in ql[64 hf + 32 (t & 1) + l] (high nibble of
+// the byte when t >= 2), its high bits in bits 2t, 2t+1 of qh[32 hf + l] and scale 8 hf + 2 t +
+// l / 16.  Lane (row, kg) takes l = 16 kg .. 16 kg + 15: one scale per lane and sub-block.
+template <int R>
+__device__ __forceinline__ void q6k_superblock(const uint8_t* __restrict__ bl, int kg, float dx,
+                                               const _Float16* __restrict__ xs_lane, float* acc) {
+  const uint32_t magic = kq_opaque_vgpr(0x64006400u);
+  const uint32_t mask_q = kq_opaque_sgpr(0x00f000f0u), mask_h = kq_opaque_sgpr(0x03000300u);
+  const uint4 scv = *reinterpret_cast<const uint4*>(bl + 192);
+  const uint32_t scw[4] = {scv.x, scv.y, scv.z, scv.w};
+  f32x16 p = {0};
 #pragma unroll
-  for (int r = 0; r < R; r++) acc[r] = 0.f;
+  for (int hf = 0; hf < 2; hf++) {
+    const uint4 hv = *reinterpret_cast<const uint4*>(bl + 128 + 32 * hf + 16 * kg);
+    const uint32_t hw[4] = {hv.x, hv.y, hv.z, hv.w};
+#pragma unroll
+    for (int qr = 0; qr < 2; qr++) {
+      const uint4 qv = *reinterpret_cast<const uint4*>(bl + 64 * hf + 32 * qr + 16 * kg);
+      const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int t = qr + 2 * h, j = 4 * hf + t;
+        const int sc = __builtin_amdgcn_sbfe((int)scw[2 * hf + (t >> 1)], 8 * (2 * (t & 1) + kg), 8);
+        const float scf = (float)sc;
+        const _Float16 sch = (_Float16)(scf * 0.0625f), ofl = (_Float16)(-64.0f * scf), ofh = (_Float16)(-96.0f * scf);
+        const f16x2 scp = {sch, sch}, oflp = {ofl, ofl}, ofhp = {ofh, ofh};
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          uint32_t fl[4], fh[4];
+#pragma unroll
+          for (int e = 0; e < 2; e++) {
+            const uint32_t q = qw[2 * s + e], hq = hw[2 * s + e];
+            const uint32_t qe = h ? q : (q << 4), qo = h ? (q >> 8) : (q >> 4);
+            const uint32_t he = hq << (8 - 2 * t), ho = t ? (hq >> (2 * t)) : hq;
+            fl[2 * e] = and_or(qe, mask_q, magic);  // bytes 0, 2 of the word: 1024 + 16 ql
+            fl[2 * e + 1] = and_or(qo, mask_q, magic);  // bytes 1, 3
+            fh[2 * e] = and_or(he, mask_h, magic);  // 1024 + 256 qh
+            fh[2 * e + 1] = and_or(ho, mask_h, magic);
+          }
+          f16x2 bl2[4], bh2[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            // (1024 + 16 ql) sc / 16 - 64 sc = sc ql;  (1024 + 256 qh) sc / 16 - 96 sc = 16 sc (qh - 2)
+            bl2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fl[e]), scp, oflp);
+            bh2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fh[e]), scp, ofhp);
+          }
+          const f16x8 blo = {bl2[0][0], bl2[0][1], bl2[1][0], bl2[1][1], bl2[2][0], bl2[2][1], bl2[3][0], bl2[3][1]};
+          const f16x8 bhi = {bh2[0][0], bh2[0][1], bh2[1][0], bh2[1][1], bh2[2][0], bh2[2][1], bh2[3][0], bh2[3][1]};
+          const f16x8 a = *reinterpret_cast<const f16x8*>(xs_lane + 32 * j + 8 * s);
+          p = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, blo, p, 0, 0, 0);
+          p = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bhi, p, 0, 0, 0);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; r++) acc[r] = fmaf(dx, p[r], acc[r]);
+}
 
-  constexpr int SBC = 4;  // superblocks per sub-chunk: one per wave
-  constexpr int NCH = 4;  // sub-chunks per chunk (kch <= 16), all in flight at once
-  constexpr int PPC = 5;  // 16-byte pieces per thread per sub-chunk: ceil(32 rows * 36 / 256)
+// ------------------------------------------------------------------ the kernel
+struct SkArgs {
+  const void* x;
+  const uint8_t* w;
+  const uint8_t* w2;    // up stack (GLU) or null
+  void* y;
+  const uint32_t* lhs;  // activation-matrix index per item, or null: item / x_div
+  const uint32_t* rhs;  // expert index per item, or null: expert 0
+  int M, N, K, rows_per_tile, kch, x_div, act;
+  int64_t x_batch_stride;   // elements between activation matrices
+  int64_t w_expert_stride;  // bytes between expert matrices
+  float limit;
+};
+
+// MB = M rounded up to a power of two (1, 2, 4, 8).  Rows of the 32-row A operand beyond MB alias
+// row (r % MB); their accumulator rows are never read.  Grid: x = row tile, y = item.
+//
+// Weight traffic: a tile (rows_per_tile rows x KCH superblocks) is fetched with coalesced
+// 16-byte loads -- consecutive lanes read consecutive 16-byte pieces of a row, so every wave
+// load covers about 1 KiB of contiguous HBM -- and parked in LDS with the row stride an odd
+// multiple of 16 bytes (keeps the row-per-lane ds_read_b128 of the MFMA operand fetch free of
+// bank conflicts).  A row-per-lane pattern straight from global memory runs 6x slower: each
+// wave load would touch 32 different cache lines for 32 bytes apiece.
+template <int C, int DT, int MB, bool GLU>
+__global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
+  using G = SkGeom<C>;
+  constexpr int R = MB < 4 ? MB : 4;  // accumulator registers carried per lane
+  constexpr int SBC = 4;              // superblocks per sub-chunk: one per wave
+  constexpr int NCH = 4;              // sub-chunks per chunk (kch <= 16)
+  constexpr int PPR = SBC * G::PP;    // 16-byte pieces per row and sub-chunk
+  constexpr int PPC = (SK_MAXROWS * PPR + SK_THREADS - 1) / SK_THREADS;  // pieces per thread and sub-chunk
   // activation staging slots per thread: slot t = (row t / XK, k-pass t % XK); a chunk holds at
   // most min(512, 1024 / MB) 8-element groups per row because kch * MB <= 32
   constexpr int XK = MB <= 2 ? 2 : 1;
   constexpr int XG = MB * XK;
 
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int M = a.M, N = a.N, K = a.K, rows_per_tile = a.rows_per_tile, kch = a.kch;
+  // layout: wt [rows_per_tile][wstride] | xs f16 [MB][kch*256] | xsum f32 [kch*8][MB] | red | scratch | dump | dq
+  const int wstride = kch * G::LBPB + (((kch * G::PP) & 1) ? 0 : 16), kchunk = kch * 256;
+  uint8_t* wt = smem;
+  _Float16* xs = reinterpret_cast<_Float16*>(smem + rows_per_tile * wstride);
+  float* xsum = reinterpret_cast<float*>(smem + rows_per_tile * wstride + (size_t)MB * kchunk * 2);
+  float* red = xsum + kch * 8 * MB;
+  float* scratch = red + SK_WAVES * R * 64;
+  uint8_t* dump = reinterpret_cast<uint8_t*>(scratch + 16) + 16 * threadIdx.x;  // per-thread 16-byte dump slot
+  uint16_t* dq = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(scratch + 16) + 16 * SK_THREADS);  // [32][16]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n_in = lane & 31, kg = lane >> 5;
+  const int nsb = K >> 8;
+  const size_t row_bytes = (size_t)nsb * G::BPB;
+  // GLU tiles hold `half` gate rows then `half` up rows; plain tiles rows_per_tile rows
+  const int half = GLU ? (rows_per_tile >> 1) : rows_per_tile;
+  const int row0 = blockIdx.x * half;
+  const int nrows = (N - row0 < half) ? (N - row0) : half;
+  const int item = blockIdx.y;
+  const size_t expert = a.rhs ? a.rhs[item] : 0;
+  const size_t xsel = a.lhs ? a.lhs[item] : (size_t)(item / a.x_div);
+  const uint8_t* wtile = a.w + expert * (size_t)a.w_expert_stride + (size_t)row0 * row_bytes;
+  const uint8_t* wtile2 = GLU ? a.w2 + expert * (size_t)a.w_expert_stride + (size_t)row0 * row_bytes : wtile;
+  const uint16_t* x16 = static_cast<const uint16_t*>(a.x) + xsel * (size_t)a.x_batch_stride;
+  // compute-phase row of this lane (spare lanes re-read tile row 0, their results are dropped)
+  const bool lane_live = GLU ? (n_in < 2 * half && (n_in < half ? n_in : n_in - half) < nrows) : n_in < nrows;
+  const int crow = lane_live ? n_in : 0;
+
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) acc[r] = 0.f;
+
   // piece map of the weight stream (see step 2): global / LDS byte offsets inside a sub-chunk
   uint32_t goff[PPC], loff[PPC];
   int ppc[PPC];
-  bool piece_ok[PPC];
+  bool piece_ok[PPC], piece_up[PPC];
   {
-    int r = tid / 36, pc = tid % 36;
+    int r = tid / PPR, pc = tid % PPR;
     StaticFor<PPC>::run([&](auto t) {
       constexpr int T = decltype(t)::value;
-      piece_ok[T] = r < nrows;
+      const bool up = GLU && r >= half;
+      const int srow = up ? r - half : r;
+      piece_ok[T] = srow < nrows && r < rows_per_tile;
+      piece_up[T] = up;
       ppc[T] = pc;
-      goff[T] = (uint32_t)r * (uint32_t)row_bytes + 16 * pc;
-      loff[T] = (uint32_t)r * (uint32_t)wstride + 16 * pc;
-      r += SK_THREADS / 36;
-      pc += SK_THREADS % 36;
-      if (pc >= 36) {
-        pc -= 36;
+      const int sbl = pc / G::PP, p = pc % G::PP;
+      goff[T] = (uint32_t)srow * (uint32_t)row_bytes + sbl * G::BPB + 16 * p;
+      loff[T] = (uint32_t)r * (uint32_t)wstride + sbl * G::LBPB + 16 * p;
+      r += SK_THREADS / PPR;
+      pc += SK_THREADS % PPR;
+      if (pc >= PPR) {
+        pc -= PPR;
         r++;
       }
     });
   }
-  uint8_t* dump = reinterpret_cast<uint8_t*>(scratch + 16) + 16 * tid;  // per-thread 16-byte dump slot
+  // side channel for the 2-byte d of q6_k: thread -> (row tid / 4, superblock tid % 4) of a sub-chunk
+  const int d_row = tid >> 2, d_sbl = tid & 3;
+  const bool d_up = GLU && d_row >= half;
+  const int d_srow = d_up ? d_row - half : d_row;
+  const bool d_ok = G::SIDE_D && d_row < rows_per_tile && d_srow < nrows;
+  const uint8_t* d_src = (d_up ? wtile2 : wtile) + (d_ok ? (size_t)d_srow * row_bytes : 0) + 208;
 
   for (int sb0 = 0; sb0 < nsb; sb0 += kch) {
     const int sbn = (nsb - sb0 < kch) ? (nsb - sb0) : kch;
     const int kc = sbn << 8, k0 = sb0 << 8;
 
     // ---- 1. activation loads first, so waiting for them does not wait for the weights
-    const int gpr = kc >> 3;         // 8-element groups per activation row in this chunk
+    const int gpr = kc >> 3;  // 8-element groups per activation row in this chunk
     u32x4 xreg[XG];
     // (loads are unconditional and branch-free -- out-of-range slots re-read valid data -- so the
     // compiler can count outstanding loads exactly and wait for the activations alone)
@@ -238,22 +359,28 @@ __global__ __launch_bounds__(SK_THREADS, 2) void q4k_skinny_kernel(const void* _
       xreg[T] = *reinterpret_cast<const u32x4*>(x16 + (size_t)m * K + k0 + 8 * kgi);
     });
 
-    // ---- 2. weight stream.  Sub-chunk c covers superblocks [4c, 4c+4) = 36 16-byte pieces per
-    // row; piece i = tid + 256 t maps to (row i / 36, piece i % 36), so consecutive lanes read
-    // consecutive 16-byte pieces of a row.  The map is the same for every sub-chunk (goff / loff
-    // below); pieces outside the tile or a ragged last sub-chunk re-read the tile's first bytes and
+    // ---- 2. weight stream.  Sub-chunk c covers superblocks [4c, 4c+4) = PPR 16-byte pieces per
+    // row; piece i = tid + 256 t maps to (row i / PPR, piece i % PPR), so consecutive lanes read
+    // consecutive 16-byte pieces of a row.  The map is the same for every sub-chunk (goff / loff);
+    // pieces outside the tile or a ragged last sub-chunk re-read the tile's first bytes and
     // land in a dump slot.  Two sub-chunks are in flight at any time (register sets c % 2); the
     // next one is issued as soon as its register set has been parked in LDS.
     u32x4 wreg[2 * PPC];
+    uint16_t dreg[2];
     auto issue = [&](auto cc) {
       constexpr int c = decltype(cc)::value;
       const int sbc = sbn - SBC * c;  // superblocks left from this sub-chunk on (uniform)
-      const uint8_t* src = wtile + (size_t)(sb0 + SBC * c) * 144;
+      const size_t sboff = (size_t)(sb0 + SBC * c) * G::BPB;
       StaticFor<PPC>::run([&](auto t) {
         constexpr int T = decltype(t)::value;
-        const bool ok = piece_ok[T] && ppc[T] < sbc * 9;
-        wreg[(c & 1) * PPC + T] = *reinterpret_cast<const u32x4*>(ok ? src + goff[T] : wtile);
+        const bool ok = piece_ok[T] && ppc[T] < sbc * G::PP;
+        const uint8_t* base = (GLU && piece_up[T]) ? wtile2 : wtile;
+        wreg[(c & 1) * PPC + T] = *reinterpret_cast<const typename G::piece_t*>(ok ? base + sboff + goff[T] : wtile);
       });
+      if constexpr (G::SIDE_D) {
+        const bool ok = d_ok && d_sbl < sbc;
+        dreg[c & 1] = *reinterpret_cast<const uint16_t*>(ok ? d_src + sboff + d_sbl * G::BPB : wtile);
+      }
     };
     issue(std::integral_constant<int, 0>{});
     issue(std::integral_constant<int, 1>{});
@@ -306,12 +433,14 @@ __global__ __launch_bounds__(SK_THREADS, 2) void q4k_skinny_kernel(const void* _
         // MFMA fragment order inside an 8-group: k0 k2 k1 k3 k4 k6 k5 k7
         const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
         *reinterpret_cast<f16x8*>(xs + (size_t)m * kchunk + kk) = v8;
-        float sum = 0.f;
+        if constexpr (G::XSUM) {
+          float sum = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; e++) sum += (float)h[e];
-        sum += __shfl_xor(sum, 1);  // 4 threads cover one 32-wide sub-block
-        sum += __shfl_xor(sum, 2);
-        if ((tid & 3) == 0) xsum[(kk >> 5) * MB + m] = sum;
+          for (int e = 0; e < 8; e++) sum += (float)h[e];
+          sum += __shfl_xor(sum, 1);  // 4 threads cover one 32-wide sub-block
+          sum += __shfl_xor(sum, 2);
+          if ((tid & 3) == 0) xsum[(kk >> 5) * MB + m] = sum;
+        }
       }
     });
 
@@ -326,21 +455,24 @@ __global__ __launch_bounds__(SK_THREADS, 2) void q4k_skinny_kernel(const void* _
       if (sbc > 0) {
         StaticFor<PPC>::run([&](auto t) {
           constexpr int T = decltype(t)::value;
-          const bool ok = piece_ok[T] && ppc[T] < sbc * 9;
-          *reinterpret_cast<u32x4*>(ok ? wt + SBC * c * 144 + loff[T] : dump) = wreg[(c & 1) * PPC + T];
+          const bool ok = piece_ok[T] && ppc[T] < sbc * G::PP;
+          *reinterpret_cast<u32x4*>(ok ? wt + SBC * c * G::LBPB + loff[T] : dump) = wreg[(c & 1) * PPC + T];
         });
+        if constexpr (G::SIDE_D) {
+          if (d_ok && d_sbl < sbc) dq[d_row * 16 + SBC * c + d_sbl] = dreg[c & 1];
+        }
       }
       if constexpr (c + 2 < NCH) issue(std::integral_constant<int, c + 2>{});
       if (sbc > 0) {
         lds_barrier();
         const int sb = SBC * c + wave;
         if (sb < sbn) {
-          Q4kRaw raw;
-          const uint4* p = reinterpret_cast<const uint4*>(wt_lane + sb * 144);
-          raw.hdr = p[0];
-#pragma unroll
-          for (int g = 0; g < 4; g++) raw.q[g] = p[1 + 2 * g + kg];
-          q4k_superblock<R, MB>(raw, xscale, xs_lane + 256 * sb, xsum_lane + 8 * MB * sb, acc);
+          if constexpr (C == KQ_Q4_K) {
+            q4k_superblock<R, MB>(wt_lane + sb * G::LBPB, kg, xscale, xs_lane + 256 * sb, xsum_lane + 8 * MB * sb, acc);
+          } else {
+            const float dx = kq::h2f(dq[crow * 16 + sb]) * xscale;
+            q6k_superblock<R>(wt_lane + sb * G::LBPB, kg, dx, xs_lane + 256 * sb, acc);
+          }
         }
       }
     });
@@ -352,60 +484,127 @@ __global__ __launch_bounds__(SK_THREADS, 2) void q4k_skinny_kernel(const void* _
   lds_barrier();
   for (int o = tid; o < R * 64; o += SK_THREADS) {
     const int r = o >> 6, l = o & 63;
+    const int m = 4 * (l >> 5) + r, n = l & 31;
+    if (m >= M || n >= nrows) continue;
     float v = 0.f;
 #pragma unroll
     for (int wv = 0; wv < SK_WAVES; wv++) v += red[(wv * R + r) * 64 + l];
-    const int m = 4 * (l >> 5) + r, n = l & 31;
-    if (m < M && n < nrows) {
-      uint16_t* yo = static_cast<uint16_t*>(y) + (size_t)m * N + row0 + n;
-      *yo = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+    if constexpr (GLU) {
+      float u = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < SK_WAVES; wv++) u += red[(wv * R + r) * 64 + l + half];
+      v = kq::glu_epilogue(a.act, v, u, a.limit, 1.0f);
     }
+    uint16_t* yo = static_cast<uint16_t*>(a.y) + ((size_t)item * M + m) * N + row0 + n;
+    *yo = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
   }
 }
 
-template <int DT, int MB>
-int launch_q4k_skinny(const void* x, const uint8_t* w, void* y, int M, int N, int K, hipStream_t s) {
-  constexpr int R = MB < 4 ? MB : 4;
-  // balanced row tiles: about two workgroups per CU, at most 32 rows each
-  int rows = (N + 511) / 512;
-  rows = (rows + 3) & ~3;
-  if (rows > 32) rows = 32;
+template <int C>
+size_t sk_lds_bytes(int rows, int kch, int MB) {
+  using G = SkGeom<C>;
+  const int R = MB < 4 ? MB : 4;
+  const size_t wstride = (size_t)kch * G::LBPB + (((kch * G::PP) & 1) ? 0 : 16);
+  return rows * wstride + (size_t)MB * kch * 512 + (size_t)kch * 8 * MB * 4 + SK_WAVES * R * 64 * 4 + 64 +
+         16 * SK_THREADS + 32 * 16 * 2;
+}
+
+template <int C, int DT, int MB, bool GLU>
+int launch_skinny(SkArgs a, int items, hipStream_t s) {
+  // balanced row tiles: about two workgroups per CU over the whole launch, at most 32 rows each
+  const int64_t total = (int64_t)a.N * items * (GLU ? 2 : 1);
+  int rows = (int)((total + 511) / 512);
+  rows = (rows + 7) & ~7;
+  if (rows > SK_MAXROWS) rows = SK_MAXROWS;
   if (rows < 8) rows = 8;
-  const int tiles = (N + rows - 1) / rows;
-  int kch = K >> 8;
-  if (kch > 16) kch = 16;            // 18 pieces per thread at most (32 rows x 16 superblocks)
+  const int half = GLU ? rows / 2 : rows;
+  const int tiles = (a.N + half - 1) / half;
+  int kch = a.K >> 8;
+  if (kch > 16) kch = 16;            // four sub-chunks of four superblocks
   if (kch * MB > 32) kch = 32 / MB;  // keep the f16 activations of a chunk within 16 KiB
-  auto lds_bytes = [&](int kc) {
-    return (size_t)rows * (kc * 144 + 16) + (size_t)MB * kc * 512 + (size_t)kc * 8 * MB * 4 + SK_WAVES * R * 64 * 4 + 64 + 16 * SK_THREADS;
-  };
-  while (kch > 1 && lds_bytes(kch) > 76 * 1024) kch >>= 1;  // two workgroups per CU must fit in 160 KiB
-  const size_t lds = lds_bytes(kch);
-  auto kern = q4k_skinny_kernel<DT, MB>;
+  while (kch > 1 && sk_lds_bytes<C>(rows, kch, MB) > 76 * 1024) kch >>= 1;  // two workgroups per CU must fit in 160 KiB
+  const size_t lds = sk_lds_bytes<C>(rows, kch, MB);
+  a.rows_per_tile = rows;
+  a.kch = kch;
+  auto kern = skinny_kernel<C, DT, MB, GLU>;
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
     KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      120 * 1024));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(SK_THREADS), lds, s, x, w, y, M, N, K, rows, kch);
+  hipLaunchKernelGGL(kern, dim3(tiles, items), dim3(SK_THREADS), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }
 
-template <int DT>
-int launch_q4k_skinny_m(const void* x, const uint8_t* w, void* y, int M, int N, int K, hipStream_t s) {
-  if (M == 1) return launch_q4k_skinny<DT, 1>(x, w, y, M, N, K, s);
-  if (M == 2) return launch_q4k_skinny<DT, 2>(x, w, y, M, N, K, s);
-  if (M <= 4) return launch_q4k_skinny<DT, 4>(x, w, y, M, N, K, s);
-  return launch_q4k_skinny<DT, 8>(x, w, y, M, N, K, s);
+template <int C, int DT, bool GLU>
+int launch_skinny_m(const SkArgs& a, int items, hipStream_t s) {
+  if (a.M == 1) return launch_skinny<C, DT, 1, GLU>(a, items, s);
+  if constexpr (GLU) {
+    return KQ_ERR_UNSUPPORTED;
+  } else {
+    if (a.M == 2) return launch_skinny<C, DT, 2, false>(a, items, s);
+    if (a.M <= 4) return launch_skinny<C, DT, 4, false>(a, items, s);
+    return launch_skinny<C, DT, 8, false>(a, items, s);
+  }
+}
+
+template <bool GLU>
+int launch_skinny_any(const SkArgs& a, int items, int codec, int dtype, hipStream_t s) {
+  if (codec == KQ_Q4_K)
+    return dtype == KQ_F16 ? launch_skinny_m<KQ_Q4_K, KQ_F16, GLU>(a, items, s)
+                           : launch_skinny_m<KQ_Q4_K, KQ_BF16, GLU>(a, items, s);
+  return dtype == KQ_F16 ? launch_skinny_m<KQ_Q6_K, KQ_F16, GLU>(a, items, s)
+                         : launch_skinny_m<KQ_Q6_K, KQ_BF16, GLU>(a, items, s);
+}
+
+bool sk_shape_ok(int M, int K, int codec, const void* x, const void* w, const void* w2) {
+  if ((codec != KQ_Q4_K && codec != KQ_Q6_K) || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return false;
+  // q4_k pieces are fetched with aligned 16-byte loads; q6_k blocks need 2-byte alignment only
+  const uintptr_t wmask = codec == KQ_Q4_K ? 15 : 1;
+  if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask)) return false;
+  return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 }
 
 }  // namespace
 
 int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
                         hipStream_t s) {
-  if (codec != KQ_Q4_K || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return KQ_ERR_UNSUPPORTED;
-  if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15)) return KQ_ERR_UNSUPPORTED;
-  if (dtype == KQ_F16) return launch_q4k_skinny_m<KQ_F16>(x, w, y, M, N, K, s);
-  return launch_q4k_skinny_m<KQ_BF16>(x, w, y, M, N, K, s);
+  if (!sk_shape_ok(M, K, codec, x, w, nullptr)) return KQ_ERR_UNSUPPORTED;
+  SkArgs a{};
+  a.x = x;
+  a.w = w;
+  a.y = y;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.x_div = 1;
+  return launch_skinny_any<false>(a, 1, codec, dtype, s);
+}
+
+int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
+                           const uint32_t* rhs, void* out, int B, int M, int N, int K, int x_div,
+                           int64_t x_batch_stride, int64_t w_expert_stride, int glu, int act, float limit, int codec,
+                           int dtype, hipStream_t s) {
+  if (!sk_shape_ok(M, K, codec, x, w, w2) || B < 1 || B > 65535) return KQ_ERR_UNSUPPORTED;
+  if (glu && (M != 1 || act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
+  const int64_t wmask = codec == KQ_Q4_K ? 15 : 1;
+  if ((w_expert_stride & wmask) || ((x_batch_stride * 2) & 15)) return KQ_ERR_UNSUPPORTED;
+  SkArgs a{};
+  a.x = x;
+  a.w = w;
+  a.w2 = w2;
+  a.y = out;
+  a.lhs = lhs;
+  a.rhs = rhs;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.x_div = x_div < 1 ? 1 : x_div;
+  a.act = act;
+  a.x_batch_stride = x_batch_stride;
+  a.w_expert_stride = w_expert_stride;
+  a.limit = limit;
+  return glu ? launch_skinny_any<true>(a, B, codec, dtype, s) : launch_skinny_any<false>(a, B, codec, dtype, s);
 }

@@ -46,6 +46,32 @@ def test_qmm_decode_and_prefill_shapes(kq, codec, M):
     assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, M)
 
 
+@pytest.mark.parametrize("codec", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 768), (3, 20000, 256), (8, 520, 4352), (2, 40, 8192), (5, 4100, 1024),
+                                   (1, 33, 2048)])
+def test_qmm_skinny_ragged_shapes(kq, codec, M, N, K):
+    """Row tiles that do not divide N, K of 1 / 3 / 17 superblocks (partial sub-chunks, two chunks)."""
+    wire = _wire(codec, N, K, seed=34)
+    for dtype in ("bfloat16", "float16"):
+        xb, xt = make_x((M, K), dtype, seed=200 + M)
+        got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+        want = O.qmm(xb, wire, codec, True, dtype)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, N, K, dtype)
+
+
+def test_qmm_skinny_unaligned_q6k_rows(kq):
+    """q6_k rows are 210-byte multiples: a wire view that starts 2 bytes into an allocation still decodes."""
+    N, K, M = 64, 768, 1
+    wire = _wire("q6_k", N, K, seed=35)
+    buf = torch.zeros(wire.size + 16, dtype=torch.uint8, device="cuda:0")
+    view = buf[2:2 + wire.size].view(N, -1)
+    view.copy_(wire_to_dev(wire))
+    xb, xt = make_x((M, K), "bfloat16", seed=36)
+    got = kq.quantized_matmul(xt, view, None, "q6_k")
+    want = O.qmm(xb, wire, "q6_k", True, "bfloat16")
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
+
+
 @pytest.mark.parametrize("codec", ["q4_k", "q8_0", "iq4_nl"])
 def test_qmm_no_transpose(kq, codec):
     K, N, M = 64, 512, 5  # W decodes to [K, N]

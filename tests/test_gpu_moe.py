@@ -103,6 +103,26 @@ def test_moe_glu_activations(kq, act, limit):
     assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
 
 
+@pytest.mark.parametrize("codec", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("E,N,K,T,R", [(6, 136, 768, 1, 4), (8, 2048, 512, 4, 2), (3, 72, 4352, 5, 3), (128, 64, 256, 1, 8)])
+def test_moe_tuned_gathered_shapes(kq, codec, E, N, K, T, R):
+    """The MFMA gathered kernels: gate/up tiles that do not divide N, 1 / 3 / 17 superblocks, many experts."""
+    gate = _stack(codec, E, N, K, seed=71)
+    up = _stack(codec, E, N, K, seed=72)
+    rng = np.random.default_rng(73)
+    idx = np.stack([rng.permutation(E)[:R] for _ in range(T)]) if R <= E else rng.integers(0, E, (T, R))
+    for dtype, act, limit in (("bfloat16", "silu", 0.0), ("float16", "gelu", 0.0), ("bfloat16", "silu_limit", 0.4)):
+        xb, xt = make_x((T, K), dtype, seed=74, scale=0.02)
+        got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act=act, limit=limit)
+        want = _glu_truth(codec, xb, gate, up, idx, act, limit, dtype=dtype)
+        assert tuple(got.shape) == (T, R, N)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype, act)
+    hb, ht = make_x((T, R, K), "bfloat16", seed=75, scale=0.02)
+    got = kq.gather_qmv_kq(ht, wire_to_dev(gate), codec, _idx_dev(idx))
+    want = O.gather_qmv(hb, gate, codec, idx, None, "bfloat16")
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, codec
+
+
 @pytest.mark.parametrize("codec", ["mxfp4", "nvfp4"])
 def test_moe_swiglu_clamp_bias(kq, codec):
     E, N, K, T, R = 4, 64, 576, 4, 2
