@@ -93,6 +93,12 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
                   int64_t x_batch_stride, int64_t w_expert_stride_bytes, int transpose, int rhs_sorted,
                   int codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* Device workspace (bytes, 256-byte aligned, may be 0) of the two MoE ops below: `glu` != 0 for
+ * kq_moe_glu_gather, 0 for kq_gather_qmv.  The batched path (more than 16 (token, expert) pairs)
+ * sorts the pairs by expert and keeps f16 activations there.  The reference allocates its own
+ * temporaries inside eval_gpu (src/kquant_moe_glu.cpp:277-382); here the caller owns them. */
+size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int codec, int dtype);
+
 /* out[t,r,:] = T(act(x[t] . G_e^T (+gb_e), x[t] . U_e^T (+ub_e))), e = idx[t,r]; f32 throughout,
  * one rounding.  x [T,K], gate/up stacks [E,N,bytes_per_row] dense, idx [T,R] uint32,
  * biases f32 [E,N] or NULL, out [T,R,N].
@@ -101,13 +107,14 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
 int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_w_dev,
                       const uint32_t* idx_dev, const float* gate_bias_dev, const float* up_bias_dev,
                       void* out_dev, int T, int R, int E, int N, int K, int act, float limit, float alpha,
-                      int codec, int dtype, void* stream);
+                      int codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
 
 /* out[t,r,:] = T(x[t,r,:] . W_e^T (+ bias_e)), e = idx[t,r].  x [T,R,K], w [E,N,bytes_per_row].
  * Replaces KQuantGatherQMVKQ (op gather_qmv_kq), reference src/kquant_moe_glu.cpp:1159-1210,
  * dispatch :331-382, kernels kq_moe_glu_kq.h:933-999. */
 int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev, const float* bias_dev,
-                  void* out_dev, int T, int R, int E, int N, int K, int codec, int dtype, void* stream);
+                  void* out_dev, int T, int R, int E, int N, int K, int codec, int dtype, void* workspace_dev,
+                  size_t workspace_bytes, void* stream);
 
 /* HOST function: wire = encode(w[rows, K] f32) (imatrix f32 [K] or NULL), rows * bytes_per_row
  * bytes written to wire_host.  Runs on the calling thread's CPU cores like the reference's

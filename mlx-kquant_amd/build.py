@@ -21,6 +21,7 @@ SOURCES = [
     ("kq_generic.hip", ["-ffp-contract=off"]),
     ("kq_mfma.hip", []),
     ("kq_gemm.hip", []),
+    ("kq_moe.hip", []),
 ]
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",

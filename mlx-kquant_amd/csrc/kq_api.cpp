@@ -184,9 +184,32 @@ static int check_moe(const char* op, int T, int R, int E, int N, int K, int code
   return KQ_OK;
 }
 
+size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int codec, int dtype) {
+  (void)dtype;
+  if (T <= 0 || R <= 0 || !codec_ok(codec)) return 0;
+  const int64_t P = (int64_t)T * R;
+  if (P > 0x7fffffff || !kq_moe_grouped_supported((int)P, E, N, K, codec)) return 0;
+  return kq_moe_grouped_workspace_bytes(glu ? T : (int)P, (int)P, E, K);
+}
+
+// Batched MoE path: returns KQ_ERR_UNSUPPORTED (error text untouched) when it does not apply.
+static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx, void* out,
+                           int T, int R, int E, int N, int K, int64_t estride, int glu, int act, float limit, int codec,
+                           int dtype, void* ws, size_t ws_bytes, hipStream_t s) {
+  const int64_t P = (int64_t)T * R;
+  if (P > 0x7fffffff || !kq_moe_grouped_supported((int)P, E, N, K, codec)) return KQ_ERR_UNSUPPORTED;
+  const int rows = glu ? T : (int)P;
+  const size_t need = kq_moe_grouped_workspace_bytes(rows, (int)P, E, K);
+  if (!ws || ws_bytes < need)
+    return kq_set_error(KQ_ERR_WORKSPACE, "%s: workspace of %zu bytes required (got %zu)", op, need, ws ? ws_bytes : 0);
+  return kq_launch_moe_grouped(x, static_cast<const uint8_t*>(w), static_cast<const uint8_t*>(w2), idx, out, rows,
+                               (int)P, E, N, K, glu ? R : 1, estride, glu, act, limit, codec, dtype, ws, s);
+}
+
 int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_w_dev, const uint32_t* idx_dev,
                       const float* gate_bias_dev, const float* up_bias_dev, void* out_dev, int T, int R, int E, int N,
-                      int K, int act, float limit, float alpha, int codec, int dtype, void* stream) {
+                      int K, int act, float limit, float alpha, int codec, int dtype, void* workspace_dev,
+                      size_t workspace_bytes, void* stream) {
   const char* op = "moe_glu_gather_kq";
   int rc = check_moe(op, T, R, E, N, K, codec, dtype);
   if (rc) return rc;
@@ -209,6 +232,10 @@ int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_
     return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
   const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
   if (!biased) {
+    const int rcg = try_moe_grouped(op, x_dev, gate_w_dev, up_w_dev, idx_dev, out_dev, T, R, E, N, K, estride, 1, act,
+                                    limit, codec, dtype, workspace_dev, workspace_bytes,
+                                    static_cast<hipStream_t>(stream));
+    if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(gate_w_dev),
                                            static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, out_dev, T * R, 1, N,
                                            K, R, K, estride, 1, act, limit, codec, dtype,
@@ -222,7 +249,8 @@ int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_
 }
 
 int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev, const float* bias_dev, void* out_dev,
-                  int T, int R, int E, int N, int K, int codec, int dtype, void* stream) {
+                  int T, int R, int E, int N, int K, int codec, int dtype, void* workspace_dev, size_t workspace_bytes,
+                  void* stream) {
   const char* op = "gather_qmv_kq";
   int rc = check_moe(op, T, R, E, N, K, codec, dtype);
   if (rc) return rc;
@@ -232,6 +260,9 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
   if (!x_dev || !w_dev || !idx_dev || !out_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
   const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
   if (!bias_dev) {
+    const int rcg = try_moe_grouped(op, x_dev, w_dev, nullptr, idx_dev, out_dev, T, R, E, N, K, estride, 0, 0, 0.f, codec,
+                                    dtype, workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
+    if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, out_dev,
                                            T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype,
                                            static_cast<hipStream_t>(stream));

@@ -75,3 +75,10 @@ size_t kq_gemm_workspace_bytes(int M, int K);
 bool kq_gemm_supported(int M, int N, int K, int codec);
 int kq_launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                    hipStream_t s);
+// Batched MoE path (q4_k / q5_k / q6_k, more than 16 pairs): pairs sorted by expert, one MFMA GEMM
+// per segment of <= 32 pairs.  rows = activation rows (T for the GLU op, T*R for the down op).
+bool kq_moe_grouped_supported(int P, int E, int N, int K, int codec);
+size_t kq_moe_grouped_workspace_bytes(int rows, int P, int E, int K);
+int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, void* out, int rows,
+                          int P, int E, int N, int K, int x_div, int64_t w_expert_stride, int glu, int act,
+                          float limit, int codec, int dtype, void* ws, hipStream_t s);

@@ -1,0 +1,246 @@
+// Building blocks shared by the matrix-core kernels (prefill GEMM, grouped MoE GEMM): wire
+// geometry of the K-quant superblocks as they travel HBM -> registers -> LDS, and the
+// per-superblock multiply-accumulate of one wave (32 weight rows x MT*32 activation rows).
+//
+// Numerics.  The B operand of v_mfma_f32_32x32x16_f16 always holds exact integers:
+//   q4_k / q5_k : sc_j*q (<= 63*31 < 2048), from 0x6400 | q = 1024 + q and one v_pk_fma_f16; the
+//                 -dmin*m_j term is one extra MFMA per superblock on the sub-block sums of x
+//                 (X_j split into two f16 halves);
+//   q6_k        : sc*(q - 32) reaches 4096, so a weight is fed as two exact terms, sc*ql (<= 1920)
+//                 and 16*sc*(qh - 2) (a multiple of 16 up to 4096): two MFMAs share one activation
+//                 fragment.
+// One f32 accumulator set collects a whole superblock and is folded into the running sum with one
+// multiply by d, so results differ from the f32 reference only by summation order.
+#pragma once
+
+#include <type_traits>
+
+#include "kq_decode.h"
+
+namespace kqmma {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// 16-byte global load from a 2-byte-aligned address (q6_k blocks are 210 bytes long): the
+// hardware serves unaligned vector loads, the type only stops the compiler from assuming more
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+
+// Compile-time loop: register arrays indexed by the loop variable are split into scalars.
+template <int N>
+struct StaticFor {
+  template <class F>
+  __device__ __forceinline__ static void run(F&& f) {
+    StaticFor<N - 1>::run(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+};
+template <>
+struct StaticFor<0> {
+  template <class F>
+  __device__ __forceinline__ static void run(F&&) {}
+};
+
+// Workgroup barrier that orders LDS traffic only (__syncthreads() would also drain every
+// outstanding global load).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+// Constants routed through registers the compiler cannot see through, so that (a & mask) | magic
+// becomes one v_and_or_b32 (VOP3 takes no literal operands on this target).
+__device__ __forceinline__ uint32_t opaque_vgpr(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+__device__ __forceinline__ uint32_t opaque_sgpr(uint32_t v) {
+  asm volatile("" : "+s"(v));
+  return v;
+}
+
+// A superblock travels as PP 16-byte pieces (q6_k: its first 208 bytes; the trailing 2-byte d
+// goes through a side channel) and is parked in LDS LBPB bytes apart.  LBPB / 16 is odd for all
+// three codecs, which keeps the row-per-lane ds_read_b128 of the fragment fetch conflict-free.
+template <int C>
+struct Wire;
+template <>
+struct Wire<KQ_Q4_K> {
+  static constexpr int BPB = 144, LBPB = 144, PP = 9, QS = 16;
+  static constexpr bool SIDE_D = false, MINS = true;
+  typedef u32x4 piece_t;
+};
+template <>
+struct Wire<KQ_Q5_K> {
+  static constexpr int BPB = 176, LBPB = 176, PP = 11, QS = 48;
+  static constexpr bool SIDE_D = false, MINS = true;
+  typedef u32x4 piece_t;
+};
+template <>
+struct Wire<KQ_Q6_K> {
+  static constexpr int BPB = 210, LBPB = 208, PP = 13, QS = 0;
+  static constexpr bool SIDE_D = true, MINS = false;
+  typedef u32x4_a2 piece_t;
+};
+
+// One superblock of one wave: weight row of this lane at b_lane (LDS), activation fragments at
+// a_lane + t*a_tile + 64 j + 16 s bytes (a_lane already includes the lane's row and 32*kg), the X
+// halves of m-block t at h_lane + t*h_tile (already including the lane's row and 16*kg).
+// acc[t] += (decoded weights) . (activations) for the MT m-blocks.
+template <int C, int MT>
+__device__ __forceinline__ void superblock_mma(const uint8_t* __restrict__ b_lane, uint16_t d_side, int kg,
+                                               const uint8_t* __restrict__ a_lane, int a_tile,
+                                               const uint8_t* __restrict__ h_lane, int h_tile, f32x16* acc) {
+  using G = Wire<C>;
+  const uint32_t magic = opaque_vgpr(0x64006400u);
+  f32x16 part[MT];
+  if constexpr (C == KQ_Q4_K || C == KQ_Q5_K) {
+    const uint32_t mask_lo = opaque_sgpr(0x000f000fu), mask_hi = opaque_sgpr(0x00f000f0u);
+    const uint4 hdr = *reinterpret_cast<const uint4*>(b_lane);
+    const float d = kq::h2f((uint16_t)(hdr.x & 0xffff));
+    const float dmin32 = kq::h2f((uint16_t)(hdr.x >> 16)) * 32.0f;
+    const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
+    const uint32_t scw[2] = {s0 & 0x3f3f3f3fu, (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)};
+    const uint32_t mnw[2] = {s1 & 0x3f3f3f3fu, ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u)};
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const uint4 qv = *reinterpret_cast<const uint4*>(b_lane + G::QS + 32 * g + 16 * kg);
+      const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
+      const uint32_t qw8[4] = {qw[0] >> 8, qw[1] >> 8, qw[2] >> 8, qw[3] >> 8};
+      uint32_t hb[4] = {0, 0, 0, 0};  // q5_k: fifth bits of this lane's 16 weights, positioned per pair
+      if constexpr (C == KQ_Q5_K) {
+        const uint4 hv = *reinterpret_cast<const uint4*>(b_lane + 16 + 16 * kg);
+        hb[0] = hv.x;
+        hb[1] = hv.y;
+        hb[2] = hv.z;
+        hb[3] = hv.w;
+      }
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int j = 2 * g + h;
+        const float scf = (float)((scw[j >> 2] >> (8 * (j & 3))) & 0xff);
+        // low nibbles read 1024 + q, high nibbles (in place) 1024 + 16 q: fold the 16 into the scale
+        const _Float16 sch = (_Float16)(h ? scf * 0.0625f : scf);
+        const _Float16 off = (_Float16)(-(h ? 64.0f : 1024.0f) * scf);
+        const f16x2 scp = {sch, sch}, offp = {off, off};
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          const uint32_t mask = h ? mask_hi : mask_lo;
+          uint32_t fr[4] = {(qw[2 * s] & mask) | magic, (qw8[2 * s] & mask) | magic, (qw[2 * s + 1] & mask) | magic,
+                            (qw8[2 * s + 1] & mask) | magic};
+          f16x2 bq[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++)  // one rounding: (1024 + q) * sc - 1024 * sc = sc * q exactly
+            bq[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fr[e]), scp, offp);
+          if constexpr (C == KQ_Q5_K) {
+            // fifth bit of weight (j, i) is bit j of qh[i]; this lane's bytes are qh[16 kg + 8 s + 0..7]
+            const _Float16 s16 = (_Float16)(16.0f * scf);
+            const uint32_t hwa = hb[2 * s] >> j, hwb = hb[2 * s + 1] >> j;
+            const _Float16 z = (_Float16)0.f;
+            const f16x2 add[4] = {{(hwa & 1) ? s16 : z, (hwa & 0x10000) ? s16 : z},
+                                  {(hwa & 0x100) ? s16 : z, (hwa & 0x1000000) ? s16 : z},
+                                  {(hwb & 1) ? s16 : z, (hwb & 0x10000) ? s16 : z},
+                                  {(hwb & 0x100) ? s16 : z, (hwb & 0x1000000) ? s16 : z}};
+#pragma unroll
+            for (int e = 0; e < 4; e++) bq[e] += add[e];
+          }
+          const f16x8 b = {bq[0][0], bq[0][1], bq[1][0], bq[1][1], bq[2][0], bq[2][1], bq[3][0], bq[3][1]};
+#pragma unroll
+          for (int t = 0; t < MT; t++) {
+            const f16x8 a = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile + 64 * j + 16 * s);
+            if (j == 0 && s == 0)
+              part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, f32x16{0}, 0, 0, 0);
+            else
+              part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, part[t], 0, 0, 0);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[t][i] = fmaf(d, part[t][i], acc[t][i]);
+
+    // mins: sum_j m_j X_j = 32 sum_j m_j (hi_j + lo_j); K slots 0..7 = hi, 8..15 = lo
+    _Float16 mj[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) mj[j] = (_Float16)(float)((mnw[j >> 2] >> (8 * (j & 3))) & 0xff);
+    const f16x8 bm = {mj[0], mj[1], mj[2], mj[3], mj[4], mj[5], mj[6], mj[7]};
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+      const f16x8 a = *reinterpret_cast<const f16x8*>(h_lane + t * h_tile);
+      part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bm, f32x16{0}, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[t][i] = fmaf(-dmin32, part[t][i], acc[t][i]);
+  } else {
+    // q6_k.  LDS block: ql[128] | qh[64] | int8 scales[16].  Weight 128 hf + 32 t + l (hf = half,
+    // t = 0..3, l = 0..31) has its low nibble in ql[64 hf + 32 (t & 1) + l] (high nibble of the byte
+    // when t >= 2), its high bits in bits 2t, 2t+1 of qh[32 hf + l] and scale 8 hf + 2 t + l / 16.
+    // Lane (row, kg) takes l = 16 kg .. 16 kg + 15: one scale per lane and sub-block.
+    const uint32_t mask_q = opaque_sgpr(0x00f000f0u), mask_h = opaque_sgpr(0x03000300u);
+    const uint4 scv = *reinterpret_cast<const uint4*>(b_lane + 192);
+    const uint32_t scw[4] = {scv.x, scv.y, scv.z, scv.w};
+#pragma unroll
+    for (int hf = 0; hf < 2; hf++) {
+      const uint4 hv = *reinterpret_cast<const uint4*>(b_lane + 128 + 32 * hf + 16 * kg);
+      const uint32_t hw[4] = {hv.x, hv.y, hv.z, hv.w};
+#pragma unroll
+      for (int qr = 0; qr < 2; qr++) {
+        const uint4 qv = *reinterpret_cast<const uint4*>(b_lane + 64 * hf + 32 * qr + 16 * kg);
+        const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const int t4 = qr + 2 * h, j = 4 * hf + t4;
+          const int sc = __builtin_amdgcn_sbfe((int)scw[2 * hf + (t4 >> 1)], 8 * (2 * (t4 & 1) + kg), 8);
+          const float scf = (float)sc;
+          const _Float16 sch = (_Float16)(scf * 0.0625f), ofl = (_Float16)(-64.0f * scf),
+                         ofh = (_Float16)(-96.0f * scf);
+          const f16x2 scp = {sch, sch}, oflp = {ofl, ofl}, ofhp = {ofh, ofh};
+#pragma unroll
+          for (int s = 0; s < 2; s++) {
+            uint32_t fl[4], fh[4];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+              const uint32_t q = qw[2 * s + e], hq = hw[2 * s + e];
+              const uint32_t qe = h ? q : (q << 4), qo = h ? (q >> 8) : (q >> 4);
+              const uint32_t he = hq << (8 - 2 * t4), ho = t4 ? (hq >> (2 * t4)) : hq;
+              fl[2 * e] = (qe & mask_q) | magic;      // bytes 0, 2 of the word: 1024 + 16 ql
+              fl[2 * e + 1] = (qo & mask_q) | magic;  // bytes 1, 3
+              fh[2 * e] = (he & mask_h) | magic;      // 1024 + 256 qh
+              fh[2 * e + 1] = (ho & mask_h) | magic;
+            }
+            f16x2 bl2[4], bh2[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              // (1024 + 16 ql) sc / 16 - 64 sc = sc ql;  (1024 + 256 qh) sc / 16 - 96 sc = 16 sc (qh - 2)
+              bl2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fl[e]), scp, oflp);
+              bh2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fh[e]), scp, ofhp);
+            }
+            const f16x8 blo = {bl2[0][0], bl2[0][1], bl2[1][0], bl2[1][1], bl2[2][0], bl2[2][1], bl2[3][0], bl2[3][1]};
+            const f16x8 bhi = {bh2[0][0], bh2[0][1], bh2[1][0], bh2[1][1], bh2[2][0], bh2[2][1], bh2[3][0], bh2[3][1]};
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+              const f16x8 a = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile + 64 * j + 16 * s);
+              if (j == 0 && s == 0)
+                part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, blo, f32x16{0}, 0, 0, 0);
+              else
+                part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, blo, part[t], 0, 0, 0);
+              part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bhi, part[t], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+    const float d = kq::h2f(d_side);
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[t][i] = fmaf(d, part[t][i], acc[t][i]);
+  }
+}
+
+}  // namespace kqmma

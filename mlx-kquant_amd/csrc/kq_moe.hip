@@ -1,0 +1,378 @@
+// Grouped MoE GEMM: the fused gate/up GLU op and the gathered down projection for many
+// (token, expert) pairs.  Pairs are counting-sorted by expert on the device and cut into segments
+// of at most 32 pairs of one expert; a workgroup multiplies one segment (the 32 activation rows of
+// v_mfma_f32_32x32x16_f16) by a 128-row slab of that expert's weights, so an expert's wire bytes are
+// streamed from HBM once per 32 pairs instead of once per pair.
+//
+// Workgroup = 4 waves.  Plain op: each wave owns 32 of the slab's 128 weight rows.  GLU: the slab
+// is 64 gate rows + the same 64 up rows (waves 0/2 gate, 1/3 up); the up waves hand their
+// accumulators to the gate waves through LDS and the epilogue act(g) * u runs before the single
+// rounding.  K advances one 256-wide superblock per step; wire bytes and the gathered activation
+// rows (converted to f16 by the activation prepass) are fetched one step ahead with coalesced
+// 16-byte loads and parked in LDS.
+#include "kq_epilogue.h"
+#include "kq_mma.h"
+
+int kq_launch_act_prepass(const void* x, void* xh, void* xhl, float* rs, int M, int K, int dtype, hipStream_t s);
+
+namespace {
+
+using namespace kqmma;
+
+constexpr int MOE_THREADS = 256;
+constexpr int SEG_M = 32;            // pairs per segment = activation rows of the MFMA
+constexpr int SLAB = 128;            // weight rows per workgroup (GLU: 64 gate + 64 up)
+constexpr int A_STRIDE = 512 + 16;   // bytes per activation row of one K step in LDS
+constexpr int SORT_THREADS = 1024;
+constexpr int SORT_MAX_E = 4096;
+
+struct Segment {
+  int expert, start, count, pad;
+};
+
+// ------------------------------------------------------------------ pair sort (one workgroup)
+// order[] = pair ids grouped by expert; segs[] = (expert, first position in order, pairs <= 32).
+// Pairs whose expert id is out of range are left out (their output rows are not written).
+__global__ __launch_bounds__(SORT_THREADS) void moe_sort_kernel(const uint32_t* __restrict__ idx, int P, int E,
+                                                               int* __restrict__ order, Segment* __restrict__ segs,
+                                                               int* __restrict__ nseg_out) {
+  __shared__ int cnt[SORT_MAX_E];     // pairs per expert, then the running cursor
+  __shared__ int scan_p[SORT_THREADS], scan_s[SORT_THREADS];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += SORT_THREADS) cnt[e] = 0;
+  __syncthreads();
+  for (int p = tid; p < P; p += SORT_THREADS) {
+    const uint32_t e = idx[p];
+    if (e < (uint32_t)E) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  // exclusive scans of pair counts and segment counts: thread t owns experts [t*ch, t*ch + ch)
+  const int ch = (E + SORT_THREADS - 1) / SORT_THREADS;
+  int lp = 0, ls = 0;
+  for (int i = 0; i < ch; i++) {
+    const int e = tid * ch + i;
+    if (e < E) {
+      lp += cnt[e];
+      ls += (cnt[e] + SEG_M - 1) / SEG_M;
+    }
+  }
+  scan_p[tid] = lp;
+  scan_s[tid] = ls;
+  __syncthreads();
+  for (int off = 1; off < SORT_THREADS; off <<= 1) {
+    const int vp = tid >= off ? scan_p[tid - off] : 0, vs = tid >= off ? scan_s[tid - off] : 0;
+    __syncthreads();
+    scan_p[tid] += vp;
+    scan_s[tid] += vs;
+    __syncthreads();
+  }
+  int bp = scan_p[tid] - lp, bs = scan_s[tid] - ls;  // exclusive prefix of this thread's experts
+  if (tid == SORT_THREADS - 1) *nseg_out = scan_s[tid];
+  for (int i = 0; i < ch; i++) {
+    const int e = tid * ch + i;
+    if (e < E) {
+      const int c = cnt[e];
+      for (int k = 0, s = bs; k < c; k += SEG_M, s++) segs[s] = Segment{e, bp + k, c - k < SEG_M ? c - k : SEG_M, 0};
+      bs += (c + SEG_M - 1) / SEG_M;
+      cnt[e] = bp;  // cursor
+      bp += c;
+    }
+  }
+  __syncthreads();
+  for (int p = tid; p < P; p += SORT_THREADS) {
+    const uint32_t e = idx[p];
+    if (e < (uint32_t)E) order[atomicAdd(&cnt[e], 1)] = p;
+  }
+}
+
+// ------------------------------------------------------------------ grouped GEMM
+struct MoeArgs {
+  const _Float16* xh;   // [rows][K] f16 activations (prepass), row = pair / x_div
+  const _Float16* xhl;  // [rows][K/256][16] X halves
+  const float* rs;      // [rows] activation scale
+  const uint8_t* w;
+  const uint8_t* w2;    // up stack (GLU) or null
+  void* y;              // [P][N]
+  const int* order;
+  const Segment* segs;
+  const int* nseg;
+  int N, K, x_div, act;
+  int64_t w_expert_stride;
+  float limit;
+};
+
+template <int C, int DT, bool GLU>
+__global__ __launch_bounds__(MOE_THREADS, 2) void moe_grouped_kernel(MoeArgs a) {
+  using G = Wire<C>;
+  constexpr int WPT = (SLAB * G::PP + MOE_THREADS - 1) / MOE_THREADS;  // wire pieces per thread per step
+  constexpr int APT = SEG_M * 32 / MOE_THREADS;                         // activation pieces per thread per step (4)
+  constexpr int NCOLS = GLU ? SLAB / 2 : SLAB;                          // output columns per workgroup
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint8_t* a_lds = smem;                                              // [32][A_STRIDE]
+  uint8_t* b_lds = a_lds + SEG_M * A_STRIDE;                          // [128][LBPB]
+  uint8_t* h_lds = b_lds + SLAB * G::LBPB;                            // [32][32] X halves
+  uint16_t* d_lds = reinterpret_cast<uint16_t*>(h_lds + SEG_M * 32);  // [128]
+  int* pair_lds = reinterpret_cast<int*>(d_lds + SLAB);               // [32] output row of each segment slot, -1 = none
+  float* rs_lds = reinterpret_cast<float*>(pair_lds + SEG_M);         // [32]
+
+  const int seg_id = blockIdx.y;
+  if (seg_id >= *a.nseg) return;  // uniform: the grid is sized for the worst case
+  const Segment seg = a.segs[seg_id];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, kg = lane >> 5;
+  const int N = a.N, K = a.K, nsb = K >> 8;
+  const size_t row_bytes = (size_t)nsb * G::BPB;
+  const int n0 = blockIdx.x * NCOLS;
+  const int ncols = N - n0 < NCOLS ? N - n0 : NCOLS;
+  const uint8_t* wtile = a.w + (size_t)seg.expert * (size_t)a.w_expert_stride + (size_t)n0 * row_bytes;
+  const uint8_t* wtile2 = GLU ? a.w2 + (size_t)seg.expert * (size_t)a.w_expert_stride + (size_t)n0 * row_bytes : wtile;
+
+  // slab row rr (= wave * 32 + l32 in the compute phase) -> (matrix, column): GLU waves alternate gate / up
+  auto slab_col = [&](int rr, bool& up) {
+    if constexpr (GLU) {
+      const int wv = rr >> 5;
+      up = wv & 1;
+      return (wv >> 1) * 32 + (rr & 31);
+    } else {
+      up = false;
+      return rr;
+    }
+  };
+
+  if (tid < SEG_M) {
+    const int pr = tid < seg.count ? a.order[seg.start + tid] : -1;
+    pair_lds[tid] = pr;
+    rs_lds[tid] = pr >= 0 ? a.rs[pr / a.x_div] : 0.f;
+  }
+
+  // piece maps.  Activations: piece i = tid + 256 t -> (slot i / 32, piece i % 32); spare slots of a
+  // short segment re-read its first pair (their results are dropped).
+  const int a_slot = tid >> 5, a_pc = tid & 31;  // + 8 slots per t
+  size_t a_goff[APT];
+  StaticFor<APT>::run([&](auto t) {
+    constexpr int T = decltype(t)::value;
+    const int slot = a_slot + 8 * T;
+    const int pr = a.order[seg.start + (slot < seg.count ? slot : 0)];
+    a_goff[T] = (size_t)(pr / a.x_div) * K + 8 * a_pc;
+  });
+  size_t h_goff;
+  {
+    const int slot = (tid & 63) >> 1;
+    const int pr = a.order[seg.start + (slot < seg.count ? slot : 0)];
+    h_goff = (size_t)(pr / a.x_div) * nsb * 16 + 8 * (tid & 1);
+  }
+  uint32_t w_goff[WPT], w_loff[WPT];
+  bool w_up[WPT];
+  {
+    int r = tid / G::PP, pc = tid % G::PP;
+    StaticFor<WPT>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      bool up;
+      const int col = slab_col(r < SLAB ? r : 0, up);
+      const bool ok = r < SLAB && col < ncols;  // rows past N and pieces past the slab re-read the slab start
+      w_up[T] = up;
+      w_goff[T] = ok ? (uint32_t)col * (uint32_t)row_bytes + 16 * pc : 0;
+      w_loff[T] = r < SLAB ? (uint32_t)r * G::LBPB + 16 * pc : 0xffffffffu;
+      r += MOE_THREADS / G::PP;
+      pc += MOE_THREADS % G::PP;
+      if (pc >= G::PP) {
+        pc -= G::PP;
+        r++;
+      }
+    });
+  }
+  // side channel for the trailing 2-byte d of a q6_k block: thread -> slab row tid % 128
+  const uint8_t* d_src;
+  {
+    bool up;
+    const int col = slab_col(tid & (SLAB - 1), up);
+    d_src = (up ? wtile2 : wtile) + (size_t)(col < ncols ? col : 0) * row_bytes + 208;
+  }
+
+  u32x4 areg[APT], wreg[WPT], hreg;
+  uint16_t dreg = 0;
+  auto issue = [&](int sb) {
+    StaticFor<APT>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      areg[T] = *reinterpret_cast<const u32x4*>(a.xh + a_goff[T] + 256 * sb);
+    });
+    StaticFor<WPT>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      const uint8_t* base = (GLU && w_up[T]) ? wtile2 : wtile;
+      wreg[T] = *reinterpret_cast<const typename G::piece_t*>(base + (size_t)sb * G::BPB + w_goff[T]);
+    });
+    if constexpr (G::SIDE_D) dreg = *reinterpret_cast<const uint16_t*>(d_src + (size_t)sb * G::BPB);
+    if constexpr (G::MINS) hreg = *reinterpret_cast<const u32x4*>(a.xhl + h_goff + (size_t)sb * 16);
+  };
+  auto park = [&]() {
+    StaticFor<APT>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      *reinterpret_cast<u32x4*>(a_lds + (a_slot + 8 * T) * A_STRIDE + 16 * a_pc) = areg[T];
+    });
+    StaticFor<WPT>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      if (w_loff[T] != 0xffffffffu) *reinterpret_cast<u32x4*>(b_lds + w_loff[T]) = wreg[T];
+    });
+    if constexpr (G::MINS) {
+      if (tid < 64) *reinterpret_cast<u32x4*>(h_lds + 16 * tid) = hreg;
+    }
+    if constexpr (G::SIDE_D) {
+      if (tid < SLAB) d_lds[tid] = dreg;
+    }
+  };
+
+  f32x16 acc[1] = {f32x16{0}};
+  const uint8_t* b_lane = b_lds + (wave * 32 + l32) * G::LBPB;
+  const uint8_t* a_lane = a_lds + l32 * A_STRIDE + 32 * kg;
+  const uint8_t* h_lane = h_lds + l32 * 32 + 16 * kg;
+
+  issue(0);
+  for (int sb = 0; sb < nsb; sb++) {
+    if (sb > 0) lds_barrier();  // everyone is done reading the previous step
+    park();
+    if (sb + 1 < nsb) issue(sb + 1);
+    lds_barrier();
+    superblock_mma<C, 1>(b_lane, G::SIDE_D ? d_lds[wave * 32 + l32] : (uint16_t)0, kg, a_lane, 0, h_lane, 0, acc);
+  }
+
+  // ---- epilogue: undo the activation scale, (GLU: combine gate and up,) round once, scatter rows
+  uint16_t* y = static_cast<uint16_t*>(a.y);
+  if constexpr (GLU) {
+    lds_barrier();  // the step buffers are free: reuse them for the up accumulators
+    float* ex = reinterpret_cast<float*>(smem);  // [2 column blocks][16][64]
+    const int nb = wave >> 1;
+    if (wave & 1) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) ex[(nb * 16 + i) * 64 + lane] = acc[0][i];
+    }
+    lds_barrier();
+    if (!(wave & 1)) {
+      const int col = nb * 32 + l32;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int slot = 8 * (i >> 2) + 4 * kg + (i & 3);
+        const int pr = pair_lds[slot];
+        if (pr >= 0 && col < ncols) {
+          const float r = rs_lds[slot];
+          const float v = kq::glu_epilogue(a.act, acc[0][i] * r, ex[(nb * 16 + i) * 64 + lane] * r, a.limit, 1.0f);
+          y[(size_t)pr * N + n0 + col] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+        }
+      }
+    }
+  } else {
+    const int col = wave * 32 + l32;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int slot = 8 * (i >> 2) + 4 * kg + (i & 3);
+      const int pr = pair_lds[slot];
+      if (pr >= 0 && col < ncols) {
+        const float v = acc[0][i] * rs_lds[slot];
+        y[(size_t)pr * N + n0 + col] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+      }
+    }
+  }
+}
+
+struct MoeWorkspace {
+  _Float16* xh;
+  _Float16* xhl;
+  float* rs;
+  int* order;
+  Segment* segs;
+  int* nseg;
+  size_t bytes;
+};
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+MoeWorkspace carve(void* ws, int rows, int P, int E, int K) {
+  MoeWorkspace m;
+  uint8_t* p = static_cast<uint8_t*>(ws);
+  size_t o = 0;
+  m.xh = reinterpret_cast<_Float16*>(p + o);
+  o += align256((size_t)rows * K * 2);
+  m.xhl = reinterpret_cast<_Float16*>(p + o);
+  o += align256((size_t)rows * (K >> 8) * 32);
+  m.rs = reinterpret_cast<float*>(p + o);
+  o += align256((size_t)rows * 4);
+  m.order = reinterpret_cast<int*>(p + o);
+  o += align256((size_t)P * 4);
+  const size_t maxseg = (size_t)E + P / SEG_M + 1;
+  m.segs = reinterpret_cast<Segment*>(p + o);
+  o += align256(maxseg * sizeof(Segment));
+  m.nseg = reinterpret_cast<int*>(p + o);
+  o += 256;
+  m.bytes = o;
+  return m;
+}
+
+template <int C, int DT, bool GLU>
+int launch_grouped(const MoeArgs& a, int P, int E, hipStream_t s) {
+  using G = Wire<C>;
+  constexpr int NCOLS = GLU ? SLAB / 2 : SLAB;
+  const int ntiles = (a.N + NCOLS - 1) / NCOLS;
+  int maxseg = E + P / SEG_M;  // sum over experts of ceil(c_e / 32) <= E + P / 32
+  if (maxseg > P) maxseg = P;
+  const size_t lds = SEG_M * A_STRIDE + SLAB * G::LBPB + SEG_M * 32 + SLAB * 2 + SEG_M * 8;
+  auto kern = moe_grouped_kernel<C, DT, GLU>;
+  hipLaunchKernelGGL(kern, dim3(ntiles, maxseg), dim3(MOE_THREADS), lds, s, a);
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
+template <bool GLU>
+int launch_grouped_any(const MoeArgs& a, int P, int E, int codec, int dtype, hipStream_t s) {
+  if (codec == KQ_Q4_K)
+    return dtype == KQ_F16 ? launch_grouped<KQ_Q4_K, KQ_F16, GLU>(a, P, E, s)
+                           : launch_grouped<KQ_Q4_K, KQ_BF16, GLU>(a, P, E, s);
+  if (codec == KQ_Q5_K)
+    return dtype == KQ_F16 ? launch_grouped<KQ_Q5_K, KQ_F16, GLU>(a, P, E, s)
+                           : launch_grouped<KQ_Q5_K, KQ_BF16, GLU>(a, P, E, s);
+  return dtype == KQ_F16 ? launch_grouped<KQ_Q6_K, KQ_F16, GLU>(a, P, E, s)
+                         : launch_grouped<KQ_Q6_K, KQ_BF16, GLU>(a, P, E, s);
+}
+
+}  // namespace
+
+bool kq_moe_grouped_supported(int P, int E, int N, int K, int codec) {
+  return (codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K) && P > 16 && E <= SORT_MAX_E && K > 0 &&
+         (K & 255) == 0 && N > 0 && (int64_t)E + P / SEG_M < 65535;
+}
+
+// rows = activation rows the prepass converts: T for the GLU op (x is [T,K]), T*R for the down op.
+size_t kq_moe_grouped_workspace_bytes(int rows, int P, int E, int K) { return carve(nullptr, rows, P, E, K).bytes; }
+
+// x: [rows][K] activations; pair p reads row p / x_div and expert idx[p]; out [P][N].
+int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, void* out, int rows,
+                          int P, int E, int N, int K, int x_div, int64_t w_expert_stride, int glu, int act,
+                          float limit, int codec, int dtype, void* ws, hipStream_t s) {
+  if (!kq_moe_grouped_supported(P, E, N, K, codec) || (glu && act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
+  const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;  // q6_k pieces are fetched with unaligned loads
+  if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
+      ((uintptr_t)w_expert_stride & wmask) || (reinterpret_cast<uintptr_t>(x) & 15) ||
+      (reinterpret_cast<uintptr_t>(ws) & 255))
+    return KQ_ERR_UNSUPPORTED;
+  const MoeWorkspace m = carve(ws, rows, P, E, K);
+  int rc = kq_launch_act_prepass(x, m.xh, m.xhl, m.rs, rows, K, dtype, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(SORT_THREADS), 0, s, idx, P, E, m.order, m.segs, m.nseg);
+  KQ_HIP_CHECK(hipGetLastError());
+  MoeArgs a{};
+  a.xh = m.xh;
+  a.xhl = m.xhl;
+  a.rs = m.rs;
+  a.w = w;
+  a.w2 = w2;
+  a.y = out;
+  a.order = m.order;
+  a.segs = m.segs;
+  a.nseg = m.nseg;
+  a.N = N;
+  a.K = K;
+  a.x_div = x_div < 1 ? 1 : x_div;
+  a.act = act;
+  a.w_expert_stride = w_expert_stride;
+  a.limit = limit;
+  return glu ? launch_grouped_any<true>(a, P, E, codec, dtype, s) : launch_grouped_any<false>(a, P, E, codec, dtype, s);
+}

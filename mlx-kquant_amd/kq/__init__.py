@@ -69,8 +69,10 @@ def _load():
     lib.kq_gather_qmm_workspace_size.restype = sz
     lib.kq_gather_qmm_workspace_size.argtypes = [i, i, i, i, i, i, i]
     lib.kq_gather_qmm.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i64, i64, i, i, i, i, vp, sz, vp]
-    lib.kq_moe_glu_gather.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, f, f, i, i, vp]
-    lib.kq_gather_qmv.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp]
+    lib.kq_moe_workspace_size.restype = sz
+    lib.kq_moe_workspace_size.argtypes = [i, i, i, i, i, i, i, i]
+    lib.kq_moe_glu_gather.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, f, f, i, i, vp, sz, vp]
+    lib.kq_gather_qmv.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, sz, vp]
     lib.kq_quantize.argtypes = [vp, vp, vp, i64, i64, i]
     _lib = lib
     return lib
@@ -327,11 +329,14 @@ def moe_glu_gather_kq(x, gate_w, up_w, kquant_type, indices, act="silu", limit=0
     T, R = idx.shape
     E, N = gate_w.shape[0], gate_w.shape[1]
     out = torch.empty((T, R, N), dtype=x.dtype, device=x.device)
+    lib = _load()
     with torch.cuda.device(x.device):
-        _check(_load().kq_moe_glu_gather(x_c.data_ptr(), gate_w.data_ptr(), up_w.data_ptr(), idx.data_ptr(),
-                                         gb.data_ptr() if biased else None, ub.data_ptr() if biased else None,
-                                         out.data_ptr(), T, R, E, N, K, _ACTS[act], float(limit), float(alpha), cid,
-                                         _DT[x.dtype], sp))
+        ws_bytes = 0 if biased else lib.kq_moe_workspace_size(T, R, E, N, K, 1, cid, _DT[x.dtype])
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+        _check(lib.kq_moe_glu_gather(x_c.data_ptr(), gate_w.data_ptr(), up_w.data_ptr(), idx.data_ptr(),
+                                     gb.data_ptr() if biased else None, ub.data_ptr() if biased else None,
+                                     out.data_ptr(), T, R, E, N, K, _ACTS[act], float(limit), float(alpha), cid,
+                                     _DT[x.dtype], ws.data_ptr() if ws is not None else None, ws_bytes, sp))
     return out
 
 
@@ -361,10 +366,13 @@ def gather_qmv_kq(x, w, kquant_type, indices, bias=None, *, stream=None):
     T, R = idx.shape
     E, N = w.shape[0], w.shape[1]
     out = torch.empty((T, R, N), dtype=x.dtype, device=x.device)
+    lib = _load()
     with torch.cuda.device(x.device):
-        _check(_load().kq_gather_qmv(x_c.data_ptr(), w.data_ptr(), idx.data_ptr(),
-                                     b.data_ptr() if b is not None else None, out.data_ptr(), T, R, E, N, K, cid,
-                                     _DT[x.dtype], sp))
+        ws_bytes = 0 if b is not None else lib.kq_moe_workspace_size(T, R, E, N, K, 0, cid, _DT[x.dtype])
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+        _check(lib.kq_gather_qmv(x_c.data_ptr(), w.data_ptr(), idx.data_ptr(),
+                                 b.data_ptr() if b is not None else None, out.data_ptr(), T, R, E, N, K, cid,
+                                 _DT[x.dtype], ws.data_ptr() if ws is not None else None, ws_bytes, sp))
     return out
 
 

@@ -115,7 +115,7 @@ def test_qmm_reference_fixtures(kq, codec):
         assert rel_l2(dev_to_bits(got), want, "float16") <= TOL
 
 
-@pytest.mark.parametrize("codec", ["q4_k", "q5_k"])
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("M,N,K", [(9, 40, 256), (200, 200, 512), (130, 384, 2304), (512, 256, 4096)])
 def test_qmm_prefill_gemm(kq, codec, M, N, K):
     """Prefill GEMM path (M > 8): ragged M and N tiles, several superblocks, both activation dtypes."""

@@ -123,6 +123,50 @@ def test_moe_tuned_gathered_shapes(kq, codec, E, N, K, T, R):
     assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, codec
 
 
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("E,N,K,T,R", [(6, 136, 768, 20, 3), (8, 200, 512, 100, 2), (128, 64, 256, 8, 8),
+                                       (5, 72, 4352, 9, 2)])
+def test_moe_grouped_batched_shapes(kq, codec, E, N, K, T, R):
+    """More than 16 pairs: the expert-sorted MFMA path (segments of <= 32 pairs; experts with none, one
+    partial or several segments; column slabs that do not divide N)."""
+    gate = _stack(codec, E, N, K, seed=81)
+    up = _stack(codec, E, N, K, seed=82)
+    rng = np.random.default_rng(83)
+    idx = rng.integers(0, E, (T, R))
+    if E == 8:
+        idx[:, 0] = 3  # one hot expert: 100+ pairs = four segments; expert 5 gets none
+        idx[idx == 5] = 6
+    for dtype, act, limit in (("bfloat16", "silu", 0.0), ("float16", "gelu", 0.0), ("bfloat16", "silu_limit", 0.4)):
+        xb, xt = make_x((T, K), dtype, seed=84, scale=0.02)
+        got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act=act, limit=limit)
+        want = _glu_truth(codec, xb, gate, up, idx, act, limit, dtype=dtype)
+        assert tuple(got.shape) == (T, R, N)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype, act)
+    for dtype in ("bfloat16", "float16"):
+        hb, ht = make_x((T, R, K), dtype, seed=85, scale=0.02)
+        got = kq.gather_qmv_kq(ht, wire_to_dev(gate), codec, _idx_dev(idx))
+        want = O.gather_qmv(hb, gate, codec, idx, None, dtype)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype)
+
+
+def test_moe_grouped_matches_per_pair_path_bitwise(kq):
+    """A pair's row does not depend on which other pairs share the call: rows of a 64-pair call equal the
+    rows of the same pairs computed in 4-pair calls (different kernels, same exact products)."""
+    codec, E, N, K, T, R = "q4_k", 8, 128, 1024, 32, 2
+    gate = _stack(codec, E, N, K, seed=86)
+    up = _stack(codec, E, N, K, seed=87)
+    idx = np.random.default_rng(88).integers(0, E, (T, R))
+    xb, xt = make_x((T, K), "bfloat16", seed=89, scale=0.02)
+    g, u = wire_to_dev(gate), wire_to_dev(up)
+    big = O.bits_to_f32(dev_to_bits(kq.moe_glu_gather_kq(xt, g, u, codec, _idx_dev(idx))), "bfloat16")
+    small = np.concatenate([O.bits_to_f32(dev_to_bits(kq.moe_glu_gather_kq(xt[t:t + 2], g, u, codec,
+                                                                         _idx_dev(idx[t:t + 2]))), "bfloat16")
+                            for t in range(0, T, 2)])
+    # both are exact products accumulated in f32 in different orders: agreement to a few bf16 ulps
+    assert np.linalg.norm(big - small) / np.linalg.norm(small) <= 2e-3
+    assert np.mean(big != small) < 0.2
+
+
 @pytest.mark.parametrize("codec", ["mxfp4", "nvfp4"])
 def test_moe_swiglu_clamp_bias(kq, codec):
     E, N, K, T, R = 4, 64, 576, 4, 2
