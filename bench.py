@@ -9,9 +9,14 @@ measured COLD: every step reads a different copy of the wire matrix, the copies 
 exceeding twice the 256 MB last-level cache, so the weight bytes come from HBM.
 value = quantized weight bytes per step / step time (HIP events on the launching stream).
 
-Extra fields: `sweep` (the other decode projections of the q4_k_m recipe at M in {1,2,4,8}),
-`prefill` (q4_k / q5_k GEMM 8192 -> 28672 at M in {512, 2048}), `roofline` for the dominant kernel
-and `cpu_baseline` (the CPU oracle timed on this box's host cores on the headline GEMV).
+Every timed call goes through the C ABI of libkq (ctypes) with outputs and workspace allocated
+beforehand, so a step is the library call and nothing else.
+
+Extra fields: `sweep` (the decode projections of the q4_k_m recipe at M in {1,2,4,8}), `prefill`
+(q4_k / q5_k / q6_k GEMM 8192 -> 28672 at M in {512, 2048}), `moe` (128 experts, top-8, hidden 2048,
+intermediate 768: fused gate/up GLU in q4_k and down in q6_k at 1 and 256 tokens), `lowbit` (M=1
+GEMV 8192 -> 8192 in the low-bit codecs), `roofline` for the dominant kernel and `cpu_baseline`
+(the CPU oracle timed on this box's host cores on the headline GEMV).
 """
 import argparse
 import json
@@ -26,6 +31,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLC_BYTES = 256 << 20
+KQ_BF16 = 2
 
 
 def synth_wire_torch(codec, rows, K, seed, device):
@@ -59,21 +65,85 @@ def quantized_weights(kq, torch, codec, N, K, seed, device):
     return wq.to(device)
 
 
-def time_matmul(kq, torch, x, copies, codec, steps, warmup):
-    """Average per-launch time (ms) over `steps` launches rotating over `copies` (events + wall)."""
-    n = len(copies)
+def time_calls(torch, calls, steps, warmup):
+    """Average time (ms) of one call over `steps` calls rotating over the closures in `calls`."""
+    n = len(calls)
     for i in range(warmup):
-        kq.quantized_matmul(x, copies[i % n], None, codec)
+        calls[i % n]()
     torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
     for i in range(steps):
-        kq.quantized_matmul(x, copies[i % n], None, codec)
+        calls[i % n]()
     ev1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     return ev0.elapsed_time(ev1) / steps, wall_ms / steps
+
+
+class Abi:
+    """Closures over the C ABI with every buffer allocated up front."""
+
+    def __init__(self, kq, torch, dev):
+        self.kq, self.torch, self.dev = kq, torch, dev
+        self.lib = kq._load()
+        self.stream = torch.cuda.current_stream().cuda_stream
+
+    def _check(self, rc):
+        if rc != 0:
+            raise RuntimeError(self.lib.kq_last_error().decode())
+
+    def qmm(self, x, w, codec, N, K):
+        torch, lib = self.torch, self.lib
+        M = x.shape[0]
+        cid = lib.kq_codec_id(codec.encode())
+        out = torch.empty((M, N), dtype=x.dtype, device=self.dev)
+        nws = lib.kq_qmm_workspace_size(M, N, K, 1, cid, KQ_BF16)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=self.dev)
+        args = (x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, 1, cid, KQ_BF16, ws.data_ptr(), nws, self.stream)
+        keep = (x, w, out, ws)
+
+        def call(_keep=keep):
+            rc = lib.kq_qmm(*args)
+            if rc:
+                self._check(rc)
+        return call
+
+    def moe_glu(self, x, gate, up, codec, idx):
+        torch, lib = self.torch, self.lib
+        (T, K), (E, N) = x.shape, gate.shape[:2]
+        R = idx.shape[1]
+        cid = lib.kq_codec_id(codec.encode())
+        out = torch.empty((T, R, N), dtype=x.dtype, device=self.dev)
+        nws = lib.kq_moe_workspace_size(T, R, E, N, K, 1, cid, KQ_BF16)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=self.dev)
+        args = (x.data_ptr(), gate.data_ptr(), up.data_ptr(), idx.data_ptr(), None, None, out.data_ptr(), T, R, E, N, K,
+                0, 0.0, 0.0, cid, KQ_BF16, ws.data_ptr(), nws, self.stream)
+        keep = (x, gate, up, idx, out, ws)
+
+        def call(_keep=keep):
+            rc = lib.kq_moe_glu_gather(*args)
+            if rc:
+                self._check(rc)
+        return call, out
+
+    def gather_qmv(self, h, w, codec, idx):
+        torch, lib = self.torch, self.lib
+        (T, R, K), (E, N) = h.shape, w.shape[:2]
+        cid = lib.kq_codec_id(codec.encode())
+        out = torch.empty((T, R, N), dtype=h.dtype, device=self.dev)
+        nws = lib.kq_moe_workspace_size(T, R, E, N, K, 0, cid, KQ_BF16)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=self.dev)
+        args = (h.data_ptr(), w.data_ptr(), idx.data_ptr(), None, out.data_ptr(), T, R, E, N, K, cid, KQ_BF16,
+                ws.data_ptr(), nws, self.stream)
+        keep = (h, w, idx, out, ws)
+
+        def call(_keep=keep):
+            rc = lib.kq_gather_qmv(*args)
+            if rc:
+                self._check(rc)
+        return call
 
 
 def cold_copies(torch, base, wbytes):
@@ -106,7 +176,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--no-sweep", action="store_true", help="skip the decode sweep and the prefill GEMM")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the sweep, prefill, MoE and low-bit sections")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -119,18 +189,23 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    abi = Abi(kq, torch, dev)
+    gx = torch.Generator(device=dev)
+    gx.manual_seed(100)
+
+    def randx(shape, scale=1.0):
+        return (torch.randn(shape, device=dev, dtype=torch.float32, generator=gx) * scale).to(torch.bfloat16)
 
     # ---------------- headline: q4_k gate/up GEMV, M = 1, cold
     codec, N, K, M = "q4_k", 14336, 4096, 1
     wbytes = N * kq.bytes_per_row(codec, K)
     base = quantized_weights(kq, torch, codec, N, K, seed=2, device=dev)
     copies = cold_copies(torch, base, wbytes)
-    gx = torch.Generator(device=dev)
-    gx.manual_seed(100)
-    x = torch.randn((M, K), device=dev, dtype=torch.float32, generator=gx).to(torch.bfloat16)
-    ms, wall_ms = time_matmul(kq, torch, x, copies, codec, args.steps, args.warmup)
+    x = randx((M, K))
+    calls = [abi.qmm(x, w, codec, N, K) for w in copies]
+    ms, wall_ms = time_calls(torch, calls, args.steps, args.warmup)
     gbs = wbytes / (ms * 1e-3) / 1e9
-    hot_ms, _ = time_matmul(kq, torch, x, copies[:1], codec, args.steps, args.warmup)
+    hot_ms, _ = time_calls(torch, calls[:1], args.steps, args.warmup)
 
     out = {
         "metric": "q4_k GEMV weight-GB/s at M=1 (cold)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
@@ -147,11 +222,12 @@ def main():
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
     }
     base_np = base.cpu().numpy() if not args.no_cpu else None
-    del copies
+    del copies, calls
 
     if not args.no_sweep:
-        sweep = []
         steps, warm = max(50, args.steps // 10), max(10, args.warmup // 10)
+        # ---------------- decode sweep (q4_k_m recipe of Llama-3-8B)
+        sweep = []
         shapes = [("q_proj", "q4_k", 4096, 4096, True), ("gate/up", "q4_k", 14336, 4096, True),
                   ("down", "q6_k", 4096, 14336, True), ("lm_head", "q6_k", 128256, 4096, False)]
         for name, c, n, k, encode in shapes:
@@ -162,25 +238,72 @@ def main():
                                                  else synth_wire_torch(c, n, k, 3, dev))
             cps = cold_copies(torch, wq, wb)
             for m in (1, 2, 4, 8):
-                xm = torch.randn((m, k), device=dev, dtype=torch.float32, generator=gx).to(torch.bfloat16)
-                t, _ = time_matmul(kq, torch, xm, cps, c, steps, warm)
+                xm = randx((m, k))
+                t, _ = time_calls(torch, [abi.qmm(xm, w, c, n, k) for w in cps], steps, warm)
                 sweep.append({"proj": name, "codec": c, "N": n, "K": k, "M": m, "us": round(t * 1e3, 2),
                               "cold_gbs": round(wb / (t * 1e-3) / 1e9, 1),
                               "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
             del cps, wq
         out["sweep"] = sweep
+
+        # ---------------- prefill GEMM
         prefill = []
-        for c in ("q4_k", "q5_k"):
+        for c in ("q4_k", "q5_k", "q6_k"):
             n, k = 28672, 8192
             wq = quantized_weights(kq, torch, c, n, k, 5, dev)
             for m in (512, 2048):
-                xm = torch.randn((m, k), device=dev, dtype=torch.float32, generator=gx).to(torch.bfloat16)
-                t, _ = time_matmul(kq, torch, xm, [wq], c, 20, 5)
+                t, _ = time_calls(torch, [abi.qmm(randx((m, k)), wq, c, n, k)], 20, 5)
                 tf = 2.0 * m * n * k / (t * 1e-3) / 1e12
                 prefill.append({"codec": c, "M": m, "N": n, "K": k, "ms": round(t, 4), "tflops": round(tf, 1),
                                 "pct_mfma_f16_peak": round(100 * tf / MFMA_F16_PEAK_TFLOPS, 2)})
             del wq
         out["prefill"] = prefill
+
+        # ---------------- MoE: 128 experts, top-8, hidden 2048, intermediate 768 (structurally valid random wire)
+        E, H, I, TOPK = 128, 2048, 768, 8
+        gate = synth_wire_torch("q4_k", E * I, H, 11, dev).reshape(E, I, -1)
+        up = synth_wire_torch("q4_k", E * I, H, 12, dev).reshape(E, I, -1)
+        down = synth_wire_torch("q6_k", E * H, I, 13, dev).reshape(E, H, -1)
+        gu_bytes = 2 * I * kq.bytes_per_row("q4_k", H)
+        dn_bytes = H * kq.bytes_per_row("q6_k", I)
+        moe = []
+        for T in (1, 256):
+            xt = randx((T, H), 0.5)
+            # 16 different routings, rotated per step, so that a step's experts are not the previous step's
+            glu_calls, dn_calls, touched = [], [], []
+            for r in range(16):
+                logits = torch.randn((T, E), device=dev, generator=gx)
+                idx = logits.topk(TOPK, dim=-1).indices.to(torch.int32).contiguous()
+                call, h = abi.moe_glu(xt, gate, up, "q4_k", idx)
+                glu_calls.append(call)
+                dn_calls.append(abi.gather_qmv(h, down, "q6_k", idx))
+                touched.append(int(idx.unique().numel()))
+            ne = sum(touched) / len(touched)
+            tg, _ = time_calls(torch, glu_calls, steps, warm)
+            td, _ = time_calls(torch, dn_calls, steps, warm)
+            moe.append({"tokens": T, "experts_touched": round(ne, 1), "glu_us": round(tg * 1e3, 2),
+                        "down_us": round(td * 1e3, 2),
+                        "glu_gbs": round(ne * gu_bytes / (tg * 1e-3) / 1e9, 1),
+                        "down_gbs": round(ne * dn_bytes / (td * 1e-3) / 1e9, 1),
+                        "pct_hbm_peak": round(100 * ne * (gu_bytes + dn_bytes) / ((tg + td) * 1e-3) / 1e9
+                                              / HBM_PEAK_GBS, 2)})
+        del gate, up, down
+        out["moe"] = moe
+
+        # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (q2_k / q3_k encoded, IQ codecs random wire)
+        lowbit = []
+        for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs"):
+            n = k = 8192
+            wb = n * kq.bytes_per_row(c, k)
+            wq = quantized_weights(kq, torch, c, n, k, 7, dev) if c in ("q2_k", "q3_k") else \
+                synth_wire_torch(c, n, k, 7, dev)
+            cps = cold_copies(torch, wq, wb)
+            t, _ = time_calls(torch, [abi.qmm(x.new_ones((1, k)), w, c, n, k) for w in cps], steps, warm)
+            lowbit.append({"codec": c, "N": n, "K": k, "M": 1, "us": round(t * 1e3, 2),
+                           "cold_gbs": round(wb / (t * 1e-3) / 1e9, 1),
+                           "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
+            del cps, wq
+        out["lowbit"] = lowbit
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(base_np, codec, K, M)
