@@ -109,8 +109,9 @@ int kq_dequantize(const void* w_dev, void* out_dev, uint64_t num_weights, int co
 
 size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int dtype) {
   (void)dtype;
-  if (transpose && codec_ok(codec) && kq_gemm_supported(M, N, K, codec)) return kq_gemm_workspace_bytes(M, K);
-  return 0;
+  if (!transpose || !codec_ok(codec)) return 0;
+  if (kq_gemm_supported(M, N, K, codec)) return kq_gemm_workspace_bytes(M, K);
+  return kq_qmm_tuned_workspace_bytes(M, N, K, codec);  // split-K partial sums of the skinny kernels (optional)
 }
 
 int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int transpose, int codec,
@@ -137,7 +138,8 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
     int rcg = kq_launch_gemm(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev, s);
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
   }
-  int rc = kq_launch_qmm_tuned(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+  int rc = kq_launch_qmm_tuned(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev,
+                               workspace_bytes, s);
   if (rc != KQ_ERR_UNSUPPORTED) return rc;
   return kq_launch_gemv_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
 }

@@ -62,8 +62,10 @@ int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2,
                              int act, float limit, float alpha, int codec, int dtype, hipStream_t s);
 // Tuned path: returns KQ_ERR_UNSUPPORTED (without touching the error text) when no tuned kernel
 // covers the request, so the caller can fall through to the generic kernels.
-int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
-                        hipStream_t s);
+// A null / short workspace is allowed: the call then runs without its split-K plan.
+size_t kq_qmm_tuned_workspace_bytes(int M, int N, int K, int codec);
+int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                        size_t ws_bytes, hipStream_t s);
 // Tuned gathered GEMV (items = (activation matrix, expert) pairs, M <= 8 rows each; with glu the
 // gate/up pair and the fused epilogue, M = 1): same fall-through contract as kq_launch_qmm_tuned.
 int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,

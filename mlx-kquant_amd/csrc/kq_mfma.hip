@@ -252,6 +252,9 @@ struct SkArgs {
   int64_t x_batch_stride;   // elements between activation matrices
   int64_t w_expert_stride;  // bytes between expert matrices
   float limit;
+  // split-K (dense calls with few row tiles): grid z = K split; partial sums [ksplit][M][N] f32
+  float* partial;
+  int ksplit, sb_per_split;
 };
 
 // MB = M rounded up to a power of two (1, 2, 4, 8).  Rows of the 32-row A operand beyond MB alias
@@ -341,8 +344,10 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
   const bool d_ok = G::SIDE_D && d_row < rows_per_tile && d_srow < nrows;
   const uint8_t* d_src = (d_up ? wtile2 : wtile) + (d_ok ? (size_t)d_srow * row_bytes : 0) + 208;
 
-  for (int sb0 = 0; sb0 < nsb; sb0 += kch) {
-    const int sbn = (nsb - sb0 < kch) ? (nsb - sb0) : kch;
+  const int sb_begin = a.ksplit > 1 ? (int)blockIdx.z * a.sb_per_split : 0;
+  const int sb_end = a.ksplit > 1 ? (sb_begin + a.sb_per_split < nsb ? sb_begin + a.sb_per_split : nsb) : nsb;
+  for (int sb0 = sb_begin; sb0 < sb_end; sb0 += kch) {
+    const int sbn = (sb_end - sb0 < kch) ? (sb_end - sb0) : kch;
     const int kc = sbn << 8, k0 = sb0 << 8;
 
     // ---- 1. activation loads first, so waiting for them does not wait for the weights
@@ -386,7 +391,7 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
     issue(std::integral_constant<int, 1>{});
 
     // ---- 3. activations -> f16 in LDS (+ per-sub-block sums)
-    if (sb0 > 0) lds_barrier();
+    if (sb0 > sb_begin) lds_barrier();
     float xscale = 1.0f, inv = 1.0f;  // true x = xscale * stored f16 x
     if constexpr (DT == KQ_BF16) {
       float amax = 0.f;
@@ -482,6 +487,22 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
 #pragma unroll
   for (int r = 0; r < R; r++) red[(wave * R + r) * 64 + lane] = acc[r];
   lds_barrier();
+  if constexpr (!GLU) {
+    if (a.ksplit > 1) {
+      // split-K: store this workgroup's partial sums; a second kernel adds the splits up in order
+      const size_t plane = (size_t)M * N;
+      for (int o = tid; o < R * 64; o += SK_THREADS) {
+        const int r = o >> 6, l = o & 63;
+        const int m = 4 * (l >> 5) + r, n = l & 31;
+        if (m >= M || n >= nrows) continue;
+        float v = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < SK_WAVES; wv++) v += red[(wv * R + r) * 64 + l];
+        a.partial[blockIdx.z * plane + (size_t)m * N + row0 + n] = v;
+      }
+      return;
+    }
+  }
   for (int o = tid; o < R * 64; o += SK_THREADS) {
     const int r = o >> 6, l = o & 63;
     const int m = 4 * (l >> 5) + r, n = l & 31;
@@ -500,6 +521,16 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
   }
 }
 
+template <int DT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, uint16_t* __restrict__ y,
+                                                            int count, int ksplit) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  float v = 0.f;
+  for (int sp = 0; sp < ksplit; sp++) v += partial[(size_t)sp * count + i];
+  y[i] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+}
+
 template <int C>
 size_t sk_lds_bytes(int rows, int kch, int MB) {
   using G = SkGeom<C>;
@@ -509,17 +540,48 @@ size_t sk_lds_bytes(int rows, int kch, int MB) {
          16 * SK_THREADS + 32 * 16 * 2;
 }
 
+// Split-K plan of a dense call: with few row tiles the K range is cut so that about 768
+// workgroups of full 32-row tiles exist; every split keeps at least one superblock per wave.
+struct SkSplit {
+  int ksplit, sb_per_split;
+};
+SkSplit sk_split_plan(int N, int K) {
+  const int nsb = K >> 8, tiles = (N + SK_MAXROWS - 1) / SK_MAXROWS;
+  SkSplit p{1, nsb};
+  if (tiles >= 384 || nsb < 8) return p;
+  int want = (768 + tiles - 1) / tiles;
+  if (want > nsb / 4) want = nsb / 4;
+  if (want < 2) return p;
+  int per = (nsb + want - 1) / want;
+  per = (per + 3) & ~3;  // whole sub-chunks
+  p.ksplit = (nsb + per - 1) / per;
+  p.sb_per_split = per;
+  if (p.ksplit < 2) return SkSplit{1, nsb};
+  return p;
+}
+
 template <int C, int DT, int MB, bool GLU>
-int launch_skinny(SkArgs a, int items, hipStream_t s) {
+int launch_skinny(SkArgs a, int items, void* ws, hipStream_t s) {
   // balanced row tiles: about two workgroups per CU over the whole launch, at most 32 rows each
   const int64_t total = (int64_t)a.N * items * (GLU ? 2 : 1);
   int rows = (int)((total + 511) / 512);
   rows = (rows + 7) & ~7;
   if (rows > SK_MAXROWS) rows = SK_MAXROWS;
   if (rows < 8) rows = 8;
+  int splits = 1;
+  a.ksplit = 1;
+  if (!GLU && items == 1 && ws) {
+    const SkSplit p = sk_split_plan(a.N, a.K);
+    if (p.ksplit > 1) {
+      rows = SK_MAXROWS;
+      splits = a.ksplit = p.ksplit;
+      a.sb_per_split = p.sb_per_split;
+      a.partial = static_cast<float*>(ws);
+    }
+  }
   const int half = GLU ? rows / 2 : rows;
   const int tiles = (a.N + half - 1) / half;
-  int kch = a.K >> 8;
+  int kch = splits > 1 ? a.sb_per_split : a.K >> 8;
   if (kch > 16) kch = 16;            // four sub-chunks of four superblocks
   if (kch * MB > 32) kch = 32 / MB;  // keep the f16 activations of a chunk within 16 KiB
   while (kch > 1 && sk_lds_bytes<C>(rows, kch, MB) > 76 * 1024) kch >>= 1;  // two workgroups per CU must fit in 160 KiB
@@ -533,30 +595,36 @@ int launch_skinny(SkArgs a, int items, hipStream_t s) {
                                      120 * 1024));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(tiles, items), dim3(SK_THREADS), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(tiles, items, splits), dim3(SK_THREADS), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
+  if (splits > 1) {
+    const int count = a.M * a.N;
+    hipLaunchKernelGGL((splitk_reduce_kernel<DT>), dim3((count + 255) / 256), dim3(256), 0, s, a.partial,
+                       static_cast<uint16_t*>(a.y), count, splits);
+    KQ_HIP_CHECK(hipGetLastError());
+  }
   return KQ_OK;
 }
 
 template <int C, int DT, bool GLU>
-int launch_skinny_m(const SkArgs& a, int items, hipStream_t s) {
-  if (a.M == 1) return launch_skinny<C, DT, 1, GLU>(a, items, s);
+int launch_skinny_m(const SkArgs& a, int items, void* ws, hipStream_t s) {
+  if (a.M == 1) return launch_skinny<C, DT, 1, GLU>(a, items, ws, s);
   if constexpr (GLU) {
     return KQ_ERR_UNSUPPORTED;
   } else {
-    if (a.M == 2) return launch_skinny<C, DT, 2, false>(a, items, s);
-    if (a.M <= 4) return launch_skinny<C, DT, 4, false>(a, items, s);
-    return launch_skinny<C, DT, 8, false>(a, items, s);
+    if (a.M == 2) return launch_skinny<C, DT, 2, false>(a, items, ws, s);
+    if (a.M <= 4) return launch_skinny<C, DT, 4, false>(a, items, ws, s);
+    return launch_skinny<C, DT, 8, false>(a, items, ws, s);
   }
 }
 
 template <bool GLU>
-int launch_skinny_any(const SkArgs& a, int items, int codec, int dtype, hipStream_t s) {
+int launch_skinny_any(const SkArgs& a, int items, int codec, int dtype, void* ws, hipStream_t s) {
   if (codec == KQ_Q4_K)
-    return dtype == KQ_F16 ? launch_skinny_m<KQ_Q4_K, KQ_F16, GLU>(a, items, s)
-                           : launch_skinny_m<KQ_Q4_K, KQ_BF16, GLU>(a, items, s);
-  return dtype == KQ_F16 ? launch_skinny_m<KQ_Q6_K, KQ_F16, GLU>(a, items, s)
-                         : launch_skinny_m<KQ_Q6_K, KQ_BF16, GLU>(a, items, s);
+    return dtype == KQ_F16 ? launch_skinny_m<KQ_Q4_K, KQ_F16, GLU>(a, items, ws, s)
+                           : launch_skinny_m<KQ_Q4_K, KQ_BF16, GLU>(a, items, ws, s);
+  return dtype == KQ_F16 ? launch_skinny_m<KQ_Q6_K, KQ_F16, GLU>(a, items, ws, s)
+                         : launch_skinny_m<KQ_Q6_K, KQ_BF16, GLU>(a, items, ws, s);
 }
 
 bool sk_shape_ok(int M, int K, int codec, const void* x, const void* w, const void* w2) {
@@ -569,8 +637,14 @@ bool sk_shape_ok(int M, int K, int codec, const void* x, const void* w, const vo
 
 }  // namespace
 
-int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
-                        hipStream_t s) {
+size_t kq_qmm_tuned_workspace_bytes(int M, int N, int K, int codec) {
+  if ((codec != KQ_Q4_K && codec != KQ_Q6_K) || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return 0;
+  const SkSplit p = sk_split_plan(N, K);
+  return p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
+}
+
+int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                        size_t ws_bytes, hipStream_t s) {
   if (!sk_shape_ok(M, K, codec, x, w, nullptr)) return KQ_ERR_UNSUPPORTED;
   SkArgs a{};
   a.x = x;
@@ -580,7 +654,8 @@ int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, 
   a.N = N;
   a.K = K;
   a.x_div = 1;
-  return launch_skinny_any<false>(a, 1, codec, dtype, s);
+  if (ws_bytes < kq_qmm_tuned_workspace_bytes(M, N, K, codec) || (reinterpret_cast<uintptr_t>(ws) & 3)) ws = nullptr;
+  return launch_skinny_any<false>(a, 1, codec, dtype, ws, s);
 }
 
 int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
@@ -606,5 +681,6 @@ int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, c
   a.x_batch_stride = x_batch_stride;
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
-  return glu ? launch_skinny_any<true>(a, B, codec, dtype, s) : launch_skinny_any<false>(a, B, codec, dtype, s);
+  return glu ? launch_skinny_any<true>(a, B, codec, dtype, nullptr, s)
+             : launch_skinny_any<false>(a, B, codec, dtype, nullptr, s);
 }
