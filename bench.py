@@ -178,6 +178,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-sweep", action="store_true", help="skip the sweep, prefill, MoE and low-bit sections")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--probe", action="store_true",
+                    help="counter probe for `rocprofv3 --pmc`: one device copy of the headline matrix (known bytes) "
+                         "followed by 20 cold launches of the headline GEMV, nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU.",
@@ -203,6 +206,17 @@ def main():
     copies = cold_copies(torch, base, wbytes)
     x = randx((M, K))
     calls = [abi.qmm(x, w, codec, N, K) for w in copies]
+    if args.probe:
+        dst = torch.empty_like(base)
+        torch.cuda.synchronize()
+        dst.copy_(copies[1])  # reference dispatch: reads and writes `wbytes` bytes
+        torch.cuda.synchronize()
+        for i in range(20):
+            calls[(i + 2) % len(calls)]()
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "copy then 20 cold GEMV launches", "copy_bytes_each_way": wbytes,
+                          "gemv_weight_bytes": wbytes}))
+        return
     ms, wall_ms = time_calls(torch, calls, args.steps, args.warmup)
     gbs = wbytes / (ms * 1e-3) / 1e9
     hot_ms, _ = time_calls(torch, calls[:1], args.steps, args.warmup)
