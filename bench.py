@@ -31,6 +31,10 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLC_BYTES = 256 << 20
+# HBM bytes one headline launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
+# `bench.py --probe`: (16237.4 KiB x 1.9983 + 28.0 KiB x 1.0), each counter scaled by what it reads for
+# the probe's plain 32256 KiB device copy.  Algorithmic bytes are 33,030,144 (weights) + 28,672 (output).
+HEADLINE_TRAFFIC_BYTES = 33_254_000
 KQ_BF16 = 2
 
 
@@ -233,7 +237,7 @@ def main():
         "hot_gbs": round(wbytes / (hot_ms * 1e-3) / 1e9, 1),
         "wall_ms_per_step": round(wall_ms, 6),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES},
     }
     base_np = base.cpu().numpy() if not args.no_cpu else None
     del copies, calls
