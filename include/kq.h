@@ -81,6 +81,10 @@ size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int 
 int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int transpose,
            int codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* Tuning hook without a counterpart in the reference: activation rows per workgroup tile of the
+ * prefill GEMM, 64 or 128 (anything else restores the default, 64).  Process-wide, not thread-safe. */
+void kq_set_gemm_tile_rows(int rows);
+
 /* out[b] = x[lhs[b]] . W[rhs[b]]^T for b < B; x batches are [M,K] matrices
  * `x_batch_stride` elements apart, experts are [N, bytes_per_row] wire matrices
  * `w_expert_stride_bytes` apart (64-bit, so strided / >2 GiB stacks work); out is

@@ -13,6 +13,8 @@
 // row-per-lane ds_read_b128 fragment fetch free of bank conflicts).
 #include "kq_mma.h"
 
+static int g_gemm_force_mt = 0;  // kq_set_gemm_tile_rows: 2 or 4 forces the tile height, 0 = default
+
 namespace {
 
 using namespace kqmma;
@@ -99,8 +101,6 @@ __global__ __launch_bounds__(PP_THREADS) void gemm_prepass_kernel(const uint16_t
 constexpr int GM_THREADS = 256;
 constexpr int BM = 128, BN = 128;
 constexpr int A_STRIDE = 512 + 16;  // bytes per activation row of one K step in LDS
-constexpr int A_BYTES = BM * A_STRIDE;
-constexpr int APT = BM * 32 / GM_THREADS;  // 16-byte activation pieces per thread per step (16)
 
 template <int C>
 struct WireGeom : Wire<C> {
@@ -108,25 +108,32 @@ struct WireGeom : Wire<C> {
   static constexpr int WPT = (BN * PPR + GM_THREADS - 1) / GM_THREADS;  // pieces per thread per step
 };
 
-template <int C, int DT>
-__global__ __launch_bounds__(GM_THREADS, 1) void kquant_gemm_kernel(const _Float16* __restrict__ xh,
+// MT = 32-row activation blocks per workgroup tile (tile = 32 MT rows x 128 columns).  MT = 4 runs one
+// workgroup per CU (one wave per SIMD) and is bound by LDS / MFMA latency it cannot hide; MT = 2 fits
+// two workgroups per CU and measured 17 - 38 % faster although each decoded fragment feeds only two
+// MFMAs (MT = 3 needs 256 registers and spills).
+template <int C, int DT, int MT>
+__global__ __launch_bounds__(GM_THREADS, MT == 4 ? 1 : 2) void kquant_gemm_kernel(const _Float16* __restrict__ xh,
                                                                     const _Float16* __restrict__ xhl,
                                                                     const float* __restrict__ rs,
                                                                     const uint8_t* __restrict__ w,
                                                                     uint16_t* __restrict__ y, int M, int N, int K,
                                                                     int mtiles) {
   using G = WireGeom<C>;
+  constexpr int TM = 32 * MT;                   // activation rows per tile
+  constexpr int A_BYTES = TM * A_STRIDE;
+  constexpr int APT = TM * 32 / GM_THREADS;     // 16-byte activation pieces per thread per step
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint8_t* a_lds = smem;                          // [BM][A_STRIDE]
+  uint8_t* a_lds = smem;                          // [TM][A_STRIDE]
   uint8_t* b_lds = smem + A_BYTES;                // [BN][LBPB]
-  uint8_t* h_lds = b_lds + BN * G::LBPB;          // [BM][32] X halves of the step
-  uint16_t* d_lds = reinterpret_cast<uint16_t*>(h_lds + BM * 32);  // [BN] side-channel d (q6_k)
+  uint8_t* h_lds = b_lds + BN * G::LBPB;          // [TM][32] X halves of the step
+  uint16_t* d_lds = reinterpret_cast<uint16_t*>(h_lds + TM * 32);  // [BN] side-channel d (q6_k)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, kg = lane >> 5;
   // consecutive workgroups share the weight columns (m fastest)
   const int mt = blockIdx.x % mtiles, nt = blockIdx.x / mtiles;
-  const int m0 = mt * BM, n0 = nt * BN;
+  const int m0 = mt * TM, n0 = nt * BN;
   const int nsb = K >> 8;
   const size_t row_bytes = (size_t)nsb * G::BPB;
   const int nrows = N - n0 < BN ? N - n0 : BN;
@@ -167,9 +174,9 @@ __global__ __launch_bounds__(GM_THREADS, 1) void kquant_gemm_kernel(const _Float
       wreg[T] = *reinterpret_cast<const typename G::piece_t*>(wtile + (size_t)sb * G::BPB + w_goff[T]);
     });
     if constexpr (G::SIDE_D) dreg = *reinterpret_cast<const uint16_t*>(d_src + (size_t)sb * G::BPB);
-    // X halves: 128 rows x 32 bytes = 256 pieces of 16 bytes
+    // X halves: TM rows x 32 bytes = 2 TM pieces of 16 bytes (threads past them re-read the first rows)
     if constexpr (G::MINS)
-      hreg = *reinterpret_cast<const u32x4*>(htile + ((size_t)(tid >> 1) * nsb + sb) * 16 + 8 * (tid & 1));
+      hreg = *reinterpret_cast<const u32x4*>(htile + ((size_t)((tid >> 1) < TM ? (tid >> 1) : 0) * nsb + sb) * 16 + 8 * (tid & 1));
   };
   auto park = [&]() {
     StaticFor<APT>::run([&](auto t) {
@@ -180,15 +187,17 @@ __global__ __launch_bounds__(GM_THREADS, 1) void kquant_gemm_kernel(const _Float
       constexpr int T = decltype(t)::value;
       if (w_loff[T] != 0xffffffffu) *reinterpret_cast<u32x4*>(b_lds + w_loff[T]) = wreg[T];
     });
-    if constexpr (G::MINS) *reinterpret_cast<u32x4*>(h_lds + 16 * tid) = hreg;
+    if constexpr (G::MINS) {
+      if (tid < 2 * TM) *reinterpret_cast<u32x4*>(h_lds + 16 * tid) = hreg;
+    }
     if constexpr (G::SIDE_D) {
       if (tid < BN) d_lds[tid] = dreg;
     }
   };
 
-  f32x16 acc[4];
+  f32x16 acc[MT];
 #pragma unroll
-  for (int t = 0; t < 4; t++) acc[t] = f32x16{0};
+  for (int t = 0; t < MT; t++) acc[t] = f32x16{0};
 
   const uint8_t* b_lane = b_lds + (wave * 32 + l32) * G::LBPB;
   const uint8_t* a_lane = a_lds + l32 * A_STRIDE + 32 * kg;
@@ -201,14 +210,14 @@ __global__ __launch_bounds__(GM_THREADS, 1) void kquant_gemm_kernel(const _Float
     if (sb + 1 < nsb) issue(sb + 1);
     lds_barrier();
 
-    superblock_mma<C, 4>(b_lane, G::SIDE_D ? d_lds[wave * 32 + l32] : (uint16_t)0, kg, a_lane, 32 * A_STRIDE, h_lane,
+    superblock_mma<C, MT>(b_lane, G::SIDE_D ? d_lds[wave * 32 + l32] : (uint16_t)0, kg, a_lane, 32 * A_STRIDE, h_lane,
                          32 * 32, acc);
   }
 
   // ---- epilogue: undo the per-row activation scale, round once, store
   const int n = n0 + wave * 32 + l32;
 #pragma unroll
-  for (int t = 0; t < 4; t++) {
+  for (int t = 0; t < MT; t++) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int m = m0 + t * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
@@ -220,19 +229,14 @@ __global__ __launch_bounds__(GM_THREADS, 1) void kquant_gemm_kernel(const _Float
   }
 }
 
-template <int C, int DT>
-int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, void* ws, hipStream_t s) {
+template <int C, int DT, int MT>
+int launch_gemm_mt(const _Float16* xh, const _Float16* xhl, const float* rs, const uint8_t* w, void* y, int M, int N,
+                   int K, hipStream_t s) {
   using G = WireGeom<C>;
-  const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-  const int mpad = mtiles * BM, nsb = K >> 8;
-  _Float16* xh = static_cast<_Float16*>(ws);
-  _Float16* xhl = xh + (size_t)mpad * K;
-  float* rs = reinterpret_cast<float*>(xhl + (size_t)mpad * nsb * 16);
-  hipLaunchKernelGGL((gemm_prepass_kernel<DT>), dim3(mpad), dim3(PP_THREADS), 0, s, static_cast<const uint16_t*>(x), xh,
-                     xhl, rs, M, K);
-  KQ_HIP_CHECK(hipGetLastError());
-  const size_t lds = A_BYTES + BN * G::LBPB + BM * 32 + BN * 2;
-  auto kern = kquant_gemm_kernel<C, DT>;
+  constexpr int TM = 32 * MT;
+  const int mtiles = (M + TM - 1) / TM, ntiles = (N + BN - 1) / BN;
+  const size_t lds = TM * A_STRIDE + BN * G::LBPB + TM * 32 + BN * 2;
+  auto kern = kquant_gemm_kernel<C, DT, MT>;
   static bool attr_set = false;
   if (!attr_set) {
     KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -243,6 +247,21 @@ int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, v
                      N, K, mtiles);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
+}
+
+
+template <int C, int DT>
+int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, void* ws, hipStream_t s) {
+  const int mpad = ((M + BM - 1) / BM) * BM, nsb = K >> 8;
+  _Float16* xh = static_cast<_Float16*>(ws);
+  _Float16* xhl = xh + (size_t)mpad * K;
+  float* rs = reinterpret_cast<float*>(xhl + (size_t)mpad * nsb * 16);
+  hipLaunchKernelGGL((gemm_prepass_kernel<DT>), dim3(mpad), dim3(PP_THREADS), 0, s, static_cast<const uint16_t*>(x), xh,
+                     xhl, rs, M, K);
+  KQ_HIP_CHECK(hipGetLastError());
+  const int mt = g_gemm_force_mt ? g_gemm_force_mt : 2;
+  if (mt == 4) return launch_gemm_mt<C, DT, 4>(xh, xhl, rs, w, y, M, N, K, s);
+  return launch_gemm_mt<C, DT, 2>(xh, xhl, rs, w, y, M, N, K, s);
 }
 
 }  // namespace
@@ -283,3 +302,5 @@ int kq_launch_act_prepass(const void* x, void* xh, void* xhl, float* rs, int M, 
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }
+
+extern "C" void kq_set_gemm_tile_rows(int rows) { g_gemm_force_mt = rows == 128 ? 4 : rows == 64 ? 2 : 0; }

@@ -103,60 +103,67 @@ __device__ __forceinline__ void superblock_mma(const uint8_t* __restrict__ b_lan
     const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
     const uint32_t scw[2] = {s0 & 0x3f3f3f3fu, (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)};
     const uint32_t mnw[2] = {s1 & 0x3f3f3f3fu, ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u)};
+    // 16 MFMA groups (sub-block j = it / 2, K-half s = it % 2).  The activation fragments of group
+    // it + 1 are requested before group it is decoded, so the LDS latency hides behind the decode
+    // and the MFMAs instead of stalling each group.
+    f16x8 afr[2][MT];
+    uint4 qv[4];
+    uint32_t hb[4] = {0, 0, 0, 0};  // q5_k: fifth bits of this lane's 16 weights, positioned per pair
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-      const uint4 qv = *reinterpret_cast<const uint4*>(b_lane + G::QS + 32 * g + 16 * kg);
-      const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
-      const uint32_t qw8[4] = {qw[0] >> 8, qw[1] >> 8, qw[2] >> 8, qw[3] >> 8};
-      uint32_t hb[4] = {0, 0, 0, 0};  // q5_k: fifth bits of this lane's 16 weights, positioned per pair
-      if constexpr (C == KQ_Q5_K) {
-        const uint4 hv = *reinterpret_cast<const uint4*>(b_lane + 16 + 16 * kg);
-        hb[0] = hv.x;
-        hb[1] = hv.y;
-        hb[2] = hv.z;
-        hb[3] = hv.w;
-      }
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const int j = 2 * g + h;
-        const float scf = (float)((scw[j >> 2] >> (8 * (j & 3))) & 0xff);
-        // low nibbles read 1024 + q, high nibbles (in place) 1024 + 16 q: fold the 16 into the scale
-        const _Float16 sch = (_Float16)(h ? scf * 0.0625f : scf);
-        const _Float16 off = (_Float16)(-(h ? 64.0f : 1024.0f) * scf);
-        const f16x2 scp = {sch, sch}, offp = {off, off};
-#pragma unroll
-        for (int s = 0; s < 2; s++) {
-          const uint32_t mask = h ? mask_hi : mask_lo;
-          uint32_t fr[4] = {(qw[2 * s] & mask) | magic, (qw8[2 * s] & mask) | magic, (qw[2 * s + 1] & mask) | magic,
-                            (qw8[2 * s + 1] & mask) | magic};
-          f16x2 bq[4];
-#pragma unroll
-          for (int e = 0; e < 4; e++)  // one rounding: (1024 + q) * sc - 1024 * sc = sc * q exactly
-            bq[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fr[e]), scp, offp);
-          if constexpr (C == KQ_Q5_K) {
-            // fifth bit of weight (j, i) is bit j of qh[i]; this lane's bytes are qh[16 kg + 8 s + 0..7]
-            const _Float16 s16 = (_Float16)(16.0f * scf);
-            const uint32_t hwa = hb[2 * s] >> j, hwb = hb[2 * s + 1] >> j;
-            const _Float16 z = (_Float16)0.f;
-            const f16x2 add[4] = {{(hwa & 1) ? s16 : z, (hwa & 0x10000) ? s16 : z},
-                                  {(hwa & 0x100) ? s16 : z, (hwa & 0x1000000) ? s16 : z},
-                                  {(hwb & 1) ? s16 : z, (hwb & 0x10000) ? s16 : z},
-                                  {(hwb & 0x100) ? s16 : z, (hwb & 0x1000000) ? s16 : z}};
-#pragma unroll
-            for (int e = 0; e < 4; e++) bq[e] += add[e];
-          }
-          const f16x8 b = {bq[0][0], bq[0][1], bq[1][0], bq[1][1], bq[2][0], bq[2][1], bq[3][0], bq[3][1]};
-#pragma unroll
-          for (int t = 0; t < MT; t++) {
-            const f16x8 a = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile + 64 * j + 16 * s);
-            if (j == 0 && s == 0)
-              part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, f32x16{0}, 0, 0, 0);
-            else
-              part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, part[t], 0, 0, 0);
-          }
-        }
-      }
+    for (int g = 0; g < 4; g++) qv[g] = *reinterpret_cast<const uint4*>(b_lane + G::QS + 32 * g + 16 * kg);
+    if constexpr (C == KQ_Q5_K) {
+      const uint4 hv = *reinterpret_cast<const uint4*>(b_lane + 16 + 16 * kg);
+      hb[0] = hv.x;
+      hb[1] = hv.y;
+      hb[2] = hv.z;
+      hb[3] = hv.w;
     }
+#pragma unroll
+    for (int t = 0; t < MT; t++) afr[0][t] = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile);
+    StaticFor<16>::run([&](auto itc) {
+      constexpr int it = decltype(itc)::value;
+      constexpr int j = it >> 1, s = it & 1, g = j >> 1, h = j & 1;
+      if constexpr (it + 1 < 16) {
+        constexpr int jn = (it + 1) >> 1, sn = (it + 1) & 1;
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+          afr[(it + 1) & 1][t] = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile + 64 * jn + 16 * sn);
+        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of this group's decode (the scheduler sinks them)
+      }
+      const uint32_t qw[4] = {qv[g].x, qv[g].y, qv[g].z, qv[g].w};
+      const float scf = (float)((scw[j >> 2] >> (8 * (j & 3))) & 0xff);
+      // low nibbles read 1024 + q, high nibbles (in place) 1024 + 16 q: fold the 16 into the scale
+      const _Float16 sch = (_Float16)(h ? scf * 0.0625f : scf);
+      const _Float16 off = (_Float16)(-(h ? 64.0f : 1024.0f) * scf);
+      const f16x2 scp = {sch, sch}, offp = {off, off};
+      const uint32_t mask = h ? mask_hi : mask_lo;
+      const uint32_t fr[4] = {(qw[2 * s] & mask) | magic, ((qw[2 * s] >> 8) & mask) | magic,
+                              (qw[2 * s + 1] & mask) | magic, ((qw[2 * s + 1] >> 8) & mask) | magic};
+      f16x2 bq[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++)  // one rounding: (1024 + q) * sc - 1024 * sc = sc * q exactly
+        bq[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fr[e]), scp, offp);
+      if constexpr (C == KQ_Q5_K) {
+        // fifth bit of weight (j, i) is bit j of qh[i]; this lane's bytes are qh[16 kg + 8 s + 0..7]
+        const _Float16 s16 = (_Float16)(16.0f * scf);
+        const uint32_t hwa = hb[2 * s] >> j, hwb = hb[2 * s + 1] >> j;
+        const _Float16 z = (_Float16)0.f;
+        const f16x2 add[4] = {{(hwa & 1) ? s16 : z, (hwa & 0x10000) ? s16 : z},
+                              {(hwa & 0x100) ? s16 : z, (hwa & 0x1000000) ? s16 : z},
+                              {(hwb & 1) ? s16 : z, (hwb & 0x10000) ? s16 : z},
+                              {(hwb & 0x100) ? s16 : z, (hwb & 0x1000000) ? s16 : z}};
+#pragma unroll
+        for (int e = 0; e < 4; e++) bq[e] += add[e];
+      }
+      const f16x8 b = {bq[0][0], bq[0][1], bq[1][0], bq[1][1], bq[2][0], bq[2][1], bq[3][0], bq[3][1]};
+#pragma unroll
+      for (int t = 0; t < MT; t++) {
+        if constexpr (it == 0)
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t], b, f32x16{0}, 0, 0, 0);
+        else
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[it & 1][t], b, part[t], 0, 0, 0);
+      }
+    });
 #pragma unroll
     for (int t = 0; t < MT; t++)
 #pragma unroll

@@ -128,6 +128,27 @@ def test_qmm_prefill_gemm(kq, codec, M, N, K):
         assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, N, K, dtype)
 
 
+def test_qmm_prefill_gemm_both_tile_heights(kq):
+    """The 128-row tile variant (kq_set_gemm_tile_rows) gives the same rounded outputs as the default 64-row one:
+    both feed the same exact products to f32 accumulators in the same order."""
+    M, N, K = 200, 384, 1024
+    lib = kq._load()
+    for codec in ("q4_k", "q5_k", "q6_k"):
+        wire = _wire(codec, N, K, seed=37)
+        xb, xt = make_x((M, K), "bfloat16", seed=38)
+        want = O.qmm(xb, wire, codec, True, "bfloat16")
+        outs = []
+        try:
+            for rows in (128, 64):
+                lib.kq_set_gemm_tile_rows(rows)
+                got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+                assert rel_l2(got, want, "bfloat16") <= TOL, (codec, rows)
+                outs.append(got)
+        finally:
+            lib.kq_set_gemm_tile_rows(0)
+        assert np.array_equal(outs[0], outs[1]), codec
+
+
 def test_qmm_prefill_gemm_wide_dynamic_range(kq):
     """bf16 activations spanning many binades and rows of very different scale: the per-row power-of-two
     scaling of the f16 conversion must keep every row within tolerance."""
