@@ -191,57 +191,66 @@ __device__ __forceinline__ void superblock_mma(const uint8_t* __restrict__ b_lan
     const uint32_t mask_q = opaque_sgpr(0x00f000f0u), mask_h = opaque_sgpr(0x03000300u);
     const uint4 scv = *reinterpret_cast<const uint4*>(b_lane + 192);
     const uint32_t scw[4] = {scv.x, scv.y, scv.z, scv.w};
+    // 16 groups in wire order: it = 8 hf + 4 qr + 2 h + s -> sub-block j = 4 hf + qr + 2 h, K-half s.
+    // The activation fragments of group it + 1 are requested before group it is decoded.
+    uint4 hv[2], qv[4];
 #pragma unroll
     for (int hf = 0; hf < 2; hf++) {
-      const uint4 hv = *reinterpret_cast<const uint4*>(b_lane + 128 + 32 * hf + 16 * kg);
-      const uint32_t hw[4] = {hv.x, hv.y, hv.z, hv.w};
+      hv[hf] = *reinterpret_cast<const uint4*>(b_lane + 128 + 32 * hf + 16 * kg);
 #pragma unroll
-      for (int qr = 0; qr < 2; qr++) {
-        const uint4 qv = *reinterpret_cast<const uint4*>(b_lane + 64 * hf + 32 * qr + 16 * kg);
-        const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          const int t4 = qr + 2 * h, j = 4 * hf + t4;
-          const int sc = __builtin_amdgcn_sbfe((int)scw[2 * hf + (t4 >> 1)], 8 * (2 * (t4 & 1) + kg), 8);
-          const float scf = (float)sc;
-          const _Float16 sch = (_Float16)(scf * 0.0625f), ofl = (_Float16)(-64.0f * scf),
-                         ofh = (_Float16)(-96.0f * scf);
-          const f16x2 scp = {sch, sch}, oflp = {ofl, ofl}, ofhp = {ofh, ofh};
-#pragma unroll
-          for (int s = 0; s < 2; s++) {
-            uint32_t fl[4], fh[4];
-#pragma unroll
-            for (int e = 0; e < 2; e++) {
-              const uint32_t q = qw[2 * s + e], hq = hw[2 * s + e];
-              const uint32_t qe = h ? q : (q << 4), qo = h ? (q >> 8) : (q >> 4);
-              const uint32_t he = hq << (8 - 2 * t4), ho = t4 ? (hq >> (2 * t4)) : hq;
-              fl[2 * e] = (qe & mask_q) | magic;      // bytes 0, 2 of the word: 1024 + 16 ql
-              fl[2 * e + 1] = (qo & mask_q) | magic;  // bytes 1, 3
-              fh[2 * e] = (he & mask_h) | magic;      // 1024 + 256 qh
-              fh[2 * e + 1] = (ho & mask_h) | magic;
-            }
-            f16x2 bl2[4], bh2[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              // (1024 + 16 ql) sc / 16 - 64 sc = sc ql;  (1024 + 256 qh) sc / 16 - 96 sc = 16 sc (qh - 2)
-              bl2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fl[e]), scp, oflp);
-              bh2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fh[e]), scp, ofhp);
-            }
-            const f16x8 blo = {bl2[0][0], bl2[0][1], bl2[1][0], bl2[1][1], bl2[2][0], bl2[2][1], bl2[3][0], bl2[3][1]};
-            const f16x8 bhi = {bh2[0][0], bh2[0][1], bh2[1][0], bh2[1][1], bh2[2][0], bh2[2][1], bh2[3][0], bh2[3][1]};
-#pragma unroll
-            for (int t = 0; t < MT; t++) {
-              const f16x8 a = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile + 64 * j + 16 * s);
-              if (j == 0 && s == 0)
-                part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, blo, f32x16{0}, 0, 0, 0);
-              else
-                part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, blo, part[t], 0, 0, 0);
-              part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bhi, part[t], 0, 0, 0);
-            }
-          }
-        }
-      }
+      for (int qr = 0; qr < 2; qr++)
+        qv[2 * hf + qr] = *reinterpret_cast<const uint4*>(b_lane + 64 * hf + 32 * qr + 16 * kg);
     }
+    f16x8 afr[2][MT];
+#pragma unroll
+    for (int t = 0; t < MT; t++) afr[0][t] = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile);
+    StaticFor<16>::run([&](auto itc) {
+      constexpr int it = decltype(itc)::value;
+      constexpr int hf = it >> 3, qr = (it >> 2) & 1, h = (it >> 1) & 1, s = it & 1;
+      constexpr int t4 = qr + 2 * h, j = 4 * hf + t4;
+      if constexpr (it + 1 < 16) {
+        constexpr int n = it + 1;
+        constexpr int jn = 4 * (n >> 3) + ((n >> 2) & 1) + 2 * ((n >> 1) & 1), sn = n & 1;
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+          afr[n & 1][t] = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile + 64 * jn + 16 * sn);
+        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of this group's decode
+      }
+      const uint32_t hw[4] = {hv[hf].x, hv[hf].y, hv[hf].z, hv[hf].w};
+      const uint32_t qw[4] = {qv[2 * hf + qr].x, qv[2 * hf + qr].y, qv[2 * hf + qr].z, qv[2 * hf + qr].w};
+      const int sc = __builtin_amdgcn_sbfe((int)scw[2 * hf + (t4 >> 1)], 8 * (2 * (t4 & 1) + kg), 8);
+      const float scf = (float)sc;
+      const _Float16 sch = (_Float16)(scf * 0.0625f), ofl = (_Float16)(-64.0f * scf), ofh = (_Float16)(-96.0f * scf);
+      const f16x2 scp = {sch, sch}, oflp = {ofl, ofl}, ofhp = {ofh, ofh};
+      uint32_t fl[4], fh[4];
+#pragma unroll
+      for (int e = 0; e < 2; e++) {
+        const uint32_t q = qw[2 * s + e], hq = hw[2 * s + e];
+        const uint32_t qe = h ? q : (q << 4), qo = h ? (q >> 8) : (q >> 4);
+        const uint32_t he = hq << (8 - 2 * t4), ho = t4 ? (hq >> (2 * t4)) : hq;
+        fl[2 * e] = (qe & mask_q) | magic;      // bytes 0, 2 of the word: 1024 + 16 ql
+        fl[2 * e + 1] = (qo & mask_q) | magic;  // bytes 1, 3
+        fh[2 * e] = (he & mask_h) | magic;      // 1024 + 256 qh
+        fh[2 * e + 1] = (ho & mask_h) | magic;
+      }
+      f16x2 bl2[4], bh2[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        // (1024 + 16 ql) sc / 16 - 64 sc = sc ql;  (1024 + 256 qh) sc / 16 - 96 sc = 16 sc (qh - 2)
+        bl2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fl[e]), scp, oflp);
+        bh2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fh[e]), scp, ofhp);
+      }
+      const f16x8 blo = {bl2[0][0], bl2[0][1], bl2[1][0], bl2[1][1], bl2[2][0], bl2[2][1], bl2[3][0], bl2[3][1]};
+      const f16x8 bhi = {bh2[0][0], bh2[0][1], bh2[1][0], bh2[1][1], bh2[2][0], bh2[2][1], bh2[3][0], bh2[3][1]};
+#pragma unroll
+      for (int t = 0; t < MT; t++) {
+        if constexpr (it == 0)
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t], blo, f32x16{0}, 0, 0, 0);
+        else
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[it & 1][t], blo, part[t], 0, 0, 0);
+        part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[it & 1][t], bhi, part[t], 0, 0, 0);
+      }
+    });
     const float d = kq::h2f(d_side);
 #pragma unroll
     for (int t = 0; t < MT; t++)
