@@ -26,7 +26,7 @@ SOURCES = [
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
     # packed-FP32 VALU forms are kept out of the generated code on purpose
-    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-fno-strict-aliasing",
     "-I", os.path.join(ROOT, "include"), "-I", CSRC, '-DKQ_GRID_BLOB="%s"' % BLOB,
 ]
 

@@ -207,7 +207,7 @@ __device__ __forceinline__ void superblock_mma(const uint8_t* __restrict__ b_lan
     StaticFor<16>::run([&](auto itc) {
       constexpr int it = decltype(itc)::value;
       constexpr int hf = it >> 3, qr = (it >> 2) & 1, h = (it >> 1) & 1, s = it & 1;
-      constexpr int t4 = qr + 2 * h, j = 4 * hf + t4;
+      constexpr int t4 = qr + 2 * h;
       if constexpr (it + 1 < 16) {
         constexpr int n = it + 1;
         constexpr int jn = 4 * (n >> 3) + ((n >> 2) & 1) + 2 * ((n >> 1) & 1), sn = n & 1;

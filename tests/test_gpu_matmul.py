@@ -59,6 +59,22 @@ def test_qmm_skinny_ragged_shapes(kq, codec, M, N, K):
         assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, N, K, dtype)
 
 
+@pytest.mark.parametrize("codec", ["mxfp4", "q8_0", "q2_k", "iq2_xxs", "q5_0"])
+def test_qmm_gemv_unaligned_rows_and_tensor_end(kq, codec):
+    """Rows that start at odd byte addresses (17 / 34 / 22-byte blocks, a view 1 byte into an allocation) and
+    a last row that ends exactly where the allocation ends."""
+    wpb, bpb = O.geometry(codec)
+    N, K, M = 37, 5 * wpb, 3
+    wire = _wire(codec, N, K, seed=39)
+    buf = torch.zeros(wire.size + 1, dtype=torch.uint8, device="cuda:0")
+    view = buf[1:].view(N, -1)
+    view.copy_(wire_to_dev(wire))
+    xb, xt = make_x((M, K), "float16", seed=40)
+    got = kq.quantized_matmul(xt, view, None, codec)
+    want = O.qmm(xb, wire, codec, True, "float16")
+    assert rel_l2(dev_to_bits(got), want, "float16") <= TOL
+
+
 def test_qmm_skinny_unaligned_q6k_rows(kq):
     """q6_k rows are 210-byte multiples: a wire view that starts 2 bytes into an allocation still decodes."""
     N, K, M = 64, 768, 1
