@@ -97,6 +97,12 @@ struct SkGeom<KQ_Q4_K> {
   typedef u32x4 piece_t;
 };
 template <>
+struct SkGeom<KQ_Q5_K> {
+  static constexpr int BPB = 176, LBPB = 176, PP = 11;
+  static constexpr bool SIDE_D = false, XSUM = true;
+  typedef u32x4 piece_t;
+};
+template <>
 struct SkGeom<KQ_Q6_K> {
   static constexpr int BPB = 210, LBPB = 208, PP = 13;
   static constexpr bool SIDE_D = true, XSUM = false;
@@ -139,22 +145,34 @@ __device__ __forceinline__ f16x8 q4k_frag(uint32_t wa, uint32_t wa8, uint32_t wb
   return __builtin_bit_cast(f16x8, v);
 }
 
-// One superblock of one 32-row tile: 16 MFMAs + the f32 fix-up on R accumulator registers.
-// bl: this lane's row of the superblock in LDS; xs_lane: this lane's A-fragment base (f16
-// index) for the superblock; xsum: X_j for the superblock, [8][XS] floats.
-template <int R, int XS>
-__device__ __forceinline__ void q4k_superblock(const uint8_t* __restrict__ bl, int kg, float xscale,
-                                               const _Float16* __restrict__ xs_lane,
-                                               const float* __restrict__ xsum, float* acc) {
+// One superblock of one 32-row tile (q4_k / q5_k): 16 MFMAs + the f32 fix-up on R accumulator
+// registers.  bl: this lane's row of the superblock in LDS; xs_lane: this lane's A-fragment base
+// (f16 index) for the superblock; xsum: X_j for the superblock, [8][XS] floats.
+// q5_k: the fifth bit of weight (sub-block j, i) is bit j of qh[i]; it is OR-ed into the code at
+// bit 4 (low-nibble sub-blocks, 1024 + q) or bit 8 (high-nibble ones, 1024 + 16 q).
+template <int C, int R, int XS>
+__device__ __forceinline__ void q45k_superblock(const uint8_t* __restrict__ bl, int kg, float xscale,
+                                                const _Float16* __restrict__ xs_lane,
+                                                const float* __restrict__ xsum, float* acc) {
+  constexpr int QS = C == KQ_Q4_K ? 16 : 48;  // offset of the nibble array
   Q4kRaw raw;
   const uint4* p4 = reinterpret_cast<const uint4*>(bl);
   raw.hdr = p4[0];
 #pragma unroll
-  for (int g = 0; g < 4; g++) raw.q[g] = p4[1 + 2 * g + kg];
+  for (int g = 0; g < 4; g++) raw.q[g] = *reinterpret_cast<const uint4*>(bl + QS + 32 * g + 16 * kg);
+  uint32_t hw[4] = {0, 0, 0, 0};
+  if constexpr (C == KQ_Q5_K) {
+    const uint4 hv = p4[1 + kg];  // qh[16 kg .. 16 kg + 15]
+    hw[0] = hv.x;
+    hw[1] = hv.y;
+    hw[2] = hv.z;
+    hw[3] = hv.w;
+  }
   float mul[8], sub[8];
   q4k_scales(raw.hdr, xscale, mul, sub);
   const uint32_t magic = kq_opaque_vgpr(0x64006400u);
   const uint32_t mask_lo = kq_opaque_sgpr(0x000f000fu), mask_hi = kq_opaque_sgpr(0x00f000f0u);
+  const uint32_t bit_lo = kq_opaque_sgpr(0x00100010u), bit_hi = kq_opaque_sgpr(0x01000100u);
 #pragma unroll
   for (int g = 0; g < 4; g++) {
     const uint32_t qw[4] = {raw.q[g].x, raw.q[g].y, raw.q[g].z, raw.q[g].w};
@@ -166,8 +184,23 @@ __device__ __forceinline__ void q4k_superblock(const uint8_t* __restrict__ bl, i
 #pragma unroll
       for (int s = 0; s < 2; s++) {
         const f16x8 a = *reinterpret_cast<const f16x8*>(xs_lane + 32 * j + 8 * s);
-        const f16x8 b = q4k_frag(qw[2 * s], qw8[2 * s], qw[2 * s + 1], qw8[2 * s + 1],
-                                 h ? mask_hi : mask_lo, magic);
+        f16x8 b = q4k_frag(qw[2 * s], qw8[2 * s], qw[2 * s + 1], qw8[2 * s + 1], h ? mask_hi : mask_lo, magic);
+        if constexpr (C == KQ_Q5_K) {
+          // even bytes of a qh word (bits j, 16 + j) go to bits 4 / 20 (h = 0) or 8 / 24 (h = 1) of the
+          // fragment word, odd bytes (bits 8 + j, 24 + j) likewise
+          const int tgt = h ? 8 : 4;
+          const uint32_t bm = h ? bit_hi : bit_lo;
+          uint4 v = __builtin_bit_cast(uint4, b);
+          const uint32_t ha = hw[2 * s], hb = hw[2 * s + 1];
+          const uint32_t ea = tgt >= j ? (ha << (tgt - j)) : (ha >> (j - tgt));
+          const uint32_t eb = tgt >= j ? (hb << (tgt - j)) : (hb >> (j - tgt));
+          const uint32_t oa = ha >> (8 + j - tgt), ob = hb >> (8 + j - tgt);
+          v.x = and_or(ea, bm, kq_opaque_vgpr(v.x));
+          v.y = and_or(oa, bm, kq_opaque_vgpr(v.y));
+          v.z = and_or(eb, bm, kq_opaque_vgpr(v.z));
+          v.w = and_or(ob, bm, kq_opaque_vgpr(v.w));
+          b = __builtin_bit_cast(f16x8, v);
+        }
         p = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, p, 0, 0, 0);
       }
 #pragma unroll
@@ -472,8 +505,9 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
         lds_barrier();
         const int sb = SBC * c + wave;
         if (sb < sbn) {
-          if constexpr (C == KQ_Q4_K) {
-            q4k_superblock<R, MB>(wt_lane + sb * G::LBPB, kg, xscale, xs_lane + 256 * sb, xsum_lane + 8 * MB * sb, acc);
+          if constexpr (C == KQ_Q4_K || C == KQ_Q5_K) {
+            q45k_superblock<C, R, MB>(wt_lane + sb * G::LBPB, kg, xscale, xs_lane + 256 * sb, xsum_lane + 8 * MB * sb,
+                                      acc);
           } else {
             const float dx = kq::h2f(dq[crow * 16 + sb]) * xscale;
             q6k_superblock<R>(wt_lane + sb * G::LBPB, kg, dx, xs_lane + 256 * sb, acc);
@@ -623,14 +657,19 @@ int launch_skinny_any(const SkArgs& a, int items, int codec, int dtype, void* ws
   if (codec == KQ_Q4_K)
     return dtype == KQ_F16 ? launch_skinny_m<KQ_Q4_K, KQ_F16, GLU>(a, items, ws, s)
                            : launch_skinny_m<KQ_Q4_K, KQ_BF16, GLU>(a, items, ws, s);
+  if (codec == KQ_Q5_K)
+    return dtype == KQ_F16 ? launch_skinny_m<KQ_Q5_K, KQ_F16, GLU>(a, items, ws, s)
+                           : launch_skinny_m<KQ_Q5_K, KQ_BF16, GLU>(a, items, ws, s);
   return dtype == KQ_F16 ? launch_skinny_m<KQ_Q6_K, KQ_F16, GLU>(a, items, ws, s)
                          : launch_skinny_m<KQ_Q6_K, KQ_BF16, GLU>(a, items, ws, s);
 }
 
+bool sk_codec_ok(int codec) { return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K; }
+
 bool sk_shape_ok(int M, int K, int codec, const void* x, const void* w, const void* w2) {
-  if ((codec != KQ_Q4_K && codec != KQ_Q6_K) || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return false;
-  // q4_k pieces are fetched with aligned 16-byte loads; q6_k blocks need 2-byte alignment only
-  const uintptr_t wmask = codec == KQ_Q4_K ? 15 : 1;
+  if (!sk_codec_ok(codec) || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return false;
+  // q4_k / q5_k pieces are fetched with aligned 16-byte loads; q6_k blocks need 2-byte alignment only
+  const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;
   if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask)) return false;
   return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 }
@@ -638,7 +677,7 @@ bool sk_shape_ok(int M, int K, int codec, const void* x, const void* w, const vo
 }  // namespace
 
 size_t kq_qmm_tuned_workspace_bytes(int M, int N, int K, int codec) {
-  if ((codec != KQ_Q4_K && codec != KQ_Q6_K) || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return 0;
+  if (!sk_codec_ok(codec) || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return 0;
   const SkSplit p = sk_split_plan(N, K);
   return p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
 }
@@ -664,7 +703,7 @@ int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, c
                            int dtype, hipStream_t s) {
   if (!sk_shape_ok(M, K, codec, x, w, w2) || B < 1 || B > 65535) return KQ_ERR_UNSUPPORTED;
   if (glu && (M != 1 || act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
-  const int64_t wmask = codec == KQ_Q4_K ? 15 : 1;
+  const int64_t wmask = codec == KQ_Q6_K ? 1 : 15;
   if ((w_expert_stride & wmask) || ((x_batch_stride * 2) & 15)) return KQ_ERR_UNSUPPORTED;
   SkArgs a{};
   a.x = x;
