@@ -90,22 +90,39 @@ __device__ __forceinline__ uint32_t kq_opaque_sgpr(uint32_t v) {
 // bytes apart, so that every block starts 16-byte aligned there.
 template <int C>
 struct SkGeom;
+// TAIL: the block's last 16 bytes [BPB - 16, BPB) travel as one extra piece and are parked at
+// LDS offset 16 PP of the block (q2_k: d / dmin, q3_k: scales + d).  XSUM: granularity of the
+// activation sums kept in LDS (0 = none).  KGOFF: consecutive weights a lane owns inside each
+// 32-weight sub-block half -- 16 (lane kg takes weights 16 kg .. 16 kg + 15 of the sub-block) or 8
+// (weights 8 kg .. 8 kg + 7 of each 16-weight scale group, so one MFMA covers one scale group).
 template <>
 struct SkGeom<KQ_Q4_K> {
-  static constexpr int BPB = 144, LBPB = 144, PP = 9;
-  static constexpr bool SIDE_D = false, XSUM = true;
+  static constexpr int BPB = 144, LBPB = 144, PP = 9, XSUM = 32, KGOFF = 16;
+  static constexpr bool SIDE_D = false, TAIL = false;
   typedef u32x4 piece_t;
 };
 template <>
 struct SkGeom<KQ_Q5_K> {
-  static constexpr int BPB = 176, LBPB = 176, PP = 11;
-  static constexpr bool SIDE_D = false, XSUM = true;
+  static constexpr int BPB = 176, LBPB = 176, PP = 11, XSUM = 32, KGOFF = 16;
+  static constexpr bool SIDE_D = false, TAIL = false;
   typedef u32x4 piece_t;
 };
 template <>
 struct SkGeom<KQ_Q6_K> {
-  static constexpr int BPB = 210, LBPB = 208, PP = 13;
-  static constexpr bool SIDE_D = true, XSUM = false;
+  static constexpr int BPB = 210, LBPB = 208, PP = 13, XSUM = 0, KGOFF = 16;
+  static constexpr bool SIDE_D = true, TAIL = false;
+  typedef u32x4_a2 piece_t;
+};
+template <>
+struct SkGeom<KQ_Q2_K> {  // LDS block: scales[16] | qs[64] | tail (wire bytes 68..83: d at +12, dmin at +14) | pad
+  static constexpr int BPB = 84, LBPB = 112, PP = 5, XSUM = 16, KGOFF = 8;
+  static constexpr bool SIDE_D = false, TAIL = true;
+  typedef u32x4_a2 piece_t;
+};
+template <>
+struct SkGeom<KQ_Q3_K> {  // LDS block: hmask[32] | qs[64] | tail (wire bytes 94..109: scales at +2, d at +14)
+  static constexpr int BPB = 110, LBPB = 112, PP = 6, XSUM = 16, KGOFF = 8;
+  static constexpr bool SIDE_D = false, TAIL = true;
   typedef u32x4_a2 piece_t;
 };
 
@@ -207,6 +224,108 @@ __device__ __forceinline__ void q45k_superblock(const uint8_t* __restrict__ bl, 
       for (int r = 0; r < R; r++) {
         acc[r] = fmaf(mul[j], p[r], acc[r]);
         acc[r] = fmaf(-sub[j], xsum[j * XS + r], acc[r]);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------ q2_k / q3_k superblocks
+// Weight 128 half + 32 si + l (l = 0..31) is the 2-bit field si of qs[32 half + l]; its scale group is
+// 8 half + 2 si + l / 16.  Lane (row, kg) owns l = 16 s + 8 kg .. + 7 of MFMA s, so every MFMA covers
+// exactly one scale group and is folded with that group's scale.  The field is masked in place and
+// reads 1024 + 4^si q; the 4^si goes into the scale.
+template <int R, int XS>
+__device__ __forceinline__ void q2k_superblock(const uint8_t* __restrict__ bl, int kg, float xscale,
+                                               const _Float16* __restrict__ xs_lane,
+                                               const float* __restrict__ xsum, float* acc) {
+  const uint32_t magic = kq_opaque_vgpr(0x64006400u);
+  const uint32_t mask[4] = {kq_opaque_sgpr(0x00030003u), kq_opaque_sgpr(0x000c000cu), kq_opaque_sgpr(0x00300030u),
+                            kq_opaque_sgpr(0x00c000c0u)};
+  const uint4 scv = *reinterpret_cast<const uint4*>(bl);
+  const uint32_t scw[4] = {scv.x, scv.y, scv.z, scv.w};
+  const uint32_t dm = *reinterpret_cast<const uint32_t*>(bl + 80 + 12);
+  const float d = kq::h2f((uint16_t)(dm & 0xffff)) * xscale, dmin = kq::h2f((uint16_t)(dm >> 16)) * xscale;
+#pragma unroll
+  for (int half = 0; half < 2; half++) {
+    const uint2 q0 = *reinterpret_cast<const uint2*>(bl + 16 + 32 * half + 8 * kg);
+    const uint2 q1 = *reinterpret_cast<const uint2*>(bl + 32 + 32 * half + 8 * kg);
+    const uint32_t qv[2][4] = {{q0.x, q0.x >> 8, q0.y, q0.y >> 8}, {q1.x, q1.x >> 8, q1.y, q1.y >> 8}};
+#pragma unroll
+    for (int si = 0; si < 4; si++) {
+      const int j = 4 * half + si;
+#pragma unroll
+      for (int s = 0; s < 2; s++) {
+        const int g = 8 * half + 2 * si + s;
+        const uint32_t scb = (scw[g >> 2] >> (8 * (g & 3))) & 0xff;
+        uint4 v;
+        v.x = and_or(qv[s][0], mask[si], magic);
+        v.y = and_or(qv[s][1], mask[si], magic);
+        v.z = and_or(qv[s][2], mask[si], magic);
+        v.w = and_or(qv[s][3], mask[si], magic);
+        const f16x8 a = *reinterpret_cast<const f16x8*>(xs_lane + 32 * j + 16 * s);
+        const f32x16 p = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, __builtin_bit_cast(f16x8, v), f32x16{0}, 0, 0, 0);
+        const float mulg = d * (float)(scb & 15) * (1.0f / (float)(1 << (2 * si)));
+        const float subg = fmaf(mulg, 1024.0f, dmin * (float)(scb >> 4));
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          acc[r] = fmaf(mulg, p[r], acc[r]);
+          acc[r] = fmaf(-subg, xsum[g * XS + r], acc[r]);
+        }
+      }
+    }
+  }
+}
+
+// q3_k: same 2-bit fields plus the high bit (bit 4 half + si of hmask[l], set = +4): the code is
+// 1024 + 4^si (q + 4 h) with zero point 4, scale d (sc - 32), sc the 6-bit scale of the group.
+template <int R, int XS>
+__device__ __forceinline__ void q3k_superblock(const uint8_t* __restrict__ bl, int kg, float xscale,
+                                               const _Float16* __restrict__ xs_lane,
+                                               const float* __restrict__ xsum, float* acc) {
+  const uint32_t magic = kq_opaque_vgpr(0x64006400u);
+  const uint32_t mask[4] = {kq_opaque_sgpr(0x00030003u), kq_opaque_sgpr(0x000c000cu), kq_opaque_sgpr(0x00300030u),
+                            kq_opaque_sgpr(0x00c000c0u)};
+  const uint32_t hmask[4] = {kq_opaque_sgpr(0x00040004u), kq_opaque_sgpr(0x00100010u), kq_opaque_sgpr(0x00400040u),
+                             kq_opaque_sgpr(0x01000100u)};
+  const uint4 tl = *reinterpret_cast<const uint4*>(bl + 96);  // wire bytes 94..109
+  // 12 scale bytes start at tail byte 2
+  const uint32_t s0 = __builtin_amdgcn_alignbyte(tl.y, tl.x, 2), s1 = __builtin_amdgcn_alignbyte(tl.z, tl.y, 2),
+                 s2 = __builtin_amdgcn_alignbyte(tl.w, tl.z, 2);
+  const float d = kq::h2f((uint16_t)(tl.w >> 16)) * xscale;
+  const uint2 h0 = *reinterpret_cast<const uint2*>(bl + 8 * kg);
+  const uint2 h1 = *reinterpret_cast<const uint2*>(bl + 16 + 8 * kg);
+  const uint32_t hv[2][4] = {{h0.x, h0.x >> 8, h0.y, h0.y >> 8}, {h1.x, h1.x >> 8, h1.y, h1.y >> 8}};
+#pragma unroll
+  for (int half = 0; half < 2; half++) {
+    const uint2 q0 = *reinterpret_cast<const uint2*>(bl + 32 + 32 * half + 8 * kg);
+    const uint2 q1 = *reinterpret_cast<const uint2*>(bl + 48 + 32 * half + 8 * kg);
+    const uint32_t qv[2][4] = {{q0.x, q0.x >> 8, q0.y, q0.y >> 8}, {q1.x, q1.x >> 8, q1.y, q1.y >> 8}};
+#pragma unroll
+    for (int si = 0; si < 4; si++) {
+      const int j = 4 * half + si;
+      const int sh = si + 2 - 4 * half;  // hmask bit 4 half + si -> code bit 2 si + 2
+#pragma unroll
+      for (int s = 0; s < 2; s++) {
+        const int g = 8 * half + 2 * si + s, k = g & 3, grp = g >> 2;
+        uint32_t lo4 = ((grp & 1) ? s1 : s0) >> (8 * k);
+        lo4 = (grp & 2) ? ((lo4 >> 4) & 15) : (lo4 & 15);
+        const uint32_t sc = lo4 | (((s2 >> (8 * k + 2 * grp)) & 3) << 4);
+        uint32_t fr[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const uint32_t hb = sh >= 0 ? (hv[s][e] << (sh >= 0 ? sh : 0)) : (hv[s][e] >> (sh < 0 ? -sh : 0));
+          fr[e] = and_or(hb, hmask[si], kq_opaque_vgpr(and_or(qv[s][e], mask[si], magic)));
+        }
+        const uint4 v = make_uint4(fr[0], fr[1], fr[2], fr[3]);
+        const f16x8 a = *reinterpret_cast<const f16x8*>(xs_lane + 32 * j + 16 * s);
+        const f32x16 p = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, __builtin_bit_cast(f16x8, v), f32x16{0}, 0, 0, 0);
+        const float mulg = d * (float)((int)sc - 32) * (1.0f / (float)(1 << (2 * si)));
+        const float subg = mulg * (1024.0f + (float)(4 << (2 * si)));
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          acc[r] = fmaf(mulg, p[r], acc[r]);
+          acc[r] = fmaf(-subg, xsum[g * XS + r], acc[r]);
+        }
       }
     }
   }
@@ -315,11 +434,11 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int M = a.M, N = a.N, K = a.K, rows_per_tile = a.rows_per_tile, kch = a.kch;
   // layout: wt [rows_per_tile][wstride] | xs f16 [MB][kch*256] | xsum f32 [kch*8][MB] | red | scratch | dump | dq
-  const int wstride = kch * G::LBPB + (((kch * G::PP) & 1) ? 0 : 16), kchunk = kch * 256;
+  const int wstride = kch * G::LBPB + (((kch * (G::LBPB / 16)) & 1) ? 0 : 16), kchunk = kch * 256;
   uint8_t* wt = smem;
   _Float16* xs = reinterpret_cast<_Float16*>(smem + rows_per_tile * wstride);
   float* xsum = reinterpret_cast<float*>(smem + rows_per_tile * wstride + (size_t)MB * kchunk * 2);
-  float* red = xsum + kch * 8 * MB;
+  float* red = xsum + kch * 16 * MB;
   float* scratch = red + SK_WAVES * R * 64;
   uint8_t* dump = reinterpret_cast<uint8_t*>(scratch + 16) + 16 * threadIdx.x;  // per-thread 16-byte dump slot
   uint16_t* dq = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(scratch + 16) + 16 * SK_THREADS);  // [32][16]
@@ -376,6 +495,10 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
   const int d_srow = d_up ? d_row - half : d_row;
   const bool d_ok = G::SIDE_D && d_row < rows_per_tile && d_srow < nrows;
   const uint8_t* d_src = (d_up ? wtile2 : wtile) + (d_ok ? (size_t)d_srow * row_bytes : 0) + 208;
+  // tail piece (last 16 bytes of a block), same thread -> (row, superblock) map
+  const bool t_ok = G::TAIL && d_row < rows_per_tile && d_srow < nrows;
+  const uint8_t* t_src = (d_up ? wtile2 : wtile) + (t_ok ? (size_t)d_srow * row_bytes : 0) + (G::BPB - 16);
+  uint8_t* t_dst = wt + d_row * wstride + d_sbl * G::LBPB + 16 * G::PP;
 
   const int sb_begin = a.ksplit > 1 ? (int)blockIdx.z * a.sb_per_split : 0;
   const int sb_end = a.ksplit > 1 ? (sb_begin + a.sb_per_split < nsb ? sb_begin + a.sb_per_split : nsb) : nsb;
@@ -403,7 +526,7 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
     // pieces outside the tile or a ragged last sub-chunk re-read the tile's first bytes and
     // land in a dump slot.  Two sub-chunks are in flight at any time (register sets c % 2); the
     // next one is issued as soon as its register set has been parked in LDS.
-    u32x4 wreg[2 * PPC];
+    u32x4 wreg[2 * PPC], treg[2];
     uint16_t dreg[2];
     auto issue = [&](auto cc) {
       constexpr int c = decltype(cc)::value;
@@ -418,6 +541,10 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
       if constexpr (G::SIDE_D) {
         const bool ok = d_ok && d_sbl < sbc;
         dreg[c & 1] = *reinterpret_cast<const uint16_t*>(ok ? d_src + sboff + d_sbl * G::BPB : wtile);
+      }
+      if constexpr (G::TAIL) {
+        const bool ok = t_ok && d_sbl < sbc;
+        treg[c & 1] = *reinterpret_cast<const u32x4_a2*>(ok ? t_src + sboff + d_sbl * G::BPB : wtile);
       }
     };
     issue(std::integral_constant<int, 0>{});
@@ -471,20 +598,24 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
         // MFMA fragment order inside an 8-group: k0 k2 k1 k3 k4 k6 k5 k7
         const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
         *reinterpret_cast<f16x8*>(xs + (size_t)m * kchunk + kk) = v8;
-        if constexpr (G::XSUM) {
+        if constexpr (G::XSUM != 0) {
           float sum = 0.f;
 #pragma unroll
           for (int e = 0; e < 8; e++) sum += (float)h[e];
-          sum += __shfl_xor(sum, 1);  // 4 threads cover one 32-wide sub-block
-          sum += __shfl_xor(sum, 2);
-          if ((tid & 3) == 0) xsum[(kk >> 5) * MB + m] = sum;
+          sum += __shfl_xor(sum, 1);  // 2 threads cover a 16-wide scale group, 4 a 32-wide sub-block
+          if constexpr (G::XSUM == 32) {
+            sum += __shfl_xor(sum, 2);
+            if ((tid & 3) == 0) xsum[(kk >> 5) * MB + m] = sum;
+          } else {
+            if ((tid & 1) == 0) xsum[(kk >> 4) * MB + m] = sum;
+          }
         }
       }
     });
 
     // ---- 4. sub-chunk by sub-chunk: park the arrived bytes in LDS, then one superblock per wave
     // while the later sub-chunks are still streaming in
-    const _Float16* xs_lane = xs + (size_t)(n_in & (MB - 1)) * kchunk + 16 * kg;
+    const _Float16* xs_lane = xs + (size_t)(n_in & (MB - 1)) * kchunk + G::KGOFF * kg;
     const float* xsum_lane = xsum + (MB == 8 ? 4 * kg : 0);
     const uint8_t* wt_lane = wt + crow * wstride;
     StaticFor<NCH>::run([&](auto cc) {
@@ -499,6 +630,9 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
         if constexpr (G::SIDE_D) {
           if (d_ok && d_sbl < sbc) dq[d_row * 16 + SBC * c + d_sbl] = dreg[c & 1];
         }
+        if constexpr (G::TAIL) {
+          *reinterpret_cast<u32x4*>((t_ok && d_sbl < sbc) ? t_dst + SBC * c * G::LBPB : dump) = treg[c & 1];
+        }
       }
       if constexpr (c + 2 < NCH) issue(std::integral_constant<int, c + 2>{});
       if (sbc > 0) {
@@ -508,6 +642,10 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
           if constexpr (C == KQ_Q4_K || C == KQ_Q5_K) {
             q45k_superblock<C, R, MB>(wt_lane + sb * G::LBPB, kg, xscale, xs_lane + 256 * sb, xsum_lane + 8 * MB * sb,
                                       acc);
+          } else if constexpr (C == KQ_Q2_K) {
+            q2k_superblock<R, MB>(wt_lane + sb * G::LBPB, kg, xscale, xs_lane + 256 * sb, xsum_lane + 16 * MB * sb, acc);
+          } else if constexpr (C == KQ_Q3_K) {
+            q3k_superblock<R, MB>(wt_lane + sb * G::LBPB, kg, xscale, xs_lane + 256 * sb, xsum_lane + 16 * MB * sb, acc);
           } else {
             const float dx = kq::h2f(dq[crow * 16 + sb]) * xscale;
             q6k_superblock<R>(wt_lane + sb * G::LBPB, kg, dx, xs_lane + 256 * sb, acc);
@@ -569,8 +707,8 @@ template <int C>
 size_t sk_lds_bytes(int rows, int kch, int MB) {
   using G = SkGeom<C>;
   const int R = MB < 4 ? MB : 4;
-  const size_t wstride = (size_t)kch * G::LBPB + (((kch * G::PP) & 1) ? 0 : 16);
-  return rows * wstride + (size_t)MB * kch * 512 + (size_t)kch * 8 * MB * 4 + SK_WAVES * R * 64 * 4 + 64 +
+  const size_t wstride = (size_t)kch * G::LBPB + (((kch * (G::LBPB / 16)) & 1) ? 0 : 16);
+  return rows * wstride + (size_t)MB * kch * 512 + (size_t)kch * 16 * MB * 4 + SK_WAVES * R * 64 * 4 + 64 +
          16 * SK_THREADS + 32 * 16 * 2;
 }
 
@@ -660,16 +798,25 @@ int launch_skinny_any(const SkArgs& a, int items, int codec, int dtype, void* ws
   if (codec == KQ_Q5_K)
     return dtype == KQ_F16 ? launch_skinny_m<KQ_Q5_K, KQ_F16, GLU>(a, items, ws, s)
                            : launch_skinny_m<KQ_Q5_K, KQ_BF16, GLU>(a, items, ws, s);
+  if (codec == KQ_Q2_K)
+    return dtype == KQ_F16 ? launch_skinny_m<KQ_Q2_K, KQ_F16, GLU>(a, items, ws, s)
+                           : launch_skinny_m<KQ_Q2_K, KQ_BF16, GLU>(a, items, ws, s);
+  if (codec == KQ_Q3_K)
+    return dtype == KQ_F16 ? launch_skinny_m<KQ_Q3_K, KQ_F16, GLU>(a, items, ws, s)
+                           : launch_skinny_m<KQ_Q3_K, KQ_BF16, GLU>(a, items, ws, s);
   return dtype == KQ_F16 ? launch_skinny_m<KQ_Q6_K, KQ_F16, GLU>(a, items, ws, s)
                          : launch_skinny_m<KQ_Q6_K, KQ_BF16, GLU>(a, items, ws, s);
 }
 
-bool sk_codec_ok(int codec) { return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K; }
+bool sk_codec_ok(int codec) {
+  return codec == KQ_Q2_K || codec == KQ_Q3_K || codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K;
+}
+// q4_k / q5_k pieces are fetched with aligned 16-byte loads; the other blocks are 2-byte multiples
+uintptr_t sk_wire_align_mask(int codec) { return (codec == KQ_Q4_K || codec == KQ_Q5_K) ? 15 : 1; }
 
 bool sk_shape_ok(int M, int K, int codec, const void* x, const void* w, const void* w2) {
   if (!sk_codec_ok(codec) || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return false;
-  // q4_k / q5_k pieces are fetched with aligned 16-byte loads; q6_k blocks need 2-byte alignment only
-  const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;
+  const uintptr_t wmask = sk_wire_align_mask(codec);
   if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask)) return false;
   return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 }
@@ -703,7 +850,7 @@ int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, c
                            int dtype, hipStream_t s) {
   if (!sk_shape_ok(M, K, codec, x, w, w2) || B < 1 || B > 65535) return KQ_ERR_UNSUPPORTED;
   if (glu && (M != 1 || act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
-  const int64_t wmask = codec == KQ_Q6_K ? 1 : 15;
+  const int64_t wmask = (int64_t)sk_wire_align_mask(codec);
   if ((w_expert_stride & wmask) || ((x_batch_stride * 2) & 15)) return KQ_ERR_UNSUPPORTED;
   SkArgs a{};
   a.x = x;

@@ -46,7 +46,7 @@ def test_qmm_decode_and_prefill_shapes(kq, codec, M):
     assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, M)
 
 
-@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("codec", ["q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("M,N,K", [(1, 1000, 768), (3, 20000, 256), (8, 520, 4352), (2, 40, 8192), (5, 4100, 1024),
                                    (1, 33, 2048)])
 def test_qmm_skinny_ragged_shapes(kq, codec, M, N, K):

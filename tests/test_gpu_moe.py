@@ -103,7 +103,7 @@ def test_moe_glu_activations(kq, act, limit):
     assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
 
 
-@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("codec", ["q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("E,N,K,T,R", [(6, 136, 768, 1, 4), (8, 2048, 512, 4, 2), (3, 72, 4352, 5, 3), (128, 64, 256, 1, 8)])
 def test_moe_tuned_gathered_shapes(kq, codec, E, N, K, T, R):
     """The MFMA gathered kernels: gate/up tiles that do not divide N, 1 / 3 / 17 superblocks, many experts."""
