@@ -308,6 +308,33 @@ def main():
         del gate, up, down
         out["moe"] = moe
 
+        # ---------------- mxfp4 MoE: 32 experts of 2880 -> 2880, top-4, 64 tokens, f32 biases, swiglu_clamp
+        E, H, TOPK, T = 32, 2880, 4, 64
+        gate = synth_wire_torch("mxfp4", E * H, H, 21, dev).reshape(E, H, -1)
+        up = synth_wire_torch("mxfp4", E * H, H, 22, dev).reshape(E, H, -1)
+        down = synth_wire_torch("mxfp4", E * H, H, 23, dev).reshape(E, H, -1)
+        gb = torch.randn((E, H), device=dev, generator=gx) * 0.01
+        ub = torch.randn((E, H), device=dev, generator=gx) * 0.01
+        db = torch.randn((E, H), device=dev, generator=gx) * 0.01
+        xt = randx((T, H), 0.5)
+        idx = torch.randn((T, E), device=dev, generator=gx).topk(TOPK, dim=-1).indices
+        kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp", limit=7.0, gate_bias=gb, up_bias=ub,
+                             alpha=1.702)
+        tg, _ = time_calls(torch, [lambda: kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp",
+                                                                 limit=7.0, gate_bias=gb, up_bias=ub, alpha=1.702)],
+                           20, 3)
+        h = kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp", limit=7.0, gate_bias=gb, up_bias=ub,
+                                 alpha=1.702)
+        td, _ = time_calls(torch, [lambda: kq.gather_qmv_kq(h, down, "mxfp4", idx, bias=db)], 20, 3)
+        mbytes = H * kq.bytes_per_row("mxfp4", H)
+        ne = int(idx.unique().numel())
+        out["moe_mxfp4"] = {"tokens": T, "experts_touched": ne, "glu_us": round(tg * 1e3, 1),
+                            "down_us": round(td * 1e3, 1),
+                            "glu_gbs": round(ne * 2 * mbytes / (tg * 1e-3) / 1e9, 1),
+                            "down_gbs": round(ne * mbytes / (td * 1e-3) / 1e9, 1),
+                            "note": "per-pair VALU kernel (biases and swiglu_clamp), timed through the Python wrapper"}
+        del gate, up, down
+
         # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (q2_k / q3_k encoded, IQ codecs random wire)
         lowbit = []
         for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs"):

@@ -22,6 +22,7 @@ SOURCES = [
     ("kq_mfma.hip", []),
     ("kq_gemm.hip", []),
     ("kq_moe.hip", []),
+    ("kq_anymma.hip", ["-ffp-contract=off"]),
 ]
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",

@@ -138,6 +138,10 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
     int rcg = kq_launch_gemm(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev, s);
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
   }
+  if (M > 8) {
+    const int rca = kq_launch_anymma_dense(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+    if (rca != KQ_ERR_UNSUPPORTED) return rca;
+  }
   int rc = kq_launch_qmm_tuned(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev,
                                workspace_bytes, s);
   if (rc != KQ_ERR_UNSUPPORTED) return rc;
@@ -190,16 +194,28 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
   (void)dtype;
   if (T <= 0 || R <= 0 || !codec_ok(codec)) return 0;
   const int64_t P = (int64_t)T * R;
-  if (P > 0x7fffffff || !kq_moe_grouped_supported((int)P, E, N, K, codec)) return 0;
-  return kq_moe_grouped_workspace_bytes(glu ? T : (int)P, (int)P, E, K);
+  if (P > 0x7fffffff) return 0;
+  if (kq_moe_grouped_supported((int)P, E, N, K, codec)) return kq_moe_grouped_workspace_bytes(glu ? T : (int)P, (int)P, E, K);
+  if (kq_anymma_moe_supported((int)P, E, N, K, codec)) return kq_anymma_moe_workspace_bytes((int)P, E);
+  return 0;
 }
 
 // Batched MoE path: returns KQ_ERR_UNSUPPORTED (error text untouched) when it does not apply.
-static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx, void* out,
-                           int T, int R, int E, int N, int K, int64_t estride, int glu, int act, float limit, int codec,
-                           int dtype, void* ws, size_t ws_bytes, hipStream_t s) {
+static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
+                           const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
+                           int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
+                           size_t ws_bytes, hipStream_t s) {
   const int64_t P = (int64_t)T * R;
-  if (P > 0x7fffffff || !kq_moe_grouped_supported((int)P, E, N, K, codec)) return KQ_ERR_UNSUPPORTED;
+  if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
+  if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
+    // every other codec, biases, swiglu_clamp: the any-codec matrix-core path
+    if (!kq_anymma_moe_supported((int)P, E, N, K, codec)) return KQ_ERR_UNSUPPORTED;
+    const size_t need = kq_anymma_moe_workspace_bytes((int)P, E);
+    if (!ws || ws_bytes < need)
+      return kq_set_error(KQ_ERR_WORKSPACE, "%s: workspace of %zu bytes required (got %zu)", op, need, ws ? ws_bytes : 0);
+    return kq_launch_anymma_moe(x, static_cast<const uint8_t*>(w), static_cast<const uint8_t*>(w2), idx, bias, bias2, out,
+                                (int)P, E, N, K, glu ? R : 1, estride, glu, act, limit, alpha, codec, dtype, ws, s);
+  }
   const int rows = glu ? T : (int)P;
   const size_t need = kq_moe_grouped_workspace_bytes(rows, (int)P, E, K);
   if (!ws || ws_bytes < need)
@@ -233,11 +249,13 @@ int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_
   if (!x_dev || !gate_w_dev || !up_w_dev || !idx_dev || !out_dev)
     return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
   const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
-  if (!biased) {
-    const int rcg = try_moe_grouped(op, x_dev, gate_w_dev, up_w_dev, idx_dev, out_dev, T, R, E, N, K, estride, 1, act,
-                                    limit, codec, dtype, workspace_dev, workspace_bytes,
+  {
+    const int rcg = try_moe_grouped(op, x_dev, gate_w_dev, up_w_dev, idx_dev, gate_bias_dev, up_bias_dev, out_dev, T, R, E,
+                                    N, K, estride, 1, act, limit, alpha, codec, dtype, workspace_dev, workspace_bytes,
                                     static_cast<hipStream_t>(stream));
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
+  }
+  if (!biased) {
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(gate_w_dev),
                                            static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, out_dev, T * R, 1, N,
                                            K, R, K, estride, 1, act, limit, codec, dtype,
@@ -261,10 +279,13 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
   if (T == 0 || R == 0 || N == 0) return KQ_OK;
   if (!x_dev || !w_dev || !idx_dev || !out_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
   const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
-  if (!bias_dev) {
-    const int rcg = try_moe_grouped(op, x_dev, w_dev, nullptr, idx_dev, out_dev, T, R, E, N, K, estride, 0, 0, 0.f, codec,
-                                    dtype, workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
+  {
+    const int rcg = try_moe_grouped(op, x_dev, w_dev, nullptr, idx_dev, bias_dev, nullptr, out_dev, T, R, E, N, K, estride,
+                                    0, 0, 0.f, 0.f, codec, dtype, workspace_dev, workspace_bytes,
+                                    static_cast<hipStream_t>(stream));
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
+  }
+  if (!bias_dev) {
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, out_dev,
                                            T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype,
                                            static_cast<hipStream_t>(stream));

@@ -84,3 +84,13 @@ size_t kq_moe_grouped_workspace_bytes(int rows, int P, int E, int K);
 int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, void* out, int rows,
                           int P, int E, int N, int K, int x_div, int64_t w_expert_stride, int glu, int act,
                           float limit, int codec, int dtype, void* ws, hipStream_t s);
+// Matrix-core GEMM for every codec (exact bf16 x 3 split of the reference-order decoded weights):
+// prefill, and the batched MoE ops with biases and every activation.
+bool kq_anymma_supported(int M, int N, int K, int codec);
+int kq_launch_anymma_dense(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
+                           hipStream_t s);
+bool kq_anymma_moe_supported(int P, int E, int N, int K, int codec);
+size_t kq_anymma_moe_workspace_bytes(int P, int E);
+int kq_launch_anymma_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
+                         const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
+                         int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, hipStream_t s);

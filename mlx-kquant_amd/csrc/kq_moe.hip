@@ -335,6 +335,14 @@ int launch_grouped_any(const MoeArgs& a, int P, int E, int codec, int dtype, hip
 
 }  // namespace
 
+int kq_launch_moe_sort(const uint32_t* idx, int P, int E, void* order, void* segs, void* nseg, hipStream_t s) {
+  if (E > SORT_MAX_E) return KQ_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(SORT_THREADS), 0, s, idx, P, E, static_cast<int*>(order),
+                     static_cast<Segment*>(segs), static_cast<int*>(nseg));
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
 bool kq_moe_grouped_supported(int P, int E, int N, int K, int codec) {
   return (codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K) && P > 16 && E <= SORT_MAX_E && K > 0 &&
          (K & 255) == 0 && N > 0 && (int64_t)E + P / SEG_M < 65535;

@@ -331,7 +331,7 @@ def moe_glu_gather_kq(x, gate_w, up_w, kquant_type, indices, act="silu", limit=0
     out = torch.empty((T, R, N), dtype=x.dtype, device=x.device)
     lib = _load()
     with torch.cuda.device(x.device):
-        ws_bytes = 0 if biased else lib.kq_moe_workspace_size(T, R, E, N, K, 1, cid, _DT[x.dtype])
+        ws_bytes = lib.kq_moe_workspace_size(T, R, E, N, K, 1, cid, _DT[x.dtype])
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
         _check(lib.kq_moe_glu_gather(x_c.data_ptr(), gate_w.data_ptr(), up_w.data_ptr(), idx.data_ptr(),
                                      gb.data_ptr() if biased else None, ub.data_ptr() if biased else None,
@@ -368,7 +368,7 @@ def gather_qmv_kq(x, w, kquant_type, indices, bias=None, *, stream=None):
     out = torch.empty((T, R, N), dtype=x.dtype, device=x.device)
     lib = _load()
     with torch.cuda.device(x.device):
-        ws_bytes = 0 if b is not None else lib.kq_moe_workspace_size(T, R, E, N, K, 0, cid, _DT[x.dtype])
+        ws_bytes = lib.kq_moe_workspace_size(T, R, E, N, K, 0, cid, _DT[x.dtype])
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
         _check(lib.kq_gather_qmv(x_c.data_ptr(), w.data_ptr(), idx.data_ptr(),
                                  b.data_ptr() if b is not None else None, out.data_ptr(), T, R, E, N, K, cid,

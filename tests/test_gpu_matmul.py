@@ -144,6 +144,22 @@ def test_qmm_prefill_gemm(kq, codec, M, N, K):
         assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, N, K, dtype)
 
 
+@pytest.mark.parametrize("codec", O.ALL_CODECS)
+def test_qmm_prefill_every_codec(kq, codec):
+    """M > 8 for every codec (the tuned K-quant GEMM or the any-codec bf16 x 3 matrix-core path), both
+    activation dtypes, N that is not a multiple of the 128-row slab, and for the 32-weight-block codecs a K
+    that is not a multiple of the 256-weight step."""
+    wpb, _ = O.geometry(codec)
+    shapes = [(40, 200, 512)] + ([(130, 72, 288)] if wpb == 32 else [(130, 72, 768)])
+    for M, N, K in shapes:
+        wire = _wire(codec, N, K, seed=61)
+        for dtype in ("bfloat16", "float16"):
+            xb, xt = make_x((M, K), dtype, seed=62)
+            got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+            want = O.qmm(xb, wire, codec, True, dtype)
+            assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, N, K, dtype)
+
+
 def test_qmm_prefill_gemm_both_tile_heights(kq):
     """The 128-row tile variant (kq_set_gemm_tile_rows) gives the same rounded outputs as the default 64-row one:
     both feed the same exact products to f32 accumulators in the same order."""

@@ -149,6 +149,47 @@ def test_moe_grouped_batched_shapes(kq, codec, E, N, K, T, R):
         assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype)
 
 
+@pytest.mark.parametrize("codec", O.ALL_CODECS)
+def test_moe_batched_every_codec(kq, codec):
+    """More than 16 pairs for every codec: the batched paths (tuned K-quant or any-codec matrix-core)."""
+    wpb, _ = O.geometry(codec)
+    E, N, K, T, R = 5, 72, (288 if wpb == 32 else 512), 12, 3
+    gate = _stack(codec, E, N, K, seed=91)
+    up = _stack(codec, E, N, K, seed=92)
+    idx = np.random.default_rng(93).integers(0, E, (T, R))
+    for dtype in ("bfloat16", "float16"):
+        xb, xt = make_x((T, K), dtype, seed=94, scale=0.02)
+        got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx))
+        want = _glu_truth(codec, xb, gate, up, idx, "silu", dtype=dtype)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype)
+        hb, ht = make_x((T, R, K), dtype, seed=95, scale=0.02)
+        got = kq.gather_qmv_kq(ht, wire_to_dev(gate), codec, _idx_dev(idx))
+        want = O.gather_qmv(hb, gate, codec, idx, None, dtype)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype)
+
+
+@pytest.mark.parametrize("codec", ["mxfp4", "nvfp4"])
+def test_moe_batched_swiglu_clamp_bias(kq, codec):
+    """Biased fp4 experts with swiglu_clamp on the batched path (64 tokens, top-4), K not a multiple of 256."""
+    E, N, K, T, R = 8, 136, 576, 64, 4
+    gate = _stack(codec, E, N, K, seed=96)
+    up = _stack(codec, E, N, K, seed=97)
+    rng = np.random.default_rng(98)
+    gb = (rng.standard_normal((E, N)) * 0.01).astype(np.float32)
+    ub = (rng.standard_normal((E, N)) * 0.01).astype(np.float32)
+    idx = np.stack([rng.permutation(E)[:R] for _ in range(T)])
+    xb, xt = make_x((T, K), "bfloat16", seed=99, scale=0.2)
+    got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act="swiglu_clamp",
+                               limit=7.0, gate_bias=torch.from_numpy(gb).cuda(), up_bias=torch.from_numpy(ub).cuda(),
+                               alpha=1.702)
+    want = _glu_truth(codec, xb, gate, up, idx, "swiglu_clamp", 7.0, 1.702, gb, ub)
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
+    hb, ht = make_x((T, R, K), "bfloat16", seed=100, scale=0.2)
+    got = kq.gather_qmv_kq(ht, wire_to_dev(gate), codec, _idx_dev(idx), bias=torch.from_numpy(gb).cuda())
+    want = O.gather_qmv(hb, gate, codec, idx, gb, "bfloat16")
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
+
+
 def test_moe_grouped_matches_per_pair_path_bitwise(kq):
     """A pair's row does not depend on which other pairs share the call: rows of a 64-pair call equal the
     rows of the same pairs computed in 4-pair calls (different kernels, same exact products)."""
