@@ -266,9 +266,11 @@ def main():
 
         # ---------------- prefill GEMM
         prefill = []
-        for c in ("q4_k", "q5_k", "q6_k"):
+        for c in ("q4_k", "q5_k", "q6_k", "q2_k", "iq4_xs"):
             n, k = 28672, 8192
-            wq = quantized_weights(kq, torch, c, n, k, 5, dev)
+            # q2_k / iq4_xs run the any-codec kernel (reference-order decode + bf16 x 3 split); iq4_xs has no
+            # encoder here and uses structurally valid random wire
+            wq = quantized_weights(kq, torch, c, n, k, 5, dev) if c != "iq4_xs" else synth_wire_torch(c, n, k, 5, dev)
             for m in (512, 2048):
                 t, _ = time_calls(torch, [abi.qmm(randx((m, k)), wq, c, n, k)], 20, 5)
                 tf = 2.0 * m * n * k / (t * 1e-3) / 1e12
@@ -332,7 +334,7 @@ def main():
                             "down_us": round(td * 1e3, 1),
                             "glu_gbs": round(ne * 2 * mbytes / (tg * 1e-3) / 1e9, 1),
                             "down_gbs": round(ne * mbytes / (td * 1e-3) / 1e9, 1),
-                            "note": "per-pair VALU kernel (biases and swiglu_clamp), timed through the Python wrapper"}
+                            "note": "any-codec matrix-core path (biases, swiglu_clamp), timed through the Python wrapper"}
         del gate, up, down
 
         # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (q2_k / q3_k encoded, IQ codecs random wire)
