@@ -61,11 +61,12 @@ def synth_wire_torch(codec, rows, K, seed, device):
 
 
 def quantized_weights(kq, torch, codec, N, K, seed, device):
-    """Seeded N(0, 0.02) f32 weights [N, K] encoded by kq.quantize (host encoder), placed on the GPU."""
+    """Seeded N(0, 0.02) f32 weights [N, K] encoded by kq.quantize (host encoder; a uniform importance
+    matrix for the IQ codecs), placed on the GPU."""
     g = torch.Generator()
     g.manual_seed(seed)
     w = torch.randn((N, K), generator=g, dtype=torch.float32) * 0.02
-    wq, _ = kq.quantize(w, codec)
+    wq, _ = kq.quantize(w, codec, torch.ones(K) if codec.startswith("iq") else None)
     return wq.to(device)
 
 
@@ -268,9 +269,8 @@ def main():
         prefill = []
         for c in ("q4_k", "q5_k", "q6_k", "q2_k", "iq4_xs"):
             n, k = 28672, 8192
-            # q2_k / iq4_xs run the any-codec kernel (reference-order decode + bf16 x 3 split); iq4_xs has no
-            # encoder here and uses structurally valid random wire
-            wq = quantized_weights(kq, torch, c, n, k, 5, dev) if c != "iq4_xs" else synth_wire_torch(c, n, k, 5, dev)
+            # q2_k / iq4_xs run the any-codec kernel (reference-order decode + bf16 x 3 split)
+            wq = quantized_weights(kq, torch, c, n, k, 5, dev)
             for m in (512, 2048):
                 t, _ = time_calls(torch, [abi.qmm(randx((m, k)), wq, c, n, k)], 20, 5)
                 tf = 2.0 * m * n * k / (t * 1e-3) / 1e12
@@ -337,12 +337,12 @@ def main():
                             "note": "any-codec matrix-core path (biases, swiglu_clamp), timed through the Python wrapper"}
         del gate, up, down
 
-        # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (q2_k / q3_k encoded, IQ codecs random wire)
+        # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (q2_k / q3_k / iq4_xs encoded, iq3_s / iq2_xxs random wire)
         lowbit = []
         for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs"):
             n = k = 8192
             wb = n * kq.bytes_per_row(c, k)
-            wq = quantized_weights(kq, torch, c, n, k, 7, dev) if c in ("q2_k", "q3_k") else \
+            wq = quantized_weights(kq, torch, c, n, k, 7, dev) if c in ("q2_k", "q3_k", "iq4_xs") else \
                 synth_wire_torch(c, n, k, 7, dev)
             cps = cold_copies(torch, wq, wb)
             t, _ = time_calls(torch, [abi.qmm(x.new_ones((1, k)), w, c, n, k) for w in cps], steps, warm)

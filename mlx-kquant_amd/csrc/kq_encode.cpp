@@ -1,5 +1,6 @@
 // Host-side wire encoders behind kq_quantize: float rows -> GGUF block bytes for the five legacy
-// 32-weight codecs and the five K-quant superblock codecs.  Like the reference's encoder
+// 32-weight codecs, the five K-quant superblock codecs and the two non-linear 4-bit codecs
+// (iq4_nl, iq4_xs).  Like the reference's encoder
 // (src/kquant_cpu_encode.cpp:38-859, ggml's search heuristics) this runs on the CPU; unlike it,
 // blocks are encoded in parallel (blocks are independent).  Operation order inside a block
 // follows the cited reference lines so that, on the same x86 host arithmetic, the bytes agree.
@@ -9,6 +10,8 @@
 //   K-quant : q4_k/q5_k :445-540, q6_k :542-628, q3_k :630-734, q2_k :736-820
 //             (round-half-to-even; super-scales written as fp16 and read back before the
 //             final re-quantisation of every weight)
+//   iq4     : iq4_nl / iq4_xs, src/kquant_iq_encode.cpp:49-214 (ggml quantize_row_iq4_nl_impl: nearest
+//             codebook entry, weighted least-squares scale, 15 trial scales around max / -127)
 #include <algorithm>
 #include <cmath>
 #include <cstring>
@@ -404,6 +407,115 @@ void enc_q2_k(const float* x, const float* im, uint8_t* b) {
   pack_2bit(lv, b + 16);
 }
 
+// ------------------------------------------------------------------ iq4_nl / iq4_xs
+// Codebook kvalues_iq4nl (src/kquant_iq_tables.h:10), ascending.
+const int8_t kIq4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+// Index of the codebook entry nearest to v; a tie goes to the upper entry (the comparison is strict).
+inline int iq4_nearest(float v) {
+  if (v <= (float)kIq4Values[0]) return 0;
+  if (v >= (float)kIq4Values[15]) return 15;
+  int lo = 0, hi = 15;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) / 2;
+    if (v < (float)kIq4Values[mid]) hi = mid; else lo = mid;
+  }
+  return v - (float)kIq4Values[hi - 1] < (float)kIq4Values[hi] - v ? hi - 1 : hi;
+}
+
+// Weighted least-squares fit of one 32-weight block: levels for inverse scale `inv`, returns sum w q x
+// and sum w q^2 through the references.
+inline void iq4_fit(const float* x, const float* wt, float inv, uint8_t* lv, float& sqx, float& sq2) {
+  sqx = sq2 = 0.f;
+  for (int j = 0; j < 32; j++) {
+    const int l = iq4_nearest(inv * x[j]);
+    if (lv) lv[j] = (uint8_t)l;
+    const float q = (float)kIq4Values[l];
+    sqx += wt[j] * q * x[j];
+    sq2 += wt[j] * q * q;
+  }
+}
+
+// kSuper = 32 (iq4_nl: [f16 d][qs 16]) or 256 (iq4_xs: [f16 d][u16 scales_h][scales_l 4][qs 128]).
+template <int kSuper>
+void enc_iq4(const float* x, const float* im, uint8_t* b) {
+  constexpr int kBlocks = kSuper / 32, kTrials = 7;
+  float sigma2 = 0.f;
+  for (int j = 0; j < kSuper; j++) sigma2 += x[j] * x[j];
+  sigma2 *= 2.f / (float)kSuper;
+
+  uint8_t lv[kSuper];
+  float scale[kBlocks];
+  float top = 0.f, top_abs = 0.f;  // block scale of largest magnitude, signed
+  for (int ib = 0; ib < kBlocks; ib++) {
+    const float* xb = x + 32 * ib;
+    float wt[32];
+    for (int j = 0; j < 32; j++) wt[j] = im ? im[32 * ib + j] * std::sqrt(sigma2 + xb[j] * xb[j]) : xb[j] * xb[j];
+    float amax = 0.f, vmax = 0.f;
+    for (int j = 0; j < 32; j++) {
+      const float ax = std::fabs(xb[j]);
+      if (ax > amax) {
+        amax = ax;
+        vmax = xb[j];
+      }
+    }
+    if (amax < 1e-15f) {
+      scale[ib] = 0.f;
+      std::memset(lv + 32 * ib, 0, 32);
+      continue;
+    }
+    // first guess: the extreme weight maps to the codebook's -127 end (sign flipped)
+    float d = -vmax / (float)kIq4Values[0];
+    float sqx, sq2;
+    iq4_fit(xb, wt, 1.f / d, lv + 32 * ib, sqx, sq2);
+    d = sq2 > 0.f ? sqx / sq2 : 0.f;
+    float best = d * sqx;
+    for (int t = -kTrials; t <= kTrials; t++) {
+      iq4_fit(xb, wt, ((float)t + (float)kIq4Values[0]) / vmax, nullptr, sqx, sq2);
+      if (sq2 > 0.f && sqx * sqx > best * sq2) {
+        d = sqx / sq2;
+        best = d * sqx;
+      }
+    }
+    scale[ib] = d;
+    if (std::fabs(d) > top_abs) {
+      top_abs = std::fabs(d);
+      top = d;
+    }
+  }
+
+  uint8_t* qs;
+  if constexpr (kBlocks == 1) {
+    qs = b + 2;
+    put_f16(b, scale[0]);
+    const float inv = scale[0] ? 1.f / scale[0] : 0.f;
+    for (int j = 0; j < 32; j++) lv[j] = (uint8_t)iq4_nearest(inv * x[j]);
+  } else {
+    // super-scale d = -top / 32, 6-bit block scales (low nibbles in scales_l, high 2 bits in scales_h),
+    // then every weight is re-quantised against its rounded block scale
+    qs = b + 8;
+    const float d = -top / 32.f;
+    put_f16(b, d);
+    const float inv = d ? 1.f / d : 0.f;
+    uint32_t sh = 0;
+    uint8_t sl[4] = {0, 0, 0, 0};
+    for (int ib = 0; ib < kBlocks; ib++) {
+      const int l = clampi(rne(inv * scale[ib]), -32, 31);
+      const float dl = d * (float)l;
+      const float invl = dl ? 1.f / dl : 0.f;
+      for (int j = 0; j < 32; j++) lv[32 * ib + j] = (uint8_t)iq4_nearest(invl * x[32 * ib + j]);
+      const int u = l + 32;
+      sl[ib / 2] |= (uint8_t)((u & 15) << (4 * (ib & 1)));
+      sh |= (uint32_t)(u >> 4) << (2 * ib);
+    }
+    b[2] = (uint8_t)(sh & 0xff);
+    b[3] = (uint8_t)(sh >> 8);
+    std::memcpy(b + 4, sl, 4);
+  }
+  for (int i = 0; i < kBlocks; i++)
+    for (int j = 0; j < 16; j++) qs[16 * i + j] = (uint8_t)(lv[32 * i + j] | (lv[32 * i + 16 + j] << 4));
+}
+
 typedef void (*BlockEnc)(const float*, const float*, uint8_t*);
 void legacy_q8_0(const float* x, const float*, uint8_t* b) { enc_q8_0(x, b); }
 void legacy_q4_0(const float* x, const float*, uint8_t* b) { enc_legacy<false, 4>(x, b); }
@@ -423,6 +535,8 @@ BlockEnc encoder_for(int codec) {
     case KQ_Q4_K: return enc_q45_k<4>;
     case KQ_Q5_K: return enc_q45_k<5>;
     case KQ_Q6_K: return enc_q6_k;
+    case KQ_IQ4_NL: return enc_iq4<32>;
+    case KQ_IQ4_XS: return enc_iq4<256>;
   }
   return nullptr;
 }
@@ -440,10 +554,11 @@ extern "C" int kq_quantize(const float* w_host, const float* imatrix_host, uint8
   if (rows == 0 || K == 0) return KQ_OK;
   if (!w_host || !wire_host) return kq_set_error(KQ_ERR_INVALID, "quantize: null buffer");
   const int64_t bpr = K / g.wpb, nblocks = rows * bpr;
-  const bool kquant = g.wpb == 256;
+  // the importance matrix steers the K-quants and the IQ codecs (flat-32 iq4_nl included); the legacy codecs ignore it
+  const bool weighted = g.wpb == 256 || codec == KQ_IQ4_NL;
   auto work = [&](int64_t b0, int64_t b1) {
     for (int64_t b = b0; b < b1; b++) {
-      const float* im = (imatrix_host && kquant) ? imatrix_host + (b % bpr) * g.wpb : nullptr;  // legacy ignores it
+      const float* im = (imatrix_host && weighted) ? imatrix_host + (b % bpr) * g.wpb : nullptr;
       enc(w_host + b * g.wpb, im, wire_host + b * g.bpb);
     }
   };

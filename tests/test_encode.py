@@ -17,7 +17,8 @@ import kq  # noqa: E402
 GOLD = os.path.join(ROOT, "tests", "golden")
 KCODECS = ["q2_k", "q3_k", "q4_k", "q5_k", "q6_k"]
 RT_BOUND = {"q8_0": 0.02, "q4_0": 0.15, "q4_1": 0.15, "q5_0": 0.10, "q5_1": 0.10, "q6_k": 0.05, "q5_k": 0.08,
-            "q4_k": 0.12, "q3_k": 0.25, "q2_k": 0.40}
+            "q4_k": 0.12, "q3_k": 0.25, "q2_k": 0.40, "iq4_nl": 0.12, "iq4_xs": 0.12}  # iq4: tests/test_iq_encode.py:34-35
+KV_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float32)
 
 
 def _enc(w, codec, imatrix=None):
@@ -66,7 +67,7 @@ def test_imatrix_changes_kquant_bytes_only():
     rng = np.random.default_rng(9)
     w = (rng.standard_normal((8, 512)) * 0.05).astype(np.float32)
     im = rng.uniform(0.1, 10.0, 512).astype(np.float32)
-    for codec in KCODECS:
+    for codec in KCODECS + ["iq4_nl", "iq4_xs"]:  # every IQ codec is importance-weighted, flat-32 iq4_nl included
         assert not np.array_equal(_enc(w, codec), _enc(w, codec, im)), codec
         rel = np.linalg.norm(O.dequantize(_enc(w, codec, im), codec) - w) / np.linalg.norm(w)
         assert rel < 1.5 * RT_BOUND[codec]
@@ -102,3 +103,40 @@ def test_legacy_closed_forms():
     wire = _enc(x, "q4_1")
     m = wire[:, 2:4].copy().view(np.float16).astype(np.float32)[:, 0]
     assert np.allclose(m, x.min(1), rtol=1e-3, atol=1e-4)
+
+
+def test_iq4_known_answer_blocks():
+    """Blocks that ARE codebook points must come back as exactly those levels and scales: a perfect fit
+    maximises the weighted correlation the scale search ranks by, so neither the first guess nor any of
+    the 15 trial scales can displace it.  Pins the codebook search, the fp16 scale slot, the 6-bit
+    scale split of iq4_xs (scales_l nibbles, scales_h pairs) and the nibble packing."""
+    rng = np.random.default_rng(11)
+    # iq4_nl: 40 blocks, scale d exactly representable in fp16, one weight at the -127 end
+    lv = rng.integers(0, 16, (40, 32))
+    lv[:, 5] = 0
+    d = (rng.integers(1, 64, 40) / 4096.0).astype(np.float32) * rng.choice([-1.0, 1.0], 40).astype(np.float32)
+    x = d[:, None] * KV_IQ4NL[lv]
+    wire = _enc(x.reshape(40, 32), "iq4_nl")
+    assert np.array_equal(wire[:, :2].copy().view(np.float16)[:, 0].astype(np.float32), d)
+    assert np.array_equal(wire[:, 2:] & 15, lv[:, :16]) and np.array_equal(wire[:, 2:] >> 4, lv[:, 16:])
+    # iq4_xs: super-scale D, block scales D * l with l in [-32, 31] and one block at -32
+    nsb = 12
+    lv = rng.integers(0, 16, (nsb, 8, 32))
+    lv[:, :, 9] = 0
+    lb = rng.integers(-32, 32, (nsb, 8))
+    lb[lb == 0] = 3
+    lb[:, 2] = -32
+    D = (rng.integers(1, 32, nsb) / 65536.0).astype(np.float32)
+    x = (D[:, None, None] * lb[:, :, None]) * KV_IQ4NL[lv]
+    wire = _enc(x.reshape(nsb, 256).astype(np.float32), "iq4_xs")
+    assert np.array_equal(wire[:, :2].copy().view(np.float16)[:, 0].astype(np.float32), D)
+    u = lb + 32
+    sl = wire[:, 4:8]
+    got_lo = np.stack([sl[:, i // 2] >> (4 * (i & 1)) & 15 for i in range(8)], axis=1)
+    sh = wire[:, 2].astype(np.uint32) | (wire[:, 3].astype(np.uint32) << 8)
+    got_hi = np.stack([(sh >> (2 * i)) & 3 for i in range(8)], axis=1)
+    assert np.array_equal(got_lo | (got_hi << 4), u)
+    qs = wire[:, 8:].reshape(nsb, 8, 16)
+    assert np.array_equal(qs & 15, lv[:, :, :16]) and np.array_equal(qs >> 4, lv[:, :, 16:])
+    # and the decoder agrees with the pre-image exactly
+    assert np.array_equal(O.dequantize(wire, "iq4_xs"), x.reshape(nsb, 256).astype(np.float32))
