@@ -160,15 +160,18 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
   (void)workspace_dev; (void)workspace_bytes; (void)rhs_sorted;
   if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: unknown codec id %d", codec);
   if (!half_dtype(dtype)) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: activations must be float16 or bfloat16");
-  if (!transpose)
-    return kq_set_error(KQ_ERR_UNSUPPORTED, "gather_qmm: transpose=false has no kernel in this build");
   if (B < 0 || M < 0 || N < 0 || K < 0) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: negative dimension");
-  if (K % kCodecs[codec].weights_per_block)
-    return kq_set_error(KQ_ERR_INVALID, "gather_qmm: K (%d) is not a multiple of %d", K,
+  const int inner = transpose ? K : N;  // the quantized (row) dimension of the expert matrices
+  if (inner % kCodecs[codec].weights_per_block)
+    return kq_set_error(KQ_ERR_INVALID, "gather_qmm: quantized row length %d is not a multiple of %d", inner,
                         kCodecs[codec].weights_per_block);
   if (B == 0 || M == 0 || N == 0) return KQ_OK;
   if (!x_dev || !w_dev || !out_dev || !lhs_idx_dev || !rhs_idx_dev)
     return kq_set_error(KQ_ERR_INVALID, "gather_qmm: null buffer");
+  if (!transpose)
+    return kq_launch_gather_nt_generic(x_dev, static_cast<const uint8_t*>(w_dev), lhs_idx_dev, rhs_idx_dev, out_dev, B,
+                                       M, N, K, x_batch_stride, w_expert_stride_bytes, codec, dtype,
+                                       static_cast<hipStream_t>(stream));
   {
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
                                            out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0, 0, 0.f,

@@ -56,6 +56,9 @@ int kq_launch_gemv_generic(const void* x, const uint8_t* w, void* y, int M, int 
                            hipStream_t s);
 int kq_launch_gemm_nt_generic(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec,
                               int dtype, hipStream_t s);
+int kq_launch_gather_nt_generic(const void* x, const uint8_t* w, const uint32_t* lhs, const uint32_t* rhs, void* out,
+                                int B, int M, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride, int codec,
+                                int dtype, hipStream_t s);
 int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
                              const uint32_t* rhs, const float* bias, const float* bias2, void* out, int B, int M,
                              int N, int K, int x_div, int64_t x_batch_stride, int64_t w_expert_stride, int glu,

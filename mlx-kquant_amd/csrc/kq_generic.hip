@@ -111,30 +111,33 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_generic_kernel(const void* __
 }
 
 // y[m, n] = sum_k x[m, k] * W[k, n] (transpose = false: W decodes to [K, N]).  One thread per
-// (m, 8 consecutive n); walks all K wire rows.
+// (m, 8 consecutive n); walks all K wire rows.  Grid z = gathered item: item b reads activation
+// matrix lhs[b] and expert rhs[b] (both null for the plain op).
 template <int C, int DT>
 __global__ __launch_bounds__(GV_THREADS) void gemm_nt_generic_kernel(const void* __restrict__ x,
                                                                      const uint8_t* __restrict__ w,
                                                                      void* __restrict__ y, int M, int N, int K,
-                                                                     const uint8_t* __restrict__ grids) {
+                                                                     const uint8_t* __restrict__ grids,
+                                                                     const uint32_t* __restrict__ lhs,
+                                                                     const uint32_t* __restrict__ rhs,
+                                                                     int64_t x_batch_stride, int64_t w_expert_stride) {
   constexpr int WPB = kq_geom(C).wpb, BPB = kq_geom(C).bpb, GPB = WPB / 8;
   const int gi = blockIdx.x * GV_THREADS + threadIdx.x;  // 8-column group
-  const int m = blockIdx.y;
+  const int m = blockIdx.y, item = blockIdx.z;
   if (gi >= N / 8) return;
   const size_t row_bytes = (size_t)(N / WPB) * BPB;
-  const uint8_t* wb = w + (size_t)(gi / GPB) * BPB;
+  const uint8_t* wb = w + (rhs ? (size_t)rhs[item] * (size_t)w_expert_stride : 0) + (size_t)(gi / GPB) * BPB;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const uint16_t* xr = static_cast<const uint16_t*>(x) + (size_t)m * K;
+  const uint16_t* xr = static_cast<const uint16_t*>(x) + (lhs ? (size_t)lhs[item] * (size_t)x_batch_stride : 0) + (size_t)m * K;
   for (int k = 0; k < K; k++) {
     float wv[8];
     kq::decode8<C>(wb + (size_t)k * row_bytes, gi % GPB, grids, wv);
     float xv = DT == KQ_F16 ? kq::h2f(xr[k]) : kq::bf162f(xr[k]);
     for (int t = 0; t < 8; t++) acc[t] = fmaf(xv, wv[t], acc[t]);
   }
-  for (int t = 0; t < 8; t++) store_y<DT>(y, (size_t)m * N + 8 * (size_t)gi + t, acc[t]);
+  for (int t = 0; t < 8; t++) store_y<DT>(y, ((size_t)item * M + m) * N + 8 * (size_t)gi + t, acc[t]);
 }
 
-// ------------------------------------------------------------ generic gathered kernels
 // One wave per (item p, output row n).  Item p reads activation matrix x[lhs[p]] (or p / x_div
 // when lhs is null) and expert rhs[p]; with GLU it also reads the `up` stack and applies the
 // fused epilogue (metal/mlx/backend/metal/kernels/kq_moe_glu_kq.h:34-60 of the reference).
@@ -268,12 +271,14 @@ struct GemvRun {
 template <int C>
 struct GemmNtRun {
   static int run(const void* x, const uint8_t* w, void* y, int M, int N, int K, int dt, const uint8_t* grids,
-                 hipStream_t s) {
-    dim3 grid((N / 8 + GV_THREADS - 1) / GV_THREADS, M), block(GV_THREADS);
+                 const uint32_t* lhs, const uint32_t* rhs, int B, int64_t xs, int64_t ws, hipStream_t s) {
+    dim3 grid((N / 8 + GV_THREADS - 1) / GV_THREADS, M, B), block(GV_THREADS);
     if (dt == KQ_F16)
-      hipLaunchKernelGGL((gemm_nt_generic_kernel<C, KQ_F16>), grid, block, 0, s, x, w, y, M, N, K, grids);
+      hipLaunchKernelGGL((gemm_nt_generic_kernel<C, KQ_F16>), grid, block, 0, s, x, w, y, M, N, K, grids, lhs, rhs, xs,
+                         ws);
     else
-      hipLaunchKernelGGL((gemm_nt_generic_kernel<C, KQ_BF16>), grid, block, 0, s, x, w, y, M, N, K, grids);
+      hipLaunchKernelGGL((gemm_nt_generic_kernel<C, KQ_BF16>), grid, block, 0, s, x, w, y, M, N, K, grids, lhs, rhs, xs,
+                         ws);
     KQ_HIP_CHECK(hipGetLastError());
     return KQ_OK;
   }
@@ -328,7 +333,18 @@ int kq_launch_gemm_nt_generic(const void* x, const uint8_t* w, void* y, int M, i
                               int dtype, hipStream_t s) {
   const uint8_t* grids = kq_device_grids();
   if (!grids) return KQ_ERR_HIP;
-  return dispatch_codec<GemmNtRun>(codec, x, w, y, M, N, K, dtype, grids, s);
+  return dispatch_codec<GemmNtRun>(codec, x, w, y, M, N, K, dtype, grids, (const uint32_t*)nullptr,
+                                   (const uint32_t*)nullptr, 1, (int64_t)0, (int64_t)0, s);
+}
+
+int kq_launch_gather_nt_generic(const void* x, const uint8_t* w, const uint32_t* lhs, const uint32_t* rhs, void* out,
+                                int B, int M, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride, int codec,
+                                int dtype, hipStream_t s) {
+  const uint8_t* grids = kq_device_grids();
+  if (!grids) return KQ_ERR_HIP;
+  if (M > 65535 || B > 65535) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: M and the batch must be below 65536");
+  return dispatch_codec<GemmNtRun>(codec, x, w, out, M, N, K, dtype, grids, lhs, rhs, B, x_batch_stride,
+                                   w_expert_stride, s);
 }
 
 int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,

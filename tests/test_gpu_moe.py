@@ -50,6 +50,21 @@ def test_gather_qmm(kq, codec, M):
     assert rel_l2(dev_to_bits(got).reshape(B, M, N), want, "float16") <= TOL
 
 
+@pytest.mark.parametrize("codec", ["q4_k", "q8_0", "iq4_nl", "q6_k"])
+def test_gather_qmm_no_transpose(kq, codec):
+    """transpose=False: every expert decodes to [K, N] (the MLA / LoRA-vjp orientation)."""
+    E, K, N, B, M = 3, 48, 512, 6, 4
+    wire = _stack(codec, E, K, N, seed=46)  # [E, K, N / wpb * bpb]
+    xb, xt = make_x((B, M, K), "float16", seed=47)
+    rng = np.random.default_rng(48)
+    lhs, rhs = rng.integers(0, B, B), rng.integers(0, E, B)
+    got = kq.gather_qmm(xt, wire_to_dev(wire), None, codec, lhs_indices=_idx_dev(lhs), rhs_indices=_idx_dev(rhs),
+                        transpose=False)
+    want = O.gather_qmm(xb, wire, codec, lhs, rhs, False, "float16")
+    assert tuple(got.shape) == (B, M, N)
+    assert rel_l2(dev_to_bits(got), want, "float16") <= TOL
+
+
 def test_gather_qmm_reference_moe_fixture_and_strided_experts(kq):
     wire = np.load(os.path.join(GOLD, "q4_k_moe.npz"))["wire"]  # [4, 128, 288]
     E, N, K, B = 4, 128, 512, 64
