@@ -84,6 +84,10 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
 /* Tuning hook without a counterpart in the reference: activation rows per workgroup tile of the
  * prefill GEMM, 64 or 128 (anything else restores the default, 64).  Process-wide, not thread-safe. */
 void kq_set_gemm_tile_rows(int rows);
+/* Tuning hook without a counterpart in the reference: 1 makes dense skinny-M calls use the
+ * workgroup-synchronous kernel (the one the gathered ops use) instead of the decoupled-wave one;
+ * 0 restores the default.  Process-wide, not thread-safe. */
+void kq_set_skinny_variant(int variant);
 
 /* out[b] = x[lhs[b]] . W[rhs[b]]^T for b < B; x batches are [M,K] matrices
  * `x_batch_stride` elements apart, experts are [N, bytes_per_row] wire matrices

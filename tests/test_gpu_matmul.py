@@ -75,6 +75,23 @@ def test_qmm_gemv_unaligned_rows_and_tensor_end(kq, codec):
     assert rel_l2(dev_to_bits(got), want, "float16") <= TOL
 
 
+@pytest.mark.parametrize("codec", ["q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+def test_qmm_skinny_both_variants(kq, codec):
+    """Dense skinny calls through the workgroup-synchronous kernel (kq_set_skinny_variant(1)) as well as the
+    default decoupled-wave one."""
+    lib = kq._load()
+    try:
+        lib.kq_set_skinny_variant(1)
+        for M, N, K in ((1, 1000, 768), (8, 520, 4352), (3, 4100, 1024)):
+            wire = _wire(codec, N, K, seed=41)
+            xb, xt = make_x((M, K), "bfloat16", seed=42)
+            got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+            want = O.qmm(xb, wire, codec, True, "bfloat16")
+            assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, M, N, K)
+    finally:
+        lib.kq_set_skinny_variant(0)
+
+
 def test_qmm_skinny_unaligned_q6k_rows(kq):
     """q6_k rows are 210-byte multiples: a wire view that starts 2 bytes into an allocation still decodes."""
     N, K, M = 64, 768, 1
