@@ -434,8 +434,8 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
   constexpr int PPR = SBC * G::PP;    // 16-byte pieces per row and sub-chunk
   constexpr int PPC = (SK_MAXROWS * PPR + SK_THREADS - 1) / SK_THREADS;  // pieces per thread and sub-chunk
   // activation staging slots per thread: slot t = (row t / XK, k-pass t % XK); a chunk holds at
-  // most min(512, 1024 / MB) 8-element groups per row because kch * MB <= 32
-  constexpr int XK = MB <= 2 ? 2 : 1;
+  // most min(512, 2048 / MB) 8-element groups per row because kch <= 16 and kch * MB <= 64
+  constexpr int XK = MB <= 4 ? 2 : 1;
   constexpr int XG = MB * XK;
   constexpr int INF = SK_INF;  // sub-chunks in flight
 
@@ -718,7 +718,7 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny2_kernel(SkArgs a) {
   constexpr int UP = (SK_MAXROWS * G::PP + 63) / 64;      // pieces per lane and unit
   constexpr int WROW = G::LBPB;                           // LDS row stride: an odd number of 16-byte pieces
   constexpr int WBUF = SK_MAXROWS * WROW + 64;            // wave buffer (+ 32 d values of q6_k)
-  constexpr int XK = MB <= 2 ? 2 : 1;
+  constexpr int XK = MB <= 4 ? 2 : 1;
   constexpr int XG = MB * XK;
   constexpr int DEPTH = SK2_DEPTH;                        // units in flight per wave
 
@@ -990,11 +990,11 @@ int launch_skinny(SkArgs a, int items, void* ws, hipStream_t s) {
   const int tiles = (a.N + half - 1) / half;
   int kch = splits > 1 ? a.sb_per_split : a.K >> 8;
   if (kch > 16) kch = 16;            // four sub-chunks of four superblocks
-  if (kch * MB > 32) kch = 32 / MB;  // keep the f16 activations of a chunk within 16 KiB
+  if (kch * MB > 64) kch = 64 / MB;  // keep the f16 activations of a chunk within 32 KiB
   if constexpr (!GLU) {
-    // dense call, M <= 2, at least two superblocks per wave: decoupled-wave variant (measured 8 - 17 % faster
-    // there; at M >= 4 or one superblock per wave the synchronous kernel wins by 5 - 12 %)
-    if (items == 1 && g_sk_variant != 1 && (g_sk_variant == 2 || (MB <= 2 && kch >= 8))) {
+    // dense call: decoupled-wave variant (measured 3 - 25 % faster than the synchronous kernel on every
+    // decode shape of the sweep)
+    if (items == 1 && g_sk_variant != 1) {
       const size_t lds2 = sk2_lds_bytes<C>(kch, MB);
       a.rows_per_tile = rows;
       a.kch = kch;
