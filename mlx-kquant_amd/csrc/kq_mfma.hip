@@ -702,25 +702,29 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
 
 // ------------------------------------------------------------------ decoupled-wave variant (dense calls)
 // Same tiles, same superblock routines, but every wave fetches, parks and consumes ITS OWN
-// superblocks (wave w owns superblocks w, w + 4, ... of the chunk): the weight stream needs no
-// workgroup barrier, so a wave that has its bytes never waits for the slowest of four.  A wave's
-// unit = one superblock of all 32 tile rows (32 PP pieces: consecutive lanes read the PP consecutive
-// pieces of a row, then the next row), parked in a wave-private LDS buffer; LDS operations of one
-// wave execute in order, so park -> fragment reads -> next park need no synchronisation.
+// superblocks: the weight stream needs no workgroup barrier, so a wave that has its bytes never
+// waits for the slowest of four.  A wave owns a run of adjacent superblocks of the chunk and moves
+// it in units of USB superblocks x 32 rows.  USB = 2: consecutive lanes read the 2 PP consecutive
+// pieces of a row (288 B for q4_k), then the next row -- reading the 33 MB gate/up matrix with
+// nothing but this pattern takes 7.3 us, with 144-byte runs 8.2 us, with whole 576-byte runs 6.7 us (as
+// fast as a linear sweep) but then nothing overlaps the decode.  USB = 1 serves short K ranges.
+// Units are parked in a wave-private LDS buffer; LDS operations of one wave execute in order, so
+// park -> fragment reads -> next park need no synchronisation.
 #ifndef SK2_DEPTH
 #define SK2_DEPTH 1
 #endif
-template <int C, int DT, int MB>
+template <int C, int DT, int MB, int USB>
 __global__ __launch_bounds__(SK_THREADS, 2) void skinny2_kernel(SkArgs a) {
   using G = SkGeom<C>;
   constexpr int R = MB < 4 ? MB : 4;
-  constexpr int NU = 4;                                   // units per wave and chunk (kch <= 16)
-  constexpr int UP = (SK_MAXROWS * G::PP + 63) / 64;      // pieces per lane and unit
-  constexpr int WROW = G::LBPB;                           // LDS row stride: an odd number of 16-byte pieces
-  constexpr int WBUF = SK_MAXROWS * WROW + 64;            // wave buffer (+ 32 d values of q6_k)
+  constexpr int NU = 4 / USB;                                  // units per wave and chunk (kch <= 16)
+  constexpr int UPIECES = SK_MAXROWS * USB * G::PP;            // pieces of a unit
+  constexpr int UP = (UPIECES + 63) / 64;                      // pieces per lane and unit
+  constexpr int WROW = USB * G::LBPB + (USB == 2 ? 16 : 0);    // LDS row stride: an odd number of 16-byte pieces
+  constexpr int WBUF = SK_MAXROWS * WROW + 128;                // wave buffer (+ 64 d values of q6_k)
   constexpr int XK = MB <= 4 ? 2 : 1;
   constexpr int XG = MB * XK;
-  constexpr int DEPTH = SK2_DEPTH;                        // units in flight per wave
+  constexpr int DEPTH = SK2_DEPTH;                             // units in flight per wave
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int M = a.M, N = a.N, K = a.K, rows_per_tile = a.rows_per_tile, kch = a.kch;
@@ -732,7 +736,7 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny2_kernel(SkArgs a) {
   float* scratch = red + SK_WAVES * R * 64;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   uint8_t* wbuf = reinterpret_cast<uint8_t*>(scratch + 16) + wave * WBUF;
-  uint16_t* dq = reinterpret_cast<uint16_t*>(wbuf + SK_MAXROWS * WROW);
+  uint16_t* dq = reinterpret_cast<uint16_t*>(wbuf + SK_MAXROWS * WROW);  // [row][USB]
 
   const int n_in = lane & 31, kg = lane >> 5;
   const int nsb = K >> 8;
@@ -747,24 +751,27 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny2_kernel(SkArgs a) {
 #pragma unroll
   for (int r = 0; r < R; r++) acc[r] = 0.f;
 
-  // piece map of a unit: piece i = lane + 64 t -> (row i / PP, piece i % PP)
+  // piece map of a unit: piece i = lane + 64 t -> (row, superblock of the unit, piece of the block)
   uint32_t goff[UP], loff[UP];
-  bool piece_ok[UP];
   StaticFor<UP>::run([&](auto t) {
     constexpr int T = decltype(t)::value;
-    const int i = lane + 64 * T, r = i / G::PP, pc = i % G::PP;
-    piece_ok[T] = r < nrows;
-    goff[T] = piece_ok[T] ? (uint32_t)r * (uint32_t)row_bytes + 16 * pc : 0;
-    loff[T] = (uint32_t)r * WROW + 16 * pc;
+    const int i = lane + 64 * T, r = i / (USB * G::PP), q = i % (USB * G::PP), sbl = q / G::PP, pc = q % G::PP;
+    goff[T] = r < nrows ? (uint32_t)r * (uint32_t)row_bytes + sbl * G::BPB + 16 * pc : 0;  // spare slots re-read the tile start
+    loff[T] = (uint32_t)r * WROW + sbl * G::LBPB + 16 * pc;
   });
-  const bool side_ok = lane < nrows;  // lanes 0..31: tail piece / d of row `lane`
-  const uint8_t* side_src = wtile + (side_ok ? (size_t)lane * row_bytes : 0);
+  // side channel (tail piece / d): lane -> (row lane / USB, superblock lane % USB)
+  const int s_row = lane / USB, s_sbl = lane % USB;
+  const bool side_ok = s_row < nrows && lane < SK_MAXROWS * USB;
+  const uint8_t* side_src = wtile + (side_ok ? (size_t)s_row * row_bytes + s_sbl * G::BPB : 0);
 
   const int sb_begin = a.ksplit > 1 ? (int)blockIdx.z * a.sb_per_split : 0;
   const int sb_end = a.ksplit > 1 ? (sb_begin + a.sb_per_split < nsb ? sb_begin + a.sb_per_split : nsb) : nsb;
   for (int sb0 = sb_begin; sb0 < sb_end; sb0 += kch) {
     const int sbn = (sb_end - sb0 < kch) ? (sb_end - sb0) : kch;
     const int kc = sbn << 8, k0 = sb0 << 8;
+    // this wave's superblocks of the chunk: USB = 2 -> a run of 2 nu adjacent ones, USB = 1 -> wave, wave + 4, ...
+    const int nu = USB == 2 ? (sbn + 7) >> 3 : NU;
+    auto unit_first = [&](int u) { return USB == 2 ? (wave * nu + u) * 2 : 4 * u + wave; };
 
     // ---- activation loads first
     const int gpr = kc >> 3;
@@ -778,13 +785,15 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny2_kernel(SkArgs a) {
       xreg[T] = *reinterpret_cast<const u32x4*>(x16 + (size_t)m * K + k0 + 8 * kgi);
     });
 
-    // ---- this wave's weight stream: unit u = superblock 4 u + wave of the chunk, DEPTH units in flight
+    // ---- this wave's weight stream, DEPTH units in flight
     u32x4 wreg[DEPTH * UP], treg[DEPTH];
     uint16_t dreg[DEPTH];
     auto issue = [&](auto uu) {
       constexpr int u = decltype(uu)::value;
-      const int sb = 4 * u + wave;
-      const bool live = sb < sbn;  // wave-uniform
+      const int sb = unit_first(u);
+      const bool live = u < nu && sb < sbn;  // wave-uniform
+      // (a unit whose second superblock lies past the chunk reads the following superblock or row:
+      // the bytes exist unless this is the matrix end, see the launcher)
       const size_t sboff = (size_t)(sb0 + (live ? sb : 0)) * G::BPB;
       StaticFor<UP>::run([&](auto t) {
         constexpr int T = decltype(t)::value;
@@ -862,18 +871,19 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny2_kernel(SkArgs a) {
     const uint8_t* wt_lane = wbuf + crow * WROW;
     StaticFor<NU>::run([&](auto uu) {
       constexpr int u = decltype(uu)::value;
-      const int sb = 4 * u + wave;
-      const bool live = sb < sbn;
+      const int sbf = unit_first(u);
+      const bool live = u < nu && sbf < sbn;
       if (live) {
         StaticFor<UP>::run([&](auto t) {
           constexpr int T = decltype(t)::value;
-          if (lane + 64 * T < SK_MAXROWS * G::PP) *reinterpret_cast<u32x4*>(wbuf + loff[T]) = wreg[(u % DEPTH) * UP + T];
+          if (lane + 64 * T < UPIECES) *reinterpret_cast<u32x4*>(wbuf + loff[T]) = wreg[(u % DEPTH) * UP + T];
         });
         if constexpr (G::SIDE_D) {
-          if (lane < SK_MAXROWS) dq[lane] = dreg[u % DEPTH];
+          if (lane < SK_MAXROWS * USB) dq[lane] = dreg[u % DEPTH];
         }
         if constexpr (G::TAIL) {
-          if (lane < SK_MAXROWS) *reinterpret_cast<u32x4*>(wbuf + lane * WROW + 16 * G::PP) = treg[u % DEPTH];
+          if (lane < SK_MAXROWS * USB)
+            *reinterpret_cast<u32x4*>(wbuf + s_row * WROW + s_sbl * G::LBPB + 16 * G::PP) = treg[u % DEPTH];
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -881,15 +891,22 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny2_kernel(SkArgs a) {
       }
       if constexpr (u + DEPTH < NU) issue(std::integral_constant<int, u + DEPTH>{});
       if (live) {
-        if constexpr (C == KQ_Q4_K || C == KQ_Q5_K) {
-          q45k_superblock<C, R, MB>(wt_lane, kg, xscale, xs_lane + 256 * sb, xsum_lane + 8 * MB * sb, acc);
-        } else if constexpr (C == KQ_Q2_K) {
-          q2k_superblock<R, MB>(wt_lane, kg, xscale, xs_lane + 256 * sb, xsum_lane + 16 * MB * sb, acc);
-        } else if constexpr (C == KQ_Q3_K) {
-          q3k_superblock<R, MB>(wt_lane, kg, xscale, xs_lane + 256 * sb, xsum_lane + 16 * MB * sb, acc);
-        } else {
-          const float dx = kq::h2f(dq[crow]) * xscale;
-          q6k_superblock<R>(wt_lane, kg, dx, xs_lane + 256 * sb, acc);
+#pragma unroll
+        for (int q = 0; q < USB; q++) {
+          const int sb = sbf + q;
+          if (sb < sbn) {
+            const uint8_t* bl = wt_lane + q * G::LBPB;
+            if constexpr (C == KQ_Q4_K || C == KQ_Q5_K) {
+              q45k_superblock<C, R, MB>(bl, kg, xscale, xs_lane + 256 * sb, xsum_lane + 8 * MB * sb, acc);
+            } else if constexpr (C == KQ_Q2_K) {
+              q2k_superblock<R, MB>(bl, kg, xscale, xs_lane + 256 * sb, xsum_lane + 16 * MB * sb, acc);
+            } else if constexpr (C == KQ_Q3_K) {
+              q3k_superblock<R, MB>(bl, kg, xscale, xs_lane + 256 * sb, xsum_lane + 16 * MB * sb, acc);
+            } else {
+              const float dx = kq::h2f(dq[crow * USB + q]) * xscale;
+              q6k_superblock<R>(bl, kg, dx, xs_lane + 256 * sb, acc);
+            }
+          }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -919,11 +936,12 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny2_kernel(SkArgs a) {
 }
 
 template <int C>
-size_t sk2_lds_bytes(int kch, int MB) {
+size_t sk2_lds_bytes(int kch, int MB, int usb) {
   using G = SkGeom<C>;
   const int R = MB < 4 ? MB : 4;
+  const size_t wrow = (size_t)usb * G::LBPB + (usb == 2 ? 16 : 0);
   return (size_t)MB * kch * 512 + (size_t)kch * 16 * MB * 4 + SK_WAVES * R * 64 * 4 + 64 +
-         SK_WAVES * (SK_MAXROWS * G::LBPB + 64);
+         SK_WAVES * (SK_MAXROWS * wrow + 128);
 }
 
 template <int DT>
@@ -995,17 +1013,28 @@ int launch_skinny(SkArgs a, int items, void* ws, hipStream_t s) {
     // dense call: decoupled-wave variant (measured 3 - 25 % faster than the synchronous kernel on every
     // decode shape of the sweep)
     if (items == 1 && g_sk_variant != 1) {
-      const size_t lds2 = sk2_lds_bytes<C>(kch, MB);
+      // Units of two adjacent superblocks read HBM in a friendlier pattern but measured 15 - 60 % slower
+      // end to end (two superblocks of decode per unit leave too little overlap), so they are only
+      // selectable through kq_set_skinny_variant(3).  Such a unit may read one superblock past an
+      // odd-length K range, i.e. into the next row: fine except at the very end of the matrix, so odd
+      // superblock counts always keep single-superblock units.
+      const bool two = g_sk_variant == 3 && kch >= 8 && ((a.K >> 8) & 1) == 0 &&
+                       (splits == 1 || (a.sb_per_split & 1) == 0);
+      const size_t lds2 = sk2_lds_bytes<C>(kch, MB, two ? 2 : 1);
       a.rows_per_tile = rows;
       a.kch = kch;
-      auto kern2 = skinny2_kernel<C, DT, MB>;
       static bool attr2_set = false;
       if (!attr2_set) {
-        KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern2),
+        KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(skinny2_kernel<C, DT, MB, 1>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 120 * 1024));
+        KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(skinny2_kernel<C, DT, MB, 2>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 120 * 1024));
         attr2_set = true;
       }
-      hipLaunchKernelGGL(kern2, dim3(tiles, 1, splits), dim3(SK_THREADS), lds2, s, a);
+      if (two)
+        hipLaunchKernelGGL((skinny2_kernel<C, DT, MB, 2>), dim3(tiles, 1, splits), dim3(SK_THREADS), lds2, s, a);
+      else
+        hipLaunchKernelGGL((skinny2_kernel<C, DT, MB, 1>), dim3(tiles, 1, splits), dim3(SK_THREADS), lds2, s, a);
       KQ_HIP_CHECK(hipGetLastError());
       if (splits > 1) {
         const int count = a.M * a.N;

@@ -77,17 +77,18 @@ def test_qmm_gemv_unaligned_rows_and_tensor_end(kq, codec):
 
 @pytest.mark.parametrize("codec", ["q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_qmm_skinny_both_variants(kq, codec):
-    """Dense skinny calls through the workgroup-synchronous kernel (kq_set_skinny_variant(1)) as well as the
-    default decoupled-wave one."""
+    """Dense skinny calls through the workgroup-synchronous kernel (kq_set_skinny_variant(1)) and the
+    two-superblock-unit form of the decoupled-wave kernel (3) as well as the default."""
     lib = kq._load()
     try:
-        lib.kq_set_skinny_variant(1)
-        for M, N, K in ((1, 1000, 768), (8, 520, 4352), (3, 4100, 1024)):
-            wire = _wire(codec, N, K, seed=41)
-            xb, xt = make_x((M, K), "bfloat16", seed=42)
-            got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
-            want = O.qmm(xb, wire, codec, True, "bfloat16")
-            assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, M, N, K)
+        for variant in (1, 3):
+            lib.kq_set_skinny_variant(variant)
+            for M, N, K in ((1, 1000, 768), (8, 520, 4352), (3, 4100, 1024), (2, 300, 4096), (5, 4200, 14336)):
+                wire = _wire(codec, N, K, seed=41)
+                xb, xt = make_x((M, K), "bfloat16", seed=42)
+                got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+                want = O.qmm(xb, wire, codec, True, "bfloat16")
+                assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, variant, M, N, K)
     finally:
         lib.kq_set_skinny_variant(0)
 
