@@ -84,10 +84,11 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
 /* Tuning hook without a counterpart in the reference: activation rows per workgroup tile of the
  * prefill GEMM, 64 or 128 (anything else restores the default, 64).  Process-wide, not thread-safe. */
 void kq_set_gemm_tile_rows(int rows);
-/* Tuning hook without a counterpart in the reference: 1 makes dense skinny-M calls use the
- * workgroup-synchronous kernel (the one the gathered ops use) instead of the decoupled-wave one, 3
- * selects two-superblock units in the decoupled-wave kernel; 0 restores the default.  Process-wide,
- * not thread-safe. */
+/* Tuning hook without a counterpart in the reference: which skinny-M kernel dense calls use.
+ * 0 = default (decoupled-wave kernel up to 4 activation rows, diagonal kernel for 5 - 8),
+ * 1 = workgroup-synchronous kernel (the one the gathered ops use), 2 = decoupled-wave kernel always,
+ * 3 = decoupled-wave kernel with two-superblock units, 4 = diagonal kernel wherever K allows it.
+ * Process-wide, not thread-safe. */
 void kq_set_skinny_variant(int variant);
 
 /* out[b] = x[lhs[b]] . W[rhs[b]]^T for b < B; x batches are [M,K] matrices

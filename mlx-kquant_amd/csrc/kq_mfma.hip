@@ -126,6 +126,20 @@ struct SkGeom<KQ_Q3_K> {  // LDS block: hmask[32] | qs[64] | tail (wire bytes 94
   typedef u32x4_a2 piece_t;
 };
 
+// Accumulator rows of the "diagonal" kernel: a lane whose MFMA column is (row r, superblock q) wants
+// D rows 8 q + 4 kg + j, i.e. registers 4 q + j of the 16 it holds.
+// (J is a template parameter: with a function argument the element access is lowered as a dynamic
+// index -- sixteen selects per pick -- before inlining can make it constant.)
+template <bool DIAG, int J>
+__device__ __forceinline__ float pick_row(const f32x16& p, int q) {
+  if constexpr (!DIAG) {
+    return p[J];
+  } else {
+    const float lo = (q & 1) ? p[4 + J] : p[J], hi = (q & 1) ? p[12 + J] : p[8 + J];
+    return (q & 2) ? hi : lo;
+  }
+}
+
 // ------------------------------------------------------------------ q4_k superblock
 struct Q4kRaw {
   uint4 hdr;
@@ -167,10 +181,10 @@ __device__ __forceinline__ f16x8 q4k_frag(uint32_t wa, uint32_t wa8, uint32_t wb
 // (f16 index) for the superblock; xsum: X_j for the superblock, [8][XS] floats.
 // q5_k: the fifth bit of weight (sub-block j, i) is bit j of qh[i]; it is OR-ed into the code at
 // bit 4 (low-nibble sub-blocks, 1024 + q) or bit 8 (high-nibble ones, 1024 + 16 q).
-template <int C, int R, int XS>
+template <int C, int R, int XS, bool DIAG = false>
 __device__ __forceinline__ void q45k_superblock(const uint8_t* __restrict__ bl, int kg, float xscale,
                                                 const _Float16* __restrict__ xs_lane,
-                                                const float* __restrict__ xsum, float* acc) {
+                                                const float* __restrict__ xsum, float* acc, int q = 0) {
   constexpr int QS = C == KQ_Q4_K ? 16 : 48;  // offset of the nibble array
   Q4kRaw raw;
   const uint4* p4 = reinterpret_cast<const uint4*>(bl);
@@ -220,11 +234,11 @@ __device__ __forceinline__ void q45k_superblock(const uint8_t* __restrict__ bl, 
         }
         p = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, p, 0, 0, 0);
       }
-#pragma unroll
-      for (int r = 0; r < R; r++) {
-        acc[r] = fmaf(mul[j], p[r], acc[r]);
+      StaticFor<R>::run([&](auto rr) {
+        constexpr int r = decltype(rr)::value;
+        acc[r] = fmaf(mul[j], pick_row<DIAG, r>(p, q), acc[r]);
         acc[r] = fmaf(-sub[j], xsum[j * XS + r], acc[r]);
-      }
+      });
     }
   }
 }
@@ -234,10 +248,10 @@ __device__ __forceinline__ void q45k_superblock(const uint8_t* __restrict__ bl, 
 // 8 half + 2 si + l / 16.  Lane (row, kg) owns l = 16 s + 8 kg .. + 7 of MFMA s, so every MFMA covers
 // exactly one scale group and is folded with that group's scale.  The field is masked in place and
 // reads 1024 + 4^si q; the 4^si goes into the scale.
-template <int R, int XS>
+template <int R, int XS, bool DIAG = false>
 __device__ __forceinline__ void q2k_superblock(const uint8_t* __restrict__ bl, int kg, float xscale,
                                                const _Float16* __restrict__ xs_lane,
-                                               const float* __restrict__ xsum, float* acc) {
+                                               const float* __restrict__ xsum, float* acc, int q = 0) {
   const uint32_t magic = kq_opaque_vgpr(0x64006400u);
   const uint32_t mask[4] = {kq_opaque_sgpr(0x00030003u), kq_opaque_sgpr(0x000c000cu), kq_opaque_sgpr(0x00300030u),
                             kq_opaque_sgpr(0x00c000c0u)};
@@ -266,11 +280,11 @@ __device__ __forceinline__ void q2k_superblock(const uint8_t* __restrict__ bl, i
         const f32x16 p = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, __builtin_bit_cast(f16x8, v), f32x16{0}, 0, 0, 0);
         const float mulg = d * (float)(scb & 15) * (1.0f / (float)(1 << (2 * si)));
         const float subg = fmaf(mulg, 1024.0f, dmin * (float)(scb >> 4));
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-          acc[r] = fmaf(mulg, p[r], acc[r]);
+        StaticFor<R>::run([&](auto rr) {
+          constexpr int r = decltype(rr)::value;
+          acc[r] = fmaf(mulg, pick_row<DIAG, r>(p, q), acc[r]);
           acc[r] = fmaf(-subg, xsum[g * XS + r], acc[r]);
-        }
+        });
       }
     }
   }
@@ -278,10 +292,10 @@ __device__ __forceinline__ void q2k_superblock(const uint8_t* __restrict__ bl, i
 
 // q3_k: same 2-bit fields plus the high bit (bit 4 half + si of hmask[l], set = +4): the code is
 // 1024 + 4^si (q + 4 h) with zero point 4, scale d (sc - 32), sc the 6-bit scale of the group.
-template <int R, int XS>
+template <int R, int XS, bool DIAG = false>
 __device__ __forceinline__ void q3k_superblock(const uint8_t* __restrict__ bl, int kg, float xscale,
                                                const _Float16* __restrict__ xs_lane,
-                                               const float* __restrict__ xsum, float* acc) {
+                                               const float* __restrict__ xsum, float* acc, int q = 0) {
   const uint32_t magic = kq_opaque_vgpr(0x64006400u);
   const uint32_t mask[4] = {kq_opaque_sgpr(0x00030003u), kq_opaque_sgpr(0x000c000cu), kq_opaque_sgpr(0x00300030u),
                             kq_opaque_sgpr(0x00c000c0u)};
@@ -321,11 +335,11 @@ __device__ __forceinline__ void q3k_superblock(const uint8_t* __restrict__ bl, i
         const f32x16 p = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, __builtin_bit_cast(f16x8, v), f32x16{0}, 0, 0, 0);
         const float mulg = d * (float)((int)sc - 32) * (1.0f / (float)(1 << (2 * si)));
         const float subg = mulg * (1024.0f + (float)(4 << (2 * si)));
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-          acc[r] = fmaf(mulg, p[r], acc[r]);
+        StaticFor<R>::run([&](auto rr) {
+          constexpr int r = decltype(rr)::value;
+          acc[r] = fmaf(mulg, pick_row<DIAG, r>(p, q), acc[r]);
           acc[r] = fmaf(-subg, xsum[g * XS + r], acc[r]);
-        }
+        });
       }
     }
   }
@@ -336,9 +350,9 @@ __device__ __forceinline__ void q3k_superblock(const uint8_t* __restrict__ bl, i
 // (hf = half, t = 0..3, l = 0..31) has its low nibble in ql[64 hf + 32 (t & 1) + l] (high nibble of
 // the byte when t >= 2), its high bits in bits 2t, 2t+1 of qh[32 hf + l] and scale 8 hf + 2 t +
 // l / 16.  Lane (row, kg) takes l = 16 kg .. 16 kg + 15: one scale per lane and sub-block.
-template <int R>
+template <int R, bool DIAG = false>
 __device__ __forceinline__ void q6k_superblock(const uint8_t* __restrict__ bl, int kg, float dx,
-                                               const _Float16* __restrict__ xs_lane, float* acc) {
+                                               const _Float16* __restrict__ xs_lane, float* acc, int q = 0) {
   const uint32_t magic = kq_opaque_vgpr(0x64006400u);
   const uint32_t mask_q = kq_opaque_sgpr(0x00f000f0u), mask_h = kq_opaque_sgpr(0x03000300u);
   const uint4 scv = *reinterpret_cast<const uint4*>(bl + 192);
@@ -388,8 +402,10 @@ __device__ __forceinline__ void q6k_superblock(const uint8_t* __restrict__ bl, i
       }
     }
   }
-#pragma unroll
-  for (int r = 0; r < R; r++) acc[r] = fmaf(dx, p[r], acc[r]);
+  StaticFor<R>::run([&](auto rr) {
+    constexpr int r = decltype(rr)::value;
+    acc[r] = fmaf(dx, pick_row<DIAG, r>(p, q), acc[r]);
+  });
 }
 
 // ------------------------------------------------------------------ the kernel
@@ -935,6 +951,231 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny2_kernel(SkArgs a) {
   }
 }
 
+// ------------------------------------------------------------------ diagonal variant (dense calls, K % 1024 == 0)
+// The 32 columns of the MFMA are 8 weight rows x 4 ADJACENT superblocks instead of 32 rows x 1
+// superblock: lane l serves row l % 8 and superblock (l % 32) / 8 of the wave's current group of
+// four, and the 32 rows of the A operand are (superblock of the group, activation row), so the
+// useful results sit on the block diagonal (D rows 8 q + m for the columns of superblock q; the rest
+// of the MFMA is idle arithmetic on matrix cores that have nothing else to do).  What it buys:
+//   * a wave's unit of weight traffic is 8 rows x 576 contiguous bytes (q4_k) instead of 32 rows x
+//     144: reading the 33 MB gate/up matrix with nothing but that pattern takes 6.7 us, as fast as a
+//     linear sweep, against 8.2 us for 144-byte runs (fewer cache lines touched per load instruction);
+//   * a wave owns its 8 rows for all of K, so there is no cross-wave reduction; the four
+//     superblock partials of a row are summed with two shuffles at the end.
+#ifndef SK3_DEPTH
+#define SK3_DEPTH 1
+#endif
+template <int C, int DT, int MB>
+__global__ __launch_bounds__(SK_THREADS, 2) void skinny3_kernel(SkArgs a) {
+  using G = SkGeom<C>;
+  constexpr int R = MB < 4 ? MB : 4;
+  constexpr int NU = 4;                                        // units (groups of 4 superblocks) per chunk
+  constexpr int UPIECES = 8 * 4 * G::PP;                       // pieces of a unit: 8 rows x 4 superblocks
+  constexpr int UP = (UPIECES + 63) / 64;
+  constexpr int WROW = 4 * G::LBPB + 16;                       // LDS row stride: an odd number of 16-byte pieces
+  constexpr int WBUF = 8 * WROW + 64;                          // wave buffer (+ 32 d values of q6_k)
+  constexpr int XK = MB <= 4 ? 2 : 1;
+  constexpr int XG = MB * XK;
+  constexpr int D3 = SK3_DEPTH;                                // units in flight per wave
+  constexpr int XSB = 256 + 32;  // f16 per superblock of activations in LDS: the four superblocks a wave reads
+                                 // together start 64 bytes apart modulo the bank window
+
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int M = a.M, N = a.N, K = a.K, kch = a.kch;
+  const int kchunk = kch * XSB + 8;  // row stride: rows start 16 bytes apart modulo the bank window
+  // layout: xs f16 [MB][kchunk] | xsum f32 [kch*16][MB] | scratch | wave buffers
+  _Float16* xs = reinterpret_cast<_Float16*>(smem);
+  float* xsum = reinterpret_cast<float*>(smem + (size_t)MB * kchunk * 2);
+  float* scratch = xsum + kch * 16 * MB;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  uint8_t* wbuf = reinterpret_cast<uint8_t*>(scratch + 16) + wave * WBUF;
+  uint16_t* dq = reinterpret_cast<uint16_t*>(wbuf + 8 * WROW);  // [q][row]
+
+  const int n_in = lane & 31, kg = lane >> 5;
+  const int r8 = n_in & 7, q4 = n_in >> 3;  // this lane's MFMA column: row r8 of the wave, superblock q4 of the group
+  const int nsb = K >> 8;
+  const size_t row_bytes = (size_t)nsb * G::BPB;
+  const int row0 = blockIdx.x * 32 + 8 * wave;  // first row of this wave
+  int nrows = N - row0;
+  nrows = nrows < 0 ? 0 : (nrows > 8 ? 8 : nrows);
+  const uint8_t* wtile = a.w + (size_t)(nrows > 0 ? row0 : 0) * row_bytes;
+  const uint16_t* x16 = static_cast<const uint16_t*>(a.x);
+  const int crow = r8 < nrows ? r8 : 0;
+
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) acc[r] = 0.f;
+
+  // piece map of a unit: piece i = lane + 64 t -> (row, superblock of the group, piece of the block)
+  uint32_t goff[UP], loff[UP];
+  StaticFor<UP>::run([&](auto t) {
+    constexpr int T = decltype(t)::value;
+    const int i = lane + 64 * T, r = i / (4 * G::PP), qq = i % (4 * G::PP), sbl = qq / G::PP, pc = qq % G::PP;
+    goff[T] = (r < nrows && i < UPIECES) ? (uint32_t)r * (uint32_t)row_bytes + sbl * G::BPB + 16 * pc : 0;
+    loff[T] = (uint32_t)r * WROW + sbl * G::LBPB + 16 * pc;
+  });
+  // side channel (tail piece / d): lane < 32 -> its own MFMA column (row r8, superblock q4)
+  const bool side_ok = lane < 32 && r8 < nrows;
+  const uint8_t* side_src = wtile + (side_ok ? (size_t)r8 * row_bytes + q4 * G::BPB : 0);
+
+  const int sb_begin = a.ksplit > 1 ? (int)blockIdx.z * a.sb_per_split : 0;
+  const int sb_end = a.ksplit > 1 ? (sb_begin + a.sb_per_split < nsb ? sb_begin + a.sb_per_split : nsb) : nsb;
+  for (int sb0 = sb_begin; sb0 < sb_end; sb0 += kch) {
+    const int sbn = (sb_end - sb0 < kch) ? (sb_end - sb0) : kch;  // a multiple of 4
+    const int kc = sbn << 8, k0 = sb0 << 8;
+
+    // ---- activation loads first
+    const int gpr = kc >> 3;
+    u32x4 xreg[XG];
+    StaticFor<XG>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      int m = T / XK;
+      m = m < M ? m : M - 1;
+      int kgi = tid + (T % XK) * SK_THREADS;
+      kgi = kgi < gpr ? kgi : 0;
+      xreg[T] = *reinterpret_cast<const u32x4*>(x16 + (size_t)m * K + k0 + 8 * kgi);
+    });
+
+    // ---- this wave's weight stream: unit u = superblocks [4 u, 4 u + 4) of its 8 rows, one unit in flight
+    u32x4 wreg[D3 * UP], treg[D3];
+    uint16_t dreg[D3];
+    auto issue = [&](auto uu) {
+      constexpr int u = decltype(uu)::value;
+      const bool live = 4 * u < sbn;  // uniform
+      const size_t sboff = (size_t)(sb0 + (live ? 4 * u : 0)) * G::BPB;
+      StaticFor<UP>::run([&](auto t) {
+        constexpr int T = decltype(t)::value;
+        wreg[(u % D3) * UP + T] = *reinterpret_cast<const typename G::piece_t*>(wtile + sboff + goff[T]);
+      });
+      if constexpr (G::SIDE_D) dreg[u % D3] = *reinterpret_cast<const uint16_t*>(side_src + sboff + 208);
+      if constexpr (G::TAIL) treg[u % D3] = *reinterpret_cast<const u32x4_a2*>(side_src + sboff + (G::BPB - 16));
+    };
+    StaticFor<D3>::run([&](auto uu) { issue(uu); });
+
+    // ---- activations -> f16 in LDS (+ sums)
+    if (sb0 > sb_begin) lds_barrier();
+    float xscale = 1.0f, inv = 1.0f;
+    if constexpr (DT == KQ_BF16) {
+      float amax = 0.f;
+      StaticFor<XG>::run([&](auto t) {
+        const u32x4 v = xreg[decltype(t)::value];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] << 16)));
+          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] & 0xffff0000u)));
+        }
+      });
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+      if (lane == 0) scratch[wave] = amax;
+      lds_barrier();
+      amax = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+      const uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff;
+      if (eb != 0 && eb != 0xff) {
+        int e = (int)eb - 127 - 14;
+        if (e < -100) e = -100;
+        xscale = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+        inv = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
+      }
+    }
+    StaticFor<XG>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      constexpr int m = T / XK;
+      const int kgi = tid + (T % XK) * SK_THREADS;
+      if (kgi < gpr) {
+        const int kk = kgi << 3;
+        const u32x4 v = xreg[T];
+        _Float16 h[8];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          if constexpr (DT == KQ_BF16) {
+            h[2 * e] = (_Float16)(__builtin_bit_cast(float, v[e] << 16) * inv);
+            h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, v[e] & 0xffff0000u) * inv);
+          } else {
+            h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] & 0xffff));
+            h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
+          }
+        }
+        const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+        *reinterpret_cast<f16x8*>(xs + (size_t)m * kchunk + (kk >> 8) * XSB + (kk & 255)) = v8;
+        if constexpr (G::XSUM != 0) {
+          float sum = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; e++) sum += (float)h[e];
+          sum += __shfl_xor(sum, 1);
+          if constexpr (G::XSUM == 32) {
+            sum += __shfl_xor(sum, 2);
+            if ((tid & 3) == 0) xsum[(kk >> 5) * MB + m] = sum;
+          } else {
+            if ((tid & 1) == 0) xsum[(kk >> 4) * MB + m] = sum;
+          }
+        }
+      }
+    });
+    lds_barrier();  // the chunk's activations are visible to every wave; from here on waves run free
+
+    // A operand: MFMA row l % 32 = (superblock q of the group, activation row): rows beyond MB alias real ones
+    const _Float16* xs_lane = xs + (size_t)(r8 & (MB - 1)) * kchunk + XSB * q4 + G::KGOFF * kg;
+    const float* xsum_lane = xsum + (size_t)(G::XSUM == 16 ? 16 : 8) * MB * q4 + (MB == 8 ? 4 * kg : 0);
+    const uint8_t* bl = wbuf + crow * WROW + q4 * G::LBPB;
+    StaticFor<NU>::run([&](auto uu) {
+      constexpr int u = decltype(uu)::value;
+      if (4 * u >= sbn) return;  // uniform
+      StaticFor<UP>::run([&](auto t) {
+        constexpr int T = decltype(t)::value;
+        if (lane + 64 * T < UPIECES) *reinterpret_cast<u32x4*>(wbuf + loff[T]) = wreg[(u % D3) * UP + T];
+      });
+      if constexpr (G::SIDE_D) {
+        if (lane < 32) dq[lane] = dreg[u % D3];
+      }
+      if constexpr (G::TAIL) {
+        if (lane < 32) *reinterpret_cast<u32x4*>(wbuf + r8 * WROW + q4 * G::LBPB + 16 * G::PP) = treg[u % D3];
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      if constexpr (u + D3 < NU) issue(std::integral_constant<int, u + D3>{});
+      constexpr int sb = 4 * u;  // superblock of q4 = 0 within the chunk
+      if constexpr (C == KQ_Q4_K || C == KQ_Q5_K) {
+        q45k_superblock<C, R, MB, true>(bl, kg, xscale, xs_lane + XSB * sb, xsum_lane + 8 * MB * sb, acc, q4);
+      } else if constexpr (C == KQ_Q2_K) {
+        q2k_superblock<R, MB, true>(bl, kg, xscale, xs_lane + XSB * sb, xsum_lane + 16 * MB * sb, acc, q4);
+      } else if constexpr (C == KQ_Q3_K) {
+        q3k_superblock<R, MB, true>(bl, kg, xscale, xs_lane + XSB * sb, xsum_lane + 16 * MB * sb, acc, q4);
+      } else {
+        const float dx = kq::h2f(dq[n_in < 32 ? (crow + 8 * q4) : 0]) * xscale;
+        q6k_superblock<R, true>(bl, kg, dx, xs_lane + XSB * sb, acc, q4);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    });
+  }
+
+  // ---- sum the four superblock partials of a row (lanes r8 + 8 q), store
+  const size_t plane = (size_t)M * N;
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    float v = acc[r];
+    v += __shfl_xor(v, 8);
+    v += __shfl_xor(v, 16);
+    const int m = 4 * kg + r;
+    if (q4 == 0 && m < M && r8 < nrows) {
+      if (a.ksplit > 1) {
+        a.partial[blockIdx.z * plane + (size_t)m * N + row0 + r8] = v;
+      } else {
+        uint16_t* yo = static_cast<uint16_t*>(a.y) + (size_t)m * N + row0 + r8;
+        *yo = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+      }
+    }
+  }
+}
+
+template <int C>
+size_t sk3_lds_bytes(int kch, int MB) {
+  using G = SkGeom<C>;
+  return (size_t)MB * (kch * 288 + 8) * 2 + (size_t)kch * 16 * MB * 4 + 64 + SK_WAVES * (8 * (4 * G::LBPB + 16) + 64);
+}
+
 template <int C>
 size_t sk2_lds_bytes(int kch, int MB, int usb) {
   using G = SkGeom<C>;
@@ -963,7 +1204,7 @@ size_t sk_lds_bytes(int rows, int kch, int MB) {
          16 * SK_THREADS + 32 * 16 * 2;
 }
 
-int g_sk_variant = 0;  // kq_set_skinny_variant: 1 forces the workgroup-synchronous kernel for dense calls
+int g_sk_variant = 0;  // kq_set_skinny_variant: 0 default, 1 synchronous, 2 decoupled, 3 two-superblock units, 4 diagonal
 
 // Split-K plan of a dense call: with few row tiles the K range is cut so that about 768
 // workgroups of full 32-row tiles exist; every split keeps at least one superblock per wave.
@@ -1013,6 +1254,32 @@ int launch_skinny(SkArgs a, int items, void* ws, hipStream_t s) {
     // dense call: decoupled-wave variant (measured 3 - 25 % faster than the synchronous kernel on every
     // decode shape of the sweep)
     if (items == 1 && g_sk_variant != 1) {
+      // Diagonal variant (a wave owns 8 rows x 4 adjacent superblocks, no cross-wave reduction): measured
+      // 4 - 10 % faster at 5 - 8 activation rows and level or slightly slower below, so it is the default
+      // only there; kq_set_skinny_variant(4) selects it wherever the shape allows.
+      const bool diag_shape = ((a.K >> 8) & 3) == 0 && (kch & 3) == 0 && (splits == 1 || (a.sb_per_split & 3) == 0);
+      if (diag_shape && (g_sk_variant == 4 || (g_sk_variant == 0 && MB == 8))) {
+        // 32-row tiles always (8 rows per wave)
+        const int tiles3 = (a.N + 31) / 32;
+        const size_t lds3 = sk3_lds_bytes<C>(kch, MB);
+        a.rows_per_tile = 32;
+        a.kch = kch;
+        static bool attr3_set = false;
+        if (!attr3_set) {
+          KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(skinny3_kernel<C, DT, MB>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 120 * 1024));
+          attr3_set = true;
+        }
+        hipLaunchKernelGGL((skinny3_kernel<C, DT, MB>), dim3(tiles3, 1, splits), dim3(SK_THREADS), lds3, s, a);
+        KQ_HIP_CHECK(hipGetLastError());
+        if (splits > 1) {
+          const int count = a.M * a.N;
+          hipLaunchKernelGGL((splitk_reduce_kernel<DT>), dim3((count + 255) / 256), dim3(256), 0, s, a.partial,
+                             static_cast<uint16_t*>(a.y), count, splits);
+          KQ_HIP_CHECK(hipGetLastError());
+        }
+        return KQ_OK;
+      }
       // Units of two adjacent superblocks read HBM in a friendlier pattern but measured 15 - 60 % slower
       // end to end (two superblocks of decode per unit leave too little overlap), so they are only
       // selectable through kq_set_skinny_variant(3).  Such a unit may read one superblock past an

@@ -77,13 +77,15 @@ def test_qmm_gemv_unaligned_rows_and_tensor_end(kq, codec):
 
 @pytest.mark.parametrize("codec", ["q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_qmm_skinny_both_variants(kq, codec):
-    """Dense skinny calls through the workgroup-synchronous kernel (kq_set_skinny_variant(1)) and the
-    two-superblock-unit form of the decoupled-wave kernel (3) as well as the default."""
+    """Dense skinny calls through every selectable kernel: workgroup-synchronous (1), decoupled-wave (2),
+    its two-superblock-unit form (3) and the diagonal kernel (4; shapes whose K is not a multiple of 1024
+    fall back to the decoupled one)."""
     lib = kq._load()
     try:
-        for variant in (1, 3):
+        for variant in (1, 2, 3, 4):
             lib.kq_set_skinny_variant(variant)
-            for M, N, K in ((1, 1000, 768), (8, 520, 4352), (3, 4100, 1024), (2, 300, 4096), (5, 4200, 14336)):
+            for M, N, K in ((1, 1000, 768), (8, 520, 4352), (3, 4100, 1024), (2, 300, 4096), (5, 4200, 14336),
+                            (7, 100, 2048)):
                 wire = _wire(codec, N, K, seed=41)
                 xb, xt = make_x((M, K), "bfloat16", seed=42)
                 got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
