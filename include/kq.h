@@ -94,12 +94,16 @@ void kq_set_skinny_variant(int variant);
 /* out[b] = x[lhs[b]] . W[rhs[b]]^T for b < B; x batches are [M,K] matrices
  * `x_batch_stride` elements apart, experts are [N, bytes_per_row] wire matrices
  * `w_expert_stride_bytes` apart (64-bit, so strided / >2 GiB stacks work); out is
- * [B, M, N] dense.  `rhs_sorted` != 0 promises rhs is non-decreasing.
+ * [B, M, N] dense.  `E` = number of matrices in the stack (entries whose rhs index is >= E are
+ * skipped by the batched path and must not occur).  `rhs_sorted` != 0 promises rhs is
+ * non-decreasing.  With a workspace of kq_gather_qmm_workspace_size bytes and more than 16 output
+ * rows (B * M) the entries are grouped by expert on the device, so an expert's wire bytes are
+ * streamed once per 32 rows instead of once per entry; without one every entry is computed on its own.
  * Replaces KQuantGatherQMM::eval_cpu, reference src/kquant_gather.cpp:470-746
  * (kquant_qmm_cpu_batch, src/kquant_cpu_decode.cpp:1361-1527). */
-size_t kq_gather_qmm_workspace_size(int B, int M, int N, int K, int transpose, int codec, int dtype);
+size_t kq_gather_qmm_workspace_size(int B, int M, int E, int N, int K, int transpose, int codec, int dtype);
 int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_dev,
-                  const uint32_t* rhs_idx_dev, void* out_dev, int B, int M, int N, int K,
+                  const uint32_t* rhs_idx_dev, void* out_dev, int B, int M, int E, int N, int K,
                   int64_t x_batch_stride, int64_t w_expert_stride_bytes, int transpose, int rhs_sorted,
                   int codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
 

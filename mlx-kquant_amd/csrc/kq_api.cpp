@@ -148,19 +148,35 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
   return kq_launch_gemv_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
 }
 
-size_t kq_gather_qmm_workspace_size(int B, int M, int N, int K, int transpose, int codec, int dtype) {
-  (void)B; (void)M; (void)N; (void)K; (void)transpose; (void)codec; (void)dtype;
-  return 0;
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// Batched gather_qmm: B * M output rows, gathered into a dense [P, K] matrix + a per-row expert id.
+static bool gather_batched_shape(int B, int M, int E, int N, int K, int transpose, int codec, int64_t* P_out) {
+  const int64_t P = (int64_t)B * M;
+  *P_out = P;
+  if (!transpose || E <= 0 || P <= 16 || P > 0x7fffffff || (K & 7)) return false;
+  return kq_moe_grouped_supported((int)P, E, N, K, codec) || kq_anymma_moe_supported((int)P, E, N, K, codec);
 }
 
+size_t kq_gather_qmm_workspace_size(int B, int M, int E, int N, int K, int transpose, int codec, int dtype) {
+  int64_t P;
+  if (B <= 0 || M <= 0 || !codec_ok(codec) || !gather_batched_shape(B, M, E, N, K, transpose, codec, &P)) return 0;
+  return align256((size_t)P * K * 2) + align256((size_t)P * 4) + kq_moe_workspace_size((int)P, 1, E, N, K, 0, codec, dtype);
+}
+
+static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
+                           const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
+                           int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
+                           size_t ws_bytes, hipStream_t s);
+
 int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_dev, const uint32_t* rhs_idx_dev,
-                  void* out_dev, int B, int M, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride_bytes,
-                  int transpose, int rhs_sorted, int codec, int dtype, void* workspace_dev, size_t workspace_bytes,
-                  void* stream) {
-  (void)workspace_dev; (void)workspace_bytes; (void)rhs_sorted;
+                  void* out_dev, int B, int M, int E, int N, int K, int64_t x_batch_stride,
+                  int64_t w_expert_stride_bytes, int transpose, int rhs_sorted, int codec, int dtype,
+                  void* workspace_dev, size_t workspace_bytes, void* stream) {
+  (void)rhs_sorted;
   if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: unknown codec id %d", codec);
   if (!half_dtype(dtype)) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: activations must be float16 or bfloat16");
-  if (B < 0 || M < 0 || N < 0 || K < 0) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: negative dimension");
+  if (B < 0 || M < 0 || N < 0 || K < 0 || E < 0) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: negative dimension");
   const int inner = transpose ? K : N;  // the quantized (row) dimension of the expert matrices
   if (inner % kCodecs[codec].weights_per_block)
     return kq_set_error(KQ_ERR_INVALID, "gather_qmm: quantized row length %d is not a multiple of %d", inner,
@@ -168,19 +184,38 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
   if (B == 0 || M == 0 || N == 0) return KQ_OK;
   if (!x_dev || !w_dev || !out_dev || !lhs_idx_dev || !rhs_idx_dev)
     return kq_set_error(KQ_ERR_INVALID, "gather_qmm: null buffer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
   if (!transpose)
     return kq_launch_gather_nt_generic(x_dev, static_cast<const uint8_t*>(w_dev), lhs_idx_dev, rhs_idx_dev, out_dev, B,
-                                       M, N, K, x_batch_stride, w_expert_stride_bytes, codec, dtype,
-                                       static_cast<hipStream_t>(stream));
+                                       M, N, K, x_batch_stride, w_expert_stride_bytes, codec, dtype, s);
+  // many output rows: gather them into a dense matrix and run the expert-grouped kernels
+  int64_t P;
+  if (workspace_dev && gather_batched_shape(B, M, E, N, K, transpose, codec, &P) &&
+      !(reinterpret_cast<uintptr_t>(workspace_dev) & 255) && !(reinterpret_cast<uintptr_t>(x_dev) & 15) &&
+      !(x_batch_stride & 7)) {
+    const size_t need = kq_gather_qmm_workspace_size(B, M, E, N, K, transpose, codec, dtype);
+    if (workspace_bytes >= need) {
+      uint8_t* wsb = static_cast<uint8_t*>(workspace_dev);
+      void* xg = wsb;
+      uint32_t* idx_rows = reinterpret_cast<uint32_t*>(wsb + align256((size_t)P * K * 2));
+      const size_t used = align256((size_t)P * K * 2) + align256((size_t)P * 4);
+      const int rcr = kq_launch_gather_rows(x_dev, lhs_idx_dev, rhs_idx_dev, xg, idx_rows, B, M, K, x_batch_stride, s);
+      if (rcr) return rcr;
+      const int rcg = try_moe_grouped("gather_qmm", xg, w_dev, nullptr, idx_rows, nullptr, nullptr, out_dev, (int)P, 1, E,
+                                      N, K, w_expert_stride_bytes, 0, 0, 0.f, 0.f, codec, dtype, wsb + used,
+                                      workspace_bytes - used, s);
+      if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
+    }
+  }
   {
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
                                            out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0, 0, 0.f,
-                                           codec, dtype, static_cast<hipStream_t>(stream));
+                                           codec, dtype, s);
     if (rct != KQ_ERR_UNSUPPORTED) return rct;
   }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
                                   nullptr, nullptr, out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0,
-                                  0, 0.f, 0.f, codec, dtype, static_cast<hipStream_t>(stream));
+                                  0, 0.f, 0.f, codec, dtype, s);
 }
 
 static int check_moe(const char* op, int T, int R, int E, int N, int K, int codec, int dtype) {

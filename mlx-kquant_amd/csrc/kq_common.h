@@ -87,6 +87,10 @@ size_t kq_moe_grouped_workspace_bytes(int rows, int P, int E, int K);
 int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, void* out, int rows,
                           int P, int E, int N, int K, int x_div, int64_t w_expert_stride, int glu, int act,
                           float limit, int codec, int dtype, void* ws, hipStream_t s);
+// Gathered activations of a batched gather_qmm: xg[b*M + m][:] = x[lhs[b]][m][:], idx_rows[b*M + m] = rhs[b]
+// (16-bit elements; K a multiple of 8, x and xg 16-byte aligned).
+int kq_launch_gather_rows(const void* x, const uint32_t* lhs, const uint32_t* rhs, void* xg, uint32_t* idx_rows, int B,
+                          int M, int K, int64_t x_batch_stride, hipStream_t s);
 // Matrix-core GEMM for every codec (exact bf16 x 3 split of the reference-order decoded weights):
 // prefill, and the batched MoE ops with biases and every activation.
 bool kq_anymma_supported(int M, int N, int K, int codec);

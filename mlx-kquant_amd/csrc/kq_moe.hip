@@ -85,6 +85,21 @@ __global__ __launch_bounds__(SORT_THREADS) void moe_sort_kernel(const uint32_t* 
   }
 }
 
+// ------------------------------------------------------------------ row gather (batched gather_qmm)
+// One workgroup per output row p = b*M + m: copies the K 16-bit activations of x[lhs[b]][m] to
+// xg[p] and notes the row's expert, so that the grouped kernels below see a plain [P, K] matrix.
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x, const uint32_t* __restrict__ lhs,
+                                                          const uint32_t* __restrict__ rhs, uint16_t* __restrict__ xg,
+                                                          uint32_t* __restrict__ idx_rows, int M, int K,
+                                                          int64_t x_batch_stride) {
+  const int p = blockIdx.x, b = p / M, m = p - b * M;
+  const uint16_t* src = x + (size_t)lhs[b] * (size_t)x_batch_stride + (size_t)m * K;
+  uint16_t* dst = xg + (size_t)p * K;
+  for (int g = threadIdx.x; g < (K >> 3); g += 256)
+    *reinterpret_cast<u32x4*>(dst + 8 * g) = *reinterpret_cast<const u32x4*>(src + 8 * g);
+  if (threadIdx.x == 0) idx_rows[p] = rhs[b];
+}
+
 // ------------------------------------------------------------------ grouped GEMM
 struct MoeArgs {
   const _Float16* xh;   // [rows][K] f16 activations (prepass), row = pair / x_div
@@ -339,6 +354,15 @@ int kq_launch_moe_sort(const uint32_t* idx, int P, int E, void* order, void* seg
   if (E > SORT_MAX_E) return KQ_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(SORT_THREADS), 0, s, idx, P, E, static_cast<int*>(order),
                      static_cast<Segment*>(segs), static_cast<int*>(nseg));
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
+int kq_launch_gather_rows(const void* x, const uint32_t* lhs, const uint32_t* rhs, void* xg, uint32_t* idx_rows, int B,
+                          int M, int K, int64_t x_batch_stride, hipStream_t s) {
+  if (B <= 0 || M <= 0) return KQ_OK;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)B * (unsigned)M), dim3(256), 0, s, static_cast<const uint16_t*>(x),
+                     lhs, rhs, static_cast<uint16_t*>(xg), idx_rows, M, K, x_batch_stride);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }

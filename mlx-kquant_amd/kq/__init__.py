@@ -67,8 +67,8 @@ def _load():
     lib.kq_qmm_workspace_size.argtypes = [i, i, i, i, i, i]
     lib.kq_qmm.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
     lib.kq_gather_qmm_workspace_size.restype = sz
-    lib.kq_gather_qmm_workspace_size.argtypes = [i, i, i, i, i, i, i]
-    lib.kq_gather_qmm.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i64, i64, i, i, i, i, vp, sz, vp]
+    lib.kq_gather_qmm_workspace_size.argtypes = [i, i, i, i, i, i, i, i]
+    lib.kq_gather_qmm.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, i64, i64, i, i, i, i, vp, sz, vp]
     lib.kq_moe_workspace_size.restype = sz
     lib.kq_moe_workspace_size.argtypes = [i, i, i, i, i, i, i, i]
     lib.kq_moe_glu_gather.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, f, f, i, i, vp, sz, vp]
@@ -255,14 +255,15 @@ def gather_qmm(x, w, scales, kquant_type, lhs_indices=None, rhs_indices=None, tr
         w3 = w.contiguous().reshape(-1, w.shape[-2], w.shape[-1])
     estride = w3.stride(0) if w3.shape[0] > 1 else w3.shape[1] * w3.shape[2]
     B = lhs.numel()
+    E = w3.shape[0]
     out = torch.empty(idx_shape + [M, N], dtype=out_type, device=x.device)
     right_sorted = bool(sorted_indices) and lhs_indices is None
     lib = _load()
     with torch.cuda.device(x.device):
-        ws_bytes = lib.kq_gather_qmm_workspace_size(B, M, N, K, int(bool(transpose)), cid, _DT[out_type])
+        ws_bytes = lib.kq_gather_qmm_workspace_size(B, M, E, N, K, int(bool(transpose)), cid, _DT[out_type])
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
-        _check(lib.kq_gather_qmm(x_c.data_ptr(), w3.data_ptr(), lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), B, M, N,
-                                 K, M * K, estride, int(bool(transpose)), int(right_sorted), cid, _DT[out_type],
+        _check(lib.kq_gather_qmm(x_c.data_ptr(), w3.data_ptr(), lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), B, M, E,
+                                 N, K, M * K, estride, int(bool(transpose)), int(right_sorted), cid, _DT[out_type],
                                  ws.data_ptr() if ws is not None else None, ws_bytes, sp))
     return out
 

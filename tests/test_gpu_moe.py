@@ -50,6 +50,26 @@ def test_gather_qmm(kq, codec, M):
     assert rel_l2(dev_to_bits(got).reshape(B, M, N), want, "float16") <= TOL
 
 
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k", "q3_k", "iq4_xs", "iq2_xxs", "q8_0", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("M", [1, 3])
+def test_gather_qmm_batched(kq, codec, M):
+    """More than 16 output rows: entries are gathered and grouped by expert on the device (the
+    sort-by-expert arm of KQuantGatherQMM::eval_cpu, src/kquant_gather.cpp:584-593).  General lhs with
+    repeats, an expert nobody picks, 2-D index arrays, both half dtypes."""
+    E, N, K, B, XB = 6, 136, 768 if codec not in ("mxfp4", "nvfp4") else 320, 44, 9
+    wire = _stack(codec, E, N, K, seed=61)
+    rng = np.random.default_rng(62)
+    lhs = rng.integers(0, XB, B)
+    rhs = rng.integers(0, E - 1, B)  # expert E-1 stays idle
+    for dtype in ("bfloat16", "float16"):
+        xb, xt = make_x((XB, M, K), dtype, seed=63, scale=0.5)
+        got = kq.gather_qmm(xt, wire_to_dev(wire), None, codec, lhs_indices=_idx_dev(lhs.reshape(4, 11)),
+                            rhs_indices=_idx_dev(rhs.reshape(4, 11)))
+        want = O.gather_qmm(xb, wire, codec, lhs, rhs, True, dtype)
+        assert tuple(got.shape) == (4, 11, M, N)
+        assert rel_l2(dev_to_bits(got).reshape(B, M, N), want, dtype) <= TOL, (codec, M, dtype)
+
+
 @pytest.mark.parametrize("codec", ["q4_k", "q8_0", "iq4_nl", "q6_k"])
 def test_gather_qmm_no_transpose(kq, codec):
     """transpose=False: every expert decodes to [K, N] (the MLA / LoRA-vjp orientation)."""
