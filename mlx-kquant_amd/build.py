@@ -23,6 +23,7 @@ SOURCES = [
     ("kq_gemm.hip", []),
     ("kq_moe.hip", []),
     ("kq_anymma.hip", ["-ffp-contract=off"]),
+    ("kq_codes.hip", []),
 ]
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",

@@ -89,6 +89,8 @@ struct AnyArgs {
   int M, N, K, x_div, act, mtiles;
   int64_t w_expert_stride;
   float limit, alpha;
+  float* partial;       // dense split-K: f32 partial sums [ksplit][M][N] (null: round and store y)
+  int steps_per_split;  // dense: K steps per blockIdx.y
 };
 
 // MODE 0 = dense, 1 = grouped, 2 = grouped GLU (slab = 64 gate + 64 up rows; waves 0/2 gate, 1/3 up)
@@ -172,13 +174,18 @@ __global__ __launch_bounds__(AM_THREADS, 1) void any_mma_kernel(AnyArgs a) {
   }
   const uint8_t* w_end2 = wbase2 + (size_t)N * row_bytes;
 
+  // dense tiles past M are zero-filled without a load (a skinny call has 32 - M such rows)
+  bool a_live[APT];
+#pragma unroll
+  for (int t = 0; t < APT; t++) a_live[t] = MODE != 0 || m0 + a_slot + 8 * t < a.M;
+
   u32x4 areg[APT], wreg[G::WPT];
   auto issue = [&](int st) {
     const int kvalid = K - AM_STEP * st;  // weights of this step that exist (>= 256 except in the last step)
 #pragma unroll
     for (int t = 0; t < APT; t++) {
       u32x4 v = {0, 0, 0, 0};
-      if (8 * a_pc < kvalid) v = *reinterpret_cast<const u32x4*>(a_src[t] + (size_t)AM_STEP * st);
+      if (8 * a_pc < kvalid && a_live[t]) v = *reinterpret_cast<const u32x4*>(a_src[t] + (size_t)AM_STEP * st);
       areg[t] = v;
     }
     const int bvalid = kvalid >= AM_STEP ? G::BYTES : (kvalid / G::WPB) * G::BPB;  // wire bytes of this step per row
@@ -238,11 +245,17 @@ __global__ __launch_bounds__(AM_THREADS, 1) void any_mma_kernel(AnyArgs a) {
   const uint8_t* b_lane = b_lds + (wave * 32 + l32) * G::LROW;
   const uint8_t* a_lane = a_lds + l32 * A_STRIDE + 16 * kg;
 
-  issue(0);
-  for (int st = 0; st < nsteps; st++) {
-    if (st > 0) lds_barrier();  // everyone is done reading the previous step
+  // dense split-K: blockIdx.y owns K steps [st0, st1)
+  int st0 = 0, st1 = nsteps;
+  if constexpr (MODE == 0) {
+    st0 = (int)blockIdx.y * a.steps_per_split;
+    st1 = st0 + a.steps_per_split < nsteps ? st0 + a.steps_per_split : nsteps;
+  }
+  issue(st0);
+  for (int st = st0; st < st1; st++) {
+    if (st > st0) lds_barrier();  // everyone is done reading the previous step
     park();
-    if (st + 1 < nsteps) issue(st + 1);
+    if (st + 1 < st1) issue(st + 1);
     lds_barrier();
     const int kvalid = K - AM_STEP * st;
 #pragma unroll 2
@@ -278,12 +291,18 @@ __global__ __launch_bounds__(AM_THREADS, 1) void any_mma_kernel(AnyArgs a) {
   auto store = [&](size_t off, float v) { y[off] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v); };
   if constexpr (MODE == 0) {
     const int n = n0 + wave * 32 + l32;
+    float* part = a.partial ? a.partial + (size_t)blockIdx.y * a.M * N : nullptr;
 #pragma unroll
     for (int t = 0; t < MT; t++)
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         const int m = m0 + t * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
-        if (m < a.M && n < N) store((size_t)m * N + n, acc[t][i]);
+        if (m < a.M && n < N) {
+          if (part)
+            part[(size_t)m * N + n] = acc[t][i];
+          else
+            store((size_t)m * N + n, acc[t][i]);
+        }
       }
   } else if constexpr (MODE == 1) {
     const int col = wave * 32 + l32;
@@ -319,6 +338,17 @@ __global__ __launch_bounds__(AM_THREADS, 1) void any_mma_kernel(AnyArgs a) {
   }
 }
 
+// y[i] = round(sum over splits of partial[split][i])
+template <int DT>
+__global__ __launch_bounds__(256) void any_splitk_reduce_kernel(const float* __restrict__ partial, uint16_t* __restrict__ y,
+                                                                int count, int splits) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  float v = 0.f;
+  for (int sp = 0; sp < splits; sp++) v += partial[(size_t)sp * count + i];
+  y[i] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+}
+
 template <int C, int DT, int MT, int MODE>
 int launch_any(const AnyArgs& a, dim3 grid, hipStream_t s) {
   using G = StepGeom<C>;
@@ -342,6 +372,25 @@ constexpr int SEG_M = 32;
 template <int C>
 struct AnyRun {
   static int run(const AnyArgs& a, int mode, int dt, int P, int E, hipStream_t s) {
+    if (mode == 0 && a.M <= 32) {
+      // skinny call: one 32-row activation tile, K split over blockIdx.y when the caller brought a workspace
+      AnyArgs b = a;
+      b.mtiles = 1;
+      const int nsteps = (a.K + AM_STEP - 1) / AM_STEP;
+      const int splits = (nsteps + a.steps_per_split - 1) / a.steps_per_split;
+      const dim3 grid((a.N + AM_BN - 1) / AM_BN, splits);
+      const int rc = dt == KQ_F16 ? launch_any<C, KQ_F16, 1, 0>(b, grid, s) : launch_any<C, KQ_BF16, 1, 0>(b, grid, s);
+      if (rc || !a.partial) return rc;
+      const int count = a.M * a.N;
+      if (dt == KQ_F16)
+        hipLaunchKernelGGL(any_splitk_reduce_kernel<KQ_F16>, dim3((count + 255) / 256), dim3(256), 0, s, a.partial,
+                           static_cast<uint16_t*>(a.y), count, splits);
+      else
+        hipLaunchKernelGGL(any_splitk_reduce_kernel<KQ_BF16>, dim3((count + 255) / 256), dim3(256), 0, s, a.partial,
+                           static_cast<uint16_t*>(a.y), count, splits);
+      KQ_HIP_CHECK(hipGetLastError());
+      return KQ_OK;
+    }
     if (mode == 0) {
       // 128-row tiles for bf16 activations, 64-row tiles for f16 (two bf16 planes in LDS)
       if (dt == KQ_BF16) {
@@ -386,9 +435,27 @@ bool kq_anymma_supported(int M, int N, int K, int codec) {
          K % kq_geom(codec).wpb == 0;
 }
 
-// Prefill GEMM, any codec.  No workspace.
+// K steps per workgroup of a skinny (M <= 32) dense call: K is split until about 512 workgroups exist.
+static int any_skinny_steps_per_split(int N, int K) {
+  const int nsteps = (K + AM_STEP - 1) / AM_STEP, tiles = (N + AM_BN - 1) / AM_BN;
+  int want = (512 + tiles - 1) / tiles;
+  if (want > nsteps) want = nsteps;
+  if (want < 1) want = 1;
+  return (nsteps + want - 1) / want;
+}
+
+// f32 partial sums of the split-K skinny call (0: no split)
+size_t kq_anymma_dense_workspace_bytes(int M, int N, int K) {
+  if (M > 32 || M <= 0 || N <= 0 || K <= 0) return 0;
+  const int nsteps = (K + AM_STEP - 1) / AM_STEP, per = any_skinny_steps_per_split(N, K);
+  const int splits = (nsteps + per - 1) / per;
+  return splits > 1 ? (size_t)splits * M * N * 4 : 0;
+}
+
+// Dense matmul, any codec: prefill tiles, or (M <= 32) one activation tile with K split across
+// workgroups when `ws` holds kq_anymma_dense_workspace_bytes.
 int kq_launch_anymma_dense(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
-                           hipStream_t s) {
+                           void* ws, size_t ws_bytes, hipStream_t s) {
   if (!kq_anymma_supported(M, N, K, codec) || (reinterpret_cast<uintptr_t>(x) & 15)) return KQ_ERR_UNSUPPORTED;
   AnyArgs a{};
   a.x = x;
@@ -400,6 +467,14 @@ int kq_launch_anymma_dense(const void* x, const uint8_t* w, void* y, int M, int 
   a.N = N;
   a.K = K;
   a.x_div = 1;
+  a.steps_per_split = (K + AM_STEP - 1) / AM_STEP;
+  if (M <= 32) {
+    const size_t need = kq_anymma_dense_workspace_bytes(M, N, K);
+    if (need && ws && ws_bytes >= need && !(reinterpret_cast<uintptr_t>(ws) & 15)) {
+      a.partial = static_cast<float*>(ws);
+      a.steps_per_split = any_skinny_steps_per_split(N, K);
+    }
+  }
   return dispatch_any(codec, a, 0, dtype, 0, 1, s);
 }
 

@@ -111,7 +111,10 @@ size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int 
   (void)dtype;
   if (!transpose || !codec_ok(codec)) return 0;
   if (kq_gemm_supported(M, N, K, codec)) return kq_gemm_workspace_bytes(M, K);
-  return kq_qmm_tuned_workspace_bytes(M, N, K, codec);  // split-K partial sums of the skinny kernels (optional)
+  // split-K partial sums (optional) of whichever skinny kernel takes the call
+  const size_t tuned = kq_qmm_tuned_workspace_bytes(M, N, K, codec);
+  const size_t any = (M > 8 && kq_anymma_supported(M, N, K, codec)) ? kq_anymma_dense_workspace_bytes(M, N, K) : 0;
+  return tuned > any ? tuned : any;
 }
 
 int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int transpose, int codec,
@@ -139,11 +142,14 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
   }
   if (M > 8) {
-    const int rca = kq_launch_anymma_dense(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+    const int rca = kq_launch_anymma_dense(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype,
+                                           workspace_dev, workspace_bytes, s);
     if (rca != KQ_ERR_UNSUPPORTED) return rca;
   }
   int rc = kq_launch_qmm_tuned(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev,
                                workspace_bytes, s);
+  if (rc != KQ_ERR_UNSUPPORTED) return rc;
+  rc = kq_launch_codes_skinny(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
   if (rc != KQ_ERR_UNSUPPORTED) return rc;
   return kq_launch_gemv_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
 }

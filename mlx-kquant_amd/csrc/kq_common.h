@@ -91,11 +91,17 @@ int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, co
 // (16-bit elements; K a multiple of 8, x and xg 16-byte aligned).
 int kq_launch_gather_rows(const void* x, const uint32_t* lhs, const uint32_t* rhs, void* xg, uint32_t* idx_rows, int B,
                           int M, int K, int64_t x_batch_stride, hipStream_t s);
+// Skinny-M (M <= 8) matrix-core kernel of the legacy / IQ / fp4 codecs: exact f16 codes in, block scales
+// applied to the f32 partial sums.  Same fall-through contract as kq_launch_qmm_tuned; no workspace.
+bool kq_codes_supported(int M, int N, int K, int codec);
+int kq_launch_codes_skinny(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
+                           hipStream_t s);
 // Matrix-core GEMM for every codec (exact bf16 x 3 split of the reference-order decoded weights):
 // prefill, and the batched MoE ops with biases and every activation.
 bool kq_anymma_supported(int M, int N, int K, int codec);
+size_t kq_anymma_dense_workspace_bytes(int M, int N, int K);
 int kq_launch_anymma_dense(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
-                           hipStream_t s);
+                           void* ws, size_t ws_bytes, hipStream_t s);
 bool kq_anymma_moe_supported(int P, int E, int N, int K, int codec);
 size_t kq_anymma_moe_workspace_bytes(int P, int E);
 int kq_launch_anymma_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,

@@ -59,6 +59,31 @@ def test_qmm_skinny_ragged_shapes(kq, codec, M, N, K):
         assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, N, K, dtype)
 
 
+NON_K = [c for c in O.ALL_CODECS if c not in ("q2_k", "q3_k", "q4_k", "q5_k", "q6_k")]
+
+
+@pytest.mark.parametrize("codec", NON_K)
+def test_qmm_skinny_codes_ragged(kq, codec):
+    """Legacy / IQ / fp4 codecs at M <= 8: K of 7 blocks (a partial last 256-weight step for the 32- and
+    64-weight blocks), a partial 128-row tile, a K long enough to be split across workgroups, both dtypes,
+    and activations spanning 30 binades (the per-step power-of-two scaling of bf16 inputs)."""
+    wpb, _ = O.geometry(codec)
+    for M, N, K in ((1, 131, 7 * wpb), (5, 40, 3 * 256), (8, 200, 8192), (2, 300, 2048 + wpb)):
+        wire = _wire(codec, N, K, seed=35)
+        for dtype in ("bfloat16", "float16"):
+            xb, xt = make_x((M, K), dtype, seed=300 + M)
+            got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+            want = O.qmm(xb, wire, codec, True, dtype)
+            assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, N, K, dtype)
+    M, N, K = 4, 64, 1024
+    wire = _wire(codec, N, K, seed=36)
+    x = np.random.default_rng(37).standard_normal((M, K)).astype(np.float32)
+    x *= np.exp2(np.random.default_rng(38).integers(-15, 15, (M, K // 256)).repeat(256, axis=1)).astype(np.float32)
+    xb = O.f32_to_bits(x, "bfloat16")
+    got = kq.quantized_matmul(bits_to_dev(xb, "bfloat16"), wire_to_dev(wire), None, codec)
+    assert rel_l2(dev_to_bits(got), O.qmm(xb, wire, codec, True, "bfloat16"), "bfloat16") <= TOL
+
+
 @pytest.mark.parametrize("codec", ["mxfp4", "q8_0", "q2_k", "iq2_xxs", "q5_0"])
 def test_qmm_gemv_unaligned_rows_and_tensor_end(kq, codec):
     """Rows that start at odd byte addresses (17 / 34 / 22-byte blocks, a view 1 byte into an allocation) and
