@@ -60,13 +60,18 @@ def synth_wire_torch(codec, rows, K, seed, device):
     return wire.reshape(rows, K // wpb * bpb)
 
 
-def quantized_weights(kq, torch, codec, N, K, seed, device):
+def quantized_weights(kq, torch, codec, N, K, seed, device, unique_rows=None):
     """Seeded N(0, 0.02) f32 weights [N, K] encoded by kq.quantize (host encoder; a uniform importance
-    matrix for the IQ codecs), placed on the GPU."""
+    matrix for the IQ codecs), placed on the GPU.  With unique_rows only that many rows are drawn and
+    encoded and the slab is repeated down the matrix (the codebook encoders search for ~1 us per weight;
+    kernel time does not depend on the values)."""
     g = torch.Generator()
     g.manual_seed(seed)
-    w = torch.randn((N, K), generator=g, dtype=torch.float32) * 0.02
+    rows = min(N, unique_rows) if unique_rows else N
+    w = torch.randn((rows, K), generator=g, dtype=torch.float32) * 0.02
     wq, _ = kq.quantize(w, codec, torch.ones(K) if codec.startswith("iq") else None)
+    if rows < N:
+        wq = wq.repeat((N + rows - 1) // rows, 1)[:N].contiguous()
     return wq.to(device)
 
 
@@ -337,13 +342,12 @@ def main():
                             "note": "any-codec matrix-core path (biases, swiglu_clamp), timed through the Python wrapper"}
         del gate, up, down
 
-        # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (q2_k / q3_k / iq4_xs encoded, iq3_s / iq2_xxs random wire)
+        # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (all five minted by kq.quantize)
         lowbit = []
         for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs"):
             n = k = 8192
             wb = n * kq.bytes_per_row(c, k)
-            wq = quantized_weights(kq, torch, c, n, k, 7, dev) if c in ("q2_k", "q3_k", "iq4_xs") else \
-                synth_wire_torch(c, n, k, 7, dev)
+            wq = quantized_weights(kq, torch, c, n, k, 7, dev, unique_rows=None if c in ("q2_k", "q3_k", "iq4_xs") else 512)
             cps = cold_copies(torch, wq, wb)
             t, _ = time_calls(torch, [abi.qmm(x.new_ones((1, k)), w, c, n, k) for w in cps], steps, warm)
             lowbit.append({"codec": c, "N": n, "K": k, "M": 1, "us": round(t * 1e3, 2),

@@ -10,6 +10,8 @@
 // IQ codebook blob linked into .rodata (data file given by -DKQ_GRID_BLOB="...").
 __asm__(".section .rodata\n"
         ".balign 16\n"
+        ".globl kq_grid_blob_host\n"
+        ".hidden kq_grid_blob_host\n"
         "kq_grid_blob_host:\n"
         ".incbin \"" KQ_GRID_BLOB "\"\n"
         ".previous\n");

@@ -1,6 +1,6 @@
 // Host-side wire encoders behind kq_quantize: float rows -> GGUF block bytes for the five legacy
-// 32-weight codecs, the five K-quant superblock codecs and the two non-linear 4-bit codecs
-// (iq4_nl, iq4_xs).  Like the reference's encoder
+// 32-weight codecs, the five K-quant superblock codecs, the two non-linear 4-bit codecs
+// (iq4_nl, iq4_xs) and three codebook codecs (iq2_xxs, iq3_xxs, iq3_s).  Like the reference's encoder
 // (src/kquant_cpu_encode.cpp:38-859, ggml's search heuristics) this runs on the CPU; unlike it,
 // blocks are encoded in parallel (blocks are independent).  Operation order inside a block
 // follows the cited reference lines so that, on the same x86 host arithmetic, the bytes agree.
@@ -12,10 +12,15 @@
 //             final re-quantisation of every weight)
 //   iq4     : iq4_nl / iq4_xs, src/kquant_iq_encode.cpp:49-214 (ggml quantize_row_iq4_nl_impl: nearest
 //             codebook entry, weighted least-squares scale, 15 trial scales around max / -127)
+//   codebook: iq2_xxs :392-598, iq3_xxs :1087-1310, iq3_s :1319-1544 (lattice search over the codebook
+//             with its neighbour index :228-331; one shared implementation driven by a traits table)
 #include <algorithm>
+#include <cfloat>
 #include <cmath>
 #include <cstring>
+#include <mutex>
 #include <thread>
+#include <utility>
 #include <vector>
 
 #include "kq_common.h"
@@ -151,7 +156,7 @@ float fit_positive(const float* x, const float* wt, int n, int nmax, uint8_t* ou
     return 0.f;
   }
   float inv = float(nmax) / vmax;
-  uint8_t lv[16];
+  uint8_t lv[32];
   float best = 0.f;
   {
     const float s = 1.0f / inv;
@@ -516,6 +521,320 @@ void enc_iq4(const float* x, const float* im, uint8_t* b) {
     for (int j = 0; j < 16; j++) qs[16 * i + j] = (uint8_t)(lv[32 * i + j] | (lv[32 * i + 16 + j] << 4));
 }
 
+// ------------------------------------------------------------------ codebook codecs (iq2_xxs, iq3_xxs, iq3_s)
+// A 32-weight sub-block is a scale times odd lattice points 2 l + 1 that must belong to a codebook
+// of 8-value (iq2) or 4-value (iq3) groups, plus one sign per weight.  The search representation
+// is derived from the decode codebooks linked into the library: the level of a value is its rank
+// among the distinct values of the codebook.  For every lattice point that is not in the codebook
+// the entries at the `rings` smallest distinct distances are kept as candidates (ties ordered by
+// entry number), as ggml's iq2xs_init_impl / iq3xs_init_impl do (reference :228-331).
+extern "C" const uint8_t kq_grid_blob_host[];
+
+struct Codebook {
+  int dim = 0, bits = 0, size = 0;
+  std::vector<int8_t> pts;     // [size][dim] coordinates 2 l + 1
+  std::vector<int32_t> slot;   // packed levels -> entry, or -(offset into near) - 1
+  std::vector<uint16_t> near;  // per off-codebook point: count, entries...
+};
+
+void build_codebook(Codebook& cb, const uint8_t* values, int size, int dim, int bits, int rings) {
+  cb.dim = dim;
+  cb.bits = bits;
+  cb.size = size;
+  bool seen[256] = {};
+  for (int i = 0; i < size * dim; i++) seen[values[i]] = true;
+  int level_of[256], nlevels = 0;
+  for (int v = 0; v < 256; v++) level_of[v] = seen[v] ? nlevels++ : -1;
+  cb.pts.resize((size_t)size * dim);
+  const int npacked = 1 << (bits * dim), mask = (1 << bits) - 1;
+  cb.slot.assign(npacked, 0);
+  std::vector<char> member(npacked, 0);
+  for (int e = 0; e < size; e++) {
+    int packed = 0;
+    for (int i = 0; i < dim; i++) {
+      const int l = level_of[values[e * dim + i]];
+      cb.pts[(size_t)e * dim + i] = int8_t(2 * l + 1);
+      packed |= l << (bits * i);
+    }
+    cb.slot[packed] = e;
+    member[packed] = 1;
+  }
+  std::vector<std::pair<int, int>> order(size);
+  for (int p = 0; p < npacked; p++) {
+    if (member[p]) continue;
+    int8_t pos[8];
+    bool reachable = true;
+    for (int i = 0; i < dim; i++) {
+      const int l = (p >> (bits * i)) & mask;
+      if (l >= nlevels) reachable = false;  // the encoder clamps levels below nlevels
+      pos[i] = int8_t(2 * l + 1);
+    }
+    if (!reachable) {
+      cb.slot[p] = 0;
+      continue;
+    }
+    for (int e = 0; e < size; e++) {
+      int d2 = 0;
+      for (int i = 0; i < dim; i++) {
+        const int df = cb.pts[(size_t)e * dim + i] - pos[i];
+        d2 += df * df;
+      }
+      order[e] = {d2, e};
+    }
+    std::sort(order.begin(), order.end());
+    const int32_t off = (int32_t)cb.near.size();
+    cb.near.push_back(0);
+    int ring = 1, cur = order[0].first, count = 0;
+    for (int e = 0; e < size; e++) {
+      if (order[e].first > cur) {
+        if (ring == rings) break;
+        cur = order[e].first;
+        ring++;
+      }
+      cb.near.push_back(uint16_t(order[e].second));
+      count++;
+    }
+    cb.near[off] = uint16_t(count);
+    cb.slot[p] = -off - 1;
+  }
+}
+
+enum { CB_IQ2XXS = 0, CB_IQ3XXS, CB_IQ3S, CB_COUNT };
+const Codebook& codebook(int which) {
+  static Codebook books[CB_COUNT];
+  static std::once_flag once[CB_COUNT];
+  std::call_once(once[which], [which] {
+    if (which == CB_IQ2XXS) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ2XXS, 256, 8, 2, 2);
+    if (which == CB_IQ3XXS) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ3XXS, 256, 4, 3, 2);
+    if (which == CB_IQ3S) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ3S, 512, 4, 3, 3);
+  });
+  return books[which];
+}
+
+// Levels of one group at inverse scale `inv`, snapped to the codebook: the rounded lattice point if it is
+// an entry, else the candidate with the least weighted error (weights sw = sqrt of the importance).
+// Returns the entry; *exact tells whether no snapping was needed.
+int snap_group(const Codebook& cb, const float* xv, const float* sw, float inv, int maxq, int8_t* lv, bool* exact) {
+  int packed = 0;
+  for (int i = 0; i < cb.dim; i++) {
+    const int l = clampi(rne(0.5f * (inv * xv[i] - 1.0f)), 0, maxq - 1);
+    lv[i] = int8_t(l);
+    packed |= l << (cb.bits * i);
+  }
+  const int32_t s = cb.slot[packed];
+  if (s >= 0) {
+    *exact = true;
+    return s;
+  }
+  *exact = false;
+  const uint16_t* cand = cb.near.data() + (-s - 1);
+  const float scale = 1.0f / inv;
+  float best = FLT_MAX;
+  int pick = -1;
+  for (int c = 1; c <= int(cand[0]); c++) {
+    const int8_t* pt = cb.pts.data() + (size_t)cand[c] * cb.dim;
+    float err = 0.f;
+    for (int i = 0; i < cb.dim; i++) {
+      const float df = scale * float(pt[i]) - xv[i];
+      err += sw[i] * df * df;
+    }
+    if (err < best) {
+      best = err;
+      pick = cand[c];
+    }
+  }
+  const int8_t* pt = cb.pts.data() + (size_t)pick * cb.dim;
+  for (int i = 0; i < cb.dim; i++) lv[i] = int8_t((pt[i] - 1) / 2);
+  return pick;
+}
+
+struct CbTraits {
+  int book, maxq;       // codebook, levels per coordinate
+  float sigma_factor;   // importance prologue
+  bool parity_signs;    // 7 stored sign bits per 8 weights (even parity enforced) vs 8
+  float zero_eps;       // sub-blocks whose largest magnitude is below this encode as zero
+  bool qp_start;        // starting scale from the positive-scale fit (iq2_xxs) vs max / (2 maxq - 1)
+  int scan;             // candidate scales -scan..scan
+  float scan_step;
+  int refine;           // 0: refit every sub-block; 1: only sub-blocks with a snapped group, all groups;
+                        // 2: only the snapped groups
+  float d_fudge;
+};
+constexpr CbTraits kIq2xxs{CB_IQ2XXS, 3, 1.0f, true, 1e-15f, true, 6, 0.1f, 0, 1.0f};
+constexpr CbTraits kIq3xxs{CB_IQ3XXS, 8, 2.0f, true, 1e-8f, false, 15, 0.2f, 2, 1.0125f};
+constexpr CbTraits kIq3s{CB_IQ3S, 8, 2.0f, false, 0.0f, false, 9, 0.2f, 1, 1.033f};
+
+// One 32-weight sub-block: magnitudes, signs, weights in; levels, codebook entries, sign bytes and the
+// scale out (ggml quantize_row_iq2_xxs_impl / iq3_xxs_impl / iq3_s_impl; reference :392-598, :1087-1310,
+// :1319-1544).
+float fit_codebook_subblock(const CbTraits& t, const float* xb, const float* imat, float sigma2, uint8_t* signs,
+                            int* entries) {
+  const Codebook& cb = codebook(t.book);
+  const int ngroups = 32 / cb.dim;
+  float wt[32], sw[32], xv[32];
+  for (int i = 0; i < 32; i++) {
+    wt[i] = imat ? imat[i] * std::sqrt(sigma2 + xb[i] * xb[i]) : xb[i] * xb[i];
+    sw[i] = std::sqrt(wt[i]);
+  }
+  for (int k = 0; k < 4; k++) {
+    uint8_t s = 0;
+    int flips = 0;
+    for (int i = 0; i < 8; i++) {
+      const float v = xb[8 * k + i];
+      xv[8 * k + i] = v >= 0.f ? v : -v;
+      if (v < 0.f) {
+        s |= uint8_t(1u << i);
+        flips++;
+      }
+    }
+    if (t.parity_signs) {
+      if (flips & 1) {  // an odd group cannot be stored: give up the sign of the least important weight
+        int imin = 0;
+        float least = wt[8 * k] * xb[8 * k] * xb[8 * k];
+        for (int i = 1; i < 8; i++) {
+          const float a = wt[8 * k + i] * xb[8 * k + i] * xb[8 * k + i];
+          if (a < least) {
+            least = a;
+            imin = i;
+          }
+        }
+        xv[8 * k + imin] = -xv[8 * k + imin];
+        s ^= uint8_t(1u << imin);
+      }
+      s &= 127;
+    }
+    signs[k] = s;
+  }
+  for (int g = 0; g < ngroups; g++) entries[g] = 0;
+  float vmax = xv[0];
+  for (int i = 1; i < 32; i++) vmax = std::max(vmax, xv[i]);
+  if (t.zero_eps > 0.f ? vmax < t.zero_eps : !(vmax != 0.f)) return 0.f;
+
+  int8_t lv[32] = {}, trial[32];
+  bool exact[8], trial_exact[8];
+  float scale, span;
+  if (t.qp_start) {
+    uint8_t tmp[32];
+    scale = fit_positive(xv, wt, 32, t.maxq + 1, tmp);
+    span = scale * float(t.maxq);
+    if (span <= 0.f) return 0.f;
+    for (int g = 0; g < ngroups; g++) exact[g] = true;
+  } else {
+    span = vmax;
+    scale = vmax / float(2 * t.maxq - 1);
+    for (int g = 0; g < ngroups; g++) exact[g] = t.refine == 2;
+  }
+  auto sums = [&](const int8_t* l, float& sqx, float& sq2) {
+    sqx = sq2 = 0.f;
+    for (int i = 0; i < 32; i++) {
+      const float q = float(2 * l[i] + 1);
+      sqx += wt[i] * xv[i] * q;
+      sq2 += wt[i] * q * q;
+    }
+  };
+  float best = 0.f;
+  for (int is = -t.scan; is <= t.scan; is++) {
+    const float inv = (float(2 * t.maxq - 1) + float(is) * t.scan_step) / span;
+    for (int g = 0; g < ngroups; g++)
+      snap_group(cb, xv + cb.dim * g, sw + cb.dim * g, inv, t.maxq, trial + cb.dim * g, &trial_exact[g]);
+    float sqx, sq2;
+    sums(trial, sqx, sq2);
+    if (sq2 > 0.f && sqx * sqx > best * sq2) {
+      scale = sqx / sq2;
+      best = scale * sqx;
+      std::memcpy(lv, trial, 32);
+      std::memcpy(exact, trial_exact, sizeof(exact));
+    }
+  }
+  bool any_snapped = false;
+  for (int g = 0; g < ngroups; g++) any_snapped |= !exact[g];
+  if (scale > 0.f && (t.refine == 0 || any_snapped)) {
+    const float inv = 1.0f / scale;
+    for (int g = 0; g < ngroups; g++) {
+      if (t.refine == 2 && exact[g]) continue;
+      bool e;
+      const int entry = snap_group(cb, xv + cb.dim * g, sw + cb.dim * g, inv, t.maxq, lv + cb.dim * g, &e);
+      const int8_t* pt = cb.pts.data() + (size_t)entry * cb.dim;
+      for (int i = 0; i < cb.dim; i++) lv[cb.dim * g + i] = int8_t((pt[i] - 1) / 2);
+    }
+    float sqx, sq2;
+    sums(lv, sqx, sq2);
+    if (sq2 > 0.f) scale = sqx / sq2;
+  }
+  if (scale < 0.f) {  // cannot happen with non-negative magnitudes; keep the wire's unsigned scale valid anyway
+    scale = -scale;
+    for (int k = 0; k < 4; k++) signs[k] = uint8_t(~signs[k]) & (t.parity_signs ? 127 : 255);
+  }
+  for (int g = 0; g < ngroups; g++) {
+    int packed = 0;
+    for (int i = 0; i < cb.dim; i++) packed |= int(lv[cb.dim * g + i]) << (cb.bits * i);
+    const int32_t s = cb.slot[packed];
+    entries[g] = s >= 0 ? s : 0;  // always an entry: every group was snapped above
+  }
+  return scale;
+}
+
+// 4-bit sub-block scale: scale ~ d (2 l + 1)
+inline int scale_level(float inv_d, float scale) { return clampi(rne(0.5f * (inv_d * scale - 1.0f)), 0, 15); }
+
+template <int kWhich>  // KQ_IQ2_XXS, KQ_IQ3_XXS, KQ_IQ3_S
+void enc_codebook(const float* x, const float* im, uint8_t* b) {
+  const CbTraits& t = kWhich == KQ_IQ2_XXS ? kIq2xxs : kWhich == KQ_IQ3_XXS ? kIq3xxs : kIq3s;
+  constexpr int kBytes = kWhich == KQ_IQ2_XXS ? 66 : kWhich == KQ_IQ3_XXS ? 98 : 110;
+  float total = 0.f;
+  for (int i = 0; i < 256; i++) total += x[i] * x[i];
+  const float sigma2 = t.sigma_factor * total / 256.0f;
+  float scales[8], top = 0.f;
+  uint8_t signs[8][4];
+  int entries[8][8];
+  for (int ib = 0; ib < 8; ib++) {
+    scales[ib] = fit_codebook_subblock(t, x + 32 * ib, im ? im + 32 * ib : nullptr, sigma2, signs[ib], entries[ib]);
+    top = std::max(top, scales[ib]);
+  }
+  std::memset(b, 0, kBytes);
+  if (!(top > 0.f)) return;
+  const float d = top / 31.0f, inv_d = 1.0f / d;
+  put_f16(b, d * t.d_fudge);
+  if constexpr (kWhich == KQ_IQ2_XXS) {
+    // per sub-block: four codebook bytes, then 4 x 7 sign bits and the 4-bit scale in one word
+    for (int ib = 0; ib < 8; ib++) {
+      uint8_t* q = b + 2 + 8 * ib;
+      uint32_t word = uint32_t(scale_level(inv_d, scales[ib])) << 28;
+      for (int k = 0; k < 4; k++) {
+        q[k] = uint8_t(scales[ib] > 0.f ? entries[ib][k] : 0);
+        if (scales[ib] > 0.f) word |= uint32_t(signs[ib][k]) << (7 * k);
+      }
+      std::memcpy(q + 4, &word, 4);
+    }
+  } else if constexpr (kWhich == KQ_IQ3_XXS) {
+    // 64 codebook bytes, then per sub-block 4 x 7 sign bits and the 4-bit scale in one word
+    for (int ib = 0; ib < 8; ib++) {
+      uint32_t word = uint32_t(scale_level(inv_d, scales[ib])) << 28;
+      for (int g = 0; g < 8; g++) b[2 + 8 * ib + g] = uint8_t(scales[ib] > 0.f ? entries[ib][g] : 0);
+      if (scales[ib] > 0.f)
+        for (int k = 0; k < 4; k++) word |= uint32_t(signs[ib][k]) << (7 * k);
+      std::memcpy(b + 66 + 4 * ib, &word, 4);
+    }
+  } else {
+    // qs[64] low entry bytes | qh[8] ninth bits | signs[32] | scales[4] (two nibbles each).  The qs and
+    // sign cursors advance only over non-zero sub-blocks while qh uses the absolute group number
+    // (reference :1329-1330, :1497-1508).
+    int qpos = 0, spos = 0;
+    for (int ib = 0; ib < 8; ib++) {
+      if (!(scales[ib] > 0.f) && !std::any_of(x + 32 * ib, x + 32 * ib + 32, [](float v) { return v != 0.f; })) continue;
+      for (int g = 0; g < 8; g++) {
+        b[2 + qpos + g] = uint8_t(entries[ib][g] & 255);
+        b[66 + ib] |= uint8_t((entries[ib][g] >> 8) << g);
+      }
+      qpos += 8;
+      for (int k = 0; k < 4; k++) b[74 + spos + k] = signs[ib][k];
+      spos += 4;
+    }
+    for (int ib = 0; ib < 8; ib += 2)
+      b[106 + ib / 2] = uint8_t(scale_level(inv_d, scales[ib]) | (scale_level(inv_d, scales[ib + 1]) << 4));
+  }
+}
+
 typedef void (*BlockEnc)(const float*, const float*, uint8_t*);
 void legacy_q8_0(const float* x, const float*, uint8_t* b) { enc_q8_0(x, b); }
 void legacy_q4_0(const float* x, const float*, uint8_t* b) { enc_legacy<false, 4>(x, b); }
@@ -537,6 +856,9 @@ BlockEnc encoder_for(int codec) {
     case KQ_Q6_K: return enc_q6_k;
     case KQ_IQ4_NL: return enc_iq4<32>;
     case KQ_IQ4_XS: return enc_iq4<256>;
+    case KQ_IQ2_XXS: return enc_codebook<KQ_IQ2_XXS>;
+    case KQ_IQ3_XXS: return enc_codebook<KQ_IQ3_XXS>;
+    case KQ_IQ3_S: return enc_codebook<KQ_IQ3_S>;
   }
   return nullptr;
 }

@@ -140,3 +140,92 @@ def test_iq4_known_answer_blocks():
     assert np.array_equal(qs & 15, lv[:, :, :16]) and np.array_equal(qs >> 4, lv[:, :, 16:])
     # and the decoder agrees with the pre-image exactly
     assert np.array_equal(O.dequantize(wire, "iq4_xs"), x.reshape(nsb, 256).astype(np.float32))
+
+
+# ------------------------------------------------------------------ codebook codecs (iq2_xxs, iq3_xxs, iq3_s)
+CB_BOUND = {"iq2_xxs": 0.45, "iq3_xxs": 0.30, "iq3_s": 0.30}  # reference tests/test_iq_encode.py:36-41
+
+
+@pytest.mark.parametrize("codec", list(CB_BOUND))
+def test_codebook_round_trip_bounds(codec):
+    """Same data recipe and bounds as the reference's IQ round-trip gate (gaussian * 0.1, |gaussian| + 0.1
+    importance, 256 x 512; tests/test_iq_encode.py:44-60, 77-96): measured there 0.36 for iq2_xxs."""
+    rng = np.random.default_rng(11)
+    w = (rng.standard_normal((256, 512)) * 0.1).astype(np.float32)
+    im = (np.abs(rng.standard_normal(512)) + 0.1).astype(np.float32)
+    wire = _enc(w, codec, im)
+    wpb, bpb = O.geometry(codec)
+    assert wire.shape == (256, 512 // wpb * bpb)
+    rel = np.linalg.norm(O.dequantize(wire, codec) - w) / np.linalg.norm(w)
+    assert rel < CB_BOUND[codec], (codec, rel)
+    assert rel > 0.02  # a 2-3 bit codec cannot be this good: guards against a vacuous decode
+    assert np.array_equal(wire, _enc(w, codec, im))
+    if codec == "iq2_xxs":
+        with pytest.raises(ValueError):
+            kq.quantize(torch.from_numpy(w), codec)  # imatrix-required, as ggml_quantize_requires_imatrix
+    else:
+        rel = np.linalg.norm(O.dequantize(_enc(w, codec), codec) - w) / np.linalg.norm(w)
+        assert rel < CB_BOUND[codec], (codec, rel)
+
+
+def _synth_lattice_wire(codec, nsb, seed):
+    """Random but structurally exact wire: every sub-block scale nibble is set, block 0 carries the
+    largest one (15), super-scale d is a power of two."""
+    rng = np.random.default_rng(seed)
+    wpb, bpb = O.geometry(codec)
+    wire = O.synth_wire(codec, nsb, seed).reshape(nsb, bpb).copy()
+    wire[:, 0:2] = np.frombuffer(np.float16(2.0 ** -6).tobytes(), dtype=np.uint8)
+    if codec == "iq2_xxs":
+        for ib in range(8):  # scale nibble = top 4 bits of the second word of a sub-block
+            wire[:, 2 + 8 * ib + 7] = (wire[:, 2 + 8 * ib + 7] & 0x0F) | ((15 if ib == 0 else rng.integers(3, 15)) << 4)
+    return wire
+
+
+def test_iq2_xxs_known_answer_blocks():
+    """Weights that ARE codebook points (decode of a valid wire) must come back as the same codebook entries
+    and signs: the rounded lattice point of every group is an entry and the sign parity is even by
+    construction.  Checks the codebook index built from the decode tables, the level <-> value map and the
+    entry / 7-bit sign packing.  Magnitudes are not exact: the search fits scale * (1, 3, 5) while the decode
+    values are (8, 25, 43), as in ggml."""
+    wire = _synth_lattice_wire("iq2_xxs", 24, 5)
+    x = O.dequantize(wire, "iq2_xxs").reshape(24, 256)
+    mine = _enc(x, "iq2_xxs", np.ones(256, np.float32))
+    a, b = wire[:, 2:].reshape(24, 8, 8), mine[:, 2:].reshape(24, 8, 8)
+    assert np.mean(a[:, :, :4] == b[:, :, :4]) > 0.97  # codebook entries
+    sa = a[:, :, 4:].copy().view(np.uint32) & 0x0FFFFFFF
+    sb = b[:, :, 4:].copy().view(np.uint32) & 0x0FFFFFFF
+    assert np.mean(sa == sb) > 0.99  # 4 x 7 sign bits
+    back = O.dequantize(mine, "iq2_xxs").reshape(24, 256)
+    assert np.linalg.norm(back - x) / np.linalg.norm(x) < 0.10
+
+
+@pytest.mark.parametrize("codec", ["iq3_xxs", "iq3_s"])
+def test_iq3_lattice_points_keep_their_shape(codec):
+    """Decode of a valid wire re-encodes to the same lattice points up to the per-sub-block scale (ggml
+    inflates d by 1.0125 / 1.033 on purpose, so magnitudes move by that factor at most)."""
+    wire = O.synth_wire(codec, 16, 6).reshape(16, -1).copy()
+    wire[:, 0:2] = np.frombuffer(np.float16(2.0 ** -5).tobytes(), dtype=np.uint8)
+    x = O.dequantize(wire, codec).reshape(16, 256)
+    back = O.dequantize(_enc(x, codec, np.ones(256, np.float32)), codec).reshape(16, 256)
+    assert np.mean(np.sign(back) == np.sign(x)) > 0.999
+    rel = np.linalg.norm(back - x) / np.linalg.norm(x)
+    assert rel < 0.08, (codec, rel)
+
+
+def test_codebook_zero_and_imatrix():
+    for codec in CB_BOUND:
+        z = np.zeros((2, 256), np.float32)
+        wire = _enc(z, codec, np.ones(256, np.float32))
+        assert not wire.any()
+        assert not O.dequantize(wire, codec).any()
+    rng = np.random.default_rng(12)
+    w = (rng.standard_normal((8, 512)) * 0.05).astype(np.float32)
+    flat = np.ones(512, np.float32)
+    steep = rng.uniform(0.05, 20.0, 512).astype(np.float32)
+    for codec in CB_BOUND:
+        a, b = _enc(w, codec, flat), _enc(w, codec, steep)
+        assert not np.array_equal(a, b), codec
+        # the importance-weighted error is what the search minimises: it must not get worse under its own weights
+        ea = np.sum(steep * (O.dequantize(a, codec) - w) ** 2)
+        eb = np.sum(steep * (O.dequantize(b, codec) - w) ** 2)
+        assert eb < ea * 1.02, (codec, ea, eb)
