@@ -191,6 +191,9 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for `rocprofv3 --pmc`: one device copy of the headline matrix (known bytes) "
                          "followed by 20 cold launches of the headline GEMV, nothing else")
+    ap.add_argument("--probe-codec", default=None, metavar="CODEC",
+                    help="counter probe for `rocprofv3 --pmc`: 20 launches of the M = 1 GEMV 8192 -> 8192 in CODEC "
+                         "(random structurally valid wire), nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU.",
@@ -208,6 +211,17 @@ def main():
 
     def randx(shape, scale=1.0):
         return (torch.randn(shape, device=dev, dtype=torch.float32, generator=gx) * scale).to(torch.bfloat16)
+
+    if args.probe_codec:
+        c, n, k = args.probe_codec, 8192, 8192
+        w = synth_wire_torch(c, n, k, 7, dev)
+        call = abi.qmm(randx((1, k)), w, c, n, k)
+        for i in range(20):
+            call()
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "20 GEMV launches", "codec": c, "N": n, "K": k, "M": 1,
+                          "weight_bytes": n * kq.bytes_per_row(c, k)}))
+        return
 
     # ---------------- headline: q4_k gate/up GEMV, M = 1, cold
     codec, N, K, M = "q4_k", 14336, 4096, 1
