@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLC_BYTES = 256 << 20
 # HBM bytes one headline launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
-# `bench.py --probe`: (16237.4 KiB x 1.9983 + 28.0 KiB x 1.0), each counter scaled by what it reads for
+# `bench.py --probe`: (16235.0 KiB x 1.9983 + 28.0 KiB x 1.0), each counter scaled by what it reads for
 # the probe's plain 32256 KiB device copy.  Algorithmic bytes are 33,030,144 (weights) + 28,672 (output).
 HEADLINE_TRAFFIC_BYTES = 33_254_000
 KQ_BF16 = 2
