@@ -194,6 +194,9 @@ def main():
     ap.add_argument("--probe-codec", default=None, metavar="CODEC",
                     help="counter probe for `rocprofv3 --pmc`: 20 launches of the M = 1 GEMV 8192 -> 8192 in CODEC "
                          "(random structurally valid wire), nothing else")
+    ap.add_argument("--probe-prefill", default=None, metavar="CODEC",
+                    help="counter probe for `rocprofv3 --pmc`: 5 launches of the prefill GEMM [2048, 8192] x "
+                         "[28672, 8192]^T in CODEC (random structurally valid wire), nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU.",
@@ -221,6 +224,17 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"probe": "20 GEMV launches", "codec": c, "N": n, "K": k, "M": 1,
                           "weight_bytes": n * kq.bytes_per_row(c, k)}))
+        return
+
+    if args.probe_prefill:
+        c, m, n, k = args.probe_prefill, 2048, 28672, 8192
+        w = synth_wire_torch(c, n, k, 7, dev)
+        call = abi.qmm(randx((m, k)), w, c, n, k)
+        for i in range(5):
+            call()
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "5 prefill GEMM launches", "codec": c, "M": m, "N": n, "K": k,
+                          "flops": 2 * m * n * k}))
         return
 
     # ---------------- headline: q4_k gate/up GEMV, M = 1, cold
@@ -353,7 +367,7 @@ def main():
                             "down_us": round(td * 1e3, 1),
                             "glu_gbs": round(ne * 2 * mbytes / (tg * 1e-3) / 1e9, 1),
                             "down_gbs": round(ne * mbytes / (td * 1e-3) / 1e9, 1),
-                            "note": "any-codec matrix-core path (biases, swiglu_clamp), timed through the Python wrapper"}
+                            "note": "grouped code-level MFMA kernel (biases, swiglu_clamp), timed through the Python wrapper"}
         del gate, up, down
 
         # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (all five minted by kq.quantize)

@@ -242,6 +242,7 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return 0;
   if (kq_moe_grouped_supported((int)P, E, N, K, codec)) return kq_moe_grouped_workspace_bytes(glu ? T : (int)P, (int)P, E, K);
+  if (kq_codes_moe_supported((int)P, E, N, K, codec)) return kq_codes_moe_workspace_bytes((int)P, E);
   if (kq_anymma_moe_supported((int)P, E, N, K, codec)) return kq_anymma_moe_workspace_bytes((int)P, E);
   return 0;
 }
@@ -254,7 +255,17 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
-    // every other codec, biases, swiglu_clamp: the any-codec matrix-core path
+    // legacy / IQ / fp4 codecs (biases and every activation included): code-level grouped kernel
+    if (kq_codes_moe_supported((int)P, E, N, K, codec)) {
+      const size_t need = kq_codes_moe_workspace_bytes((int)P, E);
+      if (!ws || ws_bytes < need)
+        return kq_set_error(KQ_ERR_WORKSPACE, "%s: workspace of %zu bytes required (got %zu)", op, need, ws ? ws_bytes : 0);
+      const int rcc = kq_launch_codes_moe(x, static_cast<const uint8_t*>(w), static_cast<const uint8_t*>(w2), idx, bias,
+                                          bias2, out, (int)P, E, N, K, glu ? R : 1, estride, glu, act, limit, alpha, codec,
+                                          dtype, ws, s);
+      if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
+    }
+    // q2_k / q3_k, and q4_k ... q6_k with biases or swiglu_clamp: the any-codec matrix-core path
     if (!kq_anymma_moe_supported((int)P, E, N, K, codec)) return KQ_ERR_UNSUPPORTED;
     const size_t need = kq_anymma_moe_workspace_bytes((int)P, E);
     if (!ws || ws_bytes < need)

@@ -18,6 +18,10 @@
 // live in LDS as f16 tables built once per workgroup.  A lane copies its row's step bytes into
 // registers with conflict-free 16-byte LDS reads and picks exactly the 8 codes its MFMA B operand
 // needs (row l % 32, K half l / 32) at compile-time offsets, so nothing decoded is shared or stored.
+//
+// The batched MoE ops (more than 16 (token, expert) pairs) use the same decode in a workgroup-tiled
+// grouped kernel (further down): 32 gathered pairs of one expert x 128 weight rows per workgroup.
+#include "kq_epilogue.h"
 #include "kq_mma.h"
 
 namespace {
@@ -621,7 +625,409 @@ int launch_codes_dt(const CkArgs& a, int dtype, hipStream_t s) {
   return KQ_ERR_UNSUPPORTED;
 }
 
+// ------------------------------------------------------------------ grouped kernel (batched MoE)
+// Pairs sorted by expert and cut into segments of at most 32 pairs of one expert (moe_sort_kernel).  A
+// workgroup multiplies a segment's gathered activation rows (the MFMA's 32 rows) by a 128-row slab of that
+// expert's wire: 4 waves x 32 weight rows, one 256-weight step at a time, wire bytes and activations
+// fetched one step ahead and parked in LDS.  GLU: the slab is 64 gate rows + the same 64 up rows (waves
+// 0 / 2 gate, 1 / 3 up); the up waves hand their sums to the gate waves through LDS and the epilogue runs
+// before the single rounding.  Same code extraction and block-scale-after-the-MFMA numerics as above.
+struct Segment {
+  int expert, start, count, pad;
+};
+
+struct CgArgs {
+  const void* x;        // [rows][K], pair p reads row p / x_div
+  const uint8_t* w;
+  const uint8_t* w2;    // up stack (GLU) or null
+  void* y;              // [P][N]
+  const float* bias;    // f32 [E][N] or null
+  const float* bias2;
+  const int* order;     // pair ids sorted by expert
+  const Segment* segs;
+  const int* nseg;
+  const uint8_t* grids;
+  int N, K, x_div, act;
+  int64_t w_expert_stride;
+  float limit, alpha;
+};
+
+constexpr int CG_THREADS = 256;
+constexpr int CG_BN = 128;
+
+template <int C>
+constexpr int grouped_lds_bytes() {
+  return 32 * XA_STRIDE + 32 * 4 + 8 * 32 * 4 + CG_BN * CodeGeom<C>::LROW + 32 * 4 + CodeGeom<C>::GRID_BYTES +
+         CodeGeom<C>::SPREAD_BYTES;
+}
+
+template <int C, int DT, bool GLU>
+__global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) {
+  using G = CodeGeom<C>;
+  constexpr int WPT = (CG_BN * G::PIECES + CG_THREADS - 1) / CG_THREADS;
+  constexpr int NCOLS = GLU ? CG_BN / 2 : CG_BN;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint8_t* a_lds = smem;                                                  // [32][XA_STRIDE] f16 activations of the step
+  float* xs_lds = reinterpret_cast<float*>(a_lds + 32 * XA_STRIDE);       // [32] activation scale per slot
+  float* xsum_lds = xs_lds + 32;                                          // [8 blocks][32 slots] (HAS_MIN)
+  uint8_t* b_lds = reinterpret_cast<uint8_t*>(xsum_lds + 8 * 32);         // [128][LROW]
+  int* pair_lds = reinterpret_cast<int*>(b_lds + CG_BN * G::LROW);        // [32] output row per slot, -1 = none
+  uint8_t* grid_lds = reinterpret_cast<uint8_t*>(pair_lds + 32);
+  uint8_t* spread_lds = grid_lds + G::GRID_BYTES;
+
+  if ((int)blockIdx.y >= *a.nseg) return;  // uniform: the grid is sized for the worst case
+  const Segment seg = a.segs[blockIdx.y];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, kg = lane >> 5;
+  const int N = a.N, K = a.K;
+  const int nsteps = (K + CK_STEP - 1) / CK_STEP;
+  const size_t row_bytes = (size_t)(K / G::WPB) * G::BPB;
+  const int n0 = blockIdx.x * NCOLS;
+  const int ncols = N - n0 < NCOLS ? N - n0 : NCOLS;
+  const uint8_t* wbase = a.w + (size_t)seg.expert * (size_t)a.w_expert_stride;
+  const uint8_t* wbase2 = GLU ? a.w2 + (size_t)seg.expert * (size_t)a.w_expert_stride : wbase;
+  const uint8_t* w_last = wbase + (size_t)N * row_bytes - 16;  // the last 16 bytes of the expert's matrix
+  const uint8_t* w_last2 = wbase2 + (size_t)N * row_bytes - 16;
+
+  // slab row rr (= wave * 32 + l32 in the compute phase) -> (matrix, column)
+  auto slab_col = [&](int rr, bool& up) {
+    if constexpr (GLU) {
+      const int wv = rr >> 5;
+      up = wv & 1;
+      return (wv >> 1) * 32 + (rr & 31);
+    } else {
+      up = false;
+      return rr;
+    }
+  };
+
+  if (tid < 32) pair_lds[tid] = tid < seg.count ? a.order[seg.start + tid] : -1;
+
+  // ---- tables
+  if constexpr (G::GRID_N > 0) {
+    const uint8_t* src = a.grids + G::GRID_OFF;
+    if constexpr (G::GRID_W == 8) {
+      for (int e = tid; e < G::GRID_N; e += CG_THREADS) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(src + 8 * e);
+        f16x8 f;
+        if constexpr (G::GRID_SIGNED)
+          f = bytes8_to_frag(v[0] ^ 0x80808080u, v[1] ^ 0x80808080u, 128.f);
+        else
+          f = bytes8_to_frag(v[0], v[1], 0.f);
+        *reinterpret_cast<f16x8*>(grid_lds + 16 * e) = f;
+      }
+    } else {
+      for (int e = tid; e < G::GRID_N; e += CG_THREADS) {
+        const uint32_t v = *reinterpret_cast<const uint32_t*>(src + 4 * e);
+        uint32_t ev, od;
+        bytes_to_f16(v, 0.f, ev, od);
+        *reinterpret_cast<u32x2*>(grid_lds + 8 * e) = u32x2{ev, od};
+      }
+    }
+  }
+  if constexpr (G::SPREAD_BYTES > 0) {
+    const uint32_t b = tid;  // 256 threads, 256 entries
+    auto bit = [&](int i) { return (b >> i) & 1u; };
+    constexpr int P = G::SPREAD_BIT;
+    *reinterpret_cast<u32x4*>(spread_lds + 16 * tid) =
+        u32x4{(bit(0) << P) | (bit(2) << (P + 16)), (bit(1) << P) | (bit(3) << (P + 16)),
+              (bit(4) << P) | (bit(6) << (P + 16)), (bit(5) << P) | (bit(7) << (P + 16))};
+  }
+  const Tables tabs{grid_lds, spread_lds};
+
+  // ---- piece maps.  Activations: piece i = tid + 256 t -> (slot i / 32, 16-byte piece i % 32).
+  const int a_slot0 = tid >> 5, a_pc = tid & 31;
+  const uint16_t* a_src[4];
+  bool a_live[4];
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const int slot = a_slot0 + 8 * t;
+    a_live[t] = slot < seg.count;
+    const size_t row = (size_t)(a.order[seg.start + (a_live[t] ? slot : 0)] / a.x_div);
+    a_src[t] = static_cast<const uint16_t*>(a.x) + row * K + 8 * a_pc;
+  }
+  const uint8_t* w_src[WPT];
+  uint32_t w_loff[WPT];
+  bool w_up[WPT];
+#pragma unroll
+  for (int t = 0; t < WPT; t++) {
+    const int i = tid + CG_THREADS * t;
+    const int r = i / G::PIECES, pc = i % G::PIECES;
+    bool up;
+    const int col = slab_col(r < CG_BN ? r : 0, up);
+    const bool ok = r < CG_BN && col < ncols;  // rows past N re-read the slab's first row
+    w_up[t] = up;
+    w_src[t] = (up ? wbase2 : wbase) + (size_t)(n0 + (ok ? col : 0)) * row_bytes + 16 * pc;
+    w_loff[t] = r < CG_BN ? (uint32_t)r * G::LROW + 16 * pc : 0xffffffffu;
+  }
+
+  u32x4 areg[4], wreg[WPT];
+  auto issue = [&](int st) {
+    const int kvalid = K - CK_STEP * st;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      u32x4 av = {0, 0, 0, 0};
+      if (a_live[t] && 8 * a_pc < kvalid) av = *reinterpret_cast<const u32x4*>(a_src[t] + (size_t)CK_STEP * st);
+      areg[t] = av;
+    }
+#pragma unroll
+    for (int t = 0; t < WPT; t++) {
+      const uint8_t* p = w_src[t] + (size_t)st * G::BYTES;
+      const uint8_t* last = w_up[t] ? w_last2 : w_last;
+      const uint8_t* q = p <= last ? p : last;  // never read past the end of the expert's matrix
+      u32x4 v = *reinterpret_cast<const u32x4_a1*>(q);
+      if (q != p) v = shr_bytes(v, (uint32_t)(p - q));
+      wreg[t] = v;
+    }
+  };
+  auto park = [&]() {
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const int slot = a_slot0 + 8 * t;
+      float xscale = 1.f;
+      _Float16 h[8];
+      if constexpr (DT == KQ_BF16) {
+        float amax = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, areg[t][e] << 16)));
+          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, areg[t][e] & 0xffff0000u)));
+        }
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));  // the slot's 32 lanes
+        float inv = 1.f;
+        const uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff;
+        if (eb != 0 && eb != 0xff) {
+          int e = (int)eb - 127 - 14;  // the largest magnitude lands in [2^14, 2^15)
+          if (e < -100) e = -100;
+          xscale = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+          inv = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          h[2 * e] = (_Float16)(__builtin_bit_cast(float, areg[t][e] << 16) * inv);
+          h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, areg[t][e] & 0xffff0000u) * inv);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(areg[t][e] & 0xffff));
+          h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(areg[t][e] >> 16));
+        }
+      }
+      const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};  // fragment order inside an 8-group
+      *reinterpret_cast<f16x8*>(a_lds + slot * XA_STRIDE + 16 * a_pc) = v8;
+      if (a_pc == 0) xs_lds[slot] = xscale;
+      if constexpr (G::HAS_MIN) {
+        float sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) sum += (float)h[e];
+        sum += __shfl_xor(sum, 1);
+        sum += __shfl_xor(sum, 2);  // 4 lanes = one 32-weight block
+        if ((a_pc & 3) == 0) xsum_lds[(a_pc >> 2) * 32 + slot] = sum;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < WPT; t++)
+      if (w_loff[t] != 0xffffffffu) *reinterpret_cast<u32x4*>(b_lds + w_loff[t]) = wreg[t];
+  };
+
+  float acc[16];  // output slots 8 (i / 4) + 4 kg + i % 4 of slab row wave * 32 + l32
+#pragma unroll
+  for (int i = 0; i < 16; i++) acc[i] = 0.f;
+  const uint8_t* b_lane = b_lds + (wave * 32 + l32) * G::LROW;
+  const uint8_t* a_lane = a_lds + l32 * XA_STRIDE + 16 * kg;
+
+  issue(0);
+  for (int st = 0; st < nsteps; st++) {
+    lds_barrier();  // tables built / everyone is done reading the previous step
+    park();
+    if (st + 1 < nsteps) issue(st + 1);
+    lds_barrier();
+    const int kvalid = K - CK_STEP * st;
+    float sacc[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) sacc[i] = 0.f;
+    constexpr int MPS = G::SB / 16;
+    auto run_step = [&](auto full_c) {
+      constexpr bool FULL = decltype(full_c)::value;
+      f32x16 part[2];
+      RowRegs<4 * G::PIECES> row;
+      StaticFor<G::PIECES>::run([&](auto pc) {
+        constexpr int P = decltype(pc)::value;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(b_lane + 16 * P);
+        row.d[4 * P] = v[0];
+        row.d[4 * P + 1] = v[1];
+        row.d[4 * P + 2] = v[2];
+        row.d[4 * P + 3] = v[3];
+      });
+      StaticFor<16>::run([&](auto jc) {
+        constexpr int J = decltype(jc)::value;
+        if (FULL || 16 * J < kvalid) {  // uniform
+          const f16x8 bv = codes<C, J>(row, kg, tabs);
+          const f16x8 av = *reinterpret_cast<const f16x8*>(a_lane + 32 * J);
+          constexpr int sbi = J / MPS, slot = sbi & 1;
+          if constexpr (J % MPS == 0)
+            part[slot] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, f32x16{0}, 0, 0, 0);
+          else
+            part[slot] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, part[slot], 0, 0, 0);
+          if constexpr (J % MPS == MPS - 1) {
+            float mn;
+            const float sc = block_scale<C, sbi>(row, mn);
+#pragma unroll
+            for (int i = 0; i < 16; i++) sacc[i] = fmaf(sc, part[slot][i], sacc[i]);
+            if constexpr (G::HAS_MIN) {
+#pragma unroll
+              for (int q = 0; q < 4; q++) {
+                const float4 xm = *reinterpret_cast<const float4*>(xsum_lds + sbi * 32 + 8 * q + 4 * kg);
+                sacc[4 * q + 0] = fmaf(mn, xm.x, sacc[4 * q + 0]);
+                sacc[4 * q + 1] = fmaf(mn, xm.y, sacc[4 * q + 1]);
+                sacc[4 * q + 2] = fmaf(mn, xm.z, sacc[4 * q + 2]);
+                sacc[4 * q + 3] = fmaf(mn, xm.w, sacc[4 * q + 3]);
+              }
+            }
+          }
+        }
+      });
+    };
+    if (kvalid >= CK_STEP)
+      run_step(std::true_type{});
+    else
+      run_step(std::false_type{});
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const float4 xs4 = *reinterpret_cast<const float4*>(xs_lds + 8 * q + 4 * kg);
+      acc[4 * q + 0] = fmaf(xs4.x, sacc[4 * q + 0], acc[4 * q + 0]);
+      acc[4 * q + 1] = fmaf(xs4.y, sacc[4 * q + 1], acc[4 * q + 1]);
+      acc[4 * q + 2] = fmaf(xs4.z, sacc[4 * q + 2], acc[4 * q + 2]);
+      acc[4 * q + 3] = fmaf(xs4.w, sacc[4 * q + 3], acc[4 * q + 3]);
+    }
+  }
+
+  // ---- epilogue
+  uint16_t* y = static_cast<uint16_t*>(a.y);
+  auto store = [&](size_t off, float v) { y[off] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v); };
+  if constexpr (!GLU) {
+    const int col = wave * 32 + l32;
+    const float bv = (a.bias && col < ncols) ? a.bias[(size_t)seg.expert * N + n0 + col] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int pr = pair_lds[8 * (i >> 2) + 4 * kg + (i & 3)];
+      if (pr >= 0 && col < ncols) store((size_t)pr * N + n0 + col, acc[i] + bv);
+    }
+  } else {
+    lds_barrier();  // the step buffers are free: reuse them for the up sums
+    float* ex = reinterpret_cast<float*>(smem);  // [2 column blocks][16][64]
+    const int nb = wave >> 1;
+    if (wave & 1) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) ex[(nb * 16 + i) * 64 + lane] = acc[i];
+    }
+    lds_barrier();
+    if (!(wave & 1)) {
+      const int col = nb * 32 + l32;
+      const bool live = col < ncols;
+      const float gb = (a.bias && live) ? a.bias[(size_t)seg.expert * N + n0 + col] : 0.f;
+      const float ub = (a.bias2 && live) ? a.bias2[(size_t)seg.expert * N + n0 + col] : 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int pr = pair_lds[8 * (i >> 2) + 4 * kg + (i & 3)];
+        if (pr >= 0 && live) {
+          const float v = kq::glu_epilogue(a.act, acc[i] + gb, ex[(nb * 16 + i) * 64 + lane] + ub, a.limit, a.alpha);
+          store((size_t)pr * N + n0 + col, v);
+        }
+      }
+    }
+  }
+}
+
+template <int C, int DT, bool GLU>
+int launch_grouped(const CgArgs& a, int P, int E, hipStream_t s) {
+  constexpr int NCOLS = GLU ? CG_BN / 2 : CG_BN;
+  int maxseg = E + P / 32;  // sum over experts of ceil(c_e / 32) <= E + P / 32
+  if (maxseg > P) maxseg = P;
+  const size_t lds = grouped_lds_bytes<C>();
+  auto kern = codes_grouped_kernel<C, DT, GLU>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((a.N + NCOLS - 1) / NCOLS, maxseg), dim3(CG_THREADS), lds, s, a);
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
+template <int C>
+int launch_grouped_any(const CgArgs& a, int P, int E, int glu, int dtype, hipStream_t s) {
+  if (glu) return dtype == KQ_F16 ? launch_grouped<C, KQ_F16, true>(a, P, E, s) : launch_grouped<C, KQ_BF16, true>(a, P, E, s);
+  return dtype == KQ_F16 ? launch_grouped<C, KQ_F16, false>(a, P, E, s) : launch_grouped<C, KQ_BF16, false>(a, P, E, s);
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
 }  // namespace
+
+// kq_moe.hip
+int kq_launch_moe_sort(const uint32_t* idx, int P, int E, void* order, void* segs, void* nseg, hipStream_t s);
+
+bool kq_codes_moe_supported(int P, int E, int N, int K, int codec) {
+  // nvfp4 (a scale per 16 weights: 16 x 16 scalings per step) does not fit the register file here and
+  // stays on the any-codec path
+  if (codec < KQ_Q4_0 || codec >= KQ_NUM_CODECS || codec == KQ_NVFP4) return false;
+  return P > 16 && E > 0 && E <= 4096 && (int64_t)E + P / 32 < 65535 && N > 0 && K > 0 && (K & 7) == 0 &&
+         K % kq_geom(codec).wpb == 0;
+}
+
+// Workspace: sorted pair list, segment table, segment count.
+size_t kq_codes_moe_workspace_bytes(int P, int E) {
+  return align256((size_t)P * 4) + align256(((size_t)E + P / 32 + 1) * sizeof(Segment)) + 256;
+}
+
+// x: [rows][K]; pair p reads row p / x_div and expert idx[p]; out [P][N].
+int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
+                        const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
+                        int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, hipStream_t s) {
+  if (!kq_codes_moe_supported(P, E, N, K, codec) || (reinterpret_cast<uintptr_t>(x) & 15) ||
+      (reinterpret_cast<uintptr_t>(ws) & 255))
+    return KQ_ERR_UNSUPPORTED;
+  uint8_t* p = static_cast<uint8_t*>(ws);
+  int* order = reinterpret_cast<int*>(p);
+  Segment* segs = reinterpret_cast<Segment*>(p + align256((size_t)P * 4));
+  int* nseg = reinterpret_cast<int*>(p + align256((size_t)P * 4) + align256(((size_t)E + P / 32 + 1) * sizeof(Segment)));
+  int rc = kq_launch_moe_sort(idx, P, E, order, segs, nseg, s);
+  if (rc) return rc;
+  CgArgs a{};
+  a.x = x;
+  a.w = w;
+  a.w2 = w2;
+  a.y = out;
+  a.bias = bias;
+  a.bias2 = bias2;
+  a.order = order;
+  a.segs = segs;
+  a.nseg = nseg;
+  a.grids = kq_device_grids();
+  if (!a.grids) return KQ_ERR_HIP;
+  a.N = N;
+  a.K = K;
+  a.x_div = x_div < 1 ? 1 : x_div;
+  a.act = act;
+  a.w_expert_stride = w_expert_stride;
+  a.limit = limit;
+  a.alpha = alpha;
+  switch (codec) {
+#define KQ_CASE(c) \
+  case c:          \
+    return launch_grouped_any<c>(a, P, E, glu, dtype, s);
+    KQ_CASE(KQ_Q4_0) KQ_CASE(KQ_Q4_1) KQ_CASE(KQ_Q5_0) KQ_CASE(KQ_Q5_1) KQ_CASE(KQ_Q8_0) KQ_CASE(KQ_IQ4_NL)
+    KQ_CASE(KQ_IQ4_XS) KQ_CASE(KQ_IQ3_S) KQ_CASE(KQ_IQ3_XXS) KQ_CASE(KQ_IQ2_XXS) KQ_CASE(KQ_IQ2_XS) KQ_CASE(KQ_IQ2_S)
+    KQ_CASE(KQ_IQ1_S) KQ_CASE(KQ_IQ1_M) KQ_CASE(KQ_MXFP4) KQ_CASE(KQ_NVFP4)
+#undef KQ_CASE
+  }
+  return KQ_ERR_UNSUPPORTED;
+}
 
 bool kq_codes_supported(int M, int N, int K, int codec) {
   if (codec < KQ_Q4_0 || codec >= KQ_NUM_CODECS) return false;  // the K-quants have their own kernels
