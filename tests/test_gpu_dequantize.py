@@ -77,7 +77,7 @@ def test_dequantize_edge_cases(kq):
 
 
 def test_dequantize_config1_size(kq):
-    # BASELINE config 1: 4096 x 4096 q4_k -> f16; full size through block independence:
+    # the reference CPU-runnable configuration, 4096 x 4096 q4_k -> f16; full size through block independence:
     # the 4096 rows are 512 distinct rows tiled, compared with the oracle on those rows.
     base = O.synth_wire("q4_k", 512 * 16, seed=21).reshape(512, 16 * 144)
     wire = np.tile(base, (8, 1))
