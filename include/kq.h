@@ -130,6 +130,18 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
                   void* out_dev, int T, int R, int E, int N, int K, int codec, int dtype, void* workspace_dev,
                   size_t workspace_bytes, void* stream);
 
+/* Router: expert scores over the E logit columns (scoring 0 = softmax, 1 = sqrt(softplus(x))), the top_k
+ * largest by score (+ bias[e] when given; smallest index first on ties) and their mixing weights:
+ * score / (sum of the picked scores (+ 1e-20 for scoring 1) if norm_topk_prob else the softmax sum)
+ * * per_expert_scale[e] * scale.  With shared_gate logits are [T, E + 1] and sigmoid(column E) is
+ * appended: scores [T, top_k + 1].  logits in `dtype` (0 / 1 / 2 = f32 / f16 / bf16), all math f32;
+ * indices uint32 [T, top_k], scores f32.  E <= 1024, top_k <= min(E, 16); scoring 1 needs norm_topk_prob.
+ * Replaces KQuantMoERouterTopK (op moe_router_topk), reference src/kquant_moe_glu.cpp:1366-1441, kernel
+ * metal/mlx/backend/metal/kernels/kq_moe_glu_kq.h:1215-1358. */
+int kq_moe_router_topk(const void* logits_dev, int dtype, int T, int E, int top_k, int norm_topk_prob,
+                       int shared_gate, const float* per_expert_scale_dev, const float* bias_dev, int scoring,
+                       float scale, uint32_t* indices_dev, float* scores_dev, void* stream);
+
 /* HOST function: wire = encode(w[rows, K] f32) (imatrix f32 [K] or NULL), rows * bytes_per_row
  * bytes written to wire_host.  Runs on the calling thread's CPU cores like the reference's
  * encoder (which is CPU-only for the IQ codecs and serial).

@@ -24,6 +24,7 @@ SOURCES = [
     ("kq_moe.hip", []),
     ("kq_anymma.hip", ["-ffp-contract=off"]),
     ("kq_codes.hip", []),
+    ("kq_router.hip", ["-ffp-contract=off"]),
 ]
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",

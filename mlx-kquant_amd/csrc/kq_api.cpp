@@ -354,3 +354,20 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
 }
 
 }  // extern "C"
+
+int kq_moe_router_topk(const void* logits_dev, int dtype, int T, int E, int top_k, int norm_topk_prob, int shared_gate,
+                       const float* per_expert_scale_dev, const float* bias_dev, int scoring, float scale,
+                       uint32_t* indices_dev, float* scores_dev, void* stream) {
+  const char* op = "moe_router_topk";
+  if (scoring != 0 && scoring != 1) return kq_set_error(KQ_ERR_INVALID, "%s: scoring must be softmax or sqrtsoftplus", op);
+  if (scoring == 1 && !norm_topk_prob) return kq_set_error(KQ_ERR_INVALID, "%s: sqrtsoftplus requires norm_topk_prob", op);
+  if (dtype != KQ_F32 && dtype != KQ_F16 && dtype != KQ_BF16)
+    return kq_set_error(KQ_ERR_INVALID, "%s: logits must be float32/float16/bfloat16", op);
+  if (T < 0 || E < 1) return kq_set_error(KQ_ERR_INVALID, "%s: bad dimension", op);
+  if (top_k < 1 || top_k > 16 || top_k > E) return kq_set_error(KQ_ERR_INVALID, "%s: top_k must be in [1, min(E, 16)]", op);
+  if (E > 1024) return kq_set_error(KQ_ERR_INVALID, "%s: requires E <= 1024", op);
+  if (T == 0) return KQ_OK;
+  if (!logits_dev || !indices_dev || !scores_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  return kq_launch_router_topk(logits_dev, dtype, T, E, top_k, norm_topk_prob, shared_gate, per_expert_scale_dev,
+                               bias_dev, scoring, scale, indices_dev, scores_dev, static_cast<hipStream_t>(stream));
+}

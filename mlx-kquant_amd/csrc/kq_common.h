@@ -114,3 +114,6 @@ size_t kq_anymma_moe_workspace_bytes(int P, int E);
 int kq_launch_anymma_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
                          const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
                          int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, hipStream_t s);
+// Router top-k (one workgroup per token): see kq_moe_router_topk in include/kq.h.
+int kq_launch_router_topk(const void* logits, int dtype, int T, int E, int top_k, int norm, int shared, const float* pes,
+                          const float* bias, int scoring, float scale, uint32_t* indices, float* scores, hipStream_t s);

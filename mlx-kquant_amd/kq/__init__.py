@@ -24,7 +24,7 @@ _GEOM = {k: (v[3], v[2]) for k, v in CODEC_GEOMETRY.items()}
 
 __all__ = [
     "codecs", "codec_has_matmul", "codec_has_moe_glu", "dequantize", "quantized_matmul", "gather_qmm",
-    "moe_glu_gather_kq", "gather_qmv_kq", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
+    "moe_glu_gather_kq", "gather_qmv_kq", "moe_router_topk", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
     "weights_per_row", "lib_path",
 ]
 
@@ -66,6 +66,7 @@ def _load():
     lib.kq_qmm_workspace_size.restype = sz
     lib.kq_qmm_workspace_size.argtypes = [i, i, i, i, i, i]
     lib.kq_qmm.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
+    lib.kq_moe_router_topk.argtypes = [vp, i, i, i, i, i, i, vp, vp, i, C.c_float, vp, vp, vp]
     lib.kq_gather_qmm_workspace_size.restype = sz
     lib.kq_gather_qmm_workspace_size.argtypes = [i, i, i, i, i, i, i, i]
     lib.kq_gather_qmm.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, i64, i64, i, i, i, i, vp, sz, vp]
@@ -375,6 +376,45 @@ def gather_qmv_kq(x, w, kquant_type, indices, bias=None, *, stream=None):
                                  b.data_ptr() if b is not None else None, out.data_ptr(), T, R, E, N, K, cid,
                                  _DT[x.dtype], ws.data_ptr() if ws is not None else None, ws_bytes, sp))
     return out
+
+
+def moe_router_topk(logits, top_k, norm_topk_prob, shared_gate=True, per_expert_scale=None, bias=None,
+                    scoring="softmax", scale=1.0, *, stream=None):
+    """Router scoring + top-k + mixing weights in one launch: returns (indices int32 [T, top_k] holding the
+    uint32 expert ids, scores float32 [T, top_k + shared_gate]) -- the inputs of the fused MoE ops.
+    Mirrors moe_router_topk, src/kquant_moe_glu.cpp:1366-1441."""
+    op = "moe_router_topk"
+    if scoring not in ("softmax", "sqrtsoftplus"):
+        raise ValueError("[kq.moe_router_topk] scoring must be softmax or sqrtsoftplus.")
+    if scoring == "sqrtsoftplus" and not norm_topk_prob:
+        raise ValueError("[kq.moe_router_topk] sqrtsoftplus requires norm_topk_prob.")
+    if logits.ndim != 2:
+        raise ValueError("[kq.moe_router_topk] logits must be 2-D [T, E + shared_gate].")
+    if logits.dtype not in _DT:
+        raise ValueError("[kq.moe_router_topk] logits must be float32/float16/bfloat16.")
+    shared = 1 if shared_gate else 0
+    T, E = logits.shape[0], logits.shape[1] - shared
+    if top_k < 1 or top_k > 16 or top_k > E:
+        raise ValueError("[kq.moe_router_topk] top_k must be in [1, min(E, 16)].")
+    if E > 1024:
+        raise ValueError("[kq.moe_router_topk] requires E <= 1024.")
+    for name, v in (("per_expert_scale", per_expert_scale), ("bias", bias)):
+        if v is not None and (v.ndim != 1 or v.shape[0] != E):
+            raise ValueError(f"[kq.moe_router_topk] {name} must be 1-D [E].")
+    _same_device(op, logits, per_expert_scale, bias)
+    sp = _stream_ptr(op, logits, stream)
+    l_c = logits.contiguous()
+    pes = per_expert_scale.to(torch.float32).contiguous() if per_expert_scale is not None else None
+    bs = bias.to(torch.float32).contiguous() if bias is not None else None
+    indices = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
+    scores = torch.empty((T, top_k + shared), dtype=torch.float32, device=logits.device)
+    with torch.cuda.device(logits.device):
+        _check(_load().kq_moe_router_topk(l_c.data_ptr(), _DT[logits.dtype], T, E, int(top_k), int(bool(norm_topk_prob)),
+                                          shared, pes.data_ptr() if pes is not None else None,
+                                          bs.data_ptr() if bs is not None else None,
+                                          1 if scoring == "sqrtsoftplus" else 0, float(scale), indices.data_ptr(),
+                                          scores.data_ptr(), sp))
+    return indices, scores
 
 
 def quantize(w, kquant_type, imatrix=None, *, stream=None):

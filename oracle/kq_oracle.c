@@ -18,6 +18,8 @@
  *                     patterns + random f32) and a closed-form bf16 RNE.
  *   qmm / gather    : pinned against numpy float64 `x @ deq(W).T`.
  *   GLU epilogue    : pinned against the numpy formulas the reference tests use.
+ *   router top-k    : pinned against the numpy formulas of the reference's router test
+ *                     (tests/test_moe_glu.py:453-551: softmax / sqrt-softplus, stable argsort, renorm).
  */
 #include "kq_oracle.h"
 
@@ -812,4 +814,68 @@ int kq_oracle_gather_qmv(int codec, void* out, const void* x, const uint8_t* w, 
   free(xf);
   free(y);
   return rc;
+}
+
+int kq_oracle_router_topk(const void* logits, int dtype, int T, int E, int top_k, int norm, int shared,
+                          const float* per_expert_scale, const float* bias, int scoring, float scale,
+                          uint32_t* indices, float* scores) {
+  /* Op contract src/kquant_moe_glu.cpp:1366-1441; kernel semantics kq_moe_glu_kq.h:1215-1358: all math
+   * in f32; top_k rounds of arg-max over p (+ bias), smallest index first on ties, the winner leaves the
+   * pool; emitted scores are the unbiased p, divided by the picked sum (norm; + 1e-20 for sqrt-softplus)
+   * or by the softmax sum, times per_expert_scale[e] and scale; shared: sigmoid of column E last. */
+  if (T < 0 || E < 1 || E > 1024 || top_k < 1 || top_k > 16 || top_k > E) return -1;
+  if (scoring != 0 && scoring != 1) return -1;
+  if (scoring == 1 && !norm) return -1;
+  float* p = (float*)malloc((size_t)E * sizeof(float));
+  for (int t = 0; t < T; t++) {
+    const size_t row = (size_t)t * (E + (shared ? 1 : 0));
+    float gsum = 1.0f;
+    if (scoring == 1) {
+      for (int e = 0; e < E; e++) {
+        const float x = load_in(logits, row + e, dtype);
+        const float z = expf(-fabsf(x));
+        const float l1p = z < 1e-4f ? fmaf(-0.5f * z, z, z) : logf(1.0f + z);
+        p[e] = sqrtf(fmaxf(x, 0.0f) + l1p);
+      }
+    } else {
+      float m = -INFINITY;
+      for (int e = 0; e < E; e++) m = fmaxf(m, load_in(logits, row + e, dtype));
+      float s = 0.f;
+      for (int e = 0; e < E; e++) {
+        p[e] = expf(load_in(logits, row + e, dtype) - m);
+        s += p[e];
+      }
+      gsum = s;
+    }
+    float win_v[16];
+    uint32_t win_i[16];
+    for (int r = 0; r < top_k; r++) {
+      float bv = -INFINITY;
+      uint32_t bi = 0xffffffffu;
+      for (int e = 0; e < E; e++) {
+        const float v = bias ? p[e] + bias[e] : p[e];
+        if (v > bv || (v == bv && (uint32_t)e < bi)) {
+          bv = v;
+          bi = (uint32_t)e;
+        }
+      }
+      if (bi == 0xffffffffu) bi = 0; /* every value NaN: keep the index in range */
+      indices[(size_t)t * top_k + r] = bi;
+      win_v[r] = p[bi];
+      win_i[r] = bi;
+      p[bi] = -INFINITY;
+    }
+    float ps = 0.f;
+    for (int r = 0; r < top_k; r++) ps += win_v[r];
+    const float denom = norm ? (scoring == 1 ? ps + 1e-20f : ps) : gsum;
+    float* srow = scores + (size_t)t * (top_k + (shared ? 1 : 0));
+    for (int r = 0; r < top_k; r++) {
+      float sv = win_v[r] / denom;
+      if (per_expert_scale) sv *= per_expert_scale[win_i[r]];
+      srow[r] = sv * scale;
+    }
+    if (shared) srow[top_k] = 1.0f / (1.0f + expf(-load_in(logits, row + E, dtype)));
+  }
+  free(p);
+  return 0;
 }

@@ -39,6 +39,11 @@ int kq_oracle_moe_glu_gather(int codec, void* out, const void* x, const uint8_t*
                              int N, int K, int act, float limit, float alpha, int dtype);
 int kq_oracle_gather_qmv(int codec, void* out, const void* x, const uint8_t* w, const uint32_t* idx,
                          const float* bias, int T, int R, int N, int K, int dtype);
+/* Router: scores (softmax = 0, sqrt(softplus) = 1) over E logit columns, top_k by score (+ bias), smallest
+ * index first on ties; logits [T][E + shared] in `dtype`, indices [T][top_k], scores f32 [T][top_k + shared]. */
+int kq_oracle_router_topk(const void* logits, int dtype, int T, int E, int top_k, int norm, int shared,
+                          const float* per_expert_scale, const float* bias, int scoring, float scale,
+                          uint32_t* indices, float* scores);
 #ifdef __cplusplus
 }
 #endif

@@ -31,6 +31,7 @@ def _load():
     lib.kq_oracle_gather_qmm.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i64, i64, i, i]
     lib.kq_oracle_moe_glu_gather.argtypes = [i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, f, f, i]
     lib.kq_oracle_gather_qmv.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i]
+    lib.kq_oracle_router_topk.argtypes = [vp, i, i, i, i, i, i, vp, vp, i, f, vp, vp]
     return lib
 
 
@@ -163,6 +164,20 @@ def gather_qmv(x, wire, codec, idx, bias=None, dtype="bfloat16"):
                                   DT[dtype])
     assert rc == 0, rc
     return out
+
+
+def router_topk(logits, dtype, top_k, norm, shared, pes=None, bias=None, scoring=0, scale=1.0):
+    """logits: numpy storage ([T, E + shared] f32, or uint16 bits for the half types)."""
+    logits = np.ascontiguousarray(logits)
+    T, E = logits.shape[0], logits.shape[1] - (1 if shared else 0)
+    p = None if pes is None else np.ascontiguousarray(pes, dtype=np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    idx = np.empty((T, top_k), dtype=np.uint32)
+    sc = np.empty((T, top_k + (1 if shared else 0)), dtype=np.float32)
+    rc = lib.kq_oracle_router_topk(_ptr(logits), DT[dtype], T, E, top_k, int(norm), int(shared), _ptr(p), _ptr(b),
+                                   scoring, scale, _ptr(idx), _ptr(sc))
+    assert rc == 0, rc
+    return idx, sc
 
 
 def synth_wire(codec, n_blocks, seed):
