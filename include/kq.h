@@ -130,6 +130,29 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
                   void* out_dev, int T, int R, int E, int N, int K, int codec, int dtype, void* workspace_dev,
                   size_t workspace_bytes, void* stream);
 
+/* out[t, r < R] as kq_moe_glu_gather (act silu or gelu, no biases); out[t, R] = the same GLU of x[t] against
+ * the block's shared expert, two single [N, bytes_per_row] matrices in `shexp_codec` (the expert codec, or
+ * q6_k / q8_0).  out [T, R + 1, N].  The workspace (kq_moe_glu_gather_shexp_workspace_size bytes, 256-byte
+ * aligned) is required.
+ * Replaces KQuantMoEGLUShexpKQ (op moe_glu_gather_shexp_kq), reference src/kquant_moe_glu.cpp:1212-1272. */
+size_t kq_moe_glu_gather_shexp_workspace_size(int T, int R, int E, int N, int K, int codec, int shexp_codec, int dtype);
+int kq_moe_glu_gather_shexp(const void* x_dev, const void* gate_w_dev, const void* up_w_dev,
+                            const void* shexp_gate_w_dev, const void* shexp_up_w_dev, const uint32_t* idx_dev,
+                            void* out_dev, int T, int R, int E, int N, int K, int act, int codec, int shexp_codec,
+                            int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
+
+/* Down projection with the routing mix folded in: out[t, :] = T(sum_s scores[t, s] * (x[t, s, :] . W_s^T)),
+ * f32 accumulation over the S slots, one rounding.  x [T, S, K], scores f32 [T, S], out [T, N].
+ * shexp_w_dev != NULL: idx is [T, S - 1], slot S - 1 multiplies the shared expert's single matrix (codec
+ * `shexp_codec`: the expert codec, or q6_k / q8_0) -- op gather_qmv_mix_kq; shexp_w_dev == NULL: idx is
+ * [T, S] and every slot gathers from the stack -- op gather_qmv_mix_ns_kq (pass shexp_codec = -1 to the
+ * size query).  The workspace (256-byte aligned) is required.
+ * Replaces KQuantGatherQMVMixKQ / KQuantGatherQMVMixNSKQ, reference src/kquant_moe_glu.cpp:1274-1364. */
+size_t kq_gather_qmv_mix_workspace_size(int T, int S, int E, int N, int K, int codec, int shexp_codec, int dtype);
+int kq_gather_qmv_mix(const void* x_dev, const void* w_dev, const void* shexp_w_dev, const uint32_t* idx_dev,
+                      const float* scores_dev, void* out_dev, int T, int S, int E, int N, int K, int codec,
+                      int shexp_codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* Router: expert scores over the E logit columns (scoring 0 = softmax, 1 = sqrt(softplus(x))), the top_k
  * largest by score (+ bias[e] when given; smallest index first on ties) and their mixing weights:
  * score / (sum of the picked scores (+ 1e-20 for scoring 1) if norm_topk_prob else the softmax sum)

@@ -89,6 +89,7 @@ struct AnyArgs {
   int M, N, K, x_div, act, mtiles;
   int64_t w_expert_stride;
   float limit, alpha;
+  KqOutMap om;          // grouped: where pair results go
   float* partial;       // dense split-K: f32 partial sums [ksplit][M][N] (null: round and store y)
   int steps_per_split;  // dense: K steps per blockIdx.y
 };
@@ -310,7 +311,8 @@ __global__ __launch_bounds__(AM_THREADS, 1) void any_mma_kernel(AnyArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int pr = pair_lds[8 * (i >> 2) + 4 * kg + (i & 3)];
-      if (pr >= 0 && col < ncols) store((size_t)pr * N + n0 + col, acc[0][i] + bv);
+      if (pr >= 0 && col < ncols)
+        kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, pr) * N + n0 + col, acc[0][i] + bv);
     }
   } else {
     lds_barrier();  // the step buffers are free: reuse them for the up accumulators
@@ -331,7 +333,7 @@ __global__ __launch_bounds__(AM_THREADS, 1) void any_mma_kernel(AnyArgs a) {
         const int pr = pair_lds[8 * (i >> 2) + 4 * kg + (i & 3)];
         if (pr >= 0 && live) {
           const float v = kq::glu_epilogue(a.act, acc[0][i] + gb, ex[(nb * 16 + i) * 64 + lane] + ub, a.limit, a.alpha);
-          store((size_t)pr * N + n0 + col, v);
+          kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, pr) * N + n0 + col, v);
         }
       }
     }
@@ -520,5 +522,6 @@ int kq_launch_anymma_moe(const void* x, const uint8_t* w, const uint8_t* w2, con
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
   a.alpha = alpha;
+  a.om = kq_out_map();
   return dispatch_any(codec, a, glu ? 2 : 1, dtype, P, E, s);
 }

@@ -40,6 +40,13 @@ constexpr int kMaxDevices = 64;
 std::mutex g_grid_mu;
 uint8_t* g_grids[kMaxDevices] = {};
 
+thread_local KqOutMap g_out_map = {1, 1, 0, 0};
+// Sets the calling thread's output map for the launches inside a scope.
+struct OutMapScope {
+  explicit OutMapScope(KqOutMap m) { g_out_map = m; }
+  ~OutMapScope() { g_out_map = KqOutMap{1, 1, 0, 0}; }
+};
+
 bool codec_ok(int c) { return c >= 0 && c < KQ_NUM_CODECS; }
 bool half_dtype(int dt) { return dt == KQ_F16 || dt == KQ_BF16; }
 
@@ -52,6 +59,8 @@ int kq_set_error(int code, const char* fmt, ...) {
   va_end(ap);
   return code;
 }
+
+const KqOutMap& kq_out_map(void) { return g_out_map; }
 
 const uint8_t* kq_device_grids(void) {
   int dev = -1;
@@ -354,6 +363,121 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
 }
 
 }  // extern "C"
+
+// ------------------------------------------------------------------ shared-expert / slot-mixing MoE ops
+static bool shexp_combo_ok(int codec, int shexp_codec) {
+  return codec_ok(codec) && codec_ok(shexp_codec) && (shexp_codec == codec || shexp_codec == KQ_Q6_K || shexp_codec == KQ_Q8_0);
+}
+
+size_t kq_moe_glu_gather_shexp_workspace_size(int T, int R, int E, int N, int K, int codec, int shexp_codec, int dtype) {
+  if (T <= 0 || R <= 0) return 0;
+  const size_t a = kq_moe_workspace_size(T, R, E, N, K, 1, codec, dtype);
+  const size_t b = kq_moe_workspace_size(T, 1, 1, N, K, 1, shexp_codec, dtype);
+  return align256((size_t)T * 4) + (a > b ? a : b);
+}
+
+int kq_moe_glu_gather_shexp(const void* x_dev, const void* gate_w_dev, const void* up_w_dev, const void* shexp_gate_w_dev,
+                            const void* shexp_up_w_dev, const uint32_t* idx_dev, void* out_dev, int T, int R, int E, int N,
+                            int K, int act, int codec, int shexp_codec, int dtype, void* workspace_dev,
+                            size_t workspace_bytes, void* stream) {
+  const char* op = "moe_glu_gather_shexp_kq";
+  if (!shexp_combo_ok(codec, shexp_codec))
+    return kq_set_error(KQ_ERR_INVALID, "%s: no fused kernel for this expert / shared-expert codec pair", op);
+  if (act != KQ_ACT_SILU && act != KQ_ACT_GELU) return kq_set_error(KQ_ERR_INVALID, "%s: act must be 'silu' or 'gelu'", op);
+  int rc = check_moe(op, T, R, E, N, K, codec, dtype);
+  if (rc) return rc;
+  rc = check_moe(op, T, 1, 1, N, K, shexp_codec, dtype);
+  if (rc) return rc;
+  if (T == 0 || N == 0) return KQ_OK;
+  if (!shexp_gate_w_dev || !shexp_up_w_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  const size_t need = kq_moe_glu_gather_shexp_workspace_size(T, R, E, N, K, codec, shexp_codec, dtype);
+  if (!workspace_dev || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace_dev) & 255))
+    return kq_set_error(KQ_ERR_WORKSPACE, "%s: 256-byte aligned workspace of %zu bytes required", op, need);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint8_t* wsb = static_cast<uint8_t*>(workspace_dev);
+  uint32_t* idx0 = reinterpret_cast<uint32_t*>(wsb);  // [T] zeros: the shared expert is a one-matrix stack
+  uint8_t* sub = wsb + align256((size_t)T * 4);
+  const size_t sub_bytes = workspace_bytes - align256((size_t)T * 4);
+  if (R > 0) {
+    OutMapScope scope(KqOutMap{R, R + 1, 0, 0});  // slot r of token t -> row t (R + 1) + r
+    rc = kq_moe_glu_gather(x_dev, gate_w_dev, up_w_dev, idx_dev, nullptr, nullptr, out_dev, T, R, E, N, K, act, 0.f, 0.f,
+                           codec, dtype, sub, sub_bytes, stream);
+    if (rc) return rc;
+  }
+  rc = kq_launch_pad_idx(nullptr, idx0, T, 1, s);  // S = 1: every entry is the padded slot, i.e. 0
+  if (rc) return rc;
+  OutMapScope scope(KqOutMap{1, R + 1, R, 0});  // token t -> row t (R + 1) + R
+  return kq_moe_glu_gather(x_dev, shexp_gate_w_dev, shexp_up_w_dev, idx0, nullptr, nullptr, out_dev, T, 1, 1, N, K, act, 0.f,
+                           0.f, shexp_codec, dtype, sub, sub_bytes, stream);
+}
+
+size_t kq_gather_qmv_mix_workspace_size(int T, int S, int E, int N, int K, int codec, int shexp_codec, int dtype) {
+  if (T <= 0 || S <= 0) return 0;
+  size_t fixed = align256((size_t)T * S * N * 4);  // f32 slot results
+  size_t sub = kq_moe_workspace_size(T, S, E, N, K, 0, codec, dtype);
+  if (shexp_codec >= 0) {
+    fixed += align256((size_t)T * S * 4) + align256((size_t)T * 4) + align256((size_t)T * K * 2);
+    const size_t b = kq_moe_workspace_size(T, 1, 1, N, K, 0, shexp_codec, dtype);
+    if (b > sub) sub = b;
+  }
+  return fixed + sub;
+}
+
+int kq_gather_qmv_mix(const void* x_dev, const void* w_dev, const void* shexp_w_dev, const uint32_t* idx_dev,
+                      const float* scores_dev, void* out_dev, int T, int S, int E, int N, int K, int codec,
+                      int shexp_codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream) {
+  const bool shared = shexp_w_dev != nullptr;
+  const char* op = shared ? "gather_qmv_mix_kq" : "gather_qmv_mix_ns_kq";
+  if (shared && !shexp_combo_ok(codec, shexp_codec))
+    return kq_set_error(KQ_ERR_INVALID, "%s: no fused kernel for this expert / shared-expert codec pair", op);
+  if (S < (shared ? 2 : 1)) return kq_set_error(KQ_ERR_INVALID, "%s: bad slot count", op);
+  int rc = check_moe(op, T, S, E, N, K, codec, dtype);
+  if (rc) return rc;
+  if (shared) {
+    rc = check_moe(op, T, 1, 1, N, K, shexp_codec, dtype);
+    if (rc) return rc;
+  }
+  if (T == 0 || N == 0) return KQ_OK;
+  if (!x_dev || !w_dev || !idx_dev || !scores_dev || !out_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  const size_t need = kq_gather_qmv_mix_workspace_size(T, S, E, N, K, codec, shared ? shexp_codec : -1, dtype);
+  if (!workspace_dev || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace_dev) & 255))
+    return kq_set_error(KQ_ERR_WORKSPACE, "%s: 256-byte aligned workspace of %zu bytes required", op, need);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint8_t* wsb = static_cast<uint8_t*>(workspace_dev);
+  float* yf = reinterpret_cast<float*>(wsb);
+  size_t o = align256((size_t)T * S * N * 4);
+  const uint32_t* idx_all = idx_dev;
+  uint32_t* idx0 = nullptr;
+  void* xs = nullptr;
+  if (shared) {
+    uint32_t* idx2 = reinterpret_cast<uint32_t*>(wsb + o);
+    o += align256((size_t)T * S * 4);
+    idx0 = reinterpret_cast<uint32_t*>(wsb + o);
+    o += align256((size_t)T * 4);
+    xs = wsb + o;
+    o += align256((size_t)T * K * 2);
+    rc = kq_launch_pad_idx(idx_dev, idx2, T, S, s);  // the shared slot rides along as expert 0; overwritten below
+    if (rc) return rc;
+    idx_all = idx2;
+  }
+  uint8_t* sub = wsb + o;
+  const size_t sub_bytes = workspace_bytes - o;
+  {
+    OutMapScope scope(KqOutMap{1, 1, 0, 1});  // f32 slot results [T][S][N]
+    rc = kq_gather_qmv(x_dev, w_dev, idx_all, nullptr, yf, T, S, E, N, K, codec, dtype, sub, sub_bytes, stream);
+    if (rc) return rc;
+  }
+  if (shared) {
+    // rows x[t][S - 1] -> dense [T][K], expert ids 0; the shared expert is a one-matrix stack
+    rc = kq_launch_gather_rows(static_cast<const uint16_t*>(x_dev) + (size_t)(S - 1) * K, nullptr, nullptr, xs, idx0, T, 1, K,
+                               (int64_t)S * K, s);
+    if (rc) return rc;
+    OutMapScope scope(KqOutMap{1, S, S - 1, 1});  // token t -> slot row t S + S - 1, f32
+    rc = kq_gather_qmv(xs, shexp_w_dev, idx0, nullptr, yf, T, 1, 1, N, K, shexp_codec, dtype, sub, sub_bytes, stream);
+    if (rc) return rc;
+  }
+  return kq_launch_mix_slots(yf, scores_dev, out_dev, T, S, N, dtype, s);
+}
 
 int kq_moe_router_topk(const void* logits_dev, int dtype, int T, int E, int top_k, int norm_topk_prob, int shared_gate,
                        const float* per_expert_scale_dev, const float* bias_dev, int scoring, float scale,

@@ -650,6 +650,7 @@ struct CgArgs {
   int N, K, x_div, act;
   int64_t w_expert_stride;
   float limit, alpha;
+  KqOutMap om;
 };
 
 constexpr int CG_THREADS = 256;
@@ -905,15 +906,14 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
   }
 
   // ---- epilogue
-  uint16_t* y = static_cast<uint16_t*>(a.y);
-  auto store = [&](size_t off, float v) { y[off] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v); };
   if constexpr (!GLU) {
     const int col = wave * 32 + l32;
     const float bv = (a.bias && col < ncols) ? a.bias[(size_t)seg.expert * N + n0 + col] : 0.f;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int pr = pair_lds[8 * (i >> 2) + 4 * kg + (i & 3)];
-      if (pr >= 0 && col < ncols) store((size_t)pr * N + n0 + col, acc[i] + bv);
+      if (pr >= 0 && col < ncols)
+        kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, pr) * N + n0 + col, acc[i] + bv);
     }
   } else {
     lds_barrier();  // the step buffers are free: reuse them for the up sums
@@ -934,7 +934,7 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
         const int pr = pair_lds[8 * (i >> 2) + 4 * kg + (i & 3)];
         if (pr >= 0 && live) {
           const float v = kq::glu_epilogue(a.act, acc[i] + gb, ex[(nb * 16 + i) * 64 + lane] + ub, a.limit, a.alpha);
-          store((size_t)pr * N + n0 + col, v);
+          kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, pr) * N + n0 + col, v);
         }
       }
     }
@@ -1017,6 +1017,7 @@ int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, cons
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
   a.alpha = alpha;
+  a.om = kq_out_map();
   switch (codec) {
 #define KQ_CASE(c) \
   case c:          \

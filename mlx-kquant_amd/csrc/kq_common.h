@@ -37,7 +37,16 @@ __host__ __device__ constexpr KqGeom kq_geom(int c) {
 #define KQ_GRID_IQ3S 31744
 #define KQ_GRID_BYTES 33792
 
+// Where the gathered / grouped kernels put the result of pair p: output row (p / in) * out + p % in + off,
+// as 16-bit values of the activation dtype or (f32 != 0) as float.  The default {1, 1, 0, 0} is row p,
+// activation dtype.  The fused MoE ops that interleave a shared-expert slot or mix the slots in f32 set
+// another map for the calling thread around their launches (kq_api.cpp); launchers copy kq_out_map().
+struct KqOutMap {
+  int in, out, off, f32;
+};
+
 // ---- host-side plumbing (kq_api.cpp) ----
+const KqOutMap& kq_out_map(void);
 int kq_set_error(int code, const char* fmt, ...);
 // Device copy of the IQ codebooks for the current device (uploaded once per device).
 const uint8_t* kq_device_grids(void);
@@ -88,7 +97,7 @@ int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, co
                           int P, int E, int N, int K, int x_div, int64_t w_expert_stride, int glu, int act,
                           float limit, int codec, int dtype, void* ws, hipStream_t s);
 // Gathered activations of a batched gather_qmm: xg[b*M + m][:] = x[lhs[b]][m][:], idx_rows[b*M + m] = rhs[b]
-// (16-bit elements; K a multiple of 8, x and xg 16-byte aligned).
+// (16-bit elements; K a multiple of 8, x and xg 16-byte aligned).  lhs == null: b; rhs == null: 0.
 int kq_launch_gather_rows(const void* x, const uint32_t* lhs, const uint32_t* rhs, void* xg, uint32_t* idx_rows, int B,
                           int M, int K, int64_t x_batch_stride, hipStream_t s);
 // Skinny-M (M <= 8) matrix-core kernel of the legacy / IQ / fp4 codecs: exact f16 codes in, block scales
@@ -103,6 +112,10 @@ size_t kq_codes_moe_workspace_bytes(int P, int E);
 int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
                         const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
                         int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, hipStream_t s);
+// Helpers of the slot-mixing ops: idx [T][S-1] -> idx2 [T][S] (last slot = expert 0), and
+// out[t][n] = T(sum_s scores[t][s] * yf[t][s][n]).
+int kq_launch_pad_idx(const uint32_t* idx, uint32_t* idx2, int T, int S, hipStream_t s);
+int kq_launch_mix_slots(const float* yf, const float* scores, void* out, int T, int S, int N, int dtype, hipStream_t s);
 // Matrix-core GEMM for every codec (exact bf16 x 3 split of the reference-order decoded weights):
 // prefill, and the batched MoE ops with biases and every activation.
 bool kq_anymma_supported(int M, int N, int K, int codec);

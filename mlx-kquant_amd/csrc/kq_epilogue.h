@@ -3,6 +3,7 @@
 #pragma once
 
 #include "kq_common.h"
+#include "kq_decode.h"
 
 namespace kq {
 __device__ __forceinline__ float glu_epilogue(int act, float g, float u, float limit, float alpha) {
@@ -23,6 +24,18 @@ __device__ __forceinline__ float glu_epilogue(int act, float g, float u, float l
   }
   const float sig = 1.0f / (1.0f + expf(-g));
   return (g * sig) * u;
+}
+
+__device__ __forceinline__ int out_row(const KqOutMap& m, int p) {
+  return m.in == m.out ? p + m.off : (p / m.in) * m.out + (p % m.in) + m.off;
+}
+// one rounding to the activation dtype (DT = KQ_F16 / KQ_BF16), or the f32 value itself
+template <int DT>
+__device__ __forceinline__ void store_result(void* y, const KqOutMap& m, size_t off, float v) {
+  if (m.f32)
+    static_cast<float*>(y)[off] = v;
+  else
+    static_cast<uint16_t*>(y)[off] = DT == KQ_F16 ? f2f16(v) : f2bf16(v);
 }
 
 }  // namespace kq

@@ -154,6 +154,7 @@ struct GatherArgs {
   int64_t x_batch_stride, w_expert_stride;
   int act;
   float limit, alpha;
+  KqOutMap om;
 };
 
 template <int C, int DT, int MT, bool GLU>
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(GV_THREADS) void gather_generic_kernel(GatherArgs a
           if (a.bias2) v2 += a.bias2[(size_t)e * a.N + n];
           v = kq::glu_epilogue(a.act, v, v2, a.limit, a.alpha);
         }
-        store_y<DT>(a.out, ((size_t)p * a.M + (m0 + m)) * a.N + n, v);
+        kq::store_result<DT>(a.out, a.om, ((size_t)kq::out_row(a.om, p) * a.M + (m0 + m)) * a.N + n, v);
       }
     }
   }
@@ -354,6 +355,6 @@ int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2,
   const uint8_t* grids = kq_device_grids();
   if (!grids) return KQ_ERR_HIP;
   GatherArgs a{x, w, w2, lhs, rhs, bias, bias2, out, B, M, N, K, x_div, x_batch_stride, w_expert_stride,
-               act, limit, alpha};
+               act, limit, alpha, kq_out_map()};
   return dispatch_codec<GatherRun>(codec, a, dtype, glu != 0, grids, s);
 }

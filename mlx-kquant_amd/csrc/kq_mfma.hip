@@ -423,6 +423,7 @@ struct SkArgs {
   // split-K (dense calls with few row tiles): grid z = K split; partial sums [ksplit][M][N] f32
   float* partial;
   int ksplit, sb_per_split;
+  KqOutMap om;  // gathered calls: output row of an item, 16-bit or f32 (dense calls: identity)
 };
 
 // MB = M rounded up to a power of two (1, 2, 4, 8).  Rows of the 32-row A operand beyond MB alias
@@ -711,8 +712,8 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
       for (int wv = 0; wv < SK_WAVES; wv++) u += red[(wv * R + r) * 64 + l + half];
       v = kq::glu_epilogue(a.act, v, u, a.limit, 1.0f);
     }
-    uint16_t* yo = static_cast<uint16_t*>(a.y) + ((size_t)item * M + m) * N + row0 + n;
-    *yo = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+    // gathered calls may remap the item's output row (M = 1 there) or ask for f32
+    kq::store_result<DT>(a.y, a.om, ((size_t)kq::out_row(a.om, item) * M + m) * N + row0 + n, v);
   }
 }
 
@@ -1236,7 +1237,10 @@ int launch_skinny(SkArgs a, int items, void* ws, hipStream_t s) {
   if (rows < 8) rows = 8;
   int splits = 1;
   a.ksplit = 1;
-  if (!GLU && items == 1 && ws) {
+  // a dense call: one item, no index arrays, the result as 16-bit values at row 0 (a gathered call of one
+  // item keeps the synchronous kernel, which honours the indices and the output map)
+  const bool dense = items == 1 && !a.lhs && !a.rhs && !a.om.f32 && a.om.in == a.om.out && a.om.off == 0;
+  if (!GLU && dense && ws) {
     const SkSplit p = sk_split_plan(a.N, a.K);
     if (p.ksplit > 1) {
       rows = SK_MAXROWS;
@@ -1253,7 +1257,7 @@ int launch_skinny(SkArgs a, int items, void* ws, hipStream_t s) {
   if constexpr (!GLU) {
     // dense call: decoupled-wave variant (measured 3 - 25 % faster than the synchronous kernel on every
     // decode shape of the sweep)
-    if (items == 1 && g_sk_variant != 1) {
+    if (dense && g_sk_variant != 1) {
       // Diagonal variant (a wave owns 8 rows x 4 adjacent superblocks, no cross-wave reduction): measured
       // 4 - 10 % faster at 5 - 8 activation rows and level or slightly slower below, so it is the default
       // only there; kq_set_skinny_variant(4) selects it wherever the shape allows.
@@ -1423,6 +1427,7 @@ int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, c
   a.x_batch_stride = x_batch_stride;
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
+  a.om = kq_out_map();
   return glu ? launch_skinny_any<true>(a, B, codec, dtype, nullptr, s)
              : launch_skinny_any<false>(a, B, codec, dtype, nullptr, s);
 }

@@ -93,11 +93,32 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __rest
                                                           uint32_t* __restrict__ idx_rows, int M, int K,
                                                           int64_t x_batch_stride) {
   const int p = blockIdx.x, b = p / M, m = p - b * M;
-  const uint16_t* src = x + (size_t)lhs[b] * (size_t)x_batch_stride + (size_t)m * K;
+  const uint16_t* src = x + (size_t)(lhs ? lhs[b] : (uint32_t)b) * (size_t)x_batch_stride + (size_t)m * K;
   uint16_t* dst = xg + (size_t)p * K;
   for (int g = threadIdx.x; g < (K >> 3); g += 256)
     *reinterpret_cast<u32x4*>(dst + 8 * g) = *reinterpret_cast<const u32x4*>(src + 8 * g);
-  if (threadIdx.x == 0) idx_rows[p] = rhs[b];
+  if (threadIdx.x == 0) idx_rows[p] = rhs ? rhs[b] : 0u;
+}
+
+// idx2[t][s] = idx[t][s] for s < S - 1, expert 0 in the last slot (its product is overwritten later)
+__global__ __launch_bounds__(256) void pad_idx_kernel(const uint32_t* __restrict__ idx, uint32_t* __restrict__ idx2, int T,
+                                                      int S) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= T * S) return;
+  const int t = i / S, s = i - t * S;
+  idx2[i] = s < S - 1 ? idx[t * (S - 1) + s] : 0u;
+}
+
+// out[t][n] = T(sum_s scores[t][s] * yf[t][s][n]), f32, slots in order
+template <int DT>
+__global__ __launch_bounds__(256) void mix_slots_kernel(const float* __restrict__ yf, const float* __restrict__ scores,
+                                                        uint16_t* __restrict__ out, int T, int S, int N) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)T * N) return;
+  const int t = (int)(i / N), n = (int)(i - (int64_t)t * N);
+  float v = 0.f;
+  for (int s = 0; s < S; s++) v = fmaf(scores[t * S + s], yf[((size_t)t * S + s) * N + n], v);
+  out[i] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
 }
 
 // ------------------------------------------------------------------ grouped GEMM
@@ -114,6 +135,7 @@ struct MoeArgs {
   int N, K, x_div, act;
   int64_t w_expert_stride;
   float limit;
+  KqOutMap om;
 };
 
 template <int C, int DT, bool GLU>
@@ -252,7 +274,6 @@ __global__ __launch_bounds__(MOE_THREADS, 2) void moe_grouped_kernel(MoeArgs a) 
   }
 
   // ---- epilogue: undo the activation scale, (GLU: combine gate and up,) round once, scatter rows
-  uint16_t* y = static_cast<uint16_t*>(a.y);
   if constexpr (GLU) {
     lds_barrier();  // the step buffers are free: reuse them for the up accumulators
     float* ex = reinterpret_cast<float*>(smem);  // [2 column blocks][16][64]
@@ -271,7 +292,7 @@ __global__ __launch_bounds__(MOE_THREADS, 2) void moe_grouped_kernel(MoeArgs a) 
         if (pr >= 0 && col < ncols) {
           const float r = rs_lds[slot];
           const float v = kq::glu_epilogue(a.act, acc[0][i] * r, ex[(nb * 16 + i) * 64 + lane] * r, a.limit, 1.0f);
-          y[(size_t)pr * N + n0 + col] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+          kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, pr) * N + n0 + col, v);
         }
       }
     }
@@ -283,7 +304,7 @@ __global__ __launch_bounds__(MOE_THREADS, 2) void moe_grouped_kernel(MoeArgs a) 
       const int pr = pair_lds[slot];
       if (pr >= 0 && col < ncols) {
         const float v = acc[0][i] * rs_lds[slot];
-        y[(size_t)pr * N + n0 + col] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+        kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, pr) * N + n0 + col, v);
       }
     }
   }
@@ -367,6 +388,24 @@ int kq_launch_gather_rows(const void* x, const uint32_t* lhs, const uint32_t* rh
   return KQ_OK;
 }
 
+int kq_launch_pad_idx(const uint32_t* idx, uint32_t* idx2, int T, int S, hipStream_t s) {
+  if (T <= 0 || S <= 0) return KQ_OK;
+  hipLaunchKernelGGL(pad_idx_kernel, dim3((T * S + 255) / 256), dim3(256), 0, s, idx, idx2, T, S);
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
+int kq_launch_mix_slots(const float* yf, const float* scores, void* out, int T, int S, int N, int dtype, hipStream_t s) {
+  if (T <= 0 || N <= 0) return KQ_OK;
+  const unsigned blocks = (unsigned)(((int64_t)T * N + 255) / 256);
+  if (dtype == KQ_F16)
+    hipLaunchKernelGGL(mix_slots_kernel<KQ_F16>, dim3(blocks), dim3(256), 0, s, yf, scores, static_cast<uint16_t*>(out), T, S, N);
+  else
+    hipLaunchKernelGGL(mix_slots_kernel<KQ_BF16>, dim3(blocks), dim3(256), 0, s, yf, scores, static_cast<uint16_t*>(out), T, S, N);
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
 bool kq_moe_grouped_supported(int P, int E, int N, int K, int codec) {
   return (codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K) && P > 16 && E <= SORT_MAX_E && K > 0 &&
          (K & 255) == 0 && N > 0 && (int64_t)E + P / SEG_M < 65535;
@@ -406,5 +445,6 @@ int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, co
   a.act = act;
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
+  a.om = kq_out_map();
   return glu ? launch_grouped_any<true>(a, P, E, codec, dtype, s) : launch_grouped_any<false>(a, P, E, codec, dtype, s);
 }

@@ -24,7 +24,8 @@ _GEOM = {k: (v[3], v[2]) for k, v in CODEC_GEOMETRY.items()}
 
 __all__ = [
     "codecs", "codec_has_matmul", "codec_has_moe_glu", "dequantize", "quantized_matmul", "gather_qmm",
-    "moe_glu_gather_kq", "gather_qmv_kq", "moe_router_topk", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
+    "moe_glu_gather_kq", "gather_qmv_kq", "moe_glu_gather_shexp_kq", "gather_qmv_mix_kq", "gather_qmv_mix_ns_kq",
+    "moe_router_topk", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
     "weights_per_row", "lib_path",
 ]
 
@@ -66,6 +67,12 @@ def _load():
     lib.kq_qmm_workspace_size.restype = sz
     lib.kq_qmm_workspace_size.argtypes = [i, i, i, i, i, i]
     lib.kq_qmm.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
+    lib.kq_moe_glu_gather_shexp_workspace_size.restype = sz
+    lib.kq_moe_glu_gather_shexp_workspace_size.argtypes = [i, i, i, i, i, i, i, i]
+    lib.kq_moe_glu_gather_shexp.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, i, vp, sz, vp]
+    lib.kq_gather_qmv_mix_workspace_size.restype = sz
+    lib.kq_gather_qmv_mix_workspace_size.argtypes = [i, i, i, i, i, i, i, i]
+    lib.kq_gather_qmv_mix.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp, sz, vp]
     lib.kq_moe_router_topk.argtypes = [vp, i, i, i, i, i, i, vp, vp, i, C.c_float, vp, vp, vp]
     lib.kq_gather_qmm_workspace_size.restype = sz
     lib.kq_gather_qmm_workspace_size.argtypes = [i, i, i, i, i, i, i, i]
@@ -376,6 +383,116 @@ def gather_qmv_kq(x, w, kquant_type, indices, bias=None, *, stream=None):
                                  b.data_ptr() if b is not None else None, out.data_ptr(), T, R, E, N, K, cid,
                                  _DT[x.dtype], ws.data_ptr() if ws is not None else None, ws_bytes, sp))
     return out
+
+
+def _shexp_codec(op, kquant_type, shexp_kquant_type):
+    """shexp_combo_has_kernel, src/kquant_moe_glu.cpp:852-858."""
+    st = shexp_kquant_type or kquant_type
+    if not (kquant_type in CODEC_GEOMETRY and st in CODEC_GEOMETRY and codec_has_moe_glu(kquant_type)
+            and codec_has_moe_glu(st) and (st == kquant_type or st in ("q6_k", "q8_0"))):
+        raise ValueError(f"[kq.{op}] no fused kernel for expert codec '{kquant_type}' with shared-expert codec '{st}'.")
+    return st
+
+
+def _check_shexp_row(op, w, kquant_type, K, N):
+    """check_kq_shexp_row, src/kquant_moe_glu.cpp:900-925."""
+    wpb, bpb = _GEOM[kquant_type]
+    if w.ndim != 2 or w.dtype != torch.uint8:
+        raise ValueError(f"[kq.{op}] shared-expert weights must be uint8 [N, bytes_per_row].")
+    if K % wpb != 0 or w.shape[0] != N or w.shape[1] != K // wpb * bpb:
+        raise ValueError(f"[kq.{op}] shared-expert weights must match the expert stack row shape.")
+    if not w.is_contiguous():
+        raise ValueError(f"[kq.{op}] weights must be row-contiguous.")
+
+
+def moe_glu_gather_shexp_kq(x, gate_w, up_w, shexp_gate_w, shexp_up_w, kquant_type, indices, act="silu",
+                            shexp_kquant_type="", *, stream=None):
+    """moe_glu_gather_kq with the block's shared expert folded in as one extra slot: [T, R + 1, N], the last
+    slot is the shared expert.  Mirrors moe_glu_gather_shexp_kq, src/kquant_moe_glu.cpp:1212-1272."""
+    op = "moe_glu_gather_shexp_kq"
+    st = _shexp_codec(op, kquant_type, shexp_kquant_type)
+    if x.ndim != 2:
+        raise ValueError("[kq.moe_glu_gather_shexp_kq] x must be 2-D [T, K].")
+    if indices.ndim != 2 or indices.shape[0] != x.shape[0]:
+        raise ValueError("[kq.moe_glu_gather_shexp_kq] indices must be [T, R].")
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("[kq.moe_glu_gather_shexp_kq] x must be float16 or bfloat16.")
+    if act not in ("silu", "gelu"):
+        raise ValueError("[kq.moe_glu_gather_shexp_kq] act must be 'silu' or 'gelu'.")
+    K = x.shape[1]
+    _check_kq_expert_stack(op, gate_w, kquant_type, K)
+    _check_kq_expert_stack(op, up_w, kquant_type, K)
+    if gate_w.shape[0] != up_w.shape[0] or gate_w.shape[1] != up_w.shape[1]:
+        raise ValueError("[kq.moe_glu_gather_shexp_kq] gate/up expert shapes must match.")
+    E, N = gate_w.shape[0], gate_w.shape[1]
+    _check_shexp_row(op, shexp_gate_w, st, K, N)
+    _check_shexp_row(op, shexp_up_w, st, K, N)
+    _same_device(op, x, gate_w, up_w, shexp_gate_w, shexp_up_w, indices)
+    sp = _stream_ptr(op, x, stream)
+    cid, _ = _codec(op, kquant_type)
+    sid, _ = _codec(op, st)
+    x_c = x.contiguous()
+    idx = _prep_idx(indices)
+    T, R = idx.shape
+    out = torch.empty((T, R + 1, N), dtype=x.dtype, device=x.device)
+    lib = _load()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.kq_moe_glu_gather_shexp_workspace_size(T, R, E, N, K, cid, sid, _DT[x.dtype])
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=x.device)
+        _check(lib.kq_moe_glu_gather_shexp(x_c.data_ptr(), gate_w.data_ptr(), up_w.data_ptr(), shexp_gate_w.data_ptr(),
+                                           shexp_up_w.data_ptr(), idx.data_ptr(), out.data_ptr(), T, R, E, N, K,
+                                           _ACTS[act], cid, sid, _DT[x.dtype], ws.data_ptr(), ws_bytes, sp))
+    return out
+
+
+def _gather_qmv_mix(op, x, w, shexp_w, kquant_type, st, indices, scores, stream):
+    if x.ndim != 3:
+        raise ValueError(f"[kq.{op}] x must be 3-D [T, S, K].")
+    T, S, K = x.shape
+    want = S - 1 if shexp_w is not None else S
+    if indices.ndim != 2 or indices.shape[0] != T or indices.shape[1] != want:
+        raise ValueError(f"[kq.{op}] indices must be [T, {'S - 1' if shexp_w is not None else 'S'}].")
+    if scores.ndim != 2 or scores.shape[0] != T or scores.shape[1] != S:
+        raise ValueError(f"[kq.{op}] scores must be [T, S].")
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError(f"[kq.{op}] x must be float16 or bfloat16.")
+    _check_kq_expert_stack(op, w, kquant_type, K)
+    E, N = w.shape[0], w.shape[1]
+    if shexp_w is not None:
+        _check_shexp_row(op, shexp_w, st, K, N)
+    _same_device(op, x, w, shexp_w, indices, scores)
+    sp = _stream_ptr(op, x, stream)
+    cid, _ = _codec(op, kquant_type)
+    sid = _codec(op, st)[0] if shexp_w is not None else -1
+    x_c = x.contiguous()
+    idx = _prep_idx(indices)
+    sc = scores.to(torch.float32).contiguous()
+    out = torch.empty((T, N), dtype=x.dtype, device=x.device)
+    lib = _load()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.kq_gather_qmv_mix_workspace_size(T, S, E, N, K, cid, sid, _DT[x.dtype])
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=x.device)
+        _check(lib.kq_gather_qmv_mix(x_c.data_ptr(), w.data_ptr(), shexp_w.data_ptr() if shexp_w is not None else None,
+                                     idx.data_ptr(), sc.data_ptr(), out.data_ptr(), T, S, E, N, K, cid, sid,
+                                     _DT[x.dtype], ws.data_ptr(), ws_bytes, sp))
+    return out
+
+
+def gather_qmv_mix_kq(x, w, shexp_w, kquant_type, indices, scores, shexp_kquant_type="", *, stream=None):
+    """Down projection with the routing mix folded in: x [T, S, K] (slot S-1 = shared expert), indices
+    [T, S-1], scores [T, S]; f32 accumulation over the S slots, returns [T, N].
+    Mirrors gather_qmv_mix_kq, src/kquant_moe_glu.cpp:1274-1323."""
+    op = "gather_qmv_mix_kq"
+    st = _shexp_codec(op, kquant_type, shexp_kquant_type)
+    if shexp_w is None:
+        raise ValueError("[kq.gather_qmv_mix_kq] shexp_w is required (use gather_qmv_mix_ns_kq without a shared expert).")
+    return _gather_qmv_mix(op, x, w, shexp_w, kquant_type, st, indices, scores, stream)
+
+
+def gather_qmv_mix_ns_kq(x, w, kquant_type, indices, scores, *, stream=None):
+    """No-shared-expert routing mix: x [T, S, K], indices [T, S], scores [T, S]; returns [T, N].
+    Mirrors gather_qmv_mix_ns_kq, src/kquant_moe_glu.cpp:1325-1364."""
+    return _gather_qmv_mix("gather_qmv_mix_ns_kq", x, w, None, kquant_type, kquant_type, indices, scores, stream)
 
 
 def moe_router_topk(logits, top_k, norm_topk_prob, shared_gate=True, per_expert_scale=None, bias=None,

@@ -18,6 +18,8 @@
  *                     patterns + random f32) and a closed-form bf16 RNE.
  *   qmm / gather    : pinned against numpy float64 `x @ deq(W).T`.
  *   GLU epilogue    : pinned against the numpy formulas the reference tests use.
+ *   shexp / mix ops : compositions of the pinned matvec and epilogue; checked against the numpy
+ *                     compositions of the reference's tests (tests/test_moe_glu.py:234-310).
  *   router top-k    : pinned against the numpy formulas of the reference's router test
  *                     (tests/test_moe_glu.py:453-551: softmax / sqrt-softplus, stable argsort, renorm).
  */
@@ -813,6 +815,72 @@ int kq_oracle_gather_qmv(int codec, void* out, const void* x, const uint8_t* w, 
   }
   free(xf);
   free(y);
+  return rc;
+}
+
+int kq_oracle_moe_glu_gather_shexp(int codec, int shexp_codec, void* out, const void* x, const uint8_t* gate_w,
+                                   const uint8_t* up_w, const uint8_t* shexp_gate_w, const uint8_t* shexp_up_w,
+                                   const uint32_t* idx, int T, int R, int N, int K, int act, int dtype) {
+  /* Op contract src/kquant_moe_glu.cpp:1212-1272: slots r < R as moe_glu_gather_kq, slot R = the same GLU
+   * against the shared expert's two matrices (f32 throughout, one rounding). */
+  const kq_oracle_codec_t* c = kq_oracle_codec(codec);
+  const kq_oracle_codec_t* sc = kq_oracle_codec(shexp_codec);
+  if (!c || !sc || K % c->weights_per_block || K % sc->weights_per_block || dtype == 0) return -1;
+  const size_t ebytes = (size_t)N * (K / c->weights_per_block) * c->bytes_per_block;
+  float* xf = (float*)malloc((size_t)K * sizeof(float));
+  float* g = (float*)malloc((size_t)N * sizeof(float));
+  float* u = (float*)malloc((size_t)N * sizeof(float));
+  int rc = 0;
+  for (int t = 0; t < T && rc == 0; t++) {
+    for (int k = 0; k < K; k++) xf[k] = load_in(x, (size_t)t * K + k, dtype);
+    for (int r = 0; r <= R && rc == 0; r++) {
+      if (r < R) {
+        const uint32_t e = idx[(size_t)t * R + r];
+        rc = kq_oracle_qmm_f32(codec, g, xf, gate_w + e * ebytes, 1, N, K, 1);
+        if (!rc) rc = kq_oracle_qmm_f32(codec, u, xf, up_w + e * ebytes, 1, N, K, 1);
+      } else {
+        rc = kq_oracle_qmm_f32(shexp_codec, g, xf, shexp_gate_w, 1, N, K, 1);
+        if (!rc) rc = kq_oracle_qmm_f32(shexp_codec, u, xf, shexp_up_w, 1, N, K, 1);
+      }
+      for (int n = 0; n < N && rc == 0; n++)
+        store_out(out, ((size_t)t * (R + 1) + r) * N + n, kq_oracle_glu_epilogue(act, g[n], u[n], 0.f, 0.f), dtype);
+    }
+  }
+  free(xf);
+  free(g);
+  free(u);
+  return rc;
+}
+
+int kq_oracle_gather_qmv_mix(int codec, int shexp_codec, void* out, const void* x, const uint8_t* w,
+                             const uint8_t* shexp_w, const uint32_t* idx, const float* scores, int T, int S, int N,
+                             int K, int dtype) {
+  /* Op contracts src/kquant_moe_glu.cpp:1274-1364: every slot's matvec in f32, the score-weighted sum
+   * accumulates in f32 in slot order, one rounding to the activation dtype. */
+  const kq_oracle_codec_t* c = kq_oracle_codec(codec);
+  if (!c || K % c->weights_per_block || dtype == 0 || S < 1) return -1;
+  const size_t ebytes = (size_t)N * (K / c->weights_per_block) * c->bytes_per_block;
+  const int routed = shexp_w ? S - 1 : S;
+  float* xf = (float*)malloc((size_t)K * sizeof(float));
+  float* y = (float*)malloc((size_t)N * sizeof(float));
+  float* acc = (float*)malloc((size_t)N * sizeof(float));
+  int rc = 0;
+  for (int t = 0; t < T && rc == 0; t++) {
+    for (int n = 0; n < N; n++) acc[n] = 0.f;
+    for (int s = 0; s < S && rc == 0; s++) {
+      for (int k = 0; k < K; k++) xf[k] = load_in(x, ((size_t)t * S + s) * K + k, dtype);
+      if (s < routed)
+        rc = kq_oracle_qmm_f32(codec, y, xf, w + idx[(size_t)t * routed + s] * ebytes, 1, N, K, 1);
+      else
+        rc = kq_oracle_qmm_f32(shexp_codec, y, xf, shexp_w, 1, N, K, 1);
+      const float sc = scores[(size_t)t * S + s];
+      for (int n = 0; n < N; n++) acc[n] = fmaf(sc, y[n], acc[n]);
+    }
+    for (int n = 0; n < N && rc == 0; n++) store_out(out, (size_t)t * N + n, acc[n], dtype);
+  }
+  free(xf);
+  free(y);
+  free(acc);
   return rc;
 }
 

@@ -39,6 +39,14 @@ int kq_oracle_moe_glu_gather(int codec, void* out, const void* x, const uint8_t*
                              int N, int K, int act, float limit, float alpha, int dtype);
 int kq_oracle_gather_qmv(int codec, void* out, const void* x, const uint8_t* w, const uint32_t* idx,
                          const float* bias, int T, int R, int N, int K, int dtype);
+/* moe_glu_gather with the shared expert as slot R: out [T][R + 1][N]. */
+int kq_oracle_moe_glu_gather_shexp(int codec, int shexp_codec, void* out, const void* x, const uint8_t* gate_w,
+                                   const uint8_t* up_w, const uint8_t* shexp_gate_w, const uint8_t* shexp_up_w,
+                                   const uint32_t* idx, int T, int R, int N, int K, int act, int dtype);
+/* out[t][:] = T(sum_s scores[t][s] * x[t][s][:] . W_s^T); shexp_w != NULL: idx [T][S-1], slot S-1 uses shexp_w. */
+int kq_oracle_gather_qmv_mix(int codec, int shexp_codec, void* out, const void* x, const uint8_t* w,
+                             const uint8_t* shexp_w, const uint32_t* idx, const float* scores, int T, int S, int N,
+                             int K, int dtype);
 /* Router: scores (softmax = 0, sqrt(softplus) = 1) over E logit columns, top_k by score (+ bias), smallest
  * index first on ties; logits [T][E + shared] in `dtype`, indices [T][top_k], scores f32 [T][top_k + shared]. */
 int kq_oracle_router_topk(const void* logits, int dtype, int T, int E, int top_k, int norm, int shared,

@@ -31,6 +31,8 @@ def _load():
     lib.kq_oracle_gather_qmm.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i64, i64, i, i]
     lib.kq_oracle_moe_glu_gather.argtypes = [i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, f, f, i]
     lib.kq_oracle_gather_qmv.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i]
+    lib.kq_oracle_moe_glu_gather_shexp.argtypes = [i, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i]
+    lib.kq_oracle_gather_qmv_mix.argtypes = [i, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i]
     lib.kq_oracle_router_topk.argtypes = [vp, i, i, i, i, i, i, vp, vp, i, f, vp, vp]
     return lib
 
@@ -162,6 +164,34 @@ def gather_qmv(x, wire, codec, idx, bias=None, dtype="bfloat16"):
     out = np.empty((T, R, N), dtype=np.uint16)
     rc = lib.kq_oracle_gather_qmv(codec_id(codec), _ptr(out), _ptr(x), _ptr(wire), _ptr(idx), _ptr(b), T, R, N, K,
                                   DT[dtype])
+    assert rc == 0, rc
+    return out
+
+
+def moe_glu_gather_shexp(x, gate, up, sgate, sup, codec, shexp_codec, idx, act="silu", dtype="bfloat16"):
+    x = np.ascontiguousarray(x)
+    idx = np.ascontiguousarray(idx, dtype=np.uint32)
+    T, K = x.shape
+    R, N = idx.shape[1], gate.shape[1]
+    out = np.empty((T, R + 1, N), dtype=np.uint16)
+    arrs = [np.ascontiguousarray(a, dtype=np.uint8) for a in (gate, up, sgate, sup)]
+    rc = lib.kq_oracle_moe_glu_gather_shexp(codec_id(codec), codec_id(shexp_codec), _ptr(out), _ptr(x), *map(_ptr, arrs),
+                                            _ptr(idx), T, R, N, K, {"silu": 0, "gelu": 1}[act], DT[dtype])
+    assert rc == 0, rc
+    return out
+
+
+def gather_qmv_mix(x, wire, shexp_wire, codec, shexp_codec, idx, scores, dtype="bfloat16"):
+    x = np.ascontiguousarray(x)
+    wire = np.ascontiguousarray(wire, dtype=np.uint8)
+    sw = None if shexp_wire is None else np.ascontiguousarray(shexp_wire, dtype=np.uint8)
+    idx = np.ascontiguousarray(idx, dtype=np.uint32)
+    sc = np.ascontiguousarray(scores, dtype=np.float32)
+    T, S, K = x.shape
+    N = wire.shape[1]
+    out = np.empty((T, N), dtype=np.uint16)
+    rc = lib.kq_oracle_gather_qmv_mix(codec_id(codec), codec_id(shexp_codec or codec), _ptr(out), _ptr(x), _ptr(wire),
+                                      _ptr(sw), _ptr(idx), _ptr(sc), T, S, N, K, DT[dtype])
     assert rc == 0, rc
     return out
 

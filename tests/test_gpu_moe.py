@@ -70,6 +70,21 @@ def test_gather_qmm_batched(kq, codec, M):
         assert rel_l2(dev_to_bits(got).reshape(B, M, N), want, dtype) <= TOL, (codec, M, dtype)
 
 
+@pytest.mark.parametrize("codec", ["q4_k", "q6_k", "q2_k", "q8_0"])
+def test_single_entry_picks_its_expert(kq, codec):
+    """A gathered call of ONE entry must still honour its expert index (it must not take the dense-call
+    kernels, which read the stack's first matrix)."""
+    E, N, K = 4, 64, 1024
+    wire = _stack(codec, E, N, K, seed=71)
+    xb, xt = make_x((1, 1, K), "bfloat16", seed=72)
+    for e in (0, 3):
+        got = kq.gather_qmm(xt, wire_to_dev(wire), None, codec, rhs_indices=_idx_dev(np.array([e])))
+        want = O.gather_qmm(xb, wire, codec, np.array([0]), np.array([e]), True, "bfloat16")
+        assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, e)
+        got = kq.gather_qmv_kq(xt, wire_to_dev(wire), codec, _idx_dev(np.array([[e]])))
+        assert rel_l2(dev_to_bits(got), O.gather_qmv(xb, wire, codec, np.array([[e]]), None, "bfloat16"), "bfloat16") <= TOL
+
+
 @pytest.mark.parametrize("codec", ["q4_k", "q8_0", "iq4_nl", "q6_k"])
 def test_gather_qmm_no_transpose(kq, codec):
     """transpose=False: every expert decodes to [K, N] (the MLA / LoRA-vjp orientation)."""
