@@ -81,6 +81,12 @@ size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int 
 int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int transpose,
            int codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* Decode-only matvec with the layer bias fused in: y[n] = T(x . W[n]^T + float(bias[n])), one activation row,
+ * bias [N] in the activation dtype, q8_0 only (as wired in the reference).
+ * Replaces KQuantQmvBias (op quantized_matmul_qmv_bias), reference src/kquant_ops.cpp:185-270. */
+int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int N, int K, int codec,
+                int dtype, void* stream);
+
 /* Tuning hook without a counterpart in the reference: activation rows per workgroup tile of the
  * prefill GEMM, 64 or 128 (anything else restores the default, 64).  Process-wide, not thread-safe. */
 void kq_set_gemm_tile_rows(int rows);

@@ -160,9 +160,24 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
   int rc = kq_launch_qmm_tuned(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev,
                                workspace_bytes, s);
   if (rc != KQ_ERR_UNSUPPORTED) return rc;
-  rc = kq_launch_codes_skinny(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+  rc = kq_launch_codes_skinny(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, y_dev, M, N, K, codec, dtype, s);
   if (rc != KQ_ERR_UNSUPPORTED) return rc;
   return kq_launch_gemv_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+}
+
+int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int N, int K, int codec,
+                int dtype, void* stream) {
+  const char* op = "quantized_matmul_qmv_bias";
+  if (codec != KQ_Q8_0) return kq_set_error(KQ_ERR_INVALID, "%s: only kquant_type 'q8_0' is wired", op);
+  if (!half_dtype(dtype)) return kq_set_error(KQ_ERR_INVALID, "%s: activations must be float16 or bfloat16", op);
+  if (N < 0 || K < 0 || K % kCodecs[codec].weights_per_block)
+    return kq_set_error(KQ_ERR_INVALID, "%s: bad dimension", op);
+  if (N == 0) return KQ_OK;
+  if (!x_dev || !w_dev || !bias_dev || !y_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  const int rc = kq_launch_codes_skinny(x_dev, static_cast<const uint8_t*>(w_dev), bias_dev, y_dev, 1, N, K, codec, dtype,
+                                        static_cast<hipStream_t>(stream));
+  if (rc == KQ_ERR_UNSUPPORTED) return kq_set_error(KQ_ERR_UNSUPPORTED, "%s: x must be 16-byte aligned", op);
+  return rc;
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }

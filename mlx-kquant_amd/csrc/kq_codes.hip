@@ -344,6 +344,7 @@ struct CkArgs {
   const void* x;  // [M][K]
   const uint8_t* w;
   void* y;        // [M][N]
+  const uint16_t* bias;  // [N] in the activation dtype, added in f32 before the rounding; or null
   const uint8_t* grids;
   int M, N, K;
 };
@@ -591,7 +592,10 @@ __global__ __launch_bounds__(CK_THREADS, 1) void codes_skinny_kernel(CkArgs a) {
 #pragma unroll
       for (int w = 0; w < CK_WAVES; w++) v += red[(w * 4 + i) * 64 + lane];
       const int m = 4 * kg + i;
-      if (m < M && n < N) y[(size_t)m * N + n] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+      if (m < M && n < N) {
+        if (a.bias) v += DT == KQ_F16 ? kq::h2f(a.bias[n]) : kq::bf162f(a.bias[n]);
+        y[(size_t)m * N + n] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+      }
     }
   }
 }
@@ -1035,13 +1039,14 @@ bool kq_codes_supported(int M, int N, int K, int codec) {
   return M > 0 && M <= CK_MAXM && N > 0 && K > 0 && K % kq_geom(codec).wpb == 0;
 }
 
-int kq_launch_codes_skinny(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
-                           hipStream_t s) {
+int kq_launch_codes_skinny(const void* x, const uint8_t* w, const void* bias, void* y, int M, int N, int K, int codec,
+                           int dtype, hipStream_t s) {
   if (!kq_codes_supported(M, N, K, codec) || (reinterpret_cast<uintptr_t>(x) & 15) || (K & 7)) return KQ_ERR_UNSUPPORTED;
   CkArgs a{};
   a.x = x;
   a.w = w;
   a.y = y;
+  a.bias = static_cast<const uint16_t*>(bias);
   a.grids = kq_device_grids();
   if (!a.grids) return KQ_ERR_HIP;
   a.M = M;

@@ -103,8 +103,9 @@ int kq_launch_gather_rows(const void* x, const uint32_t* lhs, const uint32_t* rh
 // Skinny-M (M <= 8) matrix-core kernel of the legacy / IQ / fp4 codecs: exact f16 codes in, block scales
 // applied to the f32 partial sums.  Same fall-through contract as kq_launch_qmm_tuned; no workspace.
 bool kq_codes_supported(int M, int N, int K, int codec);
-int kq_launch_codes_skinny(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
-                           hipStream_t s);
+// bias: [N] in the activation dtype (added in f32 before the single rounding) or null
+int kq_launch_codes_skinny(const void* x, const uint8_t* w, const void* bias, void* y, int M, int N, int K, int codec,
+                           int dtype, hipStream_t s);
 // Batched MoE of the same codecs (more than 16 pairs; biases and every activation): pairs sorted by expert,
 // 32-pair segments x 128-row slabs.  Workspace layout and size as the any-codec path below.
 bool kq_codes_moe_supported(int P, int E, int N, int K, int codec);

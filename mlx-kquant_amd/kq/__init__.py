@@ -23,7 +23,8 @@ from .codec_geometry import CODEC_GEOMETRY, bytes_per_row, weights_per_row
 _GEOM = {k: (v[3], v[2]) for k, v in CODEC_GEOMETRY.items()}
 
 __all__ = [
-    "codecs", "codec_has_matmul", "codec_has_moe_glu", "dequantize", "quantized_matmul", "gather_qmm",
+    "codecs", "codec_has_matmul", "codec_has_moe_glu", "dequantize", "quantized_matmul", "quantized_matmul_qmv_bias",
+    "gather_qmm",
     "moe_glu_gather_kq", "gather_qmv_kq", "moe_glu_gather_shexp_kq", "gather_qmv_mix_kq", "gather_qmv_mix_ns_kq",
     "moe_router_topk", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
     "weights_per_row", "lib_path",
@@ -67,6 +68,7 @@ def _load():
     lib.kq_qmm_workspace_size.restype = sz
     lib.kq_qmm_workspace_size.argtypes = [i, i, i, i, i, i]
     lib.kq_qmm.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
+    lib.kq_qmv_bias.argtypes = [vp, vp, vp, vp, i, i, i, i, vp]
     lib.kq_moe_glu_gather_shexp_workspace_size.restype = sz
     lib.kq_moe_glu_gather_shexp_workspace_size.argtypes = [i, i, i, i, i, i, i, i]
     lib.kq_moe_glu_gather_shexp.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, i, vp, sz, vp]
@@ -219,6 +221,37 @@ def quantized_matmul(x, w, scales, kquant_type, transpose=True, *, stream=None):
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
         _check(lib.kq_qmm(x_c.data_ptr(), w_c.data_ptr(), out.data_ptr(), M, N, K, int(bool(transpose)), cid,
                           _DT[out_type], ws.data_ptr() if ws is not None else None, ws_bytes, sp))
+    return out
+
+
+def quantized_matmul_qmv_bias(x, w, scales, bias, kquant_type, *, stream=None):
+    """Decode-only y = x @ W.T + bias with the add fused into the matvec (f32 sum, one rounding): exactly one
+    activation row, q8_0 only.  Mirrors quantized_matmul_qmv_bias, src/kquant_ops.cpp:185-270."""
+    op = "quantized_matmul_qmv_bias"
+    if kquant_type != "q8_0":
+        raise ValueError(f"[kq.quantized_matmul_qmv_bias] only kquant_type 'q8_0' is wired so far, got '{kquant_type}'.")
+    if w.dtype != torch.uint8:
+        raise ValueError("[kq.quantized_matmul_qmv_bias] w must be uint8 (raw GGUF wire bytes).")
+    if w.ndim != 2:
+        raise ValueError("[kq.quantized_matmul_qmv_bias] w must be 2D (this op is not batched); use gather_qmm for "
+                         "mixture-of-experts.")
+    cid, K, N = _expand_geometry(op, x, w, kquant_type, True)
+    if bias.ndim != 1 or bias.shape[0] != N:
+        raise ValueError(f"[kq.quantized_matmul_qmv_bias] bias must be 1D with length {N} (the output dim), got shape "
+                         f"{tuple(bias.shape)}.")
+    if x.numel() // x.shape[-1] != 1:
+        raise ValueError(f"[kq.quantized_matmul_qmv_bias] decode-only: x must carry exactly one row (got "
+                         f"{x.numel() // x.shape[-1]}). Use quantized_matmul() + a separate add for prefill/verify shapes.")
+    out_type = _out_dtype(op, x)
+    _same_device(op, x, w, bias)
+    sp = _stream_ptr(op, x, stream)
+    x_c = x.to(out_type).contiguous()
+    w_c = w.contiguous()
+    b_c = bias.to(out_type).contiguous()
+    out = torch.empty(list(x.shape[:-1]) + [N], dtype=out_type, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(_load().kq_qmv_bias(x_c.data_ptr(), w_c.data_ptr(), b_c.data_ptr(), out.data_ptr(), N, K, cid,
+                                   _DT[out_type], sp))
     return out
 
 

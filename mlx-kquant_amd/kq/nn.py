@@ -92,6 +92,9 @@ class KQuantLinear(_KQuantBase):
             self.bias = None
 
     def forward(self, x):
+        # decode (one row) with a real bias on q8_0: the add is fused into the matvec (reference :122-140)
+        if self.bias is not None and self.kquant_type == "q8_0" and x.numel() // x.shape[-1] == 1:
+            return kq.quantized_matmul_qmv_bias(x, self.weight, self.scales, self.bias, self.kquant_type)
         y = kq.quantized_matmul(x, self.weight, self.scales, self.kquant_type, transpose=True)
         if self.bias is not None:
             y = y + self.bias

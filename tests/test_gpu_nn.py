@@ -44,7 +44,13 @@ def test_linear(knn, codec, bias):
         y = layer(xt)
         want = O.bits_to_f32(O.qmm(xb.reshape(-1, K), wire, codec, True, "bfloat16"), "bfloat16").reshape(*shape[:-1], N)
         assert tuple(y.shape) == (*shape[:-1], N)
-        if bias:
+        if bias and codec == "q8_0" and shape == (1, K):
+            # fused decode path: x.W^T in f32 + the bias rounded to bf16, one rounding of the sum
+            assert y.dtype == torch.bfloat16
+            f32 = O.qmm(O.bits_to_f32(xb, "bfloat16").reshape(1, K), wire, codec, True, "float32")
+            bb = O.bits_to_f32(O.f32_to_bits(b, "bfloat16"), "bfloat16")
+            assert rel_l2(dev_to_bits(y), O.f32_to_bits(f32 + bb, "bfloat16"), "bfloat16") <= TOL
+        elif bias:
             assert y.dtype == torch.float32  # bf16 + f32 bias promotes, as in the reference
             assert _rel(y.cpu().numpy(), want + b) <= TOL
         else:
