@@ -134,3 +134,50 @@ def test_multi_linear(knn, codec):
     assert rel_l2(dev_to_bits(y).reshape(B * H, L, IN), want, "float16") <= TOL
     with pytest.raises(ValueError):
         layer(torch.zeros((B, 3, L, IN), dtype=torch.float16, device="cuda:0"))
+
+
+def test_checkpoint_and_gguf_feed_the_kernels(knn, tmp_path):
+    """float model -> kq.quantize -> checkpoint on disk -> load -> install on the GPU: the swapped layers compute
+    x @ decode(wire).T (oracle parity), and the same wire bytes travel through a GGUF file unchanged."""
+    from kq import checkpoint, gguf
+
+    class Toy(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.embed = torch.nn.Embedding(64, 256)
+            self.up = torch.nn.Linear(256, 128, bias=False)
+            self.down = torch.nn.Linear(128 * 2, 256, bias=True)
+
+        def forward(self, ids):
+            h = self.up(self.embed(ids))
+            return self.down(torch.cat([h, h], dim=-1))
+
+    torch.manual_seed(1)
+    ref = Toy()
+    state = {k: v.detach().clone() for k, v in ref.state_dict().items()}
+    tensors, per = checkpoint.quantize_state(state, {"embed": "q8_0", "up": "q4_k", "down": "q6_k"})
+    d = str(tmp_path / "toy")
+    checkpoint.save(d, tensors, per, config={"model_type": "toy"})
+    model = checkpoint.install(Toy(), checkpoint.load(d), device="cuda:0")
+    assert isinstance(model.up, knn.KQuantLinear) and model.up.weight.is_cuda
+    ids = torch.tensor([[1, 5, 9], [63, 0, 2]], device="cuda:0")
+    y = model(ids)
+    assert tuple(y.shape) == (2, 3, 256)
+    # layer by layer against the oracle on the same wire bytes
+    e = model.embed(ids)
+    want_e = O.f32_to_bits(O.bits_to_f32(O.dequantize(tensors["embed.weight"].numpy()[ids.cpu().numpy().reshape(-1)], "q8_0",
+                                                      "float16"), "float16"), "bfloat16").reshape(2, 3, 256)
+    assert np.array_equal(dev_to_bits(e), want_e)
+    h = model.up(e)
+    want_h = O.qmm(dev_to_bits(e).reshape(6, 256), tensors["up.weight"].numpy(), "q4_k", True, "bfloat16")
+    assert rel_l2(dev_to_bits(h).reshape(6, 128), want_h, "bfloat16") <= TOL
+    # and close to the float model within the codecs' error
+    y_ref = ref(ids.cpu()).detach().numpy()
+    assert _rel(y.float().cpu().numpy(), y_ref) < 0.15
+    # the same bytes through a GGUF file
+    path = str(tmp_path / "toy.gguf")
+    gguf.save_gguf(path, {"up.weight": tensors["up.weight"], "down.weight": tensors["down.weight"]},
+                   {"up.weight": "q4_k", "down.weight": "q6_k"}, {"general.architecture": "toy"})
+    g = gguf.load_gguf(path, device="cuda:0")
+    layer = knn.KQuantLinear(256, 128, False, dict(g.codecs)["up.weight"], device="cuda:0").load_wire(g.arrays["up.weight"])
+    assert torch.equal(layer(e), h)
