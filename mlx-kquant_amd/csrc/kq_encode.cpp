@@ -1,6 +1,6 @@
 // Host-side wire encoders behind kq_quantize: float rows -> GGUF block bytes for the five legacy
 // 32-weight codecs, the five K-quant superblock codecs, the two non-linear 4-bit codecs
-// (iq4_nl, iq4_xs) and three codebook codecs (iq2_xxs, iq3_xxs, iq3_s).  Like the reference's encoder
+// (iq4_nl, iq4_xs) and five codebook codecs (iq2_xxs, iq2_xs, iq2_s, iq3_xxs, iq3_s).  Like the reference's encoder
 // (src/kquant_cpu_encode.cpp:38-859, ggml's search heuristics) this runs on the CPU; unlike it,
 // blocks are encoded in parallel (blocks are independent).  Operation order inside a block
 // follows the cited reference lines so that, on the same x86 host arithmetic, the bytes agree.
@@ -12,7 +12,7 @@
 //             final re-quantisation of every weight)
 //   iq4     : iq4_nl / iq4_xs, src/kquant_iq_encode.cpp:49-214 (ggml quantize_row_iq4_nl_impl: nearest
 //             codebook entry, weighted least-squares scale, 15 trial scales around max / -127)
-//   codebook: iq2_xxs :392-598, iq3_xxs :1087-1310, iq3_s :1319-1544 (lattice search over the codebook
+//   codebook: iq2_xxs :392-598, iq2_xs :600-818, iq2_s :821-1029, iq3_xxs :1087-1310, iq3_s :1319-1544 (lattice search over the codebook
 //             with its neighbour index :228-331; one shared implementation driven by a traits table)
 #include <algorithm>
 #include <cfloat>
@@ -521,7 +521,7 @@ void enc_iq4(const float* x, const float* im, uint8_t* b) {
     for (int j = 0; j < 16; j++) qs[16 * i + j] = (uint8_t)(lv[32 * i + j] | (lv[32 * i + 16 + j] << 4));
 }
 
-// ------------------------------------------------------------------ codebook codecs (iq2_xxs, iq3_xxs, iq3_s)
+// ------------------------------------------------------------------ codebook codecs (iq2_xxs, iq2_xs, iq2_s, iq3_xxs, iq3_s)
 // A 32-weight sub-block is a scale times odd lattice points 2 l + 1 that must belong to a codebook
 // of 8-value (iq2) or 4-value (iq3) groups, plus one sign per weight.  The search representation
 // is derived from the decode codebooks linked into the library: the level of a value is its rank
@@ -599,12 +599,14 @@ void build_codebook(Codebook& cb, const uint8_t* values, int size, int dim, int 
   }
 }
 
-enum { CB_IQ2XXS = 0, CB_IQ3XXS, CB_IQ3S, CB_COUNT };
+enum { CB_IQ2XXS = 0, CB_IQ2XS, CB_IQ2S, CB_IQ3XXS, CB_IQ3S, CB_COUNT };
 const Codebook& codebook(int which) {
   static Codebook books[CB_COUNT];
   static std::once_flag once[CB_COUNT];
   std::call_once(once[which], [which] {
     if (which == CB_IQ2XXS) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ2XXS, 256, 8, 2, 2);
+    if (which == CB_IQ2XS) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ2XS, 512, 8, 2, 2);
+    if (which == CB_IQ2S) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ2S, 1024, 8, 2, 1);
     if (which == CB_IQ3XXS) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ3XXS, 256, 4, 3, 2);
     if (which == CB_IQ3S) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ3S, 512, 4, 3, 3);
   });
@@ -649,6 +651,8 @@ int snap_group(const Codebook& cb, const float* xv, const float* sw, float inv, 
 }
 
 struct CbTraits {
+  int nw;               // weights per sub-block (one scale): 32 or 16
+  float fallback_sigma; // importance without an imatrix: fallback_sigma * sigma2 + x^2
   int book, maxq;       // codebook, levels per coordinate
   float sigma_factor;   // importance prologue
   bool parity_signs;    // 7 stored sign bits per 8 weights (even parity enforced) vs 8
@@ -660,9 +664,11 @@ struct CbTraits {
                         // 2: only the snapped groups
   float d_fudge;
 };
-constexpr CbTraits kIq2xxs{CB_IQ2XXS, 3, 1.0f, true, 1e-15f, true, 6, 0.1f, 0, 1.0f};
-constexpr CbTraits kIq3xxs{CB_IQ3XXS, 8, 2.0f, true, 1e-8f, false, 15, 0.2f, 2, 1.0125f};
-constexpr CbTraits kIq3s{CB_IQ3S, 8, 2.0f, false, 0.0f, false, 9, 0.2f, 1, 1.033f};
+constexpr CbTraits kIq2xxs{32, 0.f, CB_IQ2XXS, 3, 1.0f, true, 1e-15f, true, 6, 0.1f, 0, 1.0f};
+constexpr CbTraits kIq2xs{16, 0.f, CB_IQ2XS, 3, 1.0f, true, 1e-15f, false, 9, 0.1f, 2, 1.0f};
+constexpr CbTraits kIq2s{16, 0.25f, CB_IQ2S, 3, 2.0f, false, 1e-8f, false, 9, 0.1f, 2, 0.9875f};
+constexpr CbTraits kIq3xxs{32, 0.f, CB_IQ3XXS, 8, 2.0f, true, 1e-8f, false, 15, 0.2f, 2, 1.0125f};
+constexpr CbTraits kIq3s{32, 0.f, CB_IQ3S, 8, 2.0f, false, 0.0f, false, 9, 0.2f, 1, 1.033f};
 
 // One 32-weight sub-block: magnitudes, signs, weights in; levels, codebook entries, sign bytes and the
 // scale out (ggml quantize_row_iq2_xxs_impl / iq3_xxs_impl / iq3_s_impl; reference :392-598, :1087-1310,
@@ -670,13 +676,13 @@ constexpr CbTraits kIq3s{CB_IQ3S, 8, 2.0f, false, 0.0f, false, 9, 0.2f, 1, 1.033
 float fit_codebook_subblock(const CbTraits& t, const float* xb, const float* imat, float sigma2, uint8_t* signs,
                             int* entries) {
   const Codebook& cb = codebook(t.book);
-  const int ngroups = 32 / cb.dim;
+  const int nw = t.nw, ngroups = nw / cb.dim;
   float wt[32], sw[32], xv[32];
-  for (int i = 0; i < 32; i++) {
-    wt[i] = imat ? imat[i] * std::sqrt(sigma2 + xb[i] * xb[i]) : xb[i] * xb[i];
+  for (int i = 0; i < nw; i++) {
+    wt[i] = imat ? imat[i] * std::sqrt(sigma2 + xb[i] * xb[i]) : t.fallback_sigma * sigma2 + xb[i] * xb[i];
     sw[i] = std::sqrt(wt[i]);
   }
-  for (int k = 0; k < 4; k++) {
+  for (int k = 0; k < nw / 8; k++) {
     uint8_t s = 0;
     int flips = 0;
     for (int i = 0; i < 8; i++) {
@@ -707,15 +713,15 @@ float fit_codebook_subblock(const CbTraits& t, const float* xb, const float* ima
   }
   for (int g = 0; g < ngroups; g++) entries[g] = 0;
   float vmax = xv[0];
-  for (int i = 1; i < 32; i++) vmax = std::max(vmax, xv[i]);
+  for (int i = 1; i < nw; i++) vmax = std::max(vmax, xv[i]);
   if (t.zero_eps > 0.f ? vmax < t.zero_eps : !(vmax != 0.f)) return 0.f;
 
-  int8_t lv[32] = {}, trial[32];
+  int8_t lv[32] = {}, trial[32] = {};
   bool exact[8], trial_exact[8];
   float scale, span;
   if (t.qp_start) {
     uint8_t tmp[32];
-    scale = fit_positive(xv, wt, 32, t.maxq + 1, tmp);
+    scale = fit_positive(xv, wt, nw, t.maxq + 1, tmp);
     span = scale * float(t.maxq);
     if (span <= 0.f) return 0.f;
     for (int g = 0; g < ngroups; g++) exact[g] = true;
@@ -726,7 +732,7 @@ float fit_codebook_subblock(const CbTraits& t, const float* xb, const float* ima
   }
   auto sums = [&](const int8_t* l, float& sqx, float& sq2) {
     sqx = sq2 = 0.f;
-    for (int i = 0; i < 32; i++) {
+    for (int i = 0; i < nw; i++) {
       const float q = float(2 * l[i] + 1);
       sqx += wt[i] * xv[i] * q;
       sq2 += wt[i] * q * q;
@@ -763,7 +769,7 @@ float fit_codebook_subblock(const CbTraits& t, const float* xb, const float* ima
   }
   if (scale < 0.f) {  // cannot happen with non-negative magnitudes; keep the wire's unsigned scale valid anyway
     scale = -scale;
-    for (int k = 0; k < 4; k++) signs[k] = uint8_t(~signs[k]) & (t.parity_signs ? 127 : 255);
+    for (int k = 0; k < nw / 8; k++) signs[k] = uint8_t(~signs[k]) & (t.parity_signs ? 127 : 255);
   }
   for (int g = 0; g < ngroups; g++) {
     int packed = 0;
@@ -835,6 +841,47 @@ void enc_codebook(const float* x, const float* im, uint8_t* b) {
   }
 }
 
+// iq2_xs (74 bytes: d | 32 x u16 = 9-bit entry + 7 sign bits | 8 scale bytes) and iq2_s (82 bytes: d | 32 entry
+// low bytes | 32 sign bytes | 8 bytes of entry bits 8-9 | 8 scale bytes): sixteen 16-weight sub-blocks of two
+// 8-value groups, a 4-bit scale each (reference :600-818, :821-1029).
+template <int kWhich>  // KQ_IQ2_XS, KQ_IQ2_S
+void enc_codebook16(const float* x, const float* im, uint8_t* b) {
+  const CbTraits& t = kWhich == KQ_IQ2_XS ? kIq2xs : kIq2s;
+  constexpr int kBytes = kWhich == KQ_IQ2_XS ? 74 : 82;
+  float total = 0.f;
+  for (int i = 0; i < 256; i++) total += x[i] * x[i];
+  const float sigma2 = t.sigma_factor * total / 256.0f;
+  float scales[16], top = 0.f;
+  uint8_t signs[16][4];
+  int entries[16][8];
+  for (int ib = 0; ib < 16; ib++) {
+    scales[ib] = fit_codebook_subblock(t, x + 16 * ib, im ? im + 16 * ib : nullptr, sigma2, signs[ib], entries[ib]);
+    top = std::max(top, scales[ib]);
+  }
+  std::memset(b, 0, kBytes);
+  if (!(top > 0.f)) return;
+  const float d = top / 31.0f, inv_d = 1.0f / d;
+  put_f16(b, d * t.d_fudge);
+  for (int ib = 0; ib < 16; ib++) {
+    for (int k = 0; k < 2; k++) {
+      const int g = 2 * ib + k;
+      const bool live = scales[ib] > 0.f;
+      const int entry = live ? entries[ib][k] : 0;
+      const int sg = live ? signs[ib][k] : 0;
+      if constexpr (kWhich == KQ_IQ2_XS) {
+        const uint16_t q = uint16_t(entry | (sg << 9));
+        std::memcpy(b + 2 + 2 * g, &q, 2);
+      } else {
+        b[2 + g] = uint8_t(entry & 255);
+        b[34 + g] = uint8_t(sg);
+        b[66 + g / 4] |= uint8_t((entry >> 8) << (2 * (g % 4)));
+      }
+    }
+    const int l = scale_level(inv_d, scales[ib]);
+    b[(kWhich == KQ_IQ2_XS ? 66 : 74) + ib / 2] |= uint8_t(ib % 2 ? l << 4 : l);
+  }
+}
+
 typedef void (*BlockEnc)(const float*, const float*, uint8_t*);
 void legacy_q8_0(const float* x, const float*, uint8_t* b) { enc_q8_0(x, b); }
 void legacy_q4_0(const float* x, const float*, uint8_t* b) { enc_legacy<false, 4>(x, b); }
@@ -857,6 +904,8 @@ BlockEnc encoder_for(int codec) {
     case KQ_IQ4_NL: return enc_iq4<32>;
     case KQ_IQ4_XS: return enc_iq4<256>;
     case KQ_IQ2_XXS: return enc_codebook<KQ_IQ2_XXS>;
+    case KQ_IQ2_XS: return enc_codebook16<KQ_IQ2_XS>;
+    case KQ_IQ2_S: return enc_codebook16<KQ_IQ2_S>;
     case KQ_IQ3_XXS: return enc_codebook<KQ_IQ3_XXS>;
     case KQ_IQ3_S: return enc_codebook<KQ_IQ3_S>;
   }

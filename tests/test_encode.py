@@ -143,7 +143,7 @@ def test_iq4_known_answer_blocks():
 
 
 # ------------------------------------------------------------------ codebook codecs (iq2_xxs, iq3_xxs, iq3_s)
-CB_BOUND = {"iq2_xxs": 0.45, "iq3_xxs": 0.30, "iq3_s": 0.30}  # reference tests/test_iq_encode.py:36-41
+CB_BOUND = {"iq2_xxs": 0.45, "iq2_xs": 0.45, "iq2_s": 0.45, "iq3_xxs": 0.30, "iq3_s": 0.30}  # reference tests/test_iq_encode.py:36-41
 
 
 @pytest.mark.parametrize("codec", list(CB_BOUND))
@@ -160,7 +160,7 @@ def test_codebook_round_trip_bounds(codec):
     assert rel < CB_BOUND[codec], (codec, rel)
     assert rel > 0.02  # a 2-3 bit codec cannot be this good: guards against a vacuous decode
     assert np.array_equal(wire, _enc(w, codec, im))
-    if codec == "iq2_xxs":
+    if codec in ("iq2_xxs", "iq2_xs"):
         with pytest.raises(ValueError):
             kq.quantize(torch.from_numpy(w), codec)  # imatrix-required, as ggml_quantize_requires_imatrix
     else:
@@ -197,6 +197,29 @@ def test_iq2_xxs_known_answer_blocks():
     assert np.mean(sa == sb) > 0.99  # 4 x 7 sign bits
     back = O.dequantize(mine, "iq2_xxs").reshape(24, 256)
     assert np.linalg.norm(back - x) / np.linalg.norm(x) < 0.10
+
+
+@pytest.mark.parametrize("codec", ["iq2_xs", "iq2_s"])
+def test_iq2_16_known_answer_blocks(codec):
+    """As above for the 16-weight sub-block codecs: decoded codebook points re-encode to the same entries
+    (9- / 10-bit indices split over qs and the u16 / qh fields) and the same sign bits."""
+    nsb = 24
+    wire = O.synth_wire(codec, nsb, 8).reshape(nsb, -1).copy()
+    wire[:, 0:2] = np.frombuffer(np.float16(2.0 ** -6).tobytes(), dtype=np.uint8)
+    soff = 66 if codec == "iq2_xs" else 74
+    wire[:, soff:soff + 8] |= 0x33  # no sub-block scale below 3: keeps every sub-block well above the noise floor
+    wire[:, soff] |= 0x0F
+    x = O.dequantize(wire, codec).reshape(nsb, 256)
+    mine = _enc(x, codec, np.ones(256, np.float32))
+    if codec == "iq2_xs":
+        a, b = wire[:, 2:66].copy().view(np.uint16), mine[:, 2:66].copy().view(np.uint16)
+        assert np.mean((a & 511) == (b & 511)) > 0.95 and np.mean((a >> 9) == (b >> 9)) > 0.99
+    else:
+        assert np.mean(wire[:, 2:34] == mine[:, 2:34]) > 0.95    # entry low bytes
+        assert np.mean(wire[:, 66:74] == mine[:, 66:74]) > 0.90  # entry bits 8-9, four groups per byte
+        assert np.mean(wire[:, 34:66] == mine[:, 34:66]) > 0.99  # sign bytes
+    back = O.dequantize(mine, codec).reshape(nsb, 256)
+    assert np.linalg.norm(back - x) / np.linalg.norm(x) < 0.12
 
 
 @pytest.mark.parametrize("codec", ["iq3_xxs", "iq3_s"])
