@@ -537,14 +537,18 @@ struct Codebook {
   std::vector<uint16_t> near;  // per off-codebook point: count, entries...
 };
 
-void build_codebook(Codebook& cb, const uint8_t* values, int size, int dim, int bits, int rings) {
+void build_codebook(Codebook& cb, const uint8_t* values, int size, int dim, int bits, int rings, bool is_signed = false) {
   cb.dim = dim;
   cb.bits = bits;
   cb.size = size;
   bool seen[256] = {};
   for (int i = 0; i < size * dim; i++) seen[values[i]] = true;
   int level_of[256], nlevels = 0;
-  for (int v = 0; v < 256; v++) level_of[v] = seen[v] ? nlevels++ : -1;
+  // levels by rank of the value (int8 values for the ternary codebook: -1, 0, 1)
+  for (int r = 0; r < 256; r++) {
+    const int v = is_signed ? ((r + 128) & 255) : r;  // -128 .. 127 in order, as bytes
+    level_of[v] = seen[v] ? nlevels++ : -1;
+  }
   cb.pts.resize((size_t)size * dim);
   const int npacked = 1 << (bits * dim), mask = (1 << bits) - 1;
   cb.slot.assign(npacked, 0);
@@ -599,7 +603,7 @@ void build_codebook(Codebook& cb, const uint8_t* values, int size, int dim, int 
   }
 }
 
-enum { CB_IQ2XXS = 0, CB_IQ2XS, CB_IQ2S, CB_IQ3XXS, CB_IQ3S, CB_COUNT };
+enum { CB_IQ2XXS = 0, CB_IQ2XS, CB_IQ2S, CB_IQ3XXS, CB_IQ3S, CB_IQ1, CB_COUNT };
 const Codebook& codebook(int which) {
   static Codebook books[CB_COUNT];
   static std::once_flag once[CB_COUNT];
@@ -609,6 +613,7 @@ const Codebook& codebook(int which) {
     if (which == CB_IQ2S) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ2S, 1024, 8, 2, 1);
     if (which == CB_IQ3XXS) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ3XXS, 256, 4, 3, 2);
     if (which == CB_IQ3S) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ3S, 512, 4, 3, 3);
+    if (which == CB_IQ1) build_codebook(books[which], kq_grid_blob_host + KQ_GRID_IQ1S, 2048, 8, 2, 3, true);
   });
   return books[which];
 }
@@ -882,6 +887,124 @@ void enc_codebook16(const float* x, const float* im, uint8_t* b) {
   }
 }
 
+// ------------------------------------------------------------------ iq1_s
+// 50 bytes: d | 32 entry low bytes | 8 x u16 (4 x 3 entry high bits, 3-bit scale, shift sign).  A 32-weight
+// sub-block is scale * (t + shift / 8) with t in {-1, 0, 1} drawn from the 2048-entry ternary codebook and one
+// shift sign per sub-block.  The ternary split comes from an exhaustive search over the two boundaries in the
+// sorted values (prefix sums of w x and w), for both shift signs; groups that miss the codebook snap to the
+// best of their neighbours (ggml quantize_row_iq1_s_impl; reference :1546-1798).
+void enc_iq1_s(const float* x, const float* im, uint8_t* b) {
+  const Codebook& cb = codebook(CB_IQ1);
+  constexpr float kDelta = 0.125f;
+  const float vp[3] = {-1.f + kDelta, kDelta, 1.f + kDelta}, vm[3] = {-1.f - kDelta, -kDelta, 1.f - kDelta};
+  float total = 0.f;
+  for (int i = 0; i < 256; i++) total += x[i] * x[i];
+  const float sigma2 = 2.0f * total / 256.0f;
+  float scales[8], top = 0.f;
+  int shifts[8], entries[8][4];
+  for (int ib = 0; ib < 8; ib++) {
+    const float* xb = x + 32 * ib;
+    scales[ib] = 0.f;
+    shifts[ib] = 1;
+    for (int k = 0; k < 4; k++) entries[ib][k] = 0;
+    float wt[32], vmax = 0.f;
+    for (int i = 0; i < 32; i++) {
+      wt[i] = (im ? im[32 * ib + i] : 1.0f) * std::sqrt(sigma2 + xb[i] * xb[i]);
+      vmax = std::max(vmax, std::fabs(xb[i]));
+    }
+    if (vmax < 1e-12f) continue;
+    int order[32];
+    for (int i = 0; i < 32; i++) order[i] = i;
+    std::stable_sort(order, order + 32, [&](int l, int r) { return xb[l] < xb[r]; });
+    float sx[33], sw[33];
+    sx[0] = sw[0] = 0.f;
+    for (int j = 0; j < 32; j++) {
+      sx[j + 1] = sx[j] + wt[order[j]] * xb[order[j]];
+      sw[j + 1] = sw[j] + wt[order[j]];
+    }
+    float best = -FLT_MAX, scale = vmax;
+    int b1 = -1, b2 = -1, shift = 0;
+    for (int i1 = 0; i1 <= 32; i1++)
+      for (int i2 = i1; i2 <= 32; i2++)
+        for (int sgn = 1; sgn >= -1; sgn -= 2) {
+          const float* v = sgn > 0 ? vp : vm;
+          const float sqx = (sx[i1] - sx[0]) * v[0] + (sx[i2] - sx[i1]) * v[1] + (sx[32] - sx[i2]) * v[2];
+          const float sq2 = (sw[i1] - sw[0]) * v[0] * v[0] + (sw[i2] - sw[i1]) * v[1] * v[1] + (sw[32] - sw[i2]) * v[2] * v[2];
+          if (sq2 > 0.f && sqx * sqx > best * sq2) {
+            scale = sqx / sq2;
+            best = scale * sqx;
+            b1 = i1;
+            b2 = i2;
+            shift = sgn;
+          }
+        }
+    if (b1 < 0 || shift == 0) continue;
+    int8_t lv[32];
+    for (int j = 0; j < 32; j++) lv[order[j]] = int8_t(j < b1 ? 0 : j < b2 ? 1 : 2);
+    if (scale < 0.f) {
+      for (int j = 0; j < 32; j++) lv[j] = int8_t(2 - lv[j]);
+      scale = -scale;
+      shift = -shift;
+    }
+    const float* v = shift > 0 ? vp : vm;
+    bool all_exact = true;
+    for (int k = 0; k < 4; k++) {
+      int packed = 0;
+      for (int i = 0; i < 8; i++) packed |= int(lv[8 * k + i]) << (2 * i);
+      int32_t slot = cb.slot[packed];
+      if (slot < 0) {
+        all_exact = false;
+        const uint16_t* cand = cb.near.data() + (-slot - 1);
+        float least = FLT_MAX;
+        int pick = -1;
+        for (int c = 1; c <= int(cand[0]); c++) {
+          const int8_t* pt = cb.pts.data() + (size_t)cand[c] * 8;
+          float err = 0.f;
+          for (int i = 0; i < 8; i++) {
+            const float df = scale * v[(pt[i] - 1) / 2] - xb[8 * k + i];
+            err += wt[8 * k + i] * df * df;
+          }
+          if (err < least) {
+            least = err;
+            pick = cand[c];
+          }
+        }
+        slot = pick < 0 ? 0 : pick;
+        const int8_t* pt = cb.pts.data() + (size_t)slot * 8;
+        for (int i = 0; i < 8; i++) lv[8 * k + i] = int8_t((pt[i] - 1) / 2);
+      }
+      entries[ib][k] = slot;
+    }
+    if (!all_exact) {
+      float sqx = 0.f, sq2 = 0.f;
+      for (int i = 0; i < 32; i++) {
+        const float q = v[lv[i]];
+        sqx += wt[i] * q * xb[i];
+        sq2 += wt[i] * q * q;
+      }
+      if (sqx > 0.f && sq2 > 0.f) scale = sqx / sq2;
+    }
+    scales[ib] = scale;
+    shifts[ib] = shift;
+    top = std::max(top, scale);
+  }
+  std::memset(b, 0, 50);
+  if (!(top > 0.f)) return;
+  const float d = top / 15.0f, inv_d = 1.0f / d;
+  put_f16(b, d * 1.125f);
+  for (int ib = 0; ib < 8; ib++) {
+    uint16_t h = 0;
+    for (int k = 0; k < 4; k++) {
+      b[2 + 4 * ib + k] = uint8_t(entries[ib][k] & 255);
+      h |= uint16_t((entries[ib][k] >> 8) << (3 * k));
+    }
+    int l = clampi(rne(0.5f * (inv_d * scales[ib] - 1.0f)), 0, 7);
+    if (shifts[ib] == -1) l |= 8;
+    h |= uint16_t(l << 12);
+    std::memcpy(b + 34 + 2 * ib, &h, 2);
+  }
+}
+
 typedef void (*BlockEnc)(const float*, const float*, uint8_t*);
 void legacy_q8_0(const float* x, const float*, uint8_t* b) { enc_q8_0(x, b); }
 void legacy_q4_0(const float* x, const float*, uint8_t* b) { enc_legacy<false, 4>(x, b); }
@@ -906,6 +1029,7 @@ BlockEnc encoder_for(int codec) {
     case KQ_IQ2_XXS: return enc_codebook<KQ_IQ2_XXS>;
     case KQ_IQ2_XS: return enc_codebook16<KQ_IQ2_XS>;
     case KQ_IQ2_S: return enc_codebook16<KQ_IQ2_S>;
+    case KQ_IQ1_S: return enc_iq1_s;
     case KQ_IQ3_XXS: return enc_codebook<KQ_IQ3_XXS>;
     case KQ_IQ3_S: return enc_codebook<KQ_IQ3_S>;
   }

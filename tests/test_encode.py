@@ -143,7 +143,8 @@ def test_iq4_known_answer_blocks():
 
 
 # ------------------------------------------------------------------ codebook codecs (iq2_xxs, iq3_xxs, iq3_s)
-CB_BOUND = {"iq2_xxs": 0.45, "iq2_xs": 0.45, "iq2_s": 0.45, "iq3_xxs": 0.30, "iq3_s": 0.30}  # reference tests/test_iq_encode.py:36-41
+CB_BOUND = {"iq2_xxs": 0.45, "iq2_xs": 0.45, "iq2_s": 0.45, "iq3_xxs": 0.30, "iq3_s": 0.30,
+            "iq1_s": 0.65}  # reference tests/test_iq_encode.py:36-43
 
 
 @pytest.mark.parametrize("codec", list(CB_BOUND))
@@ -160,7 +161,7 @@ def test_codebook_round_trip_bounds(codec):
     assert rel < CB_BOUND[codec], (codec, rel)
     assert rel > 0.02  # a 2-3 bit codec cannot be this good: guards against a vacuous decode
     assert np.array_equal(wire, _enc(w, codec, im))
-    if codec in ("iq2_xxs", "iq2_xs"):
+    if codec in ("iq2_xxs", "iq2_xs", "iq1_s"):
         with pytest.raises(ValueError):
             kq.quantize(torch.from_numpy(w), codec)  # imatrix-required, as ggml_quantize_requires_imatrix
     else:
@@ -252,3 +253,23 @@ def test_codebook_zero_and_imatrix():
         ea = np.sum(steep * (O.dequantize(a, codec) - w) ** 2)
         eb = np.sum(steep * (O.dequantize(b, codec) - w) ** 2)
         assert eb < ea * 1.02, (codec, ea, eb)
+
+
+def test_iq1_s_known_answer_blocks():
+    """Ternary codebook points (decode of a valid wire) re-encode to the same entries and shift signs: checks the
+    int8 level map of the 2048-entry codebook, the 11-bit entry split over qs / qh and the shift bit."""
+    nsb = 24
+    wire = O.synth_wire("iq1_s", nsb, 9).reshape(nsb, 50).copy()
+    wire[:, 0:2] = np.frombuffer(np.float16(2.0 ** -5).tobytes(), dtype=np.uint8)
+    qh = wire[:, 34:50].copy().view(np.uint16)
+    qh[:] = (qh & 0x8FFF) | (np.random.default_rng(10).integers(2, 8, qh.shape).astype(np.uint16) << 12)
+    qh[:, 0] |= 0x7000
+    wire[:, 34:50] = qh.view(np.uint8)
+    x = O.dequantize(wire, "iq1_s").reshape(nsb, 256)
+    mine = _enc(x, "iq1_s", np.ones(256, np.float32))
+    mq = mine[:, 34:50].copy().view(np.uint16)
+    assert np.mean(wire[:, 2:34] == mine[:, 2:34]) > 0.97          # entry low bytes
+    assert np.mean((qh & 0x0FFF) == (mq & 0x0FFF)) > 0.95          # 4 x 3 entry high bits
+    assert np.mean((qh & 0x8000) == (mq & 0x8000)) > 0.97          # shift signs
+    back = O.dequantize(mine, "iq1_s").reshape(nsb, 256)
+    assert np.linalg.norm(back - x) / np.linalg.norm(x) < 0.15
