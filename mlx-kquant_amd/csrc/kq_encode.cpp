@@ -1,6 +1,6 @@
 // Host-side wire encoders behind kq_quantize: float rows -> GGUF block bytes for the five legacy
 // 32-weight codecs, the five K-quant superblock codecs, the two non-linear 4-bit codecs
-// (iq4_nl, iq4_xs) and five codebook codecs (iq2_xxs, iq2_xs, iq2_s, iq3_xxs, iq3_s).  Like the reference's encoder
+// (iq4_nl, iq4_xs) and seven codebook codecs (iq2_xxs, iq2_xs, iq2_s, iq3_xxs, iq3_s, iq1_s, iq1_m).  Like the reference's encoder
 // (src/kquant_cpu_encode.cpp:38-859, ggml's search heuristics) this runs on the CPU; unlike it,
 // blocks are encoded in parallel (blocks are independent).  Operation order inside a block
 // follows the cited reference lines so that, on the same x86 host arithmetic, the bytes agree.
@@ -14,6 +14,7 @@
 //             codebook entry, weighted least-squares scale, 15 trial scales around max / -127)
 //   codebook: iq2_xxs :392-598, iq2_xs :600-818, iq2_s :821-1029, iq3_xxs :1087-1310, iq3_s :1319-1544 (lattice search over the codebook
 //             with its neighbour index :228-331; one shared implementation driven by a traits table)
+//   ternary : iq1_s :1546-1798, iq1_m :1806-2098 (two-boundary search over the sorted sub-block, codebook snap)
 #include <algorithm>
 #include <cfloat>
 #include <cmath>
@@ -888,6 +889,36 @@ void enc_codebook16(const float* x, const float* im, uint8_t* b) {
 }
 
 // ------------------------------------------------------------------ iq1_s
+// Codebook entry for eight ternary levels (0, 1, 2): the entry itself when the group is on the codebook, else
+// the neighbour closest to x under the weights at the given scale and level values; `lv` takes the levels of
+// the entry picked (reference :1500-1544, iq1_find_best_neighbour2).
+int snap_ternary(const Codebook& cb, int8_t* lv, const float* x, const float* wt, float scale, const float* v,
+                 bool* exact) {
+  int packed = 0;
+  for (int i = 0; i < 8; i++) packed |= int(lv[i]) << (2 * i);
+  const int32_t slot = cb.slot[packed];
+  if (slot >= 0) return slot;
+  *exact = false;
+  const uint16_t* cand = cb.near.data() + (-slot - 1);
+  float least = FLT_MAX;
+  int pick = 0;
+  for (int c = 1; c <= int(cand[0]); c++) {
+    const int8_t* pt = cb.pts.data() + (size_t)cand[c] * 8;
+    float err = 0.f;
+    for (int i = 0; i < 8; i++) {
+      const float df = scale * v[(pt[i] - 1) / 2] - x[i];
+      err += wt[i] * df * df;
+    }
+    if (err < least) {
+      least = err;
+      pick = cand[c];
+    }
+  }
+  const int8_t* pt = cb.pts.data() + (size_t)pick * 8;
+  for (int i = 0; i < 8; i++) lv[i] = int8_t((pt[i] - 1) / 2);
+  return pick;
+}
+
 // 50 bytes: d | 32 entry low bytes | 8 x u16 (4 x 3 entry high bits, 3-bit scale, shift sign).  A 32-weight
 // sub-block is scale * (t + shift / 8) with t in {-1, 0, 1} drawn from the 2048-entry ternary codebook and one
 // shift sign per sub-block.  The ternary split comes from an exhaustive search over the two boundaries in the
@@ -949,30 +980,9 @@ void enc_iq1_s(const float* x, const float* im, uint8_t* b) {
     const float* v = shift > 0 ? vp : vm;
     bool all_exact = true;
     for (int k = 0; k < 4; k++) {
-      int packed = 0;
-      for (int i = 0; i < 8; i++) packed |= int(lv[8 * k + i]) << (2 * i);
-      int32_t slot = cb.slot[packed];
-      if (slot < 0) {
-        all_exact = false;
-        const uint16_t* cand = cb.near.data() + (-slot - 1);
-        float least = FLT_MAX;
-        int pick = -1;
-        for (int c = 1; c <= int(cand[0]); c++) {
-          const int8_t* pt = cb.pts.data() + (size_t)cand[c] * 8;
-          float err = 0.f;
-          for (int i = 0; i < 8; i++) {
-            const float df = scale * v[(pt[i] - 1) / 2] - xb[8 * k + i];
-            err += wt[8 * k + i] * df * df;
-          }
-          if (err < least) {
-            least = err;
-            pick = cand[c];
-          }
-        }
-        slot = pick < 0 ? 0 : pick;
-        const int8_t* pt = cb.pts.data() + (size_t)slot * 8;
-        for (int i = 0; i < 8; i++) lv[8 * k + i] = int8_t((pt[i] - 1) / 2);
-      }
+      bool exact = true;
+      const int slot = snap_ternary(cb, lv + 8 * k, xb + 8 * k, wt + 8 * k, scale, v, &exact);
+      all_exact = all_exact && exact;
       entries[ib][k] = slot;
     }
     if (!all_exact) {
@@ -1005,6 +1015,124 @@ void enc_iq1_s(const float* x, const float* im, uint8_t* b) {
   }
 }
 
+// ------------------------------------------------------------------ iq1_m
+// 56 bytes: 32 entry low bytes | 16 qh bytes (two 3-bit entry tops + two shift-sign bits) | 4 x u16 (four 3-bit
+// scales; the top nibbles spell the f16 block scale).  Sixteen 16-weight sub-blocks of two 8-value groups; the
+// ternary split is shared by the sub-block, the shift sign is per group, so the boundary search scores the four
+// sign pairs from per-group prefix sums (ggml quantize_row_iq1_m_impl; reference :1806-2098).  Without an
+// importance matrix the weights are x^2.
+void enc_iq1_m(const float* x, const float* im, uint8_t* b) {
+  const Codebook& cb = codebook(CB_IQ1);
+  constexpr float kDelta = 0.125f;
+  const float vp[3] = {-1.f + kDelta, kDelta, 1.f + kDelta}, vm[3] = {-1.f - kDelta, -kDelta, 1.f - kDelta};
+  // sign pair s: group 0 takes vm when s & 2, group 1 when s & 1
+  auto values = [&](int s, int g) { return ((g == 0 ? s >> 1 : s) & 1) ? vm : vp; };
+  float total = 0.f;
+  for (int i = 0; i < 256; i++) total += x[i] * x[i];
+  const float sigma2 = 2.0f * total / 256.0f;
+  float wt[256];
+  for (int i = 0; i < 256; i++) wt[i] = im ? im[i] * std::sqrt(sigma2 + x[i] * x[i]) : x[i] * x[i];
+  float scales[16], top = 0.f;
+  int pairs[16], entries[16][2];
+  for (int ib = 0; ib < 16; ib++) {
+    const float* xb = x + 16 * ib;
+    const float* wb = wt + 16 * ib;
+    scales[ib] = 0.f;
+    pairs[ib] = 0;
+    entries[ib][0] = entries[ib][1] = std::max(0, cb.slot[0x5555]);  // the all-middle group, when the codebook has it
+    float vmax = 0.f;
+    for (int i = 0; i < 16; i++) vmax = std::max(vmax, std::fabs(xb[i]));
+    if (vmax < 1e-7f) continue;
+    int order[16];
+    for (int i = 0; i < 16; i++) order[i] = i;
+    std::stable_sort(order, order + 16, [&](int l, int r) { return xb[l] < xb[r]; });
+    float sx[2][17], sw[2][17];
+    sx[0][0] = sx[1][0] = sw[0][0] = sw[1][0] = 0.f;
+    for (int j = 0; j < 16; j++) {
+      const int i = order[j], g = i / 8;
+      sx[g][j + 1] = sx[g][j] + wb[i] * xb[i];
+      sw[g][j + 1] = sw[g][j] + wb[i];
+      sx[g ^ 1][j + 1] = sx[g ^ 1][j];
+      sw[g ^ 1][j + 1] = sw[g ^ 1][j];
+    }
+    float best = -FLT_MAX, scale = vmax;
+    int b1 = -1, b2 = -1, pair = -1;
+    for (int i1 = 0; i1 <= 16; i1++)
+      for (int i2 = i1; i2 <= 16; i2++)
+        for (int s = 0; s < 4; s++) {
+          float sqx = 0.f, sq2 = 0.f;
+          for (int g = 0; g < 2; g++) {
+            const float* v = values(s, g);
+            const float x0 = sx[g][i1], x1 = sx[g][i2] - sx[g][i1], x2 = sx[g][16] - sx[g][i2];
+            const float w0 = sw[g][i1], w1 = sw[g][i2] - sw[g][i1], w2 = sw[g][16] - sw[g][i2];
+            sqx += x0 * v[0] + x1 * v[1] + x2 * v[2];
+            sq2 += w0 * v[0] * v[0] + w1 * v[1] * v[1] + w2 * v[2] * v[2];
+          }
+          if (sq2 > 0.f && sqx * sqx > best * sq2) {
+            scale = sqx / sq2;
+            best = scale * sqx;
+            b1 = i1;
+            b2 = i2;
+            pair = s;
+          }
+        }
+    if (pair < 0) continue;
+    int8_t lv[16];
+    for (int j = 0; j < 16; j++) lv[order[j]] = int8_t(j < b1 ? 0 : j < b2 ? 1 : 2);
+    if (scale < 0.f) {  // mirror: -(t + delta) = (-t) - delta
+      for (int j = 0; j < 16; j++) lv[j] = int8_t(2 - lv[j]);
+      scale = -scale;
+      pair = 3 - pair;
+    }
+    bool all_exact = true;
+    for (int g = 0; g < 2; g++)
+      entries[ib][g] = snap_ternary(cb, lv + 8 * g, xb + 8 * g, wb + 8 * g, scale, values(pair, g), &all_exact);
+    if (!all_exact) {
+      float sqx = 0.f, sq2 = 0.f;
+      for (int i = 0; i < 16; i++) {
+        const float q = values(pair, i / 8)[lv[i]];
+        sqx += wb[i] * q * xb[i];
+        sq2 += wb[i] * q * q;
+      }
+      if (sqx > 0.f && sq2 > 0.f) scale = sqx / sq2;
+    }
+    scales[ib] = scale;
+    pairs[ib] = pair;
+    top = std::max(top, scale);
+  }
+  std::memset(b, 0, 56);
+  if (!(top > 0.f)) return;
+  float d = top / 15.0f;
+  const float inv_d = 1.0f / d;
+  uint16_t sc[4] = {0, 0, 0, 0};
+  float sqx = 0.f, sq2 = 0.f;
+  for (int ib = 0; ib < 16; ib++) {
+    const int l = clampi(rne(0.5f * (inv_d * scales[ib] - 1.0f)), 0, 7);
+    sc[ib / 4] |= uint16_t(l << (3 * (ib % 4)));
+    uint8_t h = 0;
+    for (int g = 0; g < 2; g++) {
+      const int e = entries[ib][g];
+      b[2 * ib + g] = uint8_t(e & 255);
+      h |= uint8_t((e >> 8) << (4 * g));
+      if (values(pairs[ib], g) == vm) h |= uint8_t(0x08 << (4 * g));
+      const int8_t* pt = cb.pts.data() + (size_t)e * 8;
+      for (int i = 0; i < 8; i++) {
+        const int at = 16 * ib + 8 * g + i;
+        const float q = values(pairs[ib], g)[(pt[i] - 1) / 2] * float(2 * l + 1);
+        sqx += wt[at] * q * x[at];
+        sq2 += wt[at] * q * q;
+      }
+    }
+    b[32 + ib] = h;
+  }
+  if (sq2 > 0.f) d = sqx / sq2;  // least-squares block scale for the scale levels just fixed
+  const _Float16 hd = (_Float16)(d * 1.1125f);
+  uint16_t du;
+  std::memcpy(&du, &hd, 2);
+  for (int k = 0; k < 4; k++) sc[k] |= uint16_t(((du >> (4 * k)) & 15) << 12);
+  std::memcpy(b + 48, sc, 8);
+}
+
 typedef void (*BlockEnc)(const float*, const float*, uint8_t*);
 void legacy_q8_0(const float* x, const float*, uint8_t* b) { enc_q8_0(x, b); }
 void legacy_q4_0(const float* x, const float*, uint8_t* b) { enc_legacy<false, 4>(x, b); }
@@ -1030,6 +1158,7 @@ BlockEnc encoder_for(int codec) {
     case KQ_IQ2_XS: return enc_codebook16<KQ_IQ2_XS>;
     case KQ_IQ2_S: return enc_codebook16<KQ_IQ2_S>;
     case KQ_IQ1_S: return enc_iq1_s;
+    case KQ_IQ1_M: return enc_iq1_m;
     case KQ_IQ3_XXS: return enc_codebook<KQ_IQ3_XXS>;
     case KQ_IQ3_S: return enc_codebook<KQ_IQ3_S>;
   }

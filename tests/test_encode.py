@@ -144,7 +144,7 @@ def test_iq4_known_answer_blocks():
 
 # ------------------------------------------------------------------ codebook codecs (iq2_xxs, iq3_xxs, iq3_s)
 CB_BOUND = {"iq2_xxs": 0.45, "iq2_xs": 0.45, "iq2_s": 0.45, "iq3_xxs": 0.30, "iq3_s": 0.30,
-            "iq1_s": 0.65}  # reference tests/test_iq_encode.py:36-43
+            "iq1_s": 0.65, "iq1_m": 0.65}  # reference tests/test_iq_encode.py:36-43
 
 
 @pytest.mark.parametrize("codec", list(CB_BOUND))
@@ -272,4 +272,34 @@ def test_iq1_s_known_answer_blocks():
     assert np.mean((qh & 0x0FFF) == (mq & 0x0FFF)) > 0.95          # 4 x 3 entry high bits
     assert np.mean((qh & 0x8000) == (mq & 0x8000)) > 0.97          # shift signs
     back = O.dequantize(mine, "iq1_s").reshape(nsb, 256)
+    assert np.linalg.norm(back - x) / np.linalg.norm(x) < 0.15
+
+
+def test_iq1_m_known_answer_blocks():
+    """As above for the 16-weight sub-blocks of iq1_m: entries, the two shift-sign bits per sub-block (qh bits 3 and
+    7) and the 3-bit scales come back, and the f16 block scale scattered over the four top nibbles decodes to
+    within the encoder's 1.1125 fudge of the original."""
+    nsb = 24
+    rng = np.random.default_rng(12)
+    wire = O.synth_wire("iq1_m", nsb, 13).reshape(nsb, 56).copy()
+    sc = wire[:, 48:56].copy().view(np.uint16)
+    lv = rng.integers(2, 8, (nsb, 16))
+    lv[:, 0] = 7
+    du = int(np.frombuffer(np.float16(2.0 ** -5).tobytes(), dtype=np.uint16)[0])
+    for k in range(4):
+        word = np.zeros(nsb, np.uint16)
+        for j in range(4):
+            word |= (lv[:, 4 * k + j] << (3 * j)).astype(np.uint16)
+        sc[:, k] = word | np.uint16(((du >> (4 * k)) & 15) << 12)
+    wire[:, 48:56] = sc.view(np.uint8)
+    x = O.dequantize(wire, "iq1_m").reshape(nsb, 256)
+    mine = _enc(x, "iq1_m", np.ones(256, np.float32))
+    assert np.mean(wire[:, 0:32] == mine[:, 0:32]) > 0.98                      # entry low bytes
+    assert np.mean((wire[:, 32:48] & 0x77) == (mine[:, 32:48] & 0x77)) > 0.98  # entry high bits
+    assert np.mean((wire[:, 32:48] & 0x88) == (mine[:, 32:48] & 0x88)) > 0.98  # shift signs
+    assert np.mean((mine[:, 48:56].copy().view(np.uint16) & 0xFFF) == (sc & 0xFFF)) > 0.98  # 3-bit scales
+    back = O.dequantize(mine, "iq1_m").reshape(nsb, 256)
+    assert np.linalg.norm(back - x) / np.linalg.norm(x) < 0.15
+    # without an importance matrix the x^2 weighting still lands on the same structure
+    back = O.dequantize(_enc(x, "iq1_m"), "iq1_m").reshape(nsb, 256)
     assert np.linalg.norm(back - x) / np.linalg.norm(x) < 0.15
