@@ -136,6 +136,30 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
                   void* out_dev, int T, int R, int E, int N, int K, int codec, int dtype, void* workspace_dev,
                   size_t workspace_bytes, void* stream);
 
+/* Tile map of expert-sorted routing indices, built on the device without a host sync: map uint32 [cap][3] rows
+ * of (expert, first row, rows <= 64) cutting every expert's run of rows into 64-row tiles of which only the last
+ * may be partial, in row order; counts[0] = number of valid tiles (slots past it are left untouched).
+ * cap = kq_expert_tile_map_cap(rows, n_experts) = max(rows / 64 + min(n_experts, rows), 1) bounds the tile
+ * count.  Rows whose index is >= n_experts belong to no tile.
+ * Replaces expert_tile_map (KQuantExpertTileMap), reference src/kquant.h:102-109, src/kquant_ops.cpp:422-447,
+ * src/kquant_gather.cpp:1010-1042; host-built equivalent mlx_kquant/nn.py:33-47. */
+int64_t kq_expert_tile_map_cap(int64_t rows, int n_experts);
+int kq_expert_tile_map(const uint32_t* indices_dev, int64_t rows, int n_experts, uint32_t* map_dev, int64_t cap,
+                       uint32_t* counts_dev, void* stream);
+
+/* Sorted-segment GEMM for MoE prefill: for every valid tile (expert e, first row r, n rows) of the map,
+ * out[r : r + n] = T(x[r : r + n] . W_e^T).  x [rows, K] sorted by expert, w [E, N, bytes_per_row] dense,
+ * map uint32 [n_tiles][3] and counts uint32 [1] as kq_expert_tile_map writes them (or host-built; tiles of at
+ * most 64 rows that never span experts and cover every row once).  Rows no valid tile covers hold unspecified
+ * values afterwards.  The tiles are turned into a per-row expert list on the device and the rows run through
+ * the expert-grouped kernels of kq_gather_qmv, so the workspace is kq_gather_qmm_seg_workspace_size bytes.
+ * Replaces gather_qmm_seg (KQuantGatherQMMSeg), reference src/kquant.h:111-128, src/kquant_ops.cpp:466-548,
+ * src/kquant_gather.cpp:1044-1092. */
+size_t kq_gather_qmm_seg_workspace_size(int64_t rows, int E, int N, int K, int codec, int dtype);
+int kq_gather_qmm_seg(const void* x_dev, const void* w_dev, const uint32_t* map_dev, const uint32_t* counts_dev,
+                      void* out_dev, int64_t rows, int64_t n_tiles, int E, int N, int K, int codec, int dtype,
+                      void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* out[t, r < R] as kq_moe_glu_gather (act silu or gelu, no biases); out[t, R] = the same GLU of x[t] against
  * the block's shared expert, two single [N, bytes_per_row] matrices in `shexp_codec` (the expert codec, or
  * q6_k / q8_0).  out [T, R + 1, N].  The workspace (kq_moe_glu_gather_shexp_workspace_size bytes, 256-byte

@@ -377,6 +377,72 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
                                   static_cast<hipStream_t>(stream));
 }
 
+
+// ------------------------------------------------------------------ sorted-segment prefill GEMM
+int64_t kq_expert_tile_map_cap(int64_t rows, int n_experts) {
+  if (rows < 1 || n_experts < 1) return 1;
+  const int64_t c = rows / 64 + (rows < n_experts ? rows : (int64_t)n_experts);
+  return c > 1 ? c : 1;
+}
+
+int kq_expert_tile_map(const uint32_t* indices_dev, int64_t rows, int n_experts, uint32_t* map_dev, int64_t cap,
+                       uint32_t* counts_dev, void* stream) {
+  const char* op = "expert_tile_map";
+  if (rows < 1 || n_experts < 1)
+    return kq_set_error(KQ_ERR_INVALID, "%s: indices must be non-empty and n_experts positive", op);
+  if (rows > 0x7fffffff) return kq_set_error(KQ_ERR_INVALID, "%s: too many rows", op);
+  if (cap < kq_expert_tile_map_cap(rows, n_experts))
+    return kq_set_error(KQ_ERR_INVALID, "%s: map holds %lld tiles, %lld may be needed", op, (long long)cap,
+                        (long long)kq_expert_tile_map_cap(rows, n_experts));
+  if (!indices_dev || !map_dev || !counts_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  return kq_launch_expert_tile_map(indices_dev, (int)rows, n_experts, map_dev, (int)(cap > 0x7fffffff ? 0x7fffffff : cap),
+                                   counts_dev, static_cast<hipStream_t>(stream));
+}
+
+size_t kq_gather_qmm_seg_workspace_size(int64_t rows, int E, int N, int K, int codec, int dtype) {
+  if (rows <= 0 || rows > 0x7fffffff) return 0;
+  return align256((size_t)rows * 4) + kq_moe_workspace_size((int)rows, 1, E, N, K, 0, codec, dtype);
+}
+
+int kq_gather_qmm_seg(const void* x_dev, const void* w_dev, const uint32_t* map_dev, const uint32_t* counts_dev,
+                      void* out_dev, int64_t rows, int64_t n_tiles, int E, int N, int K, int codec, int dtype,
+                      void* workspace_dev, size_t workspace_bytes, void* stream) {
+  const char* op = "gather_qmm_seg";
+  if (rows < 0 || rows > 0x7fffffff || n_tiles > 0x7fffffff) return kq_set_error(KQ_ERR_INVALID, "%s: bad dimension", op);
+  int rc = check_moe(op, (int)rows, 1, E, N, K, codec, dtype);
+  if (rc) return rc;
+  if (n_tiles < 1) return kq_set_error(KQ_ERR_INVALID, "%s: map must hold at least one tile row", op);
+  if (rows == 0 || N == 0) return KQ_OK;
+  if (!x_dev || !w_dev || !map_dev || !counts_dev || !out_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  const size_t need = kq_gather_qmm_seg_workspace_size(rows, E, N, K, codec, dtype);
+  if (!workspace_dev || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace_dev) & 255))
+    return kq_set_error(KQ_ERR_WORKSPACE, "%s: a 256-byte aligned workspace of %zu bytes is required (got %zu)", op, need,
+                        workspace_dev ? workspace_bytes : 0);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint8_t* wsb = static_cast<uint8_t*>(workspace_dev);
+  uint32_t* row_expert = reinterpret_cast<uint32_t*>(wsb);
+  const size_t used = align256((size_t)rows * 4);
+  // the grouped kernels leave out rows whose expert id is out of range; the per-row kernels know no such
+  // marker, so there an uncovered row is computed against expert 0
+  const bool grouped = kq_moe_workspace_size((int)rows, 1, E, N, K, 0, codec, dtype) > 0;
+  rc = kq_launch_tiles_to_rows(map_dev, counts_dev, (int)n_tiles, (int)rows, E, grouped ? 0xffffffffu : 0u, row_expert, s);
+  if (rc) return rc;
+  const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
+  if (grouped) {
+    const int rcg = try_moe_grouped(op, x_dev, w_dev, nullptr, row_expert, nullptr, nullptr, out_dev, (int)rows, 1, E, N, K,
+                                    estride, 0, 0, 0.f, 0.f, codec, dtype, wsb + used, workspace_bytes - used, s);
+    if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
+    // an unaligned x: rerun the row list with the marker the per-row kernels can take
+    rc = kq_launch_tiles_to_rows(map_dev, counts_dev, (int)n_tiles, (int)rows, E, 0u, row_expert, s);
+    if (rc) return rc;
+  }
+  const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, row_expert, out_dev,
+                                         (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype, s);
+  if (rct != KQ_ERR_UNSUPPORTED) return rct;
+  return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, row_expert, nullptr,
+                                  nullptr, out_dev, (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype, s);
+}
+
 }  // extern "C"
 
 // ------------------------------------------------------------------ shared-expert / slot-mixing MoE ops

@@ -121,6 +121,90 @@ __global__ __launch_bounds__(256) void mix_slots_kernel(const float* __restrict_
   out[i] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
 }
 
+// ------------------------------------------------------------------ expert tile map (sorted prefill GEMM)
+// From expert-sorted routing indices, the (expert, first row, rows <= 64) tiles of every expert's run of rows;
+// only the last tile of a run is partial.  One workgroup: each thread walks a contiguous chunk of rows (one
+// binary search for the run its chunk starts in), a block scan numbers the tiles in row order, a second walk
+// writes them.  Rows whose expert id is out of range belong to no tile.
+constexpr int TILE_ROWS = 64;
+
+__device__ __forceinline__ int first_row_of(const uint32_t* idx, int rows, uint32_t e) {  // lower bound
+  int lo = 0, hi = rows;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (idx[mid] < e) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ int end_row_of(const uint32_t* idx, int rows, uint32_t e) {  // upper bound
+  int lo = 0, hi = rows;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (idx[mid] <= e) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+__global__ __launch_bounds__(SORT_THREADS) void expert_tile_map_kernel(const uint32_t* __restrict__ idx, int rows, int E,
+                                                                      uint32_t* __restrict__ map, int cap,
+                                                                      uint32_t* __restrict__ counts) {
+  __shared__ int scan[SORT_THREADS];
+  const int tid = threadIdx.x;
+  const int ch = (rows + SORT_THREADS - 1) / SORT_THREADS;
+  const int r0 = min(tid * ch, rows), r1 = min(r0 + ch, rows);
+  int slot = 0;
+  for (int pass = 0; pass < 2; pass++) {
+    int n = 0, run_start = 0;
+    uint32_t run_e = 0xffffffffu;
+    for (int r = r0; r < r1; r++) {
+      const uint32_t e = idx[r];
+      if (r == r0 || e != run_e) {
+        run_e = e;
+        run_start = (r > r0) ? r : first_row_of(idx, rows, e);
+      }
+      if (e >= (uint32_t)E || (r - run_start) % TILE_ROWS) continue;
+      if (pass == 1 && slot + n < cap) {
+        const int left = end_row_of(idx, rows, e) - r;
+        uint32_t* t = map + 3 * (size_t)(slot + n);
+        t[0] = e;
+        t[1] = (uint32_t)r;
+        t[2] = (uint32_t)(left < TILE_ROWS ? left : TILE_ROWS);
+      }
+      n++;
+    }
+    if (pass == 1) break;
+    scan[tid] = n;
+    __syncthreads();
+    for (int off = 1; off < SORT_THREADS; off <<= 1) {
+      const int v = tid >= off ? scan[tid - off] : 0;
+      __syncthreads();
+      scan[tid] += v;
+      __syncthreads();
+    }
+    slot = scan[tid] - n;
+    if (tid == SORT_THREADS - 1) counts[0] = (uint32_t)(scan[tid] < cap ? scan[tid] : cap);
+  }
+}
+
+// row_expert[r] = `none` everywhere, then the expert of the tile that covers row r
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* __restrict__ p, int n, uint32_t v) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+__global__ __launch_bounds__(TILE_ROWS) void tiles_to_rows_kernel(const uint32_t* __restrict__ map,
+                                                                  const uint32_t* __restrict__ counts, int cap, int rows,
+                                                                  int E, uint32_t* __restrict__ row_expert) {
+  const int t = blockIdx.x;
+  const uint32_t nt = counts[0];
+  if ((uint32_t)t >= nt) return;
+  const uint32_t e = map[3 * t], start = map[3 * t + 1], n = map[3 * t + 2];
+  const uint32_t j = threadIdx.x;
+  if (e >= (uint32_t)E || j >= n || start >= (uint32_t)rows || j >= (uint32_t)rows - start) return;
+  row_expert[start + j] = e;
+}
+
 // ------------------------------------------------------------------ grouped GEMM
 struct MoeArgs {
   const _Float16* xh;   // [rows][K] f16 activations (prepass), row = pair / x_div
@@ -384,6 +468,25 @@ int kq_launch_gather_rows(const void* x, const uint32_t* lhs, const uint32_t* rh
   if (B <= 0 || M <= 0) return KQ_OK;
   hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)B * (unsigned)M), dim3(256), 0, s, static_cast<const uint16_t*>(x),
                      lhs, rhs, static_cast<uint16_t*>(xg), idx_rows, M, K, x_batch_stride);
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
+int kq_launch_expert_tile_map(const uint32_t* idx, int rows, int E, uint32_t* map, int cap, uint32_t* counts,
+                              hipStream_t s) {
+  hipLaunchKernelGGL(expert_tile_map_kernel, dim3(1), dim3(SORT_THREADS), 0, s, idx, rows, E, map, cap, counts);
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
+// row_expert[r] = expert of the tile covering row r, `none` for rows no valid tile covers
+int kq_launch_tiles_to_rows(const uint32_t* map, const uint32_t* counts, int cap, int rows, int E, uint32_t none,
+                            uint32_t* row_expert, hipStream_t s) {
+  if (rows <= 0 || cap <= 0) return KQ_OK;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, row_expert, rows, none);
+  KQ_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL(tiles_to_rows_kernel, dim3((unsigned)cap), dim3(TILE_ROWS), 0, s, map, counts, cap, rows, E,
+                     row_expert);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }

@@ -24,7 +24,7 @@ _GEOM = {k: (v[3], v[2]) for k, v in CODEC_GEOMETRY.items()}
 
 __all__ = [
     "codecs", "codec_has_matmul", "codec_has_moe_glu", "dequantize", "quantized_matmul", "quantized_matmul_qmv_bias",
-    "gather_qmm",
+    "gather_qmm", "expert_tile_map", "gather_qmm_seg",
     "moe_glu_gather_kq", "gather_qmv_kq", "moe_glu_gather_shexp_kq", "gather_qmv_mix_kq", "gather_qmv_mix_ns_kq",
     "moe_router_topk", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
     "weights_per_row", "lib_path",
@@ -84,6 +84,12 @@ def _load():
     lib.kq_moe_glu_gather.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, f, f, i, i, vp, sz, vp]
     lib.kq_gather_qmv.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, sz, vp]
     lib.kq_quantize.argtypes = [vp, vp, vp, i64, i64, i]
+    lib.kq_expert_tile_map_cap.restype = i64
+    lib.kq_expert_tile_map_cap.argtypes = [i64, i]
+    lib.kq_expert_tile_map.argtypes = [vp, i64, i, vp, i64, vp, vp]
+    lib.kq_gather_qmm_seg_workspace_size.restype = sz
+    lib.kq_gather_qmm_seg_workspace_size.argtypes = [i64, i, i, i, i, i]
+    lib.kq_gather_qmm_seg.argtypes = [vp, vp, vp, vp, vp, i64, i64, i, i, i, i, i, vp, sz, vp]
     _lib = lib
     return lib
 
@@ -306,6 +312,79 @@ def gather_qmm(x, w, scales, kquant_type, lhs_indices=None, rhs_indices=None, tr
         _check(lib.kq_gather_qmm(x_c.data_ptr(), w3.data_ptr(), lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), B, M, E,
                                  N, K, M * K, estride, int(bool(transpose)), int(right_sorted), cid, _DT[out_type],
                                  ws.data_ptr() if ws is not None else None, ws_bytes, sp))
+    return out
+
+
+def expert_tile_map(indices, n_experts, *, stream=None):
+    """Tile map of expert-sorted routing indices, built on the device: (map int32 [cap, 3] rows of
+    (expert, first row, rows <= 64), counts int32 [1] = number of valid tiles); cap = rows // 64 +
+    min(n_experts, rows) is a shape-only bound and slots past counts are uninitialised.
+    Mirrors expert_tile_map, src/kquant_ops.cpp:422-447 (uint32 there; torch has int32)."""
+    op = "expert_tile_map"
+    if indices.ndim != 1 or indices.dtype not in (torch.int32, torch.int64, torch.uint32):
+        raise ValueError(f"[kq.expert_tile_map] indices must be 1-D integer but got shape {tuple(indices.shape)} "
+                         f"dtype {indices.dtype}.")
+    rows = indices.shape[0]
+    if rows < 1 or n_experts < 1:
+        raise ValueError("[kq.expert_tile_map] indices must be non-empty and n_experts positive.")
+    if not indices.is_cuda:
+        raise RuntimeError("[kq.expert_tile_map] the indices must live on the GPU (there is no CPU implementation).")
+    sp = _stream_ptr(op, indices, stream)
+    idx = _prep_idx(indices)
+    lib = _load()
+    cap = lib.kq_expert_tile_map_cap(rows, n_experts)
+    tiles = torch.empty((cap, 3), dtype=torch.int32, device=indices.device)
+    counts = torch.empty((1,), dtype=torch.int32, device=indices.device)
+    with torch.cuda.device(indices.device):
+        _check(lib.kq_expert_tile_map(idx.data_ptr(), rows, n_experts, tiles.data_ptr(), cap, counts.data_ptr(), sp))
+    return tiles, counts
+
+
+def gather_qmm_seg(x, w, scales, kquant_type, map, counts, *, stream=None):
+    """Sorted-segment GEMM for MoE prefill: x [rows, K] sorted by expert, w [E, N, bytes_per_row]; for every valid
+    tile (expert e, first row r, n <= 64 rows) of `map` ([n_tiles, 3]; counts [1] = valid tiles) the rows
+    out[r : r + n] = x[r : r + n] @ W_e.T.  Rows no tile covers are unspecified.
+    Mirrors gather_qmm_seg, src/kquant_ops.cpp:466-548."""
+    op = "gather_qmm_seg"
+    if w.dtype != torch.uint8:
+        raise ValueError("[kq.gather_qmm_seg] w must be uint8 (raw GGUF wire bytes).")
+    cid, (wpb, bpb) = _codec(op, kquant_type)
+    if x.ndim != 2:
+        raise ValueError(f"[kq.gather_qmm_seg] x must be [rows, K] but got shape {tuple(x.shape)}.")
+    if w.ndim != 3:
+        raise ValueError(f"[kq.gather_qmm_seg] w must be (n_experts, N, bytes_per_row) but got shape {tuple(w.shape)}.")
+    ints = (torch.int32, torch.uint32)
+    if map.ndim != 2 or map.shape[1] != 3 or map.dtype not in ints or map.shape[0] < 1:
+        raise ValueError("[kq.gather_qmm_seg] map must be 32-bit integer [n_tiles >= 1, 3] (expert, row_start, num_rows) "
+                         f"but got shape {tuple(map.shape)} dtype {map.dtype}.")
+    if counts.ndim != 1 or counts.shape[0] != 1 or counts.dtype not in ints:
+        raise ValueError(f"[kq.gather_qmm_seg] counts must be 32-bit integer [1] but got shape {tuple(counts.shape)} "
+                         f"dtype {counts.dtype}.")
+    if w.shape[-1] % bpb != 0:
+        raise ValueError(f"[kq.gather_qmm_seg] KQuant weight last dim ({w.shape[-1]} bytes) is not a whole number of "
+                         f"{bpb}-byte {kquant_type} blocks.")
+    K = w.shape[-1] // bpb * wpb
+    if K != x.shape[-1]:
+        raise ValueError(f"[kq.gather_qmm_seg] x last dim ({x.shape[-1]}) does not match the expanded quantized row "
+                         f"width ({K}) for codec '{kquant_type}'.")
+    if not x.dtype.is_floating_point:
+        raise ValueError("[kq.gather_qmm_seg] Only real floating x dtypes are supported.")
+    if w.shape[1] % 8 != 0:
+        raise ValueError("[kq.gather_qmm_seg] N must be a multiple of 8.")
+    _same_device(op, x, w, map, counts)
+    sp = _stream_ptr(op, x, stream)
+    x_c = (x.to(torch.bfloat16) if x.dtype not in (torch.float16, torch.bfloat16) else x).contiguous()
+    w_c, map_c, cnt_c = w.contiguous(), map.contiguous(), counts.contiguous()
+    rows, (E, N) = x.shape[0], w.shape[:2]
+    out = torch.empty((rows, N), dtype=x_c.dtype, device=x.device)
+    if rows == 0 or N == 0:
+        return out
+    lib = _load()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.kq_gather_qmm_seg_workspace_size(rows, E, N, K, cid, _DT[x_c.dtype])
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=x.device)
+        _check(lib.kq_gather_qmm_seg(x_c.data_ptr(), w_c.data_ptr(), map_c.data_ptr(), cnt_c.data_ptr(), out.data_ptr(),
+                                     rows, map_c.shape[0], E, N, K, cid, _DT[x_c.dtype], ws.data_ptr(), ws_bytes, sp))
     return out
 
 

@@ -6,13 +6,18 @@ the reference's mlx_kquant/nn.py (KQuantEmbedding :50-101, KQuantLinear :104-160
 (`bias[indices]` expanded on axis -2 for expert stacks), an embedding gathers wire rows and decodes only
 those.
 
-What differs from the reference, on purpose: kq.gather_qmm groups its entries by expert on the device
-whenever there are more than 16 output rows, so KQuantSwitchLinear has no separate host-side
-"one GEMM per sorted expert segment" arm (reference :191-261) and never synchronises on the routing
-indices; `sorted_indices` is passed through.
+KQuantSwitchLinear keeps the reference's sorted prefill arm (:191-261): a prefill-shaped sorted call
+(x [B, 1, K], ascending 1-D indices, at least KQ_SWITCH_GEMM_MIN_ROWS rows, 512 by default, 0 disables)
+builds the tile map on the device (kq.expert_tile_map) and runs kq.gather_qmm_seg, with no host sync on the
+routing indices.  Every other call goes to kq.gather_qmm, which itself groups its entries by expert on the
+device whenever there are more than 16 output rows, so here the two arms differ in bookkeeping, not in the
+GEMM kernels behind them.
 """
 from __future__ import annotations
 
+import os
+
+import numpy as np
 import torch
 
 import kq
@@ -20,6 +25,24 @@ import kq
 from .codec_geometry import CODEC_GEOMETRY, bytes_per_row
 
 __all__ = ["KQuantEmbedding", "KQuantLinear", "KQuantSwitchLinear", "KQuantMultiLinear"]
+
+
+# kq.gather_qmm_seg tile height
+_SEG_TILE_ROWS = 64
+
+
+def _host_tile_maps(counts, device=None):
+    """Host-built equivalent of kq.expert_tile_map from per-expert row counts: (map int32 [n_tiles, 3] rows of
+    (expert, first row, rows <= 64), counts int32 [1]); only the last tile of an expert's run is partial
+    (reference :33-47)."""
+    counts = np.asarray(counts, dtype=np.int64)
+    tiles, row = [], 0
+    for e in np.flatnonzero(counts):
+        c = int(counts[e])
+        tiles += [(int(e), row + off, min(_SEG_TILE_ROWS, c - off)) for off in range(0, c, _SEG_TILE_ROWS)]
+        row += c
+    m = torch.tensor(tiles or [(0, 0, 0)], dtype=torch.int32, device=device)
+    return m, torch.tensor([len(tiles)], dtype=torch.int32, device=device)
 
 
 class _KQuantBase(torch.nn.Module):
@@ -119,11 +142,23 @@ class KQuantSwitchLinear(_KQuantBase):
             self.bias = None
 
     def forward(self, x, indices, sorted_indices=False):
+        if sorted_indices and indices.ndim == 1 and x.ndim == 3 and x.shape[0] == indices.numel() and x.shape[1] == 1:
+            min_rows = int(os.environ.get("KQ_SWITCH_GEMM_MIN_ROWS", "512"))  # read live, as the reference does
+            if min_rows > 0 and indices.numel() >= min_rows and self.weight.shape[1] % 8 == 0:
+                y = self._sorted_expert_gemm(x, indices)
+                if self.bias is not None:
+                    y = y + self.bias[indices.to(torch.int64)].unsqueeze(-2)
+                return y
         y = kq.gather_qmm(x, self.weight, self.scales, self.kquant_type, rhs_indices=indices, transpose=True,
                           sorted_indices=sorted_indices)
         if self.bias is not None:
             y = y + self.bias[indices.to(torch.int64)].unsqueeze(-2)
         return y
+
+    def _sorted_expert_gemm(self, x, indices):
+        xf = x.reshape(indices.numel(), -1)
+        maps = kq.expert_tile_map(indices, self.weight.shape[0])
+        return kq.gather_qmm_seg(xf, self.weight, self.scales, self.kquant_type, *maps)[:, None, :]
 
     def extra_repr(self):
         n, m, b = self.weight.shape

@@ -38,3 +38,43 @@ def test_validation():
         lin.load_wire(torch.zeros((96, 288), dtype=torch.uint8), bias=torch.zeros(96))
     lin.load_wire(torch.ones((96, 288), dtype=torch.uint8))
     assert int(lin.state_dict()["weight"].sum()) == 96 * 288
+
+
+def test_host_tile_maps():
+    """64-row tiles per expert run, only the last partial, absent experts skipped (reference nn.py:33-47)."""
+    m, cnt = knn._host_tile_maps([65, 0, 3, 128])
+    assert m.dtype == torch.int32 and cnt.tolist() == [5]
+    assert m.tolist() == [[0, 0, 64], [0, 64, 1], [2, 65, 3], [3, 68, 64], [3, 132, 64]]
+    m, cnt = knn._host_tile_maps([0, 0])
+    assert m.tolist() == [[0, 0, 0]] and cnt.tolist() == [0]
+
+
+def test_gather_qmm_seg_rejects_bad_inputs():
+    """Argument checks run before anything touches a device (reference tests/test_switch_gemm.py:293-319)."""
+    import kq
+
+    K, N = 512, 128
+    x = torch.zeros((64, K), dtype=torch.float16)
+    w = torch.zeros((2, N, 1056), dtype=torch.uint8)  # iq2_xxs bytes per row for K = 4096
+    s = torch.zeros((1,), dtype=torch.uint8)
+    good = torch.zeros((1, 3), dtype=torch.int32)
+    cnt = torch.zeros((1,), dtype=torch.int32)
+    with pytest.raises(ValueError):  # K mismatch
+        kq.gather_qmm_seg(x, w, s, "iq2_xxs", good, cnt)
+    x_ok = torch.zeros((64, 4096), dtype=torch.float16)
+    with pytest.raises(ValueError):  # bad map shape
+        kq.gather_qmm_seg(x_ok, w, s, "iq2_xxs", torch.zeros((3,), dtype=torch.int32), cnt)
+    with pytest.raises(ValueError):  # bad counts shape
+        kq.gather_qmm_seg(x_ok, w, s, "iq2_xxs", good, torch.zeros((2,), dtype=torch.int32))
+    with pytest.raises(ValueError):  # 3-D x
+        kq.gather_qmm_seg(torch.zeros((64, 1, 4096), dtype=torch.float16), w, s, "iq2_xxs", good, cnt)
+    with pytest.raises(ValueError):  # float wire
+        kq.gather_qmm_seg(x_ok, w.to(torch.float16), s, "iq2_xxs", good, cnt)
+    with pytest.raises(ValueError):  # unknown codec
+        kq.gather_qmm_seg(x_ok, w, s, "q9_k", good, cnt)
+    with pytest.raises(ValueError):  # expert_tile_map: float indices
+        kq.expert_tile_map(torch.zeros((8,), dtype=torch.float32), 4)
+    with pytest.raises(ValueError):  # expert_tile_map: empty
+        kq.expert_tile_map(torch.zeros((0,), dtype=torch.int32), 4)
+    with pytest.raises(RuntimeError):  # valid arguments, but no device: there is no CPU path
+        kq.gather_qmm_seg(x_ok, w, s, "iq2_xxs", good, cnt)
