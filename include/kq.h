@@ -87,8 +87,10 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
 int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int N, int K, int codec,
                 int dtype, void* stream);
 
-/* Tuning hook without a counterpart in the reference: activation rows per workgroup tile of the
- * prefill GEMM, 64 or 128 (anything else restores the default, 64).  Process-wide, not thread-safe. */
+/* Tuning hook without a counterpart in the reference: workgroup tile of the prefill GEMM.  64 = 64
+ * activation rows x 128 weight rows, 128 = 128 x 128, 256 = 64 x 256 on eight waves with two LDS stages
+ * (q4_k only; other codecs fall back to automatic); anything else restores the automatic choice.
+ * Process-wide, not thread-safe. */
 void kq_set_gemm_tile_rows(int rows);
 /* Tuning hook without a counterpart in the reference: which skinny-M kernel dense calls use.
  * 0 = default (decoupled-wave kernel up to 4 activation rows, diagonal kernel for 5 - 8),

@@ -5,15 +5,15 @@
 // inputs neither overflow nor lose bits) that also emits the sub-block sums of x as two f16 halves
 // for the q4_k / q5_k minimum term.
 //
-// Tiling.  Workgroup = 4 waves, tile 128 (M) x 128 (N), one 256-wide superblock of K per step; each
-// wave owns all 128 rows x 32 columns (4 accumulator tiles of v_mfma_f32_32x32x16_f16), so every
-// weight is decoded by exactly one wave of the workgroup.  Wire bytes and activations are fetched
+// Tiling.  Workgroup = 4 or 8 waves, tile 64 or 128 (M) x 32 per wave (N), one 256-wide superblock of K per
+// step; each wave owns all the tile's rows x 32 columns (2 or 4 accumulator tiles of
+// v_mfma_f32_32x32x16_f16), so every weight is decoded by exactly one wave of the workgroup.  Wire bytes and activations are fetched
 // with coalesced 16-byte loads into registers one step ahead and parked in LDS (activation rows
 // padded by 16 bytes, wire rows an odd number of 16-byte pieces apart, which keeps the
 // row-per-lane ds_read_b128 fragment fetch free of bank conflicts).
 #include "kq_mma.h"
 
-static int g_gemm_force_mt = 0;  // kq_set_gemm_tile_rows: 2 or 4 forces the tile height, 0 = default
+static int g_gemm_tile = 0;  // kq_set_gemm_tile_rows: 64, 128 or 256 forces the tile shape, 0 = automatic
 
 namespace {
 
@@ -98,36 +98,40 @@ __global__ __launch_bounds__(PP_THREADS) void gemm_prepass_kernel(const uint16_t
 }
 
 // ------------------------------------------------------------------ main kernel
-constexpr int GM_THREADS = 256;
-constexpr int BM = 128, BN = 128;
+constexpr int BM = 128;
 constexpr int A_STRIDE = 512 + 16;  // bytes per activation row of one K step in LDS
 
-template <int C>
+template <int C, int WAVES>
 struct WireGeom : Wire<C> {
-  static constexpr int PPR = Wire<C>::PP;                               // 16-byte pieces per row and step
-  static constexpr int WPT = (BN * PPR + GM_THREADS - 1) / GM_THREADS;  // pieces per thread per step
+  static constexpr int THREADS = 64 * WAVES, BN = 32 * WAVES;
+  static constexpr int PPR = Wire<C>::PP;                          // 16-byte pieces per row and step
+  static constexpr int WPT = (BN * PPR + THREADS - 1) / THREADS;   // pieces per thread per step
 };
 
 // MT = 32-row activation blocks per workgroup tile (tile = 32 MT rows x 128 columns).  MT = 4 runs one
 // workgroup per CU (one wave per SIMD) and is bound by LDS / MFMA latency it cannot hide; MT = 2 fits
 // two workgroups per CU and measured 17 - 38 % faster although each decoded fragment feeds only two
 // MFMAs (MT = 3 needs 256 registers and spills).
-template <int C, int DT, int MT>
-__global__ __launch_bounds__(GM_THREADS, MT == 4 ? 1 : 2) void kquant_gemm_kernel(const _Float16* __restrict__ xh,
+template <int C, int DT, int MT, int WAVES, bool DB>
+__global__ __launch_bounds__(64 * WAVES, (MT == 4 || WAVES == 8) ? 1 : 2) void kquant_gemm_kernel(const _Float16* __restrict__ xh,
                                                                     const _Float16* __restrict__ xhl,
                                                                     const float* __restrict__ rs,
                                                                     const uint8_t* __restrict__ w,
                                                                     uint16_t* __restrict__ y, int M, int N, int K,
                                                                     int mtiles) {
-  using G = WireGeom<C>;
+  using G = WireGeom<C, WAVES>;
+  constexpr int GM_THREADS = G::THREADS, BN = G::BN;
   constexpr int TM = 32 * MT;                   // activation rows per tile
   constexpr int A_BYTES = TM * A_STRIDE;
   constexpr int APT = TM * 32 / GM_THREADS;     // 16-byte activation pieces per thread per step
+  constexpr int AROWS = GM_THREADS / 32;        // activation rows one pass of the workgroup covers
+  static_assert(TM * 32 % GM_THREADS == 0 && 2 * TM <= GM_THREADS && BN <= GM_THREADS, "tile / thread count mismatch");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint8_t* a_lds = smem;                          // [TM][A_STRIDE]
-  uint8_t* b_lds = smem + A_BYTES;                // [BN][LBPB]
-  uint8_t* h_lds = b_lds + BN * G::LBPB;          // [TM][32] X halves of the step
-  uint16_t* d_lds = reinterpret_cast<uint16_t*>(h_lds + TM * 32);  // [BN] side-channel d (q6_k)
+  // one stage: activations [TM][A_STRIDE] | wire [BN][LBPB] | X halves [TM][32] | side-channel d [BN] (q6_k);
+  // DB keeps two stages so that the next step is parked while this one is multiplied
+  constexpr int STAGE = A_BYTES + BN * G::LBPB + TM * 32 + BN * 2;
+  static_assert(STAGE % 16 == 0, "stage size keeps 16-byte alignment");
+  constexpr int B_OFF = A_BYTES, H_OFF = B_OFF + BN * G::LBPB, D_OFF = H_OFF + TM * 32;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, kg = lane >> 5;
@@ -139,7 +143,7 @@ __global__ __launch_bounds__(GM_THREADS, MT == 4 ? 1 : 2) void kquant_gemm_kerne
   const int nrows = N - n0 < BN ? N - n0 : BN;
 
   // piece maps: activations piece i = tid + 256 t -> (row i / 32, piece i % 32); wire piece -> (row i / PPR, i % PPR)
-  const int a_row = tid >> 5, a_pc = tid & 31;  // + 8 rows per t
+  const int a_row = tid >> 5, a_pc = tid & 31;  // + AROWS rows per t
   uint32_t w_goff[G::WPT], w_loff[G::WPT];
   {
     int r = tid / G::PPR, pc = tid % G::PPR;
@@ -160,14 +164,14 @@ __global__ __launch_bounds__(GM_THREADS, MT == 4 ? 1 : 2) void kquant_gemm_kerne
   const _Float16* xtile = xh + (size_t)m0 * K;
   const _Float16* htile = xhl + (size_t)m0 * nsb * 16;
 
-  // side channel for the trailing 2-byte d of a q6_k block: thread -> row tid % 128
-  const uint8_t* d_src = wtile + (size_t)((tid & 127) < nrows ? (tid & 127) : 0) * row_bytes + 208;
+  // side channel for the trailing 2-byte d of a q6_k block: thread -> row tid % BN
+  const uint8_t* d_src = wtile + (size_t)((tid & (BN - 1)) < nrows ? (tid & (BN - 1)) : 0) * row_bytes + 208;
   u32x4 areg[APT], wreg[G::WPT], hreg;
   uint16_t dreg = 0;
   auto issue = [&](int sb) {
     StaticFor<APT>::run([&](auto t) {
       constexpr int T = decltype(t)::value;
-      areg[T] = *reinterpret_cast<const u32x4*>(xtile + (size_t)(a_row + 8 * T) * K + 256 * sb + 8 * a_pc);
+      areg[T] = *reinterpret_cast<const u32x4*>(xtile + (size_t)(a_row + AROWS * T) * K + 256 * sb + 8 * a_pc);
     });
     StaticFor<G::WPT>::run([&](auto t) {
       constexpr int T = decltype(t)::value;
@@ -178,40 +182,58 @@ __global__ __launch_bounds__(GM_THREADS, MT == 4 ? 1 : 2) void kquant_gemm_kerne
     if constexpr (G::MINS)
       hreg = *reinterpret_cast<const u32x4*>(htile + ((size_t)((tid >> 1) < TM ? (tid >> 1) : 0) * nsb + sb) * 16 + 8 * (tid & 1));
   };
-  auto park = [&]() {
+  auto park = [&](uint8_t* stage) {
     StaticFor<APT>::run([&](auto t) {
       constexpr int T = decltype(t)::value;
-      *reinterpret_cast<u32x4*>(a_lds + (a_row + 8 * T) * A_STRIDE + 16 * a_pc) = areg[T];
+      *reinterpret_cast<u32x4*>(stage + (a_row + AROWS * T) * A_STRIDE + 16 * a_pc) = areg[T];
     });
     StaticFor<G::WPT>::run([&](auto t) {
       constexpr int T = decltype(t)::value;
-      if (w_loff[T] != 0xffffffffu) *reinterpret_cast<u32x4*>(b_lds + w_loff[T]) = wreg[T];
+      if (w_loff[T] != 0xffffffffu) *reinterpret_cast<u32x4*>(stage + B_OFF + w_loff[T]) = wreg[T];
     });
     if constexpr (G::MINS) {
-      if (tid < 2 * TM) *reinterpret_cast<u32x4*>(h_lds + 16 * tid) = hreg;
+      if (tid < 2 * TM) *reinterpret_cast<u32x4*>(stage + H_OFF + 16 * tid) = hreg;
     }
     if constexpr (G::SIDE_D) {
-      if (tid < BN) d_lds[tid] = dreg;
+      if (tid < BN) reinterpret_cast<uint16_t*>(stage + D_OFF)[tid] = dreg;
     }
   };
-
   f32x16 acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; t++) acc[t] = f32x16{0};
 
-  const uint8_t* b_lane = b_lds + (wave * 32 + l32) * G::LBPB;
-  const uint8_t* a_lane = a_lds + l32 * A_STRIDE + 32 * kg;
-  const uint8_t* h_lane = h_lds + l32 * 32 + 16 * kg;
+  auto multiply = [&](const uint8_t* stage) {
+    const uint16_t d_side = G::SIDE_D ? reinterpret_cast<const uint16_t*>(stage + D_OFF)[wave * 32 + l32] : (uint16_t)0;
+    superblock_mma<C, MT>(stage + B_OFF + (wave * 32 + l32) * G::LBPB, d_side, kg, stage + l32 * A_STRIDE + 32 * kg,
+                         32 * A_STRIDE, stage + H_OFF + l32 * 32 + 16 * kg, 32 * 32, acc);
+  };
 
   issue(0);
-  for (int sb = 0; sb < nsb; sb++) {
-    if (sb > 0) lds_barrier();  // everyone is done reading the previous step
-    park();
-    if (sb + 1 < nsb) issue(sb + 1);
+  if constexpr (DB) {
+    // Two stages: step sb + 1 is parked into the idle stage (its loads were issued one whole step earlier),
+    // the loads of step sb + 2 go out, then step sb is multiplied; ONE barrier per step tells everyone that
+    // the stage just read may be overwritten and that the stage just written may be read.
+    park(smem);
+    if (nsb > 1) issue(1);
     lds_barrier();
-
-    superblock_mma<C, MT>(b_lane, G::SIDE_D ? d_lds[wave * 32 + l32] : (uint16_t)0, kg, a_lane, 32 * A_STRIDE, h_lane,
-                         32 * 32, acc);
+    for (int sb = 0; sb < nsb; sb++) {
+      uint8_t* cur = smem + (sb & 1) * STAGE;
+      uint8_t* nxt = smem + ((sb + 1) & 1) * STAGE;
+      if (sb + 1 < nsb) {
+        park(nxt);
+        if (sb + 2 < nsb) issue(sb + 2);
+      }
+      multiply(cur);
+      lds_barrier();
+    }
+  } else {
+    for (int sb = 0; sb < nsb; sb++) {
+      if (sb > 0) lds_barrier();  // everyone is done reading the previous step
+      park(smem);
+      if (sb + 1 < nsb) issue(sb + 1);
+      lds_barrier();
+      multiply(smem);
+    }
   }
 
   // ---- epilogue: undo the per-row activation scale, round once, store
@@ -229,21 +251,21 @@ __global__ __launch_bounds__(GM_THREADS, MT == 4 ? 1 : 2) void kquant_gemm_kerne
   }
 }
 
-template <int C, int DT, int MT>
+template <int C, int DT, int MT, int WAVES, bool DB = false>
 int launch_gemm_mt(const _Float16* xh, const _Float16* xhl, const float* rs, const uint8_t* w, void* y, int M, int N,
                    int K, hipStream_t s) {
-  using G = WireGeom<C>;
-  constexpr int TM = 32 * MT;
+  using G = WireGeom<C, WAVES>;
+  constexpr int TM = 32 * MT, BN = G::BN;
   const int mtiles = (M + TM - 1) / TM, ntiles = (N + BN - 1) / BN;
-  const size_t lds = TM * A_STRIDE + BN * G::LBPB + TM * 32 + BN * 2;
-  auto kern = kquant_gemm_kernel<C, DT, MT>;
+  const size_t lds = (size_t)(TM * A_STRIDE + BN * G::LBPB + TM * 32 + BN * 2) * (DB ? 2 : 1);
+  auto kern = kquant_gemm_kernel<C, DT, MT, WAVES, DB>;
   static bool attr_set = false;
   if (!attr_set) {
     KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(mtiles * ntiles), dim3(GM_THREADS), lds, s, xh, xhl, rs, w, static_cast<uint16_t*>(y), M,
+  hipLaunchKernelGGL(kern, dim3(mtiles * ntiles), dim3(G::THREADS), lds, s, xh, xhl, rs, w, static_cast<uint16_t*>(y), M,
                      N, K, mtiles);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
@@ -259,9 +281,22 @@ int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, v
   hipLaunchKernelGGL((gemm_prepass_kernel<DT>), dim3(mpad), dim3(PP_THREADS), 0, s, static_cast<const uint16_t*>(x), xh,
                      xhl, rs, M, K);
   KQ_HIP_CHECK(hipGetLastError());
-  const int mt = g_gemm_force_mt ? g_gemm_force_mt : 2;
-  if (mt == 4) return launch_gemm_mt<C, DT, 4>(xh, xhl, rs, w, y, M, N, K, s);
-  return launch_gemm_mt<C, DT, 2>(xh, xhl, rs, w, y, M, N, K, s);
+  // Tile shapes (activation rows x weight rows): 64 x 128, one stage, two workgroups per CU: the default;
+  // 128 x 128, one workgroup per CU: selectable only (measured slower);
+  // 64 x 256 on 8 waves with two LDS stages (q4_k; q5_k would fit but measured slower, q6_k does not fit):
+  // one barrier per step instead of two and the next step is parked while this one is multiplied, measured
+  // 5 - 9 % faster once every CU gets 8 or more workgroups, slower below (fewer, longer workgroups).
+  int tile = g_gemm_tile;
+  if (tile == 256 && C != KQ_Q4_K) tile = 0;
+  if (tile == 0) {
+    const int64_t wgs = (int64_t)((M + 63) / 64) * ((N + 255) / 256);
+    tile = (C == KQ_Q4_K && wgs >= 8 * 256) ? 256 : 64;
+  }
+  if constexpr (C == KQ_Q4_K) {
+    if (tile == 256) return launch_gemm_mt<C, DT, 2, 8, true>(xh, xhl, rs, w, y, M, N, K, s);
+  }
+  if (tile == 128) return launch_gemm_mt<C, DT, 4, 4>(xh, xhl, rs, w, y, M, N, K, s);
+  return launch_gemm_mt<C, DT, 2, 4>(xh, xhl, rs, w, y, M, N, K, s);
 }
 
 }  // namespace
@@ -303,4 +338,4 @@ int kq_launch_act_prepass(const void* x, void* xh, void* xhl, float* rs, int M, 
   return KQ_OK;
 }
 
-extern "C" void kq_set_gemm_tile_rows(int rows) { g_gemm_force_mt = rows == 128 ? 4 : rows == 64 ? 2 : 0; }
+extern "C" void kq_set_gemm_tile_rows(int rows) { g_gemm_tile = (rows == 64 || rows == 128 || rows == 256) ? rows : 0; }

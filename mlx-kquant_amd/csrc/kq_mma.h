@@ -106,7 +106,7 @@ __device__ __forceinline__ void superblock_mma(const uint8_t* __restrict__ b_lan
     // 16 MFMA groups (sub-block j = it / 2, K-half s = it % 2).  The activation fragments of group
     // it + 1 are requested before group it is decoded, so the LDS latency hides behind the decode
     // and the MFMAs instead of stalling each group.
-    f16x8 afr[2][MT];
+    f16x8 afr[2][MT], bfr[2];
     uint4 qv[4];
     uint32_t hb[4] = {0, 0, 0, 0};  // q5_k: fifth bits of this lane's 16 weights, positioned per pair
 #pragma unroll
@@ -120,16 +120,10 @@ __device__ __forceinline__ void superblock_mma(const uint8_t* __restrict__ b_lan
     }
 #pragma unroll
     for (int t = 0; t < MT; t++) afr[0][t] = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile);
-    StaticFor<16>::run([&](auto itc) {
+    // B fragment of group it: sub-block j = it / 2, K-half s = it % 2
+    auto decode = [&](auto itc) -> f16x8 {
       constexpr int it = decltype(itc)::value;
       constexpr int j = it >> 1, s = it & 1, g = j >> 1, h = j & 1;
-      if constexpr (it + 1 < 16) {
-        constexpr int jn = (it + 1) >> 1, sn = (it + 1) & 1;
-#pragma unroll
-        for (int t = 0; t < MT; t++)
-          afr[(it + 1) & 1][t] = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile + 64 * jn + 16 * sn);
-        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of this group's decode (the scheduler sinks them)
-      }
       const uint32_t qw[4] = {qv[g].x, qv[g].y, qv[g].z, qv[g].w};
       const float scf = (float)((scw[j >> 2] >> (8 * (j & 3))) & 0xff);
       // low nibbles read 1024 + q, high nibbles (in place) 1024 + 16 q: fold the 16 into the scale
@@ -155,13 +149,38 @@ __device__ __forceinline__ void superblock_mma(const uint8_t* __restrict__ b_lan
 #pragma unroll
         for (int e = 0; e < 4; e++) bq[e] += add[e];
       }
-      const f16x8 b = {bq[0][0], bq[0][1], bq[1][0], bq[1][1], bq[2][0], bq[2][1], bq[3][0], bq[3][1]};
+      return f16x8{bq[0][0], bq[0][1], bq[1][0], bq[1][1], bq[2][0], bq[2][1], bq[3][0], bq[3][1]};
+    };
+    // 16 MFMA groups, software-pipelined: while the matrix core runs the MFMAs of group it, the wave decodes
+    // the B fragment of group it + 1 and requests its activation fragments.  A wave issues in order and a
+    // second MFMA waits for the first to leave the matrix core, so vector work placed AFTER a run of MFMAs
+    // would idle behind them; the group barriers below interleave it between them instead.
+    constexpr int DEC_VALU = C == KQ_Q5_K ? 30 : 14;  // vector instructions of one decode, roughly
+    bfr[0] = decode(std::integral_constant<int, 0>{});
+    __builtin_amdgcn_sched_barrier(0);  // group 0's own fragments and decode stay out of the pipelined region
+    StaticFor<16>::run([&](auto itc) {
+      constexpr int it = decltype(itc)::value;
+      if constexpr (it + 1 < 16) {
+        constexpr int jn = (it + 1) >> 1, sn = (it + 1) & 1;
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+          afr[(it + 1) & 1][t] = *reinterpret_cast<const f16x8*>(a_lane + t * a_tile + 64 * jn + 16 * sn);
+        bfr[(it + 1) & 1] = decode(std::integral_constant<int, it + 1>{});
+      }
 #pragma unroll
       for (int t = 0; t < MT; t++) {
         if constexpr (it == 0)
-          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t], b, f32x16{0}, 0, 0, 0);
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t], bfr[0], f32x16{0}, 0, 0, 0);
         else
-          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[it & 1][t], b, part[t], 0, 0, 0);
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[it & 1][t], bfr[it & 1], part[t], 0, 0, 0);
+      }
+      if constexpr (it + 1 < 16) {
+        __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);  // the next group's fragment requests go first
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                          // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, (DEC_VALU + MT - 1) / MT, 0);   // a slice of the decode
+        }
       }
     });
 #pragma unroll

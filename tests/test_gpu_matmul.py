@@ -205,10 +205,11 @@ def test_qmm_prefill_every_codec(kq, codec):
             assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, N, K, dtype)
 
 
-def test_qmm_prefill_gemm_both_tile_heights(kq):
-    """The 128-row tile variant (kq_set_gemm_tile_rows) gives the same rounded outputs as the default 64-row one:
-    both feed the same exact products to f32 accumulators in the same order."""
-    M, N, K = 200, 384, 1024
+def test_qmm_prefill_gemm_tile_variants(kq):
+    """The 128 x 128 and the two-stage 64 x 256 tile variants (kq_set_gemm_tile_rows) give the same rounded outputs
+    as the default 64 x 128 one: all feed the same exact products to f32 accumulators in the same order.  N is no
+    multiple of 256, M none of 64, and K spans several steps so that both LDS stages are reused."""
+    M, N, K = 200, 384, 2048
     lib = kq._load()
     for codec in ("q4_k", "q5_k", "q6_k"):
         wire = _wire(codec, N, K, seed=37)
@@ -216,14 +217,30 @@ def test_qmm_prefill_gemm_both_tile_heights(kq):
         want = O.qmm(xb, wire, codec, True, "bfloat16")
         outs = []
         try:
-            for rows in (128, 64):
+            for rows in (128, 256, 64):
                 lib.kq_set_gemm_tile_rows(rows)
                 got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
                 assert rel_l2(got, want, "bfloat16") <= TOL, (codec, rows)
                 outs.append(got)
         finally:
             lib.kq_set_gemm_tile_rows(0)
-        assert np.array_equal(outs[0], outs[1]), codec
+        assert np.array_equal(outs[0], outs[2]) and np.array_equal(outs[1], outs[2]), codec
+
+
+@pytest.mark.parametrize("K", [256, 512, 768])
+def test_qmm_prefill_gemm_two_stage_short_k(kq, K):
+    """The two-stage tile with one, two and three K steps (prologue only, one parked step, stage reuse)."""
+    M, N = 70, 264
+    lib = kq._load()
+    wire = _wire("q4_k", N, K, seed=39)
+    xb, xt = make_x((M, K), "float16", seed=40)
+    want = O.qmm(xb, wire, "q4_k", True, "float16")
+    try:
+        lib.kq_set_gemm_tile_rows(256)
+        got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, "q4_k"))
+    finally:
+        lib.kq_set_gemm_tile_rows(0)
+    assert rel_l2(got, want, "float16") <= TOL
 
 
 def test_qmm_prefill_gemm_wide_dynamic_range(kq):
