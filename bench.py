@@ -15,7 +15,8 @@ beforehand, so a step is the library call and nothing else.
 Extra fields: `sweep` (the decode projections of the q4_k_m recipe at M in {1,2,4,8}), `prefill`
 (q4_k / q5_k / q6_k GEMM 8192 -> 28672 at M in {512, 2048}), `moe` (128 experts, top-8, hidden 2048,
 intermediate 768: fused gate/up GLU in q4_k and down in q6_k at 1 and 256 tokens), `lowbit` (M=1
-GEMV 8192 -> 8192 in the low-bit codecs), `roofline` for the dominant kernel and `cpu_baseline`
+GEMV 8192 -> 8192 in the low-bit codecs), `dequantize` (whole-matrix decode to f16, wire bytes in plus
+2 N K bytes out), `roofline` for the dominant kernel and `cpu_baseline`
 (the CPU oracle timed on this box's host cores on the headline GEMV).
 """
 import argparse
@@ -116,6 +117,18 @@ class Abi:
 
         def call(_keep=keep):
             rc = lib.kq_qmm(*args)
+            if rc:
+                self._check(rc)
+        return call
+
+    def dequantize(self, w, codec, N, K, out):
+        lib = self.lib
+        cid = lib.kq_codec_id(codec.encode())
+        args = (w.data_ptr(), out.data_ptr(), N * K, cid, 1, self.stream)  # dtype code 1 = float16
+        keep = (w, out)
+
+        def call(_keep=keep):
+            rc = lib.kq_dequantize(*args)
             if rc:
                 self._check(rc)
         return call
@@ -385,6 +398,22 @@ def main():
                            "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
             del cps, wq
         out["lowbit"] = lowbit
+
+        # ---------------- dequantize to f16 (random structurally valid wire): bytes = wire in + 2 N K out
+        deq = []
+        for c, n, k in (("q4_k", 4096, 4096), ("q4_k", 28672, 8192), ("q6_k", 28672, 8192), ("iq3_s", 28672, 8192),
+                        ("q8_0", 28672, 8192)):
+            wb = n * kq.bytes_per_row(c, k)
+            total = wb + 2 * n * k
+            wq = synth_wire_torch(c, n, k, 9, dev)
+            # rotate over inputs AND outputs so that neither side is served by the last-level cache
+            cps = cold_copies(torch, wq, total)
+            outs = [torch.empty((n, k), dtype=torch.float16, device=dev) for _ in cps]
+            t, _ = time_calls(torch, [abi.dequantize(w, c, n, k, o) for w, o in zip(cps, outs)], 200, 20)
+            deq.append({"codec": c, "N": n, "K": k, "us": round(t * 1e3, 2), "cold_gbs": round(total / (t * 1e-3) / 1e9, 1),
+                        "pct_hbm_peak": round(100 * total / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
+            del cps, outs, wq
+        out["dequantize"] = deq
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(base_np, codec, K, M)

@@ -12,14 +12,17 @@
 namespace {
 
 constexpr int DQ_THREADS = 256;
-constexpr int DQ_WEIGHTS = 4096;  // weights per workgroup (16 / 64 / 128 blocks)
+// Weights per workgroup: 4096 (16 / 64 / 128 blocks), or 16384 for superblock codecs on tensors large enough
+// to give every CU a few such workgroups (measured 4 - 9 % faster there, slower on small tensors and on the
+// 32-weight codecs, whose staged bytes then cost occupancy).
+constexpr int DQ_WEIGHTS = 4096, DQ_WEIGHTS_BIG = 16384;
 
-template <int C, int DT>
+template <int C, int DT, int WEIGHTS>
 __global__ __launch_bounds__(DQ_THREADS) void dequantize_kernel(const uint8_t* __restrict__ w,
                                                                 void* __restrict__ out, uint64_t num_blocks,
                                                                 const uint8_t* __restrict__ grids) {
   constexpr int WPB = kq_geom(C).wpb, BPB = kq_geom(C).bpb;
-  constexpr int NBLK = DQ_WEIGHTS / WPB;  // multiple of 16 -> chunk bytes are a multiple of 16
+  constexpr int NBLK = WEIGHTS / WPB;  // multiple of 16 -> chunk bytes are a multiple of 16
   constexpr int GPB = WPB / 8;            // 8-weight groups per block
   __shared__ __attribute__((aligned(16))) uint8_t lds[NBLK * BPB];
 
@@ -225,20 +228,28 @@ int dispatch_codec(int codec, A... a) {
 
 template <int C>
 struct DequantRun {
-  static int run(const uint8_t* w, void* out, uint64_t num_blocks, int dt, const uint8_t* grids, hipStream_t s) {
-    constexpr int NBLK = DQ_WEIGHTS / kq_geom(C).wpb;
+  template <int WEIGHTS>
+  static int launch(const uint8_t* w, void* out, uint64_t num_blocks, int dt, const uint8_t* grids, hipStream_t s) {
+    constexpr int NBLK = WEIGHTS / kq_geom(C).wpb;
     const uint64_t nwg = (num_blocks + NBLK - 1) / NBLK;
     if (nwg == 0) return KQ_OK;
     if (nwg > 0x7fffffffull) return kq_set_error(KQ_ERR_INVALID, "dequantize: tensor too large for one launch");
     dim3 grid((unsigned)nwg), block(DQ_THREADS);
     if (dt == KQ_F32)
-      hipLaunchKernelGGL((dequantize_kernel<C, KQ_F32>), grid, block, 0, s, w, out, num_blocks, grids);
+      hipLaunchKernelGGL((dequantize_kernel<C, KQ_F32, WEIGHTS>), grid, block, 0, s, w, out, num_blocks, grids);
     else if (dt == KQ_F16)
-      hipLaunchKernelGGL((dequantize_kernel<C, KQ_F16>), grid, block, 0, s, w, out, num_blocks, grids);
+      hipLaunchKernelGGL((dequantize_kernel<C, KQ_F16, WEIGHTS>), grid, block, 0, s, w, out, num_blocks, grids);
     else
-      hipLaunchKernelGGL((dequantize_kernel<C, KQ_BF16>), grid, block, 0, s, w, out, num_blocks, grids);
+      hipLaunchKernelGGL((dequantize_kernel<C, KQ_BF16, WEIGHTS>), grid, block, 0, s, w, out, num_blocks, grids);
     KQ_HIP_CHECK(hipGetLastError());
     return KQ_OK;
+  }
+  static int run(const uint8_t* w, void* out, uint64_t num_blocks, int dt, const uint8_t* grids, hipStream_t s) {
+    if constexpr (kq_geom(C).wpb == 256) {
+      if (num_blocks * 256ull >= (uint64_t)DQ_WEIGHTS_BIG * 256 * 16)
+        return launch<DQ_WEIGHTS_BIG>(w, out, num_blocks, dt, grids, s);
+    }
+    return launch<DQ_WEIGHTS>(w, out, num_blocks, dt, grids, s);
   }
 };
 

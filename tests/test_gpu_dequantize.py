@@ -86,3 +86,16 @@ def test_dequantize_config1_size(kq):
     assert got.shape == (4096, 4096)
     for r in range(8):
         assert np.array_equal(got[512 * r:512 * (r + 1)], want)
+
+
+@pytest.mark.parametrize("codec", ["q4_k", "q6_k", "iq2_xxs", "iq4_xs"])
+def test_dequantize_large_tensor_chunking(kq, codec):
+    """Tensors of 64 Mi weights and more take the 16384-weight workgroup chunk; 262176 superblocks leave a
+    ragged last workgroup (32 of 64 blocks).  Compared in slices to keep the host copies small."""
+    nblk = 262176
+    wire = O.synth_wire(codec, nblk, seed=77)
+    got = dev_to_bits(kq.dequantize(wire_to_dev(wire), None, codec, dtype=torch.float16)).reshape(-1)
+    step = 32768
+    for b0 in range(0, nblk, step):
+        want = O.dequantize(wire.reshape(nblk, -1)[b0:b0 + step], codec, "float16").reshape(-1)
+        assert np.array_equal(got[b0 * 256:b0 * 256 + want.size], want), (codec, b0)
