@@ -185,6 +185,25 @@ int kq_gather_qmv_mix(const void* x_dev, const void* w_dev, const void* shexp_w_
                       const float* scores_dev, void* out_dev, int T, int S, int E, int N, int K, int codec,
                       int shexp_codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* kq_gather_qmv_mix without a shared expert and with the expert bias (f32 [E, N]) added to every slot's product
+ * before the mix: out[t, :] = T(sum_s scores[t, s] * (x[t, s, :] . W_s^T + bias_s)).  mxfp4 / nvfp4 stacks only, as
+ * kq_gather_qmv's bias.  Workspace: kq_gather_qmv_mix_workspace_size(..., shexp_codec = -1, ...).
+ * Replaces gather_qmv_mix_bias (packed-layout op, reference src/kquant.h:321-333) once the stack is in wire form
+ * (kq_mxfp4_packed_to_wire). */
+int kq_gather_qmv_mix_bias(const void* x_dev, const void* w_dev, const float* bias_dev, const uint32_t* idx_dev,
+                           const float* scores_dev, void* out_dev, int T, int S, int E, int N, int K, int codec,
+                           int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
+
+/* mxfp4 between the MLX packed layout (uint32 codes [.., K/8], eight sequential 4-bit codes per word, 16-byte
+ * aligned; e8m0 scale bytes [.., K/32] in a tensor of their own) and the GGUF wire (17-byte blocks: scale byte,
+ * then code j in the low and code j + 16 in the high nibble of byte j).  num_blocks = number of 32-weight
+ * blocks.  The packed-layout ops of the reference (moe_glu_gather, gather_qmv_bias, gather_qmv_mix_bias,
+ * src/kquant.h:291-333) are served by converting a stack once and calling the wire-form ops. */
+int kq_mxfp4_packed_to_wire(const void* packed_dev, const void* scales_dev, void* wire_dev, int64_t num_blocks,
+                            void* stream);
+int kq_mxfp4_wire_to_packed(const void* wire_dev, void* packed_dev, void* scales_dev, int64_t num_blocks,
+                            void* stream);
+
 /* Router: expert scores over the E logit columns (scoring 0 = softmax, 1 = sqrt(softplus(x))), the top_k
  * largest by score (+ bias[e] when given; smallest index first on ties) and their mixing weights:
  * score / (sum of the picked scores (+ 1e-20 for scoring 1) if norm_topk_prob else the softmax sum)

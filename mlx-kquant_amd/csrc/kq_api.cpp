@@ -504,11 +504,11 @@ size_t kq_gather_qmv_mix_workspace_size(int T, int S, int E, int N, int K, int c
   return fixed + sub;
 }
 
-int kq_gather_qmv_mix(const void* x_dev, const void* w_dev, const void* shexp_w_dev, const uint32_t* idx_dev,
-                      const float* scores_dev, void* out_dev, int T, int S, int E, int N, int K, int codec,
-                      int shexp_codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream) {
+static int gather_qmv_mix_impl(const char* op, const void* x_dev, const void* w_dev, const void* shexp_w_dev,
+                               const float* bias_dev, const uint32_t* idx_dev, const float* scores_dev, void* out_dev, int T,
+                               int S, int E, int N, int K, int codec, int shexp_codec, int dtype, void* workspace_dev,
+                               size_t workspace_bytes, void* stream) {
   const bool shared = shexp_w_dev != nullptr;
-  const char* op = shared ? "gather_qmv_mix_kq" : "gather_qmv_mix_ns_kq";
   if (shared && !shexp_combo_ok(codec, shexp_codec))
     return kq_set_error(KQ_ERR_INVALID, "%s: no fused kernel for this expert / shared-expert codec pair", op);
   if (S < (shared ? 2 : 1)) return kq_set_error(KQ_ERR_INVALID, "%s: bad slot count", op);
@@ -545,7 +545,7 @@ int kq_gather_qmv_mix(const void* x_dev, const void* w_dev, const void* shexp_w_
   const size_t sub_bytes = workspace_bytes - o;
   {
     OutMapScope scope(KqOutMap{1, 1, 0, 1});  // f32 slot results [T][S][N]
-    rc = kq_gather_qmv(x_dev, w_dev, idx_all, nullptr, yf, T, S, E, N, K, codec, dtype, sub, sub_bytes, stream);
+    rc = kq_gather_qmv(x_dev, w_dev, idx_all, bias_dev, yf, T, S, E, N, K, codec, dtype, sub, sub_bytes, stream);
     if (rc) return rc;
   }
   if (shared) {
@@ -558,6 +558,43 @@ int kq_gather_qmv_mix(const void* x_dev, const void* w_dev, const void* shexp_w_
     if (rc) return rc;
   }
   return kq_launch_mix_slots(yf, scores_dev, out_dev, T, S, N, dtype, s);
+}
+
+int kq_gather_qmv_mix(const void* x_dev, const void* w_dev, const void* shexp_w_dev, const uint32_t* idx_dev,
+                      const float* scores_dev, void* out_dev, int T, int S, int E, int N, int K, int codec,
+                      int shexp_codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream) {
+  return gather_qmv_mix_impl(shexp_w_dev ? "gather_qmv_mix_kq" : "gather_qmv_mix_ns_kq", x_dev, w_dev, shexp_w_dev, nullptr,
+                             idx_dev, scores_dev, out_dev, T, S, E, N, K, codec, shexp_codec, dtype, workspace_dev,
+                             workspace_bytes, stream);
+}
+
+int kq_gather_qmv_mix_bias(const void* x_dev, const void* w_dev, const float* bias_dev, const uint32_t* idx_dev,
+                           const float* scores_dev, void* out_dev, int T, int S, int E, int N, int K, int codec, int dtype,
+                           void* workspace_dev, size_t workspace_bytes, void* stream) {
+  const char* op = "gather_qmv_mix_bias";
+  if (!bias_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null bias", op);
+  return gather_qmv_mix_impl(op, x_dev, w_dev, nullptr, bias_dev, idx_dev, scores_dev, out_dev, T, S, E, N, K, codec, -1,
+                             dtype, workspace_dev, workspace_bytes, stream);
+}
+
+int kq_mxfp4_packed_to_wire(const void* packed_dev, const void* scales_dev, void* wire_dev, int64_t num_blocks,
+                            void* stream) {
+  if (num_blocks < 0) return kq_set_error(KQ_ERR_INVALID, "mxfp4_packed_to_wire: negative block count");
+  if (num_blocks == 0) return KQ_OK;
+  if (!packed_dev || !scales_dev || !wire_dev) return kq_set_error(KQ_ERR_INVALID, "mxfp4_packed_to_wire: null buffer");
+  if (reinterpret_cast<uintptr_t>(packed_dev) & 15)
+    return kq_set_error(KQ_ERR_INVALID, "mxfp4_packed_to_wire: packed codes must be 16-byte aligned");
+  return kq_launch_mxfp4_repack(packed_dev, scales_dev, wire_dev, num_blocks, 1, static_cast<hipStream_t>(stream));
+}
+
+int kq_mxfp4_wire_to_packed(const void* wire_dev, void* packed_dev, void* scales_dev, int64_t num_blocks, void* stream) {
+  if (num_blocks < 0) return kq_set_error(KQ_ERR_INVALID, "mxfp4_wire_to_packed: negative block count");
+  if (num_blocks == 0) return KQ_OK;
+  if (!packed_dev || !scales_dev || !wire_dev) return kq_set_error(KQ_ERR_INVALID, "mxfp4_wire_to_packed: null buffer");
+  if (reinterpret_cast<uintptr_t>(packed_dev) & 15)
+    return kq_set_error(KQ_ERR_INVALID, "mxfp4_wire_to_packed: packed codes must be 16-byte aligned");
+  return kq_launch_mxfp4_repack(packed_dev, scales_dev, const_cast<void*>(wire_dev), num_blocks, 0,
+                                static_cast<hipStream_t>(stream));
 }
 
 int kq_moe_router_topk(const void* logits_dev, int dtype, int T, int E, int top_k, int norm_topk_prob, int shared_gate,

@@ -116,6 +116,7 @@ int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, cons
 // Helpers of the slot-mixing ops: idx [T][S-1] -> idx2 [T][S] (last slot = expert 0), and
 // out[t][n] = T(sum_s scores[t][s] * yf[t][s][n]).
 int kq_launch_pad_idx(const uint32_t* idx, uint32_t* idx2, int T, int S, hipStream_t s);
+int kq_launch_mxfp4_repack(const void* packed, const void* scales, void* wire, int64_t nblocks, int to_wire, hipStream_t s);
 int kq_launch_expert_tile_map(const uint32_t* idx, int rows, int E, uint32_t* map, int cap, uint32_t* counts,
                               hipStream_t s);
 int kq_launch_tiles_to_rows(const uint32_t* map, const uint32_t* counts, int cap, int rows, int E, uint32_t none,

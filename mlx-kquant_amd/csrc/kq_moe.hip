@@ -205,6 +205,39 @@ __global__ __launch_bounds__(TILE_ROWS) void tiles_to_rows_kernel(const uint32_t
   row_expert[start + j] = e;
 }
 
+// ------------------------------------------------------------------ mxfp4: MLX packed layout <-> GGUF wire
+// MLX keeps the 32 codes of a block in sequence (byte b = code 2b | code 2b+1 << 4, eight codes per uint32) and
+// the e8m0 scale bytes in a tensor of their own; the GGUF block is the scale byte followed by 16 bytes holding
+// code j in the low and code j + 16 in the high nibble.  One thread moves one block.
+__global__ __launch_bounds__(256) void mxfp4_packed_to_wire_kernel(const uint32_t* __restrict__ packed,
+                                                                   const uint8_t* __restrict__ scales,
+                                                                   uint8_t* __restrict__ wire, int64_t nblocks) {
+  const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (b >= nblocks) return;
+  const u32x4 v = *reinterpret_cast<const u32x4*>(packed + 4 * b);
+  const uint64_t lo = (uint64_t)v[0] | ((uint64_t)v[1] << 32), hi = (uint64_t)v[2] | ((uint64_t)v[3] << 32);
+  uint8_t* o = wire + 17 * b;
+  o[0] = scales[b];
+#pragma unroll
+  for (int j = 0; j < 16; j++) o[1 + j] = (uint8_t)(((lo >> (4 * j)) & 15) | (((hi >> (4 * j)) & 15) << 4));
+}
+
+__global__ __launch_bounds__(256) void mxfp4_wire_to_packed_kernel(const uint8_t* __restrict__ wire,
+                                                                   uint32_t* __restrict__ packed,
+                                                                   uint8_t* __restrict__ scales, int64_t nblocks) {
+  const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (b >= nblocks) return;
+  const uint8_t* in = wire + 17 * b;
+  uint64_t lo = 0, hi = 0;
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    lo |= (uint64_t)(in[1 + j] & 15) << (4 * j);
+    hi |= (uint64_t)(in[1 + j] >> 4) << (4 * j);
+  }
+  scales[b] = in[0];
+  *reinterpret_cast<u32x4*>(packed + 4 * b) = u32x4{(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
+}
+
 // ------------------------------------------------------------------ grouped GEMM
 struct MoeArgs {
   const _Float16* xh;   // [rows][K] f16 activations (prepass), row = pair / x_div
@@ -487,6 +520,21 @@ int kq_launch_tiles_to_rows(const uint32_t* map, const uint32_t* counts, int cap
   KQ_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL(tiles_to_rows_kernel, dim3((unsigned)cap), dim3(TILE_ROWS), 0, s, map, counts, cap, rows, E,
                      row_expert);
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
+int kq_launch_mxfp4_repack(const void* packed, const void* scales, void* wire, int64_t nblocks, int to_wire,
+                           hipStream_t s) {
+  if (nblocks <= 0) return KQ_OK;
+  const unsigned blocks = (unsigned)((nblocks + 255) / 256);
+  if (to_wire)
+    hipLaunchKernelGGL(mxfp4_packed_to_wire_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const uint32_t*>(packed),
+                       static_cast<const uint8_t*>(scales), static_cast<uint8_t*>(wire), nblocks);
+  else
+    hipLaunchKernelGGL(mxfp4_wire_to_packed_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const uint8_t*>(wire),
+                       static_cast<uint32_t*>(const_cast<void*>(packed)), static_cast<uint8_t*>(const_cast<void*>(scales)),
+                       nblocks);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }

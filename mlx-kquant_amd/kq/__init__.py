@@ -26,7 +26,8 @@ __all__ = [
     "codecs", "codec_has_matmul", "codec_has_moe_glu", "dequantize", "quantized_matmul", "quantized_matmul_qmv_bias",
     "gather_qmm", "expert_tile_map", "gather_qmm_seg",
     "moe_glu_gather_kq", "gather_qmv_kq", "moe_glu_gather_shexp_kq", "gather_qmv_mix_kq", "gather_qmv_mix_ns_kq",
-    "moe_router_topk", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
+    "moe_router_topk", "mxfp4_packed_to_wire", "mxfp4_wire_to_packed", "moe_glu_gather", "gather_qmv_bias",
+    "gather_qmv_mix_bias", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
     "weights_per_row", "lib_path",
 ]
 
@@ -84,6 +85,9 @@ def _load():
     lib.kq_moe_glu_gather.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, f, f, i, i, vp, sz, vp]
     lib.kq_gather_qmv.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, sz, vp]
     lib.kq_quantize.argtypes = [vp, vp, vp, i64, i64, i]
+    lib.kq_gather_qmv_mix_bias.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, sz, vp]
+    lib.kq_mxfp4_packed_to_wire.argtypes = [vp, vp, vp, i64, vp]
+    lib.kq_mxfp4_wire_to_packed.argtypes = [vp, vp, vp, i64, vp]
     lib.kq_expert_tile_map_cap.restype = i64
     lib.kq_expert_tile_map_cap.argtypes = [i64, i]
     lib.kq_expert_tile_map.argtypes = [vp, i64, i, vp, i64, vp, vp]
@@ -605,6 +609,127 @@ def gather_qmv_mix_ns_kq(x, w, kquant_type, indices, scores, *, stream=None):
     """No-shared-expert routing mix: x [T, S, K], indices [T, S], scores [T, S]; returns [T, N].
     Mirrors gather_qmv_mix_ns_kq, src/kquant_moe_glu.cpp:1325-1364."""
     return _gather_qmv_mix("gather_qmv_mix_ns_kq", x, w, None, kquant_type, kquant_type, indices, scores, stream)
+
+
+# ------------------------------------------------------------------ MLX packed mxfp4 layout
+_PACKED_INTS = (torch.int32, torch.uint32)
+
+
+def _check_packed_stack(op, w, sc, b, K):
+    """check_expert_stack, src/kquant_moe_glu.cpp:802-841 (uint32 there; torch callers may hold int32)."""
+    if w.ndim != 3 or w.dtype not in _PACKED_INTS:
+        raise ValueError(f"[kq.{op}] expert weights must be uint32 [E, N, K/8].")
+    if sc.ndim != 3 or sc.dtype != torch.uint8:
+        raise ValueError(f"[kq.{op}] expert scales must be uint8 [E, N, K/32].")
+    if w.shape[2] * 8 != K or sc.shape[2] * 32 != K:
+        raise ValueError(f"[kq.{op}] weight/scale trailing dims do not match K.")
+    if w.shape[0] != sc.shape[0] or w.shape[1] != sc.shape[1]:
+        raise ValueError(f"[kq.{op}] weight/scale expert dims do not match.")
+    if b is not None and (b.ndim != 2 or b.shape[0] != w.shape[0] or b.shape[1] != w.shape[1]):
+        raise ValueError(f"[kq.{op}] bias must be [E, N].")
+    if w.shape[1] % 8 != 0:
+        raise ValueError(f"[kq.{op}] N must be a multiple of 8.")
+    if K % 32 != 0:
+        raise ValueError(f"[kq.{op}] K must be a multiple of 32.")
+    if not w.is_contiguous() or not sc.is_contiguous():
+        raise ValueError(f"[kq.{op}] weights/scales must be row-contiguous.")
+
+
+def mxfp4_packed_to_wire(w, scales, *, stream=None):
+    """MLX packed mxfp4 (codes uint32 / int32 [..., K/8], e8m0 scales uint8 [..., K/32]) -> GGUF wire uint8
+    [..., K/32 * 17] (the two-halves nibble order of src/kquant_cpu_decode.cpp:403-418).  A device kernel; convert a
+    stack once at load time and call the wire-form ops on the result."""
+    op = "mxfp4_packed_to_wire"
+    if w.dtype not in _PACKED_INTS or scales.dtype != torch.uint8 or w.ndim < 1 or w.shape[:-1] != scales.shape[:-1] \
+            or w.shape[-1] != 4 * scales.shape[-1]:
+        raise ValueError("[kq.mxfp4_packed_to_wire] expects codes [..., K/8] (32-bit words) and uint8 scales [..., K/32].")
+    _same_device(op, w, scales)
+    sp = _stream_ptr(op, w, stream)
+    w_c, s_c = w.contiguous(), scales.contiguous()
+    wire = torch.empty(tuple(scales.shape[:-1]) + (scales.shape[-1] * 17,), dtype=torch.uint8, device=w.device)
+    with torch.cuda.device(w.device):
+        _check(_load().kq_mxfp4_packed_to_wire(w_c.data_ptr(), s_c.data_ptr(), wire.data_ptr(), s_c.numel(), sp))
+    return wire
+
+
+def mxfp4_wire_to_packed(wire, *, stream=None):
+    """The inverse of mxfp4_packed_to_wire: (codes int32 [..., K/8], scales uint8 [..., K/32])."""
+    op = "mxfp4_wire_to_packed"
+    if wire.dtype != torch.uint8 or wire.ndim < 1 or wire.shape[-1] % 17 != 0:
+        raise ValueError("[kq.mxfp4_wire_to_packed] expects uint8 wire [..., K/32 * 17].")
+    sp = _stream_ptr(op, wire, stream)
+    nb = wire.shape[-1] // 17
+    w_c = wire.contiguous()
+    packed = torch.empty(tuple(wire.shape[:-1]) + (nb * 4,), dtype=torch.int32, device=wire.device)
+    scales = torch.empty(tuple(wire.shape[:-1]) + (nb,), dtype=torch.uint8, device=wire.device)
+    with torch.cuda.device(wire.device):
+        _check(_load().kq_mxfp4_wire_to_packed(w_c.data_ptr(), packed.data_ptr(), scales.data_ptr(), scales.numel(), sp))
+    return packed, scales
+
+
+def moe_glu_gather(x, gate_w, gate_scales, gate_bias, up_w, up_scales, up_bias, indices, alpha=1.702, limit=7.0, *,
+                   stream=None):
+    """Fused gate / up expert products with expert biases and the clamped SwiGLU epilogue on MLX packed mxfp4
+    stacks: x [T, K], indices [T, R] -> [T, R, N].  The stacks are brought to wire form on the device (one pass
+    over their bytes per call; convert once with mxfp4_packed_to_wire and call moe_glu_gather_kq to avoid it).
+    Mirrors moe_glu_gather, src/kquant_moe_glu.cpp:936-986."""
+    op = "moe_glu_gather"
+    if x.ndim != 2:
+        raise ValueError("[kq.moe_glu_gather] x must be 2-D [T, K].")
+    if indices.ndim != 2 or indices.shape[0] != x.shape[0]:
+        raise ValueError("[kq.moe_glu_gather] indices must be [T, R] matching x.")
+    K = x.shape[1]
+    _check_packed_stack(op, gate_w, gate_scales, gate_bias, K)
+    _check_packed_stack(op, up_w, up_scales, up_bias, K)
+    if gate_w.shape != up_w.shape:
+        raise ValueError("[kq.moe_glu_gather] gate and up stacks must have the same shape.")
+    return moe_glu_gather_kq(x, mxfp4_packed_to_wire(gate_w, gate_scales, stream=stream),
+                             mxfp4_packed_to_wire(up_w, up_scales, stream=stream), "mxfp4", indices, act="swiglu_clamp",
+                             limit=limit, gate_bias=gate_bias, up_bias=up_bias, alpha=alpha, stream=stream)
+
+
+def gather_qmv_bias(x, w, scales, bias, indices, *, stream=None):
+    """out[t, r] = x[t, r] @ W_e.T + bias_e on an MLX packed mxfp4 stack: x [T, R, K] -> [T, R, N].
+    Mirrors gather_qmv_bias, src/kquant_moe_glu.cpp:988-1024."""
+    op = "gather_qmv_bias"
+    if x.ndim != 3:
+        raise ValueError("[kq.gather_qmv_bias] x must be 3-D [T, R, K].")
+    if indices.ndim != 2 or tuple(indices.shape) != tuple(x.shape[:2]):
+        raise ValueError("[kq.gather_qmv_bias] indices must be [T, R] matching x.")
+    _check_packed_stack(op, w, scales, bias, x.shape[2])
+    return gather_qmv_kq(x, mxfp4_packed_to_wire(w, scales, stream=stream), "mxfp4", indices, bias=bias, stream=stream)
+
+
+def gather_qmv_mix_bias(x, w, scales, bias, indices, scores, *, stream=None):
+    """gather_qmv_bias with the routing mix folded in: out[t] = sum_s scores[t, s] * (x[t, s] @ W_e.T + bias_e),
+    f32 accumulation, one rounding; x [T, S, K], indices / scores [T, S] -> [T, N].
+    Mirrors gather_qmv_mix_bias, src/kquant_moe_glu.cpp:1026-1068."""
+    op = "gather_qmv_mix_bias"
+    if x.ndim != 3:
+        raise ValueError("[kq.gather_qmv_mix_bias] x must be 3-D [T, S, K].")
+    T, S, K = x.shape
+    if indices.ndim != 2 or tuple(indices.shape) != (T, S):
+        raise ValueError("[kq.gather_qmv_mix_bias] indices must be [T, S].")
+    if scores.ndim != 2 or tuple(scores.shape) != (T, S):
+        raise ValueError("[kq.gather_qmv_mix_bias] scores must be [T, S].")
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("[kq.gather_qmv_mix_bias] x must be float16 or bfloat16.")
+    _check_packed_stack(op, w, scales, bias, K)
+    _same_device(op, x, w, scales, bias, indices, scores)
+    sp = _stream_ptr(op, x, stream)
+    wire = mxfp4_packed_to_wire(w, scales, stream=stream)
+    cid, _ = _codec(op, "mxfp4")
+    E, N = w.shape[0], w.shape[1]
+    x_c, idx = x.contiguous(), _prep_idx(indices)
+    sc, b = scores.to(torch.float32).contiguous(), bias.to(torch.float32).contiguous()
+    out = torch.empty((T, N), dtype=x.dtype, device=x.device)
+    lib = _load()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.kq_gather_qmv_mix_workspace_size(T, S, E, N, K, cid, -1, _DT[x.dtype])
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=x.device)
+        _check(lib.kq_gather_qmv_mix_bias(x_c.data_ptr(), wire.data_ptr(), b.data_ptr(), idx.data_ptr(), sc.data_ptr(),
+                                          out.data_ptr(), T, S, E, N, K, cid, _DT[x.dtype], ws.data_ptr(), ws_bytes, sp))
+    return out
 
 
 def moe_router_topk(logits, top_k, norm_topk_prob, shared_gate=True, per_expert_scale=None, bias=None,
