@@ -224,6 +224,17 @@ int kq_moe_router_topk(const void* logits_dev, int dtype, int T, int E, int top_
 int kq_quantize(const float* w_host, const float* imatrix_host, uint8_t* wire_host, int64_t rows, int64_t K,
                 int codec);
 
+/* The same encoding on the device for the codecs the reference encodes on the GPU (q8_0, q4_0/1, q5_0/1,
+ * q2_k ... q6_k; KQ_ERR_UNSUPPORTED for the IQ codecs, whose encoder is host-only there and here):
+ * w_dev [rows, K] in `w_dtype` (0 / 1 / 2 = f32 / f16 / bf16), imatrix_dev f32 [K] or NULL, wire_dev
+ * rows * bytes_per_row bytes.  One thread per block runs the host encoder's code, so the bytes equal
+ * kq_quantize's on the same values.  kq_quantize_dev_supported tells which codecs qualify.
+ * Replaces KQuantQuantize::eval_gpu (kernels metal/mlx/backend/metal/kernels/kq_quantized_encode.h),
+ * reference src/kquant_ops.cpp:550-631. */
+int kq_quantize_dev_supported(int codec);
+int kq_quantize_dev(const void* w_dev, int w_dtype, const float* imatrix_dev, void* wire_dev, int64_t rows,
+                    int64_t K, int codec, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,8 @@ SOURCES = [
     ("kq_anymma.hip", ["-ffp-contract=off"]),
     ("kq_codes.hip", []),
     ("kq_router.hip", ["-ffp-contract=off"]),
+    # the device encoder must round exactly like the host one: no fused multiply-adds
+    ("kq_encode_dev.hip", ["-ffp-contract=off"]),
 ]
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",

@@ -577,6 +577,24 @@ int kq_gather_qmv_mix_bias(const void* x_dev, const void* w_dev, const float* bi
                              dtype, workspace_dev, workspace_bytes, stream);
 }
 
+int kq_quantize_dev_supported(int codec) { return codec_ok(codec) && kq_encode_dev_supported(codec) ? 1 : 0; }
+
+int kq_quantize_dev(const void* w_dev, int w_dtype, const float* imatrix_dev, void* wire_dev, int64_t rows, int64_t K,
+                    int codec, void* stream) {
+  if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "quantize: unknown codec id %d", codec);
+  if (!kq_encode_dev_supported(codec))
+    return kq_set_error(KQ_ERR_UNSUPPORTED, "quantize: '%s' has no device encoder (use the host encoder)", kCodecs[codec].name);
+  if (w_dtype != KQ_F32 && w_dtype != KQ_F16 && w_dtype != KQ_BF16)
+    return kq_set_error(KQ_ERR_INVALID, "quantize: w must be float32, float16 or bfloat16");
+  const int wpb = kCodecs[codec].weights_per_block;
+  if (rows < 0 || K < 0 || K % wpb)
+    return kq_set_error(KQ_ERR_INVALID, "quantize: K (%lld) is not a multiple of %d", (long long)K, wpb);
+  if (rows == 0 || K == 0) return KQ_OK;
+  if (!w_dev || !wire_dev) return kq_set_error(KQ_ERR_INVALID, "quantize: null buffer");
+  return kq_launch_encode(w_dev, w_dtype, imatrix_dev, static_cast<uint8_t*>(wire_dev), rows, K, codec,
+                          static_cast<hipStream_t>(stream));
+}
+
 int kq_mxfp4_packed_to_wire(const void* packed_dev, const void* scales_dev, void* wire_dev, int64_t num_blocks,
                             void* stream) {
   if (num_blocks < 0) return kq_set_error(KQ_ERR_INVALID, "mxfp4_packed_to_wire: negative block count");

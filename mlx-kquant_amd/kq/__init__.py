@@ -85,6 +85,8 @@ def _load():
     lib.kq_moe_glu_gather.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, f, f, i, i, vp, sz, vp]
     lib.kq_gather_qmv.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, sz, vp]
     lib.kq_quantize.argtypes = [vp, vp, vp, i64, i64, i]
+    lib.kq_quantize_dev_supported.argtypes = [i]
+    lib.kq_quantize_dev.argtypes = [vp, i, vp, vp, i64, i64, i, vp]
     lib.kq_gather_qmv_mix_bias.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, sz, vp]
     lib.kq_mxfp4_packed_to_wire.argtypes = [vp, vp, vp, i64, vp]
     lib.kq_mxfp4_wire_to_packed.argtypes = [vp, vp, vp, i64, vp]
@@ -772,9 +774,10 @@ def moe_router_topk(logits, top_k, norm_topk_prob, shared_gate=True, per_expert_
 
 
 def quantize(w, kquant_type, imatrix=None, *, stream=None):
-    """Encode float weights [..., K] to wire bytes; returns (wq uint8 [..., bytes_per_row], scales uint8 [1]).
-    A host (CPU) encoder, as in the reference for the IQ codecs; the result is placed on w's device.
-    Mirrors quantize, src/kquant_ops.cpp:550-631."""
+    """Encode float weights [..., K] to wire bytes; returns (wq uint8 [..., bytes_per_row], scales uint8 [1]) on w's
+    device.  A tensor on the GPU is encoded there for the legacy and K-quant codecs (one thread per block running
+    the host encoder's code: same bytes); the IQ codecs, CPU tensors and stream="cpu" take the host encoder, as the
+    reference keeps its IQ encoders on the CPU.  Mirrors quantize, src/kquant_ops.cpp:550-631."""
     op = "quantize"
     cid, (wpb, bpb) = _codec(op, kquant_type)
     if not w.dtype.is_floating_point:
@@ -786,19 +789,28 @@ def quantize(w, kquant_type, imatrix=None, *, stream=None):
         raise ValueError(f"[kq.quantize] Last dim ({K}) must be a multiple of weights_per_block ({wpb}) for codec "
                          f"'{kquant_type}'.")
     info = _CodecInfo()
-    _load().kq_codec_get(cid, C.byref(info))
+    lib = _load()
+    lib.kq_codec_get(cid, C.byref(info))
     if not info.has_encode:
         raise ValueError(f"[kq.quantize] codec '{kquant_type}' has no encoder.")
-    im = None
     if imatrix is not None:
         if imatrix.ndim != 1 or imatrix.shape[0] != K:
             raise ValueError(f"[kq.quantize] imatrix must be 1-D with length {K}.")
-        im = imatrix.detach().to("cpu", torch.float32).contiguous()
     elif info.requires_imatrix:
         raise ValueError(f"[kq.quantize] codec '{kquant_type}' requires an importance matrix (imatrix).")
+    rows = w.numel() // K if K else 0
+    on_host = isinstance(stream, str) and stream == "cpu" or isinstance(stream, torch.device) and stream.type == "cpu"
+    if w.is_cuda and not on_host and lib.kq_quantize_dev_supported(cid):
+        sp = _stream_ptr(op, w, stream)
+        w_c = (w if w.dtype in _DT else w.to(torch.float32)).contiguous()
+        im = None if imatrix is None else imatrix.detach().to(w.device, torch.float32).contiguous()
+        wire = torch.empty(list(w.shape[:-1]) + [K // wpb * bpb], dtype=torch.uint8, device=w.device)
+        with torch.cuda.device(w.device):
+            _check(lib.kq_quantize_dev(w_c.data_ptr(), _DT[w_c.dtype], im.data_ptr() if im is not None else None,
+                                       wire.data_ptr(), rows, K, cid, sp))
+        return wire, torch.zeros(1, dtype=torch.uint8, device=w.device)
+    im = None if imatrix is None else imatrix.detach().to("cpu", torch.float32).contiguous()
     w_h = w.detach().to("cpu", torch.float32).contiguous()
-    rows = w_h.numel() // K if K else 0
     wire = torch.empty(list(w.shape[:-1]) + [K // wpb * bpb], dtype=torch.uint8)
-    _check(_load().kq_quantize(w_h.data_ptr(), im.data_ptr() if im is not None else None, wire.data_ptr(), rows, K,
-                               cid))
+    _check(lib.kq_quantize(w_h.data_ptr(), im.data_ptr() if im is not None else None, wire.data_ptr(), rows, K, cid))
     return wire.to(w.device), torch.zeros(1, dtype=torch.uint8, device=w.device)
