@@ -60,6 +60,83 @@ __device__ __forceinline__ uint32_t opaque_sgpr(uint32_t v) {
   return v;
 }
 
+// ------------------------------------------------------------------ activation prepass (one row, 256 threads)
+// Outputs for row m (rows >= M are written as zeros):
+//   xh   f16 [Mpad][K]            x * 2^-e[m], k permuted inside 8-groups to k0 k2 k1 k3 k4 k6 k5 k7
+//   xhl  f16 [Mpad][K/256][16]    per superblock: hi_j (8) then lo_j (8) with X_j = 32 (hi_j + lo_j)
+//   rs   f32 [Mpad]               2^e[m]
+// `red` = 4 floats of LDS; every thread of the workgroup must call (one barrier inside for bf16 input).
+constexpr int PP_THREADS = 256;
+
+template <int DT>
+__device__ __forceinline__ void prepass_row(const uint16_t* __restrict__ x, _Float16* __restrict__ xh,
+                                            _Float16* __restrict__ xhl, float* __restrict__ rs, int M, int K, int m,
+                                            int tid, float* red) {
+  const int ngroups = K >> 3;
+  _Float16* xo = xh + (size_t)m * K;
+  _Float16* ho = xhl + (size_t)m * (K >> 8) * 16;
+  if (m >= M) {
+    for (int g = tid; g < ngroups; g += PP_THREADS) *reinterpret_cast<u32x4*>(xo + 8 * g) = u32x4{0, 0, 0, 0};
+    for (int i = tid; i < (K >> 8) * 16; i += PP_THREADS) ho[i] = (_Float16)0.f;
+    if (tid == 0) rs[m] = 0.f;
+    return;
+  }
+  const uint16_t* xi = x + (size_t)m * K;
+  float inv = 1.f, scale = 1.f;
+  if constexpr (DT == KQ_BF16) {
+    float amax = 0.f;
+    for (int g = tid; g < ngroups; g += PP_THREADS) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(xi + 8 * g);
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] << 16)));
+        amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] & 0xffff0000u)));
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff;
+    if (eb != 0 && eb != 0xff) {
+      int e = (int)eb - 127 - 14;  // largest magnitude lands in [2^14, 2^15)
+      if (e < -100) e = -100;
+      scale = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+      inv = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
+    }
+  }
+  if (tid == 0) rs[m] = scale;
+  for (int g = tid; g < ngroups; g += PP_THREADS) {  // ngroups is a multiple of 32: whole quads stay together
+    const u32x4 v = *reinterpret_cast<const u32x4*>(xi + 8 * g);
+    _Float16 h[8];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      if constexpr (DT == KQ_BF16) {
+        h[2 * e] = (_Float16)(__builtin_bit_cast(float, v[e] << 16) * inv);
+        h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, v[e] & 0xffff0000u) * inv);
+      } else {
+        h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] & 0xffff));
+        h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
+      }
+    }
+    const f16x8 o = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+    *reinterpret_cast<f16x8*>(xo + 8 * g) = o;
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) s += (float)h[e];
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);  // 4 threads = one 32-wide sub-block
+    if ((tid & 3) == 0) {
+      const int j = g >> 2;  // global sub-block index
+      const _Float16 hi = (_Float16)(s * 0.03125f);
+      const _Float16 lo = (_Float16)((s - 32.0f * (float)hi) * 0.03125f);
+      ho[(j >> 3) * 16 + (j & 7)] = hi;
+      ho[(j >> 3) * 16 + 8 + (j & 7)] = lo;
+    }
+  }
+}
+
 // A superblock travels as PP 16-byte pieces (q6_k: its first 208 bytes; the trailing 2-byte d
 // goes through a side channel) and is parked in LDS LBPB bytes apart.  LBPB / 16 is odd for all
 // three codecs, which keeps the row-per-lane ds_read_b128 of the fragment fetch conflict-free.

@@ -33,21 +33,20 @@ struct Segment {
 // ------------------------------------------------------------------ pair sort (one workgroup)
 // order[] = pair ids grouped by expert; segs[] = (expert, first position in order, pairs <= 32).
 // Pairs whose expert id is out of range are left out (their output rows are not written).
-__global__ __launch_bounds__(SORT_THREADS) void moe_sort_kernel(const uint32_t* __restrict__ idx, int P, int E,
-                                                               int* __restrict__ order, Segment* __restrict__ segs,
-                                                               int* __restrict__ nseg_out) {
-  __shared__ int cnt[SORT_MAX_E];     // pairs per expert, then the running cursor
-  __shared__ int scan_p[SORT_THREADS], scan_s[SORT_THREADS];
+template <int THREADS>
+__device__ __forceinline__ void moe_sort_body(const uint32_t* __restrict__ idx, int P, int E, int* __restrict__ order,
+                                              Segment* __restrict__ segs, int* __restrict__ nseg_out, int* cnt,
+                                              int* scan_p, int* scan_s) {
   const int tid = threadIdx.x;
-  for (int e = tid; e < E; e += SORT_THREADS) cnt[e] = 0;
+  for (int e = tid; e < E; e += THREADS) cnt[e] = 0;
   __syncthreads();
-  for (int p = tid; p < P; p += SORT_THREADS) {
+  for (int p = tid; p < P; p += THREADS) {
     const uint32_t e = idx[p];
     if (e < (uint32_t)E) atomicAdd(&cnt[e], 1);
   }
   __syncthreads();
   // exclusive scans of pair counts and segment counts: thread t owns experts [t*ch, t*ch + ch)
-  const int ch = (E + SORT_THREADS - 1) / SORT_THREADS;
+  const int ch = (E + THREADS - 1) / THREADS;
   int lp = 0, ls = 0;
   for (int i = 0; i < ch; i++) {
     const int e = tid * ch + i;
@@ -59,7 +58,7 @@ __global__ __launch_bounds__(SORT_THREADS) void moe_sort_kernel(const uint32_t* 
   scan_p[tid] = lp;
   scan_s[tid] = ls;
   __syncthreads();
-  for (int off = 1; off < SORT_THREADS; off <<= 1) {
+  for (int off = 1; off < THREADS; off <<= 1) {
     const int vp = tid >= off ? scan_p[tid - off] : 0, vs = tid >= off ? scan_s[tid - off] : 0;
     __syncthreads();
     scan_p[tid] += vp;
@@ -67,7 +66,7 @@ __global__ __launch_bounds__(SORT_THREADS) void moe_sort_kernel(const uint32_t* 
     __syncthreads();
   }
   int bp = scan_p[tid] - lp, bs = scan_s[tid] - ls;  // exclusive prefix of this thread's experts
-  if (tid == SORT_THREADS - 1) *nseg_out = scan_s[tid];
+  if (tid == THREADS - 1) *nseg_out = scan_s[tid];
   for (int i = 0; i < ch; i++) {
     const int e = tid * ch + i;
     if (e < E) {
@@ -79,10 +78,36 @@ __global__ __launch_bounds__(SORT_THREADS) void moe_sort_kernel(const uint32_t* 
     }
   }
   __syncthreads();
-  for (int p = tid; p < P; p += SORT_THREADS) {
+  for (int p = tid; p < P; p += THREADS) {
     const uint32_t e = idx[p];
     if (e < (uint32_t)E) order[atomicAdd(&cnt[e], 1)] = p;
   }
+}
+
+__global__ __launch_bounds__(SORT_THREADS) void moe_sort_kernel(const uint32_t* __restrict__ idx, int P, int E,
+                                                               int* __restrict__ order, Segment* __restrict__ segs,
+                                                               int* __restrict__ nseg_out) {
+  __shared__ int cnt[SORT_MAX_E];     // pairs per expert, then the running cursor
+  __shared__ int scan_p[SORT_THREADS], scan_s[SORT_THREADS];
+  moe_sort_body<SORT_THREADS>(idx, P, E, order, segs, nseg_out, cnt, scan_p, scan_s);
+}
+
+// The pair sort and the activation prepass of one grouped launch in ONE kernel: workgroups 0 .. rows - 1 convert
+// one activation row each, workgroup `rows` sorts the pairs (neither depends on the other).  One launch fewer
+// per op; at 256 tokens the op time measured the same as with two launches.
+template <int DT>
+__global__ __launch_bounds__(PP_THREADS) void moe_prologue_kernel(const uint16_t* __restrict__ x, _Float16* __restrict__ xh,
+                                                                  _Float16* __restrict__ xhl, float* __restrict__ rs,
+                                                                  int rows, int K, const uint32_t* __restrict__ idx, int P,
+                                                                  int E, int* __restrict__ order,
+                                                                  Segment* __restrict__ segs, int* __restrict__ nseg_out) {
+  __shared__ int cnt[SORT_MAX_E];
+  __shared__ int scan_p[PP_THREADS], scan_s[PP_THREADS];
+  __shared__ float red[PP_THREADS / 64];
+  if ((int)blockIdx.x < rows)
+    prepass_row<DT>(x, xh, xhl, rs, rows, K, blockIdx.x, threadIdx.x, red);
+  else
+    moe_sort_body<PP_THREADS>(idx, P, E, order, segs, nseg_out, cnt, scan_p, scan_s);
 }
 
 // ------------------------------------------------------------------ row gather (batched gather_qmm)
@@ -576,9 +601,12 @@ int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, co
       (reinterpret_cast<uintptr_t>(ws) & 255))
     return KQ_ERR_UNSUPPORTED;
   const MoeWorkspace m = carve(ws, rows, P, E, K);
-  int rc = kq_launch_act_prepass(x, m.xh, m.xhl, m.rs, rows, K, dtype, s);
-  if (rc) return rc;
-  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(SORT_THREADS), 0, s, idx, P, E, m.order, m.segs, m.nseg);
+  if (dtype == KQ_F16)
+    hipLaunchKernelGGL(moe_prologue_kernel<KQ_F16>, dim3(rows + 1), dim3(PP_THREADS), 0, s, static_cast<const uint16_t*>(x),
+                       m.xh, m.xhl, m.rs, rows, K, idx, P, E, m.order, m.segs, m.nseg);
+  else
+    hipLaunchKernelGGL(moe_prologue_kernel<KQ_BF16>, dim3(rows + 1), dim3(PP_THREADS), 0, s, static_cast<const uint16_t*>(x),
+                       m.xh, m.xhl, m.rs, rows, K, idx, P, E, m.order, m.segs, m.nseg);
   KQ_HIP_CHECK(hipGetLastError());
   MoeArgs a{};
   a.xh = m.xh;
