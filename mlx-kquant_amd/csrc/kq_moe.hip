@@ -23,6 +23,13 @@ constexpr int MOE_THREADS = 256;
 constexpr int SEG_M = 32;            // pairs per segment = activation rows of the MFMA
 constexpr int SLAB = 128;            // weight rows per workgroup (GLU: 64 gate + 64 up)
 constexpr int A_STRIDE = 512 + 16;   // bytes per activation row of one K step in LDS
+// LDS stages of the grouped kernel.  Two stages (next step parked while this one is multiplied, one barrier per
+// step) cost a resident workgroup per CU and measured slower: 76.9 / 89.2 us against 72.7 / 64.7 us for the
+// GLU / down ops at 256 tokens, 128 experts.
+#ifndef KQ_MOE_STAGES
+#define KQ_MOE_STAGES 1
+#endif
+constexpr int MOE_STAGES = KQ_MOE_STAGES;
 constexpr int SORT_THREADS = 1024;
 constexpr int SORT_MAX_E = 4096;
 
@@ -287,11 +294,11 @@ __global__ __launch_bounds__(MOE_THREADS, 2) void moe_grouped_kernel(MoeArgs a) 
   constexpr int APT = SEG_M * 32 / MOE_THREADS;                         // activation pieces per thread per step (4)
   constexpr int NCOLS = GLU ? SLAB / 2 : SLAB;                          // output columns per workgroup
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint8_t* a_lds = smem;                                              // [32][A_STRIDE]
-  uint8_t* b_lds = a_lds + SEG_M * A_STRIDE;                          // [128][LBPB]
-  uint8_t* h_lds = b_lds + SLAB * G::LBPB;                            // [32][32] X halves
-  uint16_t* d_lds = reinterpret_cast<uint16_t*>(h_lds + SEG_M * 32);  // [128]
-  int* pair_lds = reinterpret_cast<int*>(d_lds + SLAB);               // [32] output row of each segment slot, -1 = none
+  // two stages of: activations [32][A_STRIDE] | wire [128][LBPB] | X halves [32][32] | side-channel d [128]
+  constexpr int B_OFF = SEG_M * A_STRIDE, H_OFF = B_OFF + SLAB * G::LBPB, D_OFF = H_OFF + SEG_M * 32;
+  constexpr int STAGE = D_OFF + SLAB * 2;
+  static_assert(STAGE % 16 == 0, "stages keep 16-byte alignment");
+  int* pair_lds = reinterpret_cast<int*>(smem + MOE_STAGES * STAGE);  // [32] output row of each segment slot, -1 = none
   float* rs_lds = reinterpret_cast<float*>(pair_lds + SEG_M);         // [32]
 
   const int seg_id = blockIdx.y;
@@ -384,40 +391,57 @@ __global__ __launch_bounds__(MOE_THREADS, 2) void moe_grouped_kernel(MoeArgs a) 
     if constexpr (G::SIDE_D) dreg = *reinterpret_cast<const uint16_t*>(d_src + (size_t)sb * G::BPB);
     if constexpr (G::MINS) hreg = *reinterpret_cast<const u32x4*>(a.xhl + h_goff + (size_t)sb * 16);
   };
-  auto park = [&]() {
+  auto park = [&](uint8_t* stage) {
     StaticFor<APT>::run([&](auto t) {
       constexpr int T = decltype(t)::value;
-      *reinterpret_cast<u32x4*>(a_lds + (a_slot + 8 * T) * A_STRIDE + 16 * a_pc) = areg[T];
+      *reinterpret_cast<u32x4*>(stage + (a_slot + 8 * T) * A_STRIDE + 16 * a_pc) = areg[T];
     });
     StaticFor<WPT>::run([&](auto t) {
       constexpr int T = decltype(t)::value;
-      if (w_loff[T] != 0xffffffffu) *reinterpret_cast<u32x4*>(b_lds + w_loff[T]) = wreg[T];
+      if (w_loff[T] != 0xffffffffu) *reinterpret_cast<u32x4*>(stage + B_OFF + w_loff[T]) = wreg[T];
     });
     if constexpr (G::MINS) {
-      if (tid < 64) *reinterpret_cast<u32x4*>(h_lds + 16 * tid) = hreg;
+      if (tid < 64) *reinterpret_cast<u32x4*>(stage + H_OFF + 16 * tid) = hreg;
     }
     if constexpr (G::SIDE_D) {
-      if (tid < SLAB) d_lds[tid] = dreg;
+      if (tid < SLAB) reinterpret_cast<uint16_t*>(stage + D_OFF)[tid] = dreg;
     }
   };
 
   f32x16 acc[1] = {f32x16{0}};
-  const uint8_t* b_lane = b_lds + (wave * 32 + l32) * G::LBPB;
-  const uint8_t* a_lane = a_lds + l32 * A_STRIDE + 32 * kg;
-  const uint8_t* h_lane = h_lds + l32 * 32 + 16 * kg;
+  auto multiply = [&](const uint8_t* stage) {
+    const uint16_t d_side = G::SIDE_D ? reinterpret_cast<const uint16_t*>(stage + D_OFF)[wave * 32 + l32] : (uint16_t)0;
+    superblock_mma<C, 1>(stage + B_OFF + (wave * 32 + l32) * G::LBPB, d_side, kg, stage + l32 * A_STRIDE + 32 * kg, 0,
+                        stage + H_OFF + l32 * 32 + 16 * kg, 0, acc);
+  };
 
   issue(0);
-  for (int sb = 0; sb < nsb; sb++) {
-    if (sb > 0) lds_barrier();  // everyone is done reading the previous step
-    park();
-    if (sb + 1 < nsb) issue(sb + 1);
+  if constexpr (MOE_STAGES == 2) {
+    // step sb + 1 is parked into the idle stage while step sb is multiplied; one barrier per step
+    park(smem);
+    if (nsb > 1) issue(1);
     lds_barrier();
-    superblock_mma<C, 1>(b_lane, G::SIDE_D ? d_lds[wave * 32 + l32] : (uint16_t)0, kg, a_lane, 0, h_lane, 0, acc);
+    for (int sb = 0; sb < nsb; sb++) {
+      if (sb + 1 < nsb) {
+        park(smem + ((sb + 1) & 1) * STAGE);
+        if (sb + 2 < nsb) issue(sb + 2);
+      }
+      multiply(smem + (sb & 1) * STAGE);
+      lds_barrier();
+    }
+  } else {
+    for (int sb = 0; sb < nsb; sb++) {
+      if (sb > 0) lds_barrier();  // everyone is done reading the previous step
+      park(smem);
+      if (sb + 1 < nsb) issue(sb + 1);
+      lds_barrier();
+      multiply(smem);
+    }
   }
 
   // ---- epilogue: undo the activation scale, (GLU: combine gate and up,) round once, scatter rows
   if constexpr (GLU) {
-    lds_barrier();  // the step buffers are free: reuse them for the up accumulators
+    if constexpr (MOE_STAGES == 1) lds_barrier();  // the step buffers are free: reuse them for the up accumulators
     float* ex = reinterpret_cast<float*>(smem);  // [2 column blocks][16][64]
     const int nb = wave >> 1;
     if (wave & 1) {
@@ -492,7 +516,7 @@ int launch_grouped(const MoeArgs& a, int P, int E, hipStream_t s) {
   const int ntiles = (a.N + NCOLS - 1) / NCOLS;
   int maxseg = E + P / SEG_M;  // sum over experts of ceil(c_e / 32) <= E + P / 32
   if (maxseg > P) maxseg = P;
-  const size_t lds = SEG_M * A_STRIDE + SLAB * G::LBPB + SEG_M * 32 + SLAB * 2 + SEG_M * 8;
+  const size_t lds = (size_t)MOE_STAGES * (SEG_M * A_STRIDE + SLAB * G::LBPB + SEG_M * 32 + SLAB * 2) + SEG_M * 8;
   auto kern = moe_grouped_kernel<C, DT, GLU>;
   hipLaunchKernelGGL(kern, dim3(ntiles, maxseg), dim3(MOE_THREADS), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
