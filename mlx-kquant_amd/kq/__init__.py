@@ -206,9 +206,35 @@ def _expand_geometry(op, x, w, kquant_type, transpose):
     return cid, inner, outer
 
 
+class _QuantizedMatmulFn(torch.autograd.Function):
+    """Gradient with respect to the activations only (the wire bytes are a frozen base): d/dx (x @ W.T) =
+    dy @ W, the same op with `transpose` flipped.  Mirrors KQuantMatmul::vjp, src/kquant_matmul.cpp:1166-1195."""
+
+    @staticmethod
+    def forward(ctx, x, w, kquant_type, transpose, stream):
+        ctx.save_for_backward(w)
+        ctx.meta = (kquant_type, bool(transpose), stream, x.dtype)
+        return _quantized_matmul_impl(x, w, kquant_type, transpose, stream)
+
+    @staticmethod
+    def backward(ctx, dy):
+        (w,) = ctx.saved_tensors
+        kquant_type, transpose, stream, x_dtype = ctx.meta
+        dx = _quantized_matmul_impl(dy, w, kquant_type, not transpose, stream)
+        return dx.to(x_dtype), None, None, None, None
+
+
 def quantized_matmul(x, w, scales, kquant_type, transpose=True, *, stream=None):
     """y = x @ W.T (transpose) or x @ W.  Output dtype = x dtype, float32 promoted to bfloat16 (the
-    activations themselves are cast first).  Mirrors quantized_matmul, src/kquant_ops.cpp:112-183."""
+    activations themselves are cast first).  Differentiable with respect to x (a frozen quantized layer passes
+    gradients to what sits upstream of it, e.g. a LoRA adapter).  Mirrors quantized_matmul,
+    src/kquant_ops.cpp:112-183."""
+    if torch.is_grad_enabled() and x.requires_grad:
+        return _QuantizedMatmulFn.apply(x, w, kquant_type, transpose, stream)
+    return _quantized_matmul_impl(x, w, kquant_type, transpose, stream)
+
+
+def _quantized_matmul_impl(x, w, kquant_type, transpose, stream):
     op = "quantized_matmul"
     if w.dtype != torch.uint8:
         raise ValueError("[kq.quantized_matmul] w must be uint8 (raw GGUF wire bytes).")
@@ -275,13 +301,50 @@ def _default_indices(t):
     return torch.arange(total, dtype=torch.int64, device=t.device).reshape(shape)
 
 
+class _GatherQmmFn(torch.autograd.Function):
+    """Gradient with respect to x only: every entry's dy[i] @ W[rhs[i]] (the op with `transpose` flipped, one
+    cotangent batch per entry) is scatter-added, in float32, into the batch of x that lhs[i] names.
+    Mirrors KQuantGatherQMM::vjp, src/kquant_gather.cpp:748-812."""
+
+    @staticmethod
+    def forward(ctx, x, w, kquant_type, lhs_indices, rhs_indices, transpose, sorted_indices, stream):
+        ctx.save_for_backward(w, lhs_indices, rhs_indices)
+        ctx.meta = (kquant_type, bool(transpose), stream, x.dtype, tuple(x.shape))
+        return _gather_qmm_impl(x, w, kquant_type, lhs_indices, rhs_indices, transpose, sorted_indices, stream)
+
+    @staticmethod
+    def backward(ctx, dy):
+        w, lhs_indices, rhs_indices = ctx.saved_tensors
+        kquant_type, transpose, stream, x_dtype, x_shape = ctx.meta
+        M, K = x_shape[-2], x_shape[-1]
+        nb = 1
+        for d in x_shape[:-2]:
+            nb *= d
+        lhs = lhs_indices if lhs_indices is not None else \
+            torch.arange(nb, dtype=torch.int64, device=dy.device).reshape(x_shape[:-2])
+        rhs = rhs_indices if rhs_indices is not None else _default_indices(w)
+        lhs, rhs = torch.broadcast_tensors(lhs, rhs)
+        B = lhs.numel()
+        g = _gather_qmm_impl(dy.reshape(B, M, dy.shape[-1]), w, kquant_type, None, rhs.reshape(B), not transpose, False,
+                             stream)
+        dx = torch.zeros((nb, M, K), dtype=torch.float32, device=dy.device)
+        dx.index_add_(0, lhs.reshape(B).to(torch.int64), g.to(torch.float32))
+        return dx.reshape(x_shape).to(x_dtype), None, None, None, None, None, None, None
+
+
 def gather_qmm(x, w, scales, kquant_type, lhs_indices=None, rhs_indices=None, transpose=True,
                sorted_indices=False, *, stream=None):
-    """out[i] = x[lhs[i]] @ W[rhs[i]].T; out shape = broadcast(lhs, rhs).shape + [M, N].
-    Mirrors gather_qmm, src/kquant_ops.cpp:293-420."""
-    op = "gather_qmm"
+    """out[i] = x[lhs[i]] @ W[rhs[i]].T; out shape = broadcast(lhs, rhs).shape + [M, N].  Differentiable with
+    respect to x.  Mirrors gather_qmm, src/kquant_ops.cpp:293-420."""
     if lhs_indices is None and rhs_indices is None:
         return quantized_matmul(x, w, scales, kquant_type, transpose, stream=stream)
+    if torch.is_grad_enabled() and x.requires_grad:
+        return _GatherQmmFn.apply(x, w, kquant_type, lhs_indices, rhs_indices, transpose, sorted_indices, stream)
+    return _gather_qmm_impl(x, w, kquant_type, lhs_indices, rhs_indices, transpose, sorted_indices, stream)
+
+
+def _gather_qmm_impl(x, w, kquant_type, lhs_indices, rhs_indices, transpose, sorted_indices, stream):
+    op = "gather_qmm"
     if w.dtype != torch.uint8:
         raise ValueError("[kq.gather_qmm] w must be uint8 (raw GGUF wire bytes).")
     _codec(op, kquant_type)
