@@ -245,6 +245,13 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
                                            codec, dtype, s);
     if (rct != KQ_ERR_UNSUPPORTED) return rct;
   }
+  {
+    // legacy / IQ / fp4 stacks, one row per entry: the code-level skinny kernel, one entry per grid row
+    const int rcc = kq_launch_codes_gather(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
+                                  nullptr, nullptr, out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0,
+                                  0, 0.f, 0.f, codec, dtype, s);
+    if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
+  }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
                                   nullptr, nullptr, out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0,
                                   0, 0.f, 0.f, codec, dtype, s);
@@ -343,6 +350,14 @@ int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_
                                            static_cast<hipStream_t>(stream));
     if (rct != KQ_ERR_UNSUPPORTED) return rct;
   }
+  {
+    // legacy / IQ / fp4 stacks, one row per entry: the code-level skinny kernel, one entry per grid row
+    const int rcc = kq_launch_codes_gather(x_dev, static_cast<const uint8_t*>(gate_w_dev),
+                                  static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, gate_bias_dev, up_bias_dev,
+                                  out_dev, T * R, 1, N, K, R, K, estride, 1, act, limit, alpha, codec, dtype,
+                                  static_cast<hipStream_t>(stream));
+    if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
+  }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(gate_w_dev),
                                   static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, gate_bias_dev, up_bias_dev,
                                   out_dev, T * R, 1, N, K, R, K, estride, 1, act, limit, alpha, codec, dtype,
@@ -371,6 +386,13 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
                                            T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype,
                                            static_cast<hipStream_t>(stream));
     if (rct != KQ_ERR_UNSUPPORTED) return rct;
+  }
+  {
+    // legacy / IQ / fp4 stacks, one row per entry: the code-level skinny kernel, one entry per grid row
+    const int rcc = kq_launch_codes_gather(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, bias_dev,
+                                  nullptr, out_dev, T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype,
+                                  static_cast<hipStream_t>(stream));
+    if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
   }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, bias_dev,
                                   nullptr, out_dev, T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype,
@@ -439,6 +461,12 @@ int kq_gather_qmm_seg(const void* x_dev, const void* w_dev, const uint32_t* map_
   const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, row_expert, out_dev,
                                          (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype, s);
   if (rct != KQ_ERR_UNSUPPORTED) return rct;
+  {
+    // legacy / IQ / fp4 stacks, one row per entry: the code-level skinny kernel, one entry per grid row
+    const int rcc = kq_launch_codes_gather(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, row_expert, nullptr,
+                                  nullptr, out_dev, (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype, s);
+    if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
+  }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, row_expert, nullptr,
                                   nullptr, out_dev, (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype, s);
 }

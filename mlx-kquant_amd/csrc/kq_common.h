@@ -116,6 +116,10 @@ int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, cons
 // Helpers of the slot-mixing ops: idx [T][S-1] -> idx2 [T][S] (last slot = expert 0), and
 // out[t][n] = T(sum_s scores[t][s] * yf[t][s][n]).
 int kq_launch_pad_idx(const uint32_t* idx, uint32_t* idx2, int T, int S, hipStream_t s);
+int kq_launch_codes_gather(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs, const uint32_t* rhs,
+                           const float* bias, const float* bias2, void* out, int B, int M, int N, int K, int x_div,
+                           int64_t x_batch_stride, int64_t w_expert_stride, int glu, int act, float limit, float alpha,
+                           int codec, int dtype, hipStream_t s);
 bool kq_encode_dev_supported(int codec);
 int kq_launch_encode(const void* w, int dtype, const float* im, uint8_t* wire, int64_t rows, int64_t K, int codec,
                      hipStream_t s);
