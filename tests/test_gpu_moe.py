@@ -301,3 +301,30 @@ def test_moe_validation_errors(kq):
         kq.gather_qmv_kq(x, w, "q4_k", idx)
     with pytest.raises(ValueError):
         kq.gather_qmv_kq(x.reshape(3, 1, K).expand(3, 2, K), w, "q4_k", idx, bias=torch.zeros((E, N), device=d))
+
+
+@pytest.mark.parametrize("codec", ["q4_1", "q5_0", "iq4_nl", "iq2_s", "iq1_m", "mxfp4", "nvfp4"])
+def test_moe_decode_entries_ragged_shapes(kq, codec):
+    """One-row entries of the legacy / IQ / fp4 codecs (MoE decode): N that is no multiple of the 16- / 32-column
+    tiles, K that is no multiple of 256 where the codec allows, repeated experts, both half dtypes; then
+    gather_qmm with lhs indices that pick rows out of order."""
+    wpb = O.geometry(codec)[0]
+    E, N, T, R = 5, 72, 2, 3
+    K = 320 if wpb == 32 else 384 if wpb == 64 else 512
+    gate = _stack(codec, E, N, K, seed=71)
+    up = _stack(codec, E, N, K, seed=72)
+    idx = np.array([[4, 0, 4], [1, 1, 3]])
+    for dtype in ("float16", "bfloat16"):
+        xb, xt = make_x((T, K), dtype, seed=73, scale=0.1)
+        for act in ("silu", "gelu"):
+            got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act=act)
+            want = _glu_truth(codec, xb, gate, up, idx, act, dtype=dtype)
+            assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype, act)
+        hb, ht = make_x((T, R, K), dtype, seed=74, scale=0.1)
+        got = kq.gather_qmv_kq(ht, wire_to_dev(gate), codec, _idx_dev(idx))
+        assert rel_l2(dev_to_bits(got), O.gather_qmv(hb, gate, codec, idx, None, dtype), dtype) <= TOL, (codec, dtype)
+    xb, xt = make_x((6, 1, K), "float16", seed=75, scale=0.1)
+    lhs, rhs = np.array([5, 0, 3, 3, 1]), np.array([2, 2, 0, 4, 1])
+    got = kq.gather_qmm(xt, wire_to_dev(gate), None, codec, lhs_indices=_idx_dev(lhs), rhs_indices=_idx_dev(rhs))
+    want = O.gather_qmm(xb, gate, codec, lhs, rhs, True, "float16")
+    assert rel_l2(dev_to_bits(got), want, "float16") <= TOL, codec
