@@ -14,7 +14,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "lib", "libkq.so")
 BLOB = os.path.join(HERE, "data", "kq_iq_grids.bin")
 
-# (source, extra flags).  kq_generic.hip holds the bit-exact decoders: no FMA contraction.
+# (source, extra flags[, object name]).  kq_generic.hip holds the bit-exact decoders: no FMA contraction.
 SOURCES = [
     ("kq_api.cpp", ["-x", "hip"]),
     ("kq_encode.cpp", ["-x", "hip"]),
@@ -23,7 +23,10 @@ SOURCES = [
     ("kq_gemm.hip", []),
     ("kq_moe.hip", []),
     ("kq_anymma.hip", ["-ffp-contract=off"]),
-    ("kq_codes.hip", []),
+    # one source, three objects: its kernel families are instantiated in parallel
+    ("kq_codes.hip", ["-DKQ_CODES_PART=1"], "kq_codes_dense"),
+    ("kq_codes.hip", ["-DKQ_CODES_PART=2"], "kq_codes_gather"),
+    ("kq_codes.hip", ["-DKQ_CODES_PART=3"], "kq_codes_grouped"),
     ("kq_router.hip", ["-ffp-contract=off"]),
     # the device encoder must round exactly like the host one: no fused multiply-adds
     ("kq_encode_dev.hip", ["-ffp-contract=off"]),
@@ -44,8 +47,8 @@ def _hipcc():
 
 
 def _compile(item):
-    src, extra = item
-    out = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    src, extra = item[0], item[1]
+    out = os.path.join(OBJ, (item[2] if len(item) > 2 else os.path.splitext(src)[0]) + ".o")
     cmd = [_hipcc()] + COMMON + extra + ["-c", os.path.join(CSRC, src), "-o", out]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     log = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
@@ -59,7 +62,7 @@ def _compile(item):
 def build_all(verbose=True):
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(os.path.dirname(LIB), exist_ok=True)
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=6) as ex:
         objs = list(ex.map(_compile, SOURCES))
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

@@ -1018,6 +1018,9 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 }  // namespace
 
 // kq_moe.hip
+// The three launcher groups below can be compiled into separate objects (KQ_CODES_PART = 1 dense, 2 gathered,
+// 3 grouped; unset = all) so that the build instantiates their kernels in parallel.
+#if !defined(KQ_CODES_PART) || KQ_CODES_PART == 3
 int kq_launch_moe_sort(const uint32_t* idx, int P, int E, void* order, void* segs, void* nseg, hipStream_t s);
 
 bool kq_codes_moe_supported(int P, int E, int N, int K, int codec) {
@@ -1078,6 +1081,9 @@ int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, cons
   return KQ_ERR_UNSUPPORTED;
 }
 
+#endif  // grouped
+
+#if !defined(KQ_CODES_PART) || KQ_CODES_PART == 1
 bool kq_codes_supported(int M, int N, int K, int codec) {
   if (codec < KQ_Q4_0 || codec >= KQ_NUM_CODECS) return false;  // the K-quants have their own kernels
   return M > 0 && M <= CK_MAXM && N > 0 && K > 0 && K % kq_geom(codec).wpb == 0;
@@ -1108,6 +1114,9 @@ int kq_launch_codes_skinny(const void* x, const uint8_t* w, const void* bias, vo
   return KQ_ERR_UNSUPPORTED;
 }
 
+#endif  // dense
+
+#if !defined(KQ_CODES_PART) || KQ_CODES_PART == 2
 // Gathered calls of up to a few entries (MoE decode): one activation row per entry (M = 1), the entry's expert
 // matrix, optional f32 biases; glu != 0 runs gate and up stacks and the fused epilogue.
 // (q8_0 stays on the plain vector kernel: int8 -> f32 costs it next to nothing, and it measured 9.1 / 8.4 us
@@ -1156,3 +1165,4 @@ int kq_launch_codes_gather(const void* x, const uint8_t* w, const uint8_t* w2, c
   }
   return KQ_ERR_UNSUPPORTED;
 }
+#endif  // gathered
