@@ -15,7 +15,8 @@ beforehand, so a step is the library call and nothing else.
 Extra fields: `sweep` (the decode projections of the q4_k_m recipe at M in {1,2,4,8}), `prefill`
 (q4_k / q5_k / q6_k GEMM 8192 -> 28672 at M in {512, 2048}), `moe` (128 experts, top-8, hidden 2048,
 intermediate 768: fused gate/up GLU in q4_k and down in q6_k at 1 and 256 tokens), `lowbit` (M=1
-GEMV 8192 -> 8192 in the low-bit codecs), `dequantize` (whole-matrix decode to f16, wire bytes in plus
+GEMV 8192 -> 8192 in the low-bit codecs), `moe_decode_lowbit` (1 token, 8 of 128 experts, IQ / mxfp4 stacks),
+`dequantize` (whole-matrix decode to f16, wire bytes in plus
 2 N K bytes out), `roofline` for the dominant kernel and `cpu_baseline`
 (the CPU oracle timed on this box's host cores on the headline GEMV).
 """
@@ -384,6 +385,26 @@ def main():
                             "down_gbs": round(ne * mbytes / (td * 1e-3) / 1e9, 1),
                             "note": "grouped code-level MFMA kernel (biases, swiglu_clamp), timed through the Python wrapper"}
         del gate, up, down
+
+        # ---------------- MoE decode (1 token, 8 of 128 experts of 2048 <-> 768) in the low-bit / fp4 codecs
+        E, H, I, TOPK = 128, 2048, 768, 8
+        dec = []
+        for c in ("iq4_xs", "iq3_s", "iq2_xxs", "mxfp4"):
+            gate = synth_wire_torch(c, E * I, H, 31, dev).reshape(E, I, -1)
+            up = synth_wire_torch(c, E * I, H, 32, dev).reshape(E, I, -1)
+            down = synth_wire_torch(c, E * H, I, 33, dev).reshape(E, H, -1)
+            calls_g, calls_d = [], []
+            for r in range(16):  # 16 routings rotated per step
+                ix = torch.randperm(E, device=dev, generator=gx)[:TOPK].reshape(1, TOPK).to(torch.int32)
+                calls_g.append(abi.moe_glu(randx((1, H), 0.5), gate, up, c, ix)[0])
+                calls_d.append(abi.gather_qmv(randx((1, TOPK, I), 0.5), down, c, ix))
+            tg, _ = time_calls(torch, calls_g, 200, 20)
+            td, _ = time_calls(torch, calls_d, 200, 20)
+            bg, bd = TOPK * 2 * I * kq.bytes_per_row(c, H), TOPK * H * kq.bytes_per_row(c, I)
+            dec.append({"codec": c, "tokens": 1, "experts": TOPK, "glu_us": round(tg * 1e3, 2), "down_us": round(td * 1e3, 2),
+                        "glu_gbs": round(bg / (tg * 1e-3) / 1e9, 1), "down_gbs": round(bd / (td * 1e-3) / 1e9, 1)})
+            del gate, up, down, calls_g, calls_d
+        out["moe_decode_lowbit"] = dec
 
         # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (all five minted by kq.quantize)
         lowbit = []
