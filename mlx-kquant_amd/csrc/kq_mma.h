@@ -174,6 +174,9 @@ __device__ __forceinline__ void superblock_mma(const uint8_t* __restrict__ b_lan
   f32x16 part[MT];
   if constexpr (C == KQ_Q4_K || C == KQ_Q5_K) {
     const uint32_t mask_lo = opaque_sgpr(0x000f000fu), mask_hi = opaque_sgpr(0x00f000f0u);
+    const uint32_t mask5_lo = opaque_sgpr(0x00100010u), mask5_hi = opaque_sgpr(0x01000100u);
+    (void)mask5_lo;
+    (void)mask5_hi;
     const uint4 hdr = *reinterpret_cast<const uint4*>(b_lane);
     const float d = kq::h2f((uint16_t)(hdr.x & 0xffff));
     const float dmin32 = kq::h2f((uint16_t)(hdr.x >> 16)) * 32.0f;
@@ -208,31 +211,33 @@ __device__ __forceinline__ void superblock_mma(const uint8_t* __restrict__ b_lan
       const _Float16 off = (_Float16)(-(h ? 64.0f : 1024.0f) * scf);
       const f16x2 scp = {sch, sch}, offp = {off, off};
       const uint32_t mask = h ? mask_hi : mask_lo;
-      const uint32_t fr[4] = {(qw[2 * s] & mask) | magic, ((qw[2 * s] >> 8) & mask) | magic,
-                              (qw[2 * s + 1] & mask) | magic, ((qw[2 * s + 1] >> 8) & mask) | magic};
+      uint32_t fr[4] = {(qw[2 * s] & mask) | magic, ((qw[2 * s] >> 8) & mask) | magic,
+                        (qw[2 * s + 1] & mask) | magic, ((qw[2 * s + 1] >> 8) & mask) | magic};
+      if constexpr (C == KQ_Q5_K) {
+        // fifth bit of weight (j, i) is bit j of qh[i]; this lane's bytes are qh[16 kg + 8 s + 0..7].  It joins the
+        // code before the conversion: bit 4 next to a low nibble (1024 + q + 16 b), bit 8 next to a high nibble
+        // held in place (1024 + 16 (q + 16 b)); both stay below 2048, so the operand is still exact.
+        constexpr int P = h ? 8 : 4;
+        const uint32_t mbit = h ? mask5_hi : mask5_lo;
+        auto place = [&](uint32_t word, int from) -> uint32_t {  // bits `from`, `from + 16` -> P, P + 16
+          return from >= P ? word >> (from - P) : word << (P - from);
+        };
+        fr[0] |= place(hb[2 * s], j) & mbit;
+        fr[1] |= place(hb[2 * s], j + 8) & mbit;
+        fr[2] |= place(hb[2 * s + 1], j) & mbit;
+        fr[3] |= place(hb[2 * s + 1], j + 8) & mbit;
+      }
       f16x2 bq[4];
 #pragma unroll
       for (int e = 0; e < 4; e++)  // one rounding: (1024 + q) * sc - 1024 * sc = sc * q exactly
         bq[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fr[e]), scp, offp);
-      if constexpr (C == KQ_Q5_K) {
-        // fifth bit of weight (j, i) is bit j of qh[i]; this lane's bytes are qh[16 kg + 8 s + 0..7]
-        const _Float16 s16 = (_Float16)(16.0f * scf);
-        const uint32_t hwa = hb[2 * s] >> j, hwb = hb[2 * s + 1] >> j;
-        const _Float16 z = (_Float16)0.f;
-        const f16x2 add[4] = {{(hwa & 1) ? s16 : z, (hwa & 0x10000) ? s16 : z},
-                              {(hwa & 0x100) ? s16 : z, (hwa & 0x1000000) ? s16 : z},
-                              {(hwb & 1) ? s16 : z, (hwb & 0x10000) ? s16 : z},
-                              {(hwb & 0x100) ? s16 : z, (hwb & 0x1000000) ? s16 : z}};
-#pragma unroll
-        for (int e = 0; e < 4; e++) bq[e] += add[e];
-      }
       return f16x8{bq[0][0], bq[0][1], bq[1][0], bq[1][1], bq[2][0], bq[2][1], bq[3][0], bq[3][1]};
     };
     // 16 MFMA groups, software-pipelined: while the matrix core runs the MFMAs of group it, the wave decodes
     // the B fragment of group it + 1 and requests its activation fragments.  A wave issues in order and a
     // second MFMA waits for the first to leave the matrix core, so vector work placed AFTER a run of MFMAs
     // would idle behind them; the group barriers below interleave it between them instead.
-    constexpr int DEC_VALU = C == KQ_Q5_K ? 30 : 14;  // vector instructions of one decode, roughly
+    constexpr int DEC_VALU = C == KQ_Q5_K ? 22 : 14;  // vector instructions of one decode, roughly
     bfr[0] = decode(std::integral_constant<int, 0>{});
     __builtin_amdgcn_sched_barrier(0);  // group 0's own fragments and decode stay out of the pipelined region
     StaticFor<16>::run([&](auto itc) {
