@@ -328,3 +328,20 @@ def test_moe_decode_entries_ragged_shapes(kq, codec):
     got = kq.gather_qmm(xt, wire_to_dev(gate), None, codec, lhs_indices=_idx_dev(lhs), rhs_indices=_idx_dev(rhs))
     want = O.gather_qmm(xb, gate, codec, lhs, rhs, True, "float16")
     assert rel_l2(dev_to_bits(got), want, "float16") <= TOL, codec
+
+
+@pytest.mark.parametrize("codec", ["q8_0", "q4_k"])
+def test_rhs_gather_more_than_32767_rows(kq, codec):
+    """A single sorted gather of 33000 one-row entries (more than a 16-bit row count, no multiple of any tile),
+    long uneven per-expert runs: every row against the oracle (reference tests/test_gather.py:197-250)."""
+    E, N, K, B = 8, 64, 256, 33000
+    wire = _stack(codec, E, N, K, seed=81)
+    rng = np.random.default_rng(82)
+    rhs = np.sort(rng.integers(0, E, B))
+    xb, xt = make_x((B, 1, K), "float16", seed=83, scale=0.1)
+    got = kq.gather_qmm(xt, wire_to_dev(wire), None, codec, rhs_indices=_idx_dev(rhs), sorted_indices=True)
+    assert tuple(got.shape) == (B, 1, N)
+    want = O.gather_qmm(xb, wire, codec, np.arange(B), rhs, True, "float16")
+    gb = dev_to_bits(got)
+    assert rel_l2(gb, want, "float16") <= TOL
+    assert rel_l2(gb[:64], want[:64], "float16") <= TOL and rel_l2(gb[-64:], want[-64:], "float16") <= TOL
