@@ -32,7 +32,6 @@ typedef u32x4 u32x4_a1 __attribute__((aligned(1)));  // the hardware serves unal
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int CK_WAVES = 8;          // waves per workgroup: they share 32 weight rows and split K
-constexpr int CK_THREADS = 64 * CK_WAVES;
 constexpr int CK_STEP = 256;         // weights of K per step
 constexpr int XA_STRIDE = 512 + 32;  // bytes per activation row of one step in LDS (rows 8 banks apart)
 constexpr int CK_MAXM = 8;
@@ -373,8 +372,19 @@ __device__ __forceinline__ void wave_sync() {
 // GMODE 0: one dense matrix.  GMODE 1: gathered, one (activation row, expert matrix) item per blockIdx.y.
 // GMODE 2: gathered GLU: the tile's 32 rows are 16 gate rows and the same 16 up rows, the epilogue act(g) * u runs
 // on the reduced sums before the single rounding.
+// Dense launches use 8 waves.  Gathered launches (many small workgroups, short K) need the whole grid resident at
+// once: the codecs whose kernel stays under 128 registers get there with 8 waves (two workgroups per CU), the
+// others use 4-wave workgroups (iq4_xs 11.9 + 8.9 -> 10.3 + 6.3 us for the GLU + down of 8 experts of 768 x 2048;
+// iq1_s went the other way, 6.8 + 5.0 -> 8.1 + 5.8 us, hence the split).
+template <int C, int GMODE>
+constexpr int ck_waves() {
+  constexpr bool small = C == KQ_IQ2_XXS || C == KQ_IQ2_XS || C == KQ_IQ2_S || C == KQ_IQ1_S || C == KQ_IQ1_M;
+  return (GMODE && !small) ? 4 : CK_WAVES;
+}
+
 template <int C, int DT, int MB, int GMODE>
-__global__ __launch_bounds__(CK_THREADS, 1) void codes_skinny_kernel(CkArgs a) {
+__global__ __launch_bounds__((64 * ck_waves<C, GMODE>()), ((ck_waves<C, GMODE>()) == 4 ? 2 : 1)) void codes_skinny_kernel(CkArgs a) {
+  constexpr int NWAVES = ck_waves<C, GMODE>(), NTHREADS = 64 * NWAVES;
   using G = CodeGeom<C>;
   constexpr int TILE_N = GMODE == 2 ? 16 : 32;  // output columns per workgroup
   constexpr int WPT = (32 * G::PIECES + 63) / 64;  // wire pieces per lane and step
@@ -408,7 +418,7 @@ __global__ __launch_bounds__(CK_THREADS, 1) void codes_skinny_kernel(CkArgs a) {
   if constexpr (G::GRID_N > 0) {
     const uint8_t* src = a.grids + G::GRID_OFF;
     if constexpr (G::GRID_W == 8) {
-      for (int e = tid; e < G::GRID_N; e += CK_THREADS) {
+      for (int e = tid; e < G::GRID_N; e += NTHREADS) {
         const u32x2 v = *reinterpret_cast<const u32x2*>(src + 8 * e);
         f16x8 f;
         if constexpr (G::GRID_SIGNED)
@@ -418,7 +428,7 @@ __global__ __launch_bounds__(CK_THREADS, 1) void codes_skinny_kernel(CkArgs a) {
         *reinterpret_cast<f16x8*>(grid_lds + 16 * e) = f;
       }
     } else {
-      for (int e = tid; e < G::GRID_N; e += CK_THREADS) {
+      for (int e = tid; e < G::GRID_N; e += NTHREADS) {
         const uint32_t v = *reinterpret_cast<const uint32_t*>(src + 4 * e);
         uint32_t ev, od;
         bytes_to_f16(v, 0.f, ev, od);
@@ -542,10 +552,10 @@ __global__ __launch_bounds__(CK_THREADS, 1) void codes_skinny_kernel(CkArgs a) {
   if (lane < CK_MAXM) xs_lds[lane] = 0.f;  // rows past MB keep a zero scale
 
   if (wave < nsteps) issue(wave);
-  for (int st = wave; st < nsteps; st += CK_WAVES) {
+  for (int st = wave; st < nsteps; st += NWAVES) {
     park();
     wave_sync();
-    if (st + CK_WAVES < nsteps) issue(st + CK_WAVES);
+    if (st + NWAVES < nsteps) issue(st + NWAVES);
     const int kvalid = K - CK_STEP * st;
     float sacc[4] = {0.f, 0.f, 0.f, 0.f};
     constexpr int MPS = G::SB / 16;  // MFMAs per scale block
@@ -605,7 +615,7 @@ __global__ __launch_bounds__(CK_THREADS, 1) void codes_skinny_kernel(CkArgs a) {
 
   // ---- the waves' partial sums meet in LDS (the step buffers are free now)
   lds_barrier();
-  float* red = reinterpret_cast<float*>(wave_base);  // [CK_WAVES][4][64]
+  float* red = reinterpret_cast<float*>(wave_base);  // [NWAVES][4][64]
 #pragma unroll
   for (int i = 0; i < 4; i++) red[(wave * 4 + i) * 64 + lane] = acc[i];
   lds_barrier();
@@ -616,7 +626,7 @@ __global__ __launch_bounds__(CK_THREADS, 1) void codes_skinny_kernel(CkArgs a) {
     for (int i = 0; i < 4; i++) {
       float v = 0.f;
 #pragma unroll
-      for (int w = 0; w < CK_WAVES; w++) v += red[(w * 4 + i) * 64 + lane];
+      for (int w = 0; w < NWAVES; w++) v += red[(w * 4 + i) * 64 + lane];
       const int m = 4 * kg + i;
       if constexpr (GMODE == 0) {
         if (m < M && n < N) {
@@ -631,7 +641,7 @@ __global__ __launch_bounds__(CK_THREADS, 1) void codes_skinny_kernel(CkArgs a) {
       } else {
         float u = 0.f;  // the up row of this column sits 16 lanes further on
 #pragma unroll
-        for (int w = 0; w < CK_WAVES; w++) u += red[(w * 4 + i) * 64 + (lane ^ 16)];
+        for (int w = 0; w < NWAVES; w++) u += red[(w * 4 + i) * 64 + (lane ^ 16)];
         if (l32 < 16 && m < M && l32 < ncols) {
           if (a.fbias) v += a.fbias[(size_t)expert * N + n];
           if (a.fbias2) u += a.fbias2[(size_t)expert * N + n];
@@ -646,8 +656,9 @@ __global__ __launch_bounds__(CK_THREADS, 1) void codes_skinny_kernel(CkArgs a) {
 template <int C, int DT, int MB, int GMODE = 0>
 int launch_codes(const CkArgs& a, hipStream_t s, int items = 1) {
   using G = CodeGeom<C>;
-  size_t lds = (size_t)G::GRID_BYTES + G::SPREAD_BYTES + (size_t)CK_WAVES * wave_lds_bytes<C>(MB);
-  const size_t red = (size_t)G::GRID_BYTES + G::SPREAD_BYTES + CK_WAVES * 4 * 64 * 4;
+  constexpr int NWAVES = ck_waves<C, GMODE>();
+  size_t lds = (size_t)G::GRID_BYTES + G::SPREAD_BYTES + (size_t)NWAVES * wave_lds_bytes<C>(MB);
+  const size_t red = (size_t)G::GRID_BYTES + G::SPREAD_BYTES + NWAVES * 4 * 64 * 4;
   if (lds < red) lds = red;
   auto kern = codes_skinny_kernel<C, DT, MB, GMODE>;
   static bool attr_set = false;
@@ -657,7 +668,7 @@ int launch_codes(const CkArgs& a, hipStream_t s, int items = 1) {
     attr_set = true;
   }
   constexpr int TILE_N = GMODE == 2 ? 16 : 32;
-  hipLaunchKernelGGL(kern, dim3((a.N + TILE_N - 1) / TILE_N, items), dim3(CK_THREADS), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3((a.N + TILE_N - 1) / TILE_N, items), dim3(64 * NWAVES), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }
