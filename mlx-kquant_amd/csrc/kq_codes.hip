@@ -372,19 +372,24 @@ __device__ __forceinline__ void wave_sync() {
 // GMODE 0: one dense matrix.  GMODE 1: gathered, one (activation row, expert matrix) item per blockIdx.y.
 // GMODE 2: gathered GLU: the tile's 32 rows are 16 gate rows and the same 16 up rows, the epilogue act(g) * u runs
 // on the reduced sums before the single rounding.
-// Dense launches use 8 waves.  Gathered launches (many small workgroups, short K) need the whole grid resident at
+// WV = waves per workgroup.  Gathered launches (many small workgroups, short K) need the whole grid resident at
 // once: the codecs whose kernel stays under 128 registers get there with 8 waves (two workgroups per CU), the
 // others use 4-wave workgroups (iq4_xs 11.9 + 8.9 -> 10.3 + 6.3 us for the GLU + down of 8 experts of 768 x 2048;
-// iq1_s went the other way, 6.8 + 5.0 -> 8.1 + 5.8 us, hence the split).
+// iq1_s went the other way, 6.8 + 5.0 -> 8.1 + 5.8 us, hence the split).  Dense launches use 8 waves, except
+// single-row calls of those larger kernels with more row tiles than CUs, where 4-wave workgroups measured 7 - 15 %
+// faster (iq4_xs 128256 x 4096: 127 -> 110 us) and 20 - 40 % slower with fewer tiles.
+template <int C>
+constexpr bool ck_small() {
+  return C == KQ_IQ2_XXS || C == KQ_IQ2_XS || C == KQ_IQ2_S || C == KQ_IQ1_S || C == KQ_IQ1_M;
+}
 template <int C, int GMODE>
 constexpr int ck_waves() {
-  constexpr bool small = C == KQ_IQ2_XXS || C == KQ_IQ2_XS || C == KQ_IQ2_S || C == KQ_IQ1_S || C == KQ_IQ1_M;
-  return (GMODE && !small) ? 4 : CK_WAVES;
+  return (GMODE && !ck_small<C>()) ? 4 : CK_WAVES;
 }
 
-template <int C, int DT, int MB, int GMODE>
-__global__ __launch_bounds__((64 * ck_waves<C, GMODE>()), ((ck_waves<C, GMODE>()) == 4 ? 2 : 1)) void codes_skinny_kernel(CkArgs a) {
-  constexpr int NWAVES = ck_waves<C, GMODE>(), NTHREADS = 64 * NWAVES;
+template <int C, int DT, int MB, int GMODE, int WV>
+__global__ __launch_bounds__((64 * WV), (WV == 4 ? 2 : 1)) void codes_skinny_kernel(CkArgs a) {
+  constexpr int NWAVES = WV, NTHREADS = 64 * NWAVES;
   using G = CodeGeom<C>;
   constexpr int TILE_N = GMODE == 2 ? 16 : 32;  // output columns per workgroup
   constexpr int WPT = (32 * G::PIECES + 63) / 64;  // wire pieces per lane and step
@@ -653,14 +658,13 @@ __global__ __launch_bounds__((64 * ck_waves<C, GMODE>()), ((ck_waves<C, GMODE>()
   }
 }
 
-template <int C, int DT, int MB, int GMODE = 0>
-int launch_codes(const CkArgs& a, hipStream_t s, int items = 1) {
+template <int C, int DT, int MB, int GMODE, int NWAVES>
+int launch_codes_wv(const CkArgs& a, hipStream_t s, int items) {
   using G = CodeGeom<C>;
-  constexpr int NWAVES = ck_waves<C, GMODE>();
   size_t lds = (size_t)G::GRID_BYTES + G::SPREAD_BYTES + (size_t)NWAVES * wave_lds_bytes<C>(MB);
   const size_t red = (size_t)G::GRID_BYTES + G::SPREAD_BYTES + NWAVES * 4 * 64 * 4;
   if (lds < red) lds = red;
-  auto kern = codes_skinny_kernel<C, DT, MB, GMODE>;
+  auto kern = codes_skinny_kernel<C, DT, MB, GMODE, NWAVES>;
   static bool attr_set = false;
   if (!attr_set) {
     KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -671,6 +675,14 @@ int launch_codes(const CkArgs& a, hipStream_t s, int items = 1) {
   hipLaunchKernelGGL(kern, dim3((a.N + TILE_N - 1) / TILE_N, items), dim3(64 * NWAVES), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
+}
+
+template <int C, int DT, int MB, int GMODE = 0>
+int launch_codes(const CkArgs& a, hipStream_t s, int items = 1) {
+  if constexpr (GMODE == 0 && MB == 1 && !ck_small<C>()) {
+    if ((a.N + 31) / 32 > 256) return launch_codes_wv<C, DT, MB, GMODE, 4>(a, s, items);
+  }
+  return launch_codes_wv<C, DT, MB, GMODE, ck_waves<C, GMODE>()>(a, s, items);
 }
 
 template <int C>

@@ -257,3 +257,16 @@ def test_qmm_prefill_gemm_wide_dynamic_range(kq):
     g, w_ = O.bits_to_f32(got, "bfloat16").astype(np.float64), O.bits_to_f32(want, "bfloat16").astype(np.float64)
     rel_rows = np.linalg.norm(g - w_, axis=1) / np.linalg.norm(w_, axis=1)
     assert rel_rows.max() <= TOL, rel_rows.max()
+
+
+@pytest.mark.parametrize("codec", ["iq4_xs", "q8_0", "mxfp4", "iq2_xxs"])
+def test_qmm_single_row_many_row_tiles(kq, codec):
+    """More row tiles than CUs (N = 8300 -> 260 tiles, the last one ragged): single-row calls of the larger
+    code-level kernels switch to 4-wave workgroups there; two rows keep 8 waves."""
+    N, K = 8300, 512 if codec != "mxfp4" else 288
+    wire = _wire(codec, N, K, seed=45)
+    for M in (1, 2):
+        xb, xt = make_x((M, K), "bfloat16", seed=46 + M)
+        got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+        want = O.qmm(xb, wire, codec, True, "bfloat16")
+        assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, M)
