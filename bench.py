@@ -10,7 +10,9 @@ exceeding twice the 256 MB last-level cache, so the weight bytes come from HBM.
 value = quantized weight bytes per step / step time (HIP events on the launching stream).
 
 Every timed call goes through the C ABI of libkq (ctypes) with outputs and workspace allocated
-beforehand, so a step is the library call and nothing else.
+beforehand.  A step is one batch of back-to-back launches (one rotation over the weight copies repeated to
+at least 100 launches), captured once into a HIP graph and replayed, so the host's launch rate does not
+enter the figure; `us_per_launch` = step time / `launches_per_step`.
 
 Extra fields: `sweep` (the decode projections of the q4_k_m recipe at M in {1,2,4,8}), `prefill`
 (q4_k / q5_k / q6_k GEMM 8192 -> 28672 at M in {512, 2048}), `moe` (128 experts, top-8, hidden 2048,
@@ -77,21 +79,81 @@ def quantized_weights(kq, torch, codec, N, K, seed, device, unique_rows=None):
     return wq.to(device)
 
 
-def time_calls(torch, calls, steps, warmup):
-    """Average time (ms) of one call over `steps` calls rotating over the closures in `calls`."""
+def _time_direct(torch, calls, launches, warm):
     n = len(calls)
-    for i in range(warmup):
+    for i in range(warm):
         calls[i % n]()
     torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
-    for i in range(steps):
+    for i in range(launches):
         calls[i % n]()
     ev1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
+    return ev0.elapsed_time(ev1) / launches, wall_ms / launches
+
+
+def capture_batch(torch, calls, batch):
+    """A HIP graph of `batch` launches rotating over the closures in `calls` (each takes the stream to launch on),
+    or None when the calls cannot be captured."""
+    n = len(calls)
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(min(n, batch)):  # first calls outside the capture: one-time setup of the library
+                calls[i](side.cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            st = torch.cuda.current_stream().cuda_stream
+            for i in range(batch):
+                calls[i % n](st)
+        return g
+    except Exception as e:  # noqa: BLE001
+        print(f"bench.py: graph capture unavailable ({e}); timing direct launches", file=sys.stderr)
+        torch.cuda.synchronize()
+        return None
+
+
+def time_graph(torch, g, batch, steps, warmup, settle_ms=30.0):
+    """`warmup` untimed replays (after enough untimed replays to bring the device to its steady clock), then
+    exactly `steps` timed ones between two events.  Returns (ms per replay, wall ms per replay)."""
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    g.replay()
+    ev1.record()
+    torch.cuda.synchronize()
+    one = max(ev0.elapsed_time(ev1), 1e-3)
+    for _ in range(int(min(2000, settle_ms / one)) + warmup):
+        g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        g.replay()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
     return ev0.elapsed_time(ev1) / steps, wall_ms / steps
+
+
+def time_calls(torch, calls, launches, warm, graph=True):
+    """Average time (ms) of one launch over about `launches` back-to-back launches rotating over the closures in
+    `calls`.  The launches are replays of a HIP graph of one rotation (at least 20 launches), so the host's launch
+    rate does not enter; calls that cannot be captured are timed as direct launches."""
+    n = len(calls)
+    batch = n * max(1, -(-20 // n))
+    g = capture_batch(torch, calls, batch) if graph else None
+    if g is None:
+        direct = [(lambda c=c: c(None)) for c in calls] if graph else calls
+        return _time_direct(torch, direct, launches, warm)
+    reps = max(1, -(-launches // batch))
+    ms, wall = time_graph(torch, g, batch, reps, max(1, warm // batch), settle_ms=10.0)
+    return ms / batch, wall / batch
 
 
 class Abi:
@@ -113,11 +175,11 @@ class Abi:
         out = torch.empty((M, N), dtype=x.dtype, device=self.dev)
         nws = lib.kq_qmm_workspace_size(M, N, K, 1, cid, KQ_BF16)
         ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=self.dev)
-        args = (x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, 1, cid, KQ_BF16, ws.data_ptr(), nws, self.stream)
+        args = (x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, 1, cid, KQ_BF16, ws.data_ptr(), nws)
         keep = (x, w, out, ws)
 
-        def call(_keep=keep):
-            rc = lib.kq_qmm(*args)
+        def call(stream=None, _keep=keep):
+            rc = lib.kq_qmm(*args, stream or self.stream)
             if rc:
                 self._check(rc)
         return call
@@ -125,11 +187,11 @@ class Abi:
     def dequantize(self, w, codec, N, K, out):
         lib = self.lib
         cid = lib.kq_codec_id(codec.encode())
-        args = (w.data_ptr(), out.data_ptr(), N * K, cid, 1, self.stream)  # dtype code 1 = float16
+        args = (w.data_ptr(), out.data_ptr(), N * K, cid, 1)  # dtype code 1 = float16
         keep = (w, out)
 
-        def call(_keep=keep):
-            rc = lib.kq_dequantize(*args)
+        def call(stream=None, _keep=keep):
+            rc = lib.kq_dequantize(*args, stream or self.stream)
             if rc:
                 self._check(rc)
         return call
@@ -143,11 +205,11 @@ class Abi:
         nws = lib.kq_moe_workspace_size(T, R, E, N, K, 1, cid, KQ_BF16)
         ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=self.dev)
         args = (x.data_ptr(), gate.data_ptr(), up.data_ptr(), idx.data_ptr(), None, None, out.data_ptr(), T, R, E, N, K,
-                0, 0.0, 0.0, cid, KQ_BF16, ws.data_ptr(), nws, self.stream)
+                0, 0.0, 0.0, cid, KQ_BF16, ws.data_ptr(), nws)
         keep = (x, gate, up, idx, out, ws)
 
-        def call(_keep=keep):
-            rc = lib.kq_moe_glu_gather(*args)
+        def call(stream=None, _keep=keep):
+            rc = lib.kq_moe_glu_gather(*args, stream or self.stream)
             if rc:
                 self._check(rc)
         return call, out
@@ -160,11 +222,11 @@ class Abi:
         nws = lib.kq_moe_workspace_size(T, R, E, N, K, 0, cid, KQ_BF16)
         ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=self.dev)
         args = (h.data_ptr(), w.data_ptr(), idx.data_ptr(), None, out.data_ptr(), T, R, E, N, K, cid, KQ_BF16,
-                ws.data_ptr(), nws, self.stream)
+                ws.data_ptr(), nws)
         keep = (h, w, idx, out, ws)
 
-        def call(_keep=keep):
-            rc = lib.kq_gather_qmv(*args)
+        def call(stream=None, _keep=keep):
+            rc = lib.kq_gather_qmv(*args, stream or self.stream)
             if rc:
                 self._check(rc)
         return call
@@ -198,8 +260,8 @@ def cpu_baseline(wire_np, codec, K, M, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=20, help="timed steps; a step is one batch of >= 100 launches")
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-sweep", action="store_true", help="skip the sweep, prefill, MoE and low-bit sections")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--probe", action="store_true",
@@ -269,13 +331,24 @@ def main():
         print(json.dumps({"probe": "copy then 20 cold GEMV launches", "copy_bytes_each_way": wbytes,
                           "gemv_weight_bytes": wbytes}))
         return
-    ms, wall_ms = time_calls(torch, calls, args.steps, args.warmup)
+    # a step = one rotation over the copies, repeated until it holds at least 100 launches, replayed as one HIP
+    # graph: back-to-back launches on one stream with no host work between them
+    lps = len(calls) * max(1, -(-100 // len(calls)))
+    g = capture_batch(torch, calls, lps)
+    if g is not None:
+        step_ms, wall_step_ms = time_graph(torch, g, lps, args.steps, args.warmup)
+    else:
+        ms1, wall1 = _time_direct(torch, [(lambda c=c: c(None)) for c in calls], lps * args.steps, lps * args.warmup)
+        step_ms, wall_step_ms = ms1 * lps, wall1 * lps
+    ms, wall_ms = step_ms / lps, wall_step_ms / lps
     gbs = wbytes / (ms * 1e-3) / 1e9
-    hot_ms, _ = time_calls(torch, calls[:1], args.steps, args.warmup)
+    hot_ms, _ = time_calls(torch, calls[:1], 2000, 200)
 
     out = {
         "metric": "q4_k GEMV weight-GB/s at M=1 (cold)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6), "higher_is_better": True,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_ms, 6), "launches_per_step": lps,
+        "us_per_launch": round(ms * 1e3, 3), "launch_mode": "hip graph replay" if g is not None else "direct",
+        "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic: seeded N(0,0.02) weights quantized by kq.quantize, N(0,1) bf16 activations",
         "config": {"workload": "decode GEMV, Llama-3-8B gate/up projection 4096->14336, q4_k, M=1, bf16 x, "
@@ -283,7 +356,7 @@ def main():
                    "codec": codec, "M": M, "N": N, "K": K},
         "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
         "hot_gbs": round(wbytes / (hot_ms * 1e-3) / 1e9, 1),
-        "wall_ms_per_step": round(wall_ms, 6),
+        "wall_ms_per_step": round(wall_step_ms, 6),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES},
     }
@@ -291,7 +364,7 @@ def main():
     del copies, calls
 
     if not args.no_sweep:
-        steps, warm = max(50, args.steps // 10), max(10, args.warmup // 10)
+        steps, warm = 400, 40  # launches per shape
         # ---------------- decode sweep (q4_k_m recipe of Llama-3-8B)
         sweep = []
         shapes = [("q_proj", "q4_k", 4096, 4096, True), ("gate/up", "q4_k", 14336, 4096, True),
@@ -373,10 +446,10 @@ def main():
                              alpha=1.702)
         tg, _ = time_calls(torch, [lambda: kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp",
                                                                  limit=7.0, gate_bias=gb, up_bias=ub, alpha=1.702)],
-                           20, 3)
+                           20, 3, graph=False)
         h = kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp", limit=7.0, gate_bias=gb, up_bias=ub,
                                  alpha=1.702)
-        td, _ = time_calls(torch, [lambda: kq.gather_qmv_kq(h, down, "mxfp4", idx, bias=db)], 20, 3)
+        td, _ = time_calls(torch, [lambda: kq.gather_qmv_kq(h, down, "mxfp4", idx, bias=db)], 20, 3, graph=False)
         mbytes = H * kq.bytes_per_row("mxfp4", H)
         ne = int(idx.unique().numel())
         out["moe_mxfp4"] = {"tokens": T, "experts_touched": ne, "glu_us": round(tg * 1e3, 1),

@@ -93,9 +93,10 @@ int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void
  * Process-wide, not thread-safe. */
 void kq_set_gemm_tile_rows(int rows);
 /* Tuning hook without a counterpart in the reference: which skinny-M kernel dense calls use.
- * 0 = default (decoupled-wave kernel up to 4 activation rows, diagonal kernel for 5 - 8),
- * 1 = workgroup-synchronous kernel (the one the gathered ops use), 2 = decoupled-wave kernel always,
- * 3 = decoupled-wave kernel with two-superblock units, 4 = diagonal kernel wherever K allows it.
+ * 0 = default (streamed kernel up to 4 activation rows of q4_k / q5_k / q6_k, else decoupled-wave kernel up to 4
+ * rows and diagonal kernel for 5 - 8), 1 = workgroup-synchronous kernel (the one the gathered ops use),
+ * 2 = decoupled-wave kernel always, 3 = decoupled-wave kernel with two-superblock units, 4 = diagonal kernel
+ * wherever K allows it, 5 = streamed kernel (direct-to-LDS weight loads) wherever it applies.
  * Process-wide, not thread-safe. */
 void kq_set_skinny_variant(int variant);
 

@@ -20,6 +20,7 @@ SOURCES = [
     ("kq_encode.cpp", ["-x", "hip"]),
     ("kq_generic.hip", ["-ffp-contract=off"]),
     ("kq_mfma.hip", []),
+    ("kq_stream.hip", ["-Wno-inline-asm"]),
     ("kq_gemm.hip", []),
     ("kq_moe.hip", []),
     ("kq_anymma.hip", ["-ffp-contract=off"]),
@@ -35,8 +36,20 @@ COMMON = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
     # packed-FP32 VALU forms are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-fno-strict-aliasing",
-    "-I", os.path.join(ROOT, "include"), "-I", CSRC, '-DKQ_GRID_BLOB="%s"' % BLOB,
+    "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-I", OBJ,
 ]
+GRID_INC = os.path.join(OBJ, "kq_iq_grids.inc")
+
+
+def _write_grid_inc():
+    """The IQ codebook data file as a C byte list (initialiser of the __device__ array in kq_api.cpp)."""
+    data = open(BLOB, "rb").read()
+    lines = [",".join(str(b) for b in data[i:i + 32]) + "," for i in range(0, len(data), 32)]
+    text = "\n".join(lines) + "\n"
+    if not os.path.exists(GRID_INC) or open(GRID_INC).read() != text:
+        with open(GRID_INC, "w") as f:
+            f.write(text)
+
 
 
 def _hipcc():
@@ -62,6 +75,7 @@ def _compile(item):
 def build_all(verbose=True):
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(os.path.dirname(LIB), exist_ok=True)
+    _write_grid_inc()
     with ThreadPoolExecutor(max_workers=6) as ex:
         objs = list(ex.map(_compile, SOURCES))
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs

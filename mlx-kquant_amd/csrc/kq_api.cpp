@@ -1,5 +1,5 @@
-// C ABI of libkq (declared in include/kq.h): argument validation, error reporting, per-device
-// codebook upload and routing to the HIP launchers.  Host-only code; compiled by hipcc as C++.
+// C ABI of libkq (declared in include/kq.h): argument validation, error reporting, the device copy of the
+// IQ codebooks and routing to the HIP launchers.  Compiled by hipcc as HIP (the codebooks are a __device__ array).
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -7,15 +7,17 @@
 
 #include "kq_common.h"
 
-// IQ codebook blob linked into .rodata (data file given by -DKQ_GRID_BLOB="...").
-__asm__(".section .rodata\n"
-        ".balign 16\n"
-        ".globl kq_grid_blob_host\n"
-        ".hidden kq_grid_blob_host\n"
-        "kq_grid_blob_host:\n"
-        ".incbin \"" KQ_GRID_BLOB "\"\n"
-        ".previous\n");
-extern "C" const uint8_t kq_grid_blob_host[];
+// IQ codebooks (33,792 bytes of ggml constants) as device-resident storage: part of the code object, so no
+// entry point allocates or copies anything for them.  The initialiser is the data file
+// data/kq_iq_grids.bin written out as a byte list by build.py (kq_iq_grids.inc in the object directory).
+// (not const: a const device array has internal linkage and cannot be looked up by symbol)
+__device__ __attribute__((aligned(16))) uint8_t kq_grid_blob_dev[KQ_GRID_BYTES] = {
+#include "kq_iq_grids.inc"
+};
+// host copy of the same bytes (the host encoders search the codebooks)
+extern "C" __attribute__((visibility("hidden"))) const uint8_t kq_grid_blob_host[KQ_GRID_BYTES] = {
+#include "kq_iq_grids.inc"
+};
 
 namespace {
 
@@ -38,7 +40,7 @@ const kq_codec_info kCodecs[KQ_NUM_CODECS] = {
 
 constexpr int kMaxDevices = 64;
 std::mutex g_grid_mu;
-uint8_t* g_grids[kMaxDevices] = {};
+const uint8_t* g_grids[kMaxDevices] = {};
 
 thread_local KqOutMap g_out_map = {1, 1, 0, 0};
 // Sets the calling thread's output map for the launches inside a scope.
@@ -71,14 +73,14 @@ const uint8_t* kq_device_grids(void) {
   }
   std::lock_guard<std::mutex> lk(g_grid_mu);
   if (!g_grids[dev]) {
-    uint8_t* p = nullptr;
-    e = hipMalloc(reinterpret_cast<void**>(&p), KQ_GRID_BYTES);
-    if (e == hipSuccess) e = hipMemcpy(p, kq_grid_blob_host, KQ_GRID_BYTES, hipMemcpyHostToDevice);
-    if (e != hipSuccess) {
-      kq_set_error(KQ_ERR_HIP, "codebook upload failed: %s", hipGetErrorString(e));
+    // every device holds its own copy of the array at its own address
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(kq_grid_blob_dev));
+    if (e != hipSuccess || !p) {
+      kq_set_error(KQ_ERR_HIP, "codebook lookup failed: %s", hipGetErrorString(e));
       return nullptr;
     }
-    g_grids[dev] = p;  // kept for the life of the process
+    g_grids[dev] = static_cast<const uint8_t*>(p);
   }
   return g_grids[dev];
 }

@@ -78,6 +78,12 @@ int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2,
 size_t kq_qmm_tuned_workspace_bytes(int M, int N, int K, int codec);
 int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                         size_t ws_bytes, hipStream_t s);
+// Streamed skinny kernel (direct-to-LDS weight stream, q4_k / q5_k / q6_k, M <= 4): same fall-through contract.
+// Needs its split-K workspace when its plan splits K (K > 4096 or few row tiles); without it the call is declined.
+bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const void* w);
+size_t kq_stream_workspace_bytes(int M, int N, int K, int codec);
+int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                         size_t ws_bytes, hipStream_t s);
 // Tuned gathered GEMV (items = (activation matrix, expert) pairs, M <= 8 rows each; with glu the
 // gate/up pair and the fused epilogue, M = 1): same fall-through contract as kq_launch_qmm_tuned.
 int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,

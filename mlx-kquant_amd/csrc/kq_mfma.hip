@@ -1207,7 +1207,7 @@ size_t sk_lds_bytes(int rows, int kch, int MB) {
          16 * SK_THREADS + 32 * 16 * 2;
 }
 
-int g_sk_variant = 0;  // kq_set_skinny_variant: 0 default, 1 synchronous, 2 decoupled, 3 two-superblock units, 4 diagonal
+int g_sk_variant = 0;  // kq_set_skinny_variant: 0 default, 1 synchronous, 2 decoupled, 3 two-superblock units, 4 diagonal, 5 streamed
 
 // Split-K plan of a dense call: with few row tiles the K range is cut so that about 768
 // workgroups of full 32-row tiles exist; every split keeps at least one superblock per wave.
@@ -1388,12 +1388,19 @@ bool sk_shape_ok(int M, int K, int codec, const void* x, const void* w, const vo
 size_t kq_qmm_tuned_workspace_bytes(int M, int N, int K, int codec) {
   if (!sk_codec_ok(codec) || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return 0;
   const SkSplit p = sk_split_plan(N, K);
-  return p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
+  const size_t own = p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
+  const size_t st = kq_stream_workspace_bytes(M, N, K, codec);
+  return own > st ? own : st;
 }
 
 int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                         size_t ws_bytes, hipStream_t s) {
   if (!sk_shape_ok(M, K, codec, x, w, nullptr)) return KQ_ERR_UNSUPPORTED;
+  // up to four activation rows of q4_k / q5_k / q6_k: the streamed kernel (variant 5), unless a test pins another
+  if (g_sk_variant == 0 || g_sk_variant == 5) {
+    const int rc = kq_launch_qmm_stream(x, w, y, M, N, K, codec, dtype, ws, ws_bytes, s);
+    if (rc != KQ_ERR_UNSUPPORTED) return rc;
+  }
   SkArgs a{};
   a.x = x;
   a.w = w;
@@ -1402,7 +1409,8 @@ int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, 
   a.N = N;
   a.K = K;
   a.x_div = 1;
-  if (ws_bytes < kq_qmm_tuned_workspace_bytes(M, N, K, codec) || (reinterpret_cast<uintptr_t>(ws) & 3)) ws = nullptr;
+  const SkSplit own = sk_split_plan(N, K);
+  if (ws_bytes < (own.ksplit > 1 ? (size_t)own.ksplit * M * N * sizeof(float) : 0) || (reinterpret_cast<uintptr_t>(ws) & 3)) ws = nullptr;
   return launch_skinny_any<false>(a, 1, codec, dtype, ws, s);
 }
 

@@ -1,0 +1,695 @@
+// Streamed skinny-M (decode) kernel: y[M,N] = x[M,K] . W^T for M <= 4, codecs q4_k / q5_k / q6_k.
+// The weight bytes go HBM -> LDS with direct-to-LDS loads (global_load_lds_dwordx4): no staging
+// registers, no LDS store instructions, and a wave keeps its next units in flight while it works.
+//
+// Mapping.  A workgroup (4 waves) owns tiles of 32 weight rows and a K range of at most 16
+// superblocks; wave w takes superblocks w, w + 4, ... of the range, a "unit" being 32 rows x one
+// superblock.  Workgroups are persistent: tile t of workgroup b is tile b + t * gridDim.x, so the
+// activations are prepared once per workgroup and the weight stream of the next tile is already on
+// its way while the current one is multiplied.
+//
+// Matrix cores.  v_mfma_f32_4x4x4_16b_f16 is sixteen independent 4 x 4 x 4 products: block b = lanes
+// 4 b .. 4 b + 3 multiplies four activation rows (A) by four weight rows (B).  Lane l serves weight
+// row l % 32 and the half kg = l / 32 of the superblock (128 weights), so no two lanes share an
+// accumulator and every lane folds its own block scales.  The eight blocks of a half-wave share one A
+// block (cbsz = 3), picked by the instruction's abid field: one register pair holds the A operands of
+// eight MFMAs, lane (kg, a, i) keeping the four activations that row i needs in MFMA number a.  The
+// activations of a whole unit are 4 (q4_k / q5_k) or 8 (q6_k) such pairs, loaded once per workgroup.
+//
+// Codes.  As in the other tuned kernels a weight enters the matrix core as an exact f16 integer made
+// with one AND-OR (0x6400 | field = 1024 + field, fields masked in place); scales, the 1024 offset and
+// the block minimum are applied in f32 to the per-lane partial sums.
+//
+// Waiting.  The compiler cannot see a direct-to-LDS load land, so these loads are issued from inline
+// assembly and every wait on them is an explicit s_waitcnt vmcnt(n): loads return in order, n is the
+// number of load instructions issued after the unit that is needed.  All other LDS traffic is ordinary
+// code.
+#include <type_traits>
+
+#include "kq_decode.h"
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int ST_WAVES = 4;
+constexpr int ST_THREADS = ST_WAVES * 64;
+constexpr int ST_ROWS = 32;
+constexpr int ST_XU = 4;  // units per wave at most (K range of a workgroup <= 16 superblocks)
+
+template <int N>
+struct SFor {
+  template <class F>
+  __device__ __forceinline__ static void run(F&& f) {
+    SFor<N - 1>::run(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+};
+template <>
+struct SFor<0> {
+  template <class F>
+  __device__ __forceinline__ static void run(F&&) {}
+};
+
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) { return (a & mask) | magic; }
+__device__ __forceinline__ uint32_t opaque_vgpr(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+__device__ __forceinline__ uint32_t opaque_sgpr(uint32_t v) {
+  asm volatile("" : "+s"(v));
+  return v;
+}
+__device__ __forceinline__ void tie_v(u32x4& v) { asm volatile("" : "+v"(v)); }
+
+// ---- direct-to-LDS loads and their waits.  LDS address of lane l: lds + 16 l (4 l for the 2-byte form).
+__device__ __forceinline__ void dma16(const uint8_t* sbase, uint32_t voff, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(sbase)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void dma2(const uint8_t* sbase, uint32_t voff, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2" ::"s"(lds), "v"(voff), "s"(sbase)
+               : "memory", "m0");
+}
+__device__ __forceinline__ u32x4 gload16(const void* p) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+template <int N>
+__device__ __forceinline__ void vmwait() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void lgkm_drain() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t*)p;
+}
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__device__ __forceinline__ void wg_lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// maximum of a non-negative value over the wave, as a wave-uniform number
+__device__ __forceinline__ float wave_max_nonneg(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, dpp_f<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, dpp_f<0x141>(v));  // row_half_mirror
+  v = fmaxf(v, dpp_f<0x140>(v));  // row_mirror
+  const uint32_t b = __builtin_bit_cast(uint32_t, v);
+  const uint32_t m0 = __builtin_amdgcn_readlane(b, 0), m1 = __builtin_amdgcn_readlane(b, 16),
+                 m2 = __builtin_amdgcn_readlane(b, 32), m3 = __builtin_amdgcn_readlane(b, 48);
+  const uint32_t m01 = m0 > m1 ? m0 : m1, m23 = m2 > m3 ? m2 : m3;
+  return __builtin_bit_cast(float, m01 > m23 ? m01 : m23);
+}
+
+// Per-codec geometry of a unit.  PP 16-byte pieces of every block travel (q6_k: the first 208 bytes, its
+// trailing d goes as one 2-byte load per row); LBPB = LDS bytes per row; NAP = A register pairs per unit;
+// XSG = activation sums per half superblock (sub-blocks of 32, q6_k: scale groups of 16).
+template <int C>
+struct StGeom;
+template <>
+struct StGeom<KQ_Q4_K> {
+  static constexpr int BPB = 144, PP = 9, LBPB = 144, NAP = 4, XSG = 4;
+  static constexpr bool SIDE_D = false;
+};
+template <>
+struct StGeom<KQ_Q5_K> {
+  static constexpr int BPB = 176, PP = 11, LBPB = 176, NAP = 4, XSG = 4;
+  static constexpr bool SIDE_D = false;
+};
+template <>
+struct StGeom<KQ_Q6_K> {
+  static constexpr int BPB = 210, PP = 13, LBPB = 208, NAP = 8, XSG = 8;
+  static constexpr bool SIDE_D = true;
+};
+template <int C>
+struct StUnit {
+  using G = StGeom<C>;
+  static constexpr int PIECES = ST_ROWS * G::PP;
+  static constexpr int FULL = PIECES / 64;                // load instructions with all 64 lanes
+  static constexpr bool HALF = (PIECES % 64) != 0;        // one more with 32 lanes
+  static constexpr int UPI = FULL + (HALF ? 1 : 0) + (G::SIDE_D ? 1 : 0);  // load instructions per unit
+  static constexpr int SLOT = ST_ROWS * G::LBPB + (G::SIDE_D ? 128 : 0);   // LDS bytes per unit
+};
+
+struct StArgs {
+  const void* x;
+  const uint8_t* w;
+  void* y;
+  int M, N, K, tiles;
+  float* partial;  // split-K: [ksplit][M][N] f32
+  int ksplit, sb_per_split;
+#ifdef KQ_ST_TS
+  uint64_t* ts;
+#endif
+};
+
+// ------------------------------------------------------------------ q4_k / q5_k unit
+// Lane (row, kg) owns sub-blocks 4 kg .. 4 kg + 3.  LDS row: d, dmin, scales[12] | (q5_k: qh[32]) | qs[128].
+// Pieces qs[64 kg + 16 pc ..), pc = 0..3: pair pc / 2 of the half, weights 16 (pc % 2) .. + 15 of the low-nibble
+// sub-block 2 (pc / 2) and of the high-nibble sub-block 2 (pc / 2) + 1.  MFMA (pc, e, h): word e of the piece,
+// nibble h; activations = A pair pc, block 2 e + h.
+template <int C, int R>
+__device__ __forceinline__ void q45k_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
+                                          const float* __restrict__ xsum, int xsum_row_stride, float* acc) {
+  constexpr int QS = C == KQ_Q4_K ? 16 : 48;
+  const u32x4 hdr = *reinterpret_cast<const u32x4*>(bl);
+  u32x4 q[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) q[i] = *reinterpret_cast<const u32x4*>(bl + QS + 64 * kg + 16 * i);
+  uint32_t hw[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if constexpr (C == KQ_Q5_K) {
+    // fifth bits: bit j of qh[l] belongs to sub-block j; shifted down by 4 kg they sit at bits 0..3 of every byte
+    const u32x4 h0 = *reinterpret_cast<const u32x4*>(bl + 16), h1 = *reinterpret_cast<const u32x4*>(bl + 32);
+    const int sh = 4 * kg;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      hw[e] = h0[e] >> sh;
+      hw[4 + e] = h1[e] >> sh;
+    }
+  }
+  float xs[R][4];
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    const float4 t4 = *reinterpret_cast<const float4*>(xsum + r * xsum_row_stride + 4 * kg);
+    xs[r][0] = t4.x;
+    xs[r][1] = t4.y;
+    xs[r][2] = t4.z;
+    xs[r][3] = t4.w;
+  }
+  // scales of this lane's four sub-blocks
+  float mul[4], sub[4];
+  {
+    const float d = kq::h2f((uint16_t)(hdr.x & 0xffff)) * xscale;
+    const float dmin = kq::h2f((uint16_t)(hdr.x >> 16)) * xscale;
+    const float d16 = d * 0.0625f;
+    const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
+    const uint32_t sc_lo = s0 & 0x3f3f3f3fu, mn_lo = s1 & 0x3f3f3f3fu;
+    const uint32_t sc_hi = (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u);
+    const uint32_t mn_hi = ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u);
+    const uint32_t scw = kg ? sc_hi : sc_lo, mnw = kg ? mn_hi : mn_lo;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const float sc = (float)((scw >> (8 * j)) & 0xff);
+      const float mn = (float)((mnw >> (8 * j)) & 0xff);
+      // even sub-blocks read low nibbles (1024 + q), odd ones high nibbles in place (1024 + 16 q)
+      mul[j] = ((j & 1) ? d16 : d) * sc;
+      sub[j] = fmaf(mul[j], 1024.0f, dmin * mn);
+    }
+  }
+  const uint32_t magic = opaque_vgpr(0x64006400u);
+  const uint32_t mask_lo = opaque_sgpr(0x000f000fu), mask_hi = opaque_sgpr(0x00f000f0u);
+  const uint32_t bit_lo = opaque_sgpr(0x00100010u), bit_hi = opaque_sgpr(0x01000100u);
+  SFor<2>::run([&](auto gg) {
+    constexpr int gl = decltype(gg)::value;
+    f32x4 p[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+    SFor<2>::run([&](auto pp) {
+      constexpr int pc = 2 * gl + decltype(pp)::value;
+      const f16x4 av = __builtin_bit_cast(f16x4, areg[pc]);
+      SFor<4>::run([&](auto ee) {
+        constexpr int e = decltype(ee)::value;
+        const uint32_t w0 = q[pc][e], w8 = w0 >> 8;
+        SFor<2>::run([&](auto hh) {
+          constexpr int h = decltype(hh)::value;
+          u32x2 bv;
+          bv.x = and_or(w0, h ? mask_hi : mask_lo, magic);  // weights l, l + 2
+          bv.y = and_or(w8, h ? mask_hi : mask_lo, magic);  // weights l + 1, l + 3
+          if constexpr (C == KQ_Q5_K) {
+            // bit jl = 2 gl + h of the four qh bytes of weights l .. l + 3 goes to bit 4 (1024 + q + 16 b) or
+            // bit 8 (1024 + 16 q + 256 b) of the 16-bit code
+            constexpr int jl = 2 * gl + h, tgt = h ? 8 : 4;
+            const uint32_t hq = hw[4 * (pc & 1) + e];
+            bv.x = and_or(hq << (tgt - jl), h ? bit_hi : bit_lo, opaque_vgpr(bv.x));
+            bv.y = and_or(hq >> (8 + jl - tgt), h ? bit_hi : bit_lo, opaque_vgpr(bv.y));
+          }
+          p[h] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, bv), p[h], 3, 2 * e + h, 0);
+        });
+      });
+    });
+    SFor<2>::run([&](auto hh) {
+      constexpr int h = decltype(hh)::value;
+      constexpr int jl = 2 * gl + h;
+      SFor<R>::run([&](auto rr) {
+        constexpr int r = decltype(rr)::value;
+        acc[r] = fmaf(mul[jl], p[h][r], acc[r]);
+        acc[r] = fmaf(-sub[jl], xs[r][jl], acc[r]);
+      });
+    });
+  });
+}
+
+// ------------------------------------------------------------------ q6_k unit
+// Lane (row, hf) owns half hf of the superblock: weights 128 hf + 32 t + l, t = 0..3, l = 0..31.  LDS row:
+// ql[128] | qh[64] | int8 scales[16]; d sits in the slot's side area (one dword per row).  Low nibble of the
+// weight: ql[64 hf + 32 (t & 1) + l] (high nibble of the byte for t >= 2); high bits: bits 2 t, 2 t + 1 of
+// qh[32 hf + l]; scale 8 hf + 2 t + l / 16.  Both fields are masked in place: 1024 + s ql with s = 1 (t < 2) or
+// 16, 1024 + 4^t qh.  Per scale group of 16 weights two accumulators P, H and
+//   sum x w = d sc (P / s + 16 H / 4^t - (1024 / s + 16 * 1024 / 4^t + 32) X).
+// MFMA (t, e): weights l = 4 e .. 4 e + 3; activations = A pair 2 t + e / 4, block 2 (e % 4) [+ 1 unused].
+template <int R>
+__device__ __forceinline__ void q6k_unit(const uint8_t* __restrict__ bl, float dx, int hf, const u32x2* areg,
+                                         const float* __restrict__ xsum, int xsum_row_stride, float* acc) {
+  u32x4 ql[4], qh[2];
+#pragma unroll
+  for (int i = 0; i < 4; i++) ql[i] = *reinterpret_cast<const u32x4*>(bl + 64 * hf + 16 * i);
+#pragma unroll
+  for (int i = 0; i < 2; i++) qh[i] = *reinterpret_cast<const u32x4*>(bl + 128 + 32 * hf + 16 * i);
+  const uint2 scw = *reinterpret_cast<const uint2*>(bl + 192 + 8 * hf);
+  float xs[R][8];
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    const float4 t0 = *reinterpret_cast<const float4*>(xsum + r * xsum_row_stride + 8 * hf);
+    const float4 t1 = *reinterpret_cast<const float4*>(xsum + r * xsum_row_stride + 8 * hf + 4);
+    xs[r][0] = t0.x; xs[r][1] = t0.y; xs[r][2] = t0.z; xs[r][3] = t0.w;
+    xs[r][4] = t1.x; xs[r][5] = t1.y; xs[r][6] = t1.z; xs[r][7] = t1.w;
+  }
+  const uint32_t magic = opaque_vgpr(0x64006400u);
+  const uint32_t mask_lo = opaque_sgpr(0x000f000fu), mask_hi = opaque_sgpr(0x00f000f0u);
+  const uint32_t mask_h[4] = {opaque_sgpr(0x00030003u), opaque_sgpr(0x000c000cu), opaque_sgpr(0x00300030u),
+                              opaque_sgpr(0x00c000c0u)};
+  uint32_t ql8[16], qh8[8];
+#pragma unroll
+  for (int i = 0; i < 16; i++) ql8[i] = ql[i >> 2][i & 3] >> 8;
+#pragma unroll
+  for (int i = 0; i < 8; i++) qh8[i] = qh[i >> 2][i & 3] >> 8;
+  SFor<4>::run([&](auto tt) {
+    constexpr int t = decltype(tt)::value;
+    SFor<2>::run([&](auto ss) {
+      constexpr int s = decltype(ss)::value;  // scale group 2 t + s: weights l = 16 s .. 16 s + 15
+      f32x4 pq = {0, 0, 0, 0}, ph = {0, 0, 0, 0};
+      SFor<4>::run([&](auto ee) {
+        constexpr int e = 4 * s + decltype(ee)::value;  // l = 4 e .. 4 e + 3
+        constexpr int wq = 8 * (t & 1) + e;             // ql word: bytes 32 (t & 1) + 4 e ..
+        const f16x4 av = __builtin_bit_cast(f16x4, areg[2 * t + e / 4]);
+        u32x2 bq, bh;
+        bq.x = and_or(ql[wq >> 2][wq & 3], t >= 2 ? mask_hi : mask_lo, magic);
+        bq.y = and_or(ql8[wq], t >= 2 ? mask_hi : mask_lo, magic);
+        bh.x = and_or(qh[e >> 2][e & 3], mask_h[t], magic);
+        bh.y = and_or(qh8[e], mask_h[t], magic);
+        pq = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, bq), pq, 3, 2 * (e & 3), 0);
+        ph = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, bh), ph, 3, 2 * (e & 3), 0);
+      });
+      constexpr int g = 2 * t + s;
+      const int sc = __builtin_amdgcn_sbfe((int)(g < 4 ? scw.x : scw.y), 8 * (g & 3), 8);
+      const float dsc = dx * (float)sc;
+      constexpr float fq = t >= 2 ? 0.0625f : 1.0f;       // 1 / s
+      constexpr float fh = 16.0f / (float)(1 << (2 * t));  // 16 / 4^t
+      constexpr float fx = 1024.0f * fq + 1024.0f * fh + 32.0f;
+      SFor<R>::run([&](auto rr) {
+        constexpr int r = decltype(rr)::value;
+        const float v = fmaf(fq, pq[r], fmaf(fh, ph[r], -fx * xs[r][g]));
+        acc[r] = fmaf(dsc, v, acc[r]);
+      });
+    });
+  });
+}
+
+// ------------------------------------------------------------------ the kernel
+// MB = M rounded up to a power of two (1, 2, 4); D = units a wave keeps in LDS (in flight or being read).
+template <int C, int DT, int MB, int D>
+__global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
+  using G = StGeom<C>;
+  using U = StUnit<C>;
+  constexpr int R = MB;
+  constexpr int NAP = G::NAP, XSG = G::XSG;
+  constexpr int XL = 2;  // 16-byte activation loads per lane and row: 4 units x 256 values
+
+#ifdef KQ_ST_TS
+  uint64_t ts[8];
+  ts[0] = __builtin_amdgcn_s_memrealtime();
+#define ST_TS(i) ts[i] = __builtin_amdgcn_s_memrealtime()
+#else
+#define ST_TS(i)
+#endif
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, kg = lane >> 5;
+  const int M = a.M, N = a.N, K = a.K, nsb = K >> 8, tiles = a.tiles;
+  const uint32_t row_bytes = (uint32_t)nsb * G::BPB;
+  const int G_x = gridDim.x;
+
+  // LDS: per wave [D slots][x fragments MB x 4 x 256 f16][x sums MB x 4 x 2 XSG f32]; then red [2][waves][R][64] f32
+  constexpr int XS_BYTES = MB * ST_XU * 512, XSUM_BYTES = MB * ST_XU * 2 * XSG * 4;
+  constexpr int WAVE_BYTES = D * U::SLOT + XS_BYTES + XSUM_BYTES;
+  uint8_t* wb = smem + wave * WAVE_BYTES;
+  _Float16* xs = reinterpret_cast<_Float16*>(wb + D * U::SLOT);
+  float* xsum = reinterpret_cast<float*>(wb + D * U::SLOT + XS_BYTES);
+  float* red_all = reinterpret_cast<float*>(smem + ST_WAVES * WAVE_BYTES);
+  const uint32_t wb_lds = lds_addr(wb);
+
+  // this workgroup's K range and this wave's units: superblocks sb_begin + wave + 4 u
+  const int sb_begin = a.ksplit > 1 ? (int)blockIdx.z * a.sb_per_split : 0;
+  int sb_end = a.ksplit > 1 ? sb_begin + a.sb_per_split : nsb;
+  sb_end = sb_end < nsb ? sb_end : nsb;
+  const int sbn = sb_end - sb_begin;
+  const int nu = sbn > wave ? (sbn - wave + ST_WAVES - 1) / ST_WAVES : 0;  // wave-uniform, 0..4
+
+  // ---- activation loads first: they are the oldest loads of the wave
+  const uint16_t* x16 = static_cast<const uint16_t*>(a.x);
+  u32x4 xreg[MB * XL];
+  SFor<MB * XL>::run([&](auto t) {
+    constexpr int T = decltype(t)::value;
+    constexpr int m = T / XL, s = T % XL;
+    const int gi = lane + 64 * s, uu = gi >> 5, grp = gi & 31;
+    int sb = wave + ST_WAVES * uu;
+    sb = sb < sbn ? sb : (wave < sbn ? wave : 0);  // spare units re-read a valid superblock
+    const int mm = m < M ? m : M - 1;
+    xreg[T] = gload16(x16 + (size_t)mm * K + (size_t)(sb_begin + sb) * 256 + 8 * grp);
+  });
+  __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled ahead of these loads
+
+  // ---- weight stream.  Piece i = lane + 64 t of a unit -> (row i / PP, piece i % PP); rows past the end of the
+  // matrix re-read the last row (their results are dropped).
+  uint32_t goff[U::FULL + 1];
+  const int row_lim = N - 1;
+  auto piece_off = [&](int i, int row0) {
+    int r = i / G::PP;
+    const int p = i - r * G::PP;
+    r = row0 + r;
+    r = r < row_lim ? r : row_lim;
+    return (uint32_t)(r - row0) * row_bytes + 16u * p;  // may be negative-free: r >= row0 whenever row0 <= row_lim
+  };
+  // (offsets are relative to the tile's first row; a tile always starts inside the matrix)
+  // Elements of the stream: (tile, unit) in tile-major order.  `it`, `iu`, `islot`: next element to issue.
+  int it = blockIdx.x, iu = 0, islot = 0, inflight = 0;
+  int goff_row0 = -1;
+  auto issue_next = [&]() {
+    if (it >= tiles) return;
+    const int row0 = it * ST_ROWS;
+    if (row0 + ST_ROWS > N && goff_row0 != row0) {  // ragged last tile: rebuild the piece map with clamped rows
+      SFor<U::FULL + 1>::run([&](auto t) { constexpr int T = decltype(t)::value; goff[T] = piece_off(lane + 64 * T, row0); });
+      goff_row0 = row0;
+    }
+    const uint8_t* base = a.w + (size_t)row0 * row_bytes + (size_t)(sb_begin + wave + ST_WAVES * iu) * G::BPB;
+    const uint32_t l0 = wb_lds + islot * U::SLOT;
+    SFor<U::FULL>::run([&](auto t) { constexpr int T = decltype(t)::value; dma16(base, goff[T], l0 + T * 1024); });
+    if constexpr (U::HALF) {
+      if (lane < 32) dma16(base, goff[U::FULL], l0 + U::FULL * 1024);
+    }
+    if constexpr (G::SIDE_D) {
+      int r = row0 + lane;
+      r = r < row_lim ? r : row_lim;
+      if (lane < 32) dma2(base + 208, (uint32_t)(r - row0) * row_bytes, l0 + ST_ROWS * G::LBPB);
+    }
+    inflight++;
+    islot = islot + 1 == D ? 0 : islot + 1;
+    if (++iu == nu) {
+      iu = 0;
+      it += G_x;
+    }
+  };
+  SFor<U::FULL + 1>::run([&](auto t) {
+    constexpr int T = decltype(t)::value;
+    const int i = lane + 64 * T, r = i / G::PP;
+    goff[T] = (uint32_t)r * row_bytes + 16u * (i - r * G::PP);
+  });
+  if (nu == 0) it = tiles;  // a wave without superblocks (short K range) only joins the barriers
+
+  // every wave of the workgroup has queued its activation loads before any weight load is queued
+  __builtin_amdgcn_s_barrier();
+  issue_next();
+  // wait for the activations alone: the first unit stays in flight
+  if (inflight) vmwait<U::UPI>(); else vmwait<0>();
+  ST_TS(1);
+  SFor<MB * XL>::run([&](auto t) { tie_v(xreg[decltype(t)::value]); });
+
+  // ---- activations -> f16 fragments (+ sums) in the wave's LDS, then this lane's A registers
+  float xscale = 1.0f, inv = 1.0f;
+  if constexpr (DT == KQ_BF16) {
+    float amax = 0.f;
+    SFor<MB * XL>::run([&](auto t) {
+      const u32x4 v = xreg[decltype(t)::value];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] << 16)));
+        amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] & 0xffff0000u)));
+      }
+    });
+    amax = wave_max_nonneg(amax);
+    // bring the largest magnitude into [2^14, 2^15): exact power-of-two scaling
+    const uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff;
+    if (eb != 0 && eb != 0xff) {
+      int e = (int)eb - 127 - 14;
+      if (e < -100) e = -100;
+      xscale = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+      inv = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
+    }
+  }
+  SFor<MB * XL>::run([&](auto t) {
+    constexpr int T = decltype(t)::value;
+    constexpr int m = T / XL, s = T % XL;
+    const int gi = lane + 64 * s, uu = gi >> 5, grp = gi & 31;
+    const u32x4 v = xreg[T];
+    _Float16 h[8];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      if constexpr (DT == KQ_BF16) {
+        h[2 * e] = (_Float16)(__builtin_bit_cast(float, v[e] << 16) * inv);
+        h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, v[e] & 0xffff0000u) * inv);
+      } else {
+        h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] & 0xffff));
+        h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
+      }
+    }
+    // MFMA fragment order inside a 4-group: k0 k2 k1 k3
+    const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+    *reinterpret_cast<f16x8*>(xs + (m * ST_XU + uu) * 256 + 8 * grp) = v8;
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) sum += (float)h[e];
+    sum += dpp_f<0xB1>(sum);  // lanes l ^ 1: 16 values
+    if constexpr (XSG == 8) {
+      if ((lane & 1) == 0) xsum[(m * ST_XU + uu) * 16 + (grp >> 1)] = sum;
+    } else {
+      sum += dpp_f<0x4E>(sum);  // lanes l ^ 2: 32 values
+      if ((lane & 3) == 0) xsum[(m * ST_XU + uu) * 8 + (grp >> 2)] = sum;
+    }
+  });
+  wave_lds_fence();
+  // A registers.  Lane (kg, fa, fi) keeps, for every unit and register pair, the four activations of row fi
+  // that MFMA block fa needs.
+  //   q4_k / q5_k: pair pc, block 2 e + h  -> k = 128 kg + 32 (2 (pc / 2) + h) + 16 (pc % 2) + 4 e
+  //   q6_k:        pair 2 t + e / 4, block 2 (e % 4) -> k = 128 hf + 32 t + 4 e  (odd blocks unused)
+  const int fa = (lane >> 2) & 7, fi = lane & 3;
+  u32x2 areg[ST_XU * NAP];
+  {
+    const uint8_t* xb = reinterpret_cast<const uint8_t*>(xs) + (fi & (MB - 1)) * (ST_XU * 512) + 256 * kg;
+    SFor<ST_XU * NAP>::run([&](auto t) {
+      constexpr int T = decltype(t)::value;
+      constexpr int u = T / NAP, pr = T % NAP;
+      int koff;  // in f16 elements inside the half
+      if constexpr (C == KQ_Q6_K)
+        koff = 32 * (pr >> 1) + 16 * (pr & 1) + 4 * (fa >> 1);
+      else
+        koff = 64 * (pr >> 1) + 32 * (fa & 1) + 16 * (pr & 1) + 4 * (fa >> 1);
+      areg[T] = *reinterpret_cast<const u32x2*>(xb + u * 512 + koff * 2);
+    });
+  }
+
+  // The other D - 1 units are queued only now: a wave that queues loads faster than the memory system takes them
+  // stalls in the issue, and the activation work above would have waited behind that stall.
+  ST_TS(2);
+  SFor<D - 1>::run([&](auto) { issue_next(); });
+  float acc[R];
+  int ct = blockIdx.x, cslot = 0;  // tile / slot being consumed
+  int parity = 0;
+  for (; ct < tiles; ct += G_x) {
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+    const int row0 = ct * ST_ROWS;
+    const int nrows = N - row0 < ST_ROWS ? N - row0 : ST_ROWS;
+    const int crow = n < nrows ? n : nrows - 1;
+    SFor<ST_XU>::run([&](auto uu) {
+      constexpr int u = decltype(uu)::value;
+      if (u < nu) {
+        // loads issued after this unit's: inflight - 1 units
+        const int younger = inflight - 1;
+        if (younger >= 3) vmwait<3 * U::UPI>();
+        else if (younger == 2) vmwait<2 * U::UPI>();
+        else if (younger == 1) vmwait<1 * U::UPI>();
+        else vmwait<0>();
+        ST_TS(3 + u);
+        const uint8_t* slot = wb + cslot * U::SLOT;
+        const uint8_t* bl = slot + crow * G::LBPB;
+        if constexpr (C == KQ_Q6_K) {
+          const float dx = kq::h2f((uint16_t)*reinterpret_cast<const uint32_t*>(slot + ST_ROWS * G::LBPB + 4 * crow)) * xscale;
+          q6k_unit<R>(bl, dx, kg, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
+        } else {
+          q45k_unit<C, R>(bl, kg, xscale, areg + u * NAP, xsum + u * 8, ST_XU * 8, acc);
+        }
+        // the slot has been read: refill it with the next element of the stream
+        lgkm_drain();
+        inflight--;
+        cslot = cslot + 1 == D ? 0 : cslot + 1;
+        issue_next();
+      }
+    });
+
+#ifdef KQ_ST_TS
+    lgkm_drain();
+    ST_TS(7);
+    if (lane == 0)
+      for (int i = 0; i < 8; i++) a.ts[((size_t)blockIdx.x * ST_WAVES + wave) * 8 + i] = ts[i];
+#endif
+    // ---- cross-wave + cross-half reduction of the tile
+    float* red = red_all + (parity * ST_WAVES + wave) * (R * 64);
+#pragma unroll
+    for (int r = 0; r < R; r++) red[r * 64 + lane] = acc[r];
+    wg_lds_barrier();
+    if (tid < R * 32) {
+      const int r = tid >> 5, nn = tid & 31;
+      float v = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < ST_WAVES; wv++) {
+        const float* rw = red_all + (parity * ST_WAVES + wv) * (R * 64);
+        v += rw[r * 64 + nn] + rw[r * 64 + nn + 32];
+      }
+      if (r < M && nn < nrows) {
+        if (a.ksplit > 1) {
+          a.partial[(size_t)blockIdx.z * M * N + (size_t)r * N + row0 + nn] = v;
+        } else {
+          uint16_t* yo = static_cast<uint16_t*>(a.y) + (size_t)r * N + row0 + nn;
+          *yo = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+        }
+      }
+    }
+    parity ^= 1;
+  }
+}
+
+template <int C, int MB, int D>
+constexpr size_t st_lds_bytes() {
+  return (size_t)ST_WAVES * (D * StUnit<C>::SLOT + MB * ST_XU * 512 + MB * ST_XU * 2 * StGeom<C>::XSG * 4) +
+         2 * ST_WAVES * MB * 64 * 4;
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void st_splitk_reduce_kernel(const float* __restrict__ partial, uint16_t* __restrict__ y,
+                                                               int count, int ksplit) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  float v = 0.f;
+  for (int sp = 0; sp < ksplit; sp++) v += partial[(size_t)sp * count + i];
+  y[i] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+}
+
+int st_num_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  return cus;
+}
+
+// K split: every workgroup gets at most 16 superblocks; with fewer row tiles than 1.5 per CU the range is cut
+// further so that about two workgroups per CU exist.
+struct StSplit {
+  int ksplit, sb_per_split;
+};
+StSplit st_split_plan(int N, int K, int cus) {
+  const int nsb = K >> 8, tiles = (N + ST_ROWS - 1) / ST_ROWS;
+  int want = (nsb + 15) / 16;
+  if (tiles * want < cus + cus / 2) {
+    int more = (2 * cus + tiles - 1) / tiles;
+    if (more > nsb / 4) more = nsb / 4;  // at least one superblock per wave
+    if (more > want) want = more;
+  }
+  if (want < 1) want = 1;
+  int per = (nsb + want - 1) / want;
+  if (per > 16) per = 16;
+  StSplit p{(nsb + per - 1) / per, per};
+  return p;
+}
+
+template <int C, int DT, int MB, int D>
+int st_launch_one(StArgs a, int splits, hipStream_t s) {
+  constexpr size_t lds = st_lds_bytes<C, MB, D>();
+  auto kern = stream_gemv_kernel<C, DT, MB, D>;
+  static bool attr_set = false;  // per instantiation
+  if (!attr_set) {
+    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  const int per_cu = lds <= 80 * 1024 ? 2 : 1;
+  int gx = per_cu * st_num_cus() / splits;
+  if (gx < 1) gx = 1;
+  if (gx > a.tiles) gx = a.tiles;
+  hipLaunchKernelGGL(kern, dim3(gx, 1, splits), dim3(ST_THREADS), lds, s, a);
+  KQ_HIP_CHECK(hipGetLastError());
+  if (splits > 1) {
+    const int count = a.M * a.N;
+    hipLaunchKernelGGL((st_splitk_reduce_kernel<DT>), dim3((count + 255) / 256), dim3(256), 0, s, a.partial,
+                       static_cast<uint16_t*>(a.y), count, splits);
+    KQ_HIP_CHECK(hipGetLastError());
+  }
+  return KQ_OK;
+}
+
+template <int C, int DT>
+int st_launch_m(const StArgs& a, int splits, hipStream_t s) {
+  constexpr int D1 = C == KQ_Q6_K ? 2 : 2;
+  if (a.M == 1) return st_launch_one<C, DT, 1, D1>(a, splits, s);
+  if (a.M == 2) return st_launch_one<C, DT, 2, 2>(a, splits, s);
+  return st_launch_one<C, DT, 4, 2>(a, splits, s);
+}
+
+bool st_codec_ok(int codec) { return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K; }
+
+}  // namespace
+
+bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const void* w) {
+  if (!st_codec_ok(codec) || M < 1 || M > 4 || N < 1 || K < 256 || (K & 255)) return false;
+  if ((int64_t)N * (K >> 8) * 210 >= (int64_t)1 << 40) return false;
+  // q4_k / q5_k pieces are fetched 16-byte aligned, q6_k blocks are 2-byte multiples
+  const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;
+  if (reinterpret_cast<uintptr_t>(w) & wmask) return false;
+  return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+}
+
+size_t kq_stream_workspace_bytes(int M, int N, int K, int codec) {
+  if (!st_codec_ok(codec) || M < 1 || M > 4 || (K & 255) || K < 256) return 0;
+  const StSplit p = st_split_plan(N, K, st_num_cus());
+  return p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
+}
+
+int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                         size_t ws_bytes, hipStream_t s) {
+  if (!kq_stream_supported(M, N, K, codec, x, w)) return KQ_ERR_UNSUPPORTED;
+  const StSplit p = st_split_plan(N, K, st_num_cus());
+  if (p.ksplit > 1 && (!ws || ws_bytes < (size_t)p.ksplit * M * N * sizeof(float) || (reinterpret_cast<uintptr_t>(ws) & 3)))
+    return KQ_ERR_UNSUPPORTED;  // the caller falls through to the kernels that can run unsplit
+  StArgs a{};
+  a.x = x;
+  a.w = w;
+  a.y = y;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.tiles = (N + ST_ROWS - 1) / ST_ROWS;
+  a.partial = static_cast<float*>(ws);
+  a.ksplit = p.ksplit;
+  a.sb_per_split = p.sb_per_split;
+  if (codec == KQ_Q4_K)
+    return dtype == KQ_F16 ? st_launch_m<KQ_Q4_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q4_K, KQ_BF16>(a, p.ksplit, s);
+  if (codec == KQ_Q5_K)
+    return dtype == KQ_F16 ? st_launch_m<KQ_Q5_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q5_K, KQ_BF16>(a, p.ksplit, s);
+  return dtype == KQ_F16 ? st_launch_m<KQ_Q6_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q6_K, KQ_BF16>(a, p.ksplit, s);
+}

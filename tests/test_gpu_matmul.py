@@ -103,11 +103,12 @@ def test_qmm_gemv_unaligned_rows_and_tensor_end(kq, codec):
 @pytest.mark.parametrize("codec", ["q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_qmm_skinny_both_variants(kq, codec):
     """Dense skinny calls through every selectable kernel: workgroup-synchronous (1), decoupled-wave (2),
-    its two-superblock-unit form (3) and the diagonal kernel (4; shapes whose K is not a multiple of 1024
-    fall back to the decoupled one)."""
+    its two-superblock-unit form (3), the diagonal kernel (4; shapes whose K is not a multiple of 1024
+    fall back to the decoupled one) and the streamed kernel (5; q4_k / q5_k / q6_k up to four rows, the rest
+    falls back)."""
     lib = kq._load()
     try:
-        for variant in (1, 2, 3, 4):
+        for variant in (1, 2, 3, 4, 5):
             lib.kq_set_skinny_variant(variant)
             for M, N, K in ((1, 1000, 768), (8, 520, 4352), (3, 4100, 1024), (2, 300, 4096), (5, 4200, 14336),
                             (7, 100, 2048)):
@@ -118,6 +119,21 @@ def test_qmm_skinny_both_variants(kq, codec):
                 assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, variant, M, N, K)
     finally:
         lib.kq_set_skinny_variant(0)
+
+
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+def test_qmm_streamed_kernel_shapes(kq, codec, dtype):
+    """The streamed kernel (default for up to four rows of q4_k / q5_k / q6_k): one to four rows, K ranges that
+    leave waves without a superblock (256, 768), K above 16 superblocks (split over grid z), a ragged last row
+    tile, a single row, and more row tiles than resident workgroups (persistent loop, N = 20000)."""
+    for M, N, K in ((1, 33, 256), (2, 31, 768), (3, 1, 1024), (4, 97, 4096), (1, 20000, 1024), (2, 1030, 5120),
+                    (1, 4100, 14336), (4, 2050, 8192)):
+        wire = _wire(codec, N, K, seed=43)
+        xb, xt = make_x((M, K), dtype, seed=44)
+        got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+        want = O.qmm(xb, wire, codec, True, dtype)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype, M, N, K)
 
 
 def test_qmm_skinny_unaligned_q6k_rows(kq):
