@@ -81,6 +81,18 @@ size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int 
 int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int transpose,
            int codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* kq_qmm for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): transpose is implied, and the workspace is a buffer of
+ * KQ_NOALLOC_SCRATCH_BYTES that lives inside the library's code object on every GPU (no hipMalloc, hipFree
+ * or other allocating call is made).  A call whose kq_qmm_workspace_size exceeds that size is rejected with
+ * KQ_ERR_WORKSPACE.  All calls on one GPU share that GPU's buffer: calls that overlap in time on the same
+ * GPU (different streams or threads) race; the buffer keeps the last call's contents, and the kernels write
+ * every element they later read, so nothing needs clearing between calls.
+ * No counterpart in the reference. */
+#define KQ_NOALLOC_SCRATCH_BYTES (4u << 20)
+int kq_qmm_noalloc(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int codec, int dtype,
+                   void* stream);
+
 /* Decode-only matvec with the layer bias fused in: y[n] = T(x . W[n]^T + float(bias[n])), one activation row,
  * bias [N] in the activation dtype, q8_0 only (as wired in the reference).
  * Replaces KQuantQmvBias (op quantized_matmul_qmv_bias), reference src/kquant_ops.cpp:185-270. */

@@ -19,6 +19,10 @@ extern "C" __attribute__((visibility("hidden"))) const uint8_t kq_grid_blob_host
 #include "kq_iq_grids.inc"
 };
 
+// Workspace of kq_qmm_noalloc: device-resident storage inside the code object.  In host code this name is only
+// a handle for hipGetSymbolAddress; kernels get the per-device address that call returns.
+static __device__ __attribute__((aligned(256))) uint8_t kq_noalloc_scratch[KQ_NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -41,6 +45,7 @@ const kq_codec_info kCodecs[KQ_NUM_CODECS] = {
 constexpr int kMaxDevices = 64;
 std::mutex g_grid_mu;
 const uint8_t* g_grids[kMaxDevices] = {};
+void* g_scratch[kMaxDevices] = {};  // per-device address of kq_noalloc_scratch
 
 thread_local KqOutMap g_out_map = {1, 1, 0, 0};
 // Sets the calling thread's output map for the launches inside a scope.
@@ -165,6 +170,35 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
   rc = kq_launch_codes_skinny(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, y_dev, M, N, K, codec, dtype, s);
   if (rc != KQ_ERR_UNSUPPORTED) return rc;
   return kq_launch_gemv_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+}
+
+int kq_qmm_noalloc(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int codec, int dtype,
+                   void* stream) {
+  if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: unknown codec id %d", codec);
+  const size_t need = kq_qmm_workspace_size(M, N, K, 1, codec, dtype);
+  if (need > KQ_NOALLOC_SCRATCH_BYTES)
+    return kq_set_error(KQ_ERR_WORKSPACE,
+                        "quantized_matmul (no-allocation entry): this shape needs %zu bytes of workspace, the built-in "
+                        "buffer holds %u; call kq_qmm with a caller-owned workspace",
+                        need, (unsigned)KQ_NOALLOC_SCRATCH_BYTES);
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return kq_set_error(KQ_ERR_HIP, "no usable HIP device: %s", hipGetErrorString(e));
+  void* scratch = nullptr;
+  {
+    std::lock_guard<std::mutex> lk(g_grid_mu);
+    if (!g_scratch[dev]) {
+      // once per device, with that device current: every GPU holds its own copy of the array
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(kq_noalloc_scratch));
+      if (e != hipSuccess || !p)
+        return kq_set_error(KQ_ERR_HIP, "scratch lookup failed: %s", hipGetErrorString(e));
+      g_scratch[dev] = p;
+    }
+    scratch = g_scratch[dev];
+  }
+  return kq_qmm(x_dev, w_dev, y_dev, M, N, K, 1, codec, dtype, scratch, KQ_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int N, int K, int codec,

@@ -69,6 +69,7 @@ def _load():
     lib.kq_qmm_workspace_size.restype = sz
     lib.kq_qmm_workspace_size.argtypes = [i, i, i, i, i, i]
     lib.kq_qmm.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
+    lib.kq_qmm_noalloc.argtypes = [vp, vp, vp, i, i, i, i, i, vp]
     lib.kq_qmv_bias.argtypes = [vp, vp, vp, vp, i, i, i, i, vp]
     lib.kq_moe_glu_gather_shexp_workspace_size.restype = sz
     lib.kq_moe_glu_gather_shexp_workspace_size.argtypes = [i, i, i, i, i, i, i, i]
