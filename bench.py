@@ -264,6 +264,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-sweep", action="store_true", help="skip the sweep, prefill, MoE and low-bit sections")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--gemm-tile", type=int, default=0,
+                    help="prefill section: force a tile shape of the prefill GEMM (kq_set_gemm_tile_rows)")
+    ap.add_argument("--only", default=None, metavar="SECTIONS",
+                    help="comma-separated extra sections to run (sweep, prefill, moe, moe_mxfp4, moe_decode_lowbit, "
+                         "lowbit, dequantize); default all")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for `rocprofv3 --pmc`: one device copy of the headline matrix (known bytes) "
                          "followed by 20 cold launches of the headline GEMV, nothing else")
@@ -363,151 +368,165 @@ def main():
     base_np = base.cpu().numpy() if not args.no_cpu else None
     del copies, calls
 
+    only = set(args.only.split(",")) if args.only else None
+
+    def want(sec):
+        return only is None or sec in only
+
     if not args.no_sweep:
         steps, warm = 400, 40  # launches per shape
         # ---------------- decode sweep (q4_k_m recipe of Llama-3-8B)
-        sweep = []
-        shapes = [("q_proj", "q4_k", 4096, 4096, True), ("gate/up", "q4_k", 14336, 4096, True),
-                  ("down", "q6_k", 4096, 14336, True), ("lm_head", "q6_k", 128256, 4096, False)]
-        for name, c, n, k, encode in shapes:
-            wb = n * kq.bytes_per_row(c, k)
-            # the 525M-weight lm_head is filled with structurally valid random wire (encoding it on
-            # the host would dominate the run); the others are encoded from N(0, 0.02)
-            wq = base if name == "gate/up" else (quantized_weights(kq, torch, c, n, k, 3, dev) if encode
-                                                 else synth_wire_torch(c, n, k, 3, dev))
-            cps = cold_copies(torch, wq, wb)
-            for m in (1, 2, 4, 8):
-                xm = randx((m, k))
-                t, _ = time_calls(torch, [abi.qmm(xm, w, c, n, k) for w in cps], steps, warm)
-                sweep.append({"proj": name, "codec": c, "N": n, "K": k, "M": m, "us": round(t * 1e3, 2),
-                              "cold_gbs": round(wb / (t * 1e-3) / 1e9, 1),
-                              "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
-            del cps, wq
-        out["sweep"] = sweep
+        if want("sweep"):
+            sweep = []
+            shapes = [("q_proj", "q4_k", 4096, 4096, True), ("gate/up", "q4_k", 14336, 4096, True),
+                      ("down", "q6_k", 4096, 14336, True), ("lm_head", "q6_k", 128256, 4096, False)]
+            for name, c, n, k, encode in shapes:
+                wb = n * kq.bytes_per_row(c, k)
+                # the 525M-weight lm_head is filled with structurally valid random wire (encoding it on
+                # the host would dominate the run); the others are encoded from N(0, 0.02)
+                wq = base if name == "gate/up" else (quantized_weights(kq, torch, c, n, k, 3, dev) if encode
+                                                     else synth_wire_torch(c, n, k, 3, dev))
+                cps = cold_copies(torch, wq, wb)
+                for m in (1, 2, 4, 8):
+                    xm = randx((m, k))
+                    t, _ = time_calls(torch, [abi.qmm(xm, w, c, n, k) for w in cps], steps, warm)
+                    sweep.append({"proj": name, "codec": c, "N": n, "K": k, "M": m, "us": round(t * 1e3, 2),
+                                  "cold_gbs": round(wb / (t * 1e-3) / 1e9, 1),
+                                  "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
+                del cps, wq
+            out["sweep"] = sweep
 
         # ---------------- prefill GEMM
-        prefill = []
-        for c in ("q4_k", "q5_k", "q6_k", "q2_k", "iq4_xs"):
-            n, k = 28672, 8192
-            # q2_k / iq4_xs run the any-codec kernel (reference-order decode + bf16 x 3 split)
-            wq = quantized_weights(kq, torch, c, n, k, 5, dev)
-            for m in (512, 2048):
-                # the device idles while the host encodes the weights: about 30 ms of launches bring it back
-                # to its steady clock before the timed ones (the first shape timed read 6 - 15 % low without)
-                t, _ = time_calls(torch, [abi.qmm(randx((m, k)), wq, c, n, k)], 20, 60 if m <= 512 else 20)
-                tf = 2.0 * m * n * k / (t * 1e-3) / 1e12
-                prefill.append({"codec": c, "M": m, "N": n, "K": k, "ms": round(t, 4), "tflops": round(tf, 1),
-                                "pct_mfma_f16_peak": round(100 * tf / MFMA_F16_PEAK_TFLOPS, 2)})
-            del wq
-        out["prefill"] = prefill
+        if want("prefill"):
+            prefill = []
+            abi.lib.kq_set_gemm_tile_rows(args.gemm_tile)
+            for c in ("q4_k", "q5_k", "q6_k", "q2_k", "iq4_xs"):
+                n, k = 28672, 8192
+                # q2_k / iq4_xs run the any-codec kernel (reference-order decode + bf16 x 3 split)
+                wq = quantized_weights(kq, torch, c, n, k, 5, dev)
+                for m in (512, 2048):
+                    # the device idles while the host encodes the weights: about 30 ms of launches bring it back
+                    # to its steady clock before the timed ones (the first shape timed read 6 - 15 % low without)
+                    t, _ = time_calls(torch, [abi.qmm(randx((m, k)), wq, c, n, k)], 20, 60 if m <= 512 else 20)
+                    tf = 2.0 * m * n * k / (t * 1e-3) / 1e12
+                    prefill.append({"codec": c, "M": m, "N": n, "K": k, "ms": round(t, 4), "tflops": round(tf, 1),
+                                    "pct_mfma_f16_peak": round(100 * tf / MFMA_F16_PEAK_TFLOPS, 2)})
+                del wq
+            abi.lib.kq_set_gemm_tile_rows(0)
+            out["prefill"] = prefill
 
         # ---------------- MoE: 128 experts, top-8, hidden 2048, intermediate 768 (structurally valid random wire)
-        E, H, I, TOPK = 128, 2048, 768, 8
-        gate = synth_wire_torch("q4_k", E * I, H, 11, dev).reshape(E, I, -1)
-        up = synth_wire_torch("q4_k", E * I, H, 12, dev).reshape(E, I, -1)
-        down = synth_wire_torch("q6_k", E * H, I, 13, dev).reshape(E, H, -1)
-        gu_bytes = 2 * I * kq.bytes_per_row("q4_k", H)
-        dn_bytes = H * kq.bytes_per_row("q6_k", I)
-        moe = []
-        for T in (1, 256):
-            xt = randx((T, H), 0.5)
-            # 16 different routings, rotated per step, so that a step's experts are not the previous step's
-            glu_calls, dn_calls, touched = [], [], []
-            for r in range(16):
-                logits = torch.randn((T, E), device=dev, generator=gx)
-                idx = logits.topk(TOPK, dim=-1).indices.to(torch.int32).contiguous()
-                call, h = abi.moe_glu(xt, gate, up, "q4_k", idx)
-                glu_calls.append(call)
-                dn_calls.append(abi.gather_qmv(h, down, "q6_k", idx))
-                touched.append(int(idx.unique().numel()))
-            ne = sum(touched) / len(touched)
-            tg, _ = time_calls(torch, glu_calls, steps, warm)
-            td, _ = time_calls(torch, dn_calls, steps, warm)
-            moe.append({"tokens": T, "experts_touched": round(ne, 1), "glu_us": round(tg * 1e3, 2),
-                        "down_us": round(td * 1e3, 2),
-                        "glu_gbs": round(ne * gu_bytes / (tg * 1e-3) / 1e9, 1),
-                        "down_gbs": round(ne * dn_bytes / (td * 1e-3) / 1e9, 1),
-                        "pct_hbm_peak": round(100 * ne * (gu_bytes + dn_bytes) / ((tg + td) * 1e-3) / 1e9
-                                              / HBM_PEAK_GBS, 2)})
-        del gate, up, down
-        out["moe"] = moe
+        if want("moe"):
+            E, H, I, TOPK = 128, 2048, 768, 8
+            gate = synth_wire_torch("q4_k", E * I, H, 11, dev).reshape(E, I, -1)
+            up = synth_wire_torch("q4_k", E * I, H, 12, dev).reshape(E, I, -1)
+            down = synth_wire_torch("q6_k", E * H, I, 13, dev).reshape(E, H, -1)
+            gu_bytes = 2 * I * kq.bytes_per_row("q4_k", H)
+            dn_bytes = H * kq.bytes_per_row("q6_k", I)
+            moe = []
+            for T in (1, 256):
+                xt = randx((T, H), 0.5)
+                # 16 different routings, rotated per step, so that a step's experts are not the previous step's
+                glu_calls, dn_calls, touched = [], [], []
+                for r in range(16):
+                    logits = torch.randn((T, E), device=dev, generator=gx)
+                    idx = logits.topk(TOPK, dim=-1).indices.to(torch.int32).contiguous()
+                    call, h = abi.moe_glu(xt, gate, up, "q4_k", idx)
+                    glu_calls.append(call)
+                    dn_calls.append(abi.gather_qmv(h, down, "q6_k", idx))
+                    touched.append(int(idx.unique().numel()))
+                ne = sum(touched) / len(touched)
+                tg, _ = time_calls(torch, glu_calls, steps, warm)
+                td, _ = time_calls(torch, dn_calls, steps, warm)
+                moe.append({"tokens": T, "experts_touched": round(ne, 1), "glu_us": round(tg * 1e3, 2),
+                            "down_us": round(td * 1e3, 2),
+                            "glu_gbs": round(ne * gu_bytes / (tg * 1e-3) / 1e9, 1),
+                            "down_gbs": round(ne * dn_bytes / (td * 1e-3) / 1e9, 1),
+                            "pct_hbm_peak": round(100 * ne * (gu_bytes + dn_bytes) / ((tg + td) * 1e-3) / 1e9
+                                                  / HBM_PEAK_GBS, 2)})
+            del gate, up, down
+            out["moe"] = moe
 
         # ---------------- mxfp4 MoE: 32 experts of 2880 -> 2880, top-4, 64 tokens, f32 biases, swiglu_clamp
-        E, H, TOPK, T = 32, 2880, 4, 64
-        gate = synth_wire_torch("mxfp4", E * H, H, 21, dev).reshape(E, H, -1)
-        up = synth_wire_torch("mxfp4", E * H, H, 22, dev).reshape(E, H, -1)
-        down = synth_wire_torch("mxfp4", E * H, H, 23, dev).reshape(E, H, -1)
-        gb = torch.randn((E, H), device=dev, generator=gx) * 0.01
-        ub = torch.randn((E, H), device=dev, generator=gx) * 0.01
-        db = torch.randn((E, H), device=dev, generator=gx) * 0.01
-        xt = randx((T, H), 0.5)
-        idx = torch.randn((T, E), device=dev, generator=gx).topk(TOPK, dim=-1).indices
-        kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp", limit=7.0, gate_bias=gb, up_bias=ub,
-                             alpha=1.702)
-        tg, _ = time_calls(torch, [lambda: kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp",
-                                                                 limit=7.0, gate_bias=gb, up_bias=ub, alpha=1.702)],
-                           20, 3, graph=False)
-        h = kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp", limit=7.0, gate_bias=gb, up_bias=ub,
+        if want("moe_mxfp4"):
+            E, H, TOPK, T = 32, 2880, 4, 64
+            gate = synth_wire_torch("mxfp4", E * H, H, 21, dev).reshape(E, H, -1)
+            up = synth_wire_torch("mxfp4", E * H, H, 22, dev).reshape(E, H, -1)
+            down = synth_wire_torch("mxfp4", E * H, H, 23, dev).reshape(E, H, -1)
+            gb = torch.randn((E, H), device=dev, generator=gx) * 0.01
+            ub = torch.randn((E, H), device=dev, generator=gx) * 0.01
+            db = torch.randn((E, H), device=dev, generator=gx) * 0.01
+            xt = randx((T, H), 0.5)
+            idx = torch.randn((T, E), device=dev, generator=gx).topk(TOPK, dim=-1).indices
+            kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp", limit=7.0, gate_bias=gb, up_bias=ub,
                                  alpha=1.702)
-        td, _ = time_calls(torch, [lambda: kq.gather_qmv_kq(h, down, "mxfp4", idx, bias=db)], 20, 3, graph=False)
-        mbytes = H * kq.bytes_per_row("mxfp4", H)
-        ne = int(idx.unique().numel())
-        out["moe_mxfp4"] = {"tokens": T, "experts_touched": ne, "glu_us": round(tg * 1e3, 1),
-                            "down_us": round(td * 1e3, 1),
-                            "glu_gbs": round(ne * 2 * mbytes / (tg * 1e-3) / 1e9, 1),
-                            "down_gbs": round(ne * mbytes / (td * 1e-3) / 1e9, 1),
-                            "note": "grouped code-level MFMA kernel (biases, swiglu_clamp), timed through the Python wrapper"}
-        del gate, up, down
+            tg, _ = time_calls(torch, [lambda: kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp",
+                                                                     limit=7.0, gate_bias=gb, up_bias=ub, alpha=1.702)],
+                               20, 3, graph=False)
+            h = kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp", limit=7.0, gate_bias=gb, up_bias=ub,
+                                     alpha=1.702)
+            td, _ = time_calls(torch, [lambda: kq.gather_qmv_kq(h, down, "mxfp4", idx, bias=db)], 20, 3, graph=False)
+            mbytes = H * kq.bytes_per_row("mxfp4", H)
+            ne = int(idx.unique().numel())
+            out["moe_mxfp4"] = {"tokens": T, "experts_touched": ne, "glu_us": round(tg * 1e3, 1),
+                                "down_us": round(td * 1e3, 1),
+                                "glu_gbs": round(ne * 2 * mbytes / (tg * 1e-3) / 1e9, 1),
+                                "down_gbs": round(ne * mbytes / (td * 1e-3) / 1e9, 1),
+                                "note": "grouped code-level MFMA kernel (biases, swiglu_clamp), timed through the Python wrapper"}
+            del gate, up, down
 
         # ---------------- MoE decode (1 token, 8 of 128 experts of 2048 <-> 768) in the low-bit / fp4 codecs
-        E, H, I, TOPK = 128, 2048, 768, 8
-        dec = []
-        for c in ("iq4_xs", "iq3_s", "iq2_xxs", "mxfp4"):
-            gate = synth_wire_torch(c, E * I, H, 31, dev).reshape(E, I, -1)
-            up = synth_wire_torch(c, E * I, H, 32, dev).reshape(E, I, -1)
-            down = synth_wire_torch(c, E * H, I, 33, dev).reshape(E, H, -1)
-            calls_g, calls_d = [], []
-            for r in range(16):  # 16 routings rotated per step
-                ix = torch.randperm(E, device=dev, generator=gx)[:TOPK].reshape(1, TOPK).to(torch.int32)
-                calls_g.append(abi.moe_glu(randx((1, H), 0.5), gate, up, c, ix)[0])
-                calls_d.append(abi.gather_qmv(randx((1, TOPK, I), 0.5), down, c, ix))
-            tg, _ = time_calls(torch, calls_g, 200, 20)
-            td, _ = time_calls(torch, calls_d, 200, 20)
-            bg, bd = TOPK * 2 * I * kq.bytes_per_row(c, H), TOPK * H * kq.bytes_per_row(c, I)
-            dec.append({"codec": c, "tokens": 1, "experts": TOPK, "glu_us": round(tg * 1e3, 2), "down_us": round(td * 1e3, 2),
-                        "glu_gbs": round(bg / (tg * 1e-3) / 1e9, 1), "down_gbs": round(bd / (td * 1e-3) / 1e9, 1)})
-            del gate, up, down, calls_g, calls_d
-        out["moe_decode_lowbit"] = dec
+        if want("moe_decode_lowbit"):
+            E, H, I, TOPK = 128, 2048, 768, 8
+            dec = []
+            for c in ("iq4_xs", "iq3_s", "iq2_xxs", "mxfp4"):
+                gate = synth_wire_torch(c, E * I, H, 31, dev).reshape(E, I, -1)
+                up = synth_wire_torch(c, E * I, H, 32, dev).reshape(E, I, -1)
+                down = synth_wire_torch(c, E * H, I, 33, dev).reshape(E, H, -1)
+                calls_g, calls_d = [], []
+                for r in range(16):  # 16 routings rotated per step
+                    ix = torch.randperm(E, device=dev, generator=gx)[:TOPK].reshape(1, TOPK).to(torch.int32)
+                    calls_g.append(abi.moe_glu(randx((1, H), 0.5), gate, up, c, ix)[0])
+                    calls_d.append(abi.gather_qmv(randx((1, TOPK, I), 0.5), down, c, ix))
+                tg, _ = time_calls(torch, calls_g, 200, 20)
+                td, _ = time_calls(torch, calls_d, 200, 20)
+                bg, bd = TOPK * 2 * I * kq.bytes_per_row(c, H), TOPK * H * kq.bytes_per_row(c, I)
+                dec.append({"codec": c, "tokens": 1, "experts": TOPK, "glu_us": round(tg * 1e3, 2), "down_us": round(td * 1e3, 2),
+                            "glu_gbs": round(bg / (tg * 1e-3) / 1e9, 1), "down_gbs": round(bd / (td * 1e-3) / 1e9, 1)})
+                del gate, up, down, calls_g, calls_d
+            out["moe_decode_lowbit"] = dec
 
         # ---------------- low-bit codecs, M = 1, 8192 -> 8192 (all five minted by kq.quantize)
-        lowbit = []
-        for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs"):
-            n = k = 8192
-            wb = n * kq.bytes_per_row(c, k)
-            wq = quantized_weights(kq, torch, c, n, k, 7, dev, unique_rows=None if c in ("q2_k", "q3_k", "iq4_xs") else 512)
-            cps = cold_copies(torch, wq, wb)
-            t, _ = time_calls(torch, [abi.qmm(x.new_ones((1, k)), w, c, n, k) for w in cps], steps, warm)
-            lowbit.append({"codec": c, "N": n, "K": k, "M": 1, "us": round(t * 1e3, 2),
-                           "cold_gbs": round(wb / (t * 1e-3) / 1e9, 1),
-                           "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
-            del cps, wq
-        out["lowbit"] = lowbit
+        if want("lowbit"):
+            lowbit = []
+            for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs"):
+                n = k = 8192
+                wb = n * kq.bytes_per_row(c, k)
+                wq = quantized_weights(kq, torch, c, n, k, 7, dev, unique_rows=None if c in ("q2_k", "q3_k", "iq4_xs") else 512)
+                cps = cold_copies(torch, wq, wb)
+                t, _ = time_calls(torch, [abi.qmm(x.new_ones((1, k)), w, c, n, k) for w in cps], steps, warm)
+                lowbit.append({"codec": c, "N": n, "K": k, "M": 1, "us": round(t * 1e3, 2),
+                               "cold_gbs": round(wb / (t * 1e-3) / 1e9, 1),
+                               "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
+                del cps, wq
+            out["lowbit"] = lowbit
 
         # ---------------- dequantize to f16 (random structurally valid wire): bytes = wire in + 2 N K out
-        deq = []
-        for c, n, k in (("q4_k", 4096, 4096), ("q4_k", 28672, 8192), ("q6_k", 28672, 8192), ("iq3_s", 28672, 8192),
-                        ("q8_0", 28672, 8192)):
-            wb = n * kq.bytes_per_row(c, k)
-            total = wb + 2 * n * k
-            wq = synth_wire_torch(c, n, k, 9, dev)
-            # rotate over inputs AND outputs so that neither side is served by the last-level cache
-            cps = cold_copies(torch, wq, total)
-            outs = [torch.empty((n, k), dtype=torch.float16, device=dev) for _ in cps]
-            t, _ = time_calls(torch, [abi.dequantize(w, c, n, k, o) for w, o in zip(cps, outs)], 200, 20)
-            deq.append({"codec": c, "N": n, "K": k, "us": round(t * 1e3, 2), "cold_gbs": round(total / (t * 1e-3) / 1e9, 1),
-                        "pct_hbm_peak": round(100 * total / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
-            del cps, outs, wq
-        out["dequantize"] = deq
+        if want("dequantize"):
+            deq = []
+            for c, n, k in (("q4_k", 4096, 4096), ("q4_k", 28672, 8192), ("q6_k", 28672, 8192), ("iq3_s", 28672, 8192),
+                            ("q8_0", 28672, 8192)):
+                wb = n * kq.bytes_per_row(c, k)
+                total = wb + 2 * n * k
+                wq = synth_wire_torch(c, n, k, 9, dev)
+                # rotate over inputs AND outputs so that neither side is served by the last-level cache
+                cps = cold_copies(torch, wq, total)
+                outs = [torch.empty((n, k), dtype=torch.float16, device=dev) for _ in cps]
+                t, _ = time_calls(torch, [abi.dequantize(w, c, n, k, o) for w, o in zip(cps, outs)], 200, 20)
+                deq.append({"codec": c, "N": n, "K": k, "us": round(t * 1e3, 2), "cold_gbs": round(total / (t * 1e-3) / 1e9, 1),
+                            "pct_hbm_peak": round(100 * total / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
+                del cps, outs, wq
+            out["dequantize"] = deq
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(base_np, codec, K, M)

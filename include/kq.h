@@ -101,7 +101,8 @@ int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void
 
 /* Tuning hook without a counterpart in the reference: workgroup tile of the prefill GEMM.  64 = 64
  * activation rows x 128 weight rows, 128 = 128 x 128, 256 = 64 x 256 on eight waves with two LDS stages
- * (q4_k only; other codecs fall back to automatic); anything else restores the automatic choice.
+ * (q4_k only; other codecs fall back to automatic), 512 = 128 x 256 on eight waves with 128-row wave tiles and
+ * direct-to-LDS loads (q4_k / q5_k; 513 = the same kernel as 128 x 128 on four waves); anything else restores the automatic choice.
  * Process-wide, not thread-safe. */
 void kq_set_gemm_tile_rows(int rows);
 /* Tuning hook without a counterpart in the reference: which skinny-M kernel dense calls use.

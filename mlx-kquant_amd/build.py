@@ -22,6 +22,7 @@ SOURCES = [
     ("kq_mfma.hip", []),
     ("kq_stream.hip", ["-Wno-inline-asm"]),
     ("kq_gemm.hip", []),
+    ("kq_gemm2.hip", ["-Wno-inline-asm"]),
     ("kq_moe.hip", []),
     ("kq_anymma.hip", ["-ffp-contract=off"]),
     # one source, three objects: its kernel families are instantiated in parallel

@@ -95,6 +95,10 @@ size_t kq_gemm_workspace_bytes(int M, int K);
 bool kq_gemm_supported(int M, int N, int K, int codec);
 int kq_launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                    hipStream_t s);
+// 128 x 256-tile prefill GEMM (q4_k / q5_k) on the outputs of the activation prepass (rows padded to 128).
+bool kq_gemm2_supported(int M, int N, int K, int codec);
+int kq_launch_gemm2(const void* xh, const void* xhl, const float* rs, const uint8_t* w, void* y, int M, int N, int K,
+                    int codec, int dtype, int shape, hipStream_t s);
 // Batched MoE path (q4_k / q5_k / q6_k, more than 16 pairs): pairs sorted by expert, one MFMA GEMM
 // per segment of <= 32 pairs.  rows = activation rows (T for the GLU op, T*R for the down op).
 bool kq_moe_grouped_supported(int P, int E, int N, int K, int codec);

@@ -13,7 +13,7 @@
 // row-per-lane ds_read_b128 fragment fetch free of bank conflicts).
 #include "kq_mma.h"
 
-static int g_gemm_tile = 0;  // kq_set_gemm_tile_rows: 64, 128 or 256 forces the tile shape, 0 = automatic
+static int g_gemm_tile = 0;  // kq_set_gemm_tile_rows: 64, 128, 256, 512 or 513 forces the tile shape, 0 = automatic
 
 namespace {
 
@@ -219,6 +219,14 @@ int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, v
   // one barrier per step instead of two and the next step is parked while this one is multiplied, measured
   // 5 - 9 % faster once every CU gets 8 or more workgroups, slower below (fewer, longer workgroups).
   int tile = g_gemm_tile;
+  // 128 x 256 tiles with 128-row wave tiles and direct-to-LDS loads (kq_gemm2.hip, q4_k / q5_k): one decoded
+  // weight fragment feeds four MFMAs instead of two.  Taken when the matrix fills the 256 CUs with whole
+  // workgroups of that size; `512` forces it, `513` its 128 x 128 / four-wave form.
+  if (tile == 512 || tile == 513 || (tile == 0 && M >= 256 && (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 256)) {
+    const int rc = kq_launch_gemm2(xh, xhl, rs, w, y, M, N, K, C, DT, tile == 513 ? 1 : 0, s);
+    if (rc != KQ_ERR_UNSUPPORTED) return rc;
+  }
+  if (tile == 512 || tile == 513) tile = 0;
   if (tile == 256 && C != KQ_Q4_K) tile = 0;
   if (tile == 0) {
     const int64_t wgs = (int64_t)((M + 63) / 64) * ((N + 255) / 256);
@@ -270,4 +278,6 @@ int kq_launch_act_prepass(const void* x, void* xh, void* xhl, float* rs, int M, 
   return KQ_OK;
 }
 
-extern "C" void kq_set_gemm_tile_rows(int rows) { g_gemm_tile = (rows == 64 || rows == 128 || rows == 256) ? rows : 0; }
+extern "C" void kq_set_gemm_tile_rows(int rows) {
+  g_gemm_tile = (rows == 64 || rows == 128 || rows == 256 || rows == 512 || rows == 513) ? rows : 0;
+}

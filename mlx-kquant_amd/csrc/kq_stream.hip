@@ -27,13 +27,15 @@
 #include <type_traits>
 
 #include "kq_decode.h"
+#include "kq_dma.h"
 
 namespace {
+
+using namespace kqdma;
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int ST_WAVES = 4;
@@ -66,28 +68,6 @@ __device__ __forceinline__ uint32_t opaque_sgpr(uint32_t v) {
 }
 __device__ __forceinline__ void tie_v(u32x4& v) { asm volatile("" : "+v"(v)); }
 
-// ---- direct-to-LDS loads and their waits.  LDS address of lane l: lds + 16 l (4 l for the 2-byte form).
-__device__ __forceinline__ void dma16(const uint8_t* sbase, uint32_t voff, uint32_t lds) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(sbase)
-               : "memory", "m0");
-}
-__device__ __forceinline__ void dma2(const uint8_t* sbase, uint32_t voff, uint32_t lds) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2" ::"s"(lds), "v"(voff), "s"(sbase)
-               : "memory", "m0");
-}
-__device__ __forceinline__ u32x4 gload16(const void* p) {
-  u32x4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-  return v;
-}
-template <int N>
-__device__ __forceinline__ void vmwait() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-__device__ __forceinline__ void lgkm_drain() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ uint32_t lds_addr(const void* p) {
-  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t*)p;
-}
 __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();

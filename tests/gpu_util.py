@@ -42,3 +42,26 @@ def rel_l2(got_bits, want_bits, dtype):
     g = O.bits_to_f32(got_bits, dtype).astype(np.float64)
     w = O.bits_to_f32(want_bits, dtype).astype(np.float64)
     return float(np.linalg.norm(g - w) / (np.linalg.norm(w) + 1e-30))
+
+
+def synth_wire_dev(codec, rows, K, seed):
+    """Structurally valid random wire minted on the GPU (random code bytes, sane scale fields so that decode stays
+    finite) for matrices too large to draw with numpy in a test: uint8 [rows, bytes_per_row]."""
+    wpb, bpb = O.geometry(codec)
+    nb = rows * (K // wpb)
+    g = torch.Generator(device=dev())
+    g.manual_seed(seed)
+    wire = torch.randint(0, 256, (nb, bpb), dtype=torch.uint8, device=dev(), generator=g)
+    d = (torch.rand(nb, 2, device=dev(), generator=g) * 0.006 + 0.004).to(torch.float16).view(torch.uint8).reshape(nb, 4)
+    off = {"q4_k": (0, 2), "q5_k": (0, 2), "q4_1": (0, 2), "q5_1": (0, 2), "q6_k": (208,), "q3_k": (108,),
+           "q2_k": (80, 82)}.get(codec, (0,))
+    if codec == "mxfp4":
+        wire[:, 0] = torch.randint(121, 130, (nb,), dtype=torch.uint8, device=dev(), generator=g)
+    elif codec == "nvfp4":
+        wire[:, 0:4] = torch.randint(0x08, 0x19, (nb, 4), dtype=torch.uint8, device=dev(), generator=g)
+    elif codec == "iq1_m":
+        raise ValueError("iq1_m keeps its scale in nibbles: mint it with oracle_lib.synth_wire")
+    else:
+        for i, o in enumerate(off):
+            wire[:, o:o + 2] = d[:, 2 * i:2 * i + 2]
+    return wire.reshape(rows, K // wpb * bpb)

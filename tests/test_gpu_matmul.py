@@ -222,9 +222,10 @@ def test_qmm_prefill_every_codec(kq, codec):
 
 
 def test_qmm_prefill_gemm_tile_variants(kq):
-    """The 128 x 128 and the two-stage 64 x 256 tile variants (kq_set_gemm_tile_rows) give the same rounded outputs
-    as the default 64 x 128 one: all feed the same exact products to f32 accumulators in the same order.  N is no
-    multiple of 256, M none of 64, and K spans several steps so that both LDS stages are reused."""
+    """The 128 x 128, the two-stage 64 x 256 and the 128 x 256 direct-to-LDS tile variants (kq_set_gemm_tile_rows)
+    give the same rounded outputs as the 64 x 128 one: all feed the same exact products to f32 accumulators in the
+    same order.  N is no multiple of 256, M none of 64, and K spans several steps so that both LDS stages are
+    reused (q6_k has no 128 x 256 kernel and falls back)."""
     M, N, K = 200, 384, 2048
     lib = kq._load()
     for codec in ("q4_k", "q5_k", "q6_k"):
@@ -233,14 +234,14 @@ def test_qmm_prefill_gemm_tile_variants(kq):
         want = O.qmm(xb, wire, codec, True, "bfloat16")
         outs = []
         try:
-            for rows in (128, 256, 64):
+            for rows in (128, 256, 512, 513, 64):
                 lib.kq_set_gemm_tile_rows(rows)
                 got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
                 assert rel_l2(got, want, "bfloat16") <= TOL, (codec, rows)
                 outs.append(got)
         finally:
             lib.kq_set_gemm_tile_rows(0)
-        assert np.array_equal(outs[0], outs[2]) and np.array_equal(outs[1], outs[2]), codec
+        assert all(np.array_equal(o, outs[-1]) for o in outs[:-1]), codec
 
 
 @pytest.mark.parametrize("K", [256, 512, 768])
@@ -257,6 +258,26 @@ def test_qmm_prefill_gemm_two_stage_short_k(kq, K):
     finally:
         lib.kq_set_gemm_tile_rows(0)
     assert rel_l2(got, want, "float16") <= TOL
+
+
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k"])
+def test_qmm_prefill_gemm_128x256_tiles(kq, codec):
+    """The direct-to-LDS kernels (512: 128 x 256 tiles, K steps of 128; 513: 128 x 128 tiles, K steps of 64): one,
+    two and nine superblocks of K (prologue only, both wire stages, stage reuse), ragged M and N tiles, both
+    activation dtypes."""
+    lib = kq._load()
+    try:
+      for rows in (512, 513):
+        lib.kq_set_gemm_tile_rows(rows)
+        for M, N, K, dtype in ((9, 40, 256, "bfloat16"), (130, 257, 512, "float16"), (300, 520, 2304, "bfloat16"),
+                               (128, 256, 1024, "bfloat16")):
+            wire = _wire(codec, N, K, seed=63)
+            xb, xt = make_x((M, K), dtype, seed=64)
+            got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+            want = O.qmm(xb, wire, codec, True, dtype)
+            assert rel_l2(got, want, dtype) <= TOL, (codec, rows, M, N, K, dtype)
+    finally:
+        lib.kq_set_gemm_tile_rows(0)
 
 
 def test_qmm_prefill_gemm_wide_dynamic_range(kq):
