@@ -492,7 +492,8 @@ bool kq_anymma_moe_supported(int P, int E, int N, int K, int codec) {
 // x: [rows][K]; pair p reads row p / x_div and expert idx[p]; out [P][N].
 int kq_launch_anymma_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
                          const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
-                         int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, hipStream_t s) {
+                         int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, KqOutMap om,
+                         hipStream_t s) {
   if (!kq_anymma_moe_supported(P, E, N, K, codec) || (reinterpret_cast<uintptr_t>(x) & 15) ||
       (reinterpret_cast<uintptr_t>(ws) & 255))
     return KQ_ERR_UNSUPPORTED;
@@ -522,6 +523,6 @@ int kq_launch_anymma_moe(const void* x, const uint8_t* w, const uint8_t* w2, con
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
   a.alpha = alpha;
-  a.om = kq_out_map();
+  a.om = om;
   return dispatch_any(codec, a, glu ? 2 : 1, dtype, P, E, s);
 }

@@ -47,13 +47,6 @@ std::mutex g_grid_mu;
 const uint8_t* g_grids[kMaxDevices] = {};
 void* g_scratch[kMaxDevices] = {};  // per-device address of kq_noalloc_scratch
 
-thread_local KqOutMap g_out_map = {1, 1, 0, 0};
-// Sets the calling thread's output map for the launches inside a scope.
-struct OutMapScope {
-  explicit OutMapScope(KqOutMap m) { g_out_map = m; }
-  ~OutMapScope() { g_out_map = KqOutMap{1, 1, 0, 0}; }
-};
-
 bool codec_ok(int c) { return c >= 0 && c < KQ_NUM_CODECS; }
 bool half_dtype(int dt) { return dt == KQ_F16 || dt == KQ_BF16; }
 
@@ -66,8 +59,6 @@ int kq_set_error(int code, const char* fmt, ...) {
   va_end(ap);
   return code;
 }
-
-const KqOutMap& kq_out_map(void) { return g_out_map; }
 
 const uint8_t* kq_device_grids(void) {
   int dev = -1;
@@ -235,7 +226,7 @@ size_t kq_gather_qmm_workspace_size(int B, int M, int E, int N, int K, int trans
 static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
                            const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
                            int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
-                           size_t ws_bytes, hipStream_t s);
+                           size_t ws_bytes, KqOutMap om, hipStream_t s);
 
 int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_dev, const uint32_t* rhs_idx_dev,
                   void* out_dev, int B, int M, int E, int N, int K, int64_t x_batch_stride,
@@ -255,7 +246,7 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (!transpose)
     return kq_launch_gather_nt_generic(x_dev, static_cast<const uint8_t*>(w_dev), lhs_idx_dev, rhs_idx_dev, out_dev, B,
-                                       M, N, K, x_batch_stride, w_expert_stride_bytes, codec, dtype, s);
+                                       M, E, N, K, x_batch_stride, w_expert_stride_bytes, codec, dtype, s);
   // many output rows: gather them into a dense matrix and run the expert-grouped kernels
   int64_t P;
   if (workspace_dev && gather_batched_shape(B, M, E, N, K, transpose, codec, &P) &&
@@ -271,26 +262,26 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
       if (rcr) return rcr;
       const int rcg = try_moe_grouped("gather_qmm", xg, w_dev, nullptr, idx_rows, nullptr, nullptr, out_dev, (int)P, 1, E,
                                       N, K, w_expert_stride_bytes, 0, 0, 0.f, 0.f, codec, dtype, wsb + used,
-                                      workspace_bytes - used, s);
+                                      workspace_bytes - used, KQ_OUT_ROWS, s);
       if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
     }
   }
   {
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
                                            out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0, 0, 0.f,
-                                           codec, dtype, s);
+                                           codec, dtype, E, KQ_OUT_ROWS, s);
     if (rct != KQ_ERR_UNSUPPORTED) return rct;
   }
   {
     // legacy / IQ / fp4 stacks, one row per entry: the code-level skinny kernel, one entry per grid row
     const int rcc = kq_launch_codes_gather(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
                                   nullptr, nullptr, out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0,
-                                  0, 0.f, 0.f, codec, dtype, s);
+                                  0, 0.f, 0.f, codec, dtype, E, KQ_OUT_ROWS, s);
     if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
   }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, lhs_idx_dev, rhs_idx_dev,
                                   nullptr, nullptr, out_dev, B, M, N, K, 1, x_batch_stride, w_expert_stride_bytes, 0,
-                                  0, 0.f, 0.f, codec, dtype, s);
+                                  0, 0.f, 0.f, codec, dtype, E, KQ_OUT_ROWS, s);
 }
 
 static int check_moe(const char* op, int T, int R, int E, int N, int K, int codec, int dtype) {
@@ -318,7 +309,7 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
                            const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
                            int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
-                           size_t ws_bytes, hipStream_t s) {
+                           size_t ws_bytes, KqOutMap om, hipStream_t s) {
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
@@ -329,7 +320,7 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
         return kq_set_error(KQ_ERR_WORKSPACE, "%s: workspace of %zu bytes required (got %zu)", op, need, ws ? ws_bytes : 0);
       const int rcc = kq_launch_codes_moe(x, static_cast<const uint8_t*>(w), static_cast<const uint8_t*>(w2), idx, bias,
                                           bias2, out, (int)P, E, N, K, glu ? R : 1, estride, glu, act, limit, alpha, codec,
-                                          dtype, ws, s);
+                                          dtype, ws, om, s);
       if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
     }
     // q2_k / q3_k, and q4_k ... q6_k with biases or swiglu_clamp: the any-codec matrix-core path
@@ -338,20 +329,21 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
     if (!ws || ws_bytes < need)
       return kq_set_error(KQ_ERR_WORKSPACE, "%s: workspace of %zu bytes required (got %zu)", op, need, ws ? ws_bytes : 0);
     return kq_launch_anymma_moe(x, static_cast<const uint8_t*>(w), static_cast<const uint8_t*>(w2), idx, bias, bias2, out,
-                                (int)P, E, N, K, glu ? R : 1, estride, glu, act, limit, alpha, codec, dtype, ws, s);
+                                (int)P, E, N, K, glu ? R : 1, estride, glu, act, limit, alpha, codec, dtype, ws, om, s);
   }
   const int rows = glu ? T : (int)P;
   const size_t need = kq_moe_grouped_workspace_bytes(rows, (int)P, E, K);
   if (!ws || ws_bytes < need)
     return kq_set_error(KQ_ERR_WORKSPACE, "%s: workspace of %zu bytes required (got %zu)", op, need, ws ? ws_bytes : 0);
   return kq_launch_moe_grouped(x, static_cast<const uint8_t*>(w), static_cast<const uint8_t*>(w2), idx, out, rows,
-                               (int)P, E, N, K, glu ? R : 1, estride, glu, act, limit, codec, dtype, ws, s);
+                               (int)P, E, N, K, glu ? R : 1, estride, glu, act, limit, codec, dtype, ws, om, s);
 }
 
-int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_w_dev, const uint32_t* idx_dev,
-                      const float* gate_bias_dev, const float* up_bias_dev, void* out_dev, int T, int R, int E, int N,
-                      int K, int act, float limit, float alpha, int codec, int dtype, void* workspace_dev,
-                      size_t workspace_bytes, void* stream) {
+// om: where the result of pair (t, r) goes; the exported op writes row t R + r of a 16-bit matrix
+static int moe_glu_gather_impl(const void* x_dev, const void* gate_w_dev, const void* up_w_dev, const uint32_t* idx_dev,
+                               const float* gate_bias_dev, const float* up_bias_dev, void* out_dev, int T, int R, int E,
+                               int N, int K, int act, float limit, float alpha, int codec, int dtype, void* workspace_dev,
+                               size_t workspace_bytes, KqOutMap om, void* stream) {
   const char* op = "moe_glu_gather_kq";
   int rc = check_moe(op, T, R, E, N, K, codec, dtype);
   if (rc) return rc;
@@ -375,14 +367,14 @@ int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_
   const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
   {
     const int rcg = try_moe_grouped(op, x_dev, gate_w_dev, up_w_dev, idx_dev, gate_bias_dev, up_bias_dev, out_dev, T, R, E,
-                                    N, K, estride, 1, act, limit, alpha, codec, dtype, workspace_dev, workspace_bytes,
+                                    N, K, estride, 1, act, limit, alpha, codec, dtype, workspace_dev, workspace_bytes, om,
                                     static_cast<hipStream_t>(stream));
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
   }
   if (!biased) {
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(gate_w_dev),
                                            static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, out_dev, T * R, 1, N,
-                                           K, R, K, estride, 1, act, limit, codec, dtype,
+                                           K, R, K, estride, 1, act, limit, codec, dtype, E, om,
                                            static_cast<hipStream_t>(stream));
     if (rct != KQ_ERR_UNSUPPORTED) return rct;
   }
@@ -390,19 +382,27 @@ int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_
     // legacy / IQ / fp4 stacks, one row per entry: the code-level skinny kernel, one entry per grid row
     const int rcc = kq_launch_codes_gather(x_dev, static_cast<const uint8_t*>(gate_w_dev),
                                   static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, gate_bias_dev, up_bias_dev,
-                                  out_dev, T * R, 1, N, K, R, K, estride, 1, act, limit, alpha, codec, dtype,
+                                  out_dev, T * R, 1, N, K, R, K, estride, 1, act, limit, alpha, codec, dtype, E, om,
                                   static_cast<hipStream_t>(stream));
     if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
   }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(gate_w_dev),
                                   static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, gate_bias_dev, up_bias_dev,
-                                  out_dev, T * R, 1, N, K, R, K, estride, 1, act, limit, alpha, codec, dtype,
+                                  out_dev, T * R, 1, N, K, R, K, estride, 1, act, limit, alpha, codec, dtype, E, om,
                                   static_cast<hipStream_t>(stream));
 }
 
-int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev, const float* bias_dev, void* out_dev,
-                  int T, int R, int E, int N, int K, int codec, int dtype, void* workspace_dev, size_t workspace_bytes,
-                  void* stream) {
+int kq_moe_glu_gather(const void* x_dev, const void* gate_w_dev, const void* up_w_dev, const uint32_t* idx_dev,
+                      const float* gate_bias_dev, const float* up_bias_dev, void* out_dev, int T, int R, int E, int N,
+                      int K, int act, float limit, float alpha, int codec, int dtype, void* workspace_dev,
+                      size_t workspace_bytes, void* stream) {
+  return moe_glu_gather_impl(x_dev, gate_w_dev, up_w_dev, idx_dev, gate_bias_dev, up_bias_dev, out_dev, T, R, E, N, K, act,
+                             limit, alpha, codec, dtype, workspace_dev, workspace_bytes, KQ_OUT_ROWS, stream);
+}
+
+static int gather_qmv_impl(const void* x_dev, const void* w_dev, const uint32_t* idx_dev, const float* bias_dev,
+                           void* out_dev, int T, int R, int E, int N, int K, int codec, int dtype, void* workspace_dev,
+                           size_t workspace_bytes, KqOutMap om, void* stream) {
   const char* op = "gather_qmv_kq";
   int rc = check_moe(op, T, R, E, N, K, codec, dtype);
   if (rc) return rc;
@@ -413,26 +413,33 @@ int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev,
   const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
   {
     const int rcg = try_moe_grouped(op, x_dev, w_dev, nullptr, idx_dev, bias_dev, nullptr, out_dev, T, R, E, N, K, estride,
-                                    0, 0, 0.f, 0.f, codec, dtype, workspace_dev, workspace_bytes,
+                                    0, 0, 0.f, 0.f, codec, dtype, workspace_dev, workspace_bytes, om,
                                     static_cast<hipStream_t>(stream));
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
   }
   if (!bias_dev) {
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, out_dev,
-                                           T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype,
+                                           T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype, E, om,
                                            static_cast<hipStream_t>(stream));
     if (rct != KQ_ERR_UNSUPPORTED) return rct;
   }
   {
     // legacy / IQ / fp4 stacks, one row per entry: the code-level skinny kernel, one entry per grid row
     const int rcc = kq_launch_codes_gather(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, bias_dev,
-                                  nullptr, out_dev, T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype,
+                                  nullptr, out_dev, T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype, E, om,
                                   static_cast<hipStream_t>(stream));
     if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
   }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, bias_dev,
-                                  nullptr, out_dev, T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype,
+                                  nullptr, out_dev, T * R, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype, E, om,
                                   static_cast<hipStream_t>(stream));
+}
+
+int kq_gather_qmv(const void* x_dev, const void* w_dev, const uint32_t* idx_dev, const float* bias_dev, void* out_dev,
+                  int T, int R, int E, int N, int K, int codec, int dtype, void* workspace_dev, size_t workspace_bytes,
+                  void* stream) {
+  return gather_qmv_impl(x_dev, w_dev, idx_dev, bias_dev, out_dev, T, R, E, N, K, codec, dtype, workspace_dev,
+                         workspace_bytes, KQ_OUT_ROWS, stream);
 }
 
 
@@ -480,31 +487,26 @@ int kq_gather_qmm_seg(const void* x_dev, const void* w_dev, const uint32_t* map_
   uint8_t* wsb = static_cast<uint8_t*>(workspace_dev);
   uint32_t* row_expert = reinterpret_cast<uint32_t*>(wsb);
   const size_t used = align256((size_t)rows * 4);
-  // the grouped kernels leave out rows whose expert id is out of range; the per-row kernels know no such
-  // marker, so there an uncovered row is computed against expert 0
-  const bool grouped = kq_moe_workspace_size((int)rows, 1, E, N, K, 0, codec, dtype) > 0;
-  rc = kq_launch_tiles_to_rows(map_dev, counts_dev, (int)n_tiles, (int)rows, E, grouped ? 0xffffffffu : 0u, row_expert, s);
+  // rows no tile covers carry an expert id outside the stack, which every kernel below leaves out
+  rc = kq_launch_tiles_to_rows(map_dev, counts_dev, (int)n_tiles, (int)rows, E, 0xffffffffu, row_expert, s);
   if (rc) return rc;
   const int64_t estride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
-  if (grouped) {
+  if (kq_moe_workspace_size((int)rows, 1, E, N, K, 0, codec, dtype) > 0) {
     const int rcg = try_moe_grouped(op, x_dev, w_dev, nullptr, row_expert, nullptr, nullptr, out_dev, (int)rows, 1, E, N, K,
-                                    estride, 0, 0, 0.f, 0.f, codec, dtype, wsb + used, workspace_bytes - used, s);
+                                    estride, 0, 0, 0.f, 0.f, codec, dtype, wsb + used, workspace_bytes - used, KQ_OUT_ROWS, s);
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
-    // an unaligned x: rerun the row list with the marker the per-row kernels can take
-    rc = kq_launch_tiles_to_rows(map_dev, counts_dev, (int)n_tiles, (int)rows, E, 0u, row_expert, s);
-    if (rc) return rc;
   }
   const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, row_expert, out_dev,
-                                         (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype, s);
+                                         (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, codec, dtype, E, KQ_OUT_ROWS, s);
   if (rct != KQ_ERR_UNSUPPORTED) return rct;
   {
     // legacy / IQ / fp4 stacks, one row per entry: the code-level skinny kernel, one entry per grid row
     const int rcc = kq_launch_codes_gather(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, row_expert, nullptr,
-                                  nullptr, out_dev, (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype, s);
+                                  nullptr, out_dev, (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype, E, KQ_OUT_ROWS, s);
     if (rcc != KQ_ERR_UNSUPPORTED) return rcc;
   }
   return kq_launch_gather_generic(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, row_expert, nullptr,
-                                  nullptr, out_dev, (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype, s);
+                                  nullptr, out_dev, (int)rows, 1, N, K, 1, K, estride, 0, 0, 0.f, 0.f, codec, dtype, E, KQ_OUT_ROWS, s);
 }
 
 }  // extern "C"
@@ -544,16 +546,16 @@ int kq_moe_glu_gather_shexp(const void* x_dev, const void* gate_w_dev, const voi
   uint8_t* sub = wsb + align256((size_t)T * 4);
   const size_t sub_bytes = workspace_bytes - align256((size_t)T * 4);
   if (R > 0) {
-    OutMapScope scope(KqOutMap{R, R + 1, 0, 0});  // slot r of token t -> row t (R + 1) + r
-    rc = kq_moe_glu_gather(x_dev, gate_w_dev, up_w_dev, idx_dev, nullptr, nullptr, out_dev, T, R, E, N, K, act, 0.f, 0.f,
-                           codec, dtype, sub, sub_bytes, stream);
+    // slot r of token t -> row t (R + 1) + r
+    rc = moe_glu_gather_impl(x_dev, gate_w_dev, up_w_dev, idx_dev, nullptr, nullptr, out_dev, T, R, E, N, K, act, 0.f, 0.f,
+                             codec, dtype, sub, sub_bytes, KqOutMap{R, R + 1, 0, 0}, stream);
     if (rc) return rc;
   }
   rc = kq_launch_pad_idx(nullptr, idx0, T, 1, s);  // S = 1: every entry is the padded slot, i.e. 0
   if (rc) return rc;
-  OutMapScope scope(KqOutMap{1, R + 1, R, 0});  // token t -> row t (R + 1) + R
-  return kq_moe_glu_gather(x_dev, shexp_gate_w_dev, shexp_up_w_dev, idx0, nullptr, nullptr, out_dev, T, 1, 1, N, K, act, 0.f,
-                           0.f, shexp_codec, dtype, sub, sub_bytes, stream);
+  // token t -> row t (R + 1) + R
+  return moe_glu_gather_impl(x_dev, shexp_gate_w_dev, shexp_up_w_dev, idx0, nullptr, nullptr, out_dev, T, 1, 1, N, K, act,
+                             0.f, 0.f, shexp_codec, dtype, sub, sub_bytes, KqOutMap{1, R + 1, R, 0}, stream);
 }
 
 size_t kq_gather_qmv_mix_workspace_size(int T, int S, int E, int N, int K, int codec, int shexp_codec, int dtype) {
@@ -607,18 +609,18 @@ static int gather_qmv_mix_impl(const char* op, const void* x_dev, const void* w_
   }
   uint8_t* sub = wsb + o;
   const size_t sub_bytes = workspace_bytes - o;
-  {
-    OutMapScope scope(KqOutMap{1, 1, 0, 1});  // f32 slot results [T][S][N]
-    rc = kq_gather_qmv(x_dev, w_dev, idx_all, bias_dev, yf, T, S, E, N, K, codec, dtype, sub, sub_bytes, stream);
-    if (rc) return rc;
-  }
+  // f32 slot results [T][S][N]
+  rc = gather_qmv_impl(x_dev, w_dev, idx_all, bias_dev, yf, T, S, E, N, K, codec, dtype, sub, sub_bytes,
+                       KqOutMap{1, 1, 0, 1}, stream);
+  if (rc) return rc;
   if (shared) {
     // rows x[t][S - 1] -> dense [T][K], expert ids 0; the shared expert is a one-matrix stack
     rc = kq_launch_gather_rows(static_cast<const uint16_t*>(x_dev) + (size_t)(S - 1) * K, nullptr, nullptr, xs, idx0, T, 1, K,
                                (int64_t)S * K, s);
     if (rc) return rc;
-    OutMapScope scope(KqOutMap{1, S, S - 1, 1});  // token t -> slot row t S + S - 1, f32
-    rc = kq_gather_qmv(xs, shexp_w_dev, idx0, nullptr, yf, T, 1, 1, N, K, shexp_codec, dtype, sub, sub_bytes, stream);
+    // token t -> slot row t S + S - 1, f32
+    rc = gather_qmv_impl(xs, shexp_w_dev, idx0, nullptr, yf, T, 1, 1, N, K, shexp_codec, dtype, sub, sub_bytes,
+                         KqOutMap{1, S, S - 1, 1}, stream);
     if (rc) return rc;
   }
   return kq_launch_mix_slots(yf, scores_dev, out_dev, T, S, N, dtype, s);

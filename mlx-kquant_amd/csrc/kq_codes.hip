@@ -358,6 +358,7 @@ struct CkArgs {
   int64_t x_item_stride, w_expert_stride;
   float limit, alpha;
   KqOutMap om;
+  int E;  // gathered calls: items whose expert id is >= E are skipped (output rows left untouched)
 };
 
 __device__ __forceinline__ void wave_sync() {
@@ -409,6 +410,7 @@ __global__ __launch_bounds__((64 * WV), (WV == 4 ? 2 : 1)) void codes_skinny_ker
   const int ncols = N - n0 < TILE_N ? N - n0 : TILE_N;
   const int item = GMODE ? (int)blockIdx.y : 0;
   const uint32_t expert = GMODE ? a.rhs[item] : 0u;
+  if (GMODE && expert >= (uint32_t)a.E) return;  // uniform over the workgroup, ahead of every barrier
   const uint8_t* wmat = a.w + (GMODE ? (size_t)expert * (size_t)a.w_expert_stride : 0);
   const uint8_t* wmat2 = GMODE == 2 ? a.w2 + (size_t)expert * (size_t)a.w_expert_stride : wmat;
   const uint8_t* w_last = wmat + (size_t)N * row_bytes - 16;    // the last 16 bytes of the matrix
@@ -1062,7 +1064,8 @@ size_t kq_codes_moe_workspace_bytes(int P, int E) {
 // x: [rows][K]; pair p reads row p / x_div and expert idx[p]; out [P][N].
 int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
                         const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
-                        int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, hipStream_t s) {
+                        int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, KqOutMap om,
+                        hipStream_t s) {
   if (!kq_codes_moe_supported(P, E, N, K, codec) || (reinterpret_cast<uintptr_t>(x) & 15) ||
       (reinterpret_cast<uintptr_t>(ws) & 255))
     return KQ_ERR_UNSUPPORTED;
@@ -1091,7 +1094,7 @@ int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, cons
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
   a.alpha = alpha;
-  a.om = kq_out_map();
+  a.om = om;
   switch (codec) {
 #define KQ_CASE(c) \
   case c:          \
@@ -1151,7 +1154,7 @@ bool kq_codes_gather_supported(int M, int N, int K, int codec) {
 int kq_launch_codes_gather(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs, const uint32_t* rhs,
                            const float* bias, const float* bias2, void* out, int B, int M, int N, int K, int x_div,
                            int64_t x_batch_stride, int64_t w_expert_stride, int glu, int act, float limit, float alpha,
-                           int codec, int dtype, hipStream_t s) {
+                           int codec, int dtype, int E, KqOutMap om, hipStream_t s) {
   if (!kq_codes_gather_supported(M, N, K, codec) || !rhs || B <= 0 || B > 65535 || (reinterpret_cast<uintptr_t>(x) & 15) ||
       (K & 7) || (x_batch_stride & 7) || (glu && !w2))
     return KQ_ERR_UNSUPPORTED;
@@ -1175,7 +1178,8 @@ int kq_launch_codes_gather(const void* x, const uint8_t* w, const uint8_t* w2, c
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
   a.alpha = alpha;
-  a.om = kq_out_map();
+  a.om = om;
+  a.E = E;
   switch (codec) {
 #define KQ_CASE(c)                                                                                               \
   case c:                                                                                                        \

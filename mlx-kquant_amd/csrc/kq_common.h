@@ -39,14 +39,14 @@ __host__ __device__ constexpr KqGeom kq_geom(int c) {
 
 // Where the gathered / grouped kernels put the result of pair p: output row (p / in) * out + p % in + off,
 // as 16-bit values of the activation dtype or (f32 != 0) as float.  The default {1, 1, 0, 0} is row p,
-// activation dtype.  The fused MoE ops that interleave a shared-expert slot or mix the slots in f32 set
-// another map for the calling thread around their launches (kq_api.cpp); launchers copy kq_out_map().
+// activation dtype.  The fused MoE ops that interleave a shared-expert slot or mix the slots in f32 pass
+// another map to the launchers (kq_api.cpp).
 struct KqOutMap {
   int in, out, off, f32;
 };
+constexpr KqOutMap KQ_OUT_ROWS = {1, 1, 0, 0};
 
 // ---- host-side plumbing (kq_api.cpp) ----
-const KqOutMap& kq_out_map(void);
 int kq_set_error(int code, const char* fmt, ...);
 // Device copy of the IQ codebooks for the current device (uploaded once per device).
 const uint8_t* kq_device_grids(void);
@@ -66,12 +66,13 @@ int kq_launch_gemv_generic(const void* x, const uint8_t* w, void* y, int M, int 
 int kq_launch_gemm_nt_generic(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec,
                               int dtype, hipStream_t s);
 int kq_launch_gather_nt_generic(const void* x, const uint8_t* w, const uint32_t* lhs, const uint32_t* rhs, void* out,
-                                int B, int M, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride, int codec,
-                                int dtype, hipStream_t s);
+                                int B, int M, int E, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride,
+                                int codec, int dtype, hipStream_t s);
 int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
                              const uint32_t* rhs, const float* bias, const float* bias2, void* out, int B, int M,
                              int N, int K, int x_div, int64_t x_batch_stride, int64_t w_expert_stride, int glu,
-                             int act, float limit, float alpha, int codec, int dtype, hipStream_t s);
+                             int act, float limit, float alpha, int codec, int dtype, int E, KqOutMap om,
+                             hipStream_t s);
 // Tuned path: returns KQ_ERR_UNSUPPORTED (without touching the error text) when no tuned kernel
 // covers the request, so the caller can fall through to the generic kernels.
 // A null / short workspace is allowed: the call then runs without its split-K plan.
@@ -86,10 +87,11 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
                          size_t ws_bytes, hipStream_t s);
 // Tuned gathered GEMV (items = (activation matrix, expert) pairs, M <= 8 rows each; with glu the
 // gate/up pair and the fused epilogue, M = 1): same fall-through contract as kq_launch_qmm_tuned.
+// The per-entry gather launchers take the stack height E and skip entries whose expert id is >= E.
 int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
                            const uint32_t* rhs, void* out, int B, int M, int N, int K, int x_div,
                            int64_t x_batch_stride, int64_t w_expert_stride, int glu, int act, float limit, int codec,
-                           int dtype, hipStream_t s);
+                           int dtype, int E, KqOutMap om, hipStream_t s);
 // Prefill GEMM (q4_k / q5_k, M > 8): needs kq_gemm_workspace_bytes(M, K) bytes of device workspace.
 size_t kq_gemm_workspace_bytes(int M, int K);
 bool kq_gemm_supported(int M, int N, int K, int codec);
@@ -105,7 +107,7 @@ bool kq_moe_grouped_supported(int P, int E, int N, int K, int codec);
 size_t kq_moe_grouped_workspace_bytes(int rows, int P, int E, int K);
 int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, void* out, int rows,
                           int P, int E, int N, int K, int x_div, int64_t w_expert_stride, int glu, int act,
-                          float limit, int codec, int dtype, void* ws, hipStream_t s);
+                          float limit, int codec, int dtype, void* ws, KqOutMap om, hipStream_t s);
 // Gathered activations of a batched gather_qmm: xg[b*M + m][:] = x[lhs[b]][m][:], idx_rows[b*M + m] = rhs[b]
 // (16-bit elements; K a multiple of 8, x and xg 16-byte aligned).  lhs == null: b; rhs == null: 0.
 int kq_launch_gather_rows(const void* x, const uint32_t* lhs, const uint32_t* rhs, void* xg, uint32_t* idx_rows, int B,
@@ -122,14 +124,15 @@ bool kq_codes_moe_supported(int P, int E, int N, int K, int codec);
 size_t kq_codes_moe_workspace_bytes(int P, int E);
 int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
                         const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
-                        int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, hipStream_t s);
+                        int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, KqOutMap om,
+                        hipStream_t s);
 // Helpers of the slot-mixing ops: idx [T][S-1] -> idx2 [T][S] (last slot = expert 0), and
 // out[t][n] = T(sum_s scores[t][s] * yf[t][s][n]).
 int kq_launch_pad_idx(const uint32_t* idx, uint32_t* idx2, int T, int S, hipStream_t s);
 int kq_launch_codes_gather(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs, const uint32_t* rhs,
                            const float* bias, const float* bias2, void* out, int B, int M, int N, int K, int x_div,
                            int64_t x_batch_stride, int64_t w_expert_stride, int glu, int act, float limit, float alpha,
-                           int codec, int dtype, hipStream_t s);
+                           int codec, int dtype, int E, KqOutMap om, hipStream_t s);
 bool kq_encode_dev_supported(int codec);
 int kq_launch_encode(const void* w, int dtype, const float* im, uint8_t* wire, int64_t rows, int64_t K, int codec,
                      hipStream_t s);
@@ -149,7 +152,8 @@ bool kq_anymma_moe_supported(int P, int E, int N, int K, int codec);
 size_t kq_anymma_moe_workspace_bytes(int P, int E);
 int kq_launch_anymma_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
                          const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
-                         int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, hipStream_t s);
+                         int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, KqOutMap om,
+                        hipStream_t s);
 // Router top-k (one workgroup per token): see kq_moe_router_topk in include/kq.h.
 int kq_launch_router_topk(const void* logits, int dtype, int T, int E, int top_k, int norm, int shared, const float* pes,
                           const float* bias, int scoring, float scale, uint32_t* indices, float* scores, hipStream_t s);

@@ -123,22 +123,28 @@ __global__ __launch_bounds__(GV_THREADS) void gemm_nt_generic_kernel(const void*
                                                                      const uint8_t* __restrict__ grids,
                                                                      const uint32_t* __restrict__ lhs,
                                                                      const uint32_t* __restrict__ rhs,
-                                                                     int64_t x_batch_stride, int64_t w_expert_stride) {
+                                                                     int64_t x_batch_stride, int64_t w_expert_stride,
+                                                                     int E) {
   constexpr int WPB = kq_geom(C).wpb, BPB = kq_geom(C).bpb, GPB = WPB / 8;
   const int gi = blockIdx.x * GV_THREADS + threadIdx.x;  // 8-column group
-  const int m = blockIdx.y, item = blockIdx.z;
+  const int item = blockIdx.z;
   if (gi >= N / 8) return;
+  const uint32_t e = rhs ? rhs[item] : 0u;
+  if (e >= (uint32_t)E) return;  // an expert id outside the stack: the entry's output is left untouched
   const size_t row_bytes = (size_t)(N / WPB) * BPB;
-  const uint8_t* wb = w + (rhs ? (size_t)rhs[item] * (size_t)w_expert_stride : 0) + (size_t)(gi / GPB) * BPB;
-  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const uint16_t* xr = static_cast<const uint16_t*>(x) + (lhs ? (size_t)lhs[item] * (size_t)x_batch_stride : 0) + (size_t)m * K;
-  for (int k = 0; k < K; k++) {
-    float wv[8];
-    kq::decode8<C>(wb + (size_t)k * row_bytes, gi % GPB, grids, wv);
-    float xv = DT == KQ_F16 ? kq::h2f(xr[k]) : kq::bf162f(xr[k]);
-    for (int t = 0; t < 8; t++) acc[t] = fmaf(xv, wv[t], acc[t]);
+  const uint8_t* wb = w + (size_t)e * (size_t)w_expert_stride + (size_t)(gi / GPB) * BPB;
+  for (int m = blockIdx.y; m < M; m += gridDim.y) {  // the grid's y extent is capped at 65535
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const uint16_t* xr =
+        static_cast<const uint16_t*>(x) + (lhs ? (size_t)lhs[item] * (size_t)x_batch_stride : 0) + (size_t)m * K;
+    for (int k = 0; k < K; k++) {
+      float wv[8];
+      kq::decode8<C>(wb + (size_t)k * row_bytes, gi % GPB, grids, wv);
+      float xv = DT == KQ_F16 ? kq::h2f(xr[k]) : kq::bf162f(xr[k]);
+      for (int t = 0; t < 8; t++) acc[t] = fmaf(xv, wv[t], acc[t]);
+    }
+    for (int t = 0; t < 8; t++) store_y<DT>(y, ((size_t)item * M + m) * N + 8 * (size_t)gi + t, acc[t]);
   }
-  for (int t = 0; t < 8; t++) store_y<DT>(y, ((size_t)item * M + m) * N + 8 * (size_t)gi + t, acc[t]);
 }
 
 // One wave per (item p, output row n).  Item p reads activation matrix x[lhs[p]] (or p / x_div
@@ -158,6 +164,7 @@ struct GatherArgs {
   int act;
   float limit, alpha;
   KqOutMap om;
+  int E;  // entries whose expert id is >= E are skipped (their output rows stay untouched)
 };
 
 template <int C, int DT, int MT, bool GLU>
@@ -172,6 +179,7 @@ __global__ __launch_bounds__(GV_THREADS) void gather_generic_kernel(GatherArgs a
   for (int64_t item = wave; item < (int64_t)a.B * a.N; item += nwaves) {
     const int p = (int)(item / a.N), n = (int)(item % a.N);
     const uint32_t e = a.rhs[p];
+    if (e >= (uint32_t)a.E) continue;  // wave-uniform
     const int64_t xi = a.lhs ? (int64_t)a.lhs[p] : (int64_t)(p / a.x_div);
     const size_t xoff = (size_t)(xi * a.x_batch_stride);
     const uint8_t* wr = a.w + (int64_t)e * a.w_expert_stride + (size_t)n * row_bytes;
@@ -283,14 +291,14 @@ struct GemvRun {
 template <int C>
 struct GemmNtRun {
   static int run(const void* x, const uint8_t* w, void* y, int M, int N, int K, int dt, const uint8_t* grids,
-                 const uint32_t* lhs, const uint32_t* rhs, int B, int64_t xs, int64_t ws, hipStream_t s) {
-    dim3 grid((N / 8 + GV_THREADS - 1) / GV_THREADS, M, B), block(GV_THREADS);
+                 const uint32_t* lhs, const uint32_t* rhs, int B, int64_t xs, int64_t ws, int E, hipStream_t s) {
+    dim3 grid((N / 8 + GV_THREADS - 1) / GV_THREADS, M < 65535 ? M : 65535, B), block(GV_THREADS);
     if (dt == KQ_F16)
       hipLaunchKernelGGL((gemm_nt_generic_kernel<C, KQ_F16>), grid, block, 0, s, x, w, y, M, N, K, grids, lhs, rhs, xs,
-                         ws);
+                         ws, E);
     else
       hipLaunchKernelGGL((gemm_nt_generic_kernel<C, KQ_BF16>), grid, block, 0, s, x, w, y, M, N, K, grids, lhs, rhs, xs,
-                         ws);
+                         ws, E);
     KQ_HIP_CHECK(hipGetLastError());
     return KQ_OK;
   }
@@ -346,26 +354,27 @@ int kq_launch_gemm_nt_generic(const void* x, const uint8_t* w, void* y, int M, i
   const uint8_t* grids = kq_device_grids();
   if (!grids) return KQ_ERR_HIP;
   return dispatch_codec<GemmNtRun>(codec, x, w, y, M, N, K, dtype, grids, (const uint32_t*)nullptr,
-                                   (const uint32_t*)nullptr, 1, (int64_t)0, (int64_t)0, s);
+                                   (const uint32_t*)nullptr, 1, (int64_t)0, (int64_t)0, 1, s);
 }
 
 int kq_launch_gather_nt_generic(const void* x, const uint8_t* w, const uint32_t* lhs, const uint32_t* rhs, void* out,
-                                int B, int M, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride, int codec,
-                                int dtype, hipStream_t s) {
+                                int B, int M, int E, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride,
+                                int codec, int dtype, hipStream_t s) {
   const uint8_t* grids = kq_device_grids();
   if (!grids) return KQ_ERR_HIP;
-  if (M > 65535 || B > 65535) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: M and the batch must be below 65536");
+  if (B > 65535) return kq_set_error(KQ_ERR_INVALID, "gather_qmm: the batch must be below 65536 entries");
   return dispatch_codec<GemmNtRun>(codec, x, w, out, M, N, K, dtype, grids, lhs, rhs, B, x_batch_stride,
-                                   w_expert_stride, s);
+                                   w_expert_stride, E, s);
 }
 
 int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
                              const uint32_t* rhs, const float* bias, const float* bias2, void* out, int B, int M,
                              int N, int K, int x_div, int64_t x_batch_stride, int64_t w_expert_stride, int glu,
-                             int act, float limit, float alpha, int codec, int dtype, hipStream_t s) {
+                             int act, float limit, float alpha, int codec, int dtype, int E, KqOutMap om,
+                             hipStream_t s) {
   const uint8_t* grids = kq_device_grids();
   if (!grids) return KQ_ERR_HIP;
   GatherArgs a{x, w, w2, lhs, rhs, bias, bias2, out, B, M, N, K, x_div, x_batch_stride, w_expert_stride,
-               act, limit, alpha, kq_out_map()};
+               act, limit, alpha, om, E};
   return dispatch_codec<GatherRun>(codec, a, dtype, glu != 0, grids, s);
 }

@@ -424,6 +424,7 @@ struct SkArgs {
   float* partial;
   int ksplit, sb_per_split;
   KqOutMap om;  // gathered calls: output row of an item, 16-bit or f32 (dense calls: identity)
+  int E;        // gathered calls: items whose expert id is >= E are skipped (output rows left untouched)
 };
 
 // MB = M rounded up to a power of two (1, 2, 4, 8).  Rows of the 32-row A operand beyond MB alias
@@ -478,6 +479,7 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_kernel(SkArgs a) {
   const int nrows = (N - row0 < half) ? (N - row0) : half;
   const int item = blockIdx.y;
   const size_t expert = a.rhs ? a.rhs[item] : 0;
+  if (a.rhs && expert >= (size_t)a.E) return;  // uniform over the workgroup, ahead of every barrier
   const size_t xsel = a.lhs ? a.lhs[item] : (size_t)(item / a.x_div);
   const uint8_t* wtile = a.w + expert * (size_t)a.w_expert_stride + (size_t)row0 * row_bytes;
   const uint8_t* wtile2 = GLU ? a.w2 + expert * (size_t)a.w_expert_stride + (size_t)row0 * row_bytes : wtile;
@@ -1417,7 +1419,7 @@ int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, 
 int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
                            const uint32_t* rhs, void* out, int B, int M, int N, int K, int x_div,
                            int64_t x_batch_stride, int64_t w_expert_stride, int glu, int act, float limit, int codec,
-                           int dtype, hipStream_t s) {
+                           int dtype, int E, KqOutMap om, hipStream_t s) {
   if (!sk_shape_ok(M, K, codec, x, w, w2) || B < 1 || B > 65535) return KQ_ERR_UNSUPPORTED;
   if (glu && (M != 1 || act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
   const int64_t wmask = (int64_t)sk_wire_align_mask(codec);
@@ -1437,7 +1439,8 @@ int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, c
   a.x_batch_stride = x_batch_stride;
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
-  a.om = kq_out_map();
+  a.om = om;
+  a.E = E;
   return glu ? launch_skinny_any<true>(a, B, codec, dtype, nullptr, s)
              : launch_skinny_any<false>(a, B, codec, dtype, nullptr, s);
 }

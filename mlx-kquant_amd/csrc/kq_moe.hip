@@ -617,7 +617,7 @@ size_t kq_moe_grouped_workspace_bytes(int rows, int P, int E, int K) { return ca
 // x: [rows][K] activations; pair p reads row p / x_div and expert idx[p]; out [P][N].
 int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, void* out, int rows,
                           int P, int E, int N, int K, int x_div, int64_t w_expert_stride, int glu, int act,
-                          float limit, int codec, int dtype, void* ws, hipStream_t s) {
+                          float limit, int codec, int dtype, void* ws, KqOutMap om, hipStream_t s) {
   if (!kq_moe_grouped_supported(P, E, N, K, codec) || (glu && act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
   const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;  // q6_k pieces are fetched with unaligned loads
   if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
@@ -648,6 +648,6 @@ int kq_launch_moe_grouped(const void* x, const uint8_t* w, const uint8_t* w2, co
   a.act = act;
   a.w_expert_stride = w_expert_stride;
   a.limit = limit;
-  a.om = kq_out_map();
+  a.om = om;
   return glu ? launch_grouped_any<true>(a, P, E, codec, dtype, s) : launch_grouped_any<false>(a, P, E, codec, dtype, s);
 }

@@ -127,6 +127,28 @@ def _stream_ptr(op: str, t: torch.Tensor, stream) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+def _on_stream(fn):
+    """`stream=` handling shared by every op: a torch.cuda.Stream other than the current one first waits for the
+    current stream (the producers of the inputs), then the whole op -- its temporaries, its workspace, its output
+    and its launches -- runs with that stream current, so the caching allocator ties every buffer to the stream
+    the kernels run on.  Inputs are marked as used on that stream.  As with any torch side stream, whoever reads
+    the result on another stream waits for this one first (`other.wait_stream(stream)`)."""
+    import functools
+
+    @functools.wraps(fn)
+    def wrapper(*args, stream=None, **kw):
+        if isinstance(stream, torch.cuda.Stream) and stream != torch.cuda.current_stream(stream.device):
+            stream.wait_stream(torch.cuda.current_stream(stream.device))
+            for a in list(args) + list(kw.values()):
+                if isinstance(a, torch.Tensor) and a.is_cuda:
+                    a.record_stream(stream)
+            with torch.cuda.stream(stream):
+                return fn(*args, stream=None, **kw)
+        return fn(*args, stream=stream, **kw)
+
+    return wrapper
+
+
 def _same_device(op, ref, *ts):
     for t in ts:
         if t is not None and t.device != ref.device:
@@ -878,3 +900,12 @@ def quantize(w, kquant_type, imatrix=None, *, stream=None):
     wire = torch.empty(list(w.shape[:-1]) + [K // wpb * bpb], dtype=torch.uint8)
     _check(lib.kq_quantize(w_h.data_ptr(), im.data_ptr() if im is not None else None, wire.data_ptr(), rows, K, cid))
     return wire.to(w.device), torch.zeros(1, dtype=torch.uint8, device=w.device)
+
+
+# every op that takes `stream=` gets the shared stream handling
+for _name in ("dequantize", "quantized_matmul", "quantized_matmul_qmv_bias", "gather_qmm", "expert_tile_map",
+              "gather_qmm_seg", "moe_glu_gather_kq", "gather_qmv_kq", "moe_glu_gather_shexp_kq", "gather_qmv_mix_kq",
+              "gather_qmv_mix_ns_kq", "mxfp4_packed_to_wire", "mxfp4_wire_to_packed", "moe_glu_gather",
+              "gather_qmv_bias", "gather_qmv_mix_bias", "moe_router_topk", "quantize"):
+    globals()[_name] = _on_stream(globals()[_name])
+del _name

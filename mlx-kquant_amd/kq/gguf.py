@@ -23,7 +23,7 @@ MAGIC = b"GGUF"
 # ggml tensor type id -> codec name (quantized) / numpy dtype (plain)
 GGML_QUANT = {2: "q4_0", 3: "q4_1", 6: "q5_0", 7: "q5_1", 8: "q8_0", 10: "q2_k", 11: "q3_k", 12: "q4_k", 13: "q5_k",
               14: "q6_k", 16: "iq2_xxs", 17: "iq2_xs", 18: "iq3_xxs", 19: "iq1_s", 20: "iq4_nl", 21: "iq3_s",
-              22: "iq2_s", 23: "iq4_xs", 29: "iq1_m", 39: "mxfp4"}
+              22: "iq2_s", 23: "iq4_xs", 29: "iq1_m", 39: "mxfp4", 40: "nvfp4"}
 GGML_PLAIN = {0: np.float32, 1: np.float16, 24: np.int8, 25: np.int16, 26: np.int32, 27: np.int64, 28: np.float64,
               30: "bfloat16"}
 _CODEC_TO_GGML = {v: k for k, v in GGML_QUANT.items()}

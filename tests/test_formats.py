@@ -93,10 +93,13 @@ def test_gguf_round_trip(tmp_path):
         "blk.0.attn_q.weight": _wire("q4_k", 32, 512, 4),
         "blk.0.ffn_gate_exps.weight": _wire("iq4_xs", 2 * 16, 256, 5).reshape(2, 16, -1),
         "token_embd.weight": _wire("q8_0", 10, 64, 6),
+        "blk.0.ffn_up_exps.weight": _wire("mxfp4", 2 * 8, 64, 7).reshape(2, 8, -1),     # ggml type 39
+        "blk.0.ffn_down_exps.weight": _wire("nvfp4", 2 * 8, 128, 8).reshape(2, 8, -1),  # ggml type 40
         "blk.0.attn_norm.weight": torch.randn(512),
         "blk.0.bias_bf16": torch.randn(4, 6).to(torch.bfloat16),
     }
-    codecs = {"blk.0.attn_q.weight": "q4_k", "blk.0.ffn_gate_exps.weight": "iq4_xs", "token_embd.weight": "q8_0"}
+    codecs = {"blk.0.attn_q.weight": "q4_k", "blk.0.ffn_gate_exps.weight": "iq4_xs", "token_embd.weight": "q8_0",
+              "blk.0.ffn_up_exps.weight": "mxfp4", "blk.0.ffn_down_exps.weight": "nvfp4"}
     meta = {"general.architecture": "llama", "llama.block_count": 1, "llama.rope.freq_base": 10000.0,
             "tokenizer.ggml.tokens": ["a", "b", "c"], "llama.flag": True, "some.ints": [1, -2, 3]}
     path = str(tmp_path / "toy.gguf")
@@ -108,6 +111,8 @@ def test_gguf_round_trip(tmp_path):
     assert g.tensor_shapes["blk.0.attn_q.weight"] == (512, 32)            # logical dims, innermost first
     assert g.tensor_shapes["blk.0.ffn_gate_exps.weight"] == (256, 16, 2)
     assert g.tensor_shapes["blk.0.bias_bf16"] == (6, 4)
+    assert g.tensor_shapes["blk.0.ffn_up_exps.weight"] == (64, 8, 2)
+    assert g.tensor_shapes["blk.0.ffn_down_exps.weight"] == (128, 8, 2)
     assert tuple(g.arrays["blk.0.attn_q.scales"].shape) == (1,)
     assert g.metadata["general.architecture"] == "llama" and g.metadata["llama.block_count"] == 1
     assert g.metadata["tokenizer.ggml.tokens"] == ["a", "b", "c"] and g.metadata["llama.flag"] is True
@@ -135,3 +140,24 @@ def test_gguf_hand_packed_bytes(tmp_path):
     open(path, "wb").write(head + b"\0" * pad + blocks[:20])
     with pytest.raises(ValueError):
         gguf.load_gguf(path)
+
+
+def test_gguf_hand_packed_fp4_types(tmp_path):
+    """ggml tensor types 39 (mxfp4: 32 weights in 17 bytes) and 40 (nvfp4: 64 weights in 36 bytes), the ids the
+    reference's reader maps (src/kquant_gguf.cpp:246-252), in a file assembled byte by byte."""
+    def s(x):
+        b = x.encode()
+        return struct.pack("<Q", len(b)) + b
+    assert O.geometry("mxfp4") == (32, 17) and O.geometry("nvfp4") == (64, 36)
+    mx = bytes(range(34))           # [K=32, N=2]: 2 rows x one 17-byte block
+    nv = bytes(range(100, 172))     # [K=64, N=2]: 2 rows x one 36-byte block
+    head = b"GGUF" + struct.pack("<IQQ", 3, 2, 0)
+    head += s("a.weight") + struct.pack("<IQQ", 2, 32, 2) + struct.pack("<IQ", 39, 0)
+    head += s("b.weight") + struct.pack("<IQQ", 2, 64, 2) + struct.pack("<IQ", 40, 64)
+    pad = (-len(head)) % 32
+    path = str(tmp_path / "fp4.gguf")
+    open(path, "wb").write(head + b"\0" * pad + mx + b"\0" * 30 + nv)
+    g = gguf.load_gguf(path)
+    assert g.codecs == [("a.weight", "mxfp4"), ("b.weight", "nvfp4")]
+    assert tuple(g.arrays["a.weight"].shape) == (2, 17) and bytes(g.arrays["a.weight"].numpy().tobytes()) == mx
+    assert tuple(g.arrays["b.weight"].shape) == (2, 36) and bytes(g.arrays["b.weight"].numpy().tobytes()) == nv
