@@ -36,9 +36,9 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLC_BYTES = 256 << 20
 # HBM bytes one headline launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
-# `bench.py --probe`: (16235.0 KiB x 1.9983 + 28.0 KiB x 1.0), each counter scaled by what it reads for
+# `bench.py --probe`: (16248.2 KiB x 1.9985 + 28.0 KiB x 1.0), each counter scaled by what it reads for
 # the probe's plain 32256 KiB device copy.  Algorithmic bytes are 33,030,144 (weights) + 28,672 (output).
-HEADLINE_TRAFFIC_BYTES = 33_254_000
+HEADLINE_TRAFFIC_BYTES = 33_280_000
 KQ_BF16 = 2
 
 
@@ -65,18 +65,30 @@ def synth_wire_torch(codec, rows, K, seed, device):
 
 
 def quantized_weights(kq, torch, codec, N, K, seed, device, unique_rows=None):
-    """Seeded N(0, 0.02) f32 weights [N, K] encoded by kq.quantize (host encoder; a uniform importance
-    matrix for the IQ codecs), placed on the GPU.  With unique_rows only that many rows are drawn and
-    encoded and the slab is repeated down the matrix (the codebook encoders search for ~1 us per weight;
-    kernel time does not depend on the values)."""
-    g = torch.Generator()
-    g.manual_seed(seed)
+    """Seeded N(0, 0.02) f32 weights [N, K] encoded by kq.quantize and placed on the GPU.  Codecs with a device
+    encoder (legacy and K-quants) are drawn and encoded on the GPU, in slabs of at most 64 Mi weights; the IQ
+    codecs go through the host encoder with a uniform importance matrix.  With unique_rows only that many rows
+    are drawn and encoded and the slab is repeated down the matrix (the codebook encoders search for ~1 us per
+    weight; kernel time does not depend on the values)."""
     rows = min(N, unique_rows) if unique_rows else N
-    w = torch.randn((rows, K), generator=g, dtype=torch.float32) * 0.02
-    wq, _ = kq.quantize(w, codec, torch.ones(K) if codec.startswith("iq") else None)
+    if kq._load().kq_quantize_dev_supported(kq._load().kq_codec_id(codec.encode())):
+        g = torch.Generator(device=device)
+        g.manual_seed(seed)
+        step = max(1, (64 << 20) // K)
+        parts = []
+        for r0 in range(0, rows, step):
+            w = torch.randn((min(step, rows - r0), K), generator=g, dtype=torch.float32, device=device) * 0.02
+            parts.append(kq.quantize(w, codec)[0])
+            del w
+        wq = parts[0] if len(parts) == 1 else torch.cat(parts)
+    else:
+        g = torch.Generator()
+        g.manual_seed(seed)
+        w = torch.randn((rows, K), generator=g, dtype=torch.float32) * 0.02
+        wq = kq.quantize(w, codec, torch.ones(K) if codec.startswith("iq") else None)[0].to(device)
     if rows < N:
         wq = wq.repeat((N + rows - 1) // rows, 1)[:N].contiguous()
-    return wq.to(device)
+    return wq
 
 
 def _time_direct(torch, calls, launches, warm):
@@ -278,6 +290,9 @@ def main():
     ap.add_argument("--probe-prefill", default=None, metavar="CODEC",
                     help="counter probe for `rocprofv3 --pmc`: 5 launches of the prefill GEMM [2048, 8192] x "
                          "[28672, 8192]^T in CODEC (random structurally valid wire), nothing else")
+    ap.add_argument("--probe-moe", type=int, default=None, metavar="TOKENS",
+                    help="counter probe for `rocprofv3 --pmc`: 10 launches each of the q4_k GLU op and the q6_k down "
+                         "op of the 128-expert top-8 MoE at TOKENS tokens, nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU.",
@@ -305,6 +320,25 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"probe": "20 GEMV launches", "codec": c, "N": n, "K": k, "M": 1,
                           "weight_bytes": n * kq.bytes_per_row(c, k)}))
+        return
+
+    if args.probe_moe:
+        E, H, I, TOPK, T = 128, 2048, 768, 8, args.probe_moe
+        gate = synth_wire_torch("q4_k", E * I, H, 11, dev).reshape(E, I, -1)
+        up = synth_wire_torch("q4_k", E * I, H, 12, dev).reshape(E, I, -1)
+        down = synth_wire_torch("q6_k", E * H, I, 13, dev).reshape(E, H, -1)
+        xt = randx((T, H), 0.5)
+        touched = []
+        for r in range(10):
+            idx = torch.randn((T, E), device=dev, generator=gx).topk(TOPK, dim=-1).indices.to(torch.int32).contiguous()
+            call, h = abi.moe_glu(xt, gate, up, "q4_k", idx)
+            call()
+            abi.gather_qmv(h, down, "q6_k", idx)()
+            touched.append(int(idx.unique().numel()))
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "10 GLU + 10 down launches", "tokens": T, "experts_touched_mean": sum(touched) / 10,
+                          "glu_bytes_per_expert": 2 * I * kq.bytes_per_row("q4_k", H),
+                          "down_bytes_per_expert": H * kq.bytes_per_row("q6_k", I)}))
         return
 
     if args.probe_prefill:
@@ -378,14 +412,11 @@ def main():
         # ---------------- decode sweep (q4_k_m recipe of Llama-3-8B)
         if want("sweep"):
             sweep = []
-            shapes = [("q_proj", "q4_k", 4096, 4096, True), ("gate/up", "q4_k", 14336, 4096, True),
-                      ("down", "q6_k", 4096, 14336, True), ("lm_head", "q6_k", 128256, 4096, False)]
-            for name, c, n, k, encode in shapes:
+            shapes = [("q_proj", "q4_k", 4096, 4096), ("gate/up", "q4_k", 14336, 4096),
+                      ("down", "q6_k", 4096, 14336), ("lm_head", "q6_k", 128256, 4096)]
+            for name, c, n, k in shapes:
                 wb = n * kq.bytes_per_row(c, k)
-                # the 525M-weight lm_head is filled with structurally valid random wire (encoding it on
-                # the host would dominate the run); the others are encoded from N(0, 0.02)
-                wq = base if name == "gate/up" else (quantized_weights(kq, torch, c, n, k, 3, dev) if encode
-                                                     else synth_wire_torch(c, n, k, 3, dev))
+                wq = base if name == "gate/up" else quantized_weights(kq, torch, c, n, k, 3, dev)
                 cps = cold_copies(torch, wq, wb)
                 for m in (1, 2, 4, 8):
                     xm = randx((m, k))
@@ -415,12 +446,12 @@ def main():
             abi.lib.kq_set_gemm_tile_rows(0)
             out["prefill"] = prefill
 
-        # ---------------- MoE: 128 experts, top-8, hidden 2048, intermediate 768 (structurally valid random wire)
+        # ---------------- MoE: 128 experts, top-8, hidden 2048, intermediate 768 (weights encoded by kq.quantize)
         if want("moe"):
             E, H, I, TOPK = 128, 2048, 768, 8
-            gate = synth_wire_torch("q4_k", E * I, H, 11, dev).reshape(E, I, -1)
-            up = synth_wire_torch("q4_k", E * I, H, 12, dev).reshape(E, I, -1)
-            down = synth_wire_torch("q6_k", E * H, I, 13, dev).reshape(E, H, -1)
+            gate = quantized_weights(kq, torch, "q4_k", E * I, H, 11, dev).reshape(E, I, -1)
+            up = quantized_weights(kq, torch, "q4_k", E * I, H, 12, dev).reshape(E, I, -1)
+            down = quantized_weights(kq, torch, "q6_k", E * H, I, 13, dev).reshape(E, H, -1)
             gu_bytes = 2 * I * kq.bytes_per_row("q4_k", H)
             dn_bytes = H * kq.bytes_per_row("q6_k", I)
             moe = []

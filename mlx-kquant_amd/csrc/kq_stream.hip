@@ -131,6 +131,7 @@ struct StArgs {
   const uint8_t* w;
   void* y;
   int M, N, K, tiles;
+  int rpt;  // weight rows per tile (<= 32): fewer than 32 evens the rows out over one round of workgroups
   float* partial;  // split-K: [ksplit][M][N] f32
   int ksplit, sb_per_split;
 #ifdef KQ_ST_TS
@@ -319,7 +320,7 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, kg = lane >> 5;
-  const int M = a.M, N = a.N, K = a.K, nsb = K >> 8, tiles = a.tiles;
+  const int M = a.M, N = a.N, K = a.K, nsb = K >> 8, tiles = a.tiles, rpt = a.rpt;
   const uint32_t row_bytes = (uint32_t)nsb * G::BPB;
   const int G_x = gridDim.x;
 
@@ -354,15 +355,16 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
   __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled ahead of these loads
 
   // ---- weight stream.  Piece i = lane + 64 t of a unit -> (row i / PP, piece i % PP); rows past the end of the
-  // matrix re-read the last row (their results are dropped).
+  // tile or of the matrix re-read the last row inside both (their results are dropped).
   uint32_t goff[U::FULL + 1];
   const int row_lim = N - 1;
   auto piece_off = [&](int i, int row0) {
     int r = i / G::PP;
     const int p = i - r * G::PP;
+    r = r < rpt ? r : rpt - 1;
     r = row0 + r;
     r = r < row_lim ? r : row_lim;
-    return (uint32_t)(r - row0) * row_bytes + 16u * p;  // may be negative-free: r >= row0 whenever row0 <= row_lim
+    return (uint32_t)(r - row0) * row_bytes + 16u * p;  // r >= row0: a tile always starts inside the matrix
   };
   // (offsets are relative to the tile's first row; a tile always starts inside the matrix)
   // Elements of the stream: (tile, unit) in tile-major order.  `it`, `iu`, `islot`: next element to issue.
@@ -370,8 +372,8 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
   int goff_row0 = -1;
   auto issue_next = [&]() {
     if (it >= tiles) return;
-    const int row0 = it * ST_ROWS;
-    if (row0 + ST_ROWS > N && goff_row0 != row0) {  // ragged last tile: rebuild the piece map with clamped rows
+    const int row0 = it * rpt;
+    if (row0 + rpt > N && goff_row0 != row0) {  // ragged last tile: rebuild the piece map with clamped rows
       SFor<U::FULL + 1>::run([&](auto t) { constexpr int T = decltype(t)::value; goff[T] = piece_off(lane + 64 * T, row0); });
       goff_row0 = row0;
     }
@@ -382,7 +384,7 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
       if (lane < 32) dma16(base, goff[U::FULL], l0 + U::FULL * 1024);
     }
     if constexpr (G::SIDE_D) {
-      int r = row0 + lane;
+      int r = row0 + (lane < rpt ? lane : rpt - 1);
       r = r < row_lim ? r : row_lim;
       if (lane < 32) dma2(base + 208, (uint32_t)(r - row0) * row_bytes, l0 + ST_ROWS * G::LBPB);
     }
@@ -396,7 +398,7 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
   SFor<U::FULL + 1>::run([&](auto t) {
     constexpr int T = decltype(t)::value;
     const int i = lane + 64 * T, r = i / G::PP;
-    goff[T] = (uint32_t)r * row_bytes + 16u * (i - r * G::PP);
+    goff[T] = (uint32_t)(r < rpt ? r : rpt - 1) * row_bytes + 16u * (i - r * G::PP);
   });
   if (nu == 0) it = tiles;  // a wave without superblocks (short K range) only joins the barriers
 
@@ -491,8 +493,8 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
   for (; ct < tiles; ct += G_x) {
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
-    const int row0 = ct * ST_ROWS;
-    const int nrows = N - row0 < ST_ROWS ? N - row0 : ST_ROWS;
+    const int row0 = ct * rpt;
+    const int nrows = N - row0 < rpt ? N - row0 : rpt;
     const int crow = n < nrows ? n : nrows - 1;
     SFor<ST_XU>::run([&](auto uu) {
       constexpr int u = decltype(uu)::value;
@@ -611,6 +613,17 @@ int st_launch_one(StArgs a, int splits, hipStream_t s) {
   const int per_cu = lds <= 80 * 1024 ? 2 : 1;
   int gx = per_cu * st_num_cus() / splits;
   if (gx < 1) gx = 1;
+  // rows per tile: when the 32-row tiles do not fill a whole number of rounds of the resident workgroups, the
+  // busiest CU decides the time (448 tiles on 512 slots: two tiles on 192 CUs, one on 64).  Spreading the rows
+  // over rounds x slots equal tiles of 24 ... 32 rows levels that; the rows a short tile leaves out cost idle lanes,
+  // not bandwidth.
+  {
+    const int tiles32 = (a.N + ST_ROWS - 1) / ST_ROWS;
+    const int rounds = (tiles32 + gx - 1) / gx;
+    const int rpt = (a.N + rounds * gx - 1) / (rounds * gx);
+    a.rpt = rpt >= 24 && rpt < ST_ROWS ? rpt : ST_ROWS;
+    a.tiles = (a.N + a.rpt - 1) / a.rpt;
+  }
   if (gx > a.tiles) gx = a.tiles;
   hipLaunchKernelGGL(kern, dim3(gx, 1, splits), dim3(ST_THREADS), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
