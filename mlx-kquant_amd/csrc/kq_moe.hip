@@ -301,7 +301,12 @@ __global__ __launch_bounds__(MOE_THREADS, 2) void moe_grouped_kernel(MoeArgs a) 
   int* pair_lds = reinterpret_cast<int*>(smem + MOE_STAGES * STAGE);  // [32] output row of each segment slot, -1 = none
   float* rs_lds = reinterpret_cast<float*>(pair_lds + SEG_M);         // [32]
 
-  const int seg_id = blockIdx.y;
+  // Workgroups go to the 8 XCDs round-robin in launch order.  Launch position L = 8 j + c runs slab j % tiles of
+  // segment 8 (j / tiles) + c: all slabs of a segment sit on one XCD, back to back, so the segment's activation
+  // rows are fetched into one L2 once instead of into all eight (grid y is a multiple of 8).
+  const int lin = blockIdx.x + gridDim.x * blockIdx.y;
+  const int slab_id = (lin >> 3) % (int)gridDim.x;
+  const int seg_id = ((lin >> 3) / (int)gridDim.x) * 8 + (lin & 7);
   if (seg_id >= *a.nseg) return;  // uniform: the grid is sized for the worst case
   const Segment seg = a.segs[seg_id];
 
@@ -309,7 +314,7 @@ __global__ __launch_bounds__(MOE_THREADS, 2) void moe_grouped_kernel(MoeArgs a) 
   const int l32 = lane & 31, kg = lane >> 5;
   const int N = a.N, K = a.K, nsb = K >> 8;
   const size_t row_bytes = (size_t)nsb * G::BPB;
-  const int n0 = blockIdx.x * NCOLS;
+  const int n0 = slab_id * NCOLS;
   const int ncols = N - n0 < NCOLS ? N - n0 : NCOLS;
   const uint8_t* wtile = a.w + (size_t)seg.expert * (size_t)a.w_expert_stride + (size_t)n0 * row_bytes;
   const uint8_t* wtile2 = GLU ? a.w2 + (size_t)seg.expert * (size_t)a.w_expert_stride + (size_t)n0 * row_bytes : wtile;
@@ -516,6 +521,7 @@ int launch_grouped(const MoeArgs& a, int P, int E, hipStream_t s) {
   const int ntiles = (a.N + NCOLS - 1) / NCOLS;
   int maxseg = E + P / SEG_M;  // sum over experts of ceil(c_e / 32) <= E + P / 32
   if (maxseg > P) maxseg = P;
+  maxseg = (maxseg + 7) & ~7;  // the kernel's launch-position map needs a multiple of 8
   const size_t lds = (size_t)MOE_STAGES * (SEG_M * A_STRIDE + SLAB * G::LBPB + SEG_M * 32 + SLAB * 2) + SEG_M * 8;
   auto kern = moe_grouped_kernel<C, DT, GLU>;
   hipLaunchKernelGGL(kern, dim3(ntiles, maxseg), dim3(MOE_THREADS), lds, s, a);

@@ -144,10 +144,12 @@ struct StArgs {
 // Pieces qs[64 kg + 16 pc ..), pc = 0..3: pair pc / 2 of the half, weights 16 (pc % 2) .. + 15 of the low-nibble
 // sub-block 2 (pc / 2) and of the high-nibble sub-block 2 (pc / 2) + 1.  MFMA (pc, e, h): word e of the piece,
 // nibble h; activations = A pair pc, block 2 e + h.
-template <int C, int R>
+// R activation rows in RG = ceil(R / 4) groups of four; group g keeps its A registers at areg[g * AS + ...].
+template <int C, int R, int AS>
 __device__ __forceinline__ void q45k_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
                                           const float* __restrict__ xsum, int xsum_row_stride, float* acc) {
   constexpr int QS = C == KQ_Q4_K ? 16 : 48;
+  constexpr int RG = (R + 3) / 4;
   const u32x4 hdr = *reinterpret_cast<const u32x4*>(bl);
   u32x4 q[4];
 #pragma unroll
@@ -197,10 +199,14 @@ __device__ __forceinline__ void q45k_unit(const uint8_t* __restrict__ bl, int kg
   const uint32_t bit_lo = opaque_sgpr(0x00100010u), bit_hi = opaque_sgpr(0x01000100u);
   SFor<2>::run([&](auto gg) {
     constexpr int gl = decltype(gg)::value;
-    f32x4 p[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+    f32x4 p[RG][2];
+#pragma unroll
+    for (int g = 0; g < RG; g++) p[g][0] = p[g][1] = f32x4{0, 0, 0, 0};
     SFor<2>::run([&](auto pp) {
       constexpr int pc = 2 * gl + decltype(pp)::value;
-      const f16x4 av = __builtin_bit_cast(f16x4, areg[pc]);
+      f16x4 av[RG];
+#pragma unroll
+      for (int g = 0; g < RG; g++) av[g] = __builtin_bit_cast(f16x4, areg[g * AS + pc]);
       SFor<4>::run([&](auto ee) {
         constexpr int e = decltype(ee)::value;
         const uint32_t w0 = q[pc][e], w8 = w0 >> 8;
@@ -217,7 +223,9 @@ __device__ __forceinline__ void q45k_unit(const uint8_t* __restrict__ bl, int kg
             bv.x = and_or(hq << (tgt - jl), h ? bit_hi : bit_lo, opaque_vgpr(bv.x));
             bv.y = and_or(hq >> (8 + jl - tgt), h ? bit_hi : bit_lo, opaque_vgpr(bv.y));
           }
-          p[h] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, bv), p[h], 3, 2 * e + h, 0);
+#pragma unroll
+          for (int g = 0; g < RG; g++)
+            p[g][h] = __builtin_amdgcn_mfma_f32_4x4x4f16(av[g], __builtin_bit_cast(f16x4, bv), p[g][h], 3, 2 * e + h, 0);
         });
       });
     });
@@ -226,7 +234,7 @@ __device__ __forceinline__ void q45k_unit(const uint8_t* __restrict__ bl, int kg
       constexpr int jl = 2 * gl + h;
       SFor<R>::run([&](auto rr) {
         constexpr int r = decltype(rr)::value;
-        acc[r] = fmaf(mul[jl], p[h][r], acc[r]);
+        acc[r] = fmaf(mul[jl], p[r / 4][h][r % 4], acc[r]);
         acc[r] = fmaf(-sub[jl], xs[r][jl], acc[r]);
       });
     });
@@ -241,9 +249,10 @@ __device__ __forceinline__ void q45k_unit(const uint8_t* __restrict__ bl, int kg
 // 16, 1024 + 4^t qh.  Per scale group of 16 weights two accumulators P, H and
 //   sum x w = d sc (P / s + 16 H / 4^t - (1024 / s + 16 * 1024 / 4^t + 32) X).
 // MFMA (t, e): weights l = 4 e .. 4 e + 3; activations = A pair 2 t + e / 4, block 2 (e % 4) [+ 1 unused].
-template <int R>
+template <int R, int AS>
 __device__ __forceinline__ void q6k_unit(const uint8_t* __restrict__ bl, float dx, int hf, const u32x2* areg,
                                          const float* __restrict__ xsum, int xsum_row_stride, float* acc) {
+  constexpr int RG = (R + 3) / 4;
   u32x4 ql[4], qh[2];
 #pragma unroll
   for (int i = 0; i < 4; i++) ql[i] = *reinterpret_cast<const u32x4*>(bl + 64 * hf + 16 * i);
@@ -271,18 +280,23 @@ __device__ __forceinline__ void q6k_unit(const uint8_t* __restrict__ bl, float d
     constexpr int t = decltype(tt)::value;
     SFor<2>::run([&](auto ss) {
       constexpr int s = decltype(ss)::value;  // scale group 2 t + s: weights l = 16 s .. 16 s + 15
-      f32x4 pq = {0, 0, 0, 0}, ph = {0, 0, 0, 0};
+      f32x4 pq[RG], ph[RG];
+#pragma unroll
+      for (int g = 0; g < RG; g++) pq[g] = ph[g] = f32x4{0, 0, 0, 0};
       SFor<4>::run([&](auto ee) {
         constexpr int e = 4 * s + decltype(ee)::value;  // l = 4 e .. 4 e + 3
         constexpr int wq = 8 * (t & 1) + e;             // ql word: bytes 32 (t & 1) + 4 e ..
-        const f16x4 av = __builtin_bit_cast(f16x4, areg[2 * t + e / 4]);
         u32x2 bq, bh;
         bq.x = and_or(ql[wq >> 2][wq & 3], t >= 2 ? mask_hi : mask_lo, magic);
         bq.y = and_or(ql8[wq], t >= 2 ? mask_hi : mask_lo, magic);
         bh.x = and_or(qh[e >> 2][e & 3], mask_h[t], magic);
         bh.y = and_or(qh8[e], mask_h[t], magic);
-        pq = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, bq), pq, 3, 2 * (e & 3), 0);
-        ph = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, bh), ph, 3, 2 * (e & 3), 0);
+#pragma unroll
+        for (int g = 0; g < RG; g++) {
+          const f16x4 av = __builtin_bit_cast(f16x4, areg[g * AS + 2 * t + e / 4]);
+          pq[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, bq), pq[g], 3, 2 * (e & 3), 0);
+          ph[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, bh), ph[g], 3, 2 * (e & 3), 0);
+        }
       });
       constexpr int g = 2 * t + s;
       const int sc = __builtin_amdgcn_sbfe((int)(g < 4 ? scw.x : scw.y), 8 * (g & 3), 8);
@@ -292,7 +306,7 @@ __device__ __forceinline__ void q6k_unit(const uint8_t* __restrict__ bl, float d
       constexpr float fx = 1024.0f * fq + 1024.0f * fh + 32.0f;
       SFor<R>::run([&](auto rr) {
         constexpr int r = decltype(rr)::value;
-        const float v = fmaf(fq, pq[r], fmaf(fh, ph[r], -fx * xs[r][g]));
+        const float v = fmaf(fq, pq[r / 4][r % 4], fmaf(fh, ph[r / 4][r % 4], -fx * xs[r][g]));
         acc[r] = fmaf(dsc, v, acc[r]);
       });
     });
@@ -300,13 +314,20 @@ __device__ __forceinline__ void q6k_unit(const uint8_t* __restrict__ bl, float d
 }
 
 // ------------------------------------------------------------------ the kernel
-// MB = M rounded up to a power of two (1, 2, 4); D = units a wave keeps in LDS (in flight or being read).
-template <int C, int DT, int MB, int D>
-__global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
+// MB = M rounded up to a power of two (1, 2, 4, 8); D = units a wave keeps in LDS (in flight or being read);
+// WGS = workgroups per CU the register budget is set for.  Eight rows are two groups of four for the 4-row
+// MFMA; their f16 fragments pass through the wave's LDS staging area two rows at a time.
+template <int MB>
+constexpr int st_xch() { return MB > 4 ? 2 : MB; }  // activation rows staged at a time
+
+template <int C, int DT, int MB, int D, int WGS>
+__global__ __launch_bounds__(ST_THREADS, WGS) void stream_gemv_kernel(StArgs a) {
   using G = StGeom<C>;
   using U = StUnit<C>;
   constexpr int R = MB;
+  constexpr int RG = (MB + 3) / 4, XCH = st_xch<MB>(), NCH = MB / XCH;
   constexpr int NAP = G::NAP, XSG = G::XSG;
+  constexpr int AS = ST_XU * NAP;  // A register pairs per row group
   constexpr int XL = 2;  // 16-byte activation loads per lane and row: 4 units x 256 values
 
 #ifdef KQ_ST_TS
@@ -325,7 +346,7 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
   const int G_x = gridDim.x;
 
   // LDS: per wave [D slots][x fragments MB x 4 x 256 f16][x sums MB x 4 x 2 XSG f32]; then red [2][waves][R][64] f32
-  constexpr int XS_BYTES = MB * ST_XU * 512, XSUM_BYTES = MB * ST_XU * 2 * XSG * 4;
+  constexpr int XS_BYTES = XCH * ST_XU * 512, XSUM_BYTES = MB * ST_XU * 2 * XSG * 4;
   constexpr int WAVE_BYTES = D * U::SLOT + XS_BYTES + XSUM_BYTES;
   uint8_t* wb = smem + wave * WAVE_BYTES;
   _Float16* xs = reinterpret_cast<_Float16*>(wb + D * U::SLOT);
@@ -432,56 +453,65 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
       inv = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
     }
   }
-  SFor<MB * XL>::run([&](auto t) {
-    constexpr int T = decltype(t)::value;
-    constexpr int m = T / XL, s = T % XL;
-    const int gi = lane + 64 * s, uu = gi >> 5, grp = gi & 31;
-    const u32x4 v = xreg[T];
-    _Float16 h[8];
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      if constexpr (DT == KQ_BF16) {
-        h[2 * e] = (_Float16)(__builtin_bit_cast(float, v[e] << 16) * inv);
-        h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, v[e] & 0xffff0000u) * inv);
-      } else {
-        h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] & 0xffff));
-        h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
-      }
-    }
-    // MFMA fragment order inside a 4-group: k0 k2 k1 k3
-    const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
-    *reinterpret_cast<f16x8*>(xs + (m * ST_XU + uu) * 256 + 8 * grp) = v8;
-    float sum = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; e++) sum += (float)h[e];
-    sum += dpp_f<0xB1>(sum);  // lanes l ^ 1: 16 values
-    if constexpr (XSG == 8) {
-      if ((lane & 1) == 0) xsum[(m * ST_XU + uu) * 16 + (grp >> 1)] = sum;
-    } else {
-      sum += dpp_f<0x4E>(sum);  // lanes l ^ 2: 32 values
-      if ((lane & 3) == 0) xsum[(m * ST_XU + uu) * 8 + (grp >> 2)] = sum;
-    }
-  });
-  wave_lds_fence();
-  // A registers.  Lane (kg, fa, fi) keeps, for every unit and register pair, the four activations of row fi
-  // that MFMA block fa needs.
+  // A registers.  Lane (kg, fa, fi) keeps, for every row group, unit and register pair, the four activations of
+  // row 4 g + fi that MFMA block fa needs.
   //   q4_k / q5_k: pair pc, block 2 e + h  -> k = 128 kg + 32 (2 (pc / 2) + h) + 16 (pc % 2) + 4 e
   //   q6_k:        pair 2 t + e / 4, block 2 (e % 4) -> k = 128 hf + 32 t + 4 e  (odd blocks unused)
   const int fa = (lane >> 2) & 7, fi = lane & 3;
-  u32x2 areg[ST_XU * NAP];
-  {
-    const uint8_t* xb = reinterpret_cast<const uint8_t*>(xs) + (fi & (MB - 1)) * (ST_XU * 512) + 256 * kg;
-    SFor<ST_XU * NAP>::run([&](auto t) {
+  u32x2 areg[RG * AS];
+  SFor<NCH>::run([&](auto cc) {
+    constexpr int c = decltype(cc)::value;  // rows c XCH .. c XCH + XCH - 1 pass through the staging area
+    if constexpr (c > 0) wave_lds_fence();  // the previous rows have been read
+    SFor<XCH * XL>::run([&](auto t) {
       constexpr int T = decltype(t)::value;
-      constexpr int u = T / NAP, pr = T % NAP;
-      int koff;  // in f16 elements inside the half
-      if constexpr (C == KQ_Q6_K)
-        koff = 32 * (pr >> 1) + 16 * (pr & 1) + 4 * (fa >> 1);
-      else
-        koff = 64 * (pr >> 1) + 32 * (fa & 1) + 16 * (pr & 1) + 4 * (fa >> 1);
-      areg[T] = *reinterpret_cast<const u32x2*>(xb + u * 512 + koff * 2);
+      constexpr int ml = T / XL, m = c * XCH + ml, s = T % XL;
+      const int gi = lane + 64 * s, uu = gi >> 5, grp = gi & 31;
+      const u32x4 v = xreg[m * XL + s];
+      _Float16 h[8];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if constexpr (DT == KQ_BF16) {
+          h[2 * e] = (_Float16)(__builtin_bit_cast(float, v[e] << 16) * inv);
+          h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, v[e] & 0xffff0000u) * inv);
+        } else {
+          h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] & 0xffff));
+          h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
+        }
+      }
+      // MFMA fragment order inside a 4-group: k0 k2 k1 k3
+      const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+      *reinterpret_cast<f16x8*>(xs + (ml * ST_XU + uu) * 256 + 8 * grp) = v8;
+      float sum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) sum += (float)h[e];
+      sum += dpp_f<0xB1>(sum);  // lanes l ^ 1: 16 values
+      if constexpr (XSG == 8) {
+        if ((lane & 1) == 0) xsum[(m * ST_XU + uu) * 16 + (grp >> 1)] = sum;
+      } else {
+        sum += dpp_f<0x4E>(sum);  // lanes l ^ 2: 32 values
+        if ((lane & 3) == 0) xsum[(m * ST_XU + uu) * 8 + (grp >> 2)] = sum;
+      }
     });
-  }
+    wave_lds_fence();
+    constexpr int g = c * XCH / 4;  // the row group these rows belong to
+    // staged row of this lane: MB <= 4 keeps all rows staged (spare lanes alias row fi % MB); MB = 8 stages
+    // rows 2 c, 2 c + 1 = rows 2 (c % 2), 2 (c % 2) + 1 of group c / 2
+    const bool mine = MB <= 4 || (fi >> 1) == (c & 1);
+    const int lrow = MB <= 4 ? (fi & (MB - 1)) : (fi & 1);
+    if (mine) {
+      const uint8_t* xb = reinterpret_cast<const uint8_t*>(xs) + lrow * (ST_XU * 512) + 256 * kg;
+      SFor<AS>::run([&](auto t) {
+        constexpr int T = decltype(t)::value;
+        constexpr int u = T / NAP, pr = T % NAP;
+        int koff;  // in f16 elements inside the half
+        if constexpr (C == KQ_Q6_K)
+          koff = 32 * (pr >> 1) + 16 * (pr & 1) + 4 * (fa >> 1);
+        else
+          koff = 64 * (pr >> 1) + 32 * (fa & 1) + 16 * (pr & 1) + 4 * (fa >> 1);
+        areg[g * AS + T] = *reinterpret_cast<const u32x2*>(xb + u * 512 + koff * 2);
+      });
+    }
+  });
 
   // The other D - 1 units are queued only now: a wave that queues loads faster than the memory system takes them
   // stalls in the issue, and the activation work above would have waited behind that stall.
@@ -510,9 +540,9 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
         const uint8_t* bl = slot + crow * G::LBPB;
         if constexpr (C == KQ_Q6_K) {
           const float dx = kq::h2f((uint16_t)*reinterpret_cast<const uint32_t*>(slot + ST_ROWS * G::LBPB + 4 * crow)) * xscale;
-          q6k_unit<R>(bl, dx, kg, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
+          q6k_unit<R, AS>(bl, dx, kg, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
         } else {
-          q45k_unit<C, R>(bl, kg, xscale, areg + u * NAP, xsum + u * 8, ST_XU * 8, acc);
+          q45k_unit<C, R, AS>(bl, kg, xscale, areg + u * NAP, xsum + u * 8, ST_XU * 8, acc);
         }
         // the slot has been read: refill it with the next element of the stream
         lgkm_drain();
@@ -556,7 +586,7 @@ __global__ __launch_bounds__(ST_THREADS, 2) void stream_gemv_kernel(StArgs a) {
 
 template <int C, int MB, int D>
 constexpr size_t st_lds_bytes() {
-  return (size_t)ST_WAVES * (D * StUnit<C>::SLOT + MB * ST_XU * 512 + MB * ST_XU * 2 * StGeom<C>::XSG * 4) +
+  return (size_t)ST_WAVES * (D * StUnit<C>::SLOT + st_xch<MB>() * ST_XU * 512 + MB * ST_XU * 2 * StGeom<C>::XSG * 4) +
          2 * ST_WAVES * MB * 64 * 4;
 }
 
@@ -604,14 +634,14 @@ StSplit st_split_plan(int N, int K, int cus) {
 template <int C, int DT, int MB, int D>
 int st_launch_one(StArgs a, int splits, hipStream_t s) {
   constexpr size_t lds = st_lds_bytes<C, MB, D>();
-  auto kern = stream_gemv_kernel<C, DT, MB, D>;
+  constexpr int WGS = lds <= 80 * 1024 ? 2 : 1;
+  auto kern = stream_gemv_kernel<C, DT, MB, D, WGS>;
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
     KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
-  const int per_cu = lds <= 80 * 1024 ? 2 : 1;
-  int gx = per_cu * st_num_cus() / splits;
+  int gx = WGS * st_num_cus() / splits;
   if (gx < 1) gx = 1;
   // rows per tile: when the 32-row tiles do not fill a whole number of rounds of the resident workgroups, the
   // busiest CU decides the time (448 tiles on 512 slots: two tiles on 192 CUs, one on 64).  Spreading the rows
@@ -641,7 +671,8 @@ int st_launch_m(const StArgs& a, int splits, hipStream_t s) {
   constexpr int D1 = C == KQ_Q6_K ? 2 : 2;
   if (a.M == 1) return st_launch_one<C, DT, 1, D1>(a, splits, s);
   if (a.M == 2) return st_launch_one<C, DT, 2, 2>(a, splits, s);
-  return st_launch_one<C, DT, 4, 2>(a, splits, s);
+  if (a.M <= 4) return st_launch_one<C, DT, 4, 2>(a, splits, s);
+  return st_launch_one<C, DT, 8, 2>(a, splits, s);
 }
 
 bool st_codec_ok(int codec) { return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K; }
@@ -649,7 +680,7 @@ bool st_codec_ok(int codec) { return codec == KQ_Q4_K || codec == KQ_Q5_K || cod
 }  // namespace
 
 bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const void* w) {
-  if (!st_codec_ok(codec) || M < 1 || M > 4 || N < 1 || K < 256 || (K & 255)) return false;
+  if (!st_codec_ok(codec) || M < 1 || M > 8 || N < 1 || K < 256 || (K & 255)) return false;
   if ((int64_t)N * (K >> 8) * 210 >= (int64_t)1 << 40) return false;
   // q4_k / q5_k pieces are fetched 16-byte aligned, q6_k blocks are 2-byte multiples
   const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;
@@ -658,7 +689,7 @@ bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const vo
 }
 
 size_t kq_stream_workspace_bytes(int M, int N, int K, int codec) {
-  if (!st_codec_ok(codec) || M < 1 || M > 4 || (K & 255) || K < 256) return 0;
+  if (!st_codec_ok(codec) || M < 1 || M > 8 || (K & 255) || K < 256) return 0;
   const StSplit p = st_split_plan(N, K, st_num_cus());
   return p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
 }
