@@ -38,10 +38,7 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int ST_WAVES = 4;
-constexpr int ST_THREADS = ST_WAVES * 64;
 constexpr int ST_ROWS = 32;
-constexpr int ST_XU = 4;  // units per wave at most (K range of a workgroup <= 16 superblocks)
 
 template <int N>
 struct SFor {
@@ -116,6 +113,27 @@ struct StGeom<KQ_Q6_K> {
   static constexpr int BPB = 210, PP = 13, LBPB = 208, NAP = 8, XSG = 8;
   static constexpr bool SIDE_D = true;
 };
+// q2_k (84 bytes) and q3_k (110): the last piece of a block starts at BPB - 16, overlapping the one before it,
+// so that whole blocks travel as 16-byte pieces.  LDS row of q2_k: scales[16] | qs[64] at 16 | piece 5 =
+// block bytes 68 .. 83 at 80 (d at 92, dmin at 94).  q3_k: hmask[32] | qs[64] at 32 | piece 6 = block bytes
+// 94 .. 109 at 96 (scales[12] at 98, d at 110).
+template <>
+struct StGeom<KQ_Q2_K> {
+  static constexpr int BPB = 84, PP = 6, LBPB = 96, NAP = 4, XSG = 8;
+  static constexpr bool SIDE_D = false;
+};
+template <>
+struct StGeom<KQ_Q3_K> {
+  static constexpr int BPB = 110, PP = 7, LBPB = 112, NAP = 4, XSG = 8;
+  static constexpr bool SIDE_D = false;
+};
+// byte offset of piece p inside a block
+template <int C>
+__device__ __forceinline__ uint32_t st_piece_off(int p) {
+  using G = StGeom<C>;
+  if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) return p == G::PP - 1 ? (uint32_t)(G::BPB - 16) : 16u * (uint32_t)p;
+  return 16u * (uint32_t)p;
+}
 template <int C>
 struct StUnit {
   using G = StGeom<C>;
@@ -241,6 +259,109 @@ __device__ __forceinline__ void q45k_unit(const uint8_t* __restrict__ bl, int kg
   });
 }
 
+// ------------------------------------------------------------------ q2_k / q3_k unit
+// Lane (row, kg) owns half kg of the superblock: weights 128 kg + 32 j + l, field j = 0..3 (bits 2 j, 2 j + 1 of
+// qs[32 kg + l]), l = 0..31; sub-block (16 weights, one scale) 8 kg + 2 j + l / 16.  Fields are masked in place:
+// 1024 + 4^j q.  q3_k: the third bit of the weight (hmask[l] bit 4 kg + j) is moved next to its field, bit
+// 2 j + 2, so the code reads 1024 + 4^j (q2 + 4 h), and the weight is q - 4.
+// MFMA (j, wi): word wi of the half, l = 4 wi .. 4 wi + 3; activations = A pair j, block wi.
+template <int C, int R, int AS>
+__device__ __forceinline__ void q23k_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
+                                          const float* __restrict__ xsum, int xsum_row_stride, float* acc) {
+  constexpr int RG = (R + 3) / 4;
+  constexpr int QS = C == KQ_Q2_K ? 16 : 32;
+  u32x4 q[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) q[i] = *reinterpret_cast<const u32x4*>(bl + QS + 32 * kg + 16 * i);
+  uint32_t w8[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) w8[i] = q[i >> 2][i & 3] >> 8;
+  uint32_t hw[8] = {0, 0, 0, 0, 0, 0, 0, 0}, hw8[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  float mul[8], sub[8];
+  if constexpr (C == KQ_Q2_K) {
+    const uint2 scw = *reinterpret_cast<const uint2*>(bl + 8 * kg);
+    const uint32_t dd = *reinterpret_cast<const uint32_t*>(bl + 92);
+    const float d = kq::h2f((uint16_t)(dd & 0xffff)) * xscale, dmin = kq::h2f((uint16_t)(dd >> 16)) * xscale;
+#pragma unroll
+    for (int sl = 0; sl < 8; sl++) {
+      const uint32_t b = ((sl < 4 ? scw.x : scw.y) >> (8 * (sl & 3))) & 0xff;
+      const float sc = (float)(b & 0xf), mn = (float)(b >> 4);
+      const float f = 1.0f / (float)(1 << (2 * (sl >> 1)));  // 1 / 4^j
+      mul[sl] = d * sc * f;
+      sub[sl] = fmaf(mul[sl], 1024.0f, dmin * mn);
+    }
+  } else {
+    const u32x4 hm0 = *reinterpret_cast<const u32x4*>(bl), hm1 = *reinterpret_cast<const u32x4*>(bl + 16);
+    const int sh = 4 * kg;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      hw[i] = hm0[i] >> sh;
+      hw[4 + i] = hm1[i] >> sh;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) hw8[i] = hw[i] >> 8;
+    // block bytes 94 .. 109 sit at 96 .. 111: scales[12] from 98, d at 110
+    const u32x4 t = *reinterpret_cast<const u32x4*>(bl + 96);
+    const uint32_t aux0 = __builtin_amdgcn_alignbyte(t[1], t[0], 2), aux1 = __builtin_amdgcn_alignbyte(t[2], t[1], 2);
+    const uint32_t tmp = __builtin_amdgcn_alignbyte(t[3], t[2], 2) >> sh;
+    const float d = kq::h2f((uint16_t)(t[3] >> 16)) * xscale;
+    const uint32_t lo = ((aux0 >> sh) & 0x0f0f0f0fu) | ((tmp & 0x03030303u) << 4);
+    const uint32_t hi = ((aux1 >> sh) & 0x0f0f0f0fu) | (((tmp >> 2) & 0x03030303u) << 4);
+#pragma unroll
+    for (int sl = 0; sl < 8; sl++) {
+      const float sc = (float)(int)(((sl < 4 ? lo : hi) >> (8 * (sl & 3))) & 0xff) - 32.0f;
+      const float f = 1.0f / (float)(1 << (2 * (sl >> 1)));
+      mul[sl] = d * sc * f;
+      sub[sl] = d * sc * (1024.0f * f + 4.0f);
+    }
+  }
+  float xs[R][8];
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    const float4 t0 = *reinterpret_cast<const float4*>(xsum + r * xsum_row_stride + 8 * kg);
+    const float4 t1 = *reinterpret_cast<const float4*>(xsum + r * xsum_row_stride + 8 * kg + 4);
+    xs[r][0] = t0.x; xs[r][1] = t0.y; xs[r][2] = t0.z; xs[r][3] = t0.w;
+    xs[r][4] = t1.x; xs[r][5] = t1.y; xs[r][6] = t1.z; xs[r][7] = t1.w;
+  }
+  const uint32_t magic = opaque_vgpr(0x64006400u);
+  const uint32_t mask_f[4] = {opaque_sgpr(0x00030003u), opaque_sgpr(0x000c000cu), opaque_sgpr(0x00300030u),
+                              opaque_sgpr(0x00c000c0u)};
+  const uint32_t bit_f[4] = {opaque_sgpr(0x00040004u), opaque_sgpr(0x00100010u), opaque_sgpr(0x00400040u),
+                             opaque_sgpr(0x01000100u)};
+  (void)bit_f;
+  SFor<4>::run([&](auto jj) {
+    constexpr int j = decltype(jj)::value;
+    f16x4 av[RG];
+#pragma unroll
+    for (int g = 0; g < RG; g++) av[g] = __builtin_bit_cast(f16x4, areg[g * AS + j]);
+    SFor<2>::run([&](auto hh) {
+      constexpr int hs = decltype(hh)::value;  // l / 16
+      f32x4 p[RG];
+#pragma unroll
+      for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
+      SFor<4>::run([&](auto ee) {
+        constexpr int wi = 4 * hs + decltype(ee)::value;
+        u32x2 bv;
+        bv.x = and_or(q[wi >> 2][wi & 3], mask_f[j], magic);  // weights l, l + 2
+        bv.y = and_or(w8[wi], mask_f[j], magic);              // weights l + 1, l + 3
+        if constexpr (C == KQ_Q3_K) {
+          bv.x = and_or(hw[wi] << (j + 2), bit_f[j], opaque_vgpr(bv.x));
+          bv.y = and_or(hw8[wi] << (j + 2), bit_f[j], opaque_vgpr(bv.y));
+        }
+#pragma unroll
+        for (int g = 0; g < RG; g++)
+          p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(av[g], __builtin_bit_cast(f16x4, bv), p[g], 3, wi, 0);
+      });
+      constexpr int sl = 2 * j + hs;
+      SFor<R>::run([&](auto rr) {
+        constexpr int r = decltype(rr)::value;
+        acc[r] = fmaf(mul[sl], p[r / 4][r % 4], acc[r]);
+        acc[r] = fmaf(-sub[sl], xs[r][sl], acc[r]);
+      });
+    });
+  });
+}
+
 // ------------------------------------------------------------------ q6_k unit
 // Lane (row, hf) owns half hf of the superblock: weights 128 hf + 32 t + l, t = 0..3, l = 0..31.  LDS row:
 // ql[128] | qh[64] | int8 scales[16]; d sits in the slot's side area (one dword per row).  Low nibble of the
@@ -320,15 +441,19 @@ __device__ __forceinline__ void q6k_unit(const uint8_t* __restrict__ bl, float d
 template <int MB>
 constexpr int st_xch() { return MB > 4 ? 2 : MB; }  // activation rows staged at a time
 
-template <int C, int DT, int MB, int D, int WGS>
-__global__ __launch_bounds__(ST_THREADS, WGS) void stream_gemv_kernel(StArgs a) {
+// XU = units (superblocks) a wave handles per tile at most: 4 or 8, i.e. K ranges of up to 16 or 32 superblocks
+// per workgroup (the A registers of all of them stay resident).
+// NW = waves per workgroup (4 or 8): wave w owns superblocks sb_begin + w + NW u of the workgroup's K range.
+template <int C, int DT, int MB, int D, int WGS, int XU, int NW>
+__global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
+  constexpr int ST_XU = XU, ST_WAVES = NW;
   using G = StGeom<C>;
   using U = StUnit<C>;
   constexpr int R = MB;
   constexpr int RG = (MB + 3) / 4, XCH = st_xch<MB>(), NCH = MB / XCH;
   constexpr int NAP = G::NAP, XSG = G::XSG;
   constexpr int AS = ST_XU * NAP;  // A register pairs per row group
-  constexpr int XL = 2;  // 16-byte activation loads per lane and row: 4 units x 256 values
+  constexpr int XL = XU / 2;  // 16-byte activation loads per lane and row: XU units x 256 values
 
 #ifdef KQ_ST_TS
   uint64_t ts[8];
@@ -359,7 +484,7 @@ __global__ __launch_bounds__(ST_THREADS, WGS) void stream_gemv_kernel(StArgs a) 
   int sb_end = a.ksplit > 1 ? sb_begin + a.sb_per_split : nsb;
   sb_end = sb_end < nsb ? sb_end : nsb;
   const int sbn = sb_end - sb_begin;
-  const int nu = sbn > wave ? (sbn - wave + ST_WAVES - 1) / ST_WAVES : 0;  // wave-uniform, 0..4
+  const int nu = sbn > wave ? (sbn - wave + ST_WAVES - 1) / ST_WAVES : 0;  // wave-uniform, 0..XU
 
   // ---- activation loads first: they are the oldest loads of the wave
   const uint16_t* x16 = static_cast<const uint16_t*>(a.x);
@@ -385,7 +510,7 @@ __global__ __launch_bounds__(ST_THREADS, WGS) void stream_gemv_kernel(StArgs a) 
     r = r < rpt ? r : rpt - 1;
     r = row0 + r;
     r = r < row_lim ? r : row_lim;
-    return (uint32_t)(r - row0) * row_bytes + 16u * p;  // r >= row0: a tile always starts inside the matrix
+    return (uint32_t)(r - row0) * row_bytes + st_piece_off<C>(p);  // r >= row0: a tile always starts inside the matrix
   };
   // (offsets are relative to the tile's first row; a tile always starts inside the matrix)
   // Elements of the stream: (tile, unit) in tile-major order.  `it`, `iu`, `islot`: next element to issue.
@@ -419,7 +544,7 @@ __global__ __launch_bounds__(ST_THREADS, WGS) void stream_gemv_kernel(StArgs a) 
   SFor<U::FULL + 1>::run([&](auto t) {
     constexpr int T = decltype(t)::value;
     const int i = lane + 64 * T, r = i / G::PP;
-    goff[T] = (uint32_t)(r < rpt ? r : rpt - 1) * row_bytes + 16u * (i - r * G::PP);
+    goff[T] = (uint32_t)(r < rpt ? r : rpt - 1) * row_bytes + st_piece_off<C>(i - r * G::PP);
   });
   if (nu == 0) it = tiles;  // a wave without superblocks (short K range) only joins the barriers
 
@@ -457,6 +582,7 @@ __global__ __launch_bounds__(ST_THREADS, WGS) void stream_gemv_kernel(StArgs a) 
   // row 4 g + fi that MFMA block fa needs.
   //   q4_k / q5_k: pair pc, block 2 e + h  -> k = 128 kg + 32 (2 (pc / 2) + h) + 16 (pc % 2) + 4 e
   //   q6_k:        pair 2 t + e / 4, block 2 (e % 4) -> k = 128 hf + 32 t + 4 e  (odd blocks unused)
+  //   q2_k / q3_k: pair j, block wi -> k = 128 kg + 32 j + 4 wi
   const int fa = (lane >> 2) & 7, fi = lane & 3;
   u32x2 areg[RG * AS];
   SFor<NCH>::run([&](auto cc) {
@@ -506,6 +632,8 @@ __global__ __launch_bounds__(ST_THREADS, WGS) void stream_gemv_kernel(StArgs a) 
         int koff;  // in f16 elements inside the half
         if constexpr (C == KQ_Q6_K)
           koff = 32 * (pr >> 1) + 16 * (pr & 1) + 4 * (fa >> 1);
+        else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K)
+          koff = 32 * pr + 4 * fa;
         else
           koff = 64 * (pr >> 1) + 32 * (fa & 1) + 16 * (pr & 1) + 4 * (fa >> 1);
         areg[g * AS + T] = *reinterpret_cast<const u32x2*>(xb + u * 512 + koff * 2);
@@ -541,6 +669,8 @@ __global__ __launch_bounds__(ST_THREADS, WGS) void stream_gemv_kernel(StArgs a) 
         if constexpr (C == KQ_Q6_K) {
           const float dx = kq::h2f((uint16_t)*reinterpret_cast<const uint32_t*>(slot + ST_ROWS * G::LBPB + 4 * crow)) * xscale;
           q6k_unit<R, AS>(bl, dx, kg, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
+        } else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) {
+          q23k_unit<C, R, AS>(bl, kg, xscale, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
         } else {
           q45k_unit<C, R, AS>(bl, kg, xscale, areg + u * NAP, xsum + u * 8, ST_XU * 8, acc);
         }
@@ -584,7 +714,7 @@ __global__ __launch_bounds__(ST_THREADS, WGS) void stream_gemv_kernel(StArgs a) 
   }
 }
 
-template <int C, int MB, int D>
+template <int C, int MB, int D, int ST_XU, int ST_WAVES>
 constexpr size_t st_lds_bytes() {
   return (size_t)ST_WAVES * (D * StUnit<C>::SLOT + st_xch<MB>() * ST_XU * 512 + MB * ST_XU * 2 * StGeom<C>::XSG * 4) +
          2 * ST_WAVES * MB * 64 * 4;
@@ -611,31 +741,45 @@ int st_num_cus() {
   return cus;
 }
 
-// K split: every workgroup gets at most 16 superblocks; with fewer row tiles than 1.5 per CU the range is cut
-// further so that about two workgroups per CU exist.
+// K split: a workgroup takes at most 16 superblocks (32 where the kernel with eight units per wave applies: codecs
+// with four A register pairs per unit, up to four rows); with fewer row tiles than g_st_fill_pct per 100 CUs the
+// range is cut further so that about two workgroups per CU exist.
 struct StSplit {
   int ksplit, sb_per_split;
 };
-StSplit st_split_plan(int N, int K, int cus) {
-  const int nsb = K >> 8, tiles = (N + ST_ROWS - 1) / ST_ROWS;
-  int want = (nsb + 15) / 16;
-  if (tiles * want < cus + cus / 2) {
+int g_st_fill_pct = 150;
+int g_st_min_rpt = 24;
+int g_st_nw8 = 1;
+int st_max_sb(int codec, int M);
+// superblocks a workgroup can take: 32 with the eight-wave kernel, which fits the LDS for up to two rows, and for
+// three or four rows of the codecs with small units
+int st_max_sb(int codec, int M) {
+  if (!g_st_nw8 || M > 4) return 16;
+  return M <= 2 || (codec != KQ_Q5_K && codec != KQ_Q6_K) ? 32 : 16;
+}
+StSplit st_split_plan(int M, int N, int K, int codec, int cus) {
+  const int nsb = K >> 8, tiles = (N + ST_ROWS - 1) / ST_ROWS, maxsb = st_max_sb(codec, M);
+  int want = (nsb + maxsb - 1) / maxsb;
+  // one or two rows: a single workgroup per CU over the whole K range beats a split with its reduction launch
+  const int fill = M <= 2 && g_st_fill_pct == 150 ? 100 : g_st_fill_pct;
+  if (tiles * want * 100 < cus * fill) {
     int more = (2 * cus + tiles - 1) / tiles;
     if (more > nsb / 4) more = nsb / 4;  // at least one superblock per wave
     if (more > want) want = more;
   }
   if (want < 1) want = 1;
   int per = (nsb + want - 1) / want;
-  if (per > 16) per = 16;
+  if (per > maxsb) per = maxsb;
   StSplit p{(nsb + per - 1) / per, per};
   return p;
 }
 
-template <int C, int DT, int MB, int D>
+template <int C, int DT, int MB, int D, int XU, int NW = 4>
 int st_launch_one(StArgs a, int splits, hipStream_t s) {
-  constexpr size_t lds = st_lds_bytes<C, MB, D>();
-  constexpr int WGS = lds <= 80 * 1024 ? 2 : 1;
-  auto kern = stream_gemv_kernel<C, DT, MB, D, WGS>;
+  constexpr size_t lds = st_lds_bytes<C, MB, D, XU, NW>();
+  static_assert(lds <= 160 * 1024, "workgroup does not fit the LDS of a CU");
+  constexpr int WGS = lds <= 80 * 1024 && NW == 4 ? 2 : 1;
+  auto kern = stream_gemv_kernel<C, DT, MB, D, WGS, XU, NW>;
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
     KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -651,11 +795,11 @@ int st_launch_one(StArgs a, int splits, hipStream_t s) {
     const int tiles32 = (a.N + ST_ROWS - 1) / ST_ROWS;
     const int rounds = (tiles32 + gx - 1) / gx;
     const int rpt = (a.N + rounds * gx - 1) / (rounds * gx);
-    a.rpt = rpt >= 24 && rpt < ST_ROWS ? rpt : ST_ROWS;
+    a.rpt = rpt >= g_st_min_rpt && rpt < ST_ROWS ? rpt : ST_ROWS;
     a.tiles = (a.N + a.rpt - 1) / a.rpt;
   }
   if (gx > a.tiles) gx = a.tiles;
-  hipLaunchKernelGGL(kern, dim3(gx, 1, splits), dim3(ST_THREADS), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(gx, 1, splits), dim3(64 * NW), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
   if (splits > 1) {
     const int count = a.M * a.N;
@@ -668,36 +812,45 @@ int st_launch_one(StArgs a, int splits, hipStream_t s) {
 
 template <int C, int DT>
 int st_launch_m(const StArgs& a, int splits, hipStream_t s) {
-  constexpr int D1 = C == KQ_Q6_K ? 2 : 2;
-  if (a.M == 1) return st_launch_one<C, DT, 1, D1>(a, splits, s);
-  if (a.M == 2) return st_launch_one<C, DT, 2, 2>(a, splits, s);
-  if (a.M <= 4) return st_launch_one<C, DT, 4, 2>(a, splits, s);
-  return st_launch_one<C, DT, 8, 2>(a, splits, s);
+  constexpr int D = 2;  // units in LDS per wave; 3 and 4 measured slower for every codec
+  if (a.sb_per_split > 16) {
+    // K ranges of 17 .. 32 superblocks: eight waves of four units (st_max_sb allows this for up to four rows).
+    // Four waves of eight units, the alternative without more waves, took 9.0 instead of 7.1 us on q2_k 8192^2.
+    if (a.M == 1) return st_launch_one<C, DT, 1, D, 4, 8>(a, splits, s);
+    if (a.M == 2) return st_launch_one<C, DT, 2, D, 4, 8>(a, splits, s);
+    if constexpr (C != KQ_Q5_K && C != KQ_Q6_K) return st_launch_one<C, DT, 4, D, 4, 8>(a, splits, s);
+  }
+  if (a.M == 1) return st_launch_one<C, DT, 1, D, 4>(a, splits, s);
+  if (a.M == 2) return st_launch_one<C, DT, 2, D, 4>(a, splits, s);
+  if (a.M <= 4) return st_launch_one<C, DT, 4, D, 4>(a, splits, s);
+  return st_launch_one<C, DT, 8, D, 4>(a, splits, s);
 }
 
-bool st_codec_ok(int codec) { return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K; }
+bool st_codec_ok(int codec) {
+  return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K || codec == KQ_Q2_K || codec == KQ_Q3_K;
+}
 
 }  // namespace
 
 bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const void* w) {
   if (!st_codec_ok(codec) || M < 1 || M > 8 || N < 1 || K < 256 || (K & 255)) return false;
   if ((int64_t)N * (K >> 8) * 210 >= (int64_t)1 << 40) return false;
-  // q4_k / q5_k pieces are fetched 16-byte aligned, q6_k blocks are 2-byte multiples
-  const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;
+  // q4_k / q5_k pieces are fetched 16-byte aligned; q6_k, q3_k blocks are 2-byte multiples, q2_k blocks 4-byte ones
+  const uintptr_t wmask = codec == KQ_Q6_K || codec == KQ_Q3_K ? 1 : codec == KQ_Q2_K ? 3 : 15;
   if (reinterpret_cast<uintptr_t>(w) & wmask) return false;
   return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 }
 
 size_t kq_stream_workspace_bytes(int M, int N, int K, int codec) {
   if (!st_codec_ok(codec) || M < 1 || M > 8 || (K & 255) || K < 256) return 0;
-  const StSplit p = st_split_plan(N, K, st_num_cus());
+  const StSplit p = st_split_plan(M, N, K, codec, st_num_cus());
   return p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
 }
 
 int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                          size_t ws_bytes, hipStream_t s) {
   if (!kq_stream_supported(M, N, K, codec, x, w)) return KQ_ERR_UNSUPPORTED;
-  const StSplit p = st_split_plan(N, K, st_num_cus());
+  const StSplit p = st_split_plan(M, N, K, codec, st_num_cus());
   if (p.ksplit > 1 && (!ws || ws_bytes < (size_t)p.ksplit * M * N * sizeof(float) || (reinterpret_cast<uintptr_t>(ws) & 3)))
     return KQ_ERR_UNSUPPORTED;  // the caller falls through to the kernels that can run unsplit
   StArgs a{};
@@ -715,5 +868,13 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
     return dtype == KQ_F16 ? st_launch_m<KQ_Q4_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q4_K, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q5_K)
     return dtype == KQ_F16 ? st_launch_m<KQ_Q5_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q5_K, KQ_BF16>(a, p.ksplit, s);
+  if (codec == KQ_Q2_K)
+    return dtype == KQ_F16 ? st_launch_m<KQ_Q2_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q2_K, KQ_BF16>(a, p.ksplit, s);
+  if (codec == KQ_Q3_K)
+    return dtype == KQ_F16 ? st_launch_m<KQ_Q3_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q3_K, KQ_BF16>(a, p.ksplit, s);
   return dtype == KQ_F16 ? st_launch_m<KQ_Q6_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q6_K, KQ_BF16>(a, p.ksplit, s);
 }
+
+extern "C" void kq_set_stream_fill(int pct) { g_st_fill_pct = pct > 0 ? pct : 150; }
+extern "C" void kq_set_stream_min_rpt(int r) { g_st_min_rpt = r > 0 ? r : 24; }
+extern "C" void kq_set_stream_nw8(int v) { g_st_nw8 = v; }
