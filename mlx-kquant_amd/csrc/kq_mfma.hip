@@ -1388,21 +1388,23 @@ bool sk_shape_ok(int M, int K, int codec, const void* x, const void* w, const vo
 }  // namespace
 
 size_t kq_qmm_tuned_workspace_bytes(int M, int N, int K, int codec) {
-  if (!sk_codec_ok(codec) || M < 1 || M > SK_MAXM || (K & 255) || K == 0) return 0;
+  if (M < 1 || M > SK_MAXM || (K & 255) || K == 0) return 0;
+  const size_t st = kq_stream_workspace_bytes(M, N, K, codec);  // also covers codecs only the streamed kernel takes
+  if (!sk_codec_ok(codec)) return st;
   const SkSplit p = sk_split_plan(N, K);
   const size_t own = p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
-  const size_t st = kq_stream_workspace_bytes(M, N, K, codec);
   return own > st ? own : st;
 }
 
 int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                         size_t ws_bytes, hipStream_t s) {
-  if (!sk_shape_ok(M, K, codec, x, w, nullptr)) return KQ_ERR_UNSUPPORTED;
-  // up to four activation rows of q4_k / q5_k / q6_k: the streamed kernel (variant 5), unless a test pins another
+  // up to eight activation rows of the K-quants, iq4_xs, iq3_s, iq2_xxs: the streamed kernel (variant 5), unless a
+  // test pins another
   if (g_sk_variant == 0 || g_sk_variant == 5) {
     const int rc = kq_launch_qmm_stream(x, w, y, M, N, K, codec, dtype, ws, ws_bytes, s);
     if (rc != KQ_ERR_UNSUPPORTED) return rc;
   }
+  if (!sk_shape_ok(M, K, codec, x, w, nullptr)) return KQ_ERR_UNSUPPORTED;
   SkArgs a{};
   a.x = x;
   a.w = w;

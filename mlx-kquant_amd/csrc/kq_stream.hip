@@ -1,12 +1,13 @@
-// Streamed skinny-M (decode) kernel: y[M,N] = x[M,K] . W^T for M <= 4, codecs q4_k / q5_k / q6_k.
+// Streamed skinny-M (decode) kernel: y[M,N] = x[M,K] . W^T for M <= 8, codecs q2_k ... q6_k, iq4_xs, iq2_xxs.
 // The weight bytes go HBM -> LDS with direct-to-LDS loads (global_load_lds_dwordx4): no staging
 // registers, no LDS store instructions, and a wave keeps its next units in flight while it works.
 //
-// Mapping.  A workgroup (4 waves) owns tiles of 32 weight rows and a K range of at most 16
-// superblocks; wave w takes superblocks w, w + 4, ... of the range, a "unit" being 32 rows x one
+// Mapping.  A workgroup (4 or 8 waves) owns tiles of up to 32 weight rows and a K range of at most 4
+// superblocks per wave; wave w takes superblocks w, w + NW, ... of the range, a "unit" being 32 rows x one
 // superblock.  Workgroups are persistent: tile t of workgroup b is tile b + t * gridDim.x, so the
 // activations are prepared once per workgroup and the weight stream of the next tile is already on
-// its way while the current one is multiplied.
+// its way while the current one is multiplied.  Longer K ranges are split over grid z with an f32
+// reduction launch behind.
 //
 // Matrix cores.  v_mfma_f32_4x4x4_16b_f16 is sixteen independent 4 x 4 x 4 products: block b = lanes
 // 4 b .. 4 b + 3 multiplies four activation rows (A) by four weight rows (B).  Lane l serves weight
@@ -16,9 +17,11 @@
 // eight MFMAs, lane (kg, a, i) keeping the four activations that row i needs in MFMA number a.  The
 // activations of a whole unit are 4 (q4_k / q5_k) or 8 (q6_k) such pairs, loaded once per workgroup.
 //
-// Codes.  As in the other tuned kernels a weight enters the matrix core as an exact f16 integer made
+// Codes.  As in the other tuned kernels a K-quant weight enters the matrix core as an exact f16 integer made
 // with one AND-OR (0x6400 | field = 1024 + field, fields masked in place); scales, the 1024 offset and
-// the block minimum are applied in f32 to the per-lane partial sums.
+// the block minimum are applied in f32 to the per-lane partial sums.  The codebook codecs read their values as
+// ready f16 from tables the workgroup builds in LDS (iq4_xs: byte -> two values; iq2_xxs: grid index -> eight
+// magnitudes, sign index -> eight sign masks).
 //
 // Waiting.  The compiler cannot see a direct-to-LDS load land, so these loads are issued from inline
 // assembly and every wait on them is an explicit s_waitcnt vmcnt(n): loads return in order, n is the
@@ -127,12 +130,39 @@ struct StGeom<KQ_Q3_K> {
   static constexpr int BPB = 110, PP = 7, LBPB = 112, NAP = 4, XSG = 8;
   static constexpr bool SIDE_D = false;
 };
+// The codebook codecs put their byte arrays on 16-byte LDS boundaries by starting pieces at odd block offsets:
+//   iq4_xs  (136): piece 0 = bytes 0 .. 15 (d, scales_h, scales_l), piece i = bytes 8 + 16 (i - 1) ..: qs[q] at 16 + q
+//   iq2_xxs  (66): pieces at 0, 2, 18, 34, 50: d at 0, the eight 8-byte groups at 16 + 8 ib
+template <>
+struct StGeom<KQ_IQ4_XS> {
+  static constexpr int BPB = 136, PP = 9, LBPB = 144, NAP = 4, XSG = 8;
+  static constexpr bool SIDE_D = false;
+};
+template <>
+struct StGeom<KQ_IQ2_XXS> {
+  static constexpr int BPB = 66, PP = 5, LBPB = 80, NAP = 4, XSG = 8;
+  static constexpr bool SIDE_D = false;
+};
 // byte offset of piece p inside a block
 template <int C>
 __device__ __forceinline__ uint32_t st_piece_off(int p) {
   using G = StGeom<C>;
   if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) return p == G::PP - 1 ? (uint32_t)(G::BPB - 16) : 16u * (uint32_t)p;
+  if constexpr (C == KQ_IQ4_XS) return p == 0 ? 0u : 16u * (uint32_t)p - 8u;
+  if constexpr (C == KQ_IQ2_XXS) return p == 0 ? 0u : 16u * (uint32_t)p - 14u;
   return 16u * (uint32_t)p;
+}
+// Order of the staged f16 activations inside a group: 0 = k0 k2 k1 k3 per four (the order the masked-in-place codes
+// leave a 32-bit word in), 1 = k0 k1 k2 k3 (codebook entries), 2 = x[j], x[j + 16] interleaved over 32 (iq4_xs: a
+// byte holds weights j and j + 16 of its sub-block).
+template <int C>
+constexpr int st_xord() { return C == KQ_IQ4_XS ? 2 : C == KQ_IQ2_XXS ? 1 : 0; }
+// LDS bytes of the decode tables a workgroup builds for itself
+//   iq4_xs:  [256] byte -> f16 pair (kvalues[low nibble], kvalues[high nibble])
+//   iq2_xxs: [256] grid entry as eight f16 | [128] sign index -> eight f16 sign masks
+template <int C>
+constexpr int st_tbl_bytes() {
+  return C == KQ_IQ4_XS ? 1024 : C == KQ_IQ2_XXS ? 4096 + 2048 : 0;
 }
 template <int C>
 struct StUnit {
@@ -149,6 +179,7 @@ struct StArgs {
   const uint8_t* w;
   void* y;
   int M, N, K, tiles;
+  const uint8_t* grids;  // device copy of the IQ codebooks (codebook codecs)
   int rpt;  // weight rows per tile (<= 32): fewer than 32 evens the rows out over one round of workgroups
   float* partial;  // split-K: [ksplit][M][N] f32
   int ksplit, sb_per_split;
@@ -362,6 +393,87 @@ __device__ __forceinline__ void q23k_unit(const uint8_t* __restrict__ bl, int kg
   });
 }
 
+// ------------------------------------------------------------------ iq4_xs unit
+// Lane (row, kg) owns sub-blocks 4 kg .. 4 kg + 3 (16 bytes of qs each; byte j = weights j and j + 16).  One table
+// read turns a byte into the f16 pair of its two codebook values; two bytes make the B operand of one MFMA,
+// whose activations are staged in the matching order x[j], x[j + 16], x[j + 1], x[j + 17].
+// MFMA (ib, q): bytes 2 q, 2 q + 1 of sub-block ib; activations = A pair ib, block q.
+template <int R, int AS>
+__device__ __forceinline__ void iq4xs_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
+                                           const uint8_t* __restrict__ tbl, float* acc) {
+  constexpr int RG = (R + 3) / 4;
+  const u32x2 hdr = *reinterpret_cast<const u32x2*>(bl);
+  const float d = kq::h2f((uint16_t)(hdr.x & 0xffff)) * xscale;
+  const uint32_t sh = (hdr.x >> 16) >> (8 * kg), sl = hdr.y >> (16 * kg);
+  SFor<4>::run([&](auto ii) {
+    constexpr int ib = decltype(ii)::value;
+    const u32x4 qv = *reinterpret_cast<const u32x4*>(bl + 16 + 64 * kg + 16 * ib);
+    f32x4 p[RG];
+#pragma unroll
+    for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
+    SFor<8>::run([&](auto qq) {
+      constexpr int q = decltype(qq)::value;
+      const uint32_t w = qv[q >> 1];
+      const uint32_t i0 = (w >> (16 * (q & 1))) & 0xff, i1 = (w >> (16 * (q & 1) + 8)) & 0xff;
+      u32x2 bv;
+      bv.x = *reinterpret_cast<const uint32_t*>(tbl + 4 * i0);
+      bv.y = *reinterpret_cast<const uint32_t*>(tbl + 4 * i1);
+#pragma unroll
+      for (int g = 0; g < RG; g++)
+        p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, areg[g * AS + ib]),
+                                                  __builtin_bit_cast(f16x4, bv), p[g], 3, q, 0);
+    });
+    const int ls = (int)(((sl >> (4 * ib)) & 15) | (((sh >> (2 * ib)) & 3) << 4));
+    const float dl = d * (float)(ls - 32);
+    SFor<R>::run([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      acc[r] = fmaf(dl, p[r / 4][r % 4], acc[r]);
+    });
+  });
+}
+
+// ------------------------------------------------------------------ iq2_xxs unit
+// Lane (row, kg) owns the 8-byte groups 4 kg .. 4 kg + 3 (32 weights each): four grid index bytes, then a word of
+// four 7-bit sign indices and the 4-bit scale.  Index -> eight f16 magnitudes, sign index -> eight f16 sign
+// masks (16-byte table reads), XOR.  MFMAs (ib, l, half): A pair ib, block 2 l + half.
+template <int R, int AS>
+__device__ __forceinline__ void iq2xxs_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
+                                            const uint8_t* __restrict__ tbl, float* acc) {
+  constexpr int RG = (R + 3) / 4;
+  const float d = kq::h2f(*reinterpret_cast<const uint16_t*>(bl)) * xscale * 0.25f;
+  const u32x4 q0 = *reinterpret_cast<const u32x4*>(bl + 16 + 32 * kg), q1 = *reinterpret_cast<const u32x4*>(bl + 32 + 32 * kg);
+  const uint8_t* stbl = tbl + 4096;
+  SFor<4>::run([&](auto ii) {
+    constexpr int ib = decltype(ii)::value;
+    const uint32_t gi = ib < 2 ? q0[2 * ib] : q1[2 * (ib - 2)], a1 = ib < 2 ? q0[2 * ib + 1] : q1[2 * (ib - 2) + 1];
+    f32x4 p[RG];
+#pragma unroll
+    for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
+    SFor<4>::run([&](auto ll) {
+      constexpr int l = decltype(ll)::value;
+      const uint32_t idx = (gi >> (8 * l)) & 0xff, si = (a1 >> (7 * l)) & 127;
+      u32x4 gv = *reinterpret_cast<const u32x4*>(tbl + 16 * idx);
+      const u32x4 sm = *reinterpret_cast<const u32x4*>(stbl + 16 * si);
+      gv[0] ^= sm[0];
+      gv[1] ^= sm[1];
+      gv[2] ^= sm[2];
+      gv[3] ^= sm[3];
+      const u32x2 lo = {gv[0], gv[1]}, hi = {gv[2], gv[3]};
+#pragma unroll
+      for (int g = 0; g < RG; g++) {
+        const f16x4 av = __builtin_bit_cast(f16x4, areg[g * AS + ib]);
+        p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, lo), p[g], 3, 2 * l, 0);
+        p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, hi), p[g], 3, 2 * l + 1, 0);
+      }
+    });
+    const float dl = d * (0.5f + (float)(a1 >> 28));
+    SFor<R>::run([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      acc[r] = fmaf(dl, p[r / 4][r % 4], acc[r]);
+    });
+  });
+}
+
 // ------------------------------------------------------------------ q6_k unit
 // Lane (row, hf) owns half hf of the superblock: weights 128 hf + 32 t + l, t = 0..3, l = 0..31.  LDS row:
 // ql[128] | qh[64] | int8 scales[16]; d sits in the slot's side area (one dword per row).  Low nibble of the
@@ -477,6 +589,8 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   _Float16* xs = reinterpret_cast<_Float16*>(wb + D * U::SLOT);
   float* xsum = reinterpret_cast<float*>(wb + D * U::SLOT + XS_BYTES);
   float* red_all = reinterpret_cast<float*>(smem + ST_WAVES * WAVE_BYTES);
+  uint8_t* tbl = smem + ST_WAVES * WAVE_BYTES + 2 * ST_WAVES * R * 64 * 4;  // decode tables (codebook codecs)
+  (void)tbl;
   const uint32_t wb_lds = lds_addr(wb);
 
   // this workgroup's K range and this wave's units: superblocks sb_begin + wave + 4 u
@@ -488,6 +602,9 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 
   // ---- activation loads first: they are the oldest loads of the wave
   const uint16_t* x16 = static_cast<const uint16_t*>(a.x);
+  // codebook codecs: threads 0 .. 127 fetch 16 bytes each of the 2 KiB grid the tables are built from
+  u32x4 greg = {0, 0, 0, 0};
+  if constexpr (C == KQ_IQ2_XXS) greg = gload16(a.grids + KQ_GRID_IQ2XXS + 16 * (tid & 127));
   u32x4 xreg[MB * XL];
   SFor<MB * XL>::run([&](auto t) {
     constexpr int T = decltype(t)::value;
@@ -555,6 +672,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   if (inflight) vmwait<U::UPI>(); else vmwait<0>();
   ST_TS(1);
   SFor<MB * XL>::run([&](auto t) { tie_v(xreg[decltype(t)::value]); });
+  tie_v(greg);
 
   // ---- activations -> f16 fragments (+ sums) in the wave's LDS, then this lane's A registers
   float xscale = 1.0f, inv = 1.0f;
@@ -583,6 +701,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   //   q4_k / q5_k: pair pc, block 2 e + h  -> k = 128 kg + 32 (2 (pc / 2) + h) + 16 (pc % 2) + 4 e
   //   q6_k:        pair 2 t + e / 4, block 2 (e % 4) -> k = 128 hf + 32 t + 4 e  (odd blocks unused)
   //   q2_k / q3_k: pair j, block wi -> k = 128 kg + 32 j + 4 wi
+  //   codebook codecs: pair ib, block b -> staged positions 128 kg + 32 ib + 4 b .. + 3
   const int fa = (lane >> 2) & 7, fi = lane & 3;
   u32x2 areg[RG * AS];
   SFor<NCH>::run([&](auto cc) {
@@ -604,9 +723,34 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
           h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
         }
       }
-      // MFMA fragment order inside a 4-group: k0 k2 k1 k3
-      const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
-      *reinterpret_cast<f16x8*>(xs + (ml * ST_XU + uu) * 256 + 8 * grp) = v8;
+      constexpr int XORD = st_xord<C>();
+      if constexpr (XORD == 0) {  // k0 k2 k1 k3 inside every group of four
+        const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+        *reinterpret_cast<f16x8*>(xs + (ml * ST_XU + uu) * 256 + 8 * grp) = v8;
+      } else if constexpr (XORD == 1) {
+        const f16x8 v8 = {h[0], h[1], h[2], h[3], h[4], h[5], h[6], h[7]};
+        *reinterpret_cast<f16x8*>(xs + (ml * ST_XU + uu) * 256 + 8 * grp) = v8;
+      } else {
+        // x[j], x[j + 16] interleaved over each 32: lanes a and a + 2 of a quad hold x[8 a ..] and x[16 + 8 a ..]
+        // and write one half each of the 16 interleaved values
+        typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
+        uint32_t own[4], par[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          own[e] = __builtin_bit_cast(uint32_t, f16x2v{h[2 * e], h[2 * e + 1]});
+          par[e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own[e], 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+        }
+        const bool high = (grp & 2) != 0;
+        // low lane: own h0..h3 with the partner's h0..h3 behind each; high lane: the partner's h4..h7 ahead of own
+        const uint32_t a0 = high ? par[2] : own[0], a1 = high ? par[3] : own[1];  // first of each pair
+        const uint32_t b0 = high ? own[2] : par[0], b1 = high ? own[3] : par[1];  // second of each pair
+        u32x4 o;
+        o[0] = (a0 & 0xffffu) | (b0 << 16);
+        o[1] = (a0 >> 16) | (b0 & 0xffff0000u);
+        o[2] = (a1 & 0xffffu) | (b1 << 16);
+        o[3] = (a1 >> 16) | (b1 & 0xffff0000u);
+        *reinterpret_cast<u32x4*>(xs + (ml * ST_XU + uu) * 256 + 32 * (grp >> 2) + 16 * (grp & 1) + (high ? 8 : 0)) = o;
+      }
       float sum = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; e++) sum += (float)h[e];
@@ -632,7 +776,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         int koff;  // in f16 elements inside the half
         if constexpr (C == KQ_Q6_K)
           koff = 32 * (pr >> 1) + 16 * (pr & 1) + 4 * (fa >> 1);
-        else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K)
+        else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K || st_tbl_bytes<C>() != 0)
           koff = 32 * pr + 4 * fa;
         else
           koff = 64 * (pr >> 1) + 32 * (fa & 1) + 16 * (pr & 1) + 4 * (fa >> 1);
@@ -640,6 +784,37 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
       });
     }
   });
+
+  // ---- decode tables of the codebook codecs (their grid bytes arrived with the activations)
+  if constexpr (C == KQ_IQ4_XS) {
+    if (tid < 256) {
+      typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
+      const f16x2v e = {(_Float16)kq::kv_iq4nl(tid & 15), (_Float16)kq::kv_iq4nl(tid >> 4)};
+      reinterpret_cast<uint32_t*>(tbl)[tid] = __builtin_bit_cast(uint32_t, e);
+    }
+  }
+  if constexpr (C == KQ_IQ2_XXS) {
+    if (tid < 128) {  // 16 grid bytes -> 16 f16 magnitudes
+      u32x4 o[2];
+#pragma unroll
+      for (int k = 0; k < 16; k += 2) {
+        typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
+        const f16x2v e = {(_Float16)(float)((greg[k >> 2] >> (8 * (k & 3))) & 0xff),
+                          (_Float16)(float)((greg[(k + 1) >> 2] >> (8 * ((k + 1) & 3))) & 0xff)};
+        o[k >> 3][(k >> 1) & 3] = __builtin_bit_cast(uint32_t, e);
+      }
+      *reinterpret_cast<u32x4*>(tbl + 32 * tid) = o[0];
+      *reinterpret_cast<u32x4*>(tbl + 32 * tid + 16) = o[1];
+    }
+    if (tid < 128) {  // sign table: 7-bit index -> eight f16 sign masks
+      const uint32_t sb = kq::ksigns((uint32_t)tid);
+      u32x4 o;
+#pragma unroll
+      for (int w = 0; w < 4; w++) o[w] = (((sb >> (2 * w)) & 1) << 15) | (((sb >> (2 * w + 1)) & 1) << 31);
+      *reinterpret_cast<u32x4*>(tbl + 4096 + 16 * tid) = o;
+    }
+  }
+  if constexpr (st_tbl_bytes<C>() != 0) wg_lds_barrier();
 
   // The other D - 1 units are queued only now: a wave that queues loads faster than the memory system takes them
   // stalls in the issue, and the activation work above would have waited behind that stall.
@@ -671,6 +846,10 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
           q6k_unit<R, AS>(bl, dx, kg, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
         } else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) {
           q23k_unit<C, R, AS>(bl, kg, xscale, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
+        } else if constexpr (C == KQ_IQ4_XS) {
+          iq4xs_unit<R, AS>(bl, kg, xscale, areg + u * NAP, tbl, acc);
+        } else if constexpr (C == KQ_IQ2_XXS) {
+          iq2xxs_unit<R, AS>(bl, kg, xscale, areg + u * NAP, tbl, acc);
         } else {
           q45k_unit<C, R, AS>(bl, kg, xscale, areg + u * NAP, xsum + u * 8, ST_XU * 8, acc);
         }
@@ -717,7 +896,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 template <int C, int MB, int D, int ST_XU, int ST_WAVES>
 constexpr size_t st_lds_bytes() {
   return (size_t)ST_WAVES * (D * StUnit<C>::SLOT + st_xch<MB>() * ST_XU * 512 + MB * ST_XU * 2 * StGeom<C>::XSG * 4) +
-         2 * ST_WAVES * MB * 64 * 4;
+         2 * ST_WAVES * MB * 64 * 4 + st_tbl_bytes<C>();
 }
 
 template <int DT>
@@ -747,15 +926,29 @@ int st_num_cus() {
 struct StSplit {
   int ksplit, sb_per_split;
 };
-int g_st_fill_pct = 150;
-int g_st_min_rpt = 24;
-int g_st_nw8 = 1;
+constexpr int g_st_fill_pct = 150;  // row tiles x splits per 100 CUs below which K is split further
+constexpr int g_st_min_rpt = 24;    // fewest rows a levelled tile may have (16 measured slower than 32)
+constexpr bool g_st_nw8 = true;
 int st_max_sb(int codec, int M);
-// superblocks a workgroup can take: 32 with the eight-wave kernel, which fits the LDS for up to two rows, and for
-// three or four rows of the codecs with small units
+// superblocks a workgroup can take: 32 with the eight-wave kernel where its LDS fits (every codec for up to two
+// rows, the codecs with small units for up to four)
+template <int C>
+constexpr int st_nw8_rows() {
+  return st_lds_bytes<C, 4, 2, 4, 8>() <= 160 * 1024 ? 4 : st_lds_bytes<C, 2, 2, 4, 8>() <= 160 * 1024 ? 2 : 0;
+}
 int st_max_sb(int codec, int M) {
-  if (!g_st_nw8 || M > 4) return 16;
-  return M <= 2 || (codec != KQ_Q5_K && codec != KQ_Q6_K) ? 32 : 16;
+  if (!g_st_nw8) return 16;
+  int rows = 0;
+  switch (codec) {
+    case KQ_Q2_K: rows = st_nw8_rows<KQ_Q2_K>(); break;
+    case KQ_Q3_K: rows = st_nw8_rows<KQ_Q3_K>(); break;
+    case KQ_Q4_K: rows = st_nw8_rows<KQ_Q4_K>(); break;
+    case KQ_Q5_K: rows = st_nw8_rows<KQ_Q5_K>(); break;
+    case KQ_Q6_K: rows = st_nw8_rows<KQ_Q6_K>(); break;
+    case KQ_IQ4_XS: rows = st_nw8_rows<KQ_IQ4_XS>(); break;
+    case KQ_IQ2_XXS: rows = st_nw8_rows<KQ_IQ2_XXS>(); break;
+  }
+  return M <= rows ? 32 : 16;
 }
 StSplit st_split_plan(int M, int N, int K, int codec, int cus) {
   const int nsb = K >> 8, tiles = (N + ST_ROWS - 1) / ST_ROWS, maxsb = st_max_sb(codec, M);
@@ -818,7 +1011,7 @@ int st_launch_m(const StArgs& a, int splits, hipStream_t s) {
     // Four waves of eight units, the alternative without more waves, took 9.0 instead of 7.1 us on q2_k 8192^2.
     if (a.M == 1) return st_launch_one<C, DT, 1, D, 4, 8>(a, splits, s);
     if (a.M == 2) return st_launch_one<C, DT, 2, D, 4, 8>(a, splits, s);
-    if constexpr (C != KQ_Q5_K && C != KQ_Q6_K) return st_launch_one<C, DT, 4, D, 4, 8>(a, splits, s);
+    if constexpr (st_nw8_rows<C>() >= 4) return st_launch_one<C, DT, 4, D, 4, 8>(a, splits, s);
   }
   if (a.M == 1) return st_launch_one<C, DT, 1, D, 4>(a, splits, s);
   if (a.M == 2) return st_launch_one<C, DT, 2, D, 4>(a, splits, s);
@@ -827,7 +1020,8 @@ int st_launch_m(const StArgs& a, int splits, hipStream_t s) {
 }
 
 bool st_codec_ok(int codec) {
-  return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K || codec == KQ_Q2_K || codec == KQ_Q3_K;
+  return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K || codec == KQ_Q2_K || codec == KQ_Q3_K ||
+         codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS;
 }
 
 }  // namespace
@@ -835,8 +1029,9 @@ bool st_codec_ok(int codec) {
 bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const void* w) {
   if (!st_codec_ok(codec) || M < 1 || M > 8 || N < 1 || K < 256 || (K & 255)) return false;
   if ((int64_t)N * (K >> 8) * 210 >= (int64_t)1 << 40) return false;
-  // q4_k / q5_k pieces are fetched 16-byte aligned; q6_k, q3_k blocks are 2-byte multiples, q2_k blocks 4-byte ones
-  const uintptr_t wmask = codec == KQ_Q6_K || codec == KQ_Q3_K ? 1 : codec == KQ_Q2_K ? 3 : 15;
+  // q4_k / q5_k pieces are fetched 16-byte aligned; iq4_xs blocks are 8-byte multiples, q2_k blocks 4-byte ones, the
+  // others 2-byte ones
+  const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : 1;
   if (reinterpret_cast<uintptr_t>(w) & wmask) return false;
   return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 }
@@ -868,6 +1063,13 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
     return dtype == KQ_F16 ? st_launch_m<KQ_Q4_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q4_K, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q5_K)
     return dtype == KQ_F16 ? st_launch_m<KQ_Q5_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q5_K, KQ_BF16>(a, p.ksplit, s);
+  if (codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS) {
+    a.grids = kq_device_grids();
+    if (!a.grids) return KQ_ERR_HIP;
+    if (codec == KQ_IQ4_XS)
+      return dtype == KQ_F16 ? st_launch_m<KQ_IQ4_XS, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_IQ4_XS, KQ_BF16>(a, p.ksplit, s);
+    return dtype == KQ_F16 ? st_launch_m<KQ_IQ2_XXS, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_IQ2_XXS, KQ_BF16>(a, p.ksplit, s);
+  }
   if (codec == KQ_Q2_K)
     return dtype == KQ_F16 ? st_launch_m<KQ_Q2_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q2_K, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q3_K)
@@ -875,6 +1077,4 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
   return dtype == KQ_F16 ? st_launch_m<KQ_Q6_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q6_K, KQ_BF16>(a, p.ksplit, s);
 }
 
-extern "C" void kq_set_stream_fill(int pct) { g_st_fill_pct = pct > 0 ? pct : 150; }
-extern "C" void kq_set_stream_min_rpt(int r) { g_st_min_rpt = r > 0 ? r : 24; }
-extern "C" void kq_set_stream_nw8(int v) { g_st_nw8 = v; }
+
