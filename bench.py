@@ -208,7 +208,8 @@ class Abi:
                 self._check(rc)
         return call
 
-    def moe_glu(self, x, gate, up, codec, idx):
+    def moe_glu(self, x, gate, up, codec, idx, act=0, limit=0.0, alpha=0.0, gate_bias=None, up_bias=None):
+        """act: 0 silu, 1 gelu, 2 silu_limit, 3 swiglu_clamp (f32 [E, N] biases)."""
         torch, lib = self.torch, self.lib
         (T, K), (E, N) = x.shape, gate.shape[:2]
         R = idx.shape[1]
@@ -216,9 +217,11 @@ class Abi:
         out = torch.empty((T, R, N), dtype=x.dtype, device=self.dev)
         nws = lib.kq_moe_workspace_size(T, R, E, N, K, 1, cid, KQ_BF16)
         ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=self.dev)
-        args = (x.data_ptr(), gate.data_ptr(), up.data_ptr(), idx.data_ptr(), None, None, out.data_ptr(), T, R, E, N, K,
-                0, 0.0, 0.0, cid, KQ_BF16, ws.data_ptr(), nws)
-        keep = (x, gate, up, idx, out, ws)
+        args = (x.data_ptr(), gate.data_ptr(), up.data_ptr(), idx.data_ptr(),
+                gate_bias.data_ptr() if gate_bias is not None else None,
+                up_bias.data_ptr() if up_bias is not None else None, out.data_ptr(), T, R, E, N, K,
+                act, float(limit), float(alpha), cid, KQ_BF16, ws.data_ptr(), nws)
+        keep = (x, gate, up, idx, out, ws, gate_bias, up_bias)
 
         def call(stream=None, _keep=keep):
             rc = lib.kq_moe_glu_gather(*args, stream or self.stream)
@@ -226,16 +229,16 @@ class Abi:
                 self._check(rc)
         return call, out
 
-    def gather_qmv(self, h, w, codec, idx):
+    def gather_qmv(self, h, w, codec, idx, bias=None):
         torch, lib = self.torch, self.lib
         (T, R, K), (E, N) = h.shape, w.shape[:2]
         cid = lib.kq_codec_id(codec.encode())
         out = torch.empty((T, R, N), dtype=h.dtype, device=self.dev)
         nws = lib.kq_moe_workspace_size(T, R, E, N, K, 0, cid, KQ_BF16)
         ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=self.dev)
-        args = (h.data_ptr(), w.data_ptr(), idx.data_ptr(), None, out.data_ptr(), T, R, E, N, K, cid, KQ_BF16,
-                ws.data_ptr(), nws)
-        keep = (h, w, idx, out, ws)
+        args = (h.data_ptr(), w.data_ptr(), idx.data_ptr(), bias.data_ptr() if bias is not None else None,
+                out.data_ptr(), T, R, E, N, K, cid, KQ_BF16, ws.data_ptr(), nws)
+        keep = (h, w, idx, out, ws, bias)
 
         def call(stream=None, _keep=keep):
             rc = lib.kq_gather_qmv(*args, stream or self.stream)
@@ -488,22 +491,18 @@ def main():
             ub = torch.randn((E, H), device=dev, generator=gx) * 0.01
             db = torch.randn((E, H), device=dev, generator=gx) * 0.01
             xt = randx((T, H), 0.5)
-            idx = torch.randn((T, E), device=dev, generator=gx).topk(TOPK, dim=-1).indices
-            kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp", limit=7.0, gate_bias=gb, up_bias=ub,
-                                 alpha=1.702)
-            tg, _ = time_calls(torch, [lambda: kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp",
-                                                                     limit=7.0, gate_bias=gb, up_bias=ub, alpha=1.702)],
-                               20, 3, graph=False)
-            h = kq.moe_glu_gather_kq(xt, gate, up, "mxfp4", idx, act="swiglu_clamp", limit=7.0, gate_bias=gb, up_bias=ub,
-                                     alpha=1.702)
-            td, _ = time_calls(torch, [lambda: kq.gather_qmv_kq(h, down, "mxfp4", idx, bias=db)], 20, 3, graph=False)
+            idx = torch.randn((T, E), device=dev, generator=gx).topk(TOPK, dim=-1).indices.to(torch.int32).contiguous()
+            glu_call, h = abi.moe_glu(xt, gate, up, "mxfp4", idx, act=3, limit=7.0, alpha=1.702, gate_bias=gb, up_bias=ub)
+            dn_call = abi.gather_qmv(h, down, "mxfp4", idx, bias=db)
+            tg, _ = time_calls(torch, [glu_call], 100, 20)
+            td, _ = time_calls(torch, [dn_call], 100, 20)
             mbytes = H * kq.bytes_per_row("mxfp4", H)
             ne = int(idx.unique().numel())
             out["moe_mxfp4"] = {"tokens": T, "experts_touched": ne, "glu_us": round(tg * 1e3, 1),
                                 "down_us": round(td * 1e3, 1),
                                 "glu_gbs": round(ne * 2 * mbytes / (tg * 1e-3) / 1e9, 1),
                                 "down_gbs": round(ne * mbytes / (td * 1e-3) / 1e9, 1),
-                                "note": "grouped code-level MFMA kernel (biases, swiglu_clamp), timed through the Python wrapper"}
+                                "note": "grouped code-level MFMA kernel (f32 biases, swiglu_clamp)"}
             del gate, up, down
 
         # ---------------- MoE decode (1 token, 8 of 128 experts of 2048 <-> 768) in the low-bit / fp4 codecs

@@ -158,11 +158,13 @@ __device__ __forceinline__ uint32_t st_piece_off(int p) {
 template <int C>
 constexpr int st_xord() { return C == KQ_IQ4_XS ? 2 : C == KQ_IQ2_XXS ? 1 : 0; }
 // LDS bytes of the decode tables a workgroup builds for itself
-//   iq4_xs:  [256] byte -> f16 pair (kvalues[low nibble], kvalues[high nibble])
+//   iq4_xs:  [256][32] byte -> f16 pair (kvalues[low nibble], kvalues[high nibble]), one copy per LDS bank: lane l
+//            reads copy l % 32, so the 64 data-dependent reads of an instruction never meet in a bank (with a single
+//            copy the bank conflicts took about half of the kernel's time)
 //   iq2_xxs: [256] grid entry as eight f16 | [128] sign index -> eight f16 sign masks
 template <int C>
 constexpr int st_tbl_bytes() {
-  return C == KQ_IQ4_XS ? 1024 : C == KQ_IQ2_XXS ? 4096 + 2048 : 0;
+  return C == KQ_IQ4_XS ? 32768 : C == KQ_IQ2_XXS ? 4096 + 2048 : 0;
 }
 template <int C>
 struct StUnit {
@@ -416,8 +418,8 @@ __device__ __forceinline__ void iq4xs_unit(const uint8_t* __restrict__ bl, int k
       const uint32_t w = qv[q >> 1];
       const uint32_t i0 = (w >> (16 * (q & 1))) & 0xff, i1 = (w >> (16 * (q & 1) + 8)) & 0xff;
       u32x2 bv;
-      bv.x = *reinterpret_cast<const uint32_t*>(tbl + 4 * i0);
-      bv.y = *reinterpret_cast<const uint32_t*>(tbl + 4 * i1);
+      bv.x = *reinterpret_cast<const uint32_t*>(tbl + 128 * i0);
+      bv.y = *reinterpret_cast<const uint32_t*>(tbl + 128 * i1);
 #pragma unroll
       for (int g = 0; g < RG; g++)
         p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, areg[g * AS + ib]),
@@ -787,10 +789,11 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 
   // ---- decode tables of the codebook codecs (their grid bytes arrived with the activations)
   if constexpr (C == KQ_IQ4_XS) {
-    if (tid < 256) {
+    for (int i = tid; i < 256 * 32; i += 64 * ST_WAVES) {  // dword i = entry i / 32, copy i % 32
       typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
-      const f16x2v e = {(_Float16)kq::kv_iq4nl(tid & 15), (_Float16)kq::kv_iq4nl(tid >> 4)};
-      reinterpret_cast<uint32_t*>(tbl)[tid] = __builtin_bit_cast(uint32_t, e);
+      const int b = i >> 5;
+      const f16x2v e = {(_Float16)kq::kv_iq4nl(b & 15), (_Float16)kq::kv_iq4nl(b >> 4)};
+      reinterpret_cast<uint32_t*>(tbl)[i] = __builtin_bit_cast(uint32_t, e);
     }
   }
   if constexpr (C == KQ_IQ2_XXS) {
@@ -847,7 +850,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         } else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) {
           q23k_unit<C, R, AS>(bl, kg, xscale, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
         } else if constexpr (C == KQ_IQ4_XS) {
-          iq4xs_unit<R, AS>(bl, kg, xscale, areg + u * NAP, tbl, acc);
+          iq4xs_unit<R, AS>(bl, kg, xscale, areg + u * NAP, tbl + 4 * (lane & 31), acc);
         } else if constexpr (C == KQ_IQ2_XXS) {
           iq2xxs_unit<R, AS>(bl, kg, xscale, areg + u * NAP, tbl, acc);
         } else {
