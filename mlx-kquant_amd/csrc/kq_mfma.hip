@@ -1,8 +1,9 @@
 // Tuned skinny-M (decode) kernels: y[M,N] = x[M,K] . W^T for M <= 8, weights streamed once from
-// HBM, all multiply-accumulates on the matrix cores.  Codecs: q4_k and q6_k.  The same kernel
-// serves the gathered ops (one grid row per (activation matrix, expert) item) and the fused
-// gate/up GLU op, where a tile holds rows [n0, n0 + h) of the gate matrix followed by the same
-// rows of the up matrix and the epilogue combines them.
+// HBM, all multiply-accumulates on the matrix cores.  Codecs: q2_k, q3_k, q4_k, q5_k, q6_k.  Dense calls
+// go to the streamed kernel of kq_stream.hip first; the kernels here serve the gathered ops (one grid
+// row per (activation matrix, expert) item) and the fused gate/up GLU op, where a tile holds rows
+// [n0, n0 + h) of the gate matrix followed by the same rows of the up matrix and the epilogue combines
+// them, and the dense calls the streamed kernel declines.
 //
 // Mapping.  One workgroup (4 waves) owns a tile of up to 32 weight rows; its waves split K by
 // superblock.  Inside a wave the weights are the B operand of v_mfma_f32_32x32x16_f16: lane l
