@@ -434,7 +434,7 @@ def main():
         if want("prefill"):
             prefill = []
             abi.lib.kq_set_gemm_tile_rows(args.gemm_tile)
-            for c in ("q4_k", "q5_k", "q6_k", "q2_k", "iq4_xs"):
+            for c in ("q4_k", "q5_k", "q6_k", "q2_k", "q3_k", "iq4_xs"):
                 n, k = 28672, 8192
                 # q2_k / iq4_xs run the any-codec kernel (reference-order decode + bf16 x 3 split)
                 wq = quantized_weights(kq, torch, c, n, k, 5, dev)

@@ -122,7 +122,8 @@ size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int 
   if (kq_gemm_supported(M, N, K, codec)) return kq_gemm_workspace_bytes(M, K);
   // split-K partial sums (optional) of whichever skinny kernel takes the call
   const size_t tuned = kq_qmm_tuned_workspace_bytes(M, N, K, codec);
-  const size_t any = (M > 8 && kq_anymma_supported(M, N, K, codec)) ? kq_anymma_dense_workspace_bytes(M, N, K) : 0;
+  size_t any = (M > 8 && kq_anymma_supported(M, N, K, codec)) ? kq_anymma_dense_workspace_bytes(M, N, K) : 0;
+  if (kq_gemm2_low_supported(M, N, K, codec) && kq_gemm2_low_workspace_bytes(M, K) > any) any = kq_gemm2_low_workspace_bytes(M, K);
   return tuned > any ? tuned : any;
 }
 
@@ -149,6 +150,10 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
                           workspace_bytes);
     int rcg = kq_launch_gemm(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev, s);
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
+  }
+  if (kq_gemm2_low_supported(M, N, K, codec) && workspace_dev && workspace_bytes >= kq_gemm2_low_workspace_bytes(M, K)) {
+    const int rcl = kq_launch_gemm2_low(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev, s);
+    if (rcl != KQ_ERR_UNSUPPORTED) return rcl;
   }
   if (M > 8) {
     const int rca = kq_launch_anymma_dense(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype,

@@ -101,6 +101,11 @@ int kq_launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K
 bool kq_gemm2_supported(int M, int N, int K, int codec);
 int kq_launch_gemm2(const void* xh, const void* xhl, const float* rs, const uint8_t* w, void* y, int M, int N, int K,
                     int codec, int dtype, int shape, hipStream_t s);
+// The same tile kernel for q2_k / q3_k (M >= 256, tiles filling the chip): runs its own activation prepass.
+bool kq_gemm2_low_supported(int M, int N, int K, int codec);
+size_t kq_gemm2_low_workspace_bytes(int M, int K);
+int kq_launch_gemm2_low(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                        hipStream_t s);
 // Batched MoE path (q4_k / q5_k / q6_k, more than 16 pairs): pairs sorted by expert, one MFMA GEMM
 // per segment of <= 32 pairs.  rows = activation rows (T for the GLU op, T*R for the down op).
 bool kq_moe_grouped_supported(int P, int E, int N, int K, int codec);

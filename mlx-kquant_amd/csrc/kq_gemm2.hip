@@ -26,11 +26,32 @@ using namespace kqmma;
 using namespace kqdma;
 
 constexpr int G2_TM = 128, G2_MT = 4;
-constexpr int G2_H_STAGE = G2_TM * 32;
+
+// Wire geometry of a weight row's superblock in LDS: PP 16-byte pieces, piece p taken from block byte off(p) and
+// parked at 16 p; HB = bytes of activation sub-block sums per row and superblock (8 or 16 hi / lo pairs).
+//   q2_k (84 B):  pieces 0 .. 4, then the block's last 16 bytes: scales[16] at 0, qs[64] at 16, d at 92, dmin at 94
+//   q3_k (110 B): pieces 0 .. 5, then the block's last 16 bytes: hmask[32] at 0, qs[64] at 32, scales[12] at 98, d at 110
+template <int C>
+struct G2Wire : Wire<C> {
+  static constexpr int HB = 32;
+  __device__ static uint32_t off(int p) { return 16u * (uint32_t)p; }
+};
+template <>
+struct G2Wire<KQ_Q2_K> {
+  static constexpr int BPB = 84, LBPB = 96, PP = 6, QS = 16, HB = 64;
+  __device__ static uint32_t off(int p) { return p == 5 ? 68u : 16u * (uint32_t)p; }
+};
+template <>
+struct G2Wire<KQ_Q3_K> {
+  static constexpr int BPB = 110, LBPB = 112, PP = 7, QS = 32, HB = 64;
+  __device__ static uint32_t off(int p) { return p == 6 ? 94u : 16u * (uint32_t)p; }
+};
+template <int C>
+constexpr bool g2_low() { return C == KQ_Q2_K || C == KQ_Q3_K; }
 
 // WAVES = 8 or 4 (tile 128 x 256 or 128 x 128), KS = K per step (128 or 64)
 template <int C, int WAVES, int KS>
-constexpr int g2_lds_bytes() { return 2 * G2_TM * KS * 2 + 2 * 32 * WAVES * Wire<C>::LBPB + 2 * G2_H_STAGE; }
+constexpr int g2_lds_bytes() { return 2 * G2_TM * KS * 2 + 2 * 32 * WAVES * G2Wire<C>::LBPB + 2 * G2_TM * G2Wire<C>::HB; }
 
 template <int C, int DT, int WAVES, int KS>
 __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_kernel(const _Float16* __restrict__ xh,
@@ -39,7 +60,11 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
                                                                      const uint8_t* __restrict__ w,
                                                                      uint16_t* __restrict__ y, int M, int N, int K,
                                                                      int mtiles) {
-  using G = Wire<C>;
+  using G = G2Wire<C>;
+  constexpr bool LOW = g2_low<C>();
+  constexpr int G2_H_STAGE = G2_TM * G::HB;
+  constexpr int H_INSTR = G2_H_STAGE / 1024;  // load instructions of the sub-block sums per superblock: 4 or 8
+  static_assert(!LOW || (WAVES == 8 && KS == 128), "q2_k / q3_k: the eight-wave shape only");
   constexpr int MT = G2_MT;
   constexpr int G2_WAVES = WAVES, G2_BN = 32 * WAVES, G2_KS = KS;
   constexpr int G2_A_STAGE = G2_TM * KS * 2;
@@ -52,7 +77,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
   constexpr int W_STAGE = G2_BN * G::LBPB;
   constexpr int W_INSTR = G2_BN * G::PP / 64;            // wire load instructions per superblock (all full waves)
   constexpr int W_PER_WAVE = (W_INSTR + G2_WAVES - 1) / G2_WAVES;
-  static_assert(W_PER_WAVE + 1 <= 7 && W_INSTR >= 4 * G2_WAVES, "the step wait covers 4 .. 7 loads per wave");
+  static_assert(W_PER_WAVE + 1 <= 7 && W_INSTR / G2_WAVES + (H_INSTR >= G2_WAVES ? 1 : 0) >= 4,
+                "the step wait covers 4 .. 7 loads per wave");
   static_assert(G2_BN * G::PP % 64 == 0, "wire tile is a whole number of 64-piece loads");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // LDS: A[2] | W[2] | H[2]
@@ -83,13 +109,14 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
     int r = i / G::PP;
     const int p = i - r * G::PP;
     r = r < nrows ? r : nrows - 1;  // rows past N re-read the last row (their columns are not stored)
-    w_voff[q] = (uint32_t)r * row_bytes + 16u * p;
+    w_voff[q] = (uint32_t)r * row_bytes + G::off(p);
   });
   const uint8_t* w_base = w + (size_t)n0 * row_bytes;
-  // X halves: 128 rows x 32 bytes = 4 loads, waves 0..3
-  const int h_i = 64 * (wave & 3) + lane;
-  const uint32_t h_voff = (uint32_t)(h_i >> 1) * (uint32_t)nsb * 32u + 16u * (h_i & 1);
-  const uint8_t* h_base = reinterpret_cast<const uint8_t*>(xhl) + (size_t)m0 * nsb * 32;
+  // X halves: 128 rows x HB bytes = H_INSTR loads, waves 0 .. H_INSTR - 1
+  constexpr int HPR = G::HB / 16;  // pieces per row
+  const int h_i = 64 * (wave & (H_INSTR - 1)) + lane;
+  const uint32_t h_voff = (uint32_t)(h_i / HPR) * (uint32_t)nsb * (uint32_t)G::HB + 16u * (h_i % HPR);
+  const uint8_t* h_base = reinterpret_cast<const uint8_t*>(xhl) + (size_t)m0 * nsb * G::HB;
 
   auto issue_a = [&](int step) {  // K step `step` (KS wide) -> A stage step % 2
     const uint8_t* base = a_base + (size_t)step * (G2_KS * 2);
@@ -104,13 +131,13 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
       constexpr int q = decltype(qq)::value;
       if (wave + G2_WAVES * q < W_INSTR) dma16(base, w_voff[q], l + q * (G2_WAVES * 1024));
     });
-    if (wave < 4) dma16(h_base + (size_t)sb * 32, h_voff, lds0 + H_OFF + (sb & 1) * G2_H_STAGE + wave * 1024);
+    if (wave < H_INSTR) dma16(h_base + (size_t)sb * G::HB, h_voff, lds0 + H_OFF + (sb & 1) * G2_H_STAGE + wave * 1024);
   };
   // load instructions of one issue_w of this wave (wave-uniform)
   int w_count = 0;
 #pragma unroll
   for (int q = 0; q < W_PER_WAVE; q++) w_count += (wave + G2_WAVES * q < W_INSTR) ? 1 : 0;
-  w_count += wave < 4 ? 1 : 0;
+  w_count += wave < H_INSTR ? 1 : 0;
 
   // ---- fragment addresses
   // A fragment of m-block t, MFMA group g of the step = (sub-block g / 2, K-half s = g % 2): lane half kg holds the
@@ -119,9 +146,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
   uint32_t a_addr[GPS];
 #pragma unroll
   for (int g = 0; g < GPS; g++)
-    a_addr[g] = (uint32_t)l32 * (16u * PR) + 16u * (uint32_t)((4 * (g >> 1) + 2 * kg + (g & 1)) ^ swz(l32));
+    a_addr[g] = (uint32_t)l32 * (16u * PR) +
+                16u * (uint32_t)((LOW ? 2 * g + kg : 4 * (g >> 1) + 2 * kg + (g & 1)) ^ swz(l32));
   const uint8_t* b_lane0 = smem + W_OFF + (wave * 32 + l32) * G::LBPB;
-  const uint8_t* h_lane0 = smem + H_OFF + l32 * 32 + 16 * kg;
+  const uint8_t* h_lane0 = smem + H_OFF + l32 * G::HB + 16 * kg;
 
   f32x16 acc[MT], part[MT];
 #pragma unroll
@@ -136,6 +164,133 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
   // per-superblock state shared by the two half steps
   float d = 0.f, dmin32 = 0.f;
   uint32_t scw[2] = {0, 0}, mnw[2] = {0, 0};
+  uint32_t lsc[4] = {0, 0, 0, 0};  // q2_k: the 16 scale / min bytes; q3_k: the 16 unpacked 6-bit scales
+  const uint32_t mask_f[4] = {opaque_sgpr(0x00030003u), opaque_sgpr(0x000c000cu), opaque_sgpr(0x00300030u),
+                              opaque_sgpr(0x00c000c0u)};
+  const uint32_t bit_f[4] = {opaque_sgpr(0x00040004u), opaque_sgpr(0x00100010u), opaque_sgpr(0x00400040u),
+                             opaque_sgpr(0x01000100u)};
+  (void)mask_f;
+  (void)bit_f;
+
+  // q2_k / q3_k step: MFMA group g of half n = part (sub-block 8 n + g, one scale): field j = g / 2 of the bytes
+  // qs[32 n + 16 (g % 2) + 8 kg .. + 7].  The field is masked in place (1024 + 4^j q; q3_k: its third bit, hmask bit
+  // 4 n + j, is moved to bit 2 j + 2 first) and one packed fma turns it into the exact integer sc q.  The rest of the
+  // weight, -dmin m_s (q2_k) or -4 d sc_s (q3_k), is two more MFMAs per superblock on the hi / lo sums of x.
+  auto k_step_low = [&](auto partc, const uint8_t* a_stage, const uint8_t* b_lane, const uint8_t* h_lane) {
+    constexpr int part_i = decltype(partc)::value;
+    if constexpr (part_i == 0) {
+      if constexpr (C == KQ_Q2_K) {
+        const uint4 sv = *reinterpret_cast<const uint4*>(b_lane);
+        lsc[0] = sv.x;
+        lsc[1] = sv.y;
+        lsc[2] = sv.z;
+        lsc[3] = sv.w;
+        const uint32_t dd = *reinterpret_cast<const uint32_t*>(b_lane + 92);
+        d = kq::h2f((uint16_t)(dd & 0xffff));
+        dmin32 = kq::h2f((uint16_t)(dd >> 16)) * 16.0f;
+      } else {
+        const uint4 t = *reinterpret_cast<const uint4*>(b_lane + 96);  // block bytes 94 .. 109
+        const uint32_t aux0 = __builtin_amdgcn_alignbyte(t.y, t.x, 2), aux1 = __builtin_amdgcn_alignbyte(t.z, t.y, 2);
+        const uint32_t tmp = __builtin_amdgcn_alignbyte(t.w, t.z, 2);
+        d = kq::h2f((uint16_t)(t.w >> 16));
+        dmin32 = d * 16.0f;
+        lsc[0] = (aux0 & 0x0f0f0f0fu) | ((tmp & 0x03030303u) << 4);
+        lsc[1] = (aux1 & 0x0f0f0f0fu) | (((tmp >> 2) & 0x03030303u) << 4);
+        lsc[2] = ((aux0 >> 4) & 0x0f0f0f0fu) | (((tmp >> 4) & 0x03030303u) << 4);
+        lsc[3] = ((aux1 >> 4) & 0x0f0f0f0fu) | (((tmp >> 6) & 0x03030303u) << 4);
+      }
+    }
+    uint2 qv[2], hv[2] = {{0, 0}, {0, 0}};
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      qv[h] = *reinterpret_cast<const uint2*>(b_lane + G::QS + 32 * part_i + 16 * h + 8 * kg);
+      if constexpr (C == KQ_Q3_K) hv[h] = *reinterpret_cast<const uint2*>(b_lane + 16 * h + 8 * kg);
+    }
+    f16x8 afr[2][MT], bfr[2];
+    auto load_a = [&](auto gc, int buf) {
+      constexpr int g = decltype(gc)::value;
+#pragma unroll
+      for (int t = 0; t < MT; t++) afr[buf][t] = *reinterpret_cast<const f16x8*>(a_stage + a_addr[g] + t * (32 * 16 * PR));
+    };
+    auto decode = [&](auto gc) -> f16x8 {
+      constexpr int g = decltype(gc)::value, j = g >> 1, h = g & 1, s = 8 * part_i + g;
+      const uint32_t sb8 = (lsc[s >> 2] >> (8 * (s & 3))) & 0xff;
+      const float scf = C == KQ_Q2_K ? (float)(sb8 & 15) : (float)(int)sb8 - 32.0f;
+      constexpr float f = 1.0f / (float)(1 << (2 * j));  // the field reads 4^j q
+      const _Float16 sch = (_Float16)(scf * f);
+      const _Float16 off = (_Float16)(-1024.0f * f * scf);
+      const f16x2 scp = {sch, sch}, offp = {off, off};
+      const uint32_t w0 = h ? qv[1].x : qv[0].x, w1 = h ? qv[1].y : qv[0].y;
+      uint32_t fr[4] = {(w0 & mask_f[j]) | magic, ((w0 >> 8) & mask_f[j]) | magic, (w1 & mask_f[j]) | magic,
+                        ((w1 >> 8) & mask_f[j]) | magic};
+      if constexpr (C == KQ_Q3_K) {
+        constexpr int from = 4 * part_i + j, to = 2 * j + 2;
+        auto place = [&](uint32_t word, int fr_bit) -> uint32_t {
+          return fr_bit >= to ? word >> (fr_bit - to) : word << (to - fr_bit);
+        };
+        const uint32_t m0 = h ? hv[1].x : hv[0].x, m1 = h ? hv[1].y : hv[0].y;
+        fr[0] |= place(m0, from) & bit_f[j];
+        fr[1] |= place(m0, from + 8) & bit_f[j];
+        fr[2] |= place(m1, from) & bit_f[j];
+        fr[3] |= place(m1, from + 8) & bit_f[j];
+      }
+      f16x2 bq[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) bq[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fr[e]), scp, offp);
+      return f16x8{bq[0][0], bq[0][1], bq[1][0], bq[1][1], bq[2][0], bq[2][1], bq[3][0], bq[3][1]};
+    };
+    constexpr int DEC_VALU = C == KQ_Q3_K ? 26 : 16;
+    load_a(std::integral_constant<int, 0>{}, 0);
+    bfr[0] = decode(std::integral_constant<int, 0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    StaticFor<GPS>::run([&](auto gc) {
+      constexpr int g = decltype(gc)::value;
+      if constexpr (g + 1 < GPS) {
+        load_a(std::integral_constant<int, g + 1>{}, (g + 1) & 1);
+        bfr[(g + 1) & 1] = decode(std::integral_constant<int, g + 1>{});
+      }
+#pragma unroll
+      for (int t = 0; t < MT; t++) {
+        if constexpr (part_i == 0 && g == 0)
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t], bfr[0], f32x16{0}, 0, 0, 0);
+        else
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[g & 1][t], bfr[g & 1], part[t], 0, 0, 0);
+      }
+      if constexpr (g + 1 < GPS) {
+        __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, (DEC_VALU + MT - 1) / MT, 0);
+        }
+      }
+    });
+    if constexpr (part_i == SPS - 1) {
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[t][i] = fmaf(d, part[t][i], acc[t][i]);
+      // the other term: sum_s c_s X_s with X_s = 16 (hi_s + lo_s); c_s = m_s (q2_k) or 4 sc_s (q3_k), s = 8 kg .. + 7
+      _Float16 cj[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const uint32_t b = (lsc[2 * kg + (j >> 2)] >> (8 * (j & 3))) & 0xff;
+        cj[j] = C == KQ_Q2_K ? (_Float16)(float)(b >> 4) : (_Float16)(4.0f * ((float)(int)b - 32.0f));
+      }
+      const f16x8 bm = {cj[0], cj[1], cj[2], cj[3], cj[4], cj[5], cj[6], cj[7]};
+#pragma unroll
+      for (int t = 0; t < MT; t++) {
+        const f16x8 ahi = *reinterpret_cast<const f16x8*>(h_lane + t * (32 * G::HB));
+        const f16x8 alo = *reinterpret_cast<const f16x8*>(h_lane + t * (32 * G::HB) + 32);
+        part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahi, bm, f32x16{0}, 0, 0, 0);
+        part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(alo, bm, part[t], 0, 0, 0);
+      }
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[t][i] = fmaf(-dmin32, part[t][i], acc[t][i]);
+    }
+  };
 
   // one step: MFMA groups it = GPS part .. GPS part + GPS - 1 of the superblock (sub-block j = it / 2, K-half s = it % 2)
   auto k_step = [&](auto partc, const uint8_t* a_stage, const uint8_t* b_lane, const uint8_t* h_lane) {
@@ -270,7 +425,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
       lds_barrier();
       if (p + 1 < SPS || sb + 1 < nsb) issue_a(step + 1);
       if (p == 0 && sb + 1 < nsb) issue_w(sb + 1);
-      k_step(pc, smem + A_OFF + (p & 1) * G2_A_STAGE, b_lane, h_lane);
+      if constexpr (LOW)
+        k_step_low(pc, smem + A_OFF + (p & 1) * G2_A_STAGE, b_lane, h_lane);
+      else
+        k_step(pc, smem + A_OFF + (p & 1) * G2_A_STAGE, b_lane, h_lane);
     });
   }
 
@@ -315,7 +473,55 @@ int launch_gemm2_shape(const _Float16* xh, const _Float16* xhl, const float* rs,
   return launch_gemm2<C, DT, 8, 128>(xh, xhl, rs, w, y, M, N, K, s);
 }
 
+// activation prepass with the sums of the 16-weight sub-blocks (q2_k / q3_k)
+template <int DT>
+__global__ __launch_bounds__(PP_THREADS) void gemm2_prepass16_kernel(const uint16_t* __restrict__ x, _Float16* __restrict__ xh,
+                                                                     _Float16* __restrict__ xhl, float* __restrict__ rs,
+                                                                     int M, int K) {
+  __shared__ float red[PP_THREADS / 64];
+  prepass_row<DT, true>(x, xh, xhl, rs, M, K, blockIdx.x, threadIdx.x, red);
+}
+
+template <int C, int DT>
+int launch_gemm2_low(const void* x, const uint8_t* w, void* y, int M, int N, int K, void* ws, hipStream_t s) {
+  const int mpad = ((M + G2_TM - 1) / G2_TM) * G2_TM, nsb = K >> 8;
+  _Float16* xh = static_cast<_Float16*>(ws);
+  _Float16* xhl = xh + (size_t)mpad * K;
+  float* rs = reinterpret_cast<float*>(xhl + (size_t)mpad * nsb * 32);
+  hipLaunchKernelGGL((gemm2_prepass16_kernel<DT>), dim3(mpad), dim3(PP_THREADS), 0, s, static_cast<const uint16_t*>(x), xh,
+                     xhl, rs, M, K);
+  KQ_HIP_CHECK(hipGetLastError());
+  return launch_gemm2<C, DT, 8, 128>(xh, xhl, rs, w, y, M, N, K, s);
+}
+
 }  // namespace
+
+// q2_k / q3_k on the 128 x 256 tile kernel: M >= 256 and enough tiles to fill the chip; the any-codec kernel keeps
+// the smaller shapes.
+bool kq_gemm2_low_supported(int M, int N, int K, int codec) {
+  return (codec == KQ_Q2_K || codec == KQ_Q3_K) && M >= 256 && K >= 256 && (K & 255) == 0 && N > 0 &&
+         (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 256 && (int64_t)N * (K >> 8) * 110 < ((int64_t)1 << 32) &&
+         (int64_t)K * 2 * 128 < ((int64_t)1 << 32);
+}
+
+size_t kq_gemm2_low_workspace_bytes(int M, int K) {
+  const size_t mpad = (size_t)((M + G2_TM - 1) / G2_TM) * G2_TM;
+  return mpad * K * 2 + mpad * (K >> 8) * 64 + mpad * 4 + 256;
+}
+
+int kq_launch_gemm2_low(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                        hipStream_t s) {
+  if (!kq_gemm2_low_supported(M, N, K, codec)) return KQ_ERR_UNSUPPORTED;
+  // q2_k blocks are 4-byte multiples, q3_k blocks 2-byte ones
+  if ((reinterpret_cast<uintptr_t>(w) & (codec == KQ_Q2_K ? 3 : 1)) || (reinterpret_cast<uintptr_t>(x) & 15) ||
+      (reinterpret_cast<uintptr_t>(ws) & 15))
+    return KQ_ERR_UNSUPPORTED;
+  if (codec == KQ_Q2_K)
+    return dtype == KQ_F16 ? launch_gemm2_low<KQ_Q2_K, KQ_F16>(x, w, y, M, N, K, ws, s)
+                           : launch_gemm2_low<KQ_Q2_K, KQ_BF16>(x, w, y, M, N, K, ws, s);
+  return dtype == KQ_F16 ? launch_gemm2_low<KQ_Q3_K, KQ_F16>(x, w, y, M, N, K, ws, s)
+                         : launch_gemm2_low<KQ_Q3_K, KQ_BF16>(x, w, y, M, N, K, ws, s);
+}
 
 // xh / xhl / rs: outputs of the activation prepass (kq_launch_act_prepass) for rows padded to a multiple of 128.
 bool kq_gemm2_supported(int M, int N, int K, int codec) {

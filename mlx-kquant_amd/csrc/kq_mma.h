@@ -64,20 +64,22 @@ __device__ __forceinline__ uint32_t opaque_sgpr(uint32_t v) {
 // Outputs for row m (rows >= M are written as zeros):
 //   xh   f16 [Mpad][K]            x * 2^-e[m], k permuted inside 8-groups to k0 k2 k1 k3 k4 k6 k5 k7
 //   xhl  f16 [Mpad][K/256][16]    per superblock: hi_j (8) then lo_j (8) with X_j = 32 (hi_j + lo_j)
+//        S16: [Mpad][K/256][32]   sums of the 16-weight sub-blocks: hi_s (16) then lo_s (16), X_s = 16 (hi_s + lo_s)
 //   rs   f32 [Mpad]               2^e[m]
 // `red` = 4 floats of LDS; every thread of the workgroup must call (one barrier inside for bf16 input).
 constexpr int PP_THREADS = 256;
 
-template <int DT>
+template <int DT, bool S16 = false>
 __device__ __forceinline__ void prepass_row(const uint16_t* __restrict__ x, _Float16* __restrict__ xh,
                                             _Float16* __restrict__ xhl, float* __restrict__ rs, int M, int K, int m,
                                             int tid, float* red) {
   const int ngroups = K >> 3;
+  constexpr int HPS = S16 ? 32 : 16;  // halves per superblock in xhl
   _Float16* xo = xh + (size_t)m * K;
-  _Float16* ho = xhl + (size_t)m * (K >> 8) * 16;
+  _Float16* ho = xhl + (size_t)m * (K >> 8) * HPS;
   if (m >= M) {
     for (int g = tid; g < ngroups; g += PP_THREADS) *reinterpret_cast<u32x4*>(xo + 8 * g) = u32x4{0, 0, 0, 0};
-    for (int i = tid; i < (K >> 8) * 16; i += PP_THREADS) ho[i] = (_Float16)0.f;
+    for (int i = tid; i < (K >> 8) * HPS; i += PP_THREADS) ho[i] = (_Float16)0.f;
     if (tid == 0) rs[m] = 0.f;
     return;
   }
@@ -126,6 +128,16 @@ __device__ __forceinline__ void prepass_row(const uint16_t* __restrict__ x, _Flo
 #pragma unroll
     for (int e = 0; e < 8; e++) s += (float)h[e];
     s += __shfl_xor(s, 1);
+    if constexpr (S16) {  // 2 threads = one 16-wide sub-block
+      if ((tid & 1) == 0) {
+        const int j = g >> 1;  // global 16-wide sub-block index
+        const _Float16 hi = (_Float16)(s * 0.0625f);
+        const _Float16 lo = (_Float16)((s - 16.0f * (float)hi) * 0.0625f);
+        ho[(j >> 4) * 32 + (j & 15)] = hi;
+        ho[(j >> 4) * 32 + 16 + (j & 15)] = lo;
+      }
+      continue;
+    }
     s += __shfl_xor(s, 2);  // 4 threads = one 32-wide sub-block
     if ((tid & 3) == 0) {
       const int j = g >> 2;  // global sub-block index
