@@ -436,7 +436,7 @@ def main():
             abi.lib.kq_set_gemm_tile_rows(args.gemm_tile)
             for c in ("q4_k", "q5_k", "q6_k", "q2_k", "q3_k", "iq4_xs"):
                 n, k = 28672, 8192
-                # q2_k / iq4_xs run the any-codec kernel (reference-order decode + bf16 x 3 split)
+                # all six run the 128 x 256 tile kernel at these shapes except q6_k (64 x 128 tiles)
                 wq = quantized_weights(kq, torch, c, n, k, 5, dev)
                 for m in (512, 2048):
                     # the device idles while the host encodes the weights: about 30 ms of launches bring it back

@@ -46,12 +46,22 @@ struct G2Wire<KQ_Q3_K> {
   static constexpr int BPB = 110, LBPB = 112, PP = 7, QS = 32, HB = 64;
   __device__ static uint32_t off(int p) { return p == 6 ? 94u : 16u * (uint32_t)p; }
 };
+//   iq4_xs (136 B): piece 0 = bytes 0 .. 15 (d, scales_h, scales_l), piece i = bytes 8 + 16 (i - 1) ..: qs[q] at 16 + q;
+//                   no sums of x are needed
+template <>
+struct G2Wire<KQ_IQ4_XS> {
+  static constexpr int BPB = 136, LBPB = 144, PP = 9, QS = 16, HB = 0;
+  __device__ static uint32_t off(int p) { return p == 0 ? 0u : 16u * (uint32_t)p - 8u; }
+};
 template <int C>
 constexpr bool g2_low() { return C == KQ_Q2_K || C == KQ_Q3_K; }
+constexpr int G2_IQ4_TBL = 1024;  // iq4_xs: [256] byte -> f16 pair (kvalues[low nibble], kvalues[high nibble])
 
 // WAVES = 8 or 4 (tile 128 x 256 or 128 x 128), KS = K per step (128 or 64)
 template <int C, int WAVES, int KS>
-constexpr int g2_lds_bytes() { return 2 * G2_TM * KS * 2 + 2 * 32 * WAVES * G2Wire<C>::LBPB + 2 * G2_TM * G2Wire<C>::HB; }
+constexpr int g2_lds_bytes() {
+  return 2 * G2_TM * KS * 2 + 2 * 32 * WAVES * G2Wire<C>::LBPB + 2 * G2_TM * G2Wire<C>::HB + (C == KQ_IQ4_XS ? G2_IQ4_TBL : 0);
+}
 
 template <int C, int DT, int WAVES, int KS>
 __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_kernel(const _Float16* __restrict__ xh,
@@ -61,10 +71,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
                                                                      uint16_t* __restrict__ y, int M, int N, int K,
                                                                      int mtiles) {
   using G = G2Wire<C>;
-  constexpr bool LOW = g2_low<C>();
+  constexpr bool LOW = g2_low<C>(), IQ4 = C == KQ_IQ4_XS;
   constexpr int G2_H_STAGE = G2_TM * G::HB;
-  constexpr int H_INSTR = G2_H_STAGE / 1024;  // load instructions of the sub-block sums per superblock: 4 or 8
-  static_assert(!LOW || (WAVES == 8 && KS == 128), "q2_k / q3_k: the eight-wave shape only");
+  constexpr int H_INSTR = G2_H_STAGE / 1024;  // load instructions of the sub-block sums per superblock: 0, 4 or 8
+  static_assert(!(LOW || IQ4) || (WAVES == 8 && KS == 128), "q2_k / q3_k / iq4_xs: the eight-wave shape only");
   constexpr int MT = G2_MT;
   constexpr int G2_WAVES = WAVES, G2_BN = 32 * WAVES, G2_KS = KS;
   constexpr int G2_A_STAGE = G2_TM * KS * 2;
@@ -77,7 +87,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
   constexpr int W_STAGE = G2_BN * G::LBPB;
   constexpr int W_INSTR = G2_BN * G::PP / 64;            // wire load instructions per superblock (all full waves)
   constexpr int W_PER_WAVE = (W_INSTR + G2_WAVES - 1) / G2_WAVES;
-  static_assert(W_PER_WAVE + 1 <= 7 && W_INSTR / G2_WAVES + (H_INSTR >= G2_WAVES ? 1 : 0) >= 4,
+  static_assert(W_PER_WAVE + 1 <= 7 && W_INSTR / G2_WAVES + (H_INSTR >= G2_WAVES ? 1 : 0) >= 4 && H_INSTR <= G2_WAVES,
                 "the step wait covers 4 .. 7 loads per wave");
   static_assert(G2_BN * G::PP % 64 == 0, "wire tile is a whole number of 64-piece loads");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -113,8 +123,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
   });
   const uint8_t* w_base = w + (size_t)n0 * row_bytes;
   // X halves: 128 rows x HB bytes = H_INSTR loads, waves 0 .. H_INSTR - 1
-  constexpr int HPR = G::HB / 16;  // pieces per row
-  const int h_i = 64 * (wave & (H_INSTR - 1)) + lane;
+  constexpr int HPR = G::HB > 0 ? G::HB / 16 : 1;  // pieces per row
+  const int h_i = 64 * (wave & (H_INSTR > 0 ? H_INSTR - 1 : 0)) + lane;
   const uint32_t h_voff = (uint32_t)(h_i / HPR) * (uint32_t)nsb * (uint32_t)G::HB + 16u * (h_i % HPR);
   const uint8_t* h_base = reinterpret_cast<const uint8_t*>(xhl) + (size_t)m0 * nsb * G::HB;
 
@@ -147,7 +157,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
 #pragma unroll
   for (int g = 0; g < GPS; g++)
     a_addr[g] = (uint32_t)l32 * (16u * PR) +
-                16u * (uint32_t)((LOW ? 2 * g + kg : 4 * (g >> 1) + 2 * kg + (g & 1)) ^ swz(l32));
+                16u * (uint32_t)((LOW || IQ4 ? 2 * g + kg : 4 * (g >> 1) + 2 * kg + (g & 1)) ^ swz(l32));
   const uint8_t* b_lane0 = smem + W_OFF + (wave * 32 + l32) * G::LBPB;
   const uint8_t* h_lane0 = smem + H_OFF + l32 * G::HB + 16 * kg;
 
@@ -293,6 +303,81 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
   };
 
   // one step: MFMA groups it = GPS part .. GPS part + GPS - 1 of the superblock (sub-block j = it / 2, K-half s = it % 2)
+  // iq4_xs step: MFMA group g of half `part` = bytes 8 (g % 2) + 4 kg .. + 3 of sub-block 4 part + g / 2.  One table
+  // read turns a byte into the f16 pair of its two codebook values (weights j and j + 16; the activations are staged in
+  // that order).  (ls - 32) kv reaches 4064 and is not always an f16 number (feeding its rounded value cost 8e-4
+  // rel-L2 on bf16 outputs), so a weight goes in as two exact terms, the even part of the scale times kv (twice a
+  // product <= 2032) and its parity times kv: two MFMAs per group on one activation fragment.
+  const uint8_t* tbl = smem + H_OFF + 2 * G2_H_STAGE;
+  if constexpr (IQ4) {
+    if (tid < 256) {
+      const f16x2 e = {(_Float16)kq::kv_iq4nl(tid & 15), (_Float16)kq::kv_iq4nl(tid >> 4)};
+      reinterpret_cast<uint32_t*>(smem + H_OFF + 2 * G2_H_STAGE)[tid] = __builtin_bit_cast(uint32_t, e);
+    }
+  }
+  uint32_t iq_sl = 0, iq_sh = 0;
+  auto k_step_iq4 = [&](auto partc, const uint8_t* a_stage, const uint8_t* b_lane) {
+    constexpr int part_i = decltype(partc)::value;
+    if constexpr (part_i == 0) {
+      const uint2 hdr = *reinterpret_cast<const uint2*>(b_lane);
+      d = kq::h2f((uint16_t)(hdr.x & 0xffff));
+      iq_sh = hdr.x >> 16;
+      iq_sl = hdr.y;
+    }
+    uint32_t qw[GPS];
+#pragma unroll
+    for (int g = 0; g < GPS; g++)
+      qw[g] = *reinterpret_cast<const uint32_t*>(b_lane + 16 + 16 * (4 * part_i + (g >> 1)) + 8 * (g & 1) + 4 * kg);
+    f16x8 afr[2][MT], bfr[2][2];
+    auto load_a = [&](auto gc, int buf) {
+      constexpr int g = decltype(gc)::value;
+#pragma unroll
+      for (int t = 0; t < MT; t++) afr[buf][t] = *reinterpret_cast<const f16x8*>(a_stage + a_addr[g] + t * (32 * 16 * PR));
+    };
+    auto decode = [&](auto gc, f16x8* out) {
+      constexpr int g = decltype(gc)::value, ib = 4 * part_i + (g >> 1);
+      const int ls = (int)(((iq_sl >> (4 * ib)) & 15) | (((iq_sh >> (2 * ib)) & 3) << 4)) - 32;
+      const int odd = ls & 1;  // ls - odd is even and at most 32 in magnitude
+      const _Float16 se = (_Float16)(float)(ls - odd), so = (_Float16)(float)odd;
+      const f16x2 sep = {se, se}, sop = {so, so};
+      f16x2 be[4], bo[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const uint32_t idx = (qw[g] >> (8 * e)) & 0xff;
+        const f16x2 kv = __builtin_bit_cast(f16x2, *reinterpret_cast<const uint32_t*>(tbl + 4 * idx));
+        be[e] = kv * sep;
+        bo[e] = kv * sop;
+      }
+      out[0] = f16x8{be[0][0], be[0][1], be[1][0], be[1][1], be[2][0], be[2][1], be[3][0], be[3][1]};
+      out[1] = f16x8{bo[0][0], bo[0][1], bo[1][0], bo[1][1], bo[2][0], bo[2][1], bo[3][0], bo[3][1]};
+    };
+    load_a(std::integral_constant<int, 0>{}, 0);
+    decode(std::integral_constant<int, 0>{}, bfr[0]);
+    StaticFor<GPS>::run([&](auto gc) {
+      constexpr int g = decltype(gc)::value;
+      if constexpr (g + 1 < GPS) {
+        load_a(std::integral_constant<int, g + 1>{}, (g + 1) & 1);
+        decode(std::integral_constant<int, g + 1>{}, bfr[(g + 1) & 1]);
+      }
+#pragma unroll
+      for (int t = 0; t < MT; t++) {
+        if constexpr (part_i == 0 && g == 0)
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t], bfr[0][0], f32x16{0}, 0, 0, 0);
+        else
+          part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[g & 1][t], bfr[g & 1][0], part[t], 0, 0, 0);
+      }
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+        part[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[g & 1][t], bfr[g & 1][1], part[t], 0, 0, 0);
+    });
+    if constexpr (part_i == SPS - 1) {
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[t][i] = fmaf(d, part[t][i], acc[t][i]);
+    }
+  };
+
   auto k_step = [&](auto partc, const uint8_t* a_stage, const uint8_t* b_lane, const uint8_t* h_lane) {
     constexpr int part_i = decltype(partc)::value;
     constexpr int NQ = GPS / 4;  // nibble pairs (32 wire bytes each) of the step
@@ -427,6 +512,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
       if (p == 0 && sb + 1 < nsb) issue_w(sb + 1);
       if constexpr (LOW)
         k_step_low(pc, smem + A_OFF + (p & 1) * G2_A_STAGE, b_lane, h_lane);
+      else if constexpr (IQ4)
+        k_step_iq4(pc, smem + A_OFF + (p & 1) * G2_A_STAGE, b_lane);
       else
         k_step(pc, smem + A_OFF + (p & 1) * G2_A_STAGE, b_lane, h_lane);
     });
@@ -482,14 +569,27 @@ __global__ __launch_bounds__(PP_THREADS) void gemm2_prepass16_kernel(const uint1
   prepass_row<DT, true>(x, xh, xhl, rs, M, K, blockIdx.x, threadIdx.x, red);
 }
 
+// activation prepass in the order of the iq4 nibble pairs (x[j], x[j + 16] interleaved)
+template <int DT>
+__global__ __launch_bounds__(PP_THREADS) void gemm2_prepass_il16_kernel(const uint16_t* __restrict__ x, _Float16* __restrict__ xh,
+                                                                        _Float16* __restrict__ xhl, float* __restrict__ rs,
+                                                                        int M, int K) {
+  __shared__ float red[PP_THREADS / 64];
+  prepass_row<DT, false, true>(x, xh, xhl, rs, M, K, blockIdx.x, threadIdx.x, red);
+}
+
 template <int C, int DT>
 int launch_gemm2_low(const void* x, const uint8_t* w, void* y, int M, int N, int K, void* ws, hipStream_t s) {
   const int mpad = ((M + G2_TM - 1) / G2_TM) * G2_TM, nsb = K >> 8;
   _Float16* xh = static_cast<_Float16*>(ws);
   _Float16* xhl = xh + (size_t)mpad * K;
   float* rs = reinterpret_cast<float*>(xhl + (size_t)mpad * nsb * 32);
-  hipLaunchKernelGGL((gemm2_prepass16_kernel<DT>), dim3(mpad), dim3(PP_THREADS), 0, s, static_cast<const uint16_t*>(x), xh,
-                     xhl, rs, M, K);
+  if constexpr (C == KQ_IQ4_XS)
+    hipLaunchKernelGGL((gemm2_prepass_il16_kernel<DT>), dim3(mpad), dim3(PP_THREADS), 0, s, static_cast<const uint16_t*>(x),
+                       xh, xhl, rs, M, K);
+  else
+    hipLaunchKernelGGL((gemm2_prepass16_kernel<DT>), dim3(mpad), dim3(PP_THREADS), 0, s, static_cast<const uint16_t*>(x), xh,
+                       xhl, rs, M, K);
   KQ_HIP_CHECK(hipGetLastError());
   return launch_gemm2<C, DT, 8, 128>(xh, xhl, rs, w, y, M, N, K, s);
 }
@@ -499,8 +599,8 @@ int launch_gemm2_low(const void* x, const uint8_t* w, void* y, int M, int N, int
 // q2_k / q3_k on the 128 x 256 tile kernel: M >= 256 and enough tiles to fill the chip; the any-codec kernel keeps
 // the smaller shapes.
 bool kq_gemm2_low_supported(int M, int N, int K, int codec) {
-  return (codec == KQ_Q2_K || codec == KQ_Q3_K) && M >= 256 && K >= 256 && (K & 255) == 0 && N > 0 &&
-         (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 256 && (int64_t)N * (K >> 8) * 110 < ((int64_t)1 << 32) &&
+  return (codec == KQ_Q2_K || codec == KQ_Q3_K || codec == KQ_IQ4_XS) && M >= 256 && K >= 256 && (K & 255) == 0 && N > 0 &&
+         (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 256 && (int64_t)N * (K >> 8) * 136 < ((int64_t)1 << 32) &&
          (int64_t)K * 2 * 128 < ((int64_t)1 << 32);
 }
 
@@ -512,13 +612,16 @@ size_t kq_gemm2_low_workspace_bytes(int M, int K) {
 int kq_launch_gemm2_low(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                         hipStream_t s) {
   if (!kq_gemm2_low_supported(M, N, K, codec)) return KQ_ERR_UNSUPPORTED;
-  // q2_k blocks are 4-byte multiples, q3_k blocks 2-byte ones
-  if ((reinterpret_cast<uintptr_t>(w) & (codec == KQ_Q2_K ? 3 : 1)) || (reinterpret_cast<uintptr_t>(x) & 15) ||
+  // q2_k blocks are 4-byte multiples, q3_k blocks 2-byte ones, iq4_xs blocks 8-byte ones
+  if ((reinterpret_cast<uintptr_t>(w) & (codec == KQ_Q2_K ? 3 : codec == KQ_IQ4_XS ? 7 : 1)) || (reinterpret_cast<uintptr_t>(x) & 15) ||
       (reinterpret_cast<uintptr_t>(ws) & 15))
     return KQ_ERR_UNSUPPORTED;
   if (codec == KQ_Q2_K)
     return dtype == KQ_F16 ? launch_gemm2_low<KQ_Q2_K, KQ_F16>(x, w, y, M, N, K, ws, s)
                            : launch_gemm2_low<KQ_Q2_K, KQ_BF16>(x, w, y, M, N, K, ws, s);
+  if (codec == KQ_IQ4_XS)
+    return dtype == KQ_F16 ? launch_gemm2_low<KQ_IQ4_XS, KQ_F16>(x, w, y, M, N, K, ws, s)
+                           : launch_gemm2_low<KQ_IQ4_XS, KQ_BF16>(x, w, y, M, N, K, ws, s);
   return dtype == KQ_F16 ? launch_gemm2_low<KQ_Q3_K, KQ_F16>(x, w, y, M, N, K, ws, s)
                          : launch_gemm2_low<KQ_Q3_K, KQ_BF16>(x, w, y, M, N, K, ws, s);
 }

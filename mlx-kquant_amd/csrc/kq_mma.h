@@ -69,7 +69,9 @@ __device__ __forceinline__ uint32_t opaque_sgpr(uint32_t v) {
 // `red` = 4 floats of LDS; every thread of the workgroup must call (one barrier inside for bf16 input).
 constexpr int PP_THREADS = 256;
 
-template <int DT, bool S16 = false>
+// IL16: xh keeps x[j], x[j + 16] interleaved over every 32 values instead (a byte of an iq4 block holds weights j
+// and j + 16 of its sub-block).
+template <int DT, bool S16 = false, bool IL16 = false>
 __device__ __forceinline__ void prepass_row(const uint16_t* __restrict__ x, _Float16* __restrict__ xh,
                                             _Float16* __restrict__ xhl, float* __restrict__ rs, int M, int K, int m,
                                             int tid, float* red) {
@@ -121,6 +123,23 @@ __device__ __forceinline__ void prepass_row(const uint16_t* __restrict__ x, _Flo
         h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] & 0xffff));
         h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
       }
+    }
+    if constexpr (IL16) {
+      // threads g and g ^ 2 hold x[8 a ..] and x[16 + 8 a ..] of a 32-block and write one half each of the 16
+      // interleaved values
+      uint32_t own[4], par[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        own[e] = (uint32_t)__builtin_bit_cast(uint16_t, h[2 * e]) | ((uint32_t)__builtin_bit_cast(uint16_t, h[2 * e + 1]) << 16);
+        par[e] = __shfl_xor(own[e], 2);
+      }
+      const bool high = (g & 2) != 0;
+      const uint32_t a0 = high ? par[2] : own[0], a1 = high ? par[3] : own[1];
+      const uint32_t b0 = high ? own[2] : par[0], b1 = high ? own[3] : par[1];
+      const u32x4 o = {(a0 & 0xffffu) | (b0 << 16), (a0 >> 16) | (b0 & 0xffff0000u), (a1 & 0xffffu) | (b1 << 16),
+                       (a1 >> 16) | (b1 & 0xffff0000u)};
+      *reinterpret_cast<u32x4*>(xo + 32 * (g >> 2) + 16 * (g & 1) + (high ? 8 : 0)) = o;
+      continue;
     }
     const f16x8 o = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
     *reinterpret_cast<f16x8*>(xo + 8 * g) = o;

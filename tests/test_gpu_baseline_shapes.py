@@ -66,10 +66,10 @@ def test_config3_prefill_8192_to_28672(kq, codec, M):
 
 
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
-@pytest.mark.parametrize("codec", ["q2_k", "q3_k"])
+@pytest.mark.parametrize("codec", ["q2_k", "q3_k", "iq4_xs"])
 @pytest.mark.parametrize("M,N,K", [(2048, 28672, 8192), (300, 16400, 512), (256, 32768, 256)])
 def test_prefill_q2k_q3k_128x256_tiles(kq, codec, M, N, K, dtype):
-    """q2_k / q3_k prefill on the 128 x 256 tile kernel (M >= 256, 256 or more tiles): the benchmark shape, a ragged
+    """q2_k / q3_k / iq4_xs prefill on the 128 x 256 tile kernel (M >= 256, 256 or more tiles): the benchmark shape, a ragged
     shape (M and N off the tile sizes, two superblocks) and a single-superblock K."""
     _check_matmul(kq, codec, M, N, K, dtype, 78, 48)
 
