@@ -288,7 +288,7 @@ struct MoeArgs {
 };
 
 template <int C, int DT, bool GLU>
-__global__ __launch_bounds__(MOE_THREADS, 2) void moe_grouped_kernel(MoeArgs a) {
+__global__ __launch_bounds__(MOE_THREADS, 3) void moe_grouped_kernel(MoeArgs a) {
   using G = Wire<C>;
   constexpr int WPT = (SLAB * G::PP + MOE_THREADS - 1) / MOE_THREADS;  // wire pieces per thread per step
   constexpr int APT = SEG_M * 32 / MOE_THREADS;                         // activation pieces per thread per step (4)
