@@ -55,7 +55,11 @@ struct CodeGeom {
                                  : C == KQ_IQ2_S ? KQ_GRID_IQ2S : (C == KQ_IQ1_S || C == KQ_IQ1_M) ? KQ_GRID_IQ1S
                                  : C == KQ_IQ3_XXS ? KQ_GRID_IQ3XXS : KQ_GRID_IQ3S;
   static constexpr bool GRID_SIGNED = C == KQ_IQ1_S || C == KQ_IQ1_M;  // int8 entries
-  static constexpr int GRID_BYTES = GRID_N * GRID_W * 2;
+  // 32-weight blocks whose byte j holds weights j and j + 16 as indices of a 16-value table (iq4_nl, mxfp4): the
+  // table in LDS maps a byte to the f16 pair of its two values, and the activations of a block are staged as
+  // x[j], x[j + 16] interleaved, so four table reads are the B operand of an MFMA with no further arithmetic
+  static constexpr bool PAIR_LUT = C == KQ_IQ4_NL || C == KQ_MXFP4;
+  static constexpr int GRID_BYTES = PAIR_LUT ? 1024 : GRID_N * GRID_W * 2;
   // 256-entry table spreading 8 bits over the 8 halves of a B operand: sign bits (bit 15) for the
   // signed codebooks, the fifth code bit (bit 4) for q5_0 / q5_1
   static constexpr bool SIGNS = C == KQ_IQ2_XXS || C == KQ_IQ2_XS || C == KQ_IQ2_S || C == KQ_IQ3_XXS || C == KQ_IQ3_S;
@@ -103,6 +107,29 @@ __device__ __forceinline__ uint32_t lut16(uint32_t n, uint32_t t0, uint32_t t1, 
   // selector bytes 0x0c / 0x0d read as 0x00 / 0xff: 0xff in every byte whose bit 3 is set
   const uint32_t mask = __builtin_amdgcn_perm(n, n, ((n >> 3) & 0x01010101u) | 0x0c0c0c0cu);
   return (hi & mask) | (lo & ~mask);
+}
+// One lane's eight consecutive activations h[0..7] (8-group `pc` of a row) to the row's staging area: in the fragment
+// order k0 k2 k1 k3 inside the group, or (PAIR) with x[j], x[j + 16] interleaved over each 32: lanes pc and pc ^ 2 of a
+// quad hold x[8 a ..] and x[16 + 8 a ..] and write one half each of the 16 interleaved values.
+template <bool PAIR>
+__device__ __forceinline__ void stage_group(uint8_t* row_lds, int pc, const _Float16* h) {
+  if constexpr (!PAIR) {
+    const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+    *reinterpret_cast<f16x8*>(row_lds + 16 * pc) = v8;
+  } else {
+    uint32_t own[4], par[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      own[e] = (uint32_t)__builtin_bit_cast(uint16_t, h[2 * e]) | ((uint32_t)__builtin_bit_cast(uint16_t, h[2 * e + 1]) << 16);
+      par[e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own[e], 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+    }
+    const bool high = (pc & 2) != 0;
+    const uint32_t a0 = high ? par[2] : own[0], a1 = high ? par[3] : own[1];
+    const uint32_t b0 = high ? own[2] : par[0], b1 = high ? own[3] : par[1];
+    const u32x4 o = {(a0 & 0xffffu) | (b0 << 16), (a0 >> 16) | (b0 & 0xffff0000u), (a1 & 0xffffu) | (b1 << 16),
+                     (a1 >> 16) | (b1 & 0xffff0000u)};
+    *reinterpret_cast<u32x4*>(row_lds + 64 * (pc >> 2) + 32 * (pc & 1) + (high ? 16 : 0)) = o;
+  }
 }
 __device__ __forceinline__ float f16bits(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (uint16_t)h); }
 
@@ -170,6 +197,14 @@ __device__ __forceinline__ f16x8 codes(const R& row, int kg, const Tables& t) {
     // 32-weight blocks: weights 0..15 = low nibbles of q[0..15], 16..31 = high nibbles
     constexpr int QOFF = C == KQ_Q4_0 || C == KQ_IQ4_NL ? 2 : C == KQ_Q4_1 ? 4 : C == KQ_Q5_0 ? 6 : C == KQ_Q5_1 ? 8 : 1;
     constexpr int boff = (J / 2) * G::BPB, off = boff + QOFF;
+    if constexpr (G::PAIR_LUT) {
+      // staged positions 16 J + 8 kg .. + 7 = bytes 8 (J % 2) + 4 kg .. + 3 of block J / 2, both nibbles of each
+      const uint32_t w = pick(kg, row.template u32<off + 8 * (J & 1)>(), row.template u32<off + 8 * (J & 1) + 4>());
+      u32x4 r;
+#pragma unroll
+      for (int e = 0; e < 4; e++) r[e] = *reinterpret_cast<const uint32_t*>(t.grid + 4 * ((w >> (8 * e)) & 0xffu));
+      return __builtin_bit_cast(f16x8, r);
+    }
     uint32_t lo = pick(kg, row.template u32<off>(), row.template u32<off + 8>());
     uint32_t hi = pick(kg, row.template u32<off + 4>(), row.template u32<off + 12>());
     if constexpr (J & 1) {
@@ -443,6 +478,13 @@ __global__ __launch_bounds__((64 * WV), (WV == 4 ? 2 : 1)) void codes_skinny_ker
       }
     }
   }
+  if constexpr (G::PAIR_LUT) {
+    if (tid < 256) {
+      const f16x2 e = C == KQ_MXFP4 ? f16x2{(_Float16)kq::kv_mxfp4(tid & 15), (_Float16)kq::kv_mxfp4(tid >> 4)}
+                                    : f16x2{(_Float16)kq::kv_iq4nl(tid & 15), (_Float16)kq::kv_iq4nl(tid >> 4)};
+      reinterpret_cast<uint32_t*>(grid_lds)[tid] = __builtin_bit_cast(uint32_t, e);
+    }
+  }
   if constexpr (G::SPREAD_BYTES > 0) {
     if (tid < 256) {
       const uint32_t b = tid;
@@ -453,7 +495,7 @@ __global__ __launch_bounds__((64 * WV), (WV == 4 ? 2 : 1)) void codes_skinny_ker
                 (bit(4) << P) | (bit(6) << (P + 16)), (bit(5) << P) | (bit(7) << (P + 16))};
     }
   }
-  if constexpr (G::GRID_N > 0 || G::SPREAD_BYTES > 0) lds_barrier();
+  if constexpr (G::GRID_N > 0 || G::SPREAD_BYTES > 0 || G::PAIR_LUT) lds_barrier();
   const Tables tabs{grid_lds, spread_lds};
 
   // ---- piece maps of this wave.  Wire: piece i = lane + 64 t -> (row i / PIECES, piece i % PIECES).
@@ -536,8 +578,7 @@ __global__ __launch_bounds__((64 * WV), (WV == 4 ? 2 : 1)) void codes_skinny_ker
           h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(areg[t][e] >> 16));
         }
       }
-      const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};  // fragment order inside an 8-group
-      *reinterpret_cast<f16x8*>(a_lds + row * XA_STRIDE + 16 * a_pc) = v8;
+      stage_group<G::PAIR_LUT>(a_lds + row * XA_STRIDE, a_pc, h);
       if (a_pc == 0) xs_lds[row] = xscale;
       if constexpr (G::HAS_MIN) {
         float sum = 0.f;
@@ -799,6 +840,13 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
       }
     }
   }
+  if constexpr (G::PAIR_LUT) {
+    if (tid < 256) {
+      const f16x2 e = C == KQ_MXFP4 ? f16x2{(_Float16)kq::kv_mxfp4(tid & 15), (_Float16)kq::kv_mxfp4(tid >> 4)}
+                                    : f16x2{(_Float16)kq::kv_iq4nl(tid & 15), (_Float16)kq::kv_iq4nl(tid >> 4)};
+      reinterpret_cast<uint32_t*>(grid_lds)[tid] = __builtin_bit_cast(uint32_t, e);
+    }
+  }
   if constexpr (G::SPREAD_BYTES > 0) {
     const uint32_t b = tid;  // 256 threads, 256 entries
     auto bit = [&](int i) { return (b >> i) & 1u; };
@@ -889,8 +937,7 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
           h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(areg[t][e] >> 16));
         }
       }
-      const f16x8 v8 = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};  // fragment order inside an 8-group
-      *reinterpret_cast<f16x8*>(a_lds + slot * XA_STRIDE + 16 * a_pc) = v8;
+      stage_group<G::PAIR_LUT>(a_lds + slot * XA_STRIDE, a_pc, h);
       if (a_pc == 0) xs_lds[slot] = xscale;
       if constexpr (G::HAS_MIN) {
         float sum = 0.f;
