@@ -305,7 +305,7 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return 0;
   if (kq_moe_grouped_supported((int)P, E, N, K, codec)) return kq_moe_grouped_workspace_bytes(glu ? T : (int)P, (int)P, E, K);
-  if (kq_codes_moe_supported((int)P, E, N, K, codec)) return kq_codes_moe_workspace_bytes((int)P, E);
+  if (kq_codes_moe_supported((int)P, E, N, K, codec)) return kq_codes_moe_workspace_bytes((int)P, E, glu ? T : (int)P, K);
   if (kq_anymma_moe_supported((int)P, E, N, K, codec)) return kq_anymma_moe_workspace_bytes((int)P, E);
   return 0;
 }
@@ -320,7 +320,7 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
     // legacy / IQ / fp4 codecs (biases and every activation included): code-level grouped kernel
     if (kq_codes_moe_supported((int)P, E, N, K, codec)) {
-      const size_t need = kq_codes_moe_workspace_bytes((int)P, E);
+      const size_t need = kq_codes_moe_workspace_bytes((int)P, E, glu ? T : (int)P, K);
       if (!ws || ws_bytes < need)
         return kq_set_error(KQ_ERR_WORKSPACE, "%s: workspace of %zu bytes required (got %zu)", op, need, ws ? ws_bytes : 0);
       const int rcc = kq_launch_codes_moe(x, static_cast<const uint8_t*>(w), static_cast<const uint8_t*>(w2), idx, bias,

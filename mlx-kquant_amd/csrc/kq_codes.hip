@@ -765,9 +765,72 @@ struct CgArgs {
   int64_t w_expert_stride;
   float limit, alpha;
   KqOutMap om;
+  // outputs of codes_prepass_kernel: per activation row and 256-wide step the f16 values in staging order (512 bytes),
+  // their power-of-two scale and (codecs with a block minimum) the sums of the eight 32-wide blocks
+  const uint8_t* xh;
+  const float* xsc;
+  const float* xsum;
 };
 
 constexpr int CG_THREADS = 256;
+
+// Activation prepass of the grouped kernel: what every workgroup used to redo for its 32 slots at every step (bf16 ->
+// f16 with an exact power-of-two scale per (row, step), staging order, block sums) is done once per row.  One
+// workgroup per row; 32 threads per step, eight steps at a time.  Steps are zero-filled past K.
+template <int DT, bool PAIR, bool SUMS>
+__global__ __launch_bounds__(256) void codes_prepass_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ xh,
+                                                            float* __restrict__ xsc, float* __restrict__ xsum, int K,
+                                                            int nsteps) {
+  const int row = blockIdx.x, tid = threadIdx.x, pc = tid & 31;
+  for (int st = tid >> 5; st < nsteps; st += 8) {
+    const int k0 = CK_STEP * st + 8 * pc;
+    u32x4 v = {0, 0, 0, 0};
+    if (k0 < K) v = *reinterpret_cast<const u32x4*>(x + (size_t)row * K + k0);
+    float xscale = 1.f;
+    _Float16 h[8];
+    if constexpr (DT == KQ_BF16) {
+      float amax = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] << 16)));
+        amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] & 0xffff0000u)));
+      }
+#pragma unroll
+      for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));  // the step's 32 lanes
+      float inv = 1.f;
+      const uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff;
+      if (eb != 0 && eb != 0xff) {
+        int e = (int)eb - 127 - 14;  // the largest magnitude lands in [2^14, 2^15)
+        if (e < -100) e = -100;
+        xscale = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+        inv = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        h[2 * e] = (_Float16)(__builtin_bit_cast(float, v[e] << 16) * inv);
+        h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, v[e] & 0xffff0000u) * inv);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] & 0xffff));
+        h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
+      }
+    }
+    const size_t rs = (size_t)row * nsteps + st;
+    stage_group<PAIR>(xh + rs * 512, pc, h);
+    if (pc == 0) xsc[rs] = xscale;
+    if constexpr (SUMS) {
+      float sum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) sum += (float)h[e];
+      sum += __shfl_xor(sum, 1);
+      sum += __shfl_xor(sum, 2);  // 4 lanes = one 32-weight block
+      if ((pc & 3) == 0) xsum[rs * 8 + (pc >> 2)] = sum;
+    }
+  }
+}
+
 constexpr int CG_BN = 128;
 
 template <int C>
@@ -859,14 +922,13 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
 
   // ---- piece maps.  Activations: piece i = tid + 256 t -> (slot i / 32, 16-byte piece i % 32).
   const int a_slot0 = tid >> 5, a_pc = tid & 31;
-  const uint16_t* a_src[4];
+  size_t a_rs[4];  // (row, step 0) index of the slot's activation row in the prepass outputs
   bool a_live[4];
 #pragma unroll
   for (int t = 0; t < 4; t++) {
     const int slot = a_slot0 + 8 * t;
     a_live[t] = slot < seg.count;
-    const size_t row = (size_t)(a.order[seg.start + (a_live[t] ? slot : 0)] / a.x_div);
-    a_src[t] = static_cast<const uint16_t*>(a.x) + row * K + 8 * a_pc;
+    a_rs[t] = (size_t)(a.order[seg.start + (a_live[t] ? slot : 0)] / a.x_div) * nsteps;
   }
   const uint8_t* w_src[WPT];
   uint32_t w_loff[WPT];
@@ -884,13 +946,21 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
   }
 
   u32x4 areg[4], wreg[WPT];
+  float sreg[4] = {0.f, 0.f, 0.f, 0.f};  // a_pc == 0: the slot's scale; a_pc 8 .. 15 (HAS_MIN): block sum a_pc - 8
   auto issue = [&](int st) {
-    const int kvalid = K - CK_STEP * st;
 #pragma unroll
     for (int t = 0; t < 4; t++) {
       u32x4 av = {0, 0, 0, 0};
-      if (a_live[t] && 8 * a_pc < kvalid) av = *reinterpret_cast<const u32x4*>(a_src[t] + (size_t)CK_STEP * st);
+      float sv = 0.f;
+      if (a_live[t]) {
+        av = *reinterpret_cast<const u32x4*>(a.xh + (a_rs[t] + st) * 512 + 16 * a_pc);
+        if (a_pc == 0) sv = a.xsc[a_rs[t] + st];
+        if constexpr (G::HAS_MIN) {
+          if (a_pc >= 8 && a_pc < 16) sv = a.xsum[(a_rs[t] + st) * 8 + (a_pc - 8)];
+        }
+      }
       areg[t] = av;
+      sreg[t] = sv;
     }
 #pragma unroll
     for (int t = 0; t < WPT; t++) {
@@ -906,46 +976,10 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
 #pragma unroll
     for (int t = 0; t < 4; t++) {
       const int slot = a_slot0 + 8 * t;
-      float xscale = 1.f;
-      _Float16 h[8];
-      if constexpr (DT == KQ_BF16) {
-        float amax = 0.f;
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, areg[t][e] << 16)));
-          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, areg[t][e] & 0xffff0000u)));
-        }
-#pragma unroll
-        for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));  // the slot's 32 lanes
-        float inv = 1.f;
-        const uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff;
-        if (eb != 0 && eb != 0xff) {
-          int e = (int)eb - 127 - 14;  // the largest magnitude lands in [2^14, 2^15)
-          if (e < -100) e = -100;
-          xscale = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
-          inv = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          h[2 * e] = (_Float16)(__builtin_bit_cast(float, areg[t][e] << 16) * inv);
-          h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, areg[t][e] & 0xffff0000u) * inv);
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(areg[t][e] & 0xffff));
-          h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(areg[t][e] >> 16));
-        }
-      }
-      stage_group<G::PAIR_LUT>(a_lds + slot * XA_STRIDE, a_pc, h);
-      if (a_pc == 0) xs_lds[slot] = xscale;
+      *reinterpret_cast<u32x4*>(a_lds + slot * XA_STRIDE + 16 * a_pc) = areg[t];
+      if (a_pc == 0) xs_lds[slot] = sreg[t];
       if constexpr (G::HAS_MIN) {
-        float sum = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) sum += (float)h[e];
-        sum += __shfl_xor(sum, 1);
-        sum += __shfl_xor(sum, 2);  // 4 lanes = one 32-weight block
-        if ((a_pc & 3) == 0) xsum_lds[(a_pc >> 2) * 32 + slot] = sum;
+        if (a_pc >= 8 && a_pc < 16) xsum_lds[(a_pc - 8) * 32 + slot] = sreg[t];
       }
     }
 #pragma unroll
@@ -1103,9 +1137,12 @@ bool kq_codes_moe_supported(int P, int E, int N, int K, int codec) {
          K % kq_geom(codec).wpb == 0;
 }
 
-// Workspace: sorted pair list, segment table, segment count.
-size_t kq_codes_moe_workspace_bytes(int P, int E) {
-  return align256((size_t)P * 4) + align256(((size_t)E + P / 32 + 1) * sizeof(Segment)) + 256;
+// Workspace: sorted pair list, segment table, segment count, then the prepass outputs for `rows` activation rows:
+// f16 steps (512 bytes each), step scales, block sums.
+size_t kq_codes_moe_workspace_bytes(int P, int E, int rows, int K) {
+  const size_t rs = (size_t)rows * ((K + CK_STEP - 1) / CK_STEP);
+  return align256((size_t)P * 4) + align256(((size_t)E + P / 32 + 1) * sizeof(Segment)) + 256 + align256(rs * 512) +
+         align256(rs * 4) + align256(rs * 32);
 }
 
 // x: [rows][K]; pair p reads row p / x_div and expert idx[p]; out [P][N].
@@ -1122,7 +1159,32 @@ int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, cons
   int* nseg = reinterpret_cast<int*>(p + align256((size_t)P * 4) + align256(((size_t)E + P / 32 + 1) * sizeof(Segment)));
   int rc = kq_launch_moe_sort(idx, P, E, order, segs, nseg, s);
   if (rc) return rc;
+  const int rows = glu ? P / (x_div < 1 ? 1 : x_div) : P, nsteps = (K + CK_STEP - 1) / CK_STEP;
+  const size_t rs = (size_t)rows * nsteps;
+  uint8_t* xh = reinterpret_cast<uint8_t*>(nseg) + 256;
+  float* xsc = reinterpret_cast<float*>(xh + align256(rs * 512));
+  float* xsum = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(xsc) + align256(rs * 4));
+  {
+    const bool pair = codec == KQ_IQ4_NL || codec == KQ_MXFP4, sums = codec == KQ_Q4_1 || codec == KQ_Q5_1;
+    const uint16_t* xi = static_cast<const uint16_t*>(x);
+#define KQ_PRE(DTV, PV, SV) \
+  hipLaunchKernelGGL((codes_prepass_kernel<DTV, PV, SV>), dim3(rows), dim3(256), 0, s, xi, xh, xsc, xsum, K, nsteps)
+    if (dtype == KQ_F16) {
+      if (pair) KQ_PRE(KQ_F16, true, false);
+      else if (sums) KQ_PRE(KQ_F16, false, true);
+      else KQ_PRE(KQ_F16, false, false);
+    } else {
+      if (pair) KQ_PRE(KQ_BF16, true, false);
+      else if (sums) KQ_PRE(KQ_BF16, false, true);
+      else KQ_PRE(KQ_BF16, false, false);
+    }
+#undef KQ_PRE
+    KQ_HIP_CHECK(hipGetLastError());
+  }
   CgArgs a{};
+  a.xh = xh;
+  a.xsc = xsc;
+  a.xsum = xsum;
   a.x = x;
   a.w = w;
   a.w2 = w2;
