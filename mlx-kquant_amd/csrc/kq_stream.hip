@@ -407,23 +407,34 @@ __device__ __forceinline__ void iq4xs_unit(const uint8_t* __restrict__ bl, int k
   const u32x2 hdr = *reinterpret_cast<const u32x2*>(bl);
   const float d = kq::h2f((uint16_t)(hdr.x & 0xffff)) * xscale;
   const uint32_t sh = (hdr.x >> 16) >> (8 * kg), sl = hdr.y >> (16 * kg);
-  SFor<4>::run([&](auto ii) {
+  // The table reads of sub-block ib + 1 are issued before the MFMAs of sub-block ib: left to itself the compiler
+  // waits for every pair of reads right before the MFMA that uses it, one LDS round trip per MFMA.
+  u32x2 bv[4][8];
+  auto lookup = [&](auto ii) {
     constexpr int ib = decltype(ii)::value;
     const u32x4 qv = *reinterpret_cast<const u32x4*>(bl + 16 + 64 * kg + 16 * ib);
+    SFor<8>::run([&](auto qq) {
+      constexpr int q = decltype(qq)::value;
+      const uint32_t w = qv[q >> 1];
+      const uint32_t i0 = (w >> (16 * (q & 1))) & 0xff, i1 = (w >> (16 * (q & 1) + 8)) & 0xff;
+      bv[ib][q].x = *reinterpret_cast<const uint32_t*>(tbl + 128 * i0);
+      bv[ib][q].y = *reinterpret_cast<const uint32_t*>(tbl + 128 * i1);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  lookup(std::integral_constant<int, 0>{});
+  SFor<4>::run([&](auto ii) {
+    constexpr int ib = decltype(ii)::value;
+    if constexpr (ib < 3) lookup(std::integral_constant<int, ib + 1>{});
     f32x4 p[RG];
 #pragma unroll
     for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
     SFor<8>::run([&](auto qq) {
       constexpr int q = decltype(qq)::value;
-      const uint32_t w = qv[q >> 1];
-      const uint32_t i0 = (w >> (16 * (q & 1))) & 0xff, i1 = (w >> (16 * (q & 1) + 8)) & 0xff;
-      u32x2 bv;
-      bv.x = *reinterpret_cast<const uint32_t*>(tbl + 128 * i0);
-      bv.y = *reinterpret_cast<const uint32_t*>(tbl + 128 * i1);
 #pragma unroll
       for (int g = 0; g < RG; g++)
         p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, areg[g * AS + ib]),
-                                                  __builtin_bit_cast(f16x4, bv), p[g], 3, q, 0);
+                                                  __builtin_bit_cast(f16x4, bv[ib][q]), p[g], 3, q, 0);
     });
     const int ls = (int)(((sl >> (4 * ib)) & 15) | (((sh >> (2 * ib)) & 3) << 4));
     const float dl = d * (float)(ls - 32);
@@ -445,22 +456,32 @@ __device__ __forceinline__ void iq2xxs_unit(const uint8_t* __restrict__ bl, int 
   const float d = kq::h2f(*reinterpret_cast<const uint16_t*>(bl)) * xscale * 0.25f;
   const u32x4 q0 = *reinterpret_cast<const u32x4*>(bl + 16 + 32 * kg), q1 = *reinterpret_cast<const u32x4*>(bl + 32 + 32 * kg);
   const uint8_t* stbl = tbl + 4096;
-  SFor<4>::run([&](auto ii) {
+  // The table reads of group ib + 1 are issued before the MFMAs of group ib (see iq4xs_unit).
+  u32x4 gv[4][4], sm[4][4];
+  uint32_t a1s[4];
+  auto lookup = [&](auto ii) {
     constexpr int ib = decltype(ii)::value;
     const uint32_t gi = ib < 2 ? q0[2 * ib] : q1[2 * (ib - 2)], a1 = ib < 2 ? q0[2 * ib + 1] : q1[2 * (ib - 2) + 1];
+    a1s[ib] = a1;
+    SFor<4>::run([&](auto ll) {
+      constexpr int l = decltype(ll)::value;
+      const uint32_t idx = (gi >> (8 * l)) & 0xff, si = (a1 >> (7 * l)) & 127;
+      gv[ib][l] = *reinterpret_cast<const u32x4*>(tbl + 16 * idx);
+      sm[ib][l] = *reinterpret_cast<const u32x4*>(stbl + 16 * si);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  lookup(std::integral_constant<int, 0>{});
+  SFor<4>::run([&](auto ii) {
+    constexpr int ib = decltype(ii)::value;
+    if constexpr (ib < 3) lookup(std::integral_constant<int, ib + 1>{});
     f32x4 p[RG];
 #pragma unroll
     for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
     SFor<4>::run([&](auto ll) {
       constexpr int l = decltype(ll)::value;
-      const uint32_t idx = (gi >> (8 * l)) & 0xff, si = (a1 >> (7 * l)) & 127;
-      u32x4 gv = *reinterpret_cast<const u32x4*>(tbl + 16 * idx);
-      const u32x4 sm = *reinterpret_cast<const u32x4*>(stbl + 16 * si);
-      gv[0] ^= sm[0];
-      gv[1] ^= sm[1];
-      gv[2] ^= sm[2];
-      gv[3] ^= sm[3];
-      const u32x2 lo = {gv[0], gv[1]}, hi = {gv[2], gv[3]};
+      const u32x4 v = gv[ib][l] ^ sm[ib][l];
+      const u32x2 lo = {v[0], v[1]}, hi = {v[2], v[3]};
 #pragma unroll
       for (int g = 0; g < RG; g++) {
         const f16x4 av = __builtin_bit_cast(f16x4, areg[g * AS + ib]);
@@ -468,7 +489,7 @@ __device__ __forceinline__ void iq2xxs_unit(const uint8_t* __restrict__ bl, int 
         p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, hi), p[g], 3, 2 * l + 1, 0);
       }
     });
-    const float dl = d * (0.5f + (float)(a1 >> 28));
+    const float dl = d * (0.5f + (float)(a1s[ib] >> 28));
     SFor<R>::run([&](auto rr) {
       constexpr int r = decltype(rr)::value;
       acc[r] = fmaf(dl, p[r / 4][r % 4], acc[r]);
@@ -789,12 +810,16 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 
   // ---- decode tables of the codebook codecs (their grid bytes arrived with the activations)
   if constexpr (C == KQ_IQ4_XS) {
-    for (int i = tid; i < 256 * 32; i += 64 * ST_WAVES) {  // dword i = entry i / 32, copy i % 32
-      typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
-      const int b = i >> 5;
-      const f16x2v e = {(_Float16)kq::kv_iq4nl(b & 15), (_Float16)kq::kv_iq4nl(b >> 4)};
-      reinterpret_cast<uint32_t*>(tbl)[i] = __builtin_bit_cast(uint32_t, e);
-    }
+    // entry b = dwords 32 b .. 32 b + 31 (one copy per LDS bank); a thread computes one entry and writes its
+    // share of the copies with 16-byte stores
+    typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
+    constexpr int TPE = 64 * ST_WAVES / 256;  // threads per entry (1 or 2)
+    const int b = tid & 255, part = tid >> 8;
+    const f16x2v e = {(_Float16)kq::kv_iq4nl(b & 15), (_Float16)kq::kv_iq4nl(b >> 4)};
+    const uint32_t ev = __builtin_bit_cast(uint32_t, e);
+    const u32x4 e4 = {ev, ev, ev, ev};
+#pragma unroll
+    for (int c = 0; c < 8 / TPE; c++) *reinterpret_cast<u32x4*>(tbl + 128 * b + (128 / TPE) * part + 16 * c) = e4;
   }
   if constexpr (C == KQ_IQ2_XXS) {
     if (tid < 128) {  // 16 grid bytes -> 16 f16 magnitudes
