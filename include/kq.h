@@ -192,7 +192,9 @@ int kq_moe_glu_gather_shexp(const void* x_dev, const void* gate_w_dev, const voi
  * shexp_w_dev != NULL: idx is [T, S - 1], slot S - 1 multiplies the shared expert's single matrix (codec
  * `shexp_codec`: the expert codec, or q6_k / q8_0) -- op gather_qmv_mix_kq; shexp_w_dev == NULL: idx is
  * [T, S] and every slot gathers from the stack -- op gather_qmv_mix_ns_kq (pass shexp_codec = -1 to the
- * size query).  The workspace (256-byte aligned) is required.
+ * size query).  Decode-sized calls (one token; up to three with a shared expert; S <= 32) run as one kernel and
+ * need no workspace (the size query returns 0, any pointer is accepted); larger calls need the 256-byte aligned
+ * workspace.  Entries whose expert id is >= E add nothing.
  * Replaces KQuantGatherQMVMixKQ / KQuantGatherQMVMixNSKQ, reference src/kquant_moe_glu.cpp:1274-1364. */
 size_t kq_gather_qmv_mix_workspace_size(int T, int S, int E, int N, int K, int codec, int shexp_codec, int dtype);
 int kq_gather_qmv_mix(const void* x_dev, const void* w_dev, const void* shexp_w_dev, const uint32_t* idx_dev,

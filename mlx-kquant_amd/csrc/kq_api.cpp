@@ -563,8 +563,20 @@ int kq_moe_glu_gather_shexp(const void* x_dev, const void* gate_w_dev, const voi
                              0.f, 0.f, shexp_codec, dtype, sub, sub_bytes, KqOutMap{1, R + 1, R, 0}, stream);
 }
 
+// Decode-sized calls run as one kernel (a workgroup per output element, the slots spread over its waves): one token,
+// or up to three when there is a shared expert (whose other form takes six launches against two); measured at
+// 128 experts of 2048 x 768 q6_k, top-8: 14.4 against 14.1 us without and 15.5 against 25.2 us with a shared
+// expert at one token.  Larger calls run the gathered matmul kernels into f32 slot rows and mix those.
+#ifndef KQ_MIX_SINGLE_TOKENS
+#define KQ_MIX_SINGLE_TOKENS 1
+#endif
+static bool mix_single_launch(int T, int S, bool shared) {
+  return KQ_MIX_SINGLE_TOKENS > 0 && S <= 32 && T <= (shared ? 3 * KQ_MIX_SINGLE_TOKENS : KQ_MIX_SINGLE_TOKENS);
+}
+
 size_t kq_gather_qmv_mix_workspace_size(int T, int S, int E, int N, int K, int codec, int shexp_codec, int dtype) {
   if (T <= 0 || S <= 0) return 0;
+  if (mix_single_launch(T, S, shexp_codec >= 0)) return 0;
   size_t fixed = align256((size_t)T * S * N * 4);  // f32 slot results
   size_t sub = kq_moe_workspace_size(T, S, E, N, K, 0, codec, dtype);
   if (shexp_codec >= 0) {
@@ -591,10 +603,17 @@ static int gather_qmv_mix_impl(const char* op, const void* x_dev, const void* w_
   }
   if (T == 0 || N == 0) return KQ_OK;
   if (!x_dev || !w_dev || !idx_dev || !scores_dev || !out_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (mix_single_launch(T, S, shared)) {
+    const int64_t expert_stride = (int64_t)N * (K / kCodecs[codec].weights_per_block) * kCodecs[codec].bytes_per_block;
+    rc = kq_launch_gather_mix_generic(x_dev, static_cast<const uint8_t*>(w_dev), static_cast<const uint8_t*>(shexp_w_dev),
+                                      idx_dev, scores_dev, bias_dev, out_dev, T, S, E, N, K, expert_stride, codec,
+                                      shared ? shexp_codec : codec, dtype, s);
+    return rc == KQ_OK ? KQ_OK : kq_set_error(rc, "%s: launch failed", op);
+  }
   const size_t need = kq_gather_qmv_mix_workspace_size(T, S, E, N, K, codec, shared ? shexp_codec : -1, dtype);
   if (!workspace_dev || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace_dev) & 255))
     return kq_set_error(KQ_ERR_WORKSPACE, "%s: 256-byte aligned workspace of %zu bytes required", op, need);
-  hipStream_t s = static_cast<hipStream_t>(stream);
   uint8_t* wsb = static_cast<uint8_t*>(workspace_dev);
   float* yf = reinterpret_cast<float*>(wsb);
   size_t o = align256((size_t)T * S * N * 4);
@@ -628,7 +647,7 @@ static int gather_qmv_mix_impl(const char* op, const void* x_dev, const void* w_
                          KqOutMap{1, S, S - 1, 1}, stream);
     if (rc) return rc;
   }
-  return kq_launch_mix_slots(yf, scores_dev, out_dev, T, S, N, dtype, s);
+  return kq_launch_mix_slots(yf, scores_dev, idx_dev, shared ? S - 1 : S, E, out_dev, T, S, N, dtype, s);
 }
 
 int kq_gather_qmv_mix(const void* x_dev, const void* w_dev, const void* shexp_w_dev, const uint32_t* idx_dev,

@@ -73,6 +73,10 @@ int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2,
                              int N, int K, int x_div, int64_t x_batch_stride, int64_t w_expert_stride, int glu,
                              int act, float limit, float alpha, int codec, int dtype, int E, KqOutMap om,
                              hipStream_t s);
+// Score-weighted slot sum in one launch (kq_generic.hip): decode-sized gather_qmv_mix calls.
+int kq_launch_gather_mix_generic(const void* x, const uint8_t* w, const uint8_t* shexp_w, const uint32_t* idx,
+                                 const float* scores, const float* bias, void* out, int T, int S, int E, int N, int K,
+                                 int64_t w_expert_stride, int codec, int shexp_codec, int dtype, hipStream_t s);
 // Tuned path: returns KQ_ERR_UNSUPPORTED (without touching the error text) when no tuned kernel
 // covers the request, so the caller can fall through to the generic kernels.
 // A null / short workspace is allowed: the call then runs without its split-K plan.
@@ -146,7 +150,8 @@ int kq_launch_expert_tile_map(const uint32_t* idx, int rows, int E, uint32_t* ma
                               hipStream_t s);
 int kq_launch_tiles_to_rows(const uint32_t* map, const uint32_t* counts, int cap, int rows, int E, uint32_t none,
                             uint32_t* row_expert, hipStream_t s);
-int kq_launch_mix_slots(const float* yf, const float* scores, void* out, int T, int S, int N, int dtype, hipStream_t s);
+int kq_launch_mix_slots(const float* yf, const float* scores, const uint32_t* idx, int routed, int E, void* out, int T,
+                        int S, int N, int dtype, hipStream_t s);
 // Matrix-core GEMM for every codec (exact bf16 x 3 split of the reference-order decoded weights):
 // prefill, and the batched MoE ops with biases and every activation.
 bool kq_anymma_supported(int M, int N, int K, int codec);

@@ -219,6 +219,97 @@ __global__ __launch_bounds__(GV_THREADS) void gather_generic_kernel(GatherArgs a
   }
 }
 
+// Score-weighted slot sum in one launch (decode-sized calls):
+// out[t][n] = T(sum_s scores[t][s] (x[t][s] . W[idx[t][s]][n] + bias[idx[t][s]][n])), f32 throughout.
+// With a shared expert the last slot reads row n of the one-matrix stack shexp_w in codec C2 (the expert codec,
+// q6_k or q8_0).  Slots whose expert id is >= E add nothing.
+struct MixArgs {
+  const void* x;           // [T][S][K]
+  const uint8_t* w;        // [E][N][row bytes]
+  const uint8_t* shexp_w;  // [N][row bytes of shexp_codec] or null
+  const uint32_t* idx;     // [T][S - 1] with a shared expert, else [T][S]
+  const float* scores;     // [T][S]
+  const float* bias;       // [E][N] or null
+  void* out;               // [T][N]
+  int T, S, E, N, K, shexp_codec;
+  int64_t w_expert_stride;
+};
+
+// this lane's share of x . w over one weight row (no reduction across the wave)
+template <int C, int DT>
+__device__ __forceinline__ float mix_row_dot(const uint8_t* wr, const void* x, size_t xoff, int ngroups, int lane,
+                                             const uint8_t* grids) {
+  constexpr int WPB = kq_geom(C).wpb, BPB = kq_geom(C).bpb, GPB = WPB / 8;
+  float acc = 0.f;
+  for (int gi = lane; gi < ngroups; gi += 64) {
+    float wv[8], xv[8];
+    kq::decode8<C>(wr + (size_t)(gi / GPB) * BPB, gi % GPB, grids, wv);
+    load_x8<DT>(x, xoff + 8 * (size_t)gi, xv);
+    for (int t = 0; t < 8; t++) acc = fmaf(xv[t], wv[t], acc);
+  }
+  return acc;
+}
+
+// One workgroup (four waves) per (token t, output row n): wave w takes the slots w, w + 4, ...; a lane sums
+// score * (its share of the dot product) over the wave's slots, the wave reduces once, and the four wave sums are
+// added in wave order.
+template <int C, int DT>
+__global__ __launch_bounds__(GV_THREADS) void gather_mix_generic_kernel(MixArgs a, const uint8_t* __restrict__ grids) {
+  __shared__ float part[GV_THREADS / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const size_t row_bytes = (size_t)(a.K / kq_geom(C).wpb) * kq_geom(C).bpb;
+  const int ngroups = a.K / 8;
+  const int routed = a.shexp_w ? a.S - 1 : a.S;
+  for (int64_t item = blockIdx.x; item < (int64_t)a.T * a.N; item += gridDim.x) {
+    const int t = (int)(item / a.N), n = (int)(item % a.N);
+    float tot = 0.f, btot = 0.f;
+    for (int sl = wave; sl < a.S; sl += GV_THREADS / 64) {  // wave-uniform control flow
+      const size_t xoff = ((size_t)t * a.S + sl) * a.K;
+      const float score = a.scores[(size_t)t * a.S + sl];
+      float v;
+      if (sl < routed) {
+        const uint32_t e = a.idx[(size_t)t * routed + sl];
+        if (e >= (uint32_t)a.E) continue;
+        v = mix_row_dot<C, DT>(a.w + (int64_t)e * a.w_expert_stride + (size_t)n * row_bytes, a.x, xoff, ngroups, lane, grids);
+        if (a.bias) btot = fmaf(score, a.bias[(size_t)e * a.N + n], btot);
+      } else if (a.shexp_codec == KQ_Q6_K) {
+        v = mix_row_dot<KQ_Q6_K, DT>(a.shexp_w + (size_t)n * (a.K / 256) * 210, a.x, xoff, ngroups, lane, grids);
+      } else if (a.shexp_codec == KQ_Q8_0) {
+        v = mix_row_dot<KQ_Q8_0, DT>(a.shexp_w + (size_t)n * (a.K / 32) * 34, a.x, xoff, ngroups, lane, grids);
+      } else {
+        v = mix_row_dot<C, DT>(a.shexp_w + (size_t)n * row_bytes, a.x, xoff, ngroups, lane, grids);
+      }
+      tot = fmaf(score, v, tot);
+    }
+    for (int off = 32; off > 0; off >>= 1) tot += __shfl_xor(tot, off);
+    if (lane == 0) part[wave] = tot + btot;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float r = part[0];
+      for (int w = 1; w < GV_THREADS / 64; w++) r += part[w];
+      uint16_t* o = static_cast<uint16_t*>(a.out) + (size_t)t * a.N + n;
+      *o = DT == KQ_F16 ? kq::f2f16(r) : kq::f2bf16(r);
+    }
+    __syncthreads();
+  }
+}
+
+template <int C>
+struct MixRun {
+  static int run(MixArgs a, int dt, const uint8_t* grids, hipStream_t s) {
+    const int64_t items = (int64_t)a.T * a.N;
+    if (items == 0) return KQ_OK;
+    int64_t nwg = items;
+    if (nwg > 65536) nwg = 65536;
+    if (dt == KQ_F16)
+      hipLaunchKernelGGL((gather_mix_generic_kernel<C, KQ_F16>), dim3((unsigned)nwg), dim3(GV_THREADS), 0, s, a, grids);
+    else
+      hipLaunchKernelGGL((gather_mix_generic_kernel<C, KQ_BF16>), dim3((unsigned)nwg), dim3(GV_THREADS), 0, s, a, grids);
+    KQ_HIP_CHECK(hipGetLastError());
+    return KQ_OK;
+  }
+};
+
 template <template <int> class F, typename... A>
 int dispatch_codec(int codec, A... a) {
   switch (codec) {
@@ -377,4 +468,16 @@ int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2,
   GatherArgs a{x, w, w2, lhs, rhs, bias, bias2, out, B, M, N, K, x_div, x_batch_stride, w_expert_stride,
                act, limit, alpha, om, E};
   return dispatch_codec<GatherRun>(codec, a, dtype, glu != 0, grids, s);
+}
+
+// x [T][S][K], idx [T][S] (or [T][S - 1] with a shared expert, whose one-matrix stack shexp_w supplies the last
+// slot), scores [T][S], out [T][N].  shexp_codec: the expert codec, q6_k or q8_0.
+int kq_launch_gather_mix_generic(const void* x, const uint8_t* w, const uint8_t* shexp_w, const uint32_t* idx,
+                                 const float* scores, const float* bias, void* out, int T, int S, int E, int N, int K,
+                                 int64_t w_expert_stride, int codec, int shexp_codec, int dtype, hipStream_t s) {
+  const uint8_t* grids = kq_device_grids();
+  if (!grids) return KQ_ERR_HIP;
+  if (shexp_w && shexp_codec != codec && shexp_codec != KQ_Q6_K && shexp_codec != KQ_Q8_0) return KQ_ERR_UNSUPPORTED;
+  MixArgs a{x, w, shexp_w, idx, scores, bias, out, T, S, E, N, K, shexp_w ? shexp_codec : codec, w_expert_stride};
+  return dispatch_codec<MixRun>(codec, a, dtype, grids, s);
 }

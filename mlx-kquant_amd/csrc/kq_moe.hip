@@ -181,15 +181,21 @@ __global__ __launch_bounds__(256) void pad_idx_kernel(const uint32_t* __restrict
   idx2[i] = s < S - 1 ? idx[t * (S - 1) + s] : 0u;
 }
 
-// out[t][n] = T(sum_s scores[t][s] * yf[t][s][n]), f32, slots in order
+// out[t][n] = T(sum_s scores[t][s] * yf[t][s][n]), f32, slots in order.  idx [T][routed]: the expert ids of the
+// first `routed` slots; a slot whose id is >= E was skipped by the matmul kernels (its row of yf holds nothing)
+// and adds nothing.
 template <int DT>
 __global__ __launch_bounds__(256) void mix_slots_kernel(const float* __restrict__ yf, const float* __restrict__ scores,
+                                                        const uint32_t* __restrict__ idx, int routed, int E,
                                                         uint16_t* __restrict__ out, int T, int S, int N) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= (int64_t)T * N) return;
   const int t = (int)(i / N), n = (int)(i - (int64_t)t * N);
   float v = 0.f;
-  for (int s = 0; s < S; s++) v = fmaf(scores[t * S + s], yf[((size_t)t * S + s) * N + n], v);
+  for (int s = 0; s < S; s++) {
+    if (s < routed && idx[(size_t)t * routed + s] >= (uint32_t)E) continue;
+    v = fmaf(scores[t * S + s], yf[((size_t)t * S + s) * N + n], v);
+  }
   out[i] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
 }
 
@@ -641,13 +647,16 @@ int kq_launch_pad_idx(const uint32_t* idx, uint32_t* idx2, int T, int S, hipStre
   return KQ_OK;
 }
 
-int kq_launch_mix_slots(const float* yf, const float* scores, void* out, int T, int S, int N, int dtype, hipStream_t s) {
+int kq_launch_mix_slots(const float* yf, const float* scores, const uint32_t* idx, int routed, int E, void* out, int T,
+                        int S, int N, int dtype, hipStream_t s) {
   if (T <= 0 || N <= 0) return KQ_OK;
   const unsigned blocks = (unsigned)(((int64_t)T * N + 255) / 256);
   if (dtype == KQ_F16)
-    hipLaunchKernelGGL(mix_slots_kernel<KQ_F16>, dim3(blocks), dim3(256), 0, s, yf, scores, static_cast<uint16_t*>(out), T, S, N);
+    hipLaunchKernelGGL(mix_slots_kernel<KQ_F16>, dim3(blocks), dim3(256), 0, s, yf, scores, idx, routed, E,
+                       static_cast<uint16_t*>(out), T, S, N);
   else
-    hipLaunchKernelGGL(mix_slots_kernel<KQ_BF16>, dim3(blocks), dim3(256), 0, s, yf, scores, static_cast<uint16_t*>(out), T, S, N);
+    hipLaunchKernelGGL(mix_slots_kernel<KQ_BF16>, dim3(blocks), dim3(256), 0, s, yf, scores, idx, routed, E,
+                       static_cast<uint16_t*>(out), T, S, N);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }
