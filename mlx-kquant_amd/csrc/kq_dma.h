@@ -29,6 +29,12 @@ __device__ __forceinline__ u32x4 gload16(const void* p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
   return v;
 }
+typedef uint32_t u32x2_dma __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32x2_dma gload8(const void* p) {
+  u32x2_dma v;
+  asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
 template <int N>
 __device__ __forceinline__ void vmwait() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");

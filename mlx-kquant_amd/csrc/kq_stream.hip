@@ -1,4 +1,4 @@
-// Streamed skinny-M (decode) kernel: y[M,N] = x[M,K] . W^T for M <= 8, codecs q2_k ... q6_k, iq4_xs, iq2_xxs.
+// Streamed skinny-M (decode) kernel: y[M,N] = x[M,K] . W^T for M <= 8, codecs q2_k ... q6_k, iq4_xs, iq3_s, iq2_xxs.
 // The weight bytes go HBM -> LDS with direct-to-LDS loads (global_load_lds_dwordx4): no staging
 // registers, no LDS store instructions, and a wave keeps its next units in flight while it works.
 //
@@ -21,7 +21,10 @@
 // with one AND-OR (0x6400 | field = 1024 + field, fields masked in place); scales, the 1024 offset and
 // the block minimum are applied in f32 to the per-lane partial sums.  The codebook codecs read their values as
 // ready f16 from tables the workgroup builds in LDS (iq4_xs: byte -> two values; iq2_xxs: grid index -> eight
-// magnitudes, sign index -> eight sign masks).
+// magnitudes, sign index -> eight sign masks; iq3_s: 9-bit grid index -> four magnitudes, sign byte -> eight sign
+// masks).  These kernels are bound by the LDS once the table reads of a wave meet in a bank, so the one-row
+// kernels spend their spare LDS on that: a copy of the table per bank group (iq4_xs, iq2_xxs) or entries with the
+// signs already applied (iq3_s).
 //
 // Waiting.  The compiler cannot see a direct-to-LDS load land, so these loads are issued from inline
 // assembly and every wait on them is an explicit s_waitcnt vmcnt(n): loads return in order, n is the
@@ -67,6 +70,7 @@ __device__ __forceinline__ uint32_t opaque_sgpr(uint32_t v) {
   return v;
 }
 __device__ __forceinline__ void tie_v(u32x4& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void tie_v2(u32x2& v) { asm volatile("" : "+v"(v)); }
 
 __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -143,6 +147,17 @@ struct StGeom<KQ_IQ2_XXS> {
   static constexpr int BPB = 66, PP = 5, LBPB = 80, NAP = 4, XSG = 8;
   static constexpr bool SIDE_D = false;
 };
+//   iq3_s  (110): pieces at 2, 18, .., 82 and 94; d travels as a 2-byte load per row.  LDS row: qs[64] at 0,
+//                 qh[8] at 64, sign words 0..5 at 72 + 4 k, block bytes 94 .. 109 at 96 (sign words 6, 7 at 100,
+//                 104; scales[4] at 108)
+template <>
+struct StGeom<KQ_IQ3_S> {
+  static constexpr int BPB = 110, PP = 7, LBPB = 112, NAP = 4, XSG = 8;
+  static constexpr bool SIDE_D = true;
+};
+// block byte of the f16 d that travels on its own (SIDE_D)
+template <int C>
+constexpr uint32_t st_side_d_off() { return C == KQ_Q6_K ? 208u : 0u; }
 // byte offset of piece p inside a block
 template <int C>
 __device__ __forceinline__ uint32_t st_piece_off(int p) {
@@ -150,21 +165,34 @@ __device__ __forceinline__ uint32_t st_piece_off(int p) {
   if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) return p == G::PP - 1 ? (uint32_t)(G::BPB - 16) : 16u * (uint32_t)p;
   if constexpr (C == KQ_IQ4_XS) return p == 0 ? 0u : 16u * (uint32_t)p - 8u;
   if constexpr (C == KQ_IQ2_XXS) return p == 0 ? 0u : 16u * (uint32_t)p - 14u;
+  if constexpr (C == KQ_IQ3_S) return p == 6 ? 94u : 16u * (uint32_t)p + 2u;
   return 16u * (uint32_t)p;
 }
 // Order of the staged f16 activations inside a group: 0 = k0 k2 k1 k3 per four (the order the masked-in-place codes
 // leave a 32-bit word in), 1 = k0 k1 k2 k3 (codebook entries), 2 = x[j], x[j + 16] interleaved over 32 (iq4_xs: a
 // byte holds weights j and j + 16 of its sub-block).
 template <int C>
-constexpr int st_xord() { return C == KQ_IQ4_XS ? 2 : C == KQ_IQ2_XXS ? 1 : 0; }
+constexpr int st_xord() { return C == KQ_IQ4_XS ? 2 : C == KQ_IQ2_XXS || C == KQ_IQ3_S ? 1 : 0; }
 // LDS bytes of the decode tables a workgroup builds for itself
 //   iq4_xs:  [256][32] byte -> f16 pair (kvalues[low nibble], kvalues[high nibble]), one copy per LDS bank: lane l
 //            reads copy l % 32, so the 64 data-dependent reads of an instruction never meet in a bank (with a single
 //            copy the bank conflicts took about half of the kernel's time)
 //   iq2_xxs: [256] grid entry as eight f16 | [128] sign index -> eight f16 sign masks
-template <int C>
+//   iq3_s:   [512] grid entry as four f16 | [256] sign byte -> eight f16 sign masks; the one-row eight-wave kernel
+//            has the LDS for [16 sign nibbles][512] entries with the signs applied (64 KiB, in front of the plain
+//            entries it is built from): one table read per four weights and no XOR.  With the two-table form the
+//            kernel is bound by the LDS (88 % busy, 63 % of that bank conflicts of the data-dependent reads).
+template <int C, int MB = 0, int NW = 0>
+constexpr bool st_iq3s_merged() { return C == KQ_IQ3_S && MB == 1 && NW == 8; }
+// iq2_xxs, one-row eight-wave kernel: 16 copies of both tables, entry e copy c at 256 e + 16 c, lane l reads copy
+// l % 16, so the sixteen lanes of a 16-byte read never meet in a bank (with single copies the kernel is bound by the
+// LDS: 90 % busy, 60 % of that bank conflicts).
+template <int C, int MB = 0, int NW = 0>
+constexpr int st_iq2_copies() { return C == KQ_IQ2_XXS && MB == 1 && NW == 8 ? 16 : 1; }
+template <int C, int MB = 0, int NW = 0>
 constexpr int st_tbl_bytes() {
-  return C == KQ_IQ4_XS ? 32768 : C == KQ_IQ2_XXS ? 4096 + 2048 : 0;
+  return C == KQ_IQ4_XS ? 32768 : C == KQ_IQ2_XXS ? (4096 + 2048) * st_iq2_copies<C, MB, NW>() :
+         st_iq3s_merged<C, MB, NW>() ? 65536 + 4096 : C == KQ_IQ3_S ? 4096 + 4096 : 0;
 }
 template <int C>
 struct StUnit {
@@ -449,13 +477,14 @@ __device__ __forceinline__ void iq4xs_unit(const uint8_t* __restrict__ bl, int k
 // Lane (row, kg) owns the 8-byte groups 4 kg .. 4 kg + 3 (32 weights each): four grid index bytes, then a word of
 // four 7-bit sign indices and the 4-bit scale.  Index -> eight f16 magnitudes, sign index -> eight f16 sign
 // masks (16-byte table reads), XOR.  MFMAs (ib, l, half): A pair ib, block 2 l + half.
-template <int R, int AS>
+// COP copies of every table entry, 16 bytes apart (tbl already points at the lane's copy).
+template <int R, int AS, int COP>
 __device__ __forceinline__ void iq2xxs_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
                                             const uint8_t* __restrict__ tbl, float* acc) {
   constexpr int RG = (R + 3) / 4;
   const float d = kq::h2f(*reinterpret_cast<const uint16_t*>(bl)) * xscale * 0.25f;
   const u32x4 q0 = *reinterpret_cast<const u32x4*>(bl + 16 + 32 * kg), q1 = *reinterpret_cast<const u32x4*>(bl + 32 + 32 * kg);
-  const uint8_t* stbl = tbl + 4096;
+  const uint8_t* stbl = tbl + 4096 * COP;
   // The table reads of group ib + 1 are issued before the MFMAs of group ib (see iq4xs_unit).
   u32x4 gv[4][4], sm[4][4];
   uint32_t a1s[4];
@@ -466,8 +495,8 @@ __device__ __forceinline__ void iq2xxs_unit(const uint8_t* __restrict__ bl, int 
     SFor<4>::run([&](auto ll) {
       constexpr int l = decltype(ll)::value;
       const uint32_t idx = (gi >> (8 * l)) & 0xff, si = (a1 >> (7 * l)) & 127;
-      gv[ib][l] = *reinterpret_cast<const u32x4*>(tbl + 16 * idx);
-      sm[ib][l] = *reinterpret_cast<const u32x4*>(stbl + 16 * si);
+      gv[ib][l] = *reinterpret_cast<const u32x4*>(tbl + 16 * COP * idx);
+      sm[ib][l] = *reinterpret_cast<const u32x4*>(stbl + 16 * COP * si);
     });
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -490,6 +519,73 @@ __device__ __forceinline__ void iq2xxs_unit(const uint8_t* __restrict__ bl, int 
       }
     });
     const float dl = d * (0.5f + (float)(a1s[ib] >> 28));
+    SFor<R>::run([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      acc[r] = fmaf(dl, p[r / 4][r % 4], acc[r]);
+    });
+  });
+}
+
+// ------------------------------------------------------------------ iq3_s unit
+// Lane (row, kg) owns the 32-weight blocks 4 kg .. 4 kg + 3: eight index bytes each (the ninth index bit is bit j
+// of the block's qh byte), four sign bytes (one per eight weights) and a 4-bit scale.  Index -> four f16
+// magnitudes (8-byte table read), sign byte -> eight f16 sign masks (16-byte read), XOR.  MFMAs (ib, l, half):
+// index 2 l + half of the block; A pair ib, block 2 l + half.
+// MERGED: tbl holds [16][512] entries with the signs of a nibble applied; index | nibble << 9.
+template <int R, int AS, bool MERGED>
+__device__ __forceinline__ void iq3s_unit(const uint8_t* __restrict__ bl, int kg, float dx, const u32x2* areg,
+                                          const uint8_t* __restrict__ tbl, float* acc) {
+  constexpr int RG = (R + 3) / 4;
+  const u32x4 qa = *reinterpret_cast<const u32x4*>(bl + 32 * kg), qb = *reinterpret_cast<const u32x4*>(bl + 32 * kg + 16);
+  const uint32_t qh = *reinterpret_cast<const uint32_t*>(bl + 64 + 4 * kg);
+  const uint32_t scw = *reinterpret_cast<const uint32_t*>(bl + 108) >> (16 * kg);
+  const uint8_t* sgp = bl + 72 + 16 * kg;
+  const uint8_t* stbl = tbl + 4096;
+  u32x2 gv[4][8];
+  u32x4 sm[4][4];
+  auto lookup = [&](auto ii) {
+    constexpr int ib = decltype(ii)::value;
+    const uint32_t w0 = ib < 2 ? qa[2 * ib] : qb[2 * (ib - 2)], w1 = ib < 2 ? qa[2 * ib + 1] : qb[2 * (ib - 2) + 1];
+    const uint32_t hb = qh >> (8 * ib);
+    // sign words 6 and 7 of the block sit four bytes further (behind the two bytes the last piece repeats)
+    const uint32_t sw = *reinterpret_cast<const uint32_t*>(sgp + 4 * ib + (ib >= 2 ? 4 * kg : 0));
+    SFor<8>::run([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      const uint32_t w = j < 4 ? w0 : w1;
+      uint32_t idx = ((w >> (8 * (j & 3))) & 0xff) | (((hb >> j) & 1) << 8);
+      if constexpr (MERGED) idx |= ((sw >> (4 * j)) & 15) << 9;
+      gv[ib][j] = *reinterpret_cast<const u32x2*>(tbl + 8 * idx);
+    });
+    if constexpr (!MERGED) {
+      SFor<4>::run([&](auto ll) {
+        constexpr int l = decltype(ll)::value;
+        sm[ib][l] = *reinterpret_cast<const u32x4*>(stbl + 16 * ((sw >> (8 * l)) & 0xff));
+      });
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  lookup(std::integral_constant<int, 0>{});
+  SFor<4>::run([&](auto ii) {
+    constexpr int ib = decltype(ii)::value;
+    if constexpr (ib < 3) lookup(std::integral_constant<int, ib + 1>{});
+    f32x4 p[RG];
+#pragma unroll
+    for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
+    SFor<4>::run([&](auto ll) {
+      constexpr int l = decltype(ll)::value;
+      u32x2 lo = gv[ib][2 * l], hi = gv[ib][2 * l + 1];
+      if constexpr (!MERGED) {
+        lo = u32x2{lo[0] ^ sm[ib][l][0], lo[1] ^ sm[ib][l][1]};
+        hi = u32x2{hi[0] ^ sm[ib][l][2], hi[1] ^ sm[ib][l][3]};
+      }
+#pragma unroll
+      for (int g = 0; g < RG; g++) {
+        const f16x4 av = __builtin_bit_cast(f16x4, areg[g * AS + ib]);
+        p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, lo), p[g], 3, 2 * l, 0);
+        p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, __builtin_bit_cast(f16x4, hi), p[g], 3, 2 * l + 1, 0);
+      }
+    });
+    const float dl = dx * (float)(1 + 2 * (int)((scw >> (4 * ib)) & 15));
     SFor<R>::run([&](auto rr) {
       constexpr int r = decltype(rr)::value;
       acc[r] = fmaf(dl, p[r / 4][r % 4], acc[r]);
@@ -627,7 +723,21 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   const uint16_t* x16 = static_cast<const uint16_t*>(a.x);
   // codebook codecs: threads 0 .. 127 fetch 16 bytes each of the 2 KiB grid the tables are built from
   u32x4 greg = {0, 0, 0, 0};
-  if constexpr (C == KQ_IQ2_XXS) greg = gload16(a.grids + KQ_GRID_IQ2XXS + 16 * (tid & 127));
+  // replicated iq2_xxs tables: the sixteen lanes of a quarter wave write the sixteen copies of one entry (a wave
+  // store covers 1 KiB of consecutive LDS); wave w converts the grid entries 32 i + 4 w + lane / 16, i = 0 .. 7
+  constexpr int IQ2_COP = st_iq2_copies<C, MB, NW>();
+  u32x2 gq[IQ2_COP > 1 ? 8 : 1];
+  if constexpr (C == KQ_IQ2_XXS) {
+    if constexpr (IQ2_COP == 1) {
+      greg = gload16(a.grids + KQ_GRID_IQ2XXS + 16 * (tid & 127));
+    } else {
+      SFor<8>::run([&](auto ii) {
+        constexpr int i = decltype(ii)::value;
+        gq[i] = gload8(a.grids + KQ_GRID_IQ2XXS + 8 * (32 * i + 4 * wave + (lane >> 4)));
+      });
+    }
+  }
+  if constexpr (C == KQ_IQ3_S) greg = gload16(a.grids + KQ_GRID_IQ3S + 16 * (tid & 127));  // four entries
   u32x4 xreg[MB * XL];
   SFor<MB * XL>::run([&](auto t) {
     constexpr int T = decltype(t)::value;
@@ -672,7 +782,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
     if constexpr (G::SIDE_D) {
       int r = row0 + (lane < rpt ? lane : rpt - 1);
       r = r < row_lim ? r : row_lim;
-      if (lane < 32) dma2(base + 208, (uint32_t)(r - row0) * row_bytes, l0 + ST_ROWS * G::LBPB);
+      if (lane < 32) dma2(base + st_side_d_off<C>(), (uint32_t)(r - row0) * row_bytes, l0 + ST_ROWS * G::LBPB);
     }
     inflight++;
     islot = islot + 1 == D ? 0 : islot + 1;
@@ -696,6 +806,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   ST_TS(1);
   SFor<MB * XL>::run([&](auto t) { tie_v(xreg[decltype(t)::value]); });
   tie_v(greg);
+  if constexpr (IQ2_COP > 1) SFor<8>::run([&](auto ii) { tie_v2(gq[decltype(ii)::value]); });
 
   // ---- activations -> f16 fragments (+ sums) in the wave's LDS, then this lane's A registers
   float xscale = 1.0f, inv = 1.0f;
@@ -821,7 +932,31 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 #pragma unroll
     for (int c = 0; c < 8 / TPE; c++) *reinterpret_cast<u32x4*>(tbl + 128 * b + (128 / TPE) * part + 16 * c) = e4;
   }
-  if constexpr (C == KQ_IQ2_XXS) {
+  if constexpr (C == KQ_IQ2_XXS && st_iq2_copies<C, MB, NW>() > 1) {
+    constexpr int COP = st_iq2_copies<C, MB, NW>();
+    static_assert(COP == 1 || (COP == 16 && NW == 8), "eight waves write 16 copies");
+    typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
+    uint8_t* dst = tbl + 256 * (4 * wave + (lane >> 4)) + 16 * (lane & 15);
+    SFor<8>::run([&](auto ii) {  // grid entries: eight bytes -> eight f16
+      constexpr int i = decltype(ii)::value;
+      u32x4 o;
+#pragma unroll
+      for (int k = 0; k < 8; k += 2) {
+        const uint32_t gw = gq[i][k >> 2];
+        const f16x2v e = {(_Float16)(float)((gw >> (8 * (k & 3))) & 0xff), (_Float16)(float)((gw >> (8 * ((k + 1) & 3))) & 0xff)};
+        o[k >> 1] = __builtin_bit_cast(uint32_t, e);
+      }
+      *reinterpret_cast<u32x4*>(dst + 256 * 32 * i) = o;
+    });
+    SFor<4>::run([&](auto ii) {  // sign indices 32 i + 4 w + lane / 16 -> eight f16 sign masks
+      constexpr int i = decltype(ii)::value;
+      const uint32_t sb = kq::ksigns((uint32_t)(32 * i + 4 * wave + (lane >> 4)));
+      u32x4 o;
+#pragma unroll
+      for (int w = 0; w < 4; w++) o[w] = (((sb >> (2 * w)) & 1) << 15) | (((sb >> (2 * w + 1)) & 1) << 31);
+      *reinterpret_cast<u32x4*>(dst + 4096 * COP + 256 * 32 * i) = o;
+    });
+  } else if constexpr (C == KQ_IQ2_XXS) {
     if (tid < 128) {  // 16 grid bytes -> 16 f16 magnitudes
       u32x4 o[2];
 #pragma unroll
@@ -839,6 +974,39 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
       u32x4 o;
 #pragma unroll
       for (int w = 0; w < 4; w++) o[w] = (((sb >> (2 * w)) & 1) << 15) | (((sb >> (2 * w + 1)) & 1) << 31);
+      *reinterpret_cast<u32x4*>(tbl + 4096 + 16 * tid) = o;
+    }
+  }
+  if constexpr (C == KQ_IQ3_S) {
+    constexpr bool MERGED = st_iq3s_merged<C, MB, NW>();
+    uint8_t* plain = MERGED ? tbl + 65536 : tbl;
+    if (tid < 128) {  // four grid entries of four bytes -> four times four f16 magnitudes
+      typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
+      u32x4 o[2];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const uint32_t gw = greg[e];
+        const f16x2v e0 = {(_Float16)(float)(gw & 0xff), (_Float16)(float)((gw >> 8) & 0xff)};
+        const f16x2v e1 = {(_Float16)(float)((gw >> 16) & 0xff), (_Float16)(float)(gw >> 24)};
+        o[e >> 1][2 * (e & 1)] = __builtin_bit_cast(uint32_t, e0);
+        o[e >> 1][2 * (e & 1) + 1] = __builtin_bit_cast(uint32_t, e1);
+      }
+      *reinterpret_cast<u32x4*>(plain + 32 * tid) = o[0];
+      *reinterpret_cast<u32x4*>(plain + 32 * tid + 16) = o[1];
+    }
+    if constexpr (MERGED) {
+      static_assert(!MERGED || 64 * NW == 512, "one thread per grid entry");
+      wg_lds_barrier();
+      const u32x2 e = *reinterpret_cast<const u32x2*>(plain + 8 * tid);
+      SFor<16>::run([&](auto nn) {
+        constexpr uint32_t nib = decltype(nn)::value;
+        constexpr uint32_t m0 = ((nib & 1) << 15) | ((nib & 2) << 30), m1 = ((nib & 4) << 13) | ((nib & 8) << 28);
+        *reinterpret_cast<u32x2*>(tbl + 8 * (tid | (nib << 9))) = u32x2{e[0] ^ m0, e[1] ^ m1};
+      });
+    } else if (tid < 256) {  // sign byte -> eight f16 sign masks
+      u32x4 o;
+#pragma unroll
+      for (int w = 0; w < 4; w++) o[w] = ((((uint32_t)tid >> (2 * w)) & 1) << 15) | ((((uint32_t)tid >> (2 * w + 1)) & 1) << 31);
       *reinterpret_cast<u32x4*>(tbl + 4096 + 16 * tid) = o;
     }
   }
@@ -877,7 +1045,11 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         } else if constexpr (C == KQ_IQ4_XS) {
           iq4xs_unit<R, AS>(bl, kg, xscale, areg + u * NAP, tbl + 4 * (lane & 31), acc);
         } else if constexpr (C == KQ_IQ2_XXS) {
-          iq2xxs_unit<R, AS>(bl, kg, xscale, areg + u * NAP, tbl, acc);
+          constexpr int COP = st_iq2_copies<C, MB, NW>();
+          iq2xxs_unit<R, AS, COP>(bl, kg, xscale, areg + u * NAP, COP > 1 ? tbl + 16 * (lane & 15) : tbl, acc);
+        } else if constexpr (C == KQ_IQ3_S) {
+          const float dx = kq::h2f((uint16_t)*reinterpret_cast<const uint32_t*>(slot + ST_ROWS * G::LBPB + 4 * crow)) * xscale;
+          iq3s_unit<R, AS, st_iq3s_merged<C, MB, NW>()>(bl, kg, dx, areg + u * NAP, tbl, acc);
         } else {
           q45k_unit<C, R, AS>(bl, kg, xscale, areg + u * NAP, xsum + u * 8, ST_XU * 8, acc);
         }
@@ -924,7 +1096,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 template <int C, int MB, int D, int ST_XU, int ST_WAVES>
 constexpr size_t st_lds_bytes() {
   return (size_t)ST_WAVES * (D * StUnit<C>::SLOT + st_xch<MB>() * ST_XU * 512 + MB * ST_XU * 2 * StGeom<C>::XSG * 4) +
-         2 * ST_WAVES * MB * 64 * 4 + st_tbl_bytes<C>();
+         2 * ST_WAVES * MB * 64 * 4 + st_tbl_bytes<C, MB, ST_WAVES>();
 }
 
 template <int DT>
@@ -975,6 +1147,7 @@ int st_max_sb(int codec, int M) {
     case KQ_Q6_K: rows = st_nw8_rows<KQ_Q6_K>(); break;
     case KQ_IQ4_XS: rows = st_nw8_rows<KQ_IQ4_XS>(); break;
     case KQ_IQ2_XXS: rows = st_nw8_rows<KQ_IQ2_XXS>(); break;
+    case KQ_IQ3_S: rows = st_nw8_rows<KQ_IQ3_S>(); break;
   }
   return M <= rows ? 32 : 16;
 }
@@ -1049,7 +1222,7 @@ int st_launch_m(const StArgs& a, int splits, hipStream_t s) {
 
 bool st_codec_ok(int codec) {
   return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K || codec == KQ_Q2_K || codec == KQ_Q3_K ||
-         codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS;
+         codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S;
 }
 
 }  // namespace
@@ -1091,9 +1264,11 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
     return dtype == KQ_F16 ? st_launch_m<KQ_Q4_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q4_K, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q5_K)
     return dtype == KQ_F16 ? st_launch_m<KQ_Q5_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q5_K, KQ_BF16>(a, p.ksplit, s);
-  if (codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS) {
+  if (codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S) {
     a.grids = kq_device_grids();
     if (!a.grids) return KQ_ERR_HIP;
+    if (codec == KQ_IQ3_S)
+      return dtype == KQ_F16 ? st_launch_m<KQ_IQ3_S, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_IQ3_S, KQ_BF16>(a, p.ksplit, s);
     if (codec == KQ_IQ4_XS)
       return dtype == KQ_F16 ? st_launch_m<KQ_IQ4_XS, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_IQ4_XS, KQ_BF16>(a, p.ksplit, s);
     return dtype == KQ_F16 ? st_launch_m<KQ_IQ2_XXS, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_IQ2_XXS, KQ_BF16>(a, p.ksplit, s);
