@@ -921,16 +921,17 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 
   // ---- decode tables of the codebook codecs (their grid bytes arrived with the activations)
   if constexpr (C == KQ_IQ4_XS) {
-    // entry b = dwords 32 b .. 32 b + 31 (one copy per LDS bank); a thread computes one entry and writes its
-    // share of the copies with 16-byte stores
+    // entry b = dwords 32 b .. 32 b + 31 (one copy per LDS bank).  Eight lanes write the 128 bytes of an entry, so
+    // a wave store covers 1 KiB of consecutive LDS (entry-per-lane stores, 128 bytes apart, all meet in two banks)
     typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
-    constexpr int TPE = 64 * ST_WAVES / 256;  // threads per entry (1 or 2)
-    const int b = tid & 255, part = tid >> 8;
-    const f16x2v e = {(_Float16)kq::kv_iq4nl(b & 15), (_Float16)kq::kv_iq4nl(b >> 4)};
-    const uint32_t ev = __builtin_bit_cast(uint32_t, e);
-    const u32x4 e4 = {ev, ev, ev, ev};
+    constexpr int PER_WAVE = 256 / 8 / ST_WAVES;  // store instructions per wave: 8 entries each
 #pragma unroll
-    for (int c = 0; c < 8 / TPE; c++) *reinterpret_cast<u32x4*>(tbl + 128 * b + (128 / TPE) * part + 16 * c) = e4;
+    for (int i = 0; i < PER_WAVE; i++) {
+      const int b = 8 * (PER_WAVE * wave + i) + (lane >> 3);
+      const f16x2v e = {(_Float16)kq::kv_iq4nl(b & 15), (_Float16)kq::kv_iq4nl(b >> 4)};
+      const uint32_t ev = __builtin_bit_cast(uint32_t, e);
+      *reinterpret_cast<u32x4*>(tbl + 128 * b + 16 * (lane & 7)) = u32x4{ev, ev, ev, ev};
+    }
   }
   if constexpr (C == KQ_IQ2_XXS && st_iq2_copies<C, MB, NW>() > 1) {
     constexpr int COP = st_iq2_copies<C, MB, NW>();
