@@ -59,7 +59,12 @@ struct CodeGeom {
   // table in LDS maps a byte to the f16 pair of its two values, and the activations of a block are staged as
   // x[j], x[j + 16] interleaved, so four table reads are the B operand of an MFMA with no further arithmetic
   static constexpr bool PAIR_LUT = C == KQ_IQ4_NL || C == KQ_MXFP4;
+  // pair table: 256 entries of 4 bytes.  The grouped kernel keeps one copy per LDS bank (entry b copy c at
+  // 128 b + 4 c, lane l reads copy l % 32: the 64 data-dependent reads of an instruction never meet in a bank),
+  // + 1 KiB for the plain table the copies are made from; the per-entry kernel, whose launches are too short to
+  // earn the 32 KiB build back, keeps the plain table.
   static constexpr int GRID_BYTES = PAIR_LUT ? 1024 : GRID_N * GRID_W * 2;
+  static constexpr int GROUPED_GRID_BYTES = PAIR_LUT ? 32768 + 1024 : GRID_BYTES;
   // 256-entry table spreading 8 bits over the 8 halves of a B operand: sign bits (bit 15) for the
   // signed codebooks, the fifth code bit (bit 4) for q5_0 / q5_1
   static constexpr bool SIGNS = C == KQ_IQ2_XXS || C == KQ_IQ2_XS || C == KQ_IQ2_S || C == KQ_IQ3_XXS || C == KQ_IQ3_S;
@@ -180,6 +185,7 @@ __device__ __forceinline__ uint32_t pick(int kg, uint32_t a, uint32_t b) { retur
 struct Tables {
   const uint8_t* grid;    // f16 codebook (LDS)
   const uint8_t* spread;  // 256 x 16-byte bit-spread table (LDS)
+  int pair_shift;         // log2 of the byte distance between pair-table entries (2, or 7 with a copy per bank)
 };
 
 // The B operand of MFMA J (weights 16 J + 8 kg .. + 7 of the step) of the row whose step bytes are in
@@ -202,7 +208,8 @@ __device__ __forceinline__ f16x8 codes(const R& row, int kg, const Tables& t) {
       const uint32_t w = pick(kg, row.template u32<off + 8 * (J & 1)>(), row.template u32<off + 8 * (J & 1) + 4>());
       u32x4 r;
 #pragma unroll
-      for (int e = 0; e < 4; e++) r[e] = *reinterpret_cast<const uint32_t*>(t.grid + 4 * ((w >> (8 * e)) & 0xffu));
+      for (int e = 0; e < 4; e++)
+        r[e] = *reinterpret_cast<const uint32_t*>(t.grid + (((w >> (8 * e)) & 0xffu) << t.pair_shift));
       return __builtin_bit_cast(f16x8, r);
     }
     uint32_t lo = pick(kg, row.template u32<off>(), row.template u32<off + 8>());
@@ -496,7 +503,7 @@ __global__ __launch_bounds__((64 * WV), (WV == 4 ? 2 : 1)) void codes_skinny_ker
     }
   }
   if constexpr (G::GRID_N > 0 || G::SPREAD_BYTES > 0 || G::PAIR_LUT) lds_barrier();
-  const Tables tabs{grid_lds, spread_lds};
+  const Tables tabs{grid_lds, spread_lds, 2};
 
   // ---- piece maps of this wave.  Wire: piece i = lane + 64 t -> (row i / PIECES, piece i % PIECES).
   // Activations: lane -> (row lane / 32 + 2 t, 16-byte piece lane % 32).
@@ -835,7 +842,7 @@ constexpr int CG_BN = 128;
 
 template <int C>
 constexpr int grouped_lds_bytes() {
-  return 32 * XA_STRIDE + 32 * 4 + 8 * 32 * 4 + CG_BN * CodeGeom<C>::LROW + 32 * 4 + CodeGeom<C>::GRID_BYTES +
+  return 32 * XA_STRIDE + 32 * 4 + 8 * 32 * 4 + CG_BN * CodeGeom<C>::LROW + 32 * 4 + CodeGeom<C>::GROUPED_GRID_BYTES +
          CodeGeom<C>::SPREAD_BYTES;
 }
 
@@ -851,7 +858,7 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
   uint8_t* b_lds = reinterpret_cast<uint8_t*>(xsum_lds + 8 * 32);         // [128][LROW]
   int* pair_lds = reinterpret_cast<int*>(b_lds + CG_BN * G::LROW);        // [32] output row per slot, -1 = none
   uint8_t* grid_lds = reinterpret_cast<uint8_t*>(pair_lds + 32);
-  uint8_t* spread_lds = grid_lds + G::GRID_BYTES;
+  uint8_t* spread_lds = grid_lds + G::GROUPED_GRID_BYTES;
 
   if ((int)blockIdx.y >= *a.nseg) return;  // uniform: the grid is sized for the worst case
   const Segment seg = a.segs[blockIdx.y];
@@ -904,10 +911,18 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
     }
   }
   if constexpr (G::PAIR_LUT) {
+    // one entry per thread into a plain table, then eight lanes write the 128 bytes of an entry's copies: a wave
+    // store covers consecutive LDS
+    uint32_t* plain = reinterpret_cast<uint32_t*>(grid_lds + 32768);
     if (tid < 256) {
       const f16x2 e = C == KQ_MXFP4 ? f16x2{(_Float16)kq::kv_mxfp4(tid & 15), (_Float16)kq::kv_mxfp4(tid >> 4)}
                                     : f16x2{(_Float16)kq::kv_iq4nl(tid & 15), (_Float16)kq::kv_iq4nl(tid >> 4)};
-      reinterpret_cast<uint32_t*>(grid_lds)[tid] = __builtin_bit_cast(uint32_t, e);
+      plain[tid] = __builtin_bit_cast(uint32_t, e);
+    }
+    lds_barrier();
+    for (int i = tid; i < 256 * 8; i += CG_THREADS) {
+      const uint32_t ev = plain[i >> 3];
+      *reinterpret_cast<u32x4*>(grid_lds + 16 * i) = u32x4{ev, ev, ev, ev};
     }
   }
   if constexpr (G::SPREAD_BYTES > 0) {
@@ -918,7 +933,7 @@ __global__ __launch_bounds__(CG_THREADS, 2) void codes_grouped_kernel(CgArgs a) 
         u32x4{(bit(0) << P) | (bit(2) << (P + 16)), (bit(1) << P) | (bit(3) << (P + 16)),
               (bit(4) << P) | (bit(6) << (P + 16)), (bit(5) << P) | (bit(7) << (P + 16))};
   }
-  const Tables tabs{grid_lds, spread_lds};
+  const Tables tabs{G::PAIR_LUT ? grid_lds + 4 * (tid & 31) : grid_lds, spread_lds, 7};
 
   // ---- piece maps.  Activations: piece i = tid + 256 t -> (slot i / 32, 16-byte piece i % 32).
   const int a_slot0 = tid >> 5, a_pc = tid & 31;
