@@ -1425,6 +1425,12 @@ int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, c
                            int dtype, int E, KqOutMap om, hipStream_t s) {
   if (!sk_shape_ok(M, K, codec, x, w, w2) || B < 1 || B > 65535) return KQ_ERR_UNSUPPORTED;
   if (glu && (M != 1 || act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
+  // one activation row per entry, entries in order of x (MoE decode): the streamed kernel
+  if (M == 1 && !lhs && rhs && x_batch_stride == K && g_sk_variant == 0) {
+    const int rcs = kq_launch_gather_stream(x, w, glu ? w2 : nullptr, rhs, out, B, N, K, x_div, w_expert_stride, act, limit,
+                                            codec, dtype, E, om, s);
+    if (rcs != KQ_ERR_UNSUPPORTED) return rcs;
+  }
   const int64_t wmask = (int64_t)sk_wire_align_mask(codec);
   if ((w_expert_stride & wmask) || ((x_batch_stride * 2) & 15)) return KQ_ERR_UNSUPPORTED;
   SkArgs a{};

@@ -33,6 +33,7 @@
 #include <type_traits>
 
 #include "kq_decode.h"
+#include "kq_epilogue.h"
 #include "kq_dma.h"
 
 namespace {
@@ -213,6 +214,15 @@ struct StArgs {
   int rpt;  // weight rows per tile (<= 32): fewer than 32 evens the rows out over one round of workgroups
   float* partial;  // split-K: [ksplit][M][N] f32
   int ksplit, sb_per_split;
+  // gathered calls (one activation row per entry, MoE decode): entry p = blockIdx.x / tiles_per_entry multiplies row
+  // p / x_div of x by rows of expert rhs[p] (w, and w2 = the up stack of the fused gate / up form) into output row
+  // out_row(om, p); entries whose expert id is >= E are skipped
+  const uint8_t* w2;
+  const uint32_t* rhs;
+  int tiles_per_entry, x_div, E, act;
+  float limit;
+  int64_t w_expert_stride;
+  KqOutMap om;
 #ifdef KQ_ST_TS
   uint64_t* ts;
 #endif
@@ -675,9 +685,14 @@ constexpr int st_xch() { return MB > 4 ? 2 : MB; }  // activation rows staged at
 // XU = units (superblocks) a wave handles per tile at most: 4 or 8, i.e. K ranges of up to 16 or 32 superblocks
 // per workgroup (the A registers of all of them stay resident).
 // NW = waves per workgroup (4 or 8): wave w owns superblocks sb_begin + w + NW u of the workgroup's K range.
-template <int C, int DT, int MB, int D, int WGS, int XU, int NW>
+// GM = 0: dense.  GM = 1: gathered, one tile of one entry per workgroup.  GM = 2: gathered gate / up pair: a
+// superblock is two units (the gate rows, then the same rows of the up matrix) with an accumulator each, and the
+// tile's result is act(gate) * up.
+template <int C, int DT, int MB, int D, int WGS, int XU, int NW, int GM = 0>
 __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
+  static_assert(GM == 0 || MB == 1, "gathered entries carry one activation row");
   constexpr int ST_XU = XU, ST_WAVES = NW;
+  constexpr int UPS = GM == 2 ? 2 : 1;  // units per superblock
   using G = StGeom<C>;
   using U = StUnit<C>;
   constexpr int R = MB;
@@ -697,9 +712,22 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, kg = lane >> 5;
-  const int M = a.M, N = a.N, K = a.K, nsb = K >> 8, tiles = a.tiles, rpt = a.rpt;
+  const int M = a.M, N = a.N, K = a.K, nsb = K >> 8, rpt = a.rpt;
   const uint32_t row_bytes = (uint32_t)nsb * G::BPB;
-  const int G_x = gridDim.x;
+  // gathered: this workgroup's entry and its tile inside the entry's matrix (the tile loop below runs once)
+  const int g_entry = GM ? __builtin_amdgcn_readfirstlane((int)blockIdx.x / a.tiles_per_entry) : 0;
+  const int g_tile = GM ? (int)blockIdx.x - g_entry * a.tiles_per_entry : 0;
+  const uint8_t* wmat = a.w;
+  const uint8_t* wmat2 = a.w;
+  if constexpr (GM != 0) {
+    const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.rhs[g_entry]);
+    if (e >= (uint32_t)a.E) return;  // the whole workgroup, ahead of every barrier
+    wmat = a.w + (int64_t)e * a.w_expert_stride;
+    if constexpr (GM == 2) wmat2 = a.w2 + (int64_t)e * a.w_expert_stride;
+  }
+  const int tiles = GM ? g_tile + 1 : a.tiles;
+  const int tile0 = GM ? g_tile : (int)blockIdx.x;
+  const int G_x = GM ? 1 << 30 : (int)gridDim.x;
 
   // LDS: per wave [D slots][x fragments MB x 4 x 256 f16][x sums MB x 4 x 2 XSG f32]; then red [2][waves][R][64] f32
   constexpr int XS_BYTES = XCH * ST_XU * 512, XSUM_BYTES = MB * ST_XU * 2 * XSG * 4;
@@ -708,7 +736,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   _Float16* xs = reinterpret_cast<_Float16*>(wb + D * U::SLOT);
   float* xsum = reinterpret_cast<float*>(wb + D * U::SLOT + XS_BYTES);
   float* red_all = reinterpret_cast<float*>(smem + ST_WAVES * WAVE_BYTES);
-  uint8_t* tbl = smem + ST_WAVES * WAVE_BYTES + 2 * ST_WAVES * R * 64 * 4;  // decode tables (codebook codecs)
+  uint8_t* tbl = smem + ST_WAVES * WAVE_BYTES + UPS * 2 * ST_WAVES * R * 64 * 4;  // decode tables (codebook codecs)
   (void)tbl;
   const uint32_t wb_lds = lds_addr(wb);
 
@@ -717,10 +745,10 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   int sb_end = a.ksplit > 1 ? sb_begin + a.sb_per_split : nsb;
   sb_end = sb_end < nsb ? sb_end : nsb;
   const int sbn = sb_end - sb_begin;
-  const int nu = sbn > wave ? (sbn - wave + ST_WAVES - 1) / ST_WAVES : 0;  // wave-uniform, 0..XU
+  const int nu = UPS * (sbn > wave ? (sbn - wave + ST_WAVES - 1) / ST_WAVES : 0);  // wave-uniform, 0..XU
 
   // ---- activation loads first: they are the oldest loads of the wave
-  const uint16_t* x16 = static_cast<const uint16_t*>(a.x);
+  const uint16_t* x16 = static_cast<const uint16_t*>(a.x) + (GM ? (size_t)(g_entry / a.x_div) * K : 0);
   // codebook codecs: threads 0 .. 127 fetch 16 bytes each of the 2 KiB grid the tables are built from
   u32x4 greg = {0, 0, 0, 0};
   // replicated iq2_xxs tables: the sixteen lanes of a quarter wave write the sixteen copies of one entry (a wave
@@ -764,7 +792,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   };
   // (offsets are relative to the tile's first row; a tile always starts inside the matrix)
   // Elements of the stream: (tile, unit) in tile-major order.  `it`, `iu`, `islot`: next element to issue.
-  int it = blockIdx.x, iu = 0, islot = 0, inflight = 0;
+  int it = tile0, iu = 0, islot = 0, inflight = 0;
   int goff_row0 = -1;
   auto issue_next = [&]() {
     if (it >= tiles) return;
@@ -773,8 +801,9 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
       SFor<U::FULL + 1>::run([&](auto t) { constexpr int T = decltype(t)::value; goff[T] = piece_off(lane + 64 * T, row0); });
       goff_row0 = row0;
     }
-    const uint8_t* base = a.w + (size_t)row0 * row_bytes + (size_t)(sb_begin + wave + ST_WAVES * iu) * G::BPB;
-    const uint32_t l0 = wb_lds + islot * U::SLOT;
+    const uint8_t* base = ((GM == 2 && (iu & 1)) ? wmat2 : wmat) + (size_t)row0 * row_bytes +
+                          (size_t)(sb_begin + wave + ST_WAVES * (iu / UPS)) * G::BPB;
+    const uint32_t l0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(wb_lds + islot * U::SLOT));
     SFor<U::FULL>::run([&](auto t) { constexpr int T = decltype(t)::value; dma16(base, goff[T], l0 + T * 1024); });
     if constexpr (U::HALF) {
       if (lane < 32) dma16(base, goff[U::FULL], l0 + U::FULL * 1024);
@@ -1017,12 +1046,13 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   // stalls in the issue, and the activation work above would have waited behind that stall.
   ST_TS(2);
   SFor<D - 1>::run([&](auto) { issue_next(); });
-  float acc[R];
-  int ct = blockIdx.x, cslot = 0;  // tile / slot being consumed
+  float acc_a[R], acc_b[GM == 2 ? R : 1];
+  int ct = tile0, cslot = 0;  // tile / slot being consumed
   int parity = 0;
   for (; ct < tiles; ct += G_x) {
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.f;
+    for (int r = 0; r < R; r++) acc_a[r] = 0.f;
+    acc_b[0] = 0.f;
     const int row0 = ct * rpt;
     const int nrows = N - row0 < rpt ? N - row0 : rpt;
     const int crow = n < nrows ? n : nrows - 1;
@@ -1038,21 +1068,23 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         ST_TS(3 + u);
         const uint8_t* slot = wb + cslot * U::SLOT;
         const uint8_t* bl = slot + crow * G::LBPB;
+        constexpr int us = u / UPS;  // the wave's superblock this unit belongs to
+        float* acc = (GM == 2 && (u & 1)) ? acc_b : acc_a;
         if constexpr (C == KQ_Q6_K) {
           const float dx = kq::h2f((uint16_t)*reinterpret_cast<const uint32_t*>(slot + ST_ROWS * G::LBPB + 4 * crow)) * xscale;
-          q6k_unit<R, AS>(bl, dx, kg, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
+          q6k_unit<R, AS>(bl, dx, kg, areg + us * NAP, xsum + us * 16, ST_XU * 16, acc);
         } else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) {
-          q23k_unit<C, R, AS>(bl, kg, xscale, areg + u * NAP, xsum + u * 16, ST_XU * 16, acc);
+          q23k_unit<C, R, AS>(bl, kg, xscale, areg + us * NAP, xsum + us * 16, ST_XU * 16, acc);
         } else if constexpr (C == KQ_IQ4_XS) {
-          iq4xs_unit<R, AS>(bl, kg, xscale, areg + u * NAP, tbl + 4 * (lane & 31), acc);
+          iq4xs_unit<R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc);
         } else if constexpr (C == KQ_IQ2_XXS) {
           constexpr int COP = st_iq2_copies<C, MB, NW>();
-          iq2xxs_unit<R, AS, COP>(bl, kg, xscale, areg + u * NAP, COP > 1 ? tbl + 16 * (lane & 15) : tbl, acc);
+          iq2xxs_unit<R, AS, COP>(bl, kg, xscale, areg + us * NAP, COP > 1 ? tbl + 16 * (lane & 15) : tbl, acc);
         } else if constexpr (C == KQ_IQ3_S) {
           const float dx = kq::h2f((uint16_t)*reinterpret_cast<const uint32_t*>(slot + ST_ROWS * G::LBPB + 4 * crow)) * xscale;
-          iq3s_unit<R, AS, st_iq3s_merged<C, MB, NW>()>(bl, kg, dx, areg + u * NAP, tbl, acc);
+          iq3s_unit<R, AS, st_iq3s_merged<C, MB, NW>()>(bl, kg, dx, areg + us * NAP, tbl, acc);
         } else {
-          q45k_unit<C, R, AS>(bl, kg, xscale, areg + u * NAP, xsum + u * 8, ST_XU * 8, acc);
+          q45k_unit<C, R, AS>(bl, kg, xscale, areg + us * NAP, xsum + us * 8, ST_XU * 8, acc);
         }
         // the slot has been read: refill it with the next element of the stream
         lgkm_drain();
@@ -1069,19 +1101,26 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
       for (int i = 0; i < 8; i++) a.ts[((size_t)blockIdx.x * ST_WAVES + wave) * 8 + i] = ts[i];
 #endif
     // ---- cross-wave + cross-half reduction of the tile
-    float* red = red_all + (parity * ST_WAVES + wave) * (R * 64);
+    float* red = red_all + (parity * ST_WAVES + wave) * (UPS * R * 64);
 #pragma unroll
-    for (int r = 0; r < R; r++) red[r * 64 + lane] = acc[r];
+    for (int r = 0; r < R; r++) red[r * 64 + lane] = acc_a[r];
+    if constexpr (GM == 2) red[R * 64 + lane] = acc_b[0];
     wg_lds_barrier();
     if (tid < R * 32) {
       const int r = tid >> 5, nn = tid & 31;
-      float v = 0.f;
+      float v = 0.f, vu = 0.f;
 #pragma unroll
       for (int wv = 0; wv < ST_WAVES; wv++) {
-        const float* rw = red_all + (parity * ST_WAVES + wv) * (R * 64);
+        const float* rw = red_all + (parity * ST_WAVES + wv) * (UPS * R * 64);
         v += rw[r * 64 + nn] + rw[r * 64 + nn + 32];
+        if constexpr (GM == 2) vu += rw[R * 64 + nn] + rw[R * 64 + nn + 32];
       }
-      if (r < M && nn < nrows) {
+      if constexpr (GM != 0) {
+        if (nn < nrows) {
+          if constexpr (GM == 2) v = kq::glu_epilogue(a.act, v, vu, a.limit, 1.0f);
+          kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, g_entry) * N + row0 + nn, v);
+        }
+      } else if (r < M && nn < nrows) {
         if (a.ksplit > 1) {
           a.partial[(size_t)blockIdx.z * M * N + (size_t)r * N + row0 + nn] = v;
         } else {
@@ -1094,10 +1133,10 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   }
 }
 
-template <int C, int MB, int D, int ST_XU, int ST_WAVES>
+template <int C, int MB, int D, int ST_XU, int ST_WAVES, int GM = 0>
 constexpr size_t st_lds_bytes() {
   return (size_t)ST_WAVES * (D * StUnit<C>::SLOT + st_xch<MB>() * ST_XU * 512 + MB * ST_XU * 2 * StGeom<C>::XSG * 4) +
-         2 * ST_WAVES * MB * 64 * 4 + st_tbl_bytes<C, MB, ST_WAVES>();
+         (GM == 2 ? 2 : 1) * 2 * ST_WAVES * MB * 64 * 4 + st_tbl_bytes<C, MB, ST_WAVES>();
 }
 
 template <int DT>
@@ -1221,6 +1260,36 @@ int st_launch_m(const StArgs& a, int splits, hipStream_t s) {
   return st_launch_one<C, DT, 8, D, 4>(a, splits, s);
 }
 
+// Gathered calls: one workgroup per (entry, 32-row tile); NW waves share the entry's K range, XU = 4 units per
+// wave, i.e. at most 4 NW superblocks (2 NW for the gate / up pair, whose superblocks are two units).
+template <int C, int DT, int NW, int GM>
+int st_launch_gather(StArgs a, int entries, hipStream_t s) {
+  constexpr int D = 2, XU = 4;
+  constexpr size_t lds = st_lds_bytes<C, 1, D, XU, NW, GM>();
+  static_assert(lds <= 160 * 1024, "workgroup does not fit the LDS of a CU");
+  constexpr int WGS = lds <= 80 * 1024 && NW == 4 ? 2 : 1;
+  auto kern = stream_gemv_kernel<C, DT, 1, D, WGS, XU, NW, GM>;
+  static bool attr_set = false;  // per instantiation
+  if (!attr_set) {
+    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  a.rpt = ST_ROWS;
+  a.tiles_per_entry = (a.N + ST_ROWS - 1) / ST_ROWS;
+  a.tiles = a.tiles_per_entry;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(entries * a.tiles_per_entry)), dim3(64 * NW), lds, s, a);
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
+template <int C, int DT>
+int st_launch_gather_nw(const StArgs& a, int entries, bool glu, hipStream_t s) {
+  const int nsb = a.K >> 8;
+  // gate / up pair: two units per superblock; beyond four superblocks eight waves keep a wave at two to four units
+  if (glu) return nsb <= 4 ? st_launch_gather<C, DT, 4, 2>(a, entries, s) : st_launch_gather<C, DT, 8, 2>(a, entries, s);
+  return nsb <= 16 ? st_launch_gather<C, DT, 4, 1>(a, entries, s) : st_launch_gather<C, DT, 8, 1>(a, entries, s);
+}
+
 bool st_codec_ok(int codec) {
   return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K || codec == KQ_Q2_K || codec == KQ_Q3_K ||
          codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S;
@@ -1281,4 +1350,44 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
   return dtype == KQ_F16 ? st_launch_m<KQ_Q6_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q6_K, KQ_BF16>(a, p.ksplit, s);
 }
 
-
+// Gathered matvec of MoE decode on the streamed kernel: entry p (0 .. entries - 1) multiplies row p / x_div of x
+// [.., K] by the [N, K] matrix of expert rhs[p] (w; with w2 the fused gate / up form act(x . gate) * (x . up)) into
+// output row out_row(om, p).  q4_k / q5_k / q6_k, K of at most 32 superblocks (16 for the fused form).
+int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* rhs, void* out,
+                            int entries, int N, int K, int x_div, int64_t w_expert_stride, int act, float limit,
+                            int codec, int dtype, int E, KqOutMap om, hipStream_t s) {
+  if (codec != KQ_Q4_K && codec != KQ_Q5_K && codec != KQ_Q6_K) return KQ_ERR_UNSUPPORTED;
+  if (entries < 1 || entries > 64 || N < 1 || K < 256 || (K & 255) || !rhs) return KQ_ERR_UNSUPPORTED;
+  const bool glu = w2 != nullptr;
+  if ((K >> 8) > (glu ? 16 : 32) || (glu && act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
+  if ((int64_t)entries * ((N + ST_ROWS - 1) / ST_ROWS) > 65535 * 16) return KQ_ERR_UNSUPPORTED;
+  const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;
+  if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
+      ((uintptr_t)w_expert_stride & wmask) || (reinterpret_cast<uintptr_t>(x) & 15) || ((K * 2) & 15))
+    return KQ_ERR_UNSUPPORTED;
+  StArgs a{};
+  a.x = x;
+  a.w = w;
+  a.w2 = w2;
+  a.rhs = rhs;
+  a.y = out;
+  a.M = 1;
+  a.N = N;
+  a.K = K;
+  a.ksplit = 1;
+  a.sb_per_split = K >> 8;
+  a.x_div = x_div < 1 ? 1 : x_div;
+  a.E = E;
+  a.act = act;
+  a.limit = limit;
+  a.w_expert_stride = w_expert_stride;
+  a.om = om;
+  if (codec == KQ_Q4_K)
+    return dtype == KQ_F16 ? st_launch_gather_nw<KQ_Q4_K, KQ_F16>(a, entries, glu, s)
+                           : st_launch_gather_nw<KQ_Q4_K, KQ_BF16>(a, entries, glu, s);
+  if (codec == KQ_Q5_K)
+    return dtype == KQ_F16 ? st_launch_gather_nw<KQ_Q5_K, KQ_F16>(a, entries, glu, s)
+                           : st_launch_gather_nw<KQ_Q5_K, KQ_BF16>(a, entries, glu, s);
+  return dtype == KQ_F16 ? st_launch_gather_nw<KQ_Q6_K, KQ_F16>(a, entries, glu, s)
+                         : st_launch_gather_nw<KQ_Q6_K, KQ_BF16>(a, entries, glu, s);
+}
