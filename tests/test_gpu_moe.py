@@ -345,3 +345,32 @@ def test_rhs_gather_more_than_32767_rows(kq, codec):
     gb = dev_to_bits(got)
     assert rel_l2(gb, want, "float16") <= TOL
     assert rel_l2(gb[:64], want[:64], "float16") <= TOL and rel_l2(gb[-64:], want[-64:], "float16") <= TOL
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("N,K,T,R,act", [
+    (72, 768, 1, 8, "silu"),       # ragged rows (72 = 2 tiles + 8), three superblocks: four-wave form, one unit a wave
+    (96, 3072, 2, 4, "gelu"),      # twelve superblocks: eight-wave fused form, two tokens share the activations
+    (40, 4096, 1, 3, "silu"),      # sixteen superblocks, the longest K of the fused form
+    (64, 6144, 2, 2, "silu"),      # past it for the fused form (older kernel), inside the plain form's 32
+])
+def test_moe_decode_entries_on_the_streamed_kernel(kq, codec, N, K, T, R, act, dtype):
+    """Up to 16 (token, expert) entries of a K-quant stack run the gathered mode of the streamed kernel: fused
+    gate / up (two units per superblock) and the plain down projection."""
+    E = 5
+    gate, up, down = _stack(codec, E, N, K, 201), _stack(codec, E, N, K, 202), _stack(codec, E, N, K, 203)
+    rng = np.random.default_rng(204)
+    idx = rng.integers(0, E, (T, R))
+    xb, xt = make_x((T, K), dtype, seed=205, scale=0.1)
+    h = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act=act)
+    assert tuple(h.shape) == (T, R, N)
+    assert rel_l2(dev_to_bits(h), _glu_truth(codec, xb, gate, up, idx, act, dtype=dtype), dtype) <= TOL
+    xb2, xt2 = make_x((T, R, K), dtype, seed=206, scale=0.1)
+    y = kq.gather_qmv_kq(xt2, wire_to_dev(down), codec, _idx_dev(idx))
+    assert tuple(y.shape) == (T, R, N)
+    assert rel_l2(dev_to_bits(y), O.gather_qmv(xb2, down, codec, idx, None, dtype), dtype) <= TOL
+    # the entries agree with a dense matmul against the expert's matrix (the dense streamed kernel)
+    e0 = int(idx[0, 0])
+    dense = kq.quantized_matmul(xt2[0, :1].contiguous(), wire_to_dev(down[e0]), None, codec)
+    assert rel_l2(dev_to_bits(y[0, 0:1]), dev_to_bits(dense), dtype) <= TOL

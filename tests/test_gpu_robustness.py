@@ -162,3 +162,35 @@ def test_qmm_replayed_from_a_hip_graph(kq, codec, M):
         assert torch.equal(y_graph, y_eager), (codec, rep)
         other = torch.randn(256, 256, device="cuda:0")
         (other @ other).sum().item()  # the program's own eager work between replays
+
+
+@pytest.mark.parametrize("codec,K", [("q4_k", 1024), ("q6_k", 512)])
+def test_fused_gate_up_skips_expert_ids_outside_the_stack(kq, codec, K):
+    """kq_moe_glu_gather with 8 entries (the gathered mode of the streamed kernel): entries whose expert id is >= E
+    leave their output rows as they were, the others are computed."""
+    lib = kq._load()
+    cid = lib.kq_codec_id(codec.encode())
+    E, N, T, R = 3, 48, 4, 2
+    gate = _wire(codec, E * N, K, 95).reshape(E, N, -1)
+    up = _wire(codec, E * N, K, 96).reshape(E, N, -1)
+    g_dev, u_dev = wire_to_dev(gate), wire_to_dev(up)
+    xb, xt = make_x((T, K), "bfloat16", seed=97, scale=0.1)
+    idx = np.array([[0, 3], [2, 0xFFFFFFFF], [1, 1], [7, 0]], dtype=np.uint32)
+    idx_t = torch.from_numpy(idx.view(np.int32).copy()).cuda()
+    out = torch.full((T, R, N), 5.0, dtype=torch.bfloat16, device="cuda:0")
+    nws = lib.kq_moe_workspace_size(T, R, E, N, K, 1, cid, KQ_BF16)
+    ws = torch.empty(max(nws, 256), dtype=torch.uint8, device="cuda:0")
+    rc = lib.kq_moe_glu_gather(xt.data_ptr(), g_dev.data_ptr(), u_dev.data_ptr(), idx_t.data_ptr(), None, None,
+                               out.data_ptr(), T, R, E, N, K, 0, 0.0, 0.0, cid, KQ_BF16, ws.data_ptr(), nws,
+                               torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.kq_last_error()
+    torch.cuda.synchronize()
+    got = dev_to_bits(out)
+    for t in range(T):
+        for r in range(R):
+            if idx[t, r] >= E:
+                assert np.all(O.bits_to_f32(got[t, r], "bfloat16") == 5.0), (codec, t, r)
+            else:
+                want = O.moe_glu_gather(xb[t:t + 1], gate, up, codec, idx[t:t + 1, r:r + 1].astype(np.int64), "silu",
+                                        dtype="bfloat16")
+                assert rel_l2(got[t:t + 1, r:r + 1], want, "bfloat16") <= TOL, (codec, t, r)
