@@ -183,17 +183,18 @@ constexpr int st_xord() { return C == KQ_IQ4_XS ? 2 : C == KQ_IQ2_XXS || C == KQ
 //            has the LDS for [16 sign nibbles][512] entries with the signs applied (64 KiB, in front of the plain
 //            entries it is built from): one table read per four weights and no XOR.  With the two-table form the
 //            kernel is bound by the LDS (88 % busy, 63 % of that bank conflicts of the data-dependent reads).
-template <int C, int MB = 0, int NW = 0>
-constexpr bool st_iq3s_merged() { return C == KQ_IQ3_S && MB == 1 && NW == 8; }
+template <int C, int MB = 0, int NW = 0, int GM = 0>
+constexpr bool st_iq3s_merged() { return C == KQ_IQ3_S && MB == 1 && NW == 8 && GM == 0; }
 // iq2_xxs, one-row eight-wave kernel: 16 copies of both tables, entry e copy c at 256 e + 16 c, lane l reads copy
 // l % 16, so the sixteen lanes of a 16-byte read never meet in a bank (with single copies the kernel is bound by the
 // LDS: 90 % busy, 60 % of that bank conflicts).
-template <int C, int MB = 0, int NW = 0>
-constexpr int st_iq2_copies() { return C == KQ_IQ2_XXS && MB == 1 && NW == 8 ? 16 : 1; }
-template <int C, int MB = 0, int NW = 0>
+template <int C, int MB = 0, int NW = 0, int GM = 0>
+constexpr int st_iq2_copies() { return C == KQ_IQ2_XXS && MB == 1 && NW == 8 && GM == 0 ? 16 : 1; }
+// (gathered launches, whose workgroups live for one to four units, keep the plain iq2_xxs / iq3_s tables)
+template <int C, int MB = 0, int NW = 0, int GM = 0>
 constexpr int st_tbl_bytes() {
-  return C == KQ_IQ4_XS ? 32768 : C == KQ_IQ2_XXS ? (4096 + 2048) * st_iq2_copies<C, MB, NW>() :
-         st_iq3s_merged<C, MB, NW>() ? 65536 + 4096 : C == KQ_IQ3_S ? 4096 + 4096 : 0;
+  return C == KQ_IQ4_XS ? 32768 : C == KQ_IQ2_XXS ? (4096 + 2048) * st_iq2_copies<C, MB, NW, GM>() :
+         st_iq3s_merged<C, MB, NW, GM>() ? 65536 + 4096 : C == KQ_IQ3_S ? 4096 + 4096 : 0;
 }
 template <int C>
 struct StUnit {
@@ -753,7 +754,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   u32x4 greg = {0, 0, 0, 0};
   // replicated iq2_xxs tables: the sixteen lanes of a quarter wave write the sixteen copies of one entry (a wave
   // store covers 1 KiB of consecutive LDS); wave w converts the grid entries 32 i + 4 w + lane / 16, i = 0 .. 7
-  constexpr int IQ2_COP = st_iq2_copies<C, MB, NW>();
+  constexpr int IQ2_COP = st_iq2_copies<C, MB, NW, GM>();
   u32x2 gq[IQ2_COP > 1 ? 8 : 1];
   if constexpr (C == KQ_IQ2_XXS) {
     if constexpr (IQ2_COP == 1) {
@@ -962,8 +963,8 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
       *reinterpret_cast<u32x4*>(tbl + 128 * b + 16 * (lane & 7)) = u32x4{ev, ev, ev, ev};
     }
   }
-  if constexpr (C == KQ_IQ2_XXS && st_iq2_copies<C, MB, NW>() > 1) {
-    constexpr int COP = st_iq2_copies<C, MB, NW>();
+  if constexpr (C == KQ_IQ2_XXS && st_iq2_copies<C, MB, NW, GM>() > 1) {
+    constexpr int COP = st_iq2_copies<C, MB, NW, GM>();
     static_assert(COP == 1 || (COP == 16 && NW == 8), "eight waves write 16 copies");
     typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
     uint8_t* dst = tbl + 256 * (4 * wave + (lane >> 4)) + 16 * (lane & 15);
@@ -1008,7 +1009,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
     }
   }
   if constexpr (C == KQ_IQ3_S) {
-    constexpr bool MERGED = st_iq3s_merged<C, MB, NW>();
+    constexpr bool MERGED = st_iq3s_merged<C, MB, NW, GM>();
     uint8_t* plain = MERGED ? tbl + 65536 : tbl;
     if (tid < 128) {  // four grid entries of four bytes -> four times four f16 magnitudes
       typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
@@ -1078,11 +1079,11 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         } else if constexpr (C == KQ_IQ4_XS) {
           iq4xs_unit<R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc);
         } else if constexpr (C == KQ_IQ2_XXS) {
-          constexpr int COP = st_iq2_copies<C, MB, NW>();
+          constexpr int COP = st_iq2_copies<C, MB, NW, GM>();
           iq2xxs_unit<R, AS, COP>(bl, kg, xscale, areg + us * NAP, COP > 1 ? tbl + 16 * (lane & 15) : tbl, acc);
         } else if constexpr (C == KQ_IQ3_S) {
           const float dx = kq::h2f((uint16_t)*reinterpret_cast<const uint32_t*>(slot + ST_ROWS * G::LBPB + 4 * crow)) * xscale;
-          iq3s_unit<R, AS, st_iq3s_merged<C, MB, NW>()>(bl, kg, dx, areg + us * NAP, tbl, acc);
+          iq3s_unit<R, AS, st_iq3s_merged<C, MB, NW, GM>()>(bl, kg, dx, areg + us * NAP, tbl, acc);
         } else {
           q45k_unit<C, R, AS>(bl, kg, xscale, areg + us * NAP, xsum + us * 8, ST_XU * 8, acc);
         }
@@ -1136,7 +1137,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 template <int C, int MB, int D, int ST_XU, int ST_WAVES, int GM = 0>
 constexpr size_t st_lds_bytes() {
   return (size_t)ST_WAVES * (D * StUnit<C>::SLOT + st_xch<MB>() * ST_XU * 512 + MB * ST_XU * 2 * StGeom<C>::XSG * 4) +
-         (GM == 2 ? 2 : 1) * 2 * ST_WAVES * MB * 64 * 4 + st_tbl_bytes<C, MB, ST_WAVES>();
+         (GM == 2 ? 2 : 1) * 2 * ST_WAVES * MB * 64 * 4 + st_tbl_bytes<C, MB, ST_WAVES, GM>();
 }
 
 template <int DT>
@@ -1297,6 +1298,8 @@ bool st_codec_ok(int codec) {
 
 }  // namespace
 
+// The dense and the gathered launchers can be compiled into separate objects (KQ_STREAM_PART = 1 dense, 2 gathered).
+#if !defined(KQ_STREAM_PART) || KQ_STREAM_PART == 1
 bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const void* w) {
   if (!st_codec_ok(codec) || M < 1 || M > 8 || N < 1 || K < 256 || (K & 255)) return false;
   if ((int64_t)N * (K >> 8) * 210 >= (int64_t)1 << 40) return false;
@@ -1350,18 +1353,21 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
   return dtype == KQ_F16 ? st_launch_m<KQ_Q6_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q6_K, KQ_BF16>(a, p.ksplit, s);
 }
 
+#endif  // dense part
+
+#if !defined(KQ_STREAM_PART) || KQ_STREAM_PART == 2
 // Gathered matvec of MoE decode on the streamed kernel: entry p (0 .. entries - 1) multiplies row p / x_div of x
 // [.., K] by the [N, K] matrix of expert rhs[p] (w; with w2 the fused gate / up form act(x . gate) * (x . up)) into
-// output row out_row(om, p).  q4_k / q5_k / q6_k, K of at most 32 superblocks (16 for the fused form).
+// output row out_row(om, p).  Every codec of the streamed kernel, K of at most 32 superblocks (16 for the fused form).
 int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* rhs, void* out,
                             int entries, int N, int K, int x_div, int64_t w_expert_stride, int act, float limit,
                             int codec, int dtype, int E, KqOutMap om, hipStream_t s) {
-  if (codec != KQ_Q4_K && codec != KQ_Q5_K && codec != KQ_Q6_K) return KQ_ERR_UNSUPPORTED;
+  if (!st_codec_ok(codec)) return KQ_ERR_UNSUPPORTED;
   if (entries < 1 || entries > 64 || N < 1 || K < 256 || (K & 255) || !rhs) return KQ_ERR_UNSUPPORTED;
   const bool glu = w2 != nullptr;
   if ((K >> 8) > (glu ? 16 : 32) || (glu && act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
   if ((int64_t)entries * ((N + ST_ROWS - 1) / ST_ROWS) > 65535 * 16) return KQ_ERR_UNSUPPORTED;
-  const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;
+  const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : 1;
   if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
       ((uintptr_t)w_expert_stride & wmask) || (reinterpret_cast<uintptr_t>(x) & 15) || ((K * 2) & 15))
     return KQ_ERR_UNSUPPORTED;
@@ -1382,12 +1388,19 @@ int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, 
   a.limit = limit;
   a.w_expert_stride = w_expert_stride;
   a.om = om;
-  if (codec == KQ_Q4_K)
-    return dtype == KQ_F16 ? st_launch_gather_nw<KQ_Q4_K, KQ_F16>(a, entries, glu, s)
-                           : st_launch_gather_nw<KQ_Q4_K, KQ_BF16>(a, entries, glu, s);
-  if (codec == KQ_Q5_K)
-    return dtype == KQ_F16 ? st_launch_gather_nw<KQ_Q5_K, KQ_F16>(a, entries, glu, s)
-                           : st_launch_gather_nw<KQ_Q5_K, KQ_BF16>(a, entries, glu, s);
-  return dtype == KQ_F16 ? st_launch_gather_nw<KQ_Q6_K, KQ_F16>(a, entries, glu, s)
-                         : st_launch_gather_nw<KQ_Q6_K, KQ_BF16>(a, entries, glu, s);
+  if (codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S) {
+    a.grids = kq_device_grids();
+    if (!a.grids) return KQ_ERR_HIP;
+  }
+  switch (codec) {
+#define KQ_CASE(c)                                                                    \
+  case c:                                                                             \
+    return dtype == KQ_F16 ? st_launch_gather_nw<c, KQ_F16>(a, entries, glu, s)       \
+                           : st_launch_gather_nw<c, KQ_BF16>(a, entries, glu, s);
+    KQ_CASE(KQ_Q2_K) KQ_CASE(KQ_Q3_K) KQ_CASE(KQ_Q4_K) KQ_CASE(KQ_Q5_K) KQ_CASE(KQ_Q6_K) KQ_CASE(KQ_IQ4_XS)
+    KQ_CASE(KQ_IQ3_S) KQ_CASE(KQ_IQ2_XXS)
+#undef KQ_CASE
+  }
+  return KQ_ERR_UNSUPPORTED;
 }
+#endif  // gathered part

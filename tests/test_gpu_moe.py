@@ -348,7 +348,7 @@ def test_rhs_gather_more_than_32767_rows(kq, codec):
 
 
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
-@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k", "q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs"])
 @pytest.mark.parametrize("N,K,T,R,act", [
     (72, 768, 1, 8, "silu"),       # ragged rows (72 = 2 tiles + 8), three superblocks: four-wave form, one unit a wave
     (96, 3072, 2, 4, "gelu"),      # twelve superblocks: eight-wave fused form, two tokens share the activations
@@ -356,7 +356,7 @@ def test_rhs_gather_more_than_32767_rows(kq, codec):
     (64, 6144, 2, 2, "silu"),      # past it for the fused form (older kernel), inside the plain form's 32
 ])
 def test_moe_decode_entries_on_the_streamed_kernel(kq, codec, N, K, T, R, act, dtype):
-    """Up to 16 (token, expert) entries of a K-quant stack run the gathered mode of the streamed kernel: fused
+    """Up to 16 (token, expert) entries of a stack in one of the streamed kernel's codecs run its gathered mode: fused
     gate / up (two units per superblock) and the plain down projection."""
     E = 5
     gate, up, down = _stack(codec, E, N, K, 201), _stack(codec, E, N, K, 202), _stack(codec, E, N, K, 203)
