@@ -311,12 +311,22 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 }
 
 // Batched MoE path: returns KQ_ERR_UNSUPPORTED (error text untouched) when it does not apply.
+// Up to this many (token, expert) pairs of a q4_k / q5_k / q6_k stack the per-entry streamed kernel is the faster
+// route (128 experts of 2048 <-> 768, top-8, fused gate / up + down: 3 tokens 17.5 + 16.3 against 28.0 + 20.5 us,
+// 6 tokens 25.2 + 27.3 against 28.3 + 27.4, 8 tokens 30.0 + 33.7 against 35.1 + 32.9).
+#ifndef KQ_PER_ENTRY_MAX_PAIRS
+#define KQ_PER_ENTRY_MAX_PAIRS 48
+#endif
 static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
                            const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
                            int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
                            size_t ws_bytes, KqOutMap om, hipStream_t s) {
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
+  // few entries: the per-entry kernels (the caller tries them next) beat the prologue + grouped-kernel pair
+  if (P <= KQ_PER_ENTRY_MAX_PAIRS && P > 16 && !bias && !bias2 && (codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K) &&
+      (!glu || act != KQ_ACT_SWIGLU_CLAMP) && (K >> 8) <= (glu ? 16 : 32) && (K & 255) == 0)
+    return KQ_ERR_UNSUPPORTED;
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
     // legacy / IQ / fp4 codecs (biases and every activation included): code-level grouped kernel
     if (kq_codes_moe_supported((int)P, E, N, K, codec)) {

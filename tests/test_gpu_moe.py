@@ -354,10 +354,11 @@ def test_rhs_gather_more_than_32767_rows(kq, codec):
     (96, 3072, 2, 4, "gelu"),      # twelve superblocks: eight-wave fused form, two tokens share the activations
     (40, 4096, 1, 3, "silu"),      # sixteen superblocks, the longest K of the fused form
     (64, 6144, 2, 2, "silu"),      # past it for the fused form (older kernel), inside the plain form's 32
+    (64, 1024, 10, 4, "silu"),     # 40 entries: still one workgroup per (entry, tile) for q4_k / q5_k / q6_k
 ])
 def test_moe_decode_entries_on_the_streamed_kernel(kq, codec, N, K, T, R, act, dtype):
-    """Up to 16 (token, expert) entries of a stack in one of the streamed kernel's codecs run its gathered mode: fused
-    gate / up (two units per superblock) and the plain down projection."""
+    """Up to 16 (token, expert) entries of a stack in one of the streamed kernel's codecs (48 for q4_k / q5_k / q6_k)
+    run its gathered mode: fused gate / up (two units per superblock) and the plain down projection."""
     E = 5
     gate, up, down = _stack(codec, E, N, K, 201), _stack(codec, E, N, K, 202), _stack(codec, E, N, K, 203)
     rng = np.random.default_rng(204)

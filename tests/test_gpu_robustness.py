@@ -61,7 +61,8 @@ def test_ops_on_a_side_stream_see_their_inputs(kq):
                                      ("q2_k", 256)])
 def test_expert_ids_outside_the_stack_are_skipped(kq, codec, K, T):
     """Entries whose expert id is >= E are left out (their output rows keep what they held); the others are
-    computed as usual.  8 entries run the per-entry kernels (tuned, code-level, generic), 24 the grouped ones."""
+    computed as usual.  8 entries run the per-entry kernels (streamed, code-level, generic), 24 the grouped ones
+    (q4_k / q6_k: still the per-entry streamed kernel)."""
     lib = kq._load()
     cid = lib.kq_codec_id(codec.encode())
     E, N, R = 3, 64, 2
