@@ -1166,10 +1166,15 @@ int st_num_cus() {
 // range is cut further so that about two workgroups per CU exist.
 struct StSplit {
   int ksplit, sb_per_split;
+  int rpt;  // rows per tile the plan asks for (0: 32, levelled by the launcher)
 };
 constexpr int g_st_fill_pct = 150;  // row tiles x splits per 100 CUs below which K is split further
 constexpr int g_st_min_rpt = 24;    // fewest rows a levelled tile may have (16 measured slower than 32)
 constexpr bool g_st_nw8 = true;
+#ifndef KQ_ST_SHORT_TILES
+#define KQ_ST_SHORT_TILES 1
+#endif
+constexpr bool g_st_short_tiles = KQ_ST_SHORT_TILES != 0;
 int st_max_sb(int codec, int M);
 // superblocks a workgroup can take: 32 with the eight-wave kernel where its LDS fits (every codec for up to two
 // rows, the codecs with small units for up to four)
@@ -1203,9 +1208,16 @@ StSplit st_split_plan(int M, int N, int K, int codec, int cus) {
     if (more > want) want = more;
   }
   if (want < 1) want = 1;
+  // one or two rows, fewer 32-row tiles than CUs and a K range one eight-wave workgroup can take: shorter tiles
+  // (one per CU) instead of a K split, which would add the reduction launch (4096 x 4096: 7.0 -> 5.6 us)
+  if (g_st_short_tiles && want > 1 && M <= 4 && maxsb >= 32 && nsb >= 8 && nsb <= 32 && tiles < cus) {
+    int r = (N + cus - 1) / cus;
+    if (r < 8) r = 8;
+    if (r < ST_ROWS) return StSplit{1, nsb > 16 ? nsb : 17, r};  // sb_per_split > 16 selects the eight-wave kernel
+  }
   int per = (nsb + want - 1) / want;
   if (per > maxsb) per = maxsb;
-  StSplit p{(nsb + per - 1) / per, per};
+  StSplit p{(nsb + per - 1) / per, per, 0};
   return p;
 }
 
@@ -1226,7 +1238,9 @@ int st_launch_one(StArgs a, int splits, hipStream_t s) {
   // busiest CU decides the time (448 tiles on 512 slots: two tiles on 192 CUs, one on 64).  Spreading the rows
   // over rounds x slots equal tiles of 24 ... 32 rows levels that; the rows a short tile leaves out cost idle lanes,
   // not bandwidth.
-  {
+  if (a.rpt > 0) {  // the plan's short tiles
+    a.tiles = (a.N + a.rpt - 1) / a.rpt;
+  } else {
     const int tiles32 = (a.N + ST_ROWS - 1) / ST_ROWS;
     const int rounds = (tiles32 + gx - 1) / gx;
     const int rpt = (a.N + rounds * gx - 1) / (rounds * gx);
@@ -1333,6 +1347,7 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
   a.partial = static_cast<float*>(ws);
   a.ksplit = p.ksplit;
   a.sb_per_split = p.sb_per_split;
+  a.rpt = p.rpt;
   if (codec == KQ_Q4_K)
     return dtype == KQ_F16 ? st_launch_m<KQ_Q4_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q4_K, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q5_K)
