@@ -127,11 +127,13 @@ def test_qmm_streamed_kernel_shapes(kq, codec, dtype):
     """The streamed kernel (default for up to eight rows of q4_k / q5_k / q6_k): one to eight rows (five and more
     run two groups of four), K ranges that leave waves without a superblock (256, 768), K above 16 superblocks
     (split over grid z), a ragged last row tile, a single row, row counts that level to tiles of fewer than 32
-    rows (14336 -> 28, 15000 -> 30) and more row tiles than resident workgroups (persistent loop, N = 20000)."""
+    rows (14336 -> 28, 15000 -> 30), more row tiles than resident workgroups (persistent loop, N = 20000), and
+    small shapes of up to four rows that run short tiles (8 or 16 rows, 4096 x 4096, 1000 x 2048, 97 x 4096)
+    on eight-wave workgroups instead of a K split."""
     for M, N, K in ((1, 33, 256), (2, 31, 768), (3, 1, 1024), (4, 97, 4096), (1, 20000, 1024), (2, 1030, 5120),
                     (1, 4100, 14336), (4, 2050, 8192), (5, 33, 256), (8, 97, 4096), (7, 1030, 5120), (6, 2050, 8192),
                     (8, 20000, 1024), (5, 1, 768), (1, 14336, 512), (8, 15000, 256), (3, 14336, 1024), (1, 8192, 8192),
-                    (2, 300, 6144), (4, 8200, 7936)):
+                    (2, 300, 6144), (4, 8200, 7936), (1, 4096, 4096), (3, 1000, 2048)):
         wire = _wire(codec, N, K, seed=43)
         xb, xt = make_x((M, K), dtype, seed=44)
         got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
