@@ -332,7 +332,7 @@ __global__ __launch_bounds__(AM_THREADS, 1) void any_mma_kernel(AnyArgs a) {
       for (int i = 0; i < 16; i++) {
         const int pr = pair_lds[8 * (i >> 2) + 4 * kg + (i & 3)];
         if (pr >= 0 && live) {
-          const float v = kq::glu_epilogue(a.act, acc[0][i] + gb, ex[(nb * 16 + i) * 64 + lane] + ub, a.limit, a.alpha);
+          const float v = kq::glu_epilogue_fast(a.act, acc[0][i] + gb, ex[(nb * 16 + i) * 64 + lane] + ub, a.limit, a.alpha);
           kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, pr) * N + n0 + col, v);
         }
       }

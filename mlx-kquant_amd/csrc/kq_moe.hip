@@ -493,24 +493,28 @@ __global__ __launch_bounds__(MOE_THREADS, 3) void moe_grouped_kernel(MoeArgs a) 
   // ---- epilogue: undo the activation scale, (GLU: combine gate and up,) round once, scatter rows
   if constexpr (GLU) {
     if constexpr (MOE_STAGES == 1) lds_barrier();  // the step buffers are free: reuse them for the up accumulators
+    // The gate wave (even) and the up wave (odd) of a column block swap half of their accumulators and finish eight
+    // outputs each: the gate wave registers 0 .. 7, the up wave 8 .. 15.
     float* ex = reinterpret_cast<float*>(smem);  // [2 column blocks][16][64]
     const int nb = wave >> 1;
-    if (wave & 1) {
+    const bool upw = (wave & 1) != 0;
 #pragma unroll
-      for (int i = 0; i < 16; i++) ex[(nb * 16 + i) * 64 + lane] = acc[0][i];
+    for (int i = 0; i < 8; i++) {
+      const int give = upw ? i : 8 + i;  // the register the partner finishes
+      ex[(nb * 16 + give) * 64 + lane] = upw ? acc[0][i] : acc[0][8 + i];
     }
     lds_barrier();
-    if (!(wave & 1)) {
-      const int col = nb * 32 + l32;
+    const int col = nb * 32 + l32;
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        const int slot = 8 * (i >> 2) + 4 * kg + (i & 3);
-        const int pr = pair_lds[slot];
-        if (pr >= 0 && col < ncols) {
-          const float r = rs_lds[slot];
-          const float v = kq::glu_epilogue(a.act, acc[0][i] * r, ex[(nb * 16 + i) * 64 + lane] * r, a.limit, 1.0f);
-          kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, pr) * N + n0 + col, v);
-        }
+    for (int j = 0; j < 8; j++) {
+      const int i = upw ? 8 + j : j;
+      const int slot = 8 * (i >> 2) + 4 * kg + (i & 3);
+      const int pr = pair_lds[slot];
+      if (pr >= 0 && col < ncols) {
+        const float r = rs_lds[slot];
+        const float mine = (upw ? acc[0][8 + j] : acc[0][j]) * r, other = ex[(nb * 16 + i) * 64 + lane] * r;
+        const float v = kq::glu_epilogue_fast(a.act, upw ? other : mine, upw ? mine : other, a.limit, 1.0f);
+        kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, pr) * N + n0 + col, v);
       }
     }
   } else {
