@@ -560,13 +560,30 @@ __device__ __forceinline__ void iq3s_unit(const uint8_t* __restrict__ bl, int kg
     const uint32_t hb = qh >> (8 * ib);
     // sign words 6 and 7 of the block sit four bytes further (behind the two bytes the last piece repeats)
     const uint32_t sw = *reinterpret_cast<const uint32_t*>(sgp + 4 * ib + (ib >= 2 ? 4 * kg : 0));
-    SFor<8>::run([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      const uint32_t w = j < 4 ? w0 : w1;
-      uint32_t idx = ((w >> (8 * (j & 3))) & 0xff) | (((hb >> j) & 1) << 8);
-      if constexpr (MERGED) idx |= ((sw >> (4 * j)) & 15) << 9;
-      gv[ib][j] = *reinterpret_cast<const u32x2*>(tbl + 8 * idx);
-    });
+    if constexpr (MERGED) {
+      // 13-bit table index of value j = index byte | high bit << 8 | sign nibble << 9, built two per dword with byte
+      // permutes: the high bits spread to the low bit of each byte (even and odd values apart, by a 24-bit multiply
+      // whose partial products meet only beside the kept bits), the sign nibbles shifted beside them, then
+      // interleaved with the index bytes.
+      const uint32_t he = __umul24(hb & 0x55u, 0x41041u) & 0x01010101u;
+      const uint32_t ho = __umul24((hb >> 1) & 0x55u, 0x41041u) & 0x01010101u;
+      const uint32_t ce = ((sw << 1) & 0x1e1e1e1eu) | he, co = ((sw >> 3) & 0x1e1e1e1eu) | ho;
+      const uint32_t c03 = __builtin_amdgcn_perm(co, ce, 0x05010400u), c47 = __builtin_amdgcn_perm(co, ce, 0x07030602u);
+      const uint32_t pr[4] = {__builtin_amdgcn_perm(c03, w0, 0x05010400u), __builtin_amdgcn_perm(c03, w0, 0x07030602u),
+                              __builtin_amdgcn_perm(c47, w1, 0x05010400u), __builtin_amdgcn_perm(c47, w1, 0x07030602u)};
+      SFor<8>::run([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        const uint32_t idx = (j & 1) ? pr[j / 2] >> 16 : pr[j / 2] & 0xffffu;
+        gv[ib][j] = *reinterpret_cast<const u32x2*>(tbl + 8 * idx);
+      });
+    } else {
+      SFor<8>::run([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        const uint32_t w = j < 4 ? w0 : w1;
+        const uint32_t idx = ((w >> (8 * (j & 3))) & 0xff) | (((hb >> j) & 1) << 8);
+        gv[ib][j] = *reinterpret_cast<const u32x2*>(tbl + 8 * idx);
+      });
+    }
     if constexpr (!MERGED) {
       SFor<4>::run([&](auto ll) {
         constexpr int l = decltype(ll)::value;
