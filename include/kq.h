@@ -73,7 +73,10 @@ int kq_dequantize(const void* w_dev, void* out_dev, uint64_t num_weights, int co
 /* y[M,N] = x[M,K] . W^T  (transpose != 0, W decodes to [N,K])  or  x[M,K] . W (transpose == 0,
  * W decodes to [K,N]).  x and y have dtype `dtype` (KQ_F16 / KQ_BF16; the op layer casts f32
  * activations to bf16 first, as the reference does); accumulation is f32 with one rounding
- * to `dtype`.  Workspace: kq_qmm_workspace_size bytes of device memory (may be 0).
+ * to `dtype`.  Workspace: kq_qmm_workspace_size bytes of device memory (may be 0).  With transpose == 0 the
+ * workspace is optional (f32 partial sums of a K range cut over the grid, for calls with few output tiles;
+ * without it the call runs uncut), the weights are split into two bf16 terms (16 significant bits) and the
+ * op is the reference's qmm_n, src/kquant_matmul.cpp:455-527.
  * Replaces kquant_qmm_cpu<T>, reference src/kquant_cpu_decode.h:54-70 /
  * src/kquant_cpu_decode.cpp:1209-1359 (called by KQuantMatmul::eval_cpu,
  * src/kquant_matmul.cpp:1104-1164). */

@@ -20,6 +20,7 @@ SOURCES = [
     ("kq_encode.cpp", ["-x", "hip"]),
     ("kq_generic.hip", ["-ffp-contract=off"]),
     ("kq_mfma.hip", []),
+    ("kq_nt.hip", ["-ffp-contract=off"]),
     # one source, two objects: the dense and the gathered launchers instantiate their kernels in parallel
     ("kq_stream.hip", ["-Wno-inline-asm", "-DKQ_STREAM_PART=1"], "kq_stream_dense"),
     ("kq_stream.hip", ["-Wno-inline-asm", "-DKQ_STREAM_PART=2"], "kq_stream_gather"),

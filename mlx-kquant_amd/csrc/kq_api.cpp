@@ -118,7 +118,8 @@ int kq_dequantize(const void* w_dev, void* out_dev, uint64_t num_weights, int co
 
 size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int dtype) {
   (void)dtype;
-  if (!transpose || !codec_ok(codec)) return 0;
+  if (!codec_ok(codec)) return 0;
+  if (!transpose) return kq_nt_workspace_bytes(M, N, K);  // optional: partial sums of a K range cut over the grid
   if (kq_gemm_supported(M, N, K, codec)) return kq_gemm_workspace_bytes(M, K);
   // split-K partial sums (optional) of whichever skinny kernel takes the call
   const size_t tuned = kq_qmm_tuned_workspace_bytes(M, N, K, codec);
@@ -141,8 +142,12 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
   if (M == 0 || N == 0) return KQ_OK;
   if (!x_dev || !w_dev || !y_dev) return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: null buffer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (!transpose)
+  if (!transpose) {
+    const int rcn = kq_launch_nt_mfma(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, y_dev, 1, M, 1, N, K,
+                                      0, 0, codec, dtype, workspace_dev, workspace_bytes, s);
+    if (rcn != KQ_ERR_UNSUPPORTED) return rcn;
     return kq_launch_gemm_nt_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
+  }
   if (kq_gemm_supported(M, N, K, codec)) {
     const size_t need = kq_gemm_workspace_bytes(M, K);
     if (!workspace_dev || workspace_bytes < need)
@@ -249,9 +254,13 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
   if (!x_dev || !w_dev || !out_dev || !lhs_idx_dev || !rhs_idx_dev)
     return kq_set_error(KQ_ERR_INVALID, "gather_qmm: null buffer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (!transpose)
+  if (!transpose) {
+    const int rcn = kq_launch_nt_mfma(x_dev, static_cast<const uint8_t*>(w_dev), lhs_idx_dev, rhs_idx_dev, out_dev, B, M,
+                                      E, N, K, x_batch_stride, w_expert_stride_bytes, codec, dtype, nullptr, 0, s);
+    if (rcn != KQ_ERR_UNSUPPORTED) return rcn;
     return kq_launch_gather_nt_generic(x_dev, static_cast<const uint8_t*>(w_dev), lhs_idx_dev, rhs_idx_dev, out_dev, B,
                                        M, E, N, K, x_batch_stride, w_expert_stride_bytes, codec, dtype, s);
+  }
   // many output rows: gather them into a dense matrix and run the expert-grouped kernels
   int64_t P;
   if (workspace_dev && gather_batched_shape(B, M, E, N, K, transpose, codec, &P) &&

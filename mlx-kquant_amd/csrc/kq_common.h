@@ -68,6 +68,12 @@ int kq_launch_gemm_nt_generic(const void* x, const uint8_t* w, void* y, int M, i
 int kq_launch_gather_nt_generic(const void* x, const uint8_t* w, const uint32_t* lhs, const uint32_t* rhs, void* out,
                                 int B, int M, int E, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride,
                                 int codec, int dtype, hipStream_t s);
+// kq_nt.hip: transpose = false on the matrix cores (dense: lhs = rhs = null, B = E = 1); KQ_ERR_UNSUPPORTED when
+// the output is not 16-byte aligned.  Dense calls with few tiles cut K when given kq_nt_workspace_bytes of workspace.
+size_t kq_nt_workspace_bytes(int M, int N, int K);
+int kq_launch_nt_mfma(const void* x, const uint8_t* w, const uint32_t* lhs, const uint32_t* rhs, void* out, int B,
+                      int M, int E, int N, int K, int64_t x_batch_stride, int64_t w_expert_stride, int codec, int dtype,
+                      void* ws, size_t ws_bytes, hipStream_t s);
 int kq_launch_gather_generic(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs,
                              const uint32_t* rhs, const float* bias, const float* bias2, void* out, int B, int M,
                              int N, int K, int x_div, int64_t x_batch_stride, int64_t w_expert_stride, int glu,

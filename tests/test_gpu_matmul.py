@@ -165,6 +165,26 @@ def test_qmm_no_transpose(kq, codec):
     assert rel_l2(dev_to_bits(got), want, "float16") <= TOL
 
 
+@pytest.mark.parametrize("codec", O.ALL_CODECS)
+def test_qmm_no_transpose_every_codec_on_the_matrix_cores(kq, codec):
+    """transpose=False (src/kquant_matmul.cpp:455-527 of the reference): the reduction runs over wire rows.  Shapes
+    with a ragged last 32-row step, a K that is no multiple of 8, more than 32 activation rows and a column count
+    that does not fill the last 128-column tile, in both activation types."""
+    shapes = [(1, 128, 512, "bfloat16", 1), (5, 50, 768, "float16", 2), (40, 27, 256, "bfloat16", 3),
+              (3, 16, 1280, "float16", 4)]
+    if codec in ("q4_k", "q6_k", "q8_0", "iq3_s", "mxfp4"):  # long K, few tiles: the K range is cut over the grid
+        shapes += [(3, 1024, 256, "float16", 6), (20, 1000, 256, "bfloat16", 7)]
+    if O.geometry(codec)[0] == 32:
+        shapes.append((2, 70, 352, "bfloat16", 5))
+    for (M, K, N, dtype, seed) in shapes:
+        wire = _wire(codec, K, N, seed=70 + seed)
+        xb, xt = make_x((M, K), dtype, seed=80 + seed)
+        got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec, transpose=False)
+        want = O.qmm(xb, wire, codec, False, dtype)
+        assert tuple(got.shape) == (M, N)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, K, N, dtype)
+
+
 def test_qmm_dtype_rules_and_shapes(kq):
     N, K = 64, 256
     wire = _wire("q4_k", N, K, seed=34)
