@@ -326,6 +326,16 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 #ifndef KQ_PER_ENTRY_MAX_PAIRS
 #define KQ_PER_ENTRY_MAX_PAIRS 48
 #endif
+// q2_k / q3_k stacks have no expert-grouped kernel of their own (their batched route is the any-codec kernel), so
+// the per-entry kernel stays ahead much longer (same stacks, fused gate / up + down, us: 64 pairs 21.9 + 20.1
+// against 87.9 + 47.6 for q2_k, 36.0 + 24.6 against 113.9 + 60.3 for q3_k; 256 pairs 67 + 61 against 154 + 76 and
+// 126 + 76 against 200 + 106; 512 pairs 125 + 116 against 156 + 86 and 245 + 144 against 202 + 108).
+#ifndef KQ_PER_ENTRY_MAX_PAIRS_LOW
+#define KQ_PER_ENTRY_MAX_PAIRS_LOW 256
+#endif
+#ifndef KQ_PER_ENTRY_MAX_PAIRS_IQ
+#define KQ_PER_ENTRY_MAX_PAIRS_IQ 64
+#endif
 static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
                            const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
                            int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
@@ -333,7 +343,12 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
   // few entries: the per-entry kernels (the caller tries them next) beat the prologue + grouped-kernel pair
-  if (P <= KQ_PER_ENTRY_MAX_PAIRS && P > 16 && !bias && !bias2 && (codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K) &&
+  const bool grouped_codec = codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K;
+  const bool low_codec = codec == KQ_Q2_K || codec == KQ_Q3_K;  // their batched route is the any-codec kernel
+  const bool iq_codec = codec == KQ_IQ4_XS || codec == KQ_IQ3_S || codec == KQ_IQ2_XXS;
+  if (P > 16 && !bias && !bias2 &&
+      ((grouped_codec && P <= KQ_PER_ENTRY_MAX_PAIRS) || (low_codec && P <= KQ_PER_ENTRY_MAX_PAIRS_LOW) ||
+       (iq_codec && P <= KQ_PER_ENTRY_MAX_PAIRS_IQ)) &&
       (!glu || act != KQ_ACT_SWIGLU_CLAMP) && (K >> 8) <= (glu ? 16 : 32) && (K & 255) == 0)
     return KQ_ERR_UNSUPPORTED;
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {

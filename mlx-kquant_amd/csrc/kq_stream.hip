@@ -1391,11 +1391,14 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
 // Gathered matvec of MoE decode on the streamed kernel: entry p (0 .. entries - 1) multiplies row p / x_div of x
 // [.., K] by the [N, K] matrix of expert rhs[p] (w; with w2 the fused gate / up form act(x . gate) * (x . up)) into
 // output row out_row(om, p).  Every codec of the streamed kernel, K of at most 32 superblocks (16 for the fused form).
+#ifndef KQ_GATHER_STREAM_MAX_ENTRIES
+#define KQ_GATHER_STREAM_MAX_ENTRIES 256
+#endif
 int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* rhs, void* out,
                             int entries, int N, int K, int x_div, int64_t w_expert_stride, int act, float limit,
                             int codec, int dtype, int E, KqOutMap om, hipStream_t s) {
   if (!st_codec_ok(codec)) return KQ_ERR_UNSUPPORTED;
-  if (entries < 1 || entries > 64 || N < 1 || K < 256 || (K & 255) || !rhs) return KQ_ERR_UNSUPPORTED;
+  if (entries < 1 || entries > KQ_GATHER_STREAM_MAX_ENTRIES || N < 1 || K < 256 || (K & 255) || !rhs) return KQ_ERR_UNSUPPORTED;
   const bool glu = w2 != nullptr;
   if ((K >> 8) > (glu ? 16 : 32) || (glu && act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
   if ((int64_t)entries * ((N + ST_ROWS - 1) / ST_ROWS) > 65535 * 16) return KQ_ERR_UNSUPPORTED;

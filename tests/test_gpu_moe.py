@@ -173,6 +173,28 @@ def test_moe_tuned_gathered_shapes(kq, codec, E, N, K, T, R):
     assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, codec
 
 
+@pytest.mark.parametrize("codec,T", [("q2_k", 50), ("q2_k", 80), ("q3_k", 50), ("q3_k", 80), ("iq4_xs", 15),
+                                     ("iq4_xs", 20), ("iq3_s", 15), ("iq3_s", 20), ("iq2_xxs", 15), ("iq2_xxs", 20)])
+def test_moe_low_bit_routes_either_side_of_the_entry_threshold(kq, codec, T):
+    """q2_k / q3_k stacks run entry by entry on the streamed kernel up to 256 (token, expert) pairs and on the
+    any-codec kernel above; iq4_xs / iq3_s / iq2_xxs switch to the code-level grouped kernel above 64 pairs.  The
+    token counts (x 4 experts each) sit on either side."""
+    E, N, K, R = 6, 136, 768, 4
+    gate = _stack(codec, E, N, K, seed=91)
+    up = _stack(codec, E, N, K, seed=92)
+    rng = np.random.default_rng(93)
+    idx = np.stack([rng.permutation(E)[:R] for _ in range(T)])
+    xb, xt = make_x((T, K), "bfloat16", seed=94, scale=0.05)
+    got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act="silu")
+    want = _glu_truth(codec, xb, gate, up, idx, "silu", 0.0, dtype="bfloat16")
+    assert tuple(got.shape) == (T, R, N)
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, T)
+    hb, ht = make_x((T, R, K), "float16", seed=95, scale=0.05)
+    got = kq.gather_qmv_kq(ht, wire_to_dev(gate), codec, _idx_dev(idx))
+    want = O.gather_qmv(hb, gate, codec, idx, None, "float16")
+    assert rel_l2(dev_to_bits(got), want, "float16") <= TOL, (codec, T)
+
+
 @pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("E,N,K,T,R", [(6, 136, 768, 20, 3), (8, 200, 512, 100, 2), (128, 64, 256, 8, 8),
                                        (5, 72, 4352, 9, 2)])
