@@ -351,6 +351,10 @@ __global__ __launch_bounds__(256) void any_splitk_reduce_kernel(const float* __r
   y[i] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
 }
 
+// 32-row activation groups per workgroup of a dense call: 128-row tiles for bf16 activations, 64-row tiles for
+// f16 (two bf16 planes in LDS), smaller ones for fewer rows
+int any_dense_mt(int M, int dt) { return M <= 32 ? 1 : (M <= 64 || dt == KQ_F16) ? 2 : 4; }
+
 template <int C, int DT, int MT, int MODE>
 int launch_any(const AnyArgs& a, dim3 grid, hipStream_t s) {
   using G = StepGeom<C>;
@@ -374,14 +378,22 @@ constexpr int SEG_M = 32;
 template <int C>
 struct AnyRun {
   static int run(const AnyArgs& a, int mode, int dt, int P, int E, hipStream_t s) {
-    if (mode == 0 && a.M <= 32) {
-      // skinny call: one 32-row activation tile, K split over blockIdx.y when the caller brought a workspace
+    if (mode == 0) {
+      // one to four 32-row activation groups per workgroup; K split over blockIdx.y when the caller brought a
+      // workspace (a.partial) and the plan asked for it
       AnyArgs b = a;
-      b.mtiles = 1;
+      const int mt = any_dense_mt(a.M, dt);
+      b.mtiles = (a.M + 32 * mt - 1) / (32 * mt);
       const int nsteps = (a.K + AM_STEP - 1) / AM_STEP;
       const int splits = (nsteps + a.steps_per_split - 1) / a.steps_per_split;
-      const dim3 grid((a.N + AM_BN - 1) / AM_BN, splits);
-      const int rc = dt == KQ_F16 ? launch_any<C, KQ_F16, 1, 0>(b, grid, s) : launch_any<C, KQ_BF16, 1, 0>(b, grid, s);
+      const dim3 grid(b.mtiles * ((a.N + AM_BN - 1) / AM_BN), splits);
+      int rc;
+      if (mt == 1)
+        rc = dt == KQ_F16 ? launch_any<C, KQ_F16, 1, 0>(b, grid, s) : launch_any<C, KQ_BF16, 1, 0>(b, grid, s);
+      else if (mt == 2)
+        rc = dt == KQ_F16 ? launch_any<C, KQ_F16, 2, 0>(b, grid, s) : launch_any<C, KQ_BF16, 2, 0>(b, grid, s);
+      else
+        rc = launch_any<C, KQ_BF16, 4, 0>(b, grid, s);
       if (rc || !a.partial) return rc;
       const int count = a.M * a.N;
       if (dt == KQ_F16)
@@ -392,17 +404,6 @@ struct AnyRun {
                            static_cast<uint16_t*>(a.y), count, splits);
       KQ_HIP_CHECK(hipGetLastError());
       return KQ_OK;
-    }
-    if (mode == 0) {
-      // 128-row tiles for bf16 activations, 64-row tiles for f16 (two bf16 planes in LDS)
-      if (dt == KQ_BF16) {
-        AnyArgs b = a;
-        b.mtiles = (a.M + 127) / 128;
-        return launch_any<C, KQ_BF16, 4, 0>(b, dim3(b.mtiles * ((a.N + AM_BN - 1) / AM_BN)), s);
-      }
-      AnyArgs b = a;
-      b.mtiles = (a.M + 63) / 64;
-      return launch_any<C, KQ_F16, 2, 0>(b, dim3(b.mtiles * ((a.N + AM_BN - 1) / AM_BN)), s);
     }
     int maxseg = E + P / SEG_M;
     if (maxseg > P) maxseg = P;
@@ -437,25 +438,30 @@ bool kq_anymma_supported(int M, int N, int K, int codec) {
          K % kq_geom(codec).wpb == 0;
 }
 
-// K steps per workgroup of a skinny (M <= 32) dense call: K is split until about 512 workgroups exist.
-static int any_skinny_steps_per_split(int N, int K) {
-  const int nsteps = (K + AM_STEP - 1) / AM_STEP, tiles = (N + AM_BN - 1) / AM_BN;
-  int want = (512 + tiles - 1) / tiles;
+// K steps per workgroup of a dense call: K is split until about 512 workgroups exist (calls of more than 32 rows
+// with 256 tiles or more run unsplit), with the partial sums held to 64 MiB.
+static int any_steps_per_split(int M, int N, int K, int dt) {
+  const int mt = any_dense_mt(M, dt);
+  const int64_t tiles = (int64_t)((N + AM_BN - 1) / AM_BN) * ((M + 32 * mt - 1) / (32 * mt));
+  const int nsteps = (K + AM_STEP - 1) / AM_STEP;
+  int64_t want = (M > 32 && tiles >= 256) ? 1 : (512 + tiles - 1) / tiles;
+  const int64_t cap = ((int64_t)64 << 20) / ((int64_t)M * N * 4);
+  if (want > cap) want = cap;
   if (want > nsteps) want = nsteps;
   if (want < 1) want = 1;
-  return (nsteps + want - 1) / want;
+  return (int)((nsteps + want - 1) / want);
 }
 
-// f32 partial sums of the split-K skinny call (0: no split)
-size_t kq_anymma_dense_workspace_bytes(int M, int N, int K) {
-  if (M > 32 || M <= 0 || N <= 0 || K <= 0) return 0;
-  const int nsteps = (K + AM_STEP - 1) / AM_STEP, per = any_skinny_steps_per_split(N, K);
+// f32 partial sums of the split-K call (0: no split)
+size_t kq_anymma_dense_workspace_bytes(int M, int N, int K, int dtype) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const int nsteps = (K + AM_STEP - 1) / AM_STEP, per = any_steps_per_split(M, N, K, dtype);
   const int splits = (nsteps + per - 1) / per;
   return splits > 1 ? (size_t)splits * M * N * 4 : 0;
 }
 
-// Dense matmul, any codec: prefill tiles, or (M <= 32) one activation tile with K split across
-// workgroups when `ws` holds kq_anymma_dense_workspace_bytes.
+// Dense matmul, any codec; K is split across workgroups when the call has few tiles and `ws` holds
+// kq_anymma_dense_workspace_bytes.
 int kq_launch_anymma_dense(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
                            void* ws, size_t ws_bytes, hipStream_t s) {
   if (!kq_anymma_supported(M, N, K, codec) || (reinterpret_cast<uintptr_t>(x) & 15)) return KQ_ERR_UNSUPPORTED;
@@ -470,12 +476,10 @@ int kq_launch_anymma_dense(const void* x, const uint8_t* w, void* y, int M, int 
   a.K = K;
   a.x_div = 1;
   a.steps_per_split = (K + AM_STEP - 1) / AM_STEP;
-  if (M <= 32) {
-    const size_t need = kq_anymma_dense_workspace_bytes(M, N, K);
-    if (need && ws && ws_bytes >= need && !(reinterpret_cast<uintptr_t>(ws) & 15)) {
-      a.partial = static_cast<float*>(ws);
-      a.steps_per_split = any_skinny_steps_per_split(N, K);
-    }
+  const size_t need = kq_anymma_dense_workspace_bytes(M, N, K, dtype);
+  if (need && ws && ws_bytes >= need && !(reinterpret_cast<uintptr_t>(ws) & 15)) {
+    a.partial = static_cast<float*>(ws);
+    a.steps_per_split = any_steps_per_split(M, N, K, dtype);
   }
   return dispatch_any(codec, a, 0, dtype, 0, 1, s);
 }

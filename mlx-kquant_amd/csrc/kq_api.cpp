@@ -123,7 +123,7 @@ size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int 
   if (kq_gemm_supported(M, N, K, codec)) return kq_gemm_workspace_bytes(M, K);
   // split-K partial sums (optional) of whichever skinny kernel takes the call
   const size_t tuned = kq_qmm_tuned_workspace_bytes(M, N, K, codec);
-  size_t any = (M > 8 && kq_anymma_supported(M, N, K, codec)) ? kq_anymma_dense_workspace_bytes(M, N, K) : 0;
+  size_t any = (M > 8 && kq_anymma_supported(M, N, K, codec)) ? kq_anymma_dense_workspace_bytes(M, N, K, dtype) : 0;
   if (kq_gemm2_low_supported(M, N, K, codec) && kq_gemm2_low_workspace_bytes(M, K) > any) any = kq_gemm2_low_workspace_bytes(M, K);
   return tuned > any ? tuned : any;
 }

@@ -165,7 +165,7 @@ int kq_launch_mix_slots(const float* yf, const float* scores, const uint32_t* id
 // Matrix-core GEMM for every codec (exact bf16 x 3 split of the reference-order decoded weights):
 // prefill, and the batched MoE ops with biases and every activation.
 bool kq_anymma_supported(int M, int N, int K, int codec);
-size_t kq_anymma_dense_workspace_bytes(int M, int N, int K);
+size_t kq_anymma_dense_workspace_bytes(int M, int N, int K, int dtype);
 int kq_launch_anymma_dense(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype,
                            void* ws, size_t ws_bytes, hipStream_t s);
 bool kq_anymma_moe_supported(int P, int E, int N, int K, int codec);
