@@ -87,8 +87,10 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
 /* kq_qmm for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): transpose is implied, and the workspace is a buffer of
  * KQ_NOALLOC_SCRATCH_BYTES that lives inside the library's code object on every GPU (no hipMalloc, hipFree
- * or other allocating call is made).  A call whose kq_qmm_workspace_size exceeds that size is rejected with
- * KQ_ERR_WORKSPACE.  All calls on one GPU share that GPU's buffer: calls that overlap in time on the same
+ * or other allocating call is made).  A call that cannot run in that size (the prefill GEMM of q4_k / q5_k /
+ * q6_k keeps its converted activations there: about 2.2 * M * K bytes) is rejected with KQ_ERR_WORKSPACE; the
+ * optional part of kq_qmm_workspace_size (partial sums of a K range cut over the grid) is used when it fits
+ * and left out otherwise.  All calls on one GPU share that GPU's buffer: calls that overlap in time on the same
  * GPU (different streams or threads) race; the buffer keeps the last call's contents, and the kernels write
  * every element they later read, so nothing needs clearing between calls.
  * No counterpart in the reference. */

@@ -120,7 +120,7 @@ size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int 
   (void)dtype;
   if (!codec_ok(codec)) return 0;
   if (!transpose) return kq_nt_workspace_bytes(M, N, K);  // optional: partial sums of a K range cut over the grid
-  if (kq_gemm_supported(M, N, K, codec)) return kq_gemm_workspace_bytes(M, K);
+  if (kq_gemm_supported(M, N, K, codec)) return kq_gemm_workspace_bytes(M, N, K);
   // split-K partial sums (optional) of whichever skinny kernel takes the call
   const size_t tuned = kq_qmm_tuned_workspace_bytes(M, N, K, codec);
   size_t any = (M > 8 && kq_anymma_supported(M, N, K, codec)) ? kq_anymma_dense_workspace_bytes(M, N, K, dtype) : 0;
@@ -149,11 +149,12 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
     return kq_launch_gemm_nt_generic(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, s);
   }
   if (kq_gemm_supported(M, N, K, codec)) {
-    const size_t need = kq_gemm_workspace_bytes(M, K);
+    const size_t need = kq_gemm_workspace_min_bytes(M, K);
     if (!workspace_dev || workspace_bytes < need)
       return kq_set_error(KQ_ERR_WORKSPACE, "quantized_matmul: workspace of %zu bytes required (got %zu)", need,
                           workspace_bytes);
-    int rcg = kq_launch_gemm(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev, s);
+    int rcg = kq_launch_gemm(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev,
+                             workspace_bytes, s);
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
   }
   if (kq_gemm2_low_supported(M, N, K, codec) && workspace_dev && workspace_bytes >= kq_gemm2_low_workspace_bytes(M, K)) {
@@ -176,7 +177,9 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
 int kq_qmm_noalloc(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int codec, int dtype,
                    void* stream) {
   if (!codec_ok(codec)) return kq_set_error(KQ_ERR_INVALID, "quantized_matmul: unknown codec id %d", codec);
-  const size_t need = kq_qmm_workspace_size(M, N, K, 1, codec, dtype);
+  // what the call cannot run without (the prefill GEMM's converted activations); partial sums of a K range cut
+  // over the grid are optional and are left out when they do not fit
+  const size_t need = kq_gemm_supported(M, N, K, codec) ? kq_gemm_workspace_min_bytes(M, K) : 0;
   if (need > KQ_NOALLOC_SCRATCH_BYTES)
     return kq_set_error(KQ_ERR_WORKSPACE,
                         "quantized_matmul (no-allocation entry): this shape needs %zu bytes of workspace, the built-in "

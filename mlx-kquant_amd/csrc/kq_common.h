@@ -106,11 +106,13 @@ int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, c
                            const uint32_t* rhs, void* out, int B, int M, int N, int K, int x_div,
                            int64_t x_batch_stride, int64_t w_expert_stride, int glu, int act, float limit, int codec,
                            int dtype, int E, KqOutMap om, hipStream_t s);
-// Prefill GEMM (q4_k / q5_k, M > 8): needs kq_gemm_workspace_bytes(M, K) bytes of device workspace.
-size_t kq_gemm_workspace_bytes(int M, int K);
+// Prefill GEMM (q4_k / q5_k / q6_k, M > 8): needs kq_gemm_workspace_min_bytes(M, K) bytes of device workspace
+// (converted activations); with kq_gemm_workspace_bytes(M, N, K) a call with few tiles cuts K over the grid.
+size_t kq_gemm_workspace_min_bytes(int M, int K);
+size_t kq_gemm_workspace_bytes(int M, int N, int K);
 bool kq_gemm_supported(int M, int N, int K, int codec);
 int kq_launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
-                   hipStream_t s);
+                   size_t ws_bytes, hipStream_t s);
 // 128 x 256-tile prefill GEMM (q4_k / q5_k) on the outputs of the activation prepass (rows padded to 128).
 bool kq_gemm2_supported(int M, int N, int K, int codec);
 int kq_launch_gemm2(const void* xh, const void* xhl, const float* rs, const uint8_t* w, void* y, int M, int N, int K,

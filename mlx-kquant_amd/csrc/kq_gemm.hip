@@ -50,7 +50,10 @@ __global__ __launch_bounds__(64 * WAVES, (MT == 4 || WAVES == 8) ? 1 : 2) void k
                                                                     const float* __restrict__ rs,
                                                                     const uint8_t* __restrict__ w,
                                                                     uint16_t* __restrict__ y, int M, int N, int K,
-                                                                    int mtiles) {
+                                                                    int mtiles, int sb_per_split,
+                                                                    float* __restrict__ part) {
+  // part != null: grid y cuts the superblocks into ranges of sb_per_split, whose scaled f32 sums go to
+  // part[range][M][N] and are added by gemm_splitk_reduce_kernel
   using G = WireGeom<C, WAVES>;
   constexpr int GM_THREADS = G::THREADS, BN = G::BN;
   constexpr int TM = 32 * MT;                   // activation rows per tile
@@ -70,8 +73,10 @@ __global__ __launch_bounds__(64 * WAVES, (MT == 4 || WAVES == 8) ? 1 : 2) void k
   // consecutive workgroups share the weight columns (m fastest)
   const int mt = blockIdx.x % mtiles, nt = blockIdx.x / mtiles;
   const int m0 = mt * TM, n0 = nt * BN;
-  const int nsb = K >> 8;
-  const size_t row_bytes = (size_t)nsb * G::BPB;
+  const int nsb_all = K >> 8;
+  const int sb0 = part ? (int)blockIdx.y * sb_per_split : 0;
+  const int nsb = part ? (sb0 + sb_per_split < nsb_all ? sb_per_split : nsb_all - sb0) : nsb_all;  // steps of this workgroup
+  const size_t row_bytes = (size_t)nsb_all * G::BPB;
   const int nrows = N - n0 < BN ? N - n0 : BN;
 
   // piece maps: activations piece i = tid + 256 t -> (row i / 32, piece i % 32); wire piece -> (row i / PPR, i % PPR)
@@ -92,9 +97,9 @@ __global__ __launch_bounds__(64 * WAVES, (MT == 4 || WAVES == 8) ? 1 : 2) void k
       }
     });
   }
-  const uint8_t* wtile = w + (size_t)n0 * row_bytes;
-  const _Float16* xtile = xh + (size_t)m0 * K;
-  const _Float16* htile = xhl + (size_t)m0 * nsb * 16;
+  const uint8_t* wtile = w + (size_t)n0 * row_bytes + (size_t)sb0 * G::BPB;
+  const _Float16* xtile = xh + (size_t)m0 * K + 256 * (size_t)sb0;
+  const _Float16* htile = xhl + ((size_t)m0 * nsb_all + sb0) * 16;
 
   // side channel for the trailing 2-byte d of a q6_k block: thread -> row tid % BN
   const uint8_t* d_src = wtile + (size_t)((tid & (BN - 1)) < nrows ? (tid & (BN - 1)) : 0) * row_bytes + 208;
@@ -112,7 +117,7 @@ __global__ __launch_bounds__(64 * WAVES, (MT == 4 || WAVES == 8) ? 1 : 2) void k
     if constexpr (G::SIDE_D) dreg = *reinterpret_cast<const uint16_t*>(d_src + (size_t)sb * G::BPB);
     // X halves: TM rows x 32 bytes = 2 TM pieces of 16 bytes (threads past them re-read the first rows)
     if constexpr (G::MINS)
-      hreg = *reinterpret_cast<const u32x4*>(htile + ((size_t)((tid >> 1) < TM ? (tid >> 1) : 0) * nsb + sb) * 16 + 8 * (tid & 1));
+      hreg = *reinterpret_cast<const u32x4*>(htile + ((size_t)((tid >> 1) < TM ? (tid >> 1) : 0) * nsb_all + sb) * 16 + 8 * (tid & 1));
   };
   auto park = [&](uint8_t* stage) {
     StaticFor<APT>::run([&](auto t) {
@@ -177,15 +182,49 @@ __global__ __launch_bounds__(64 * WAVES, (MT == 4 || WAVES == 8) ? 1 : 2) void k
       const int m = m0 + t * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
       if (m < M && n < N) {
         const float v = acc[t][i] * rs[m];
-        y[(size_t)m * N + n] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+        if (part)
+          part[((size_t)blockIdx.y * M + m) * N + n] = v;
+        else
+          y[(size_t)m * N + n] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
       }
     }
   }
 }
 
+// y[i] = round(sum over the K ranges of part[range][i]), ranges added in order
+template <int DT>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part, uint16_t* __restrict__ y,
+                                                                 size_t count, int splits) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  float v = 0.f;
+  for (int sp = 0; sp < splits; sp++) v += part[(size_t)sp * count + i];
+  y[i] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+}
+
+// Superblocks per workgroup of a call on 64 x 128 tiles: K is cut while at most 512 workgroups exist (at least two
+// superblocks each) and the partial sums stay within 8 MiB (their write and read cost about 0.5 us per MiB: cut in
+// three, 128 rows on 14336 x 4096 went from 39 to 50 us); calls with 256 tiles or more run uncut (returns K / 256).
+int gemm_sb_per_split(int M, int N, int K) {
+  const int nsb = K >> 8;
+  const int64_t tiles = (int64_t)((M + 63) / 64) * ((N + 127) / 128);
+  if (tiles >= 256 || nsb < 4) return nsb;
+  int64_t want = 512 / tiles;
+  const int64_t cap = ((int64_t)8 << 20) / ((int64_t)M * N * 4);
+  if (want > cap) want = cap;
+  if (want > nsb / 2) want = nsb / 2;
+  if (want < 2) return nsb;
+  return (int)((nsb + want - 1) / want);
+}
+
+size_t gemm_base_bytes(int M, int K) {
+  const size_t mpad = (size_t)((M + BM - 1) / BM) * BM;
+  return mpad * K * 2 + mpad * (K >> 8) * 32 + mpad * 4 + 256;
+}
+
 template <int C, int DT, int MT, int WAVES, bool DB = false>
 int launch_gemm_mt(const _Float16* xh, const _Float16* xhl, const float* rs, const uint8_t* w, void* y, int M, int N,
-                   int K, hipStream_t s) {
+                   int K, hipStream_t s, int sb_per_split = 0, float* part = nullptr) {
   using G = WireGeom<C, WAVES>;
   constexpr int TM = 32 * MT, BN = G::BN;
   const int mtiles = (M + TM - 1) / TM, ntiles = (N + BN - 1) / BN;
@@ -197,15 +236,21 @@ int launch_gemm_mt(const _Float16* xh, const _Float16* xhl, const float* rs, con
                                      (int)lds));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(mtiles * ntiles), dim3(G::THREADS), lds, s, xh, xhl, rs, w, static_cast<uint16_t*>(y), M,
-                     N, K, mtiles);
+  const int splits = part ? ((K >> 8) + sb_per_split - 1) / sb_per_split : 1;
+  hipLaunchKernelGGL(kern, dim3(mtiles * ntiles, splits), dim3(G::THREADS), lds, s, xh, xhl, rs, w,
+                     static_cast<uint16_t*>(y), M, N, K, mtiles, sb_per_split, part);
+  if (part) {
+    const size_t count = (size_t)M * N;
+    hipLaunchKernelGGL((gemm_splitk_reduce_kernel<DT>), dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, part,
+                       static_cast<uint16_t*>(y), count, splits);
+  }
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }
 
 
 template <int C, int DT>
-int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, void* ws, hipStream_t s) {
+int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, void* ws, size_t ws_bytes, hipStream_t s) {
   const int mpad = ((M + BM - 1) / BM) * BM, nsb = K >> 8;
   _Float16* xh = static_cast<_Float16*>(ws);
   _Float16* xhl = xh + (size_t)mpad * K;
@@ -236,14 +281,32 @@ int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, v
     if (tile == 256) return launch_gemm_mt<C, DT, 2, 8, true>(xh, xhl, rs, w, y, M, N, K, s);
   }
   if (tile == 128) return launch_gemm_mt<C, DT, 4, 4>(xh, xhl, rs, w, y, M, N, K, s);
+  // few tiles: cut K over the grid when the workspace also holds the partial sums
+  const int per = g_gemm_tile == 0 ? gemm_sb_per_split(M, N, K) : nsb;
+  if (per < nsb) {
+    const size_t base = (gemm_base_bytes(M, K) + 255) & ~(size_t)255;
+    const int splits = (nsb + per - 1) / per;
+    if (ws_bytes >= base + (size_t)splits * M * N * 4)
+      return launch_gemm_mt<C, DT, 2, 4>(xh, xhl, rs, w, y, M, N, K, s, per,
+                                         reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + base));
+  }
   return launch_gemm_mt<C, DT, 2, 4>(xh, xhl, rs, w, y, M, N, K, s);
 }
 
 }  // namespace
 
-size_t kq_gemm_workspace_bytes(int M, int K) {
-  const size_t mpad = (size_t)((M + BM - 1) / BM) * BM;
-  return mpad * K * 2 + mpad * (K >> 8) * 32 + mpad * 4 + 256;
+// Required part of the workspace: converted activations, block sums, row scales
+size_t kq_gemm_workspace_min_bytes(int M, int K) { return gemm_base_bytes(M, K); }
+
+// ... plus the f32 partial sums of a K range cut over the grid (calls with few tiles; optional: a call whose
+// workspace holds only the required part runs uncut)
+size_t kq_gemm_workspace_bytes(int M, int N, int K) {
+  const size_t base = gemm_base_bytes(M, K);
+  if (M <= 0 || N <= 0 || K < 256) return base;
+  if (M >= 256 && (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 256) return base;
+  const int nsb = K >> 8, per = gemm_sb_per_split(M, N, K);
+  if (per >= nsb) return base;
+  return ((base + 255) & ~(size_t)255) + (size_t)((nsb + per - 1) / per) * M * N * 4;
 }
 
 bool kq_gemm_supported(int M, int N, int K, int codec) {
@@ -251,19 +314,19 @@ bool kq_gemm_supported(int M, int N, int K, int codec) {
 }
 
 int kq_launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
-                   hipStream_t s) {
+                   size_t ws_bytes, hipStream_t s) {
   if (!kq_gemm_supported(M, N, K, codec)) return KQ_ERR_UNSUPPORTED;
   const uintptr_t wmask = codec == KQ_Q6_K ? 1 : 15;  // q6_k pieces are fetched with unaligned loads
   if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(ws) & 15))
     return KQ_ERR_UNSUPPORTED;
   if (codec == KQ_Q6_K)
-    return dtype == KQ_F16 ? launch_gemm<KQ_Q6_K, KQ_F16>(x, w, y, M, N, K, ws, s)
-                           : launch_gemm<KQ_Q6_K, KQ_BF16>(x, w, y, M, N, K, ws, s);
+    return dtype == KQ_F16 ? launch_gemm<KQ_Q6_K, KQ_F16>(x, w, y, M, N, K, ws, ws_bytes, s)
+                           : launch_gemm<KQ_Q6_K, KQ_BF16>(x, w, y, M, N, K, ws, ws_bytes, s);
   if (codec == KQ_Q4_K)
-    return dtype == KQ_F16 ? launch_gemm<KQ_Q4_K, KQ_F16>(x, w, y, M, N, K, ws, s)
-                           : launch_gemm<KQ_Q4_K, KQ_BF16>(x, w, y, M, N, K, ws, s);
-  return dtype == KQ_F16 ? launch_gemm<KQ_Q5_K, KQ_F16>(x, w, y, M, N, K, ws, s)
-                         : launch_gemm<KQ_Q5_K, KQ_BF16>(x, w, y, M, N, K, ws, s);
+    return dtype == KQ_F16 ? launch_gemm<KQ_Q4_K, KQ_F16>(x, w, y, M, N, K, ws, ws_bytes, s)
+                           : launch_gemm<KQ_Q4_K, KQ_BF16>(x, w, y, M, N, K, ws, ws_bytes, s);
+  return dtype == KQ_F16 ? launch_gemm<KQ_Q5_K, KQ_F16>(x, w, y, M, N, K, ws, ws_bytes, s)
+                         : launch_gemm<KQ_Q5_K, KQ_BF16>(x, w, y, M, N, K, ws, ws_bytes, s);
 }
 
 int kq_launch_act_prepass(const void* x, void* xh, void* xhl, float* rs, int M, int K, int dtype, hipStream_t s) {
