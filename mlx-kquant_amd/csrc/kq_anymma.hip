@@ -3,11 +3,12 @@
 // do not cover (legacy, IQ, fp4, biases, swiglu_clamp).
 //
 // Numerics.  A wave decodes its 32 weight columns with the reference-order decoders of
-// kq_decode.h (f32, bit-identical to dequantize) and splits every f32 weight into three bf16
-// terms by truncation, w = b1 + b2 + b3 exactly (8 + 8 + 8 significand bits; bf16 has the f32
-// exponent range, so no codec scale can overflow or underflow).  Activations are bf16 as given, or
+// kq_decode.h (f32, bit-identical to dequantize) and splits every f32 weight into two bf16
+// terms, the truncation and the remainder rounded to nearest (16 significand bits, an error below
+// 2^-17 of the weight; bf16 has the f32 exponent range, so no codec scale can overflow or
+// underflow; KQ_ANY_TERMS = 3 builds the exact three-term form).  Activations are bf16 as given, or
 // f16 split exactly into two bf16 terms.  v_mfma_f32_32x32x16_bf16 then forms exact products and
-// accumulates in f32: the result differs from the f32 reference by summation order only.
+// accumulates in f32.
 //
 // Tiling.  Workgroup = 4 waves, tile = (32 MT activation rows) x 128 weight rows, K advances one
 // 256-weight step (a superblock, or 8 / 4 of the 32 / 64-weight blocks; the last step of a K that is
@@ -74,6 +75,27 @@ __device__ __forceinline__ void split3(const float* w, uint32_t* o1, uint32_t* o
     o3[i] = (t3[0] >> 16) | t3[1];
   }
 }
+
+// f32 -> bf16 by truncation + the remainder rounded to nearest (v_cvt_pk_bf16_f32): 16 significand bits, an error
+// below 2^-17 of the weight.  Two terms instead of three take a third off the MFMAs and 2.5 vector instructions per
+// weight off the split; the kernel is bound by both.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void split2(const float* w, uint32_t* o1, uint32_t* o2) {
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const float v0 = w[2 * i], v1 = w[2 * i + 1];
+    const uint32_t b0 = __builtin_bit_cast(uint32_t, v0), b1 = __builtin_bit_cast(uint32_t, v1);
+    o1[i] = __builtin_amdgcn_perm(b1, b0, 0x07060302u);
+    const float r0 = v0 - __builtin_bit_cast(float, b0 & 0xffff0000u);
+    const float r1 = v1 - __builtin_bit_cast(float, b1 & 0xffff0000u);
+    const bf16x2_t lo = {(__bf16)r0, (__bf16)r1};
+    o2[i] = __builtin_bit_cast(uint32_t, lo);
+  }
+}
+
+#ifndef KQ_ANY_TERMS
+#define KQ_ANY_TERMS 2
+#endif
 
 struct AnyArgs {
   const void* x;        // dense: [M][K]; grouped: [rows][K], pair p reads row p / x_div
@@ -269,8 +291,11 @@ __global__ __launch_bounds__(AM_THREADS, 1) void any_mma_kernel(AnyArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; e++) w8[e] = 0.f;
       }
-      uint32_t b1[4], b2[4], b3[4];
-      split3(w8, b1, b2, b3);
+      uint32_t b1[4], b2[4], b3[4] = {0u, 0u, 0u, 0u};
+      if constexpr (KQ_ANY_TERMS == 3)
+        split3(w8, b1, b2, b3);
+      else
+        split2(w8, b1, b2);
       const bf16x8 f1 = __builtin_bit_cast(bf16x8, make_uint4(b1[0], b1[1], b1[2], b1[3]));
       const bf16x8 f2 = __builtin_bit_cast(bf16x8, make_uint4(b2[0], b2[1], b2[2], b2[3]));
       const bf16x8 f3 = __builtin_bit_cast(bf16x8, make_uint4(b3[0], b3[1], b3[2], b3[3]));
@@ -281,7 +306,7 @@ __global__ __launch_bounds__(AM_THREADS, 1) void any_mma_kernel(AnyArgs a) {
           const bf16x8 av = *reinterpret_cast<const bf16x8*>(a_lane + (pl * TM + t * 32) * A_STRIDE + 32 * i);
           acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, f1, acc[t], 0, 0, 0);
           acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, f2, acc[t], 0, 0, 0);
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, f3, acc[t], 0, 0, 0);
+          if constexpr (KQ_ANY_TERMS == 3) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, f3, acc[t], 0, 0, 0);
         }
       }
     }
