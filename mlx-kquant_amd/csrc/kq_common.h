@@ -164,7 +164,7 @@ int kq_launch_tiles_to_rows(const uint32_t* map, const uint32_t* counts, int cap
                             uint32_t* row_expert, hipStream_t s);
 int kq_launch_mix_slots(const float* yf, const float* scores, const uint32_t* idx, int routed, int E, void* out, int T,
                         int S, int N, int dtype, hipStream_t s);
-// Matrix-core GEMM for every codec (exact bf16 x 3 split of the reference-order decoded weights):
+// Matrix-core GEMM for every codec (two-term bf16 split of the reference-order decoded weights):
 // prefill, and the batched MoE ops with biases and every activation.
 bool kq_anymma_supported(int M, int N, int K, int codec);
 size_t kq_anymma_dense_workspace_bytes(int M, int N, int K, int dtype);

@@ -232,7 +232,7 @@ def test_qmm_prefill_gemm(kq, codec, M, N, K):
 
 @pytest.mark.parametrize("codec", O.ALL_CODECS)
 def test_qmm_prefill_every_codec(kq, codec):
-    """M > 8 for every codec (the tuned K-quant GEMM or the any-codec bf16 x 3 matrix-core path), both
+    """M > 8 for every codec (the tuned K-quant GEMM or the any-codec bf16 matrix-core path), both
     activation dtypes, N that is not a multiple of the 128-row slab, and for the 32-weight-block codecs a K
     that is not a multiple of the 256-weight step."""
     wpb, _ = O.geometry(codec)
