@@ -26,7 +26,7 @@ __all__ = [
     "codecs", "codec_has_matmul", "codec_has_moe_glu", "dequantize", "quantized_matmul", "quantized_matmul_qmv_bias",
     "gather_qmm", "expert_tile_map", "gather_qmm_seg",
     "moe_glu_gather_kq", "gather_qmv_kq", "moe_glu_gather_shexp_kq", "gather_qmv_mix_kq", "gather_qmv_mix_ns_kq",
-    "moe_router_topk", "mxfp4_packed_to_wire", "mxfp4_wire_to_packed", "moe_glu_gather", "gather_qmv_bias",
+    "moe_router_topk", "mxfp4_packed_to_wire", "mxfp4_wire_to_packed", "set_packed_cache", "moe_glu_gather", "gather_qmv_bias",
     "gather_qmv_mix_bias", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
     "weights_per_row", "lib_path",
 ]
@@ -740,6 +740,45 @@ def mxfp4_packed_to_wire(w, scales, *, stream=None):
     return wire
 
 
+# Wire forms of the packed stacks the three packed-layout ops below were called with: the reference's kernels read
+# the packed layout directly (src/kquant_moe_glu.cpp:149-275); here a stack is rewritten to wire form on the device
+# the first time an op sees it and the result is kept for as long as the packed tensors live and stay unmodified
+# (torch's version counters), so a model that calls these ops every step converts each stack once.  The copy costs
+# 17/16 of the stack's bytes of device memory; set_packed_cache(0) turns the cache off (one conversion per call).
+_PACKED_CACHE = {}
+_PACKED_CACHE_MAX = 256
+
+
+def set_packed_cache(max_entries: int) -> None:
+    """Number of packed mxfp4 stacks whose wire form is kept between calls (0: convert on every call)."""
+    global _PACKED_CACHE_MAX
+    _PACKED_CACHE_MAX = max(0, int(max_entries))
+    _PACKED_CACHE.clear()
+
+
+def _wire_of_packed(w, scales, stream):
+    import weakref
+    if _PACKED_CACHE_MAX == 0:
+        return mxfp4_packed_to_wire(w, scales, stream=stream)
+    key = (w.data_ptr(), scales.data_ptr(), tuple(w.shape), str(w.device))
+    hit = _PACKED_CACHE.get(key)
+    if hit is not None:
+        wref, sref, ver, wire, ev = hit
+        if wref() is w and sref() is scales and ver == (w._version, scales._version):
+            if not ev.query():  # still in flight: order the consumer's stream after the conversion
+                (stream if isinstance(stream, torch.cuda.Stream) else torch.cuda.current_stream(w.device)).wait_event(ev)
+            return wire
+        _PACKED_CACHE.pop(key, None)
+    wire = mxfp4_packed_to_wire(w, scales, stream=stream)
+    ev = torch.cuda.Event()
+    ev.record(stream if isinstance(stream, torch.cuda.Stream) else torch.cuda.current_stream(w.device))
+    if len(_PACKED_CACHE) >= _PACKED_CACHE_MAX:
+        _PACKED_CACHE.pop(next(iter(_PACKED_CACHE)))
+    _PACKED_CACHE[key] = (weakref.ref(w), weakref.ref(scales), (w._version, scales._version), wire, ev)
+    weakref.finalize(w, _PACKED_CACHE.pop, key, None)
+    return wire
+
+
 def mxfp4_wire_to_packed(wire, *, stream=None):
     """The inverse of mxfp4_packed_to_wire: (codes int32 [..., K/8], scales uint8 [..., K/32])."""
     op = "mxfp4_wire_to_packed"
@@ -771,8 +810,8 @@ def moe_glu_gather(x, gate_w, gate_scales, gate_bias, up_w, up_scales, up_bias, 
     _check_packed_stack(op, up_w, up_scales, up_bias, K)
     if gate_w.shape != up_w.shape:
         raise ValueError("[kq.moe_glu_gather] gate and up stacks must have the same shape.")
-    return moe_glu_gather_kq(x, mxfp4_packed_to_wire(gate_w, gate_scales, stream=stream),
-                             mxfp4_packed_to_wire(up_w, up_scales, stream=stream), "mxfp4", indices, act="swiglu_clamp",
+    return moe_glu_gather_kq(x, _wire_of_packed(gate_w, gate_scales, stream),
+                             _wire_of_packed(up_w, up_scales, stream), "mxfp4", indices, act="swiglu_clamp",
                              limit=limit, gate_bias=gate_bias, up_bias=up_bias, alpha=alpha, stream=stream)
 
 
@@ -785,7 +824,7 @@ def gather_qmv_bias(x, w, scales, bias, indices, *, stream=None):
     if indices.ndim != 2 or tuple(indices.shape) != tuple(x.shape[:2]):
         raise ValueError("[kq.gather_qmv_bias] indices must be [T, R] matching x.")
     _check_packed_stack(op, w, scales, bias, x.shape[2])
-    return gather_qmv_kq(x, mxfp4_packed_to_wire(w, scales, stream=stream), "mxfp4", indices, bias=bias, stream=stream)
+    return gather_qmv_kq(x, _wire_of_packed(w, scales, stream), "mxfp4", indices, bias=bias, stream=stream)
 
 
 def gather_qmv_mix_bias(x, w, scales, bias, indices, scores, *, stream=None):
@@ -805,7 +844,7 @@ def gather_qmv_mix_bias(x, w, scales, bias, indices, scores, *, stream=None):
     _check_packed_stack(op, w, scales, bias, K)
     _same_device(op, x, w, scales, bias, indices, scores)
     sp = _stream_ptr(op, x, stream)
-    wire = mxfp4_packed_to_wire(w, scales, stream=stream)
+    wire = _wire_of_packed(w, scales, stream)
     cid, _ = _codec(op, "mxfp4")
     E, N = w.shape[0], w.shape[1]
     x_c, idx = x.contiguous(), _prep_idx(indices)

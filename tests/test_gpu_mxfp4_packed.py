@@ -108,3 +108,33 @@ def test_mix_bias_matches_ns_op_with_zero_bias(kq):
                                idx, sc)
     b = kq.gather_qmv_mix_ns_kq(ht, wire_to_dev(_wire_from_codes(codes, scales)), "mxfp4", idx, sc)
     assert torch.equal(a, b)
+
+
+def test_packed_stack_wire_form_is_kept_and_follows_in_place_changes(kq):
+    """The packed-layout ops keep a stack's wire form between calls: a second call on the same tensors gives the
+    same bytes, an in-place change of the stack is seen by the next call, and with the cache off every call converts."""
+    E, N, K, T, R = 3, 64, 288, 5, 2
+    rng = np.random.default_rng(17)
+    gc, gs, gw = _packed_stack(E, N, K, seed=12)
+    gb = (rng.standard_normal((E, N)) * 0.01).astype(np.float32)
+    idx = rng.integers(0, E, (T, R))
+    idx_dev = torch.from_numpy(idx).cuda()
+    hb, ht = make_x((T, R, K), "bfloat16", seed=19, scale=0.2)
+    w_dev, s_dev, b_dev = _dev_words(gw), torch.from_numpy(gs).cuda(), torch.from_numpy(gb).cuda()
+    first = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+    again = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+    assert torch.equal(first, again)
+    assert rel_l2(dev_to_bits(first), O.gather_qmv(hb, _wire_from_codes(gc, gs), "mxfp4", idx, gb, "bfloat16"), "bfloat16") <= TOL
+    # double every weight of the stack in place (scale exponents + 1): the kept wire form must not be used
+    s_dev.add_(1)
+    gs2 = gs + 1
+    changed = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+    want = O.gather_qmv(hb, _wire_from_codes(gc, gs2), "mxfp4", idx, gb, "bfloat16")
+    assert rel_l2(dev_to_bits(changed), want, "bfloat16") <= TOL
+    assert not torch.equal(changed, first)
+    try:
+        kq.set_packed_cache(0)
+        off = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+        assert torch.equal(off, changed)
+    finally:
+        kq.set_packed_cache(256)
