@@ -336,6 +336,16 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 #ifndef KQ_PER_ENTRY_MAX_PAIRS_LOW
 #define KQ_PER_ENTRY_MAX_PAIRS_LOW 256
 #endif
+// The legacy / other IQ / fp4 codecs: the code-level per-entry kernel against the code-level grouped kernel (same
+// stacks, us: mxfp4 32 pairs 24.9 + 21.0 against 37.4 + 22.7, 64 pairs 41.2 + 36.1 against 53.8 + 34.1; q4_0 64 pairs
+// 39.2 + 27.7 against 52.6 + 33.4; iq2_xs 48 pairs 33.6 + 29.8 against 40.7 + 26.6, even at 64).  nvfp4's batched
+// route is the any-codec kernel: 64 pairs 68 + 51 against 128 + 71, 128 pairs 127 + 96 against 158 + 96, behind at 256.
+#ifndef KQ_PER_ENTRY_MAX_PAIRS_CODES
+#define KQ_PER_ENTRY_MAX_PAIRS_CODES 48
+#endif
+#ifndef KQ_PER_ENTRY_MAX_PAIRS_NVFP4
+#define KQ_PER_ENTRY_MAX_PAIRS_NVFP4 128
+#endif
 #ifndef KQ_PER_ENTRY_MAX_PAIRS_IQ
 #define KQ_PER_ENTRY_MAX_PAIRS_IQ 64
 #endif
@@ -349,6 +359,11 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
   const bool grouped_codec = codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K;
   const bool low_codec = codec == KQ_Q2_K || codec == KQ_Q3_K;  // their batched route is the any-codec kernel
   const bool iq_codec = codec == KQ_IQ4_XS || codec == KQ_IQ3_S || codec == KQ_IQ2_XXS;
+  // the other codecs' per-entry kernel is the code-level one, which takes biases and every activation
+  const bool codes_codec = !grouped_codec && !low_codec && !iq_codec;
+  if (codes_codec && P > 16 && P <= (codec == KQ_NVFP4 ? KQ_PER_ENTRY_MAX_PAIRS_NVFP4 : KQ_PER_ENTRY_MAX_PAIRS_CODES) &&
+      kq_codes_gather_supported(1, N, K, codec))
+    return KQ_ERR_UNSUPPORTED;
   if (P > 16 && !bias && !bias2 &&
       ((grouped_codec && P <= KQ_PER_ENTRY_MAX_PAIRS) || (low_codec && P <= KQ_PER_ENTRY_MAX_PAIRS_LOW) ||
        (iq_codec && P <= KQ_PER_ENTRY_MAX_PAIRS_IQ)) &&

@@ -141,6 +141,7 @@ int kq_launch_codes_skinny(const void* x, const uint8_t* w, const void* bias, vo
                            int dtype, hipStream_t s);
 // Batched MoE of the same codecs (more than 16 pairs; biases and every activation): pairs sorted by expert,
 // 32-pair segments x 128-row slabs.  Workspace layout and size as the any-codec path below.
+bool kq_codes_gather_supported(int M, int N, int K, int codec);
 bool kq_codes_moe_supported(int P, int E, int N, int K, int codec);
 size_t kq_codes_moe_workspace_bytes(int P, int E, int rows, int K);
 int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,

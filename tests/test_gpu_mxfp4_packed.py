@@ -61,9 +61,9 @@ def test_layout_converters(kq):
     assert np.array_equal(back_w.cpu().numpy().view(np.uint32), words) and np.array_equal(back_s.cpu().numpy(), scales)
 
 
-@pytest.mark.parametrize("T,R", [(3, 2), (64, 4)])
+@pytest.mark.parametrize("T,R", [(3, 2), (10, 4), (64, 4)])
 def test_packed_ops_match_wire_oracle(kq, T, R):
-    """Per-entry (T * R <= 16) and batched paths; gpt-oss style biases, alpha = 1.702, limit = 7."""
+    """Per-entry (up to 48 pairs) and batched paths; gpt-oss style biases, alpha = 1.702, limit = 7."""
     E, N, K = 4, 64, 576
     rng = np.random.default_rng(7)
     gc, gs, gw = _packed_stack(E, N, K, seed=2)
