@@ -19,7 +19,8 @@ Extra fields: `sweep` (the decode projections of the q4_k_m recipe at M in {1,2,
 intermediate 768: fused gate/up GLU in q4_k and down in q6_k at 1 and 256 tokens), `lowbit` (M=1
 GEMV 8192 -> 8192 in the low-bit codecs), `moe_decode_lowbit` (1 token, 8 of 128 experts, IQ / mxfp4 stacks),
 `dequantize` (whole-matrix decode to f16, wire bytes in plus
-2 N K bytes out), `roofline` for the dominant kernel and `cpu_baseline`
+2 N K bytes out), `mid_m` (16 ... 64 activation rows on 4096-wide matrices), `no_transpose` (transpose = 0:
+128 gathered entries of (M x 128) . (128 x 512), and dense 4096 x 4096), `roofline` for the dominant kernel and `cpu_baseline`
 (the CPU oracle timed on this box's host cores on the headline GEMV).
 """
 import argparse
@@ -196,6 +197,40 @@ class Abi:
                 self._check(rc)
         return call
 
+    def qmm_nt(self, x, w, codec, K, N):
+        """transpose = 0: x [M, K] . W, W stored as K wire rows of N weights."""
+        torch, lib = self.torch, self.lib
+        M = x.shape[0]
+        cid = lib.kq_codec_id(codec.encode())
+        out = torch.empty((M, N), dtype=x.dtype, device=self.dev)
+        nws = lib.kq_qmm_workspace_size(M, N, K, 0, cid, KQ_BF16)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=self.dev)
+        args = (x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, 0, cid, KQ_BF16, ws.data_ptr(), nws)
+        keep = (x, w, out, ws)
+
+        def call(stream=None, _keep=keep):
+            rc = lib.kq_qmm(*args, stream or self.stream)
+            if rc:
+                self._check(rc)
+        return call
+
+    def gather_nt(self, x, w, codec, rhs, E, K, N):
+        """transpose = 0, gathered: entry b = x[b] ([M, K]) . W[rhs[b]], every expert K wire rows of N weights."""
+        torch, lib = self.torch, self.lib
+        B, M = x.shape[0], x.shape[1]
+        cid = lib.kq_codec_id(codec.encode())
+        out = torch.empty((B, M, N), dtype=x.dtype, device=self.dev)
+        lhs = torch.arange(B, dtype=torch.int32, device=self.dev)
+        args = (x.data_ptr(), w.data_ptr(), lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), B, M, E, N, K, M * K,
+                w.numel() // E, 0, 0, cid, KQ_BF16, 0, 0)
+        keep = (x, w, out, lhs, rhs)
+
+        def call(stream=None, _keep=keep):
+            rc = lib.kq_gather_qmm(*args, stream or self.stream)
+            if rc:
+                self._check(rc)
+        return call
+
     def dequantize(self, w, codec, N, K, out):
         lib = self.lib
         cid = lib.kq_codec_id(codec.encode())
@@ -283,7 +318,7 @@ def main():
                     help="prefill section: force a tile shape of the prefill GEMM (kq_set_gemm_tile_rows)")
     ap.add_argument("--only", default=None, metavar="SECTIONS",
                     help="comma-separated extra sections to run (sweep, prefill, moe, moe_mxfp4, moe_decode_lowbit, "
-                         "lowbit, dequantize); default all")
+                         "lowbit, dequantize, mid_m, no_transpose); default all")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for `rocprofv3 --pmc`: one device copy of the headline matrix (known bytes) "
                          "followed by 20 cold launches of the headline GEMV, nothing else")
@@ -557,6 +592,42 @@ def main():
                             "pct_hbm_peak": round(100 * total / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
                 del cps, outs, wq
             out["dequantize"] = deq
+
+        # ---------------- between decode and prefill: 16 ... 64 rows on matrices with few tiles (K cut over the grid)
+        if want("mid_m"):
+            mid = []
+            for c, n, k, m in (("q4_k", 4096, 4096, 16), ("q4_k", 4096, 4096, 64), ("q4_k", 14336, 4096, 32),
+                               ("q6_k", 4096, 4096, 16), ("q8_0", 4096, 4096, 64), ("q2_k", 4096, 4096, 64)):
+                wb = n * kq.bytes_per_row(c, k)
+                wq = synth_wire_torch(c, n, k, 11, dev)
+                cps = cold_copies(torch, wq, wb)
+                xm = randx((m, k))
+                t, _ = time_calls(torch, [abi.qmm(xm, w, c, n, k) for w in cps], 200, 20)
+                mid.append({"codec": c, "N": n, "K": k, "M": m, "us": round(t * 1e3, 2),
+                            "tflops": round(2.0 * m * n * k / (t * 1e-3) / 1e12, 1),
+                            "cold_gbs": round(wb / (t * 1e-3) / 1e9, 1)})
+                del cps, wq
+            out["mid_m"] = mid
+
+        # ---------------- transpose = 0 (reduction over wire rows): MLA-shaped gathered entries and dense calls
+        if want("no_transpose"):
+            nt = []
+            for c in ("q4_k", "q8_0"):
+                E, k, n = 128, 128, 512
+                wq = synth_wire_torch(c, E * k, n, 13, dev)
+                rhs = torch.arange(E, dtype=torch.int32, device=dev)
+                for m in (1, 64):
+                    t, _ = time_calls(torch, [abi.gather_nt(randx((E, m, k)), wq, c, rhs, E, k, n)], 200, 20)
+                    nt.append({"codec": c, "entries": E, "M": m, "K": k, "N": n, "us": round(t * 1e3, 2)})
+                del wq
+            for m in (1, 32, 512):
+                k = n = 4096
+                wq = synth_wire_torch("q4_k", k, n, 14, dev)
+                t, _ = time_calls(torch, [abi.qmm_nt(randx((m, k)), wq, "q4_k", k, n)], 200, 20)
+                nt.append({"codec": "q4_k", "entries": 1, "M": m, "K": k, "N": n, "us": round(t * 1e3, 2),
+                           "tflops": round(2.0 * m * n * k / (t * 1e-3) / 1e12, 1)})
+                del wq
+            out["no_transpose"] = nt
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(base_np, codec, K, M)
