@@ -31,6 +31,10 @@ typedef uint32_t u32_a1 __attribute__((aligned(1)));  // the hardware serves una
 
 constexpr int NT_WAVES = 4, NT_THREADS = 64 * NT_WAVES;
 constexpr int NT_KSTEP = 32, NT_COLS = 128;
+// Codecs whose 32-row form does not fit 256 registers (it spills up to 248 bytes per lane) take 64-row tiles on one
+// wave per SIMD beyond 32 rows (q6_k 4096 x 4096, 512 rows: 292 -> 146 us); for the others the 64-row form measured
+// level or slower (q8_0 93 -> 111 us).
+constexpr bool nt_wide(int codec) { return codec == KQ_Q6_K; }
 
 struct NtArgs {
   const void* x;
@@ -72,9 +76,10 @@ struct NtGeom {
   static constexpr int STAGE_BYTES = NT_WAVES * NT_KSTEP * STRIDE;
 };
 
-// MR = 16-row groups of activations per workgroup (1: up to 16 rows, 2: 32)
+// MR = 16-row groups of activations per workgroup (1: up to 16 rows, 2: 32, 4: 64 rows on one wave per SIMD, for
+// calls of many rows: every decoded weight then feeds four MFMAs)
 template <int C, int DT, int MR>
-__global__ __launch_bounds__(NT_THREADS, 2) void gemm_nt_mfma_kernel(NtArgs a, const uint8_t* __restrict__ grids) {
+__global__ __launch_bounds__(NT_THREADS, MR == 4 ? 1 : 2) void gemm_nt_mfma_kernel(NtArgs a, const uint8_t* __restrict__ grids) {
   using G = NtGeom<C>;
   constexpr int BPB = G::BPB, GPB = G::GPB, PDW = G::PDW, STRIDE = G::STRIDE, NDW = G::NDW;
   constexpr int RED_BYTES = 2 * 32 * MR * 64 * 4;  // two waves' accumulators; shares the space of the staging areas
@@ -290,7 +295,7 @@ __global__ __launch_bounds__(256) void nt_reduce_kernel(const float* __restrict_
 
 // K ranges of a dense call: enough workgroups for two per CU, at least eight steps each
 int nt_ksplit(int M, int N, int K) {
-  const int mr = M <= 16 ? 1 : 2;
+  const int mr = M <= 16 ? 1 : 2;  // (the 64-row form of nt_wide codecs halves the tiles: the plan stays on the safe side)
   const int64_t tiles = (int64_t)((N + NT_COLS - 1) / NT_COLS) * ((M + 16 * mr - 1) / (16 * mr));
   const int steps = (K + NT_KSTEP - 1) / NT_KSTEP;
   if (tiles >= 256 || steps < 16) return 1;
@@ -313,10 +318,13 @@ struct NtRun {
     }
   }
   static int run(const NtArgs& a, int B, int dt, const uint8_t* grids, hipStream_t s) {
-    if (a.M <= 16)
+    if (a.M <= 16) {
       dt == KQ_F16 ? go<KQ_F16, 1>(a, B, grids, s) : go<KQ_BF16, 1>(a, B, grids, s);
-    else
+    } else if (nt_wide(C) && a.M > 32) {
+      if constexpr (nt_wide(C)) dt == KQ_F16 ? go<KQ_F16, 4>(a, B, grids, s) : go<KQ_BF16, 4>(a, B, grids, s);
+    } else {
       dt == KQ_F16 ? go<KQ_F16, 2>(a, B, grids, s) : go<KQ_BF16, 2>(a, B, grids, s);
+    }
     KQ_HIP_CHECK(hipGetLastError());
     return KQ_OK;
   }
