@@ -96,9 +96,11 @@ size_t kq_stream_workspace_bytes(int M, int N, int K, int codec);
 int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                          size_t ws_bytes, hipStream_t s);
 // Gathered matvec (MoE decode, one activation row per entry) on the streamed kernel; UNSUPPORTED -> older kernels.
-int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* rhs, void* out,
-                            int entries, int N, int K, int x_div, int64_t w_expert_stride, int act, float limit,
-                            int codec, int dtype, int E, KqOutMap om, hipStream_t s);
+// Entry p reads activation row p / x_div of x, or (lhs != null) the row at x + lhs[p] * x_row_stride.
+int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs, const uint32_t* rhs,
+                            void* out, int entries, int N, int K, int x_div, int64_t x_row_stride,
+                            int64_t w_expert_stride, int act, float limit, int codec, int dtype, int E, KqOutMap om,
+                            hipStream_t s);
 // Tuned gathered GEMV (items = (activation matrix, expert) pairs, M <= 8 rows each; with glu the
 // gate/up pair and the fused epilogue, M = 1): same fall-through contract as kq_launch_qmm_tuned.
 // The per-entry gather launchers take the stack height E and skip entries whose expert id is >= E.

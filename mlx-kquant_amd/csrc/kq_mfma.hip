@@ -1423,11 +1423,12 @@ int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, c
                            const uint32_t* rhs, void* out, int B, int M, int N, int K, int x_div,
                            int64_t x_batch_stride, int64_t w_expert_stride, int glu, int act, float limit, int codec,
                            int dtype, int E, KqOutMap om, hipStream_t s) {
-  // one activation row per entry, entries in order of x (MoE decode): the streamed kernel, which also takes the
-  // codebook codecs it has units for
-  if (M == 1 && !lhs && rhs && x_batch_stride == K && g_sk_variant == 0 && B >= 1 && (!glu || act != KQ_ACT_SWIGLU_CLAMP)) {
-    const int rcs = kq_launch_gather_stream(x, w, glu ? w2 : nullptr, rhs, out, B, N, K, x_div, w_expert_stride, act, limit,
-                                            codec, dtype, E, om, s);
+  // one activation row per entry (MoE decode: entries in order of x; gather_qmm: any row index): the streamed
+  // kernel, which also takes the codebook codecs it has units for
+  if (M == 1 && rhs && (lhs || x_batch_stride == K) && g_sk_variant == 0 && B >= 1 &&
+      (!glu || act != KQ_ACT_SWIGLU_CLAMP)) {
+    const int rcs = kq_launch_gather_stream(x, w, glu ? w2 : nullptr, lhs, rhs, out, B, N, K, x_div, x_batch_stride,
+                                            w_expert_stride, act, limit, codec, dtype, E, om, s);
     if (rcs != KQ_ERR_UNSUPPORTED) return rcs;
   }
   if (!sk_shape_ok(M, K, codec, x, w, w2) || B < 1 || B > 65535) return KQ_ERR_UNSUPPORTED;

@@ -220,6 +220,8 @@ struct StArgs {
   // out_row(om, p); entries whose expert id is >= E are skipped
   const uint8_t* w2;
   const uint32_t* rhs;
+  const uint32_t* lhs;     // null, or the entry's activation row: x + lhs[p] * x_row_stride (x_div is then unused)
+  int64_t x_row_stride;
   int tiles_per_entry, x_div, E, act;
   float limit;
   int64_t w_expert_stride;
@@ -766,7 +768,10 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   const int nu = UPS * (sbn > wave ? (sbn - wave + ST_WAVES - 1) / ST_WAVES : 0);  // wave-uniform, 0..XU
 
   // ---- activation loads first: they are the oldest loads of the wave
-  const uint16_t* x16 = static_cast<const uint16_t*>(a.x) + (GM ? (size_t)(g_entry / a.x_div) * K : 0);
+  const uint16_t* x16 = static_cast<const uint16_t*>(a.x);
+  if constexpr (GM != 0)
+    x16 += a.lhs ? (size_t)__builtin_amdgcn_readfirstlane((int)a.lhs[g_entry]) * (size_t)a.x_row_stride
+                 : (size_t)(g_entry / a.x_div) * K;
   // codebook codecs: threads 0 .. 127 fetch 16 bytes each of the 2 KiB grid the tables are built from
   u32x4 greg = {0, 0, 0, 0};
   // replicated iq2_xxs tables: the sixteen lanes of a quarter wave write the sixteen copies of one entry (a wave
@@ -1394,9 +1399,10 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
 #ifndef KQ_GATHER_STREAM_MAX_ENTRIES
 #define KQ_GATHER_STREAM_MAX_ENTRIES 256
 #endif
-int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* rhs, void* out,
-                            int entries, int N, int K, int x_div, int64_t w_expert_stride, int act, float limit,
-                            int codec, int dtype, int E, KqOutMap om, hipStream_t s) {
+int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs, const uint32_t* rhs,
+                            void* out, int entries, int N, int K, int x_div, int64_t x_row_stride,
+                            int64_t w_expert_stride, int act, float limit, int codec, int dtype, int E, KqOutMap om,
+                            hipStream_t s) {
   if (!st_codec_ok(codec)) return KQ_ERR_UNSUPPORTED;
   if (entries < 1 || entries > KQ_GATHER_STREAM_MAX_ENTRIES || N < 1 || K < 256 || (K & 255) || !rhs) return KQ_ERR_UNSUPPORTED;
   const bool glu = w2 != nullptr;
@@ -1404,13 +1410,16 @@ int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, 
   if ((int64_t)entries * ((N + ST_ROWS - 1) / ST_ROWS) > 65535 * 16) return KQ_ERR_UNSUPPORTED;
   const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : 1;
   if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
-      ((uintptr_t)w_expert_stride & wmask) || (reinterpret_cast<uintptr_t>(x) & 15) || ((K * 2) & 15))
+      ((uintptr_t)w_expert_stride & wmask) || (reinterpret_cast<uintptr_t>(x) & 15) || ((K * 2) & 15) ||
+      (lhs && ((x_row_stride * 2) & 15)))
     return KQ_ERR_UNSUPPORTED;
   StArgs a{};
   a.x = x;
   a.w = w;
   a.w2 = w2;
   a.rhs = rhs;
+  a.lhs = lhs;
+  a.x_row_stride = x_row_stride;
   a.y = out;
   a.M = 1;
   a.N = N;

@@ -316,12 +316,22 @@ def quantized_matmul_qmv_bias(x, w, scales, bias, kquant_type, *, stream=None):
     return out
 
 
+_ARANGE = {}
+
+
 def _default_indices(t):
+    """0 .. (batch entries - 1) in the batch shape of t; the tensors are constants and are kept per (device, count)."""
     shape = t.shape[:-2]
     total = 1
     for d in shape:
         total *= d
-    return torch.arange(total, dtype=torch.int64, device=t.device).reshape(shape)
+    key = (str(t.device), total)
+    a = _ARANGE.get(key)
+    if a is None:
+        if len(_ARANGE) > 64:
+            _ARANGE.clear()
+        a = _ARANGE[key] = torch.arange(total, dtype=torch.int32, device=t.device)
+    return a.reshape(shape)
 
 
 class _GatherQmmFn(torch.autograd.Function):
@@ -383,8 +393,8 @@ def _gather_qmm_impl(x, w, kquant_type, lhs_indices, rhs_indices, transpose, sor
     rhs = rhs_indices if rhs_indices is not None else _default_indices(w)
     lhs, rhs = torch.broadcast_tensors(lhs, rhs)
     idx_shape = list(lhs.shape)
-    lhs = lhs.to(torch.int64).reshape(-1).to(torch.int32).contiguous()  # uint32 bit pattern
-    rhs = rhs.to(torch.int64).reshape(-1).to(torch.int32).contiguous()
+    lhs = _prep_idx(lhs).reshape(-1)  # uint32 bit pattern
+    rhs = _prep_idx(rhs).reshape(-1)
     M = x.shape[-2]
     x_c = x.to(out_type).reshape(-1, M, K).contiguous()
     # the expert (leading) dim of w may be strided; rows inside one expert must be packed
@@ -496,6 +506,11 @@ def _check_kq_expert_stack(op, w, kquant_type, K):
 
 
 def _prep_idx(idx):
+    """Index tensor as the contiguous uint32 bit pattern the ABI reads; int32 / uint32 inputs cost no kernel."""
+    if idx.dtype == torch.int32:
+        return idx.contiguous()
+    if idx.dtype == torch.uint32:
+        return idx.contiguous().view(torch.int32)
     return idx.to(torch.int64).to(torch.int32).contiguous()
 
 
