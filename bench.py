@@ -620,7 +620,7 @@ def main():
                     t, _ = time_calls(torch, [abi.gather_nt(randx((E, m, k)), wq, c, rhs, E, k, n)], 200, 20)
                     nt.append({"codec": c, "entries": E, "M": m, "K": k, "N": n, "us": round(t * 1e3, 2)})
                 del wq
-            for m in (1, 32, 512):
+            for m in (1, 32, 512, 2048):
                 k = n = 4096
                 wq = synth_wire_torch("q4_k", k, n, 14, dev)
                 t, _ = time_calls(torch, [abi.qmm_nt(randx((m, k)), wq, "q4_k", k, n)], 200, 20)

@@ -18,7 +18,8 @@
 // of K in turn and their accumulators meet in LDS.  A wave copies the 32 row pieces of its step (the wire bytes of
 // the tile's columns, contiguous per row; for the 256-weight codecs the whole superblock, which two column tiles
 // share) into its own LDS area with dword loads issued one step ahead, and the decoders read the bytes from there:
-// decoding straight from global memory costs about 130 byte-wide loads a step.
+// decoding straight from global memory costs about 130 byte-wide loads a step.  Calls of 96 rows and more run
+// gemm_nt_wide_kernel below, which decodes a step once for 128 activation rows.
 #include <type_traits>
 
 #include "kq_decode.h"
@@ -35,6 +36,11 @@ constexpr int NT_KSTEP = 32, NT_COLS = 128;
 // wave per SIMD beyond 32 rows (q6_k 4096 x 4096, 512 rows: 292 -> 146 us); for the others the 64-row form measured
 // level or slower (q8_0 93 -> 111 us).
 constexpr bool nt_wide(int codec) { return codec == KQ_Q6_K; }
+// Calls of this many activation rows take the kernel that decodes a step once for 128 rows
+#ifndef KQ_NT_SHARED_ROWS
+#define KQ_NT_SHARED_ROWS 96
+#endif
+constexpr int NT_SHARED_ROWS = KQ_NT_SHARED_ROWS;
 
 struct NtArgs {
   const void* x;
@@ -271,6 +277,184 @@ __global__ __launch_bounds__(NT_THREADS, MR == 4 ? 1 : 2) void gemm_nt_mfma_kern
   }
 }
 
+// Many activation rows: 128 (MRW = 2) or 256 (MRW = 4) rows x 128 columns per workgroup.  Every wave owns a quarter
+// of the rows and the four walk the
+// K steps together, so the 4096 weights of a step are decoded ONCE per workgroup instead of once per 32 rows: wave w
+// decodes rows 8w ... 8w + 7 of the step's 32 (lane (c, part): rows 8w + 2 part, + 1 of column group c), writes them
+// as packed bf16 pairs where the MFMA operands of all four waves lie (LDS, [k group h][t][c] x 16 bytes, hi and lo
+// planes), and after one barrier every wave reads its 16 operands back.  Staging and operand buffers are double:
+// one barrier per step.
+template <int C, int DT, int MRW>
+__global__ __launch_bounds__(NT_THREADS, 2) void gemm_nt_wide_kernel(NtArgs a, const uint8_t* __restrict__ grids) {
+  using G = NtGeom<C>;
+  constexpr int BPB = G::BPB, GPB = G::GPB, PDW = G::PDW, STRIDE = G::STRIDE;
+  constexpr int STG = NT_KSTEP * STRIDE;               // one staging buffer: the step's 32 row pieces
+  constexpr int NDWW = (NT_KSTEP * PDW + NT_THREADS - 1) / NT_THREADS;  // dwords a thread copies per step
+  constexpr int PLANE = 4 * 8 * 16 * 16;               // one operand plane: [h][t][c] x 16 bytes
+  constexpr int OPB = 2 * PLANE;                       // hi + lo
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STG + 2 * OPB];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 15, h = lane >> 4;  // h: k group as operand reader, row pair as decoder
+  const int item = a.ksplit > 1 ? 0 : blockIdx.z, split = a.ksplit > 1 ? blockIdx.z : 0;
+  const uint32_t e = a.rhs ? a.rhs[item] : 0u;
+  if (e >= (uint32_t)a.E) return;  // the whole workgroup leaves: the entry's output rows stay untouched
+  const int tile = blockIdx.x;
+  const int ngroups = a.N / 8;
+  const int gi = tile * 16 + c;
+  const bool col_ok = gi < ngroups;
+  const size_t row_bytes = (size_t)(a.N / G::WPB) * BPB;
+  const int pi = G::SUPER ? tile >> 1 : tile;
+  const int gp = (col_ok ? gi : ngroups - 1) - pi * (G::PCOLS / 8);
+  const uint8_t* wt = a.w + (size_t)e * (size_t)a.w_expert_stride + (size_t)pi * G::PIECE;
+  const int cols_here = a.N - G::PCOLS * pi < G::PCOLS ? a.N - G::PCOLS * pi : G::PCOLS;
+  const int piece_here = cols_here / G::WPB * BPB;
+  const int blk_off = (gp / GPB) * BPB + (8 * wave + 2 * h) * STRIDE;  // this lane's first row inside a staging buffer
+  const int g = gp % GPB, klast = a.K - 1;
+  const int m0 = blockIdx.y * (64 * MRW) + 16 * MRW * wave;
+  const uint16_t* xr[MRW];
+#pragma unroll
+  for (int q = 0; q < MRW; q++) {
+    const int mrow = m0 + 16 * q + c < a.M ? m0 + 16 * q + c : a.M - 1;
+    xr[q] = static_cast<const uint16_t*>(a.x) + (a.lhs ? (size_t)a.lhs[item] * (size_t)a.x_batch_stride : 0) +
+            (size_t)mrow * a.K;
+  }
+  f32x4 acc[MRW][8];
+#pragma unroll
+  for (int q = 0; q < MRW; q++)
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc[q][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  uint32_t wreg[NDWW], xreg[MRW][4];
+  auto fetch = [&](int st) {  // as in gemm_nt_mfma_kernel, the step's pieces spread over the whole workgroup
+#pragma unroll
+    for (int j = 0; j < NDWW; j++) {
+      const int idx = tid + NT_THREADS * j < NT_KSTEP * PDW ? tid + NT_THREADS * j : NT_KSTEP * PDW - 1;
+      const int row = idx / PDW, boff = 4 * (idx - row * PDW);
+      const int eoff = boff < piece_here - 4 ? boff : piece_here - 4;
+      const int k = NT_KSTEP * st + row < a.K ? NT_KSTEP * st + row : klast;
+      const uint32_t v = *reinterpret_cast<const u32_a1*>(wt + (size_t)k * row_bytes + eoff);
+      wreg[j] = v >> (8 * ((boff - eoff) & 3));
+    }
+    const int k0 = NT_KSTEP * st + 8 * h;
+#pragma unroll
+    for (int q = 0; q < MRW; q++) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) xreg[q][j] = 0u;
+      if (a.x_vec) {
+        const uint4 v = *reinterpret_cast<const uint4*>(xr[q] + (k0 < a.K ? k0 : 0));
+        const bool in = k0 < a.K;
+        xreg[q][0] = in ? v.x : 0u, xreg[q][1] = in ? v.y : 0u, xreg[q][2] = in ? v.z : 0u, xreg[q][3] = in ? v.w : 0u;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+          if (k0 + i < a.K) xreg[q][i >> 1] |= (uint32_t)xr[q][k0 + i] << (16 * (i & 1));
+      }
+    }
+  };
+  auto park = [&](uint8_t* stage) {
+#pragma unroll
+    for (int j = 0; j < NDWW; j++) {
+      const int idx = tid + NT_THREADS * j;
+      if (idx < NT_KSTEP * PDW) *reinterpret_cast<uint32_t*>(stage + 4 * idx) = wreg[j];
+    }
+  };
+
+  const int steps_all = (a.K + NT_KSTEP - 1) / NT_KSTEP;
+  const int st_begin = split * a.steps_per_split;
+  const int nsteps = st_begin + a.steps_per_split < steps_all ? st_begin + a.steps_per_split : steps_all;
+  if (st_begin < nsteps) {
+    fetch(st_begin);
+    park(lds);
+  }
+  for (int st = st_begin; st < nsteps; st++) {
+    const int b = (st - st_begin) & 1;
+    const uint8_t* stage = lds + b * STG;
+    uint8_t* opnd = lds + 2 * STG + b * OPB;
+    bf16x8 ah[MRW], al[MRW];
+#pragma unroll
+    for (int q = 0; q < MRW; q++) {
+      if constexpr (DT == KQ_BF16) {
+        ah[q] = __builtin_bit_cast(bf16x8, make_uint4(xreg[q][0], xreg[q][1], xreg[q][2], xreg[q][3]));
+      } else {
+        uint32_t hi[4], lo[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const float f0 = kq::h2f((uint16_t)(xreg[q][j] & 0xffffu)), f1 = kq::h2f((uint16_t)(xreg[q][j] >> 16));
+          hi[j] = pack_hi(f0, f1);
+          lo[j] = pack_hi(f0 - trunc_bf16(f0), f1 - trunc_bf16(f1));
+        }
+        ah[q] = __builtin_bit_cast(bf16x8, make_uint4(hi[0], hi[1], hi[2], hi[3]));
+        al[q] = __builtin_bit_cast(bf16x8, make_uint4(lo[0], lo[1], lo[2], lo[3]));
+      }
+    }
+    if (st == st_begin) __syncthreads();  // the first staging buffer is complete (later ones: the barrier below)
+    if (st + 1 < nsteps) fetch(st + 1);
+    {  // decode this lane's two rows and put them where the operands lie
+      float w0[8], w1[8];
+      kq::decode8<C>(stage + blk_off, g, grids, w0);
+      kq::decode8<C>(stage + blk_off + STRIDE, g, grids, w1);
+      uint8_t* dst = opnd + ((wave * 8) * 16 + c) * 16 + 4 * h;
+#pragma unroll
+      for (int t = 0; t < 8; t++) {
+        *reinterpret_cast<uint32_t*>(dst + t * 256) = pack_hi(w0[t], w1[t]);
+        *reinterpret_cast<uint32_t*>(dst + t * 256 + PLANE) =
+            pack_rne(w0[t] - trunc_bf16(w0[t]), w1[t] - trunc_bf16(w1[t]));
+      }
+    }
+    if (st + 1 < nsteps) park(lds + (b ^ 1) * STG);
+    __syncthreads();  // operands of this step are complete; the other staging buffer is written
+    const uint8_t* src = opnd + ((h * 8) * 16 + c) * 16;
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      const bf16x8 wh = *reinterpret_cast<const bf16x8*>(src + t * 256);
+      const bf16x8 wl = *reinterpret_cast<const bf16x8*>(src + t * 256 + PLANE);
+#pragma unroll
+      for (int q = 0; q < MRW; q++) {
+        acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[q], wh, acc[q][t], 0, 0, 0);
+        acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[q], wl, acc[q][t], 0, 0, 0);
+        if constexpr (DT == KQ_F16) acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[q], wh, acc[q][t], 0, 0, 0);
+      }
+    }
+  }
+
+  if (!col_ok) return;
+  if (a.ksplit > 1) {
+    float* pb = a.part + (size_t)split * a.M * a.N + 8 * (size_t)gi;
+#pragma unroll
+    for (int q = 0; q < MRW; q++) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int m = m0 + 16 * q + 4 * h + r;
+        if (m < a.M) {
+          float4* o = reinterpret_cast<float4*>(pb + (size_t)m * a.N);
+          o[0] = make_float4(acc[q][0][r], acc[q][1][r], acc[q][2][r], acc[q][3][r]);
+          o[1] = make_float4(acc[q][4][r], acc[q][5][r], acc[q][6][r], acc[q][7][r]);
+        }
+      }
+    }
+    return;
+  }
+  uint16_t* yb = static_cast<uint16_t*>(a.y) + (size_t)item * a.M * a.N + 8 * (size_t)gi;
+#pragma unroll
+  for (int q = 0; q < MRW; q++) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int m = m0 + 16 * q + 4 * h + r;
+      if (m < a.M) {
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const float v0 = acc[q][2 * j][r], v1 = acc[q][2 * j + 1][r];
+          const uint16_t lo = DT == KQ_F16 ? kq::f2f16(v0) : kq::f2bf16(v0);
+          const uint16_t hi = DT == KQ_F16 ? kq::f2f16(v1) : kq::f2bf16(v1);
+          o[j] = (uint32_t)lo | ((uint32_t)hi << 16);
+        }
+        *reinterpret_cast<uint4*>(yb + (size_t)m * a.N) = make_uint4(o[0], o[1], o[2], o[3]);
+      }
+    }
+  }
+}
+
 // y[i] = sum over the K ranges of part[s][i], 8 outputs per thread, ranges added in order
 template <int DT>
 __global__ __launch_bounds__(256) void nt_reduce_kernel(const float* __restrict__ part, void* __restrict__ y,
@@ -295,8 +479,8 @@ __global__ __launch_bounds__(256) void nt_reduce_kernel(const float* __restrict_
 
 // K ranges of a dense call: enough workgroups for two per CU, at least eight steps each
 int nt_ksplit(int M, int N, int K) {
-  const int mr = M <= 16 ? 1 : 2;  // (the 64-row form of nt_wide codecs halves the tiles: the plan stays on the safe side)
-  const int64_t tiles = (int64_t)((N + NT_COLS - 1) / NT_COLS) * ((M + 16 * mr - 1) / (16 * mr));
+  const int rows = M <= 16 ? 16 : M < NT_SHARED_ROWS ? 32 : 128;  // activation rows per workgroup
+  const int64_t tiles = (int64_t)((N + NT_COLS - 1) / NT_COLS) * ((M + rows - 1) / rows);
   const int steps = (K + NT_KSTEP - 1) / NT_KSTEP;
   if (tiles >= 256 || steps < 16) return 1;
   int s = (int)((512 + tiles - 1) / tiles);
@@ -317,8 +501,22 @@ struct NtRun {
                          groups, a.ksplit);
     }
   }
+  template <int DT>
+  static void go_shared(const NtArgs& a, int B, const uint8_t* grids, hipStream_t s) {
+    // (256-row tiles, MRW = 4, measured slower: 316 against 223 us at 2048 rows of 4096 x 4096 q4_k; their 212 - 250
+    // registers leave two workgroups per CU where the 128-row form runs three)
+    dim3 grid((a.N + NT_COLS - 1) / NT_COLS, (a.M + 127) / 128, a.ksplit > 1 ? a.ksplit : B);
+    hipLaunchKernelGGL((gemm_nt_wide_kernel<C, DT, 2>), grid, dim3(NT_THREADS), 0, s, a, grids);
+    if (a.ksplit > 1) {
+      const size_t groups = (size_t)a.M * a.N / 8;
+      hipLaunchKernelGGL((nt_reduce_kernel<DT>), dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s, a.part, a.y,
+                         groups, a.ksplit);
+    }
+  }
   static int run(const NtArgs& a, int B, int dt, const uint8_t* grids, hipStream_t s) {
-    if (a.M <= 16) {
+    if (a.M >= NT_SHARED_ROWS) {
+      dt == KQ_F16 ? go_shared<KQ_F16>(a, B, grids, s) : go_shared<KQ_BF16>(a, B, grids, s);
+    } else if (a.M <= 16) {
       dt == KQ_F16 ? go<KQ_F16, 1>(a, B, grids, s) : go<KQ_BF16, 1>(a, B, grids, s);
     } else if (nt_wide(C) && a.M > 32) {
       if constexpr (nt_wide(C)) dt == KQ_F16 ? go<KQ_F16, 4>(a, B, grids, s) : go<KQ_BF16, 4>(a, B, grids, s);

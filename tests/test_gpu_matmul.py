@@ -174,6 +174,10 @@ def test_qmm_no_transpose_every_codec_on_the_matrix_cores(kq, codec):
               (3, 16, 1280, "float16", 4)]
     if codec in ("q4_k", "q6_k", "q8_0", "iq3_s", "mxfp4"):  # long K, few tiles: the K range is cut over the grid
         shapes += [(3, 1024, 256, "float16", 6), (20, 1000, 256, "bfloat16", 7)]
+    # 96 rows and more: the kernel that decodes a step once per 128 rows (ragged rows, odd step counts, K cut)
+    shapes += [(100, 72, 256, "bfloat16", 8), (200, 33, 512, "float16", 9)]
+    if codec in ("q4_k", "q6_k", "q8_0", "iq2_xxs", "nvfp4"):
+        shapes.append((130, 1056, 256, "bfloat16", 10))
     if O.geometry(codec)[0] == 32:
         shapes.append((2, 70, 352, "bfloat16", 5))
     for (M, K, N, dtype, seed) in shapes:
@@ -183,6 +187,18 @@ def test_qmm_no_transpose_every_codec_on_the_matrix_cores(kq, codec):
         want = O.qmm(xb, wire, codec, False, dtype)
         assert tuple(got.shape) == (M, N)
         assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, K, N, dtype)
+
+
+@pytest.mark.parametrize("codec,M,K,N,dtype", [("q4_k", 2048, 64, 4096, "bfloat16"), ("q8_0", 2100, 40, 4096, "float16"),
+                                               ("q6_k", 2050, 96, 4096, "bfloat16")])
+def test_qmm_no_transpose_many_rows(kq, codec, M, K, N, dtype):
+    """transpose=False with thousands of activation rows (a ragged last row tile, a ragged last K step)."""
+    wire = _wire(codec, K, N, seed=90)
+    xb, xt = make_x((M, K), dtype, seed=91)
+    got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec, transpose=False)
+    want = O.qmm(xb, wire, codec, False, dtype)
+    assert tuple(got.shape) == (M, N)
+    assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, M, K, N, dtype)
 
 
 def test_qmm_dtype_rules_and_shapes(kq):
