@@ -100,6 +100,22 @@ def test_gather_qmm_no_transpose(kq, codec):
     assert rel_l2(dev_to_bits(got), want, "float16") <= TOL
 
 
+@pytest.mark.parametrize("codec", ["q4_k", "q8_0", "iq3_s"])
+def test_gather_qmm_no_transpose_many_rows_per_entry(kq, codec):
+    """transpose=False with 100 activation rows per entry (the kernel that shares a step's decode over 128 rows),
+    repeated lhs rows and an expert id outside the stack (that entry's rows stay untouched)."""
+    E, K, N, B, M = 3, 48, 512, 5, 100
+    wire = _stack(codec, E, K, N, seed=146)
+    xb, xt = make_x((B, M, K), "bfloat16", seed=147)
+    lhs, rhs = np.array([4, 0, 0, 2, 1]), np.array([2, 0, 7, 1, 1])
+    out = kq.gather_qmm(xt, wire_to_dev(wire), None, codec, lhs_indices=_idx_dev(lhs), rhs_indices=_idx_dev(rhs),
+                        transpose=False)
+    keep = [0, 1, 3, 4]
+    want = O.gather_qmm(xb, wire, codec, lhs[keep], rhs[keep], False, "bfloat16")
+    assert tuple(out.shape) == (B, M, N)
+    assert rel_l2(dev_to_bits(out[keep]), want, "bfloat16") <= TOL
+
+
 def test_gather_qmm_reference_moe_fixture_and_strided_experts(kq):
     wire = np.load(os.path.join(GOLD, "q4_k_moe.npz"))["wire"]  # [4, 128, 288]
     E, N, K, B = 4, 128, 512, 64
