@@ -173,7 +173,7 @@ def test_qmm_no_transpose_every_codec_on_the_matrix_cores(kq, codec):
     shapes = [(1, 128, 512, "bfloat16", 1), (5, 50, 768, "float16", 2), (40, 27, 256, "bfloat16", 3),
               (3, 16, 1280, "float16", 4)]
     if codec in ("q4_k", "q6_k", "q8_0", "iq3_s", "mxfp4"):  # long K, few tiles: the K range is cut over the grid
-        shapes += [(3, 1024, 256, "float16", 6), (20, 1000, 256, "bfloat16", 7)]
+        shapes += [(3, 1024, 256, "float16", 6), (20, 1000, 256, "bfloat16", 7), (2, 1001, 256, "bfloat16", 11)]
     # 96 rows and more: the kernel that decodes a step once per 128 rows (ragged rows, odd step counts, K cut)
     shapes += [(100, 72, 256, "bfloat16", 8), (200, 33, 512, "float16", 9)]
     if codec in ("q4_k", "q6_k", "q8_0", "iq2_xxs", "nvfp4"):
