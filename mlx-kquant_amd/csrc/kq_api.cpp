@@ -239,7 +239,8 @@ size_t kq_gather_qmm_workspace_size(int B, int M, int E, int N, int K, int trans
 static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
                            const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
                            int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
-                           size_t ws_bytes, KqOutMap om, hipStream_t s);
+                           size_t ws_bytes, KqOutMap om, hipStream_t s, int entry_rows = 1);
+static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int N, int K);
 
 int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_dev, const uint32_t* rhs_idx_dev,
                   void* out_dev, int B, int M, int E, int N, int K, int64_t x_batch_stride,
@@ -267,6 +268,7 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
   // many output rows: gather them into a dense matrix and run the expert-grouped kernels
   int64_t P;
   if (workspace_dev && gather_batched_shape(B, M, E, N, K, transpose, codec, &P) &&
+      !per_entry_route(P, M, false, 0, 0, codec, N, K) &&
       !(reinterpret_cast<uintptr_t>(workspace_dev) & 255) && !(reinterpret_cast<uintptr_t>(x_dev) & 15) &&
       !(x_batch_stride & 7)) {
     const size_t need = kq_gather_qmm_workspace_size(B, M, E, N, K, transpose, codec, dtype);
@@ -279,7 +281,7 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
       if (rcr) return rcr;
       const int rcg = try_moe_grouped("gather_qmm", xg, w_dev, nullptr, idx_rows, nullptr, nullptr, out_dev, (int)P, 1, E,
                                       N, K, w_expert_stride_bytes, 0, 0, 0.f, 0.f, codec, dtype, wsb + used,
-                                      workspace_bytes - used, KQ_OUT_ROWS, s);
+                                      workspace_bytes - used, KQ_OUT_ROWS, s, M);
       if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
     }
   }
@@ -349,26 +351,32 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 #ifndef KQ_PER_ENTRY_MAX_PAIRS_IQ
 #define KQ_PER_ENTRY_MAX_PAIRS_IQ 64
 #endif
-static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
-                           const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
-                           int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
-                           size_t ws_bytes, KqOutMap om, hipStream_t s) {
-  const int64_t P = (int64_t)T * R;
-  if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
-  // few entries: the per-entry kernels (the caller tries them next) beat the prologue + grouped-kernel pair
+// True when a call of P (token, expert) pairs is better served entry by entry than by the sorted, expert-grouped
+// kernels.  entry_rows = activation rows per entry of the caller's per-entry fallback (1 for the MoE ops; gather_qmm's
+// M): the per-entry kernels take one row per entry, the older K-quant ones up to eight.
+static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int N, int K) {
+  if (P <= 16) return false;  // the callers never reach the grouped route with so few pairs
   const bool grouped_codec = codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K;
   const bool low_codec = codec == KQ_Q2_K || codec == KQ_Q3_K;  // their batched route is the any-codec kernel
   const bool iq_codec = codec == KQ_IQ4_XS || codec == KQ_IQ3_S || codec == KQ_IQ2_XXS;
   // the other codecs' per-entry kernel is the code-level one, which takes biases and every activation
-  const bool codes_codec = !grouped_codec && !low_codec && !iq_codec;
-  if (codes_codec && P > 16 && P <= (codec == KQ_NVFP4 ? KQ_PER_ENTRY_MAX_PAIRS_NVFP4 : KQ_PER_ENTRY_MAX_PAIRS_CODES) &&
-      kq_codes_gather_supported(1, N, K, codec))
-    return KQ_ERR_UNSUPPORTED;
-  if (P > 16 && !bias && !bias2 &&
-      ((grouped_codec && P <= KQ_PER_ENTRY_MAX_PAIRS) || (low_codec && P <= KQ_PER_ENTRY_MAX_PAIRS_LOW) ||
-       (iq_codec && P <= KQ_PER_ENTRY_MAX_PAIRS_IQ)) &&
-      (!glu || act != KQ_ACT_SWIGLU_CLAMP) && (K >> 8) <= (glu ? 16 : 32) && (K & 255) == 0)
-    return KQ_ERR_UNSUPPORTED;
+  if (!grouped_codec && !low_codec && !iq_codec)
+    return entry_rows == 1 && P <= (codec == KQ_NVFP4 ? KQ_PER_ENTRY_MAX_PAIRS_NVFP4 : KQ_PER_ENTRY_MAX_PAIRS_CODES) &&
+           kq_codes_gather_supported(1, N, K, codec);
+  if (has_bias || (glu && act == KQ_ACT_SWIGLU_CLAMP) || (K >> 8) > (glu ? 16 : 32) || (K & 255)) return false;
+  if (grouped_codec) return P <= KQ_PER_ENTRY_MAX_PAIRS && entry_rows <= 8;
+  return entry_rows == 1 && P <= (low_codec ? KQ_PER_ENTRY_MAX_PAIRS_LOW : KQ_PER_ENTRY_MAX_PAIRS_IQ);
+}
+
+static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
+                           const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
+                           int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
+                           size_t ws_bytes, KqOutMap om, hipStream_t s, int entry_rows) {
+  // entry_rows: activation rows per entry of the CALLER's per-entry fallback (1 for the MoE ops; gather_qmm's M)
+  const int64_t P = (int64_t)T * R;
+  if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
+  // few entries: the per-entry kernels (the caller tries them next) beat the prologue + grouped-kernel pair
+  if (per_entry_route(P, entry_rows, bias || bias2, glu, act, codec, N, K)) return KQ_ERR_UNSUPPORTED;
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
     // legacy / IQ / fp4 codecs (biases and every activation included): code-level grouped kernel
     if (kq_codes_moe_supported((int)P, E, N, K, codec)) {

@@ -70,6 +70,22 @@ def test_gather_qmm_batched(kq, codec, M):
         assert rel_l2(dev_to_bits(got).reshape(B, M, N), want, dtype) <= TOL, (codec, M, dtype)
 
 
+@pytest.mark.parametrize("codec", ["q4_k", "q2_k", "iq4_xs", "mxfp4", "nvfp4", "q8_0"])
+@pytest.mark.parametrize("B,M", [(10, 3), (3, 12)])
+def test_gather_qmm_few_entries_of_several_rows(kq, codec, B, M):
+    """17 ... 48 output rows made of entries with several activation rows each: the one-row-per-entry kernels do not
+    apply, whatever the pair count says."""
+    E, N, K = 5, 136, 512 if codec not in ("mxfp4", "nvfp4") else 320
+    wire = _stack(codec, E, N, K, seed=161)
+    rng = np.random.default_rng(162)
+    lhs, rhs = rng.integers(0, B, B), rng.integers(0, E, B)
+    xb, xt = make_x((B, M, K), "bfloat16", seed=163, scale=0.5)
+    got = kq.gather_qmm(xt, wire_to_dev(wire), None, codec, lhs_indices=_idx_dev(lhs), rhs_indices=_idx_dev(rhs))
+    want = O.gather_qmm(xb, wire, codec, lhs, rhs, True, "bfloat16")
+    assert tuple(got.shape) == (B, M, N)
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, B, M)
+
+
 @pytest.mark.parametrize("codec", ["q4_k", "q6_k", "q2_k", "q8_0"])
 def test_single_entry_picks_its_expert(kq, codec):
     """A gathered call of ONE entry must still honour its expert index (it must not take the dense-call
