@@ -348,6 +348,11 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 #ifndef KQ_PER_ENTRY_MAX_PAIRS_NVFP4
 #define KQ_PER_ENTRY_MAX_PAIRS_NVFP4 128
 #endif
+// q8_0: the streamed per-entry kernel against the code-level grouped kernel (same stacks, us: 32 pairs 21.0 + 15.0
+// against 38.8 + 23.2, 64 pairs 38.8 + 28.0 against 55.7 + 36.8, 128 pairs 74.3 + 53.0 against 71.4 + 48.6).
+#ifndef KQ_PER_ENTRY_MAX_PAIRS_Q8
+#define KQ_PER_ENTRY_MAX_PAIRS_Q8 64
+#endif
 #ifndef KQ_PER_ENTRY_MAX_PAIRS_IQ
 #define KQ_PER_ENTRY_MAX_PAIRS_IQ 64
 #endif
@@ -359,13 +364,15 @@ static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, i
   const bool grouped_codec = codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K;
   const bool low_codec = codec == KQ_Q2_K || codec == KQ_Q3_K;  // their batched route is the any-codec kernel
   const bool iq_codec = codec == KQ_IQ4_XS || codec == KQ_IQ3_S || codec == KQ_IQ2_XXS;
+  const bool q8 = codec == KQ_Q8_0;  // per-entry kernel: the streamed one; batched: the code-level grouped kernel
   // the other codecs' per-entry kernel is the code-level one, which takes biases and every activation
-  if (!grouped_codec && !low_codec && !iq_codec)
+  if (!grouped_codec && !low_codec && !iq_codec && !q8)
     return entry_rows == 1 && P <= (codec == KQ_NVFP4 ? KQ_PER_ENTRY_MAX_PAIRS_NVFP4 : KQ_PER_ENTRY_MAX_PAIRS_CODES) &&
            kq_codes_gather_supported(1, N, K, codec);
   if (has_bias || (glu && act == KQ_ACT_SWIGLU_CLAMP) || (K >> 8) > (glu ? 16 : 32) || (K & 255)) return false;
   if (grouped_codec) return P <= KQ_PER_ENTRY_MAX_PAIRS && entry_rows <= 8;
-  return entry_rows == 1 && P <= (low_codec ? KQ_PER_ENTRY_MAX_PAIRS_LOW : KQ_PER_ENTRY_MAX_PAIRS_IQ);
+  return entry_rows == 1 &&
+         P <= (low_codec ? KQ_PER_ENTRY_MAX_PAIRS_LOW : q8 ? KQ_PER_ENTRY_MAX_PAIRS_Q8 : KQ_PER_ENTRY_MAX_PAIRS_IQ);
 }
 
 static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,

@@ -1269,8 +1269,9 @@ int kq_launch_codes_skinny(const void* x, const uint8_t* w, const void* bias, vo
 #if !defined(KQ_CODES_PART) || KQ_CODES_PART == 2
 // Gathered calls of up to a few entries (MoE decode): one activation row per entry (M = 1), the entry's expert
 // matrix, optional f32 biases; glu != 0 runs gate and up stacks and the fused epilogue.
-// (q8_0 stays on the plain vector kernel: int8 -> f32 costs it next to nothing, and it measured 9.1 / 8.4 us
-// against 12.7 / 9.0 us here for the GLU / down ops of 8 experts of 768 x 2048.)
+// (q8_0 entries are not taken here: the streamed kernel has a q8_0 unit, and where that declines - a K that is no
+// multiple of 256 - the plain vector kernel measured 9.1 / 8.4 us against 12.7 / 9.0 us here for the GLU / down ops
+// of 8 experts of 768 x 2048.)
 bool kq_codes_gather_supported(int M, int N, int K, int codec) {
   return M == 1 && codec != KQ_Q8_0 && kq_codes_supported(M, N, K, codec);
 }

@@ -24,7 +24,8 @@
 // magnitudes, sign index -> eight sign masks; iq3_s: 9-bit grid index -> four magnitudes, sign byte -> eight sign
 // masks).  These kernels are bound by the LDS once the table reads of a wave meet in a bank, so the one-row
 // kernels spend their spare LDS on that: a copy of the table per bank group (iq4_xs, iq2_xxs) or entries with the
-// signs already applied (iq3_s).
+// signs already applied (iq3_s).  q8_0 (eight 34-byte blocks per unit row) needs no table: a byte permute and one
+// exact packed subtraction turn a quant byte into its f16 value.
 //
 // Waiting.  The compiler cannot see a direct-to-LDS load land, so these loads are issued from inline
 // assembly and every wait on them is an explicit s_waitcnt vmcnt(n): loads return in order, n is the
@@ -156,6 +157,12 @@ struct StGeom<KQ_IQ3_S> {
   static constexpr int BPB = 110, PP = 7, LBPB = 112, NAP = 4, XSG = 8;
   static constexpr bool SIDE_D = true;
 };
+//   q8_0: a "superblock" is eight 34-byte blocks (272 bytes), copied as they lie
+template <>
+struct StGeom<KQ_Q8_0> {
+  static constexpr int BPB = 272, PP = 17, LBPB = 272, NAP = 4, XSG = 4;
+  static constexpr bool SIDE_D = false;
+};
 // block byte of the f16 d that travels on its own (SIDE_D)
 template <int C>
 constexpr uint32_t st_side_d_off() { return C == KQ_Q6_K ? 208u : 0u; }
@@ -173,7 +180,7 @@ __device__ __forceinline__ uint32_t st_piece_off(int p) {
 // leave a 32-bit word in), 1 = k0 k1 k2 k3 (codebook entries), 2 = x[j], x[j + 16] interleaved over 32 (iq4_xs: a
 // byte holds weights j and j + 16 of its sub-block).
 template <int C>
-constexpr int st_xord() { return C == KQ_IQ4_XS ? 2 : C == KQ_IQ2_XXS || C == KQ_IQ3_S ? 1 : 0; }
+constexpr int st_xord() { return C == KQ_IQ4_XS ? 2 : C == KQ_IQ2_XXS || C == KQ_IQ3_S || C == KQ_Q8_0 ? 1 : 0; }
 // LDS bytes of the decode tables a workgroup builds for itself
 //   iq4_xs:  [256][32] byte -> f16 pair (kvalues[low nibble], kvalues[high nibble]), one copy per LDS bank: lane l
 //            reads copy l % 32, so the 64 data-dependent reads of an instruction never meet in a bank (with a single
@@ -432,6 +439,58 @@ __device__ __forceinline__ void q23k_unit(const uint8_t* __restrict__ bl, int kg
         acc[r] = fmaf(mul[sl], p[r / 4][r % 4], acc[r]);
         acc[r] = fmaf(-sub[sl], xs[r][sl], acc[r]);
       });
+    });
+  });
+}
+
+// ------------------------------------------------------------------ q8_0 unit
+// Lane (row, kg) owns blocks 4 kg .. 4 kg + 3 of the row's eight: 136 bytes at 136 kg, read as 34 dwords.  A block
+// at an even position has its quants 2 bytes past a dword boundary (realigned with v_alignbyte), an odd one on it.
+// A quant byte b becomes the f16 1024 + (b ^ 0x80) = q + 1152 by a byte permute, and the exact packed subtraction of
+// 1152 leaves q.  MFMA (ib, q): weights 4 q .. 4 q + 3 of block ib; activations = A pair ib, block q.
+template <int R, int AS>
+__device__ __forceinline__ void q80_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
+                                         float* acc) {
+  constexpr int RG = (R + 3) / 4;
+  typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
+  const uint8_t* p8 = bl + 136 * kg;
+  uint32_t w[34];
+#pragma unroll
+  for (int i = 0; i < 17; i++) {
+    const u32x2 v = *reinterpret_cast<const u32x2*>(p8 + 8 * i);
+    w[2 * i] = v.x;
+    w[2 * i + 1] = v.y;
+  }
+  const uint32_t flip = opaque_sgpr(0x80808080u), magic = opaque_vgpr(0x64646464u);
+  const f16x2v off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+  SFor<4>::run([&](auto ii) {
+    constexpr int ib = decltype(ii)::value;
+    // byte offset of block ib inside the 136: 34 ib -> dword 8.5 ib
+    constexpr int d0 = (34 * ib) / 4;            // dword holding d
+    constexpr bool even = (ib & 1) == 0;         // d in the low half of dword d0, quants straddle dwords
+    const float dl = kq::h2f((uint16_t)(even ? (w[d0] & 0xffffu) : (w[d0] >> 16))) * xscale;
+    f32x4 p[RG];
+#pragma unroll
+    for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
+    SFor<8>::run([&](auto qq) {
+      constexpr int q = decltype(qq)::value;
+      uint32_t qd;
+      if constexpr (even)
+        qd = __builtin_amdgcn_alignbyte(w[d0 + q + 1], w[d0 + q], 2);
+      else
+        qd = w[d0 + 1 + q];
+      qd ^= flip;
+      u32x2 bv;
+      bv.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2v, __builtin_amdgcn_perm(magic, qd, 0x04010400u)) + off);
+      bv.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2v, __builtin_amdgcn_perm(magic, qd, 0x04030402u)) + off);
+#pragma unroll
+      for (int g = 0; g < RG; g++)
+        p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, areg[g * AS + ib]),
+                                                  __builtin_bit_cast(f16x4, bv), p[g], 3, q, 0);
+    });
+    SFor<R>::run([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      acc[r] = fmaf(dl, p[r / 4][r % 4], acc[r]);
     });
   });
 }
@@ -962,7 +1021,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         int koff;  // in f16 elements inside the half
         if constexpr (C == KQ_Q6_K)
           koff = 32 * (pr >> 1) + 16 * (pr & 1) + 4 * (fa >> 1);
-        else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K || st_tbl_bytes<C>() != 0)
+        else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K || C == KQ_Q8_0 || st_tbl_bytes<C>() != 0)
           koff = 32 * pr + 4 * fa;
         else
           koff = 64 * (pr >> 1) + 32 * (fa & 1) + 16 * (pr & 1) + 4 * (fa >> 1);
@@ -1098,6 +1157,8 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
           q6k_unit<R, AS>(bl, dx, kg, areg + us * NAP, xsum + us * 16, ST_XU * 16, acc);
         } else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) {
           q23k_unit<C, R, AS>(bl, kg, xscale, areg + us * NAP, xsum + us * 16, ST_XU * 16, acc);
+        } else if constexpr (C == KQ_Q8_0) {
+          q80_unit<R, AS>(bl, kg, xscale, areg + us * NAP, acc);
         } else if constexpr (C == KQ_IQ4_XS) {
           iq4xs_unit<R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc);
         } else if constexpr (C == KQ_IQ2_XXS) {
@@ -1202,7 +1263,8 @@ int st_max_sb(int codec, int M);
 // rows, the codecs with small units for up to four)
 template <int C>
 constexpr int st_nw8_rows() {
-  return st_lds_bytes<C, 4, 2, 4, 8>() <= 160 * 1024 ? 4 : st_lds_bytes<C, 2, 2, 4, 8>() <= 160 * 1024 ? 2 : 0;
+  return st_lds_bytes<C, 4, 2, 4, 8>() <= 160 * 1024 ? 4 : st_lds_bytes<C, 2, 2, 4, 8>() <= 160 * 1024 ? 2 :
+         st_lds_bytes<C, 1, 2, 4, 8>() <= 160 * 1024 ? 1 : 0;
 }
 int st_max_sb(int codec, int M) {
   if (!g_st_nw8) return 16;
@@ -1216,6 +1278,7 @@ int st_max_sb(int codec, int M) {
     case KQ_IQ4_XS: rows = st_nw8_rows<KQ_IQ4_XS>(); break;
     case KQ_IQ2_XXS: rows = st_nw8_rows<KQ_IQ2_XXS>(); break;
     case KQ_IQ3_S: rows = st_nw8_rows<KQ_IQ3_S>(); break;
+    case KQ_Q8_0: rows = st_nw8_rows<KQ_Q8_0>(); break;
   }
   return M <= rows ? 32 : 16;
 }
@@ -1287,8 +1350,10 @@ int st_launch_m(const StArgs& a, int splits, hipStream_t s) {
   if (a.sb_per_split > 16) {
     // K ranges of 17 .. 32 superblocks: eight waves of four units (st_max_sb allows this for up to four rows).
     // Four waves of eight units, the alternative without more waves, took 9.0 instead of 7.1 us on q2_k 8192^2.
-    if (a.M == 1) return st_launch_one<C, DT, 1, D, 4, 8>(a, splits, s);
-    if (a.M == 2) return st_launch_one<C, DT, 2, D, 4, 8>(a, splits, s);
+    if constexpr (st_nw8_rows<C>() >= 1)
+      if (a.M == 1) return st_launch_one<C, DT, 1, D, 4, 8>(a, splits, s);
+    if constexpr (st_nw8_rows<C>() >= 2)
+      if (a.M == 2) return st_launch_one<C, DT, 2, D, 4, 8>(a, splits, s);
     if constexpr (st_nw8_rows<C>() >= 4) return st_launch_one<C, DT, 4, D, 4, 8>(a, splits, s);
   }
   if (a.M == 1) return st_launch_one<C, DT, 1, D, 4>(a, splits, s);
@@ -1323,13 +1388,21 @@ template <int C, int DT>
 int st_launch_gather_nw(const StArgs& a, int entries, bool glu, hipStream_t s) {
   const int nsb = a.K >> 8;
   // gate / up pair: two units per superblock; beyond four superblocks eight waves keep a wave at two to four units
-  if (glu) return nsb <= 4 ? st_launch_gather<C, DT, 4, 2>(a, entries, s) : st_launch_gather<C, DT, 8, 2>(a, entries, s);
-  return nsb <= 16 ? st_launch_gather<C, DT, 4, 1>(a, entries, s) : st_launch_gather<C, DT, 8, 1>(a, entries, s);
+  // (a codec whose eight-wave workgroup does not fit the LDS stays on four waves as far as their units reach)
+  if (glu) {
+    if (nsb <= 4) return st_launch_gather<C, DT, 4, 2>(a, entries, s);
+    if constexpr (st_lds_bytes<C, 1, 2, 4, 8, 2>() <= 160 * 1024) return st_launch_gather<C, DT, 8, 2>(a, entries, s);
+    if (nsb <= 8) return st_launch_gather<C, DT, 4, 2>(a, entries, s);
+    return KQ_ERR_UNSUPPORTED;
+  }
+  if (nsb <= 16) return st_launch_gather<C, DT, 4, 1>(a, entries, s);
+  if constexpr (st_lds_bytes<C, 1, 2, 4, 8, 1>() <= 160 * 1024) return st_launch_gather<C, DT, 8, 1>(a, entries, s);
+  return KQ_ERR_UNSUPPORTED;
 }
 
 bool st_codec_ok(int codec) {
   return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K || codec == KQ_Q2_K || codec == KQ_Q3_K ||
-         codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S;
+         codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S || codec == KQ_Q8_0;
 }
 
 }  // namespace
@@ -1338,7 +1411,7 @@ bool st_codec_ok(int codec) {
 #if !defined(KQ_STREAM_PART) || KQ_STREAM_PART == 1
 bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const void* w) {
   if (!st_codec_ok(codec) || M < 1 || M > 8 || N < 1 || K < 256 || (K & 255)) return false;
-  if ((int64_t)N * (K >> 8) * 210 >= (int64_t)1 << 40) return false;
+  if ((int64_t)N * (K >> 8) * 272 >= (int64_t)1 << 40) return false;
   // q4_k / q5_k pieces are fetched 16-byte aligned; iq4_xs blocks are 8-byte multiples, q2_k blocks 4-byte ones, the
   // others 2-byte ones
   const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : 1;
@@ -1383,6 +1456,8 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
       return dtype == KQ_F16 ? st_launch_m<KQ_IQ4_XS, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_IQ4_XS, KQ_BF16>(a, p.ksplit, s);
     return dtype == KQ_F16 ? st_launch_m<KQ_IQ2_XXS, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_IQ2_XXS, KQ_BF16>(a, p.ksplit, s);
   }
+  if (codec == KQ_Q8_0)
+    return dtype == KQ_F16 ? st_launch_m<KQ_Q8_0, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q8_0, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q2_K)
     return dtype == KQ_F16 ? st_launch_m<KQ_Q2_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q2_K, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q3_K)
@@ -1442,7 +1517,7 @@ int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, 
     return dtype == KQ_F16 ? st_launch_gather_nw<c, KQ_F16>(a, entries, glu, s)       \
                            : st_launch_gather_nw<c, KQ_BF16>(a, entries, glu, s);
     KQ_CASE(KQ_Q2_K) KQ_CASE(KQ_Q3_K) KQ_CASE(KQ_Q4_K) KQ_CASE(KQ_Q5_K) KQ_CASE(KQ_Q6_K) KQ_CASE(KQ_IQ4_XS)
-    KQ_CASE(KQ_IQ3_S) KQ_CASE(KQ_IQ2_XXS)
+    KQ_CASE(KQ_IQ3_S) KQ_CASE(KQ_IQ2_XXS) KQ_CASE(KQ_Q8_0)
 #undef KQ_CASE
   }
   return KQ_ERR_UNSUPPORTED;
