@@ -353,6 +353,12 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 #ifndef KQ_PER_ENTRY_MAX_PAIRS_Q8
 #define KQ_PER_ENTRY_MAX_PAIRS_Q8 64
 #endif
+// iq4_nl / q4_0 / mxfp4 calls the streamed kernel takes (no biases, no swiglu_clamp, K a multiple of 256), against the
+// code-level grouped kernel (same stacks, us: mxfp4 32 pairs 20.2 + 16.5 against 37.4 + 22.7, 64 pairs 37.2 + 30.1
+// against 50.1 + 30.5, 96 pairs 54.5 + 43.7 against 58.3 + 37.3; q4_0 64 pairs 33.3 + 28.3 against 48.0 + 25.8).
+#ifndef KQ_PER_ENTRY_MAX_PAIRS_NIB
+#define KQ_PER_ENTRY_MAX_PAIRS_NIB 64
+#endif
 #ifndef KQ_PER_ENTRY_MAX_PAIRS_IQ
 #define KQ_PER_ENTRY_MAX_PAIRS_IQ 64
 #endif
@@ -365,11 +371,17 @@ static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, i
   const bool low_codec = codec == KQ_Q2_K || codec == KQ_Q3_K;  // their batched route is the any-codec kernel
   const bool iq_codec = codec == KQ_IQ4_XS || codec == KQ_IQ3_S || codec == KQ_IQ2_XXS;
   const bool q8 = codec == KQ_Q8_0;  // per-entry kernel: the streamed one; batched: the code-level grouped kernel
+  const bool streamed_shape =
+      !(has_bias || (glu && act == KQ_ACT_SWIGLU_CLAMP) || (K >> 8) > (glu ? 16 : 32) || (K & 255));
+  // iq4_nl / q4_0 / mxfp4 entries the streamed kernel takes; the others fall to the code-level rule below
+  if ((codec == KQ_IQ4_NL || codec == KQ_Q4_0 || codec == KQ_MXFP4) && streamed_shape && entry_rows == 1 &&
+      P <= KQ_PER_ENTRY_MAX_PAIRS_NIB)
+    return true;
   // the other codecs' per-entry kernel is the code-level one, which takes biases and every activation
   if (!grouped_codec && !low_codec && !iq_codec && !q8)
     return entry_rows == 1 && P <= (codec == KQ_NVFP4 ? KQ_PER_ENTRY_MAX_PAIRS_NVFP4 : KQ_PER_ENTRY_MAX_PAIRS_CODES) &&
            kq_codes_gather_supported(1, N, K, codec);
-  if (has_bias || (glu && act == KQ_ACT_SWIGLU_CLAMP) || (K >> 8) > (glu ? 16 : 32) || (K & 255)) return false;
+  if (!streamed_shape) return false;
   if (grouped_codec) return P <= KQ_PER_ENTRY_MAX_PAIRS && entry_rows <= 8;
   return entry_rows == 1 &&
          P <= (low_codec ? KQ_PER_ENTRY_MAX_PAIRS_LOW : q8 ? KQ_PER_ENTRY_MAX_PAIRS_Q8 : KQ_PER_ENTRY_MAX_PAIRS_IQ);

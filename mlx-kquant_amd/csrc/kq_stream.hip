@@ -1,4 +1,5 @@
-// Streamed skinny-M (decode) kernel: y[M,N] = x[M,K] . W^T for M <= 8, codecs q2_k ... q6_k, iq4_xs, iq3_s, iq2_xxs.
+// Streamed skinny-M (decode) kernel: y[M,N] = x[M,K] . W^T for M <= 8, codecs q2_k ... q6_k, iq4_xs, iq3_s, iq2_xxs,
+// q8_0, iq4_nl, q4_0, mxfp4 (the 32-weight-block codecs with K a multiple of 256).
 // The weight bytes go HBM -> LDS with direct-to-LDS loads (global_load_lds_dwordx4): no staging
 // registers, no LDS store instructions, and a wave keeps its next units in flight while it works.
 //
@@ -25,7 +26,9 @@
 // masks).  These kernels are bound by the LDS once the table reads of a wave meet in a bank, so the one-row
 // kernels spend their spare LDS on that: a copy of the table per bank group (iq4_xs, iq2_xxs) or entries with the
 // signs already applied (iq3_s).  q8_0 (eight 34-byte blocks per unit row) needs no table: a byte permute and one
-// exact packed subtraction turn a quant byte into its f16 value.
+// exact packed subtraction turn a quant byte into its f16 value.  iq4_nl, q4_0 and mxfp4 (eight 18- or 17-byte blocks
+// per unit row, a quant byte holding weights j and j + 16 of its block) share the iq4_xs table with their own sixteen
+// values in it.
 //
 // Waiting.  The compiler cannot see a direct-to-LDS load land, so these loads are issued from inline
 // assembly and every wait on them is an explicit s_waitcnt vmcnt(n): loads return in order, n is the
@@ -163,6 +166,26 @@ struct StGeom<KQ_Q8_0> {
   static constexpr int BPB = 272, PP = 17, LBPB = 272, NAP = 4, XSG = 4;
   static constexpr bool SIDE_D = false;
 };
+//   iq4_nl / q4_0 (eight 18-byte blocks = 144 bytes, copied as they lie) and mxfp4 (eight 17-byte blocks = 136
+//   bytes, the last piece starting at 120 like q2_k's): a byte holds weights j and j + 16 of its block, as in iq4_xs
+template <>
+struct StGeom<KQ_IQ4_NL> {
+  static constexpr int BPB = 144, PP = 9, LBPB = 144, NAP = 4, XSG = 8;
+  static constexpr bool SIDE_D = false;
+};
+template <>
+struct StGeom<KQ_Q4_0> {
+  static constexpr int BPB = 144, PP = 9, LBPB = 144, NAP = 4, XSG = 8;
+  static constexpr bool SIDE_D = false;
+};
+template <>
+struct StGeom<KQ_MXFP4> {
+  static constexpr int BPB = 136, PP = 9, LBPB = 144, NAP = 4, XSG = 8;
+  static constexpr bool SIDE_D = false;
+};
+// codecs decoded through the byte -> f16 pair table (one copy per LDS bank)
+template <int C>
+constexpr bool st_pair_table() { return C == KQ_IQ4_XS || C == KQ_IQ4_NL || C == KQ_Q4_0 || C == KQ_MXFP4; }
 // block byte of the f16 d that travels on its own (SIDE_D)
 template <int C>
 constexpr uint32_t st_side_d_off() { return C == KQ_Q6_K ? 208u : 0u; }
@@ -170,7 +193,8 @@ constexpr uint32_t st_side_d_off() { return C == KQ_Q6_K ? 208u : 0u; }
 template <int C>
 __device__ __forceinline__ uint32_t st_piece_off(int p) {
   using G = StGeom<C>;
-  if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) return p == G::PP - 1 ? (uint32_t)(G::BPB - 16) : 16u * (uint32_t)p;
+  if constexpr (C == KQ_Q2_K || C == KQ_Q3_K || C == KQ_MXFP4)
+    return p == G::PP - 1 ? (uint32_t)(G::BPB - 16) : 16u * (uint32_t)p;
   if constexpr (C == KQ_IQ4_XS) return p == 0 ? 0u : 16u * (uint32_t)p - 8u;
   if constexpr (C == KQ_IQ2_XXS) return p == 0 ? 0u : 16u * (uint32_t)p - 14u;
   if constexpr (C == KQ_IQ3_S) return p == 6 ? 94u : 16u * (uint32_t)p + 2u;
@@ -180,7 +204,7 @@ __device__ __forceinline__ uint32_t st_piece_off(int p) {
 // leave a 32-bit word in), 1 = k0 k1 k2 k3 (codebook entries), 2 = x[j], x[j + 16] interleaved over 32 (iq4_xs: a
 // byte holds weights j and j + 16 of its sub-block).
 template <int C>
-constexpr int st_xord() { return C == KQ_IQ4_XS ? 2 : C == KQ_IQ2_XXS || C == KQ_IQ3_S || C == KQ_Q8_0 ? 1 : 0; }
+constexpr int st_xord() { return st_pair_table<C>() ? 2 : C == KQ_IQ2_XXS || C == KQ_IQ3_S || C == KQ_Q8_0 ? 1 : 0; }
 // LDS bytes of the decode tables a workgroup builds for itself
 //   iq4_xs:  [256][32] byte -> f16 pair (kvalues[low nibble], kvalues[high nibble]), one copy per LDS bank: lane l
 //            reads copy l % 32, so the 64 data-dependent reads of an instruction never meet in a bank (with a single
@@ -200,7 +224,7 @@ constexpr int st_iq2_copies() { return C == KQ_IQ2_XXS && MB == 1 && NW == 8 && 
 // (gathered launches, whose workgroups live for one to four units, keep the plain iq2_xxs / iq3_s tables)
 template <int C, int MB = 0, int NW = 0, int GM = 0>
 constexpr int st_tbl_bytes() {
-  return C == KQ_IQ4_XS ? 32768 : C == KQ_IQ2_XXS ? (4096 + 2048) * st_iq2_copies<C, MB, NW, GM>() :
+  return st_pair_table<C>() ? 32768 : C == KQ_IQ2_XXS ? (4096 + 2048) * st_iq2_copies<C, MB, NW, GM>() :
          st_iq3s_merged<C, MB, NW, GM>() ? 65536 + 4096 : C == KQ_IQ3_S ? 4096 + 4096 : 0;
 }
 template <int C>
@@ -538,6 +562,80 @@ __device__ __forceinline__ void iq4xs_unit(const uint8_t* __restrict__ bl, int k
     });
     const int ls = (int)(((sl >> (4 * ib)) & 15) | (((sh >> (2 * ib)) & 3) << 4));
     const float dl = d * (float)(ls - 32);
+    SFor<R>::run([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      acc[r] = fmaf(dl, p[r / 4][r % 4], acc[r]);
+    });
+  });
+}
+
+// ------------------------------------------------------------------ iq4_nl / q4_0 / mxfp4 unit
+// Lane (row, kg) owns blocks 4 kg .. 4 kg + 3 of the row's eight (18 or 17 bytes each: scale, then 16 bytes whose
+// byte j holds weights j and j + 16).  The blocks' bytes are read as dwords and the 16 quant bytes of a block are
+// brought onto dword boundaries with v_alignbyte; everything else is the iq4_xs unit: table read per byte, MFMA
+// (ib, q) on bytes 2 q, 2 q + 1 of block ib, block scale on the partial sum.
+template <int C, int R, int AS>
+__device__ __forceinline__ void nib32_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
+                                           const uint8_t* __restrict__ tbl, float* acc) {
+  constexpr int RG = (R + 3) / 4;
+  constexpr int BB = C == KQ_MXFP4 ? 17 : 18;   // block bytes
+  constexpr int HB = C == KQ_MXFP4 ? 1 : 2;     // scale bytes in front of the quants
+  constexpr int NDW = 4 * BB / 4;               // 17 or 18 dwords per lane
+  uint32_t w[NDW + 1];
+  if constexpr (C == KQ_MXFP4) {
+    // LDS row: block bytes 0 .. 127 as they lie, bytes 120 .. 135 again at 128: this lane's bytes 68 kg .. 68 kg + 67
+    // are contiguous for kg = 0; for kg = 1 bytes 128 .. 135 sit at 136
+#pragma unroll
+    for (int i = 0; i < 15; i++) w[i] = *reinterpret_cast<const uint32_t*>(bl + 68 * kg + 4 * i);
+    w[15] = *reinterpret_cast<const uint32_t*>(bl + (kg ? 136 : 60));
+    w[16] = *reinterpret_cast<const uint32_t*>(bl + (kg ? 140 : 64));
+    w[17] = 0u;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 9; i++) {
+      const u32x2 v = *reinterpret_cast<const u32x2*>(bl + 72 * kg + 8 * i);
+      w[2 * i] = v.x;
+      w[2 * i + 1] = v.y;
+    }
+    w[18] = 0u;
+  }
+  u32x2 bv[4][8];
+  auto lookup = [&](auto ii) {
+    constexpr int ib = decltype(ii)::value;
+    constexpr int o = BB * ib + HB, base = o / 4, sh = o % 4;  // first quant byte of the block
+    uint32_t qv[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      qv[i] = sh == 0 ? w[base + i] : __builtin_amdgcn_alignbyte(w[base + i + 1], w[base + i], sh);
+    SFor<8>::run([&](auto qq) {
+      constexpr int q = decltype(qq)::value;
+      const uint32_t ww = qv[q >> 1];
+      const uint32_t i0 = (ww >> (16 * (q & 1))) & 0xff, i1 = (ww >> (16 * (q & 1) + 8)) & 0xff;
+      bv[ib][q].x = *reinterpret_cast<const uint32_t*>(tbl + 128 * i0);
+      bv[ib][q].y = *reinterpret_cast<const uint32_t*>(tbl + 128 * i1);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  lookup(std::integral_constant<int, 0>{});
+  SFor<4>::run([&](auto ii) {
+    constexpr int ib = decltype(ii)::value;
+    if constexpr (ib < 3) lookup(std::integral_constant<int, ib + 1>{});
+    f32x4 p[RG];
+#pragma unroll
+    for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
+    SFor<8>::run([&](auto qq) {
+      constexpr int q = decltype(qq)::value;
+#pragma unroll
+      for (int g = 0; g < RG; g++)
+        p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, areg[g * AS + ib]),
+                                                  __builtin_bit_cast(f16x4, bv[ib][q]), p[g], 3, q, 0);
+    });
+    constexpr int so = BB * ib;  // scale byte(s) of the block
+    float dl;
+    if constexpr (C == KQ_MXFP4)
+      dl = kq::e8m0_half((w[so / 4] >> (8 * (so % 4))) & 0xffu) * xscale;
+    else
+      dl = kq::h2f((uint16_t)((w[so / 4] >> (8 * (so % 4))) & 0xffffu)) * xscale;
     SFor<R>::run([&](auto rr) {
       constexpr int r = decltype(rr)::value;
       acc[r] = fmaf(dl, p[r / 4][r % 4], acc[r]);
@@ -1031,7 +1129,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   });
 
   // ---- decode tables of the codebook codecs (their grid bytes arrived with the activations)
-  if constexpr (C == KQ_IQ4_XS) {
+  if constexpr (st_pair_table<C>()) {
     // entry b = dwords 32 b .. 32 b + 31 (one copy per LDS bank).  Eight lanes write the 128 bytes of an entry, so
     // a wave store covers 1 KiB of consecutive LDS (entry-per-lane stores, 128 bytes apart, all meet in two banks)
     typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
@@ -1039,7 +1137,12 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) {
       const int b = 8 * (PER_WAVE * wave + i) + (lane >> 3);
-      const f16x2v e = {(_Float16)kq::kv_iq4nl(b & 15), (_Float16)kq::kv_iq4nl(b >> 4)};
+      auto val = [](int i) -> float {
+        if constexpr (C == KQ_MXFP4) return kq::kv_mxfp4(i);
+        else if constexpr (C == KQ_Q4_0) return (float)(i - 8);
+        else return kq::kv_iq4nl(i);
+      };
+      const f16x2v e = {(_Float16)val(b & 15), (_Float16)val(b >> 4)};
       const uint32_t ev = __builtin_bit_cast(uint32_t, e);
       *reinterpret_cast<u32x4*>(tbl + 128 * b + 16 * (lane & 7)) = u32x4{ev, ev, ev, ev};
     }
@@ -1161,6 +1264,8 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
           q80_unit<R, AS>(bl, kg, xscale, areg + us * NAP, acc);
         } else if constexpr (C == KQ_IQ4_XS) {
           iq4xs_unit<R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc);
+        } else if constexpr (C == KQ_IQ4_NL || C == KQ_Q4_0 || C == KQ_MXFP4) {
+          nib32_unit<C, R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc);
         } else if constexpr (C == KQ_IQ2_XXS) {
           constexpr int COP = st_iq2_copies<C, MB, NW, GM>();
           iq2xxs_unit<R, AS, COP>(bl, kg, xscale, areg + us * NAP, COP > 1 ? tbl + 16 * (lane & 15) : tbl, acc);
@@ -1279,6 +1384,9 @@ int st_max_sb(int codec, int M) {
     case KQ_IQ2_XXS: rows = st_nw8_rows<KQ_IQ2_XXS>(); break;
     case KQ_IQ3_S: rows = st_nw8_rows<KQ_IQ3_S>(); break;
     case KQ_Q8_0: rows = st_nw8_rows<KQ_Q8_0>(); break;
+    case KQ_IQ4_NL: rows = st_nw8_rows<KQ_IQ4_NL>(); break;
+    case KQ_Q4_0: rows = st_nw8_rows<KQ_Q4_0>(); break;
+    case KQ_MXFP4: rows = st_nw8_rows<KQ_MXFP4>(); break;
   }
   return M <= rows ? 32 : 16;
 }
@@ -1402,7 +1510,8 @@ int st_launch_gather_nw(const StArgs& a, int entries, bool glu, hipStream_t s) {
 
 bool st_codec_ok(int codec) {
   return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K || codec == KQ_Q2_K || codec == KQ_Q3_K ||
-         codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S || codec == KQ_Q8_0;
+         codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S || codec == KQ_Q8_0 || codec == KQ_IQ4_NL ||
+         codec == KQ_Q4_0 || codec == KQ_MXFP4;
 }
 
 }  // namespace
@@ -1414,7 +1523,7 @@ bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const vo
   if ((int64_t)N * (K >> 8) * 272 >= (int64_t)1 << 40) return false;
   // q4_k / q5_k pieces are fetched 16-byte aligned; iq4_xs blocks are 8-byte multiples, q2_k blocks 4-byte ones, the
   // others 2-byte ones
-  const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : 1;
+  const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : codec == KQ_MXFP4 ? 0 : 1;
   if (reinterpret_cast<uintptr_t>(w) & wmask) return false;
   return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 }
@@ -1458,6 +1567,12 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
   }
   if (codec == KQ_Q8_0)
     return dtype == KQ_F16 ? st_launch_m<KQ_Q8_0, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q8_0, KQ_BF16>(a, p.ksplit, s);
+  if (codec == KQ_IQ4_NL)
+    return dtype == KQ_F16 ? st_launch_m<KQ_IQ4_NL, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_IQ4_NL, KQ_BF16>(a, p.ksplit, s);
+  if (codec == KQ_Q4_0)
+    return dtype == KQ_F16 ? st_launch_m<KQ_Q4_0, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q4_0, KQ_BF16>(a, p.ksplit, s);
+  if (codec == KQ_MXFP4)
+    return dtype == KQ_F16 ? st_launch_m<KQ_MXFP4, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_MXFP4, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q2_K)
     return dtype == KQ_F16 ? st_launch_m<KQ_Q2_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q2_K, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q3_K)
@@ -1483,7 +1598,7 @@ int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, 
   const bool glu = w2 != nullptr;
   if ((K >> 8) > (glu ? 16 : 32) || (glu && act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
   if ((int64_t)entries * ((N + ST_ROWS - 1) / ST_ROWS) > 65535 * 16) return KQ_ERR_UNSUPPORTED;
-  const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : 1;
+  const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : codec == KQ_MXFP4 ? 0 : 1;
   if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
       ((uintptr_t)w_expert_stride & wmask) || (reinterpret_cast<uintptr_t>(x) & 15) || ((K * 2) & 15) ||
       (lhs && ((x_row_stride * 2) & 15)))
@@ -1517,7 +1632,7 @@ int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, 
     return dtype == KQ_F16 ? st_launch_gather_nw<c, KQ_F16>(a, entries, glu, s)       \
                            : st_launch_gather_nw<c, KQ_BF16>(a, entries, glu, s);
     KQ_CASE(KQ_Q2_K) KQ_CASE(KQ_Q3_K) KQ_CASE(KQ_Q4_K) KQ_CASE(KQ_Q5_K) KQ_CASE(KQ_Q6_K) KQ_CASE(KQ_IQ4_XS)
-    KQ_CASE(KQ_IQ3_S) KQ_CASE(KQ_IQ2_XXS) KQ_CASE(KQ_Q8_0)
+    KQ_CASE(KQ_IQ3_S) KQ_CASE(KQ_IQ2_XXS) KQ_CASE(KQ_Q8_0) KQ_CASE(KQ_IQ4_NL) KQ_CASE(KQ_Q4_0) KQ_CASE(KQ_MXFP4)
 #undef KQ_CASE
   }
   return KQ_ERR_UNSUPPORTED;

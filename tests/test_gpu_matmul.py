@@ -121,7 +121,8 @@ def test_qmm_skinny_both_variants(kq, codec):
         lib.kq_set_skinny_variant(0)
 
 
-@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k", "q2_k", "q3_k", "iq4_xs", "iq2_xxs", "iq3_s", "q8_0"])
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k", "q2_k", "q3_k", "iq4_xs", "iq2_xxs", "iq3_s", "q8_0", "iq4_nl",
+                                   "q4_0", "mxfp4"])
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
 def test_qmm_streamed_kernel_shapes(kq, codec, dtype):
     """The streamed kernel (default for up to eight rows of q4_k / q5_k / q6_k): one to eight rows (five and more
