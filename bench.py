@@ -561,13 +561,17 @@ def main():
                 del gate, up, down, calls_g, calls_d
             out["moe_decode_lowbit"] = dec
 
-        # ---------------- low-bit codecs (and q8_0), M = 1, 8192 -> 8192 (all minted by kq.quantize)
+        # ---------------- low-bit codecs (and q8_0, 4-bit block codecs), M = 1, 8192 -> 8192 (minted by kq.quantize)
         if want("lowbit"):
             lowbit = []
-            for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs", "q8_0"):
+            for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs", "q8_0", "q4_0", "iq4_nl", "mxfp4"):
                 n = k = 8192
                 wb = n * kq.bytes_per_row(c, k)
-                wq = quantized_weights(kq, torch, c, n, k, 7, dev, unique_rows=None if c in ("q2_k", "q3_k", "iq4_xs", "q8_0") else 512)
+                if c == "mxfp4":  # no encoder in the reference: random structurally valid wire
+                    wq = synth_wire_torch(c, n, k, 7, dev).reshape(n, -1)
+                else:
+                    wq = quantized_weights(kq, torch, c, n, k, 7, dev,
+                                           unique_rows=None if c in ("q2_k", "q3_k", "iq4_xs", "q8_0", "q4_0") else 512)
                 cps = cold_copies(torch, wq, wb)
                 t, _ = time_calls(torch, [abi.qmm(x.new_ones((1, k)), w, c, n, k) for w in cps], steps, warm)
                 lowbit.append({"codec": c, "N": n, "K": k, "M": 1, "us": round(t * 1e3, 2),
