@@ -564,10 +564,10 @@ def main():
         # ---------------- low-bit codecs (and q8_0, 4-bit block codecs), M = 1, 8192 -> 8192 (minted by kq.quantize)
         if want("lowbit"):
             lowbit = []
-            for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs", "q8_0", "q4_0", "iq4_nl", "mxfp4"):
+            for c in ("q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs", "q8_0", "q4_0", "iq4_nl", "mxfp4", "nvfp4"):
                 n = k = 8192
                 wb = n * kq.bytes_per_row(c, k)
-                if c == "mxfp4":  # no encoder in the reference: random structurally valid wire
+                if c in ("mxfp4", "nvfp4"):  # no encoder in the reference: random structurally valid wire
                     wq = synth_wire_torch(c, n, k, 7, dev).reshape(n, -1)
                 else:
                     wq = quantized_weights(kq, torch, c, n, k, 7, dev,

@@ -356,6 +356,11 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 // iq4_nl / q4_0 / mxfp4 calls the streamed kernel takes (no biases, no swiglu_clamp, K a multiple of 256), against the
 // code-level grouped kernel (same stacks, us: mxfp4 32 pairs 20.2 + 16.5 against 37.4 + 22.7, 64 pairs 37.2 + 30.1
 // against 50.1 + 30.5, 96 pairs 54.5 + 43.7 against 58.3 + 37.3; q4_0 64 pairs 33.3 + 28.3 against 48.0 + 25.8).
+// nvfp4 calls the streamed kernel takes, against the any-codec kernel (us: 128 pairs 71.6 + 58.4 entry by entry,
+// 160 pairs 87 + 72 against 187 + 92, 256 pairs 138 + 113 against 213 + 105); the streamed kernel stops at 256 entries.
+#ifndef KQ_PER_ENTRY_MAX_PAIRS_NVFP4_STREAMED
+#define KQ_PER_ENTRY_MAX_PAIRS_NVFP4_STREAMED 256
+#endif
 #ifndef KQ_PER_ENTRY_MAX_PAIRS_NIB
 #define KQ_PER_ENTRY_MAX_PAIRS_NIB 64
 #endif
@@ -373,10 +378,11 @@ static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, i
   const bool q8 = codec == KQ_Q8_0;  // per-entry kernel: the streamed one; batched: the code-level grouped kernel
   const bool streamed_shape =
       !(has_bias || (glu && act == KQ_ACT_SWIGLU_CLAMP) || (K >> 8) > (glu ? 16 : 32) || (K & 255));
-  // iq4_nl / q4_0 / mxfp4 entries the streamed kernel takes; the others fall to the code-level rule below
+  // iq4_nl / q4_0 / mxfp4 / nvfp4 entries the streamed kernel takes; the others fall to the code-level rule below
   if ((codec == KQ_IQ4_NL || codec == KQ_Q4_0 || codec == KQ_MXFP4) && streamed_shape && entry_rows == 1 &&
       P <= KQ_PER_ENTRY_MAX_PAIRS_NIB)
     return true;
+  if (codec == KQ_NVFP4 && streamed_shape && entry_rows == 1 && P <= KQ_PER_ENTRY_MAX_PAIRS_NVFP4_STREAMED) return true;
   // the other codecs' per-entry kernel is the code-level one, which takes biases and every activation
   if (!grouped_codec && !low_codec && !iq_codec && !q8)
     return entry_rows == 1 && P <= (codec == KQ_NVFP4 ? KQ_PER_ENTRY_MAX_PAIRS_NVFP4 : KQ_PER_ENTRY_MAX_PAIRS_CODES) &&

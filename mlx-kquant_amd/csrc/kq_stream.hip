@@ -1,5 +1,5 @@
 // Streamed skinny-M (decode) kernel: y[M,N] = x[M,K] . W^T for M <= 8, codecs q2_k ... q6_k, iq4_xs, iq3_s, iq2_xxs,
-// q8_0, iq4_nl, q4_0, mxfp4 (the 32-weight-block codecs with K a multiple of 256).
+// q8_0, iq4_nl, q4_0, mxfp4, nvfp4 (the 32- and 64-weight-block codecs with K a multiple of 256).
 // The weight bytes go HBM -> LDS with direct-to-LDS loads (global_load_lds_dwordx4): no staging
 // registers, no LDS store instructions, and a wave keeps its next units in flight while it works.
 //
@@ -28,7 +28,7 @@
 // signs already applied (iq3_s).  q8_0 (eight 34-byte blocks per unit row) needs no table: a byte permute and one
 // exact packed subtraction turn a quant byte into its f16 value.  iq4_nl, q4_0 and mxfp4 (eight 18- or 17-byte blocks
 // per unit row, a quant byte holding weights j and j + 16 of its block) share the iq4_xs table with their own sixteen
-// values in it.
+// values in it; nvfp4 (a byte = weights j and j + 8 of 16 with a scale of their own) does too.
 //
 // Waiting.  The compiler cannot see a direct-to-LDS load land, so these loads are issued from inline
 // assembly and every wait on them is an explicit s_waitcnt vmcnt(n): loads return in order, n is the
@@ -183,9 +183,18 @@ struct StGeom<KQ_MXFP4> {
   static constexpr int BPB = 136, PP = 9, LBPB = 144, NAP = 4, XSG = 8;
   static constexpr bool SIDE_D = false;
 };
+//   nvfp4: four 36-byte blocks of 64 weights (four e4m3 scales, then 8 bytes per 16 weights whose byte j holds
+//   weights j and j + 8 of its 16), 144 bytes copied as they lie
+template <>
+struct StGeom<KQ_NVFP4> {
+  static constexpr int BPB = 144, PP = 9, LBPB = 144, NAP = 4, XSG = 8;
+  static constexpr bool SIDE_D = false;
+};
 // codecs decoded through the byte -> f16 pair table (one copy per LDS bank)
 template <int C>
-constexpr bool st_pair_table() { return C == KQ_IQ4_XS || C == KQ_IQ4_NL || C == KQ_Q4_0 || C == KQ_MXFP4; }
+constexpr bool st_pair_table() {
+  return C == KQ_IQ4_XS || C == KQ_IQ4_NL || C == KQ_Q4_0 || C == KQ_MXFP4 || C == KQ_NVFP4;
+}
 // block byte of the f16 d that travels on its own (SIDE_D)
 template <int C>
 constexpr uint32_t st_side_d_off() { return C == KQ_Q6_K ? 208u : 0u; }
@@ -202,9 +211,11 @@ __device__ __forceinline__ uint32_t st_piece_off(int p) {
 }
 // Order of the staged f16 activations inside a group: 0 = k0 k2 k1 k3 per four (the order the masked-in-place codes
 // leave a 32-bit word in), 1 = k0 k1 k2 k3 (codebook entries), 2 = x[j], x[j + 16] interleaved over 32 (iq4_xs: a
-// byte holds weights j and j + 16 of its sub-block).
+// byte holds weights j and j + 16 of its sub-block), 3 = x[j], x[j + 8] interleaved over 16 (nvfp4).
 template <int C>
-constexpr int st_xord() { return st_pair_table<C>() ? 2 : C == KQ_IQ2_XXS || C == KQ_IQ3_S || C == KQ_Q8_0 ? 1 : 0; }
+constexpr int st_xord() {
+  return C == KQ_NVFP4 ? 3 : st_pair_table<C>() ? 2 : C == KQ_IQ2_XXS || C == KQ_IQ3_S || C == KQ_Q8_0 ? 1 : 0;
+}
 // LDS bytes of the decode tables a workgroup builds for itself
 //   iq4_xs:  [256][32] byte -> f16 pair (kvalues[low nibble], kvalues[high nibble]), one copy per LDS bank: lane l
 //            reads copy l % 32, so the 64 data-dependent reads of an instruction never meet in a bank (with a single
@@ -569,15 +580,25 @@ __device__ __forceinline__ void iq4xs_unit(const uint8_t* __restrict__ bl, int k
   });
 }
 
-// ------------------------------------------------------------------ iq4_nl / q4_0 / mxfp4 unit
+// ------------------------------------------------------------------ iq4_nl / q4_0 / mxfp4 / nvfp4 unit
 // Lane (row, kg) owns blocks 4 kg .. 4 kg + 3 of the row's eight (18 or 17 bytes each: scale, then 16 bytes whose
 // byte j holds weights j and j + 16).  The blocks' bytes are read as dwords and the 16 quant bytes of a block are
 // brought onto dword boundaries with v_alignbyte; everything else is the iq4_xs unit: table read per byte, MFMA
-// (ib, q) on bytes 2 q, 2 q + 1 of block ib, block scale on the partial sum.
+// (ib, q) on bytes 2 q, 2 q + 1 of block ib, block scale on the partial sum.  nvfp4: the lane's 72 bytes are two
+// 36-byte blocks, all fields on dword boundaries; "block" ib is then a pair of 16-weight groups with a scale each.
+// half of an unsigned e4m3 scale (0 and 0x7f decode to 0), the value kq::ue4m3_half returns, without branches
+__device__ __forceinline__ float ue4m3_half_fast(uint32_t x) {
+  const uint32_t ex = (x >> 3) & 15u, man = x & 7u;
+  const float normal = __builtin_bit_cast(float, ((ex + 119u) << 23) | (man << 20));
+  const float sub = (float)man * 0x1p-10f;
+  const float v = ex ? normal : sub;
+  return x == 0x7fu ? 0.0f : v;
+}
 template <int C, int R, int AS>
 __device__ __forceinline__ void nib32_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
                                            const uint8_t* __restrict__ tbl, float* acc) {
   constexpr int RG = (R + 3) / 4;
+  constexpr bool NV = C == KQ_NVFP4;            // 36-byte blocks of 64: scale bytes 0 .. 3, 8 quant bytes per 16 weights
   constexpr int BB = C == KQ_MXFP4 ? 17 : 18;   // block bytes
   constexpr int HB = C == KQ_MXFP4 ? 1 : 2;     // scale bytes in front of the quants
   constexpr int NDW = 4 * BB / 4;               // 17 or 18 dwords per lane
@@ -602,7 +623,8 @@ __device__ __forceinline__ void nib32_unit(const uint8_t* __restrict__ bl, int k
   u32x2 bv[4][8];
   auto lookup = [&](auto ii) {
     constexpr int ib = decltype(ii)::value;
-    constexpr int o = BB * ib + HB, base = o / 4, sh = o % 4;  // first quant byte of the block
+    // first quant byte of the block (nvfp4: of the 16 bytes of groups 2 (ib % 2), 2 (ib % 2) + 1 of block ib / 2)
+    constexpr int o = NV ? 36 * (ib / 2) + 4 + 16 * (ib % 2) : BB * ib + HB, base = o / 4, sh = o % 4;
     uint32_t qv[4];
 #pragma unroll
     for (int i = 0; i < 4; i++)
@@ -620,16 +642,31 @@ __device__ __forceinline__ void nib32_unit(const uint8_t* __restrict__ bl, int k
   SFor<4>::run([&](auto ii) {
     constexpr int ib = decltype(ii)::value;
     if constexpr (ib < 3) lookup(std::integral_constant<int, ib + 1>{});
-    f32x4 p[RG];
+    f32x4 p[RG], p2[RG];  // p2: the second 16 weights of the 32 (nvfp4: a scale of their own)
 #pragma unroll
-    for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
+    for (int g = 0; g < RG; g++) p[g] = p2[g] = f32x4{0, 0, 0, 0};
     SFor<8>::run([&](auto qq) {
       constexpr int q = decltype(qq)::value;
 #pragma unroll
-      for (int g = 0; g < RG; g++)
-        p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, areg[g * AS + ib]),
-                                                  __builtin_bit_cast(f16x4, bv[ib][q]), p[g], 3, q, 0);
+      for (int g = 0; g < RG; g++) {
+        if constexpr (NV && q >= 4)
+          p2[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, areg[g * AS + ib]),
+                                                     __builtin_bit_cast(f16x4, bv[ib][q]), p2[g], 3, q, 0);
+        else
+          p[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, areg[g * AS + ib]),
+                                                    __builtin_bit_cast(f16x4, bv[ib][q]), p[g], 3, q, 0);
+      }
     });
+    if constexpr (NV) {
+      const uint32_t sw = w[9 * (ib / 2)] >> (16 * (ib % 2));
+      const float d0 = ue4m3_half_fast(sw & 0xffu) * xscale, d1 = ue4m3_half_fast((sw >> 8) & 0xffu) * xscale;
+      SFor<R>::run([&](auto rr) {
+        constexpr int r = decltype(rr)::value;
+        acc[r] = fmaf(d0, p[r / 4][r % 4], acc[r]);
+        acc[r] = fmaf(d1, p2[r / 4][r % 4], acc[r]);
+      });
+      return;
+    }
     constexpr int so = BB * ib;  // scale byte(s) of the block
     float dl;
     if constexpr (C == KQ_MXFP4)
@@ -1075,15 +1112,19 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         *reinterpret_cast<f16x8*>(xs + (ml * ST_XU + uu) * 256 + 8 * grp) = v8;
       } else {
         // x[j], x[j + 16] interleaved over each 32: lanes a and a + 2 of a quad hold x[8 a ..] and x[16 + 8 a ..]
-        // and write one half each of the 16 interleaved values
+        // and write one half each of the 16 interleaved values (XORD 3: x[j], x[j + 8] over each 16, lanes a and
+        // a + 1)
         typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
         uint32_t own[4], par[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           own[e] = __builtin_bit_cast(uint32_t, f16x2v{h[2 * e], h[2 * e + 1]});
-          par[e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own[e], 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+          if constexpr (XORD == 2)
+            par[e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own[e], 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+          else
+            par[e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own[e], 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
         }
-        const bool high = (grp & 2) != 0;
+        const bool high = (grp & (XORD == 2 ? 2 : 1)) != 0;
         // low lane: own h0..h3 with the partner's h0..h3 behind each; high lane: the partner's h4..h7 ahead of own
         const uint32_t a0 = high ? par[2] : own[0], a1 = high ? par[3] : own[1];  // first of each pair
         const uint32_t b0 = high ? own[2] : par[0], b1 = high ? own[3] : par[1];  // second of each pair
@@ -1092,7 +1133,10 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         o[1] = (a0 >> 16) | (b0 & 0xffff0000u);
         o[2] = (a1 & 0xffffu) | (b1 << 16);
         o[3] = (a1 >> 16) | (b1 & 0xffff0000u);
-        *reinterpret_cast<u32x4*>(xs + (ml * ST_XU + uu) * 256 + 32 * (grp >> 2) + 16 * (grp & 1) + (high ? 8 : 0)) = o;
+        if constexpr (XORD == 2)
+          *reinterpret_cast<u32x4*>(xs + (ml * ST_XU + uu) * 256 + 32 * (grp >> 2) + 16 * (grp & 1) + (high ? 8 : 0)) = o;
+        else
+          *reinterpret_cast<u32x4*>(xs + (ml * ST_XU + uu) * 256 + 16 * (grp >> 1) + (high ? 8 : 0)) = o;
       }
       float sum = 0.f;
 #pragma unroll
@@ -1138,7 +1182,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
     for (int i = 0; i < PER_WAVE; i++) {
       const int b = 8 * (PER_WAVE * wave + i) + (lane >> 3);
       auto val = [](int i) -> float {
-        if constexpr (C == KQ_MXFP4) return kq::kv_mxfp4(i);
+        if constexpr (C == KQ_MXFP4 || C == KQ_NVFP4) return kq::kv_mxfp4(i);
         else if constexpr (C == KQ_Q4_0) return (float)(i - 8);
         else return kq::kv_iq4nl(i);
       };
@@ -1264,7 +1308,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
           q80_unit<R, AS>(bl, kg, xscale, areg + us * NAP, acc);
         } else if constexpr (C == KQ_IQ4_XS) {
           iq4xs_unit<R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc);
-        } else if constexpr (C == KQ_IQ4_NL || C == KQ_Q4_0 || C == KQ_MXFP4) {
+        } else if constexpr (C == KQ_IQ4_NL || C == KQ_Q4_0 || C == KQ_MXFP4 || C == KQ_NVFP4) {
           nib32_unit<C, R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc);
         } else if constexpr (C == KQ_IQ2_XXS) {
           constexpr int COP = st_iq2_copies<C, MB, NW, GM>();
@@ -1387,6 +1431,7 @@ int st_max_sb(int codec, int M) {
     case KQ_IQ4_NL: rows = st_nw8_rows<KQ_IQ4_NL>(); break;
     case KQ_Q4_0: rows = st_nw8_rows<KQ_Q4_0>(); break;
     case KQ_MXFP4: rows = st_nw8_rows<KQ_MXFP4>(); break;
+    case KQ_NVFP4: rows = st_nw8_rows<KQ_NVFP4>(); break;
   }
   return M <= rows ? 32 : 16;
 }
@@ -1511,7 +1556,7 @@ int st_launch_gather_nw(const StArgs& a, int entries, bool glu, hipStream_t s) {
 bool st_codec_ok(int codec) {
   return codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K || codec == KQ_Q2_K || codec == KQ_Q3_K ||
          codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S || codec == KQ_Q8_0 || codec == KQ_IQ4_NL ||
-         codec == KQ_Q4_0 || codec == KQ_MXFP4;
+         codec == KQ_Q4_0 || codec == KQ_MXFP4 || codec == KQ_NVFP4;
 }
 
 }  // namespace
@@ -1573,6 +1618,8 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
     return dtype == KQ_F16 ? st_launch_m<KQ_Q4_0, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q4_0, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_MXFP4)
     return dtype == KQ_F16 ? st_launch_m<KQ_MXFP4, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_MXFP4, KQ_BF16>(a, p.ksplit, s);
+  if (codec == KQ_NVFP4)
+    return dtype == KQ_F16 ? st_launch_m<KQ_NVFP4, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_NVFP4, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q2_K)
     return dtype == KQ_F16 ? st_launch_m<KQ_Q2_K, KQ_F16>(a, p.ksplit, s) : st_launch_m<KQ_Q2_K, KQ_BF16>(a, p.ksplit, s);
   if (codec == KQ_Q3_K)
@@ -1633,6 +1680,7 @@ int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, 
                            : st_launch_gather_nw<c, KQ_BF16>(a, entries, glu, s);
     KQ_CASE(KQ_Q2_K) KQ_CASE(KQ_Q3_K) KQ_CASE(KQ_Q4_K) KQ_CASE(KQ_Q5_K) KQ_CASE(KQ_Q6_K) KQ_CASE(KQ_IQ4_XS)
     KQ_CASE(KQ_IQ3_S) KQ_CASE(KQ_IQ2_XXS) KQ_CASE(KQ_Q8_0) KQ_CASE(KQ_IQ4_NL) KQ_CASE(KQ_Q4_0) KQ_CASE(KQ_MXFP4)
+    KQ_CASE(KQ_NVFP4)
 #undef KQ_CASE
   }
   return KQ_ERR_UNSUPPORTED;

@@ -122,7 +122,7 @@ def test_qmm_skinny_both_variants(kq, codec):
 
 
 @pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k", "q2_k", "q3_k", "iq4_xs", "iq2_xxs", "iq3_s", "q8_0", "iq4_nl",
-                                   "q4_0", "mxfp4"])
+                                   "q4_0", "mxfp4", "nvfp4"])
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
 def test_qmm_streamed_kernel_shapes(kq, codec, dtype):
     """The streamed kernel (default for up to eight rows of q4_k / q5_k / q6_k): one to eight rows (five and more

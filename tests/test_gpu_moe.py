@@ -208,9 +208,9 @@ def test_moe_tuned_gathered_shapes(kq, codec, E, N, K, T, R):
 @pytest.mark.parametrize("codec,T", [("q2_k", 50), ("q2_k", 80), ("q3_k", 50), ("q3_k", 80), ("iq4_xs", 15),
                                      ("iq4_xs", 20), ("iq3_s", 15), ("iq3_s", 20), ("iq2_xxs", 15), ("iq2_xxs", 20),
                                      ("q8_0", 15), ("q8_0", 20), ("mxfp4", 15), ("mxfp4", 20), ("q4_0", 15),
-                                     ("q4_0", 20), ("iq4_nl", 15), ("iq4_nl", 20)])
+                                     ("q4_0", 20), ("iq4_nl", 15), ("iq4_nl", 20), ("nvfp4", 50), ("nvfp4", 80)])
 def test_moe_low_bit_routes_either_side_of_the_entry_threshold(kq, codec, T):
-    """q2_k / q3_k stacks run entry by entry on the streamed kernel up to 256 (token, expert) pairs and on the
+    """q2_k / q3_k / nvfp4 stacks run entry by entry on the streamed kernel up to 256 (token, expert) pairs, on the
     any-codec kernel above; iq4_xs / iq3_s / iq2_xxs / q8_0 / mxfp4 / q4_0 / iq4_nl switch to the code-level grouped
     kernel above 64 pairs.  The
     token counts (x 4 experts each) sit on either side."""
@@ -406,7 +406,7 @@ def test_rhs_gather_more_than_32767_rows(kq, codec):
 
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
 @pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k", "q2_k", "q3_k", "iq4_xs", "iq3_s", "iq2_xxs", "q8_0", "iq4_nl",
-                                   "q4_0", "mxfp4"])
+                                   "q4_0", "mxfp4", "nvfp4"])
 @pytest.mark.parametrize("N,K,T,R,act", [
     (72, 768, 1, 8, "silu"),       # ragged rows (72 = 2 tiles + 8), three superblocks: four-wave form, one unit a wave
     (96, 3072, 2, 4, "gelu"),      # twelve superblocks: eight-wave fused form, two tokens share the activations
