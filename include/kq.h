@@ -137,8 +137,8 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
 /* Device workspace (bytes, 256-byte aligned, may be 0) of the two MoE ops below: `glu` != 0 for
  * kq_moe_glu_gather, 0 for kq_gather_qmv.  The batched path (more than 16 (token, expert) pairs; more than 48
  * for q4_k / q5_k / q6_k and the legacy / fp4 / other IQ stacks, 64 for iq4_xs / iq3_s / iq2_xxs / q8_0 and for
- * unbiased iq4_nl / q4_0 / mxfp4 calls, 128 for nvfp4 with biases,
- * 256 for q2_k / q3_k / nvfp4)
+ * iq4_nl / q4_0 / mxfp4 with K a multiple of 256,
+ * 256 for q2_k / q3_k / nvfp4; for stacks of fewer than 128 experts these limits shrink in proportion, E / 128)
  * sorts the pairs by expert and keeps f16 activations there.  The reference allocates its own
  * temporaries inside eval_gpu (src/kquant_moe_glu.cpp:277-382); here the caller owns them. */
 size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int codec, int dtype);

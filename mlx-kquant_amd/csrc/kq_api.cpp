@@ -240,7 +240,7 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
                            const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
                            int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
                            size_t ws_bytes, KqOutMap om, hipStream_t s, int entry_rows = 1);
-static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int N, int K);
+static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int E, int N, int K);
 
 int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_dev, const uint32_t* rhs_idx_dev,
                   void* out_dev, int B, int M, int E, int N, int K, int64_t x_batch_stride,
@@ -268,7 +268,7 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
   // many output rows: gather them into a dense matrix and run the expert-grouped kernels
   int64_t P;
   if (workspace_dev && gather_batched_shape(B, M, E, N, K, transpose, codec, &P) &&
-      !per_entry_route(P, M, false, 0, 0, codec, N, K) &&
+      !per_entry_route(P, M, false, 0, 0, codec, E, N, K) &&
       !(reinterpret_cast<uintptr_t>(workspace_dev) & 255) && !(reinterpret_cast<uintptr_t>(x_dev) & 15) &&
       !(x_batch_stride & 7)) {
     const size_t need = kq_gather_qmm_workspace_size(B, M, E, N, K, transpose, codec, dtype);
@@ -353,7 +353,7 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 #ifndef KQ_PER_ENTRY_MAX_PAIRS_Q8
 #define KQ_PER_ENTRY_MAX_PAIRS_Q8 64
 #endif
-// iq4_nl / q4_0 / mxfp4 calls the streamed kernel takes (no biases, no swiglu_clamp, K a multiple of 256), against the
+// iq4_nl / q4_0 / mxfp4 calls the streamed kernel takes (K a multiple of 256), against the
 // code-level grouped kernel (same stacks, us: mxfp4 32 pairs 20.2 + 16.5 against 37.4 + 22.7, 64 pairs 37.2 + 30.1
 // against 50.1 + 30.5, 96 pairs 54.5 + 43.7 against 58.3 + 37.3; q4_0 64 pairs 33.3 + 28.3 against 48.0 + 25.8).
 // nvfp4 calls the streamed kernel takes, against the any-codec kernel (us: 128 pairs 71.6 + 58.4 entry by entry,
@@ -370,27 +370,38 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 // True when a call of P (token, expert) pairs is better served entry by entry than by the sorted, expert-grouped
 // kernels.  entry_rows = activation rows per entry of the caller's per-entry fallback (1 for the MoE ops; gather_qmm's
 // M): the per-entry kernels take one row per entry, the older K-quant ones up to eight.
-static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int N, int K) {
+// The pair counts above were measured on stacks of 128 experts.  Entry by entry every pair reads its expert's matrix
+// again while the grouped kernels read a matrix once per call, so what decides is how many pairs share an expert:
+// the limits shrink in proportion for shorter stacks (32 experts of 3072 x 3072 in mxfp4, 64 pairs: 188 + 81 us entry
+// by entry against 118 + 68 grouped).
+static int64_t per_entry_limit(int limit, int E) {
+  const int64_t scaled = (int64_t)limit * E / 128;
+  return scaled < limit ? scaled : limit;
+}
+static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int E, int N, int K) {
   if (P <= 16) return false;  // the callers never reach the grouped route with so few pairs
   const bool grouped_codec = codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K;
   const bool low_codec = codec == KQ_Q2_K || codec == KQ_Q3_K;  // their batched route is the any-codec kernel
   const bool iq_codec = codec == KQ_IQ4_XS || codec == KQ_IQ3_S || codec == KQ_IQ2_XXS;
   const bool q8 = codec == KQ_Q8_0;  // per-entry kernel: the streamed one; batched: the code-level grouped kernel
-  const bool streamed_shape =
-      !(has_bias || (glu && act == KQ_ACT_SWIGLU_CLAMP) || (K >> 8) > (glu ? 16 : 32) || (K & 255));
-  // iq4_nl / q4_0 / mxfp4 / nvfp4 entries the streamed kernel takes; the others fall to the code-level rule below
-  if ((codec == KQ_IQ4_NL || codec == KQ_Q4_0 || codec == KQ_MXFP4) && streamed_shape && entry_rows == 1 &&
-      P <= KQ_PER_ENTRY_MAX_PAIRS_NIB)
+  const bool streamed_k = !((K >> 8) > (glu ? 16 : 32) || (K & 255));
+  const bool streamed_shape = streamed_k && !(has_bias || (glu && act == KQ_ACT_SWIGLU_CLAMP));
+  // iq4_nl / q4_0 / mxfp4 / nvfp4 entries the streamed kernel takes (biases and swiglu_clamp included); the others
+  // fall to the code-level rule below
+  if ((codec == KQ_IQ4_NL || codec == KQ_Q4_0 || codec == KQ_MXFP4) && streamed_k && entry_rows == 1 &&
+      P <= per_entry_limit(KQ_PER_ENTRY_MAX_PAIRS_NIB, E))
     return true;
-  if (codec == KQ_NVFP4 && streamed_shape && entry_rows == 1 && P <= KQ_PER_ENTRY_MAX_PAIRS_NVFP4_STREAMED) return true;
+  if (codec == KQ_NVFP4 && streamed_k && entry_rows == 1 && P <= per_entry_limit(KQ_PER_ENTRY_MAX_PAIRS_NVFP4_STREAMED, E))
+    return true;
   // the other codecs' per-entry kernel is the code-level one, which takes biases and every activation
   if (!grouped_codec && !low_codec && !iq_codec && !q8)
-    return entry_rows == 1 && P <= (codec == KQ_NVFP4 ? KQ_PER_ENTRY_MAX_PAIRS_NVFP4 : KQ_PER_ENTRY_MAX_PAIRS_CODES) &&
+    return entry_rows == 1 &&
+           P <= per_entry_limit(codec == KQ_NVFP4 ? KQ_PER_ENTRY_MAX_PAIRS_NVFP4 : KQ_PER_ENTRY_MAX_PAIRS_CODES, E) &&
            kq_codes_gather_supported(1, N, K, codec);
   if (!streamed_shape) return false;
-  if (grouped_codec) return P <= KQ_PER_ENTRY_MAX_PAIRS && entry_rows <= 8;
+  if (grouped_codec) return P <= per_entry_limit(KQ_PER_ENTRY_MAX_PAIRS, E) && entry_rows <= 8;
   return entry_rows == 1 &&
-         P <= (low_codec ? KQ_PER_ENTRY_MAX_PAIRS_LOW : q8 ? KQ_PER_ENTRY_MAX_PAIRS_Q8 : KQ_PER_ENTRY_MAX_PAIRS_IQ);
+         P <= per_entry_limit(low_codec ? KQ_PER_ENTRY_MAX_PAIRS_LOW : q8 ? KQ_PER_ENTRY_MAX_PAIRS_Q8 : KQ_PER_ENTRY_MAX_PAIRS_IQ, E);
 }
 
 static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
@@ -401,7 +412,7 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
   // few entries: the per-entry kernels (the caller tries them next) beat the prologue + grouped-kernel pair
-  if (per_entry_route(P, entry_rows, bias || bias2, glu, act, codec, N, K)) return KQ_ERR_UNSUPPORTED;
+  if (per_entry_route(P, entry_rows, bias || bias2, glu, act, codec, E, N, K)) return KQ_ERR_UNSUPPORTED;
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
     // legacy / IQ / fp4 codecs (biases and every activation included): code-level grouped kernel
     if (kq_codes_moe_supported((int)P, E, N, K, codec)) {
@@ -461,6 +472,14 @@ static int moe_glu_gather_impl(const void* x_dev, const void* gate_w_dev, const 
                                     static_cast<hipStream_t>(stream));
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
   }
+  if (kq_stream_full_epilogue(codec) && (biased || act == KQ_ACT_SWIGLU_CLAMP)) {
+    // fp4 stacks with biases / swiglu_clamp: the streamed kernel's gathered mode carries both
+    const int rcs = kq_launch_gather_stream(x_dev, static_cast<const uint8_t*>(gate_w_dev),
+                                            static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, out_dev, T * R, N, K,
+                                            R, K, estride, act, limit, alpha, gate_bias_dev, up_bias_dev, codec, dtype, E,
+                                            om, static_cast<hipStream_t>(stream));
+    if (rcs != KQ_ERR_UNSUPPORTED) return rcs;
+  }
   if (!biased) {
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(gate_w_dev),
                                            static_cast<const uint8_t*>(up_w_dev), nullptr, idx_dev, out_dev, T * R, 1, N,
@@ -506,6 +525,12 @@ static int gather_qmv_impl(const void* x_dev, const void* w_dev, const uint32_t*
                                     0, 0, 0.f, 0.f, codec, dtype, workspace_dev, workspace_bytes, om,
                                     static_cast<hipStream_t>(stream));
     if (rcg != KQ_ERR_UNSUPPORTED) return rcg;
+  }
+  if (bias_dev && kq_stream_full_epilogue(codec)) {
+    const int rcs = kq_launch_gather_stream(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, out_dev,
+                                            T * R, N, K, 1, K, estride, 0, 0.f, 1.0f, bias_dev, nullptr, codec, dtype, E, om,
+                                            static_cast<hipStream_t>(stream));
+    if (rcs != KQ_ERR_UNSUPPORTED) return rcs;
   }
   if (!bias_dev) {
     const int rct = kq_launch_gather_tuned(x_dev, static_cast<const uint8_t*>(w_dev), nullptr, nullptr, idx_dev, out_dev,

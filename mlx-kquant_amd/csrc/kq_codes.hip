@@ -1269,8 +1269,8 @@ int kq_launch_codes_skinny(const void* x, const uint8_t* w, const void* bias, vo
 #if !defined(KQ_CODES_PART) || KQ_CODES_PART == 2
 // Gathered calls of up to a few entries (MoE decode): one activation row per entry (M = 1), the entry's expert
 // matrix, optional f32 biases; glu != 0 runs gate and up stacks and the fused epilogue.
-// (iq4_nl / q4_0 / mxfp4 entries come here only when the streamed kernel declines them: biases, swiglu_clamp, a K
-// that is no multiple of 256.)
+// (iq4_nl / q4_0 / mxfp4 / nvfp4 entries come here only when the streamed kernel declines them: a K that is no
+// multiple of 256, more than 16 (32) superblocks.)
 // (q8_0 entries are not taken here: the streamed kernel has a q8_0 unit, and where that declines - a K that is no
 // multiple of 256 - the plain vector kernel measured 9.1 / 8.4 us against 12.7 / 9.0 us here for the GLU / down ops
 // of 8 experts of 768 x 2048.)

@@ -96,11 +96,17 @@ size_t kq_stream_workspace_bytes(int M, int N, int K, int codec);
 int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                          size_t ws_bytes, hipStream_t s);
 // Gathered matvec (MoE decode, one activation row per entry) on the streamed kernel; UNSUPPORTED -> older kernels.
-// Entry p reads activation row p / x_div of x, or (lhs != null) the row at x + lhs[p] * x_row_stride.
+// Entry p reads activation row p / x_div of x, or (lhs != null) the row at x + lhs[p] * x_row_stride.  bias / bias2:
+// null, or f32 [E][N] added to the gate (or plain) and up sums; alpha: the sigmoid slope of swiglu_clamp.
 int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs, const uint32_t* rhs,
                             void* out, int entries, int N, int K, int x_div, int64_t x_row_stride,
-                            int64_t w_expert_stride, int act, float limit, int codec, int dtype, int E, KqOutMap om,
-                            hipStream_t s);
+                            int64_t w_expert_stride, int act, float limit, float alpha, const float* bias,
+                            const float* bias2, int codec, int dtype, int E, KqOutMap om, hipStream_t s);
+// codecs whose gathered calls the streamed kernel also takes with biases and swiglu_clamp (the fp4 stacks that carry
+// them, and the two codecs that share their unit)
+inline bool kq_stream_full_epilogue(int codec) {
+  return codec == KQ_MXFP4 || codec == KQ_NVFP4 || codec == KQ_IQ4_NL || codec == KQ_Q4_0;
+}
 // Tuned gathered GEMV (items = (activation matrix, expert) pairs, M <= 8 rows each; with glu the
 // gate/up pair and the fused epilogue, M = 1): same fall-through contract as kq_launch_qmm_tuned.
 // The per-entry gather launchers take the stack height E and skip entries whose expert id is >= E.

@@ -1428,7 +1428,7 @@ int kq_launch_gather_tuned(const void* x, const uint8_t* w, const uint8_t* w2, c
   if (M == 1 && rhs && (lhs || x_batch_stride == K) && g_sk_variant == 0 && B >= 1 &&
       (!glu || act != KQ_ACT_SWIGLU_CLAMP)) {
     const int rcs = kq_launch_gather_stream(x, w, glu ? w2 : nullptr, lhs, rhs, out, B, N, K, x_div, x_batch_stride,
-                                            w_expert_stride, act, limit, codec, dtype, E, om, s);
+                                            w_expert_stride, act, limit, 1.0f, nullptr, nullptr, codec, dtype, E, om, s);
     if (rcs != KQ_ERR_UNSUPPORTED) return rcs;
   }
   if (!sk_shape_ok(M, K, codec, x, w, w2) || B < 1 || B > 65535) return KQ_ERR_UNSUPPORTED;

@@ -265,7 +265,9 @@ struct StArgs {
   const uint32_t* lhs;     // null, or the entry's activation row: x + lhs[p] * x_row_stride (x_div is then unused)
   int64_t x_row_stride;
   int tiles_per_entry, x_div, E, act;
-  float limit;
+  float limit, alpha;
+  const float* bias;   // null, or f32 [E][N] added to the (gate) sums before the epilogue
+  const float* bias2;  // the same for the up sums of the fused form
   int64_t w_expert_stride;
   KqOutMap om;
 #ifdef KQ_ST_TS
@@ -933,9 +935,11 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   const int g_tile = GM ? (int)blockIdx.x - g_entry * a.tiles_per_entry : 0;
   const uint8_t* wmat = a.w;
   const uint8_t* wmat2 = a.w;
+  uint32_t g_expert = 0;
   if constexpr (GM != 0) {
     const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.rhs[g_entry]);
     if (e >= (uint32_t)a.E) return;  // the whole workgroup, ahead of every barrier
+    g_expert = e;
     wmat = a.w + (int64_t)e * a.w_expert_stride;
     if constexpr (GM == 2) wmat2 = a.w2 + (int64_t)e * a.w_expert_stride;
   }
@@ -1350,7 +1354,11 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
       }
       if constexpr (GM != 0) {
         if (nn < nrows) {
-          if constexpr (GM == 2) v = kq::glu_epilogue(a.act, v, vu, a.limit, 1.0f);
+          if (a.bias) v += a.bias[(size_t)g_expert * N + row0 + nn];
+          if constexpr (GM == 2) {
+            if (a.bias2) vu += a.bias2[(size_t)g_expert * N + row0 + nn];
+            v = kq::glu_epilogue(a.act, v, vu, a.limit, a.alpha);
+          }
           kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, g_entry) * N + row0 + nn, v);
         }
       } else if (r < M && nn < nrows) {
@@ -1638,12 +1646,12 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
 #endif
 int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs, const uint32_t* rhs,
                             void* out, int entries, int N, int K, int x_div, int64_t x_row_stride,
-                            int64_t w_expert_stride, int act, float limit, int codec, int dtype, int E, KqOutMap om,
-                            hipStream_t s) {
+                            int64_t w_expert_stride, int act, float limit, float alpha, const float* bias,
+                            const float* bias2, int codec, int dtype, int E, KqOutMap om, hipStream_t s) {
   if (!st_codec_ok(codec)) return KQ_ERR_UNSUPPORTED;
   if (entries < 1 || entries > KQ_GATHER_STREAM_MAX_ENTRIES || N < 1 || K < 256 || (K & 255) || !rhs) return KQ_ERR_UNSUPPORTED;
   const bool glu = w2 != nullptr;
-  if ((K >> 8) > (glu ? 16 : 32) || (glu && act == KQ_ACT_SWIGLU_CLAMP)) return KQ_ERR_UNSUPPORTED;
+  if ((K >> 8) > (glu ? 16 : 32) || (!glu && bias2)) return KQ_ERR_UNSUPPORTED;
   if ((int64_t)entries * ((N + ST_ROWS - 1) / ST_ROWS) > 65535 * 16) return KQ_ERR_UNSUPPORTED;
   const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : codec == KQ_MXFP4 ? 0 : 1;
   if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
@@ -1667,6 +1675,9 @@ int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, 
   a.E = E;
   a.act = act;
   a.limit = limit;
+  a.alpha = alpha;
+  a.bias = bias;
+  a.bias2 = bias2;
   a.w_expert_stride = w_expert_stride;
   a.om = om;
   if (codec == KQ_IQ4_XS || codec == KQ_IQ2_XXS || codec == KQ_IQ3_S) {

@@ -213,8 +213,8 @@ def test_moe_low_bit_routes_either_side_of_the_entry_threshold(kq, codec, T):
     """q2_k / q3_k / nvfp4 stacks run entry by entry on the streamed kernel up to 256 (token, expert) pairs, on the
     any-codec kernel above; iq4_xs / iq3_s / iq2_xxs / q8_0 / mxfp4 / q4_0 / iq4_nl switch to the code-level grouped
     kernel above 64 pairs.  The
-    token counts (x 4 experts each) sit on either side."""
-    E, N, K, R = 6, 136, 768, 4
+    token counts (x 4 experts each) sit on either side.  (128 experts: the pair limits shrink with shorter stacks.)"""
+    E, N, K, R = 128, 136, 768, 4
     gate = _stack(codec, E, N, K, seed=91)
     up = _stack(codec, E, N, K, seed=92)
     rng = np.random.default_rng(93)
@@ -336,6 +336,35 @@ def test_moe_swiglu_clamp_bias(kq, codec):
     assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
 
 
+@pytest.mark.parametrize("codec", ["mxfp4", "nvfp4"])
+@pytest.mark.parametrize("T,R", [(1, 4), (3, 4), (10, 4), (15, 4), (20, 4)])
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+def test_moe_swiglu_clamp_bias_on_the_streamed_kernel(kq, codec, T, R, dtype):
+    """Biased fp4 experts with swiglu_clamp and K a multiple of 256: up to 64 (mxfp4) or 256 (nvfp4) pairs run entry
+    by entry on the streamed kernel, whose epilogue adds the f32 biases; 80 pairs of mxfp4 take the grouped kernel.
+    Ragged N (two tiles + 8 rows), a limit small enough to clamp, the down op with its bias."""
+    E, N, K = 128, 72, 768
+    gate = _stack(codec, E, N, K, seed=261)
+    up = _stack(codec, E, N, K, seed=262)
+    rng = np.random.default_rng(263)
+    gb = (rng.standard_normal((E, N)) * 0.05).astype(np.float32)
+    ub = (rng.standard_normal((E, N)) * 0.05).astype(np.float32)
+    idx = np.stack([rng.permutation(E)[:R] for _ in range(T)])
+    xb, xt = make_x((T, K), dtype, seed=264, scale=0.2)
+    g, u, ix = wire_to_dev(gate), wire_to_dev(up), _idx_dev(idx)
+    gbt, ubt = torch.from_numpy(gb).cuda(), torch.from_numpy(ub).cuda()
+    got = kq.moe_glu_gather_kq(xt, g, u, codec, ix, act="swiglu_clamp", limit=7.0, gate_bias=gbt, up_bias=ubt, alpha=1.702)
+    want = _glu_truth(codec, xb, gate, up, idx, "swiglu_clamp", 7.0, 1.702, gb, ub, dtype=dtype)
+    assert rel_l2(dev_to_bits(got), want, dtype) <= TOL
+    got = kq.moe_glu_gather_kq(xt, g, u, codec, ix, act="swiglu_clamp", limit=0.75, gate_bias=ubt, up_bias=gbt, alpha=1.2)
+    want = _glu_truth(codec, xb, gate, up, idx, "swiglu_clamp", 0.75, 1.2, ub, gb, dtype=dtype)
+    assert rel_l2(dev_to_bits(got), want, dtype) <= TOL
+    hb, ht = make_x((T, R, K), dtype, seed=265, scale=0.2)
+    got = kq.gather_qmv_kq(ht, g, codec, ix, bias=gbt)
+    want = O.gather_qmv(hb, gate, codec, idx, gb, dtype)
+    assert rel_l2(dev_to_bits(got), want, dtype) <= TOL
+
+
 def test_moe_validation_errors(kq):
     d = torch.device("cuda:0")
     E, N, K = 2, 16, 256
@@ -417,7 +446,7 @@ def test_rhs_gather_more_than_32767_rows(kq, codec):
 def test_moe_decode_entries_on_the_streamed_kernel(kq, codec, N, K, T, R, act, dtype):
     """Up to 16 (token, expert) entries of a stack in one of the streamed kernel's codecs (48 for q4_k / q5_k / q6_k)
     run its gathered mode: fused gate / up (two units per superblock) and the plain down projection."""
-    E = 5
+    E = 5 if T * R <= 16 else 130  # beyond 16 entries the per-entry route needs a tall stack
     gate, up, down = _stack(codec, E, N, K, 201), _stack(codec, E, N, K, 202), _stack(codec, E, N, K, 203)
     rng = np.random.default_rng(204)
     idx = rng.integers(0, E, (T, R))
