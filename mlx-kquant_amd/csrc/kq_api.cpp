@@ -214,6 +214,10 @@ int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void
     return kq_set_error(KQ_ERR_INVALID, "%s: bad dimension", op);
   if (N == 0) return KQ_OK;
   if (!x_dev || !w_dev || !bias_dev || !y_dev) return kq_set_error(KQ_ERR_INVALID, "%s: null buffer", op);
+  // the streamed kernel where its plan needs no K split (this op has no workspace), else the code-level kernel
+  const int rcs = kq_launch_qmm_stream(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, 1, N, K, codec, dtype, nullptr, 0,
+                                       static_cast<hipStream_t>(stream), bias_dev);
+  if (rcs != KQ_ERR_UNSUPPORTED) return rcs;
   const int rc = kq_launch_codes_skinny(x_dev, static_cast<const uint8_t*>(w_dev), bias_dev, y_dev, 1, N, K, codec, dtype,
                                         static_cast<hipStream_t>(stream));
   if (rc == KQ_ERR_UNSUPPORTED) return kq_set_error(KQ_ERR_UNSUPPORTED, "%s: x must be 16-byte aligned", op);

@@ -94,7 +94,7 @@ int kq_launch_qmm_tuned(const void* x, const uint8_t* w, void* y, int M, int N, 
 bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const void* w);
 size_t kq_stream_workspace_bytes(int M, int N, int K, int codec);
 int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
-                         size_t ws_bytes, hipStream_t s);
+                         size_t ws_bytes, hipStream_t s, const void* bias = nullptr);
 // Gathered matvec (MoE decode, one activation row per entry) on the streamed kernel; UNSUPPORTED -> older kernels.
 // Entry p reads activation row p / x_div of x, or (lhs != null) the row at x + lhs[p] * x_row_stride.  bias / bias2:
 // null, or f32 [E][N] added to the gate (or plain) and up sums; alpha: the sigmoid slope of swiglu_clamp.

@@ -256,6 +256,7 @@ struct StArgs {
   const uint8_t* grids;  // device copy of the IQ codebooks (codebook codecs)
   int rpt;  // weight rows per tile (<= 32): fewer than 32 evens the rows out over one round of workgroups
   float* partial;  // split-K: [ksplit][M][N] f32
+  const uint16_t* bias16;  // dense calls without a K split: null, or [N] in the activation dtype, added in f32
   int ksplit, sb_per_split;
   // gathered calls (one activation row per entry, MoE decode): entry p = blockIdx.x / tiles_per_entry multiplies row
   // p / x_div of x by rows of expert rhs[p] (w, and w2 = the up stack of the fused gate / up form) into output row
@@ -1365,6 +1366,7 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         if (a.ksplit > 1) {
           a.partial[(size_t)blockIdx.z * M * N + (size_t)r * N + row0 + nn] = v;
         } else {
+          if (a.bias16) v += DT == KQ_F16 ? kq::h2f(a.bias16[row0 + nn]) : kq::bf162f(a.bias16[row0 + nn]);
           uint16_t* yo = static_cast<uint16_t*>(a.y) + (size_t)r * N + row0 + nn;
           *yo = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
         }
@@ -1588,9 +1590,10 @@ size_t kq_stream_workspace_bytes(int M, int N, int K, int codec) {
 }
 
 int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
-                         size_t ws_bytes, hipStream_t s) {
+                         size_t ws_bytes, hipStream_t s, const void* bias) {
   if (!kq_stream_supported(M, N, K, codec, x, w)) return KQ_ERR_UNSUPPORTED;
   const StSplit p = st_split_plan(M, N, K, codec, st_num_cus());
+  if (bias && p.ksplit > 1) return KQ_ERR_UNSUPPORTED;  // the bias joins the sum in the unsplit epilogue only
   if (p.ksplit > 1 && (!ws || ws_bytes < (size_t)p.ksplit * M * N * sizeof(float) || (reinterpret_cast<uintptr_t>(ws) & 3)))
     return KQ_ERR_UNSUPPORTED;  // the caller falls through to the kernels that can run unsplit
   StArgs a{};
@@ -1602,6 +1605,7 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
   a.K = K;
   a.tiles = (N + ST_ROWS - 1) / ST_ROWS;
   a.partial = static_cast<float*>(ws);
+  a.bias16 = static_cast<const uint16_t*>(bias);
   a.ksplit = p.ksplit;
   a.sb_per_split = p.sb_per_split;
   a.rpt = p.rpt;

@@ -142,6 +142,24 @@ def test_qmm_streamed_kernel_shapes(kq, codec, dtype):
         assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype, M, N, K)
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+@pytest.mark.parametrize("N,K", [(264, 512), (4096, 4096), (1000, 8192), (33, 256), (97, 320), (20000, 1024)])
+def test_qmv_bias_fused_decode(kq, N, K, dtype):
+    """q8_0 decode with the bias added to the f32 sum before the single rounding (quantized_matmul_qmv_bias): the
+    streamed kernel where K is a multiple of 256 and its plan needs no K split, the code-level kernel otherwise
+    (K = 320; 264 x 512 and 33 x 256 are too small to fill the chip unsplit)."""
+    wire = _wire("q8_0", N, K, seed=301)
+    xb, xt = make_x((1, K), dtype, seed=302)
+    b = np.random.default_rng(303).standard_normal(N).astype(np.float32)
+    bbits = O.f32_to_bits(b, dtype)
+    bt = torch.from_numpy(bbits.view(np.int16)).cuda().view(torch.bfloat16 if dtype == "bfloat16" else torch.float16)
+    got = kq.quantized_matmul_qmv_bias(xt, wire_to_dev(wire), None, bt, "q8_0")
+    f32 = O.qmm(O.bits_to_f32(xb, dtype).reshape(1, K), wire, "q8_0", True, "float32")
+    want = O.f32_to_bits(f32 + O.bits_to_f32(bbits, dtype), dtype)
+    assert tuple(got.shape) == (1, N) and got.dtype == xt.dtype
+    assert rel_l2(dev_to_bits(got), want, dtype) <= TOL
+
+
 def test_qmm_skinny_unaligned_q6k_rows(kq):
     """q6_k rows are 210-byte multiples: a wire view that starts 2 bytes into an allocation still decodes."""
     N, K, M = 64, 768, 1
