@@ -17,7 +17,7 @@ enter the figure; `us_per_launch` = step time / `launches_per_step`.
 Extra fields: `sweep` (the decode projections of the q4_k_m recipe at M in {1,2,4,8}), `prefill`
 (q4_k / q5_k / q6_k GEMM 8192 -> 28672 at M in {512, 2048}), `moe` (128 experts, top-8, hidden 2048,
 intermediate 768: fused gate/up GLU in q4_k and down in q6_k at 1 and 256 tokens), `lowbit` (M=1
-GEMV 8192 -> 8192 in the low-bit codecs), `moe_decode_lowbit` (1 token, 8 of 128 experts, IQ / mxfp4 stacks),
+GEMV 8192 -> 8192 in the low-bit codecs), `moe_decode_lowbit` (1 token, 8 of 128 experts, IQ / fp4 / q8_0 stacks),
 `dequantize` (whole-matrix decode to f16, wire bytes in plus
 2 N K bytes out), `mid_m` (16 ... 64 activation rows on 4096-wide matrices), `no_transpose` (transpose = 0:
 128 gathered entries of (M x 128) . (128 x 512), and dense 4096 x 4096), `roofline` for the dominant kernel and `cpu_baseline`
@@ -544,7 +544,7 @@ def main():
         if want("moe_decode_lowbit"):
             E, H, I, TOPK = 128, 2048, 768, 8
             dec = []
-            for c in ("iq4_xs", "iq3_s", "iq2_xxs", "mxfp4"):
+            for c in ("iq4_xs", "iq3_s", "iq2_xxs", "mxfp4", "nvfp4", "q8_0"):
                 gate = synth_wire_torch(c, E * I, H, 31, dev).reshape(E, I, -1)
                 up = synth_wire_torch(c, E * I, H, 32, dev).reshape(E, I, -1)
                 down = synth_wire_torch(c, E * H, I, 33, dev).reshape(E, H, -1)
