@@ -18,6 +18,7 @@ Extra fields: `sweep` (the decode projections of the q4_k_m recipe at M in {1,2,
 (q4_k / q5_k / q6_k GEMM 8192 -> 28672 at M in {512, 2048}), `moe` (128 experts, top-8, hidden 2048,
 intermediate 768: fused gate/up GLU in q4_k and down in q6_k at 1 and 256 tokens), `lowbit` (M=1
 GEMV 8192 -> 8192 in the low-bit codecs), `moe_decode_lowbit` (1 token, 8 of 128 experts, IQ / fp4 / q8_0 stacks),
+`read_ceiling` (stock read-only reduction and device copy on buffers of the GEMV's sizes, cold),
 `dequantize` (whole-matrix decode to f16, wire bytes in plus
 2 N K bytes out), `mid_m` (16 ... 64 activation rows on 4096-wide matrices), `no_transpose` (transpose = 0:
 128 gathered entries of (M x 128) . (128 x 512), and dense 4096 x 4096), `roofline` for the dominant kernel and `cpu_baseline`
@@ -287,6 +288,35 @@ def cold_copies(torch, base, wbytes):
     return [base] + [base.clone() for _ in range(ncopies - 1)]
 
 
+def read_ceiling(torch, dev, sizes):
+    """What this box's memory system delivers to stock kernels on buffers of the GEMV's sizes, cold (rotating
+    over copies that together exceed twice the last-level cache) and timed like the GEMV (HIP-graph replays):
+    a read-only reduction (torch.sum over an int32 view: bytes read) and the runtime's device-to-device copy
+    (bytes read + bytes written).  Stated next to the 8 TB/s peak so that a GEMV rate can be compared with what
+    a plain reader reaches on the same part."""
+    rows = []
+    for label, nbytes in sizes:
+        n32 = nbytes // 4
+        ncopies = max(2, (2 * LLC_BYTES + nbytes - 1) // nbytes + 1)
+        srcs = [torch.randint(-2 ** 31, 2 ** 31 - 1, (n32,), dtype=torch.int32, device=dev) for _ in range(ncopies)]
+        acc = torch.empty((), dtype=torch.int64, device=dev)
+        dsts = [torch.empty_like(srcs[0]) for _ in range(ncopies)]
+
+        def summer(v):
+            return lambda stream=None: torch.sum(v, dtype=torch.int64, out=acc)
+
+        def copier(v, d):
+            return lambda stream=None: d.copy_(v)
+
+        ts, _ = time_calls(torch, [summer(v) for v in srcs], 200, 20)
+        tc, _ = time_calls(torch, [copier(v, d) for v, d in zip(srcs, dsts)], 200, 20)
+        rows.append({"buffer": label, "bytes": n32 * 4,
+                     "sum_int32_us": round(ts * 1e3, 2), "sum_int32_read_gbs": round(n32 * 4 / (ts * 1e-3) / 1e9, 1),
+                     "copy_us": round(tc * 1e3, 2), "copy_read_plus_write_gbs": round(2 * n32 * 4 / (tc * 1e-3) / 1e9, 1)})
+        del srcs, dsts
+    return rows
+
+
 def cpu_baseline(wire_np, codec, K, M, budget_s=12.0):
     """The CPU oracle (a port of the reference's threaded scalar eval_cpu path) on the same GEMV."""
     import numpy as np
@@ -439,6 +469,9 @@ def main():
     }
     base_np = base.cpu().numpy() if not args.no_cpu else None
     del copies, calls
+    # the box's attainable bandwidth with stock kernels, on the sizes of the headline matrix and of lm_head
+    out["read_ceiling"] = read_ceiling(torch, dev, [("gate/up q4_k wire, 33 MB", wbytes),
+                                                    ("lm_head q6_k wire, 431 MB", 128256 * kq.bytes_per_row("q6_k", 4096))])
 
     only = set(args.only.split(",")) if args.only else None
 

@@ -92,7 +92,9 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
  * optional part of kq_qmm_workspace_size (partial sums of a K range cut over the grid) is used when it fits
  * and left out otherwise.  All calls on one GPU share that GPU's buffer: calls that overlap in time on the same
  * GPU (different streams or threads) race; the buffer keeps the last call's contents, and the kernels write
- * every element they later read, so nothing needs clearing between calls.
+ * every element they later read, so nothing needs clearing between calls.  The first call of a shape on a
+ * device looks the buffer's address up and sets kernel attributes: make one eager call of each shape before
+ * capturing it into a HIP graph.
  * No counterpart in the reference. */
 #define KQ_NOALLOC_SCRATCH_BYTES (4u << 20)
 int kq_qmm_noalloc(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int K, int codec, int dtype,
@@ -107,15 +109,18 @@ int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void
 /* Tuning hook without a counterpart in the reference: workgroup tile of the prefill GEMM.  64 = 64
  * activation rows x 128 weight rows, 128 = 128 x 128, 256 = 64 x 256 on eight waves with two LDS stages
  * (q4_k only; other codecs fall back to automatic), 512 = 128 x 256 on eight waves with 128-row wave tiles and
- * direct-to-LDS loads (q4_k / q5_k; 513 = the same kernel as 128 x 128 on four waves); anything else restores the automatic choice.
+ * direct-to-LDS loads (q2_k / q3_k / q4_k / q5_k / iq4_xs; 513 = the same kernel as 128 x 128 on four waves);
+ * anything else restores the automatic choice.
  * Process-wide, not thread-safe. */
 void kq_set_gemm_tile_rows(int rows);
 /* Tuning hook without a counterpart in the reference: which skinny-M kernel dense calls use.
- * 0 = default (streamed kernel up to 4 activation rows of q4_k / q5_k / q6_k, else decoupled-wave kernel up to 4
- * rows and diagonal kernel for 5 - 8), 1 = workgroup-synchronous kernel (the one the gathered ops use),
- * 2 = decoupled-wave kernel always, 3 = decoupled-wave kernel with two-superblock units, 4 = diagonal kernel
- * wherever K allows it, 5 = streamed kernel (direct-to-LDS weight loads) wherever it applies.
- * Process-wide, not thread-safe. */
+ * 0 = default: the streamed kernel (direct-to-LDS weight loads) for up to 8 activation rows of every codec it
+ * has a unit for (q2_k ... q6_k, iq4_xs, iq3_s, iq2_xxs, q8_0, q4_0, iq4_nl, mxfp4, nvfp4); calls it declines (a
+ * split plan without workspace, unaligned activations) fall to the older K-quant kernels: decoupled-wave up to
+ * 4 rows, diagonal for 5 - 8.  The other values pin one of those older kernels for q2_k ... q6_k so that tests
+ * reach them: 1 = workgroup-synchronous kernel (the one multi-row gathered entries use), 2 = decoupled-wave
+ * kernel always, 3 = decoupled-wave kernel with two-superblock units, 4 = diagonal kernel wherever K allows it;
+ * 5 = same as 0.  Process-wide, not thread-safe. */
 void kq_set_skinny_variant(int variant);
 
 /* out[b] = x[lhs[b]] . W[rhs[b]]^T for b < B; x batches are [M,K] matrices

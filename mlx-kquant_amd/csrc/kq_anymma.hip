@@ -387,12 +387,7 @@ int launch_any(const AnyArgs& a, dim3 grid, hipStream_t s) {
   size_t lds = (size_t)NA * 32 * MT * A_STRIDE + (size_t)AM_BN * G::LROW + 128;
   if (MODE == 2 && lds < 8192 + 128) lds = 8192 + 128;
   auto kern = any_mma_kernel<C, DT, MT, MODE>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)lds));
-    attr_set = true;
-  }
+  KQ_SET_MAX_LDS_ONCE((kern), lds);
   hipLaunchKernelGGL(kern, grid, dim3(AM_THREADS), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;

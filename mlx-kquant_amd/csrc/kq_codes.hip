@@ -715,12 +715,7 @@ int launch_codes_wv(const CkArgs& a, hipStream_t s, int items) {
   const size_t red = (size_t)G::GRID_BYTES + G::SPREAD_BYTES + NWAVES * 4 * 64 * 4;
   if (lds < red) lds = red;
   auto kern = codes_skinny_kernel<C, DT, MB, GMODE, NWAVES>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)lds));
-    attr_set = true;
-  }
+  KQ_SET_MAX_LDS_ONCE((kern), lds);
   constexpr int TILE_N = GMODE == 2 ? 16 : 32;
   hipLaunchKernelGGL(kern, dim3((a.N + TILE_N - 1) / TILE_N, items), dim3(64 * NWAVES), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
@@ -1117,12 +1112,7 @@ int launch_grouped(const CgArgs& a, int P, int E, hipStream_t s) {
   if (maxseg > P) maxseg = P;
   const size_t lds = grouped_lds_bytes<C>();
   auto kern = codes_grouped_kernel<C, DT, GLU>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)lds));
-    attr_set = true;
-  }
+  KQ_SET_MAX_LDS_ONCE((kern), lds);
   hipLaunchKernelGGL(kern, dim3((a.N + NCOLS - 1) / NCOLS, maxseg), dim3(CG_THREADS), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;

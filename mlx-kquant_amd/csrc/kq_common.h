@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "kq.h"
 
 enum KqCodec : int {
@@ -56,6 +58,21 @@ const uint8_t* kq_device_grids(void);
     hipError_t _e = (expr);                                                             \
     if (_e != hipSuccess)                                                               \
       return kq_set_error(KQ_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(_e));  \
+  } while (0)
+
+// hipFuncSetAttribute applies to the current device only: one flag per (call site = kernel instantiation, device).
+// Two host threads may both set the attribute the first time; the call is idempotent.
+#define KQ_SET_MAX_LDS_ONCE(kern, bytes)                                                          \
+  do {                                                                                            \
+    static std::atomic<uint64_t> _kq_done{0};                                                     \
+    int _kq_dev = 0;                                                                              \
+    KQ_HIP_CHECK(hipGetDevice(&_kq_dev));                                                         \
+    const uint64_t _kq_bit = 1ull << (_kq_dev & 63);                                              \
+    if (!(_kq_done.load(std::memory_order_acquire) & _kq_bit)) {                                  \
+      KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                       \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes))); \
+      _kq_done.fetch_or(_kq_bit, std::memory_order_release);                                      \
+    }                                                                                             \
   } while (0)
 
 // ---- per-op launchers implemented in the .hip files ----

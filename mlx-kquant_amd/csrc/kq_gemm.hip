@@ -230,12 +230,7 @@ int launch_gemm_mt(const _Float16* xh, const _Float16* xhl, const float* rs, con
   const int mtiles = (M + TM - 1) / TM, ntiles = (N + BN - 1) / BN;
   const size_t lds = (size_t)(TM * A_STRIDE + BN * G::LBPB + TM * 32 + BN * 2) * (DB ? 2 : 1);
   auto kern = kquant_gemm_kernel<C, DT, MT, WAVES, DB>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)lds));
-    attr_set = true;
-  }
+  KQ_SET_MAX_LDS_ONCE((kern), lds);
   const int splits = part ? ((K >> 8) + sb_per_split - 1) / sb_per_split : 1;
   hipLaunchKernelGGL(kern, dim3(mtiles * ntiles, splits), dim3(G::THREADS), lds, s, xh, xhl, rs, w,
                      static_cast<uint16_t*>(y), M, N, K, mtiles, sb_per_split, part);

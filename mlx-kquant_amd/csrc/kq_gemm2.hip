@@ -542,11 +542,7 @@ int launch_gemm2(const _Float16* xh, const _Float16* xhl, const float* rs, const
   constexpr int lds = g2_lds_bytes<C, WAVES, KS>();
   static_assert(lds <= 160 * 1024, "tile does not fit the LDS of a CU");
   auto kern = kquant_gemm2_kernel<C, DT, WAVES, KS>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    attr_set = true;
-  }
+  KQ_SET_MAX_LDS_ONCE((kern), lds);
   hipLaunchKernelGGL(kern, dim3(mtiles * ntiles), dim3(64 * WAVES), lds, s, xh, xhl, rs, w, static_cast<uint16_t*>(y), M, N,
                      K, mtiles);
   KQ_HIP_CHECK(hipGetLastError());

@@ -1273,12 +1273,7 @@ int launch_skinny(SkArgs a, int items, void* ws, hipStream_t s) {
         const size_t lds3 = sk3_lds_bytes<C>(kch, MB);
         a.rows_per_tile = 32;
         a.kch = kch;
-        static bool attr3_set = false;
-        if (!attr3_set) {
-          KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(skinny3_kernel<C, DT, MB>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 120 * 1024));
-          attr3_set = true;
-        }
+        KQ_SET_MAX_LDS_ONCE((skinny3_kernel<C, DT, MB>), 120 * 1024);
         hipLaunchKernelGGL((skinny3_kernel<C, DT, MB>), dim3(tiles3, 1, splits), dim3(SK_THREADS), lds3, s, a);
         KQ_HIP_CHECK(hipGetLastError());
         if (splits > 1) {
@@ -1299,14 +1294,8 @@ int launch_skinny(SkArgs a, int items, void* ws, hipStream_t s) {
       const size_t lds2 = sk2_lds_bytes<C>(kch, MB, two ? 2 : 1);
       a.rows_per_tile = rows;
       a.kch = kch;
-      static bool attr2_set = false;
-      if (!attr2_set) {
-        KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(skinny2_kernel<C, DT, MB, 1>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 120 * 1024));
-        KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(skinny2_kernel<C, DT, MB, 2>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 120 * 1024));
-        attr2_set = true;
-      }
+      KQ_SET_MAX_LDS_ONCE((skinny2_kernel<C, DT, MB, 1>), 120 * 1024);
+      KQ_SET_MAX_LDS_ONCE((skinny2_kernel<C, DT, MB, 2>), 120 * 1024);
       if (two)
         hipLaunchKernelGGL((skinny2_kernel<C, DT, MB, 2>), dim3(tiles, 1, splits), dim3(SK_THREADS), lds2, s, a);
       else
@@ -1326,12 +1315,7 @@ int launch_skinny(SkArgs a, int items, void* ws, hipStream_t s) {
   a.rows_per_tile = rows;
   a.kch = kch;
   auto kern = skinny_kernel<C, DT, MB, GLU>;
-  static bool attr_set = false;  // per instantiation
-  if (!attr_set) {
-    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     120 * 1024));
-    attr_set = true;
-  }
+  KQ_SET_MAX_LDS_ONCE((kern), 120 * 1024);
   hipLaunchKernelGGL(kern, dim3(tiles, items, splits), dim3(SK_THREADS), lds, s, a);
   KQ_HIP_CHECK(hipGetLastError());
   if (splits > 1) {

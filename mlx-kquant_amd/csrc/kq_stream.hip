@@ -1393,14 +1393,16 @@ __global__ __launch_bounds__(256) void st_splitk_reduce_kernel(const float* __re
 }
 
 int st_num_cus() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    cus = n;
+  // compute units of the current device, looked up once per device
+  static std::atomic<int> cus[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev].store(n, std::memory_order_relaxed);
   }
-  return cus;
+  return n;
 }
 
 // K split: a workgroup takes at most 16 superblocks (32 where the kernel with eight units per wave applies: codecs
@@ -1475,11 +1477,7 @@ int st_launch_one(StArgs a, int splits, hipStream_t s) {
   static_assert(lds <= 160 * 1024, "workgroup does not fit the LDS of a CU");
   constexpr int WGS = lds <= 80 * 1024 && NW == 4 ? 2 : 1;
   auto kern = stream_gemv_kernel<C, DT, MB, D, WGS, XU, NW>;
-  static bool attr_set = false;  // per instantiation
-  if (!attr_set) {
-    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
-  }
+  KQ_SET_MAX_LDS_ONCE((kern), lds);
   int gx = WGS * st_num_cus() / splits;
   if (gx < 1) gx = 1;
   // rows per tile: when the 32-row tiles do not fill a whole number of rounds of the resident workgroups, the
@@ -1534,11 +1532,7 @@ int st_launch_gather(StArgs a, int entries, hipStream_t s) {
   static_assert(lds <= 160 * 1024, "workgroup does not fit the LDS of a CU");
   constexpr int WGS = lds <= 80 * 1024 && NW == 4 ? 2 : 1;
   auto kern = stream_gemv_kernel<C, DT, 1, D, WGS, XU, NW, GM>;
-  static bool attr_set = false;  // per instantiation
-  if (!attr_set) {
-    KQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
-  }
+  KQ_SET_MAX_LDS_ONCE((kern), lds);
   a.rpt = ST_ROWS;
   a.tiles_per_entry = (a.N + ST_ROWS - 1) / ST_ROWS;
   a.tiles = a.tiles_per_entry;

@@ -26,7 +26,7 @@ __all__ = [
     "codecs", "codec_has_matmul", "codec_has_moe_glu", "dequantize", "quantized_matmul", "quantized_matmul_qmv_bias",
     "gather_qmm", "expert_tile_map", "gather_qmm_seg",
     "moe_glu_gather_kq", "gather_qmv_kq", "moe_glu_gather_shexp_kq", "gather_qmv_mix_kq", "gather_qmv_mix_ns_kq",
-    "moe_router_topk", "mxfp4_packed_to_wire", "mxfp4_wire_to_packed", "set_packed_cache", "moe_glu_gather", "gather_qmv_bias",
+    "moe_router_topk", "mxfp4_packed_to_wire", "mxfp4_wire_to_packed", "set_packed_cache", "invalidate_packed_cache", "moe_glu_gather", "gather_qmv_bias",
     "gather_qmv_mix_bias", "quantize", "codec_geometry", "CODEC_GEOMETRY", "bytes_per_row",
     "weights_per_row", "lib_path",
 ]
@@ -755,20 +755,41 @@ def mxfp4_packed_to_wire(w, scales, *, stream=None):
     return wire
 
 
-# Wire forms of the packed stacks the three packed-layout ops below were called with: the reference's kernels read
-# the packed layout directly (src/kquant_moe_glu.cpp:149-275); here a stack is rewritten to wire form on the device
-# the first time an op sees it and the result is kept for as long as the packed tensors live and stay unmodified
-# (torch's version counters), so a model that calls these ops every step converts each stack once.  The copy costs
-# 17/16 of the stack's bytes of device memory; set_packed_cache(0) turns the cache off (one conversion per call).
+# Wire forms of packed stacks.  The reference's kernels read the packed layout directly on every call
+# (src/kquant_moe_glu.cpp:149-275); here a stack is rewritten to wire form on the device before the wire-form
+# kernels run, once per call by default.  set_packed_cache(n) lets the three packed-layout ops below keep the wire
+# form of up to n stacks between calls (17/16 of a stack's bytes of device memory each).  A kept wire form is used
+# again only while the same two tensor objects are passed and their torch version counters stand still; writes that
+# bypass those counters (w.data.copy_(), set_(), a kernel writing through data_ptr()) are not seen, so a caller who
+# reloads weights that way calls invalidate_packed_cache(w) afterwards.  That is why the cache is off by default.
 _PACKED_CACHE = {}
-_PACKED_CACHE_MAX = 256
+_PACKED_CACHE_MAX = 0
 
 
 def set_packed_cache(max_entries: int) -> None:
-    """Number of packed mxfp4 stacks whose wire form is kept between calls (0: convert on every call)."""
+    """Number of packed mxfp4 stacks whose wire form is kept between calls (0, the default: convert on every call).
+    A kept wire form follows in-place changes made through torch ops on the tensor itself; after a write torch's
+    version counters do not see (w.data.copy_(), set_(), raw-pointer writes) call invalidate_packed_cache."""
     global _PACKED_CACHE_MAX
     _PACKED_CACHE_MAX = max(0, int(max_entries))
-    _PACKED_CACHE.clear()
+    _drop_packed(list(_PACKED_CACHE))
+
+
+def invalidate_packed_cache(w=None) -> None:
+    """Forget the kept wire form of the packed stack whose codes tensor is w (every stack when w is None)."""
+    _drop_packed([k for k, v in _PACKED_CACHE.items() if w is None or v[0]() is w or v[1]() is w])
+
+
+def _drop_packed(keys):
+    # A dropped wire form may still be read by kernels in flight: every stream other than the allocating one that
+    # used it was named to the caching allocator with record_stream, so the block is not handed out again before
+    # those streams pass the point of release.
+    for k in keys:
+        _PACKED_CACHE.pop(k, None)
+
+
+def _consumer_stream(t, stream):
+    return stream if isinstance(stream, torch.cuda.Stream) else torch.cuda.current_stream(t.device)
 
 
 def _wire_of_packed(w, scales, stream):
@@ -776,20 +797,24 @@ def _wire_of_packed(w, scales, stream):
     if _PACKED_CACHE_MAX == 0:
         return mxfp4_packed_to_wire(w, scales, stream=stream)
     key = (w.data_ptr(), scales.data_ptr(), tuple(w.shape), str(w.device))
+    cs = _consumer_stream(w, stream)
     hit = _PACKED_CACHE.get(key)
     if hit is not None:
-        wref, sref, ver, wire, ev = hit
+        wref, sref, ver, wire, ev, made_on = hit
         if wref() is w and sref() is scales and ver == (w._version, scales._version):
-            if not ev.query():  # still in flight: order the consumer's stream after the conversion
-                (stream if isinstance(stream, torch.cuda.Stream) else torch.cuda.current_stream(w.device)).wait_event(ev)
+            if cs != made_on:
+                cs.wait_event(ev)          # order this stream after the conversion
+                wire.record_stream(cs)     # and keep the block from reuse while this stream reads it
             return wire
-        _PACKED_CACHE.pop(key, None)
+        _drop_packed([key])
     wire = mxfp4_packed_to_wire(w, scales, stream=stream)
     ev = torch.cuda.Event()
-    ev.record(stream if isinstance(stream, torch.cuda.Stream) else torch.cuda.current_stream(w.device))
-    if len(_PACKED_CACHE) >= _PACKED_CACHE_MAX:
-        _PACKED_CACHE.pop(next(iter(_PACKED_CACHE)))
-    _PACKED_CACHE[key] = (weakref.ref(w), weakref.ref(scales), (w._version, scales._version), wire, ev)
+    ev.record(cs)
+    if cs != torch.cuda.current_stream(w.device):
+        wire.record_stream(cs)             # allocated on the current stream, written and read on cs
+    while len(_PACKED_CACHE) >= _PACKED_CACHE_MAX:
+        _drop_packed([next(iter(_PACKED_CACHE))])
+    _PACKED_CACHE[key] = (weakref.ref(w), weakref.ref(scales), (w._version, scales._version), wire, ev, cs)
     weakref.finalize(w, _PACKED_CACHE.pop, key, None)
     return wire
 

@@ -1,5 +1,7 @@
-"""GPU parity: the device encoder behind kq.quantize writes the host encoder's bytes (the host encoder is pinned
-against the reference's fixtures in tests/test_encode.py), and what it writes decodes within the codec's bound."""
+"""GPU parity: the device encoder behind kq.quantize reproduces the reference's own fixture bytes inside the
+reference's x86-vs-Metal band, writes the host encoder's bytes, and what it writes decodes within the codec's bound."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -41,6 +43,44 @@ def test_device_encoder_writes_host_bytes(kq, codec):
     live = [r for r in range(rows) if r not in (3, 9)]  # the outlier row is covered by the byte comparison only
     assert np.linalg.norm(back[live] - w[live]) / np.linalg.norm(w[live]) < BOUND[codec]
     assert not back[3].any()
+
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+KCODECS = ["q2_k", "q3_k", "q4_k", "q5_k", "q6_k"]
+
+
+@pytest.mark.parametrize("codec", KCODECS)
+def test_device_encoder_reproduces_reference_fixture_bytes(kq, codec):
+    """The device encoder against the reference's own vectors, directly: the committed wire fixtures were minted
+    by the reference's encoder from default_rng(1234) (tests/gen_fixtures.py:62-63) on Metal, and the reference's
+    x86 encoder lands within a few ULP-tie bytes of them (tests/test_encode.py:203-250).  kq.quantize on cuda:0
+    must land in the same band, and what it writes must decode to what the fixture decodes to."""
+    gold = np.load(os.path.join(GOLD, f"{codec}.npz"))["wire"]
+    w = (np.random.default_rng(1234).standard_normal((256, 512)) * 0.1).astype(np.float32)
+    dev, _ = kq.quantize(torch.from_numpy(w).cuda(), codec)
+    mine = dev.cpu().numpy()
+    assert mine.shape == gold.shape
+    frac = np.mean(mine != gold)
+    assert frac < 2e-3, (codec, frac)
+    a, b = O.dequantize(mine, codec), O.dequantize(gold, codec)
+    assert np.linalg.norm(a - b) / np.linalg.norm(b) < 2e-2
+    # the fixture's bytes, decoded on the device, are the oracle's decode bit for bit
+    got = kq.dequantize(torch.from_numpy(gold).cuda(), None, codec, dtype=torch.float32).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32).ravel(), b.view(np.uint32).ravel())
+
+
+def test_device_encoder_reproduces_reference_moe_fixture_bytes(kq):
+    """Same for the expert-stack fixtures (default_rng(4321), four experts of 128 x 512, tests/gen_fixtures.py:80-89)."""
+    rng = np.random.default_rng(4321)
+    ws = [(rng.standard_normal((128, 512)) * 0.1).astype(np.float32) for _ in range(4 * len(KCODECS))]
+    for ci, codec in enumerate(KCODECS):
+        gold = np.load(os.path.join(GOLD, f"{codec}_moe.npz"))["wire"]
+        stack = np.stack(ws[4 * ci:4 * ci + 4])
+        dev, _ = kq.quantize(torch.from_numpy(stack).cuda(), codec)   # leading (expert) dimension kept
+        mine = dev.cpu().numpy()
+        assert mine.shape == gold.shape
+        for e in range(4):
+            assert np.mean(mine[e] != gold[e]) < 3e-3, (codec, e)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -111,8 +111,10 @@ def test_mix_bias_matches_ns_op_with_zero_bias(kq):
 
 
 def test_packed_stack_wire_form_is_kept_and_follows_in_place_changes(kq):
-    """The packed-layout ops keep a stack's wire form between calls: a second call on the same tensors gives the
-    same bytes, an in-place change of the stack is seen by the next call, and with the cache off every call converts."""
+    """By default every call converts the packed stack, so any write to it is seen.  With set_packed_cache(n) a
+    stack's wire form is kept between calls: a second call gives the same bytes, an in-place change through torch
+    ops is seen by the next call, a write that bypasses torch's version counters is seen after
+    invalidate_packed_cache, and a call on another stream uses the kept form correctly."""
     E, N, K, T, R = 3, 64, 288, 5, 2
     rng = np.random.default_rng(17)
     gc, gs, gw = _packed_stack(E, N, K, seed=12)
@@ -121,20 +123,44 @@ def test_packed_stack_wire_form_is_kept_and_follows_in_place_changes(kq):
     idx_dev = torch.from_numpy(idx).cuda()
     hb, ht = make_x((T, R, K), "bfloat16", seed=19, scale=0.2)
     w_dev, s_dev, b_dev = _dev_words(gw), torch.from_numpy(gs).cuda(), torch.from_numpy(gb).cuda()
-    first = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
-    again = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
-    assert torch.equal(first, again)
-    assert rel_l2(dev_to_bits(first), O.gather_qmv(hb, _wire_from_codes(gc, gs), "mxfp4", idx, gb, "bfloat16"), "bfloat16") <= TOL
-    # double every weight of the stack in place (scale exponents + 1): the kept wire form must not be used
-    s_dev.add_(1)
-    gs2 = gs + 1
-    changed = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
-    want = O.gather_qmv(hb, _wire_from_codes(gc, gs2), "mxfp4", idx, gb, "bfloat16")
-    assert rel_l2(dev_to_bits(changed), want, "bfloat16") <= TOL
-    assert not torch.equal(changed, first)
+
+    def want(scales):
+        return O.gather_qmv(hb, _wire_from_codes(gc, scales), "mxfp4", idx, gb, "bfloat16")
+
+    # default: no cache, a write through .data (which torch's version counter does not see) changes the result
+    base = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+    assert rel_l2(dev_to_bits(base), want(gs), "bfloat16") <= TOL
+    s_dev.data.add_(1)
+    bumped = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+    assert rel_l2(dev_to_bits(bumped), want(gs + 1), "bfloat16") <= TOL
+    assert not torch.equal(bumped, base)
+    s_dev.data.sub_(1)
     try:
-        kq.set_packed_cache(0)
-        off = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
-        assert torch.equal(off, changed)
+        kq.set_packed_cache(8)
+        first = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+        again = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+        assert torch.equal(first, again) and torch.equal(first, base)
+        # a consumer on another stream waits for the conversion and reads the same bytes
+        side = torch.cuda.Stream()
+        other = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev, stream=side)
+        side.synchronize()
+        assert torch.equal(other, first)
+        # double every weight of the stack in place (scale exponents + 1): the kept wire form must not be used
+        s_dev.add_(1)
+        changed = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+        assert rel_l2(dev_to_bits(changed), want(gs + 1), "bfloat16") <= TOL
+        assert not torch.equal(changed, first)
+        # a write the version counters miss needs the explicit call
+        s_dev.data.add_(1)
+        kq.invalidate_packed_cache(w_dev)
+        reloaded = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+        assert rel_l2(dev_to_bits(reloaded), want(gs + 2), "bfloat16") <= TOL
+        assert not torch.equal(reloaded, changed)
+        # eviction at the entry limit keeps the results right
+        kq.set_packed_cache(1)
+        w2, s2 = w_dev.clone(), s_dev.clone()
+        a2 = kq.gather_qmv_bias(ht, w2, s2, b_dev, idx_dev)
+        a1 = kq.gather_qmv_bias(ht, w_dev, s_dev, b_dev, idx_dev)
+        assert torch.equal(a1, reloaded) and torch.equal(a2, reloaded)
     finally:
-        kq.set_packed_cache(256)
+        kq.set_packed_cache(0)

@@ -65,3 +65,56 @@ def test_noalloc_refuses_oversized_workspace(kq):
                             torch.cuda.current_stream().cuda_stream)
     assert rc == KQ_ERR_WORKSPACE
     assert b"workspace" in lib.kq_last_error()
+
+
+def test_noalloc_leaves_device_memory_alone(kq):
+    """The property the entry point exists for: the free device memory reported by the runtime is the same before
+    and after a first-of-its-shape call and a repeated call (torch's caching allocator is not involved: every buffer
+    is made beforehand, the library's own buffer lives in its code object)."""
+    lib = kq._load()
+    cid = lib.kq_codec_id(b"q5_k")
+    M, N, K = 2, 2048, 4096  # a shape no other test of this file has run: first-use set-up of its kernel included
+    wire = O.synth_wire("q5_k", N * K // 256, seed=61).reshape(N, K // 256 * 176)
+    w = wire_to_dev(wire)
+    xb, xt = make_x((M, K), "bfloat16", seed=62)
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device=w.device)
+    stream = torch.cuda.current_stream().cuda_stream
+    # load the library's code object and take the buffer's address with another shape first
+    _both(kq, lib, "q4_k", 1, 512, 1024, "bfloat16", 63)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        assert lib.kq_qmm_noalloc(xt.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K, cid, KQ_BF16, stream) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    assert rel_l2(dev_to_bits(y), O.qmm(xb, wire, "q5_k", True, "bfloat16"), "bfloat16") <= 1e-3
+
+
+def test_noalloc_replayed_from_a_hip_graph(kq):
+    """The advertised use: kq_qmm_noalloc captured into a HIP graph after one eager call of the same shape (the
+    first call on a device looks the buffer up and sets kernel attributes, which is set-up work and stays outside
+    a capture), replayed several times with the built-in buffer dirtied by another shape between the replays."""
+    lib = kq._load()
+    cid = lib.kq_codec_id(b"q4_k")
+    M, N, K = 1, 4096, 4096  # split-K plan: partial sums in the built-in buffer
+    wire = O.synth_wire("q4_k", N * K // 256, seed=71).reshape(N, K // 256 * 144)
+    w = wire_to_dev(wire)
+    xb, xt = make_x((M, K), "bfloat16", seed=72)
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device=w.device)
+    cur = torch.cuda.current_stream().cuda_stream
+    assert lib.kq_qmm_noalloc(xt.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K, cid, KQ_BF16, cur) == 0
+    torch.cuda.synchronize()
+    eager = dev_to_bits(y).copy()
+    assert rel_l2(eager, O.qmm(xb, wire, "q4_k", True, "bfloat16"), "bfloat16") <= 1e-3
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        st = torch.cuda.current_stream().cuda_stream
+        assert lib.kq_qmm_noalloc(xt.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K, cid, KQ_BF16, st) == 0
+    for rep in range(3):
+        _both(kq, lib, "q6_k", 3, 1024, 2048, "float16", 80 + rep)  # another shape writes over the buffer
+        y.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(dev_to_bits(y), eager), rep
