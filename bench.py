@@ -303,7 +303,7 @@ def read_ceiling(torch, dev, sizes):
         dsts = [torch.empty_like(srcs[0]) for _ in range(ncopies)]
 
         def summer(v):
-            return lambda stream=None: torch.sum(v, dtype=torch.int64, out=acc)
+            return lambda stream=None: torch.sum(v, dim=(0,), dtype=torch.int64, out=acc)
 
         def copier(v, d):
             return lambda stream=None: d.copy_(v)
@@ -354,10 +354,12 @@ def main():
                          "followed by 20 cold launches of the headline GEMV, nothing else")
     ap.add_argument("--probe-codec", default=None, metavar="CODEC",
                     help="counter probe for `rocprofv3 --pmc`: 20 launches of the M = 1 GEMV 8192 -> 8192 in CODEC "
-                         "(random structurally valid wire), nothing else")
+                         "(random structurally valid wire; --gemm-tile applies), nothing else")
     ap.add_argument("--probe-prefill", default=None, metavar="CODEC",
                     help="counter probe for `rocprofv3 --pmc`: 5 launches of the prefill GEMM [2048, 8192] x "
                          "[28672, 8192]^T in CODEC (random structurally valid wire), nothing else")
+    ap.add_argument("--probe-n", type=int, default=28672, metavar="N",
+                    help="weight rows of the --probe-prefill matrix (24576 = whole rounds of 256 x 256 tiles on 256 CUs)")
     ap.add_argument("--probe-moe", type=int, default=None, metavar="TOKENS",
                     help="counter probe for `rocprofv3 --pmc`: 10 launches each of the q4_k GLU op and the q6_k down "
                          "op of the 128-expert top-8 MoE at TOKENS tokens, nothing else")
@@ -410,7 +412,8 @@ def main():
         return
 
     if args.probe_prefill:
-        c, m, n, k = args.probe_prefill, 2048, 28672, 8192
+        c, m, n, k = args.probe_prefill, 2048, args.probe_n, 8192
+        abi.lib.kq_set_gemm_tile_rows(args.gemm_tile)
         w = synth_wire_torch(c, n, k, 7, dev)
         call = abi.qmm(randx((m, k)), w, c, n, k)
         for i in range(5):

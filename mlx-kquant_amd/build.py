@@ -26,6 +26,7 @@ SOURCES = [
     ("kq_stream.hip", ["-Wno-inline-asm", "-DKQ_STREAM_PART=2"], "kq_stream_gather"),
     ("kq_gemm.hip", []),
     ("kq_gemm2.hip", ["-Wno-inline-asm"]),
+    ("kq_gemm3.hip", ["-Wno-inline-asm"]),
     ("kq_moe.hip", []),
     ("kq_anymma.hip", ["-ffp-contract=off"]),
     # one source, three objects: its kernel families are instantiated in parallel

@@ -141,7 +141,12 @@ int kq_launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K
 // 128 x 256-tile prefill GEMM (q4_k / q5_k) on the outputs of the activation prepass (rows padded to 128).
 bool kq_gemm2_supported(int M, int N, int K, int codec);
 int kq_launch_gemm2(const void* xh, const void* xhl, const float* rs, const uint8_t* w, void* y, int M, int N, int K,
-                    int codec, int dtype, int shape, hipStream_t s);
+                    int codec, int dtype, int shape, hipStream_t s, int nt0 = 0, int ntiles = -1);
+// 256 x 256-tile prefill GEMM (q4_k / q5_k, 256-row wave tiles on one accumulator set) on the same prepass outputs
+// (mrows >= M prepared rows): column tiles nt0 .. nt0 + ntiles - 1 of 256 weight rows each.
+bool kq_gemm3_supported(int M, int mrows, int N, int K, int codec);
+int kq_launch_gemm3(const void* xh, const void* xhl, const float* rs, const uint8_t* w, void* y, int M, int mrows, int N,
+                    int K, int codec, int dtype, int nt0, int ntiles, hipStream_t s);
 // The same tile kernel for q2_k / q3_k (M >= 256, tiles filling the chip): runs its own activation prepass.
 bool kq_gemm2_low_supported(int M, int N, int K, int codec);
 size_t kq_gemm2_low_workspace_bytes(int M, int K);

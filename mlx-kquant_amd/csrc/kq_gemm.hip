@@ -13,7 +13,7 @@
 // row-per-lane ds_read_b128 fragment fetch free of bank conflicts).
 #include "kq_mma.h"
 
-static int g_gemm_tile = 0;  // kq_set_gemm_tile_rows: 64, 128, 256, 512 or 513 forces the tile shape, 0 = automatic
+static int g_gemm_tile = 0;  // kq_set_gemm_tile_rows: 64, 128, 256, 512, 513 or 1024 forces the tile shape, 0 = automatic
 
 namespace {
 
@@ -244,6 +244,19 @@ int launch_gemm_mt(const _Float16* xh, const _Float16* xhl, const float* rs, con
 }
 
 
+int gemm_num_cus() {
+  // compute units of the current device, looked up once per device
+  static std::atomic<int> cus[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
 template <int C, int DT>
 int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, void* ws, size_t ws_bytes, hipStream_t s) {
   const int mpad = ((M + BM - 1) / BM) * BM, nsb = K >> 8;
@@ -262,11 +275,34 @@ int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, v
   // 128 x 256 tiles with 128-row wave tiles and direct-to-LDS loads (kq_gemm2.hip, q4_k / q5_k): one decoded
   // weight fragment feeds four MFMAs instead of two.  Taken when the matrix fills the 256 CUs with whole
   // workgroups of that size; `512` forces it, `513` its 128 x 128 / four-wave form.
+  if constexpr (C != KQ_Q6_K) {
+    // 256 x 256 tiles with 256-row wave tiles on one accumulator set (kq_gemm3.hip): a decoded fragment feeds eight
+    // MFMAs.  Such tiles are few (2048 x 28672: 896 on 256 CUs), so they take the column tiles that fill whole rounds
+    // of one workgroup per CU and the 128 x 256 kernel takes the rest (there: 96 + 16 column tiles = 3 + 1 rounds);
+    // a matrix of less than one round runs on them whole when it fills three quarters of the CUs (512 x 28672: 224
+    // workgroups, 10 % faster than 448 of the 128-row kernel).  `1024` forces them for every column tile, `512` /
+    // `513` keep the 128-row kernels.
+    const int nt256 = (N + 255) / 256;
+    if (tile == 1024 && kq_gemm3_supported(M, mpad, N, K, C)) return kq_launch_gemm3(xh, xhl, rs, w, y, M, mpad, N, K, C, DT, 0, nt256, s);
+    if (tile == 0 && M >= 256 && kq_gemm3_supported(M, mpad, N, K, C)) {
+      const int mt256 = (M + 255) / 256, cus = gemm_num_cus();
+      const int64_t tiles = (int64_t)mt256 * nt256;
+      int tall = (int)((tiles / cus) * cus / mt256);  // column tiles in whole rounds
+      if (tall == 0 && 4 * tiles >= 3 * (int64_t)cus) tall = nt256;
+      if (tall > 0) {
+        int rc = kq_launch_gemm3(xh, xhl, rs, w, y, M, mpad, N, K, C, DT, 0, tall, s);
+        if (rc != KQ_OK || tall == nt256) return rc;
+        rc = kq_launch_gemm2(xh, xhl, rs, w, y, M, N, K, C, DT, 0, s, tall, nt256 - tall);
+        if (rc != KQ_ERR_UNSUPPORTED) return rc;
+        return kq_launch_gemm3(xh, xhl, rs, w, y, M, mpad, N, K, C, DT, tall, nt256 - tall, s);
+      }
+    }
+  }
   if (tile == 512 || tile == 513 || (tile == 0 && M >= 256 && (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 256)) {
     const int rc = kq_launch_gemm2(xh, xhl, rs, w, y, M, N, K, C, DT, tile == 513 ? 1 : 0, s);
     if (rc != KQ_ERR_UNSUPPORTED) return rc;
   }
-  if (tile == 512 || tile == 513) tile = 0;
+  if (tile == 512 || tile == 513 || tile == 1024) tile = 0;
   if (tile == 256 && C != KQ_Q4_K) tile = 0;
   if (tile == 0) {
     const int64_t wgs = (int64_t)((M + 63) / 64) * ((N + 255) / 256);
@@ -337,5 +373,5 @@ int kq_launch_act_prepass(const void* x, void* xh, void* xhl, float* rs, int M, 
 }
 
 extern "C" void kq_set_gemm_tile_rows(int rows) {
-  g_gemm_tile = (rows == 64 || rows == 128 || rows == 256 || rows == 512 || rows == 513) ? rows : 0;
+  g_gemm_tile = (rows == 64 || rows == 128 || rows == 256 || rows == 512 || rows == 513 || rows == 1024) ? rows : 0;
 }

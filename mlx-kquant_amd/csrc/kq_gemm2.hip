@@ -69,7 +69,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
                                                                      const float* __restrict__ rs,
                                                                      const uint8_t* __restrict__ w,
                                                                      uint16_t* __restrict__ y, int M, int N, int K,
-                                                                     int mtiles) {
+                                                                     int mtiles, int nt0) {
   using G = G2Wire<C>;
   constexpr bool LOW = g2_low<C>(), IQ4 = C == KQ_IQ4_XS;
   constexpr int G2_H_STAGE = G2_TM * G::HB;
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, kg = lane >> 5;
-  const int mt = blockIdx.x % mtiles, nt = blockIdx.x / mtiles;  // consecutive workgroups share the weight columns
+  const int mt = blockIdx.x % mtiles, nt = nt0 + blockIdx.x / mtiles;  // consecutive workgroups share the weight columns
   const int m0 = mt * G2_TM, n0 = nt * G2_BN;
   const int nsb = K >> 8;
   const uint32_t row_bytes = (uint32_t)nsb * G::BPB;
@@ -536,24 +536,25 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void kquant_gemm2_k
 
 template <int C, int DT, int WAVES, int KS>
 int launch_gemm2(const _Float16* xh, const _Float16* xhl, const float* rs, const uint8_t* w, void* y, int M, int N, int K,
-                 hipStream_t s) {
+                 hipStream_t s, int nt0 = 0, int ntiles_sel = -1) {
   constexpr int BN = 32 * WAVES;
-  const int mtiles = (M + G2_TM - 1) / G2_TM, ntiles = (N + BN - 1) / BN;
+  const int mtiles = (M + G2_TM - 1) / G2_TM, ntiles = ntiles_sel >= 0 ? ntiles_sel : (N + BN - 1) / BN;
+  if (ntiles == 0) return KQ_OK;
   constexpr int lds = g2_lds_bytes<C, WAVES, KS>();
   static_assert(lds <= 160 * 1024, "tile does not fit the LDS of a CU");
   auto kern = kquant_gemm2_kernel<C, DT, WAVES, KS>;
   KQ_SET_MAX_LDS_ONCE((kern), lds);
   hipLaunchKernelGGL(kern, dim3(mtiles * ntiles), dim3(64 * WAVES), lds, s, xh, xhl, rs, w, static_cast<uint16_t*>(y), M, N,
-                     K, mtiles);
+                     K, mtiles, nt0);
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }
 
 template <int C, int DT>
 int launch_gemm2_shape(const _Float16* xh, const _Float16* xhl, const float* rs, const uint8_t* w, void* y, int M, int N,
-                       int K, int shape, hipStream_t s) {
+                       int K, int shape, hipStream_t s, int nt0, int ntiles) {
   if (shape == 1) return launch_gemm2<C, DT, 4, 64>(xh, xhl, rs, w, y, M, N, K, s);
-  return launch_gemm2<C, DT, 8, 128>(xh, xhl, rs, w, y, M, N, K, s);
+  return launch_gemm2<C, DT, 8, 128>(xh, xhl, rs, w, y, M, N, K, s, nt0, ntiles);
 }
 
 // activation prepass with the sums of the 16-weight sub-blocks (q2_k / q3_k)
@@ -628,16 +629,16 @@ bool kq_gemm2_supported(int M, int N, int K, int codec) {
          (int64_t)N * (K >> 8) * 176 < ((int64_t)1 << 32) && (int64_t)K * 2 * 128 < ((int64_t)1 << 32);
 }
 
-// shape 0: 128 x 256 tiles on eight waves, K steps of 128; shape 1: 128 x 128 tiles on four waves, K steps of 64
-// (two workgroups per CU)
+// shape 0: 128 x 256 tiles on eight waves, K steps of 128 (column tiles nt0 .. nt0 + ntiles - 1; ntiles < 0: all);
+// shape 1: 128 x 128 tiles on four waves, K steps of 64 (two workgroups per CU, always the whole matrix)
 int kq_launch_gemm2(const void* xh, const void* xhl, const float* rs, const uint8_t* w, void* y, int M, int N, int K,
-                    int codec, int dtype, int shape, hipStream_t s) {
+                    int codec, int dtype, int shape, hipStream_t s, int nt0, int ntiles) {
   if (!kq_gemm2_supported(M, N, K, codec)) return KQ_ERR_UNSUPPORTED;
   const _Float16* a = static_cast<const _Float16*>(xh);
   const _Float16* h = static_cast<const _Float16*>(xhl);
   if (codec == KQ_Q4_K)
-    return dtype == KQ_F16 ? launch_gemm2_shape<KQ_Q4_K, KQ_F16>(a, h, rs, w, y, M, N, K, shape, s)
-                           : launch_gemm2_shape<KQ_Q4_K, KQ_BF16>(a, h, rs, w, y, M, N, K, shape, s);
-  return dtype == KQ_F16 ? launch_gemm2_shape<KQ_Q5_K, KQ_F16>(a, h, rs, w, y, M, N, K, shape, s)
-                         : launch_gemm2_shape<KQ_Q5_K, KQ_BF16>(a, h, rs, w, y, M, N, K, shape, s);
+    return dtype == KQ_F16 ? launch_gemm2_shape<KQ_Q4_K, KQ_F16>(a, h, rs, w, y, M, N, K, shape, s, nt0, ntiles)
+                           : launch_gemm2_shape<KQ_Q4_K, KQ_BF16>(a, h, rs, w, y, M, N, K, shape, s, nt0, ntiles);
+  return dtype == KQ_F16 ? launch_gemm2_shape<KQ_Q5_K, KQ_F16>(a, h, rs, w, y, M, N, K, shape, s, nt0, ntiles)
+                         : launch_gemm2_shape<KQ_Q5_K, KQ_BF16>(a, h, rs, w, y, M, N, K, shape, s, nt0, ntiles);
 }

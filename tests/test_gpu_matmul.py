@@ -340,6 +340,62 @@ def test_qmm_prefill_gemm_128x256_tiles(kq, codec):
         lib.kq_set_gemm_tile_rows(0)
 
 
+@pytest.mark.parametrize("codec", ["q4_k", "q5_k"])
+def test_qmm_prefill_gemm_256x256_tiles(kq, codec):
+    """The 256-row kernel (kq_set_gemm_tile_rows(1024): running sums kept in units of the current superblock scale):
+    one, two, four and nine superblocks of K (prologue only, both wire stages, stage reuse), ragged M and N tiles,
+    fewer rows than a tile, both activation dtypes; and the automatic choice, which splits the column tiles between
+    this kernel and the 128-row one."""
+    lib = kq._load()
+    try:
+        for rows in (1024, 0):
+            lib.kq_set_gemm_tile_rows(rows)
+            for M, N, K, dtype in ((64, 40, 256, "bfloat16"), (130, 257, 512, "float16"), (300, 520, 2304, "bfloat16"),
+                                   (256, 256, 1024, "bfloat16"), (513, 700, 1024, "float16")):
+                wire = _wire(codec, N, K, seed=63)
+                xb, xt = make_x((M, K), dtype, seed=64)
+                got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+                want = O.qmm(xb, wire, codec, True, dtype)
+                assert rel_l2(got, want, dtype) <= TOL, (codec, rows, M, N, K, dtype)
+    finally:
+        lib.kq_set_gemm_tile_rows(0)
+
+
+def test_qmm_prefill_gemm_256x256_tiles_scale_corner_cases(kq):
+    """Superblocks the unit chain of the 256-row kernel must survive: d = 0 with a live dmin (the unit is kept and the
+    integers are fed as zeros), a subnormal d next to a large dmin, d falling and rising by 2^20 between neighbouring
+    superblocks, dmin = 0, and a first superblock with d = 0.  Every output row is checked on its own."""
+    lib = kq._load()
+    M, N, K = 256, 256, 2048
+    nsb = K // 256
+    wire = _wire("q4_k", N, K, seed=91).reshape(N, nsb, 144).copy()
+
+    def put(rows, sb, d, dmin):
+        wire[rows, sb, 0:2] = np.frombuffer(np.float16(d).tobytes(), dtype=np.uint8)
+        wire[rows, sb, 2:4] = np.frombuffer(np.float16(dmin).tobytes(), dtype=np.uint8)
+
+    put(slice(0, 64), 0, 0.0, 0.01)          # first superblock without a scale
+    put(slice(0, 64), 3, 0.0, 0.02)          # d = 0 in the middle, live minima
+    put(slice(64, 128), 2, 6e-8, 3.0)        # subnormal d, dmin / d = 5e7
+    put(slice(64, 128), 5, 1e-5, 0.0)        # no minima
+    put(slice(128, 192), 1, 8.0, 0.001)      # the unit jumps up by about 2^10 ...
+    put(slice(128, 192), 2, 1e-5, 0.001)     # ... and down by 2^20
+    put(slice(192, 256), 4, 0.0, 0.0)        # an all-zero superblock
+    wire = wire.reshape(N, nsb * 144)
+    xb, xt = make_x((M, K), "bfloat16", seed=92)
+    want = O.bits_to_f32(O.qmm(xb, wire, "q4_k", True, "bfloat16"), "bfloat16").astype(np.float64)
+    try:
+        lib.kq_set_gemm_tile_rows(1024)
+        got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, "q4_k"))
+    finally:
+        lib.kq_set_gemm_tile_rows(0)
+    g = O.bits_to_f32(got, "bfloat16").astype(np.float64)
+    assert np.isfinite(g).all()
+    for c0 in range(0, N, 64):  # per group of weight rows: the corner cases do not hide behind the ordinary columns
+        blk = slice(c0, c0 + 64)
+        assert np.linalg.norm(g[:, blk] - want[:, blk]) / np.linalg.norm(want[:, blk]) <= TOL, c0
+
+
 def test_qmm_prefill_gemm_wide_dynamic_range(kq):
     """bf16 activations spanning many binades and rows of very different scale: the per-row power-of-two
     scaling of the f16 conversion must keep every row within tolerance."""
