@@ -33,6 +33,7 @@ SOURCES = [
     ("kq_codes.hip", ["-DKQ_CODES_PART=1"], "kq_codes_dense"),
     ("kq_codes.hip", ["-DKQ_CODES_PART=2"], "kq_codes_gather"),
     ("kq_codes.hip", ["-DKQ_CODES_PART=3"], "kq_codes_grouped"),
+    ("kq_fp4.hip", []),
     ("kq_router.hip", ["-ffp-contract=off"]),
     # the device encoder must round exactly like the host one: no fused multiply-adds
     ("kq_encode_dev.hip", ["-ffp-contract=off"]),

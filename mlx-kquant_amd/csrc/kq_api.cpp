@@ -323,6 +323,11 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return 0;
   if (kq_moe_grouped_supported((int)P, E, N, K, codec)) return kq_moe_grouped_workspace_bytes(glu ? T : (int)P, (int)P, E, K);
+  if (kq_fp4_moe_supported((int)P, E, N, K, codec)) {  // mxfp4: block-scaled MFMA path, else the code-level kernel
+    const size_t a = kq_fp4_moe_workspace_bytes((int)P, E, glu ? T : (int)P, K);
+    const size_t b = kq_codes_moe_supported((int)P, E, N, K, codec) ? kq_codes_moe_workspace_bytes((int)P, E, glu ? T : (int)P, K) : 0;
+    return a > b ? a : b;
+  }
   if (kq_codes_moe_supported((int)P, E, N, K, codec)) return kq_codes_moe_workspace_bytes((int)P, E, glu ? T : (int)P, K);
   if (kq_anymma_moe_supported((int)P, E, N, K, codec)) return kq_anymma_moe_workspace_bytes((int)P, E);
   return 0;
@@ -418,6 +423,16 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
   // few entries: the per-entry kernels (the caller tries them next) beat the prologue + grouped-kernel pair
   if (per_entry_route(P, entry_rows, bias || bias2, glu, act, codec, E, N, K)) return KQ_ERR_UNSUPPORTED;
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
+    // mxfp4: the wire blocks go into the block-scaled matrix instruction undecoded (kq_fp4.hip)
+    if (kq_fp4_moe_supported((int)P, E, N, K, codec)) {
+      const size_t need = kq_fp4_moe_workspace_bytes((int)P, E, glu ? T : (int)P, K);
+      if (!ws || ws_bytes < need)
+        return kq_set_error(KQ_ERR_WORKSPACE, "%s: workspace of %zu bytes required (got %zu)", op, need, ws ? ws_bytes : 0);
+      const int rcf = kq_launch_fp4_moe(x, static_cast<const uint8_t*>(w), static_cast<const uint8_t*>(w2), idx, bias, bias2,
+                                        out, (int)P, E, N, K, glu ? R : 1, estride, glu, act, limit, alpha, codec, dtype, ws,
+                                        om, s);
+      if (rcf != KQ_ERR_UNSUPPORTED) return rcf;
+    }
     // legacy / IQ / fp4 codecs (biases and every activation included): code-level grouped kernel
     if (kq_codes_moe_supported((int)P, E, N, K, codec)) {
       const size_t need = kq_codes_moe_workspace_bytes((int)P, E, glu ? T : (int)P, K);

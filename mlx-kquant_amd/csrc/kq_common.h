@@ -178,6 +178,14 @@ int kq_launch_codes_moe(const void* x, const uint8_t* w, const uint8_t* w2, cons
                         const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
                         int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, KqOutMap om,
                         hipStream_t s);
+// Batched MoE of mxfp4 stacks on the block-scaled matrix instruction (wire blocks undecoded, activations as e4m3
+// terms); same contract and workspace layout idea as kq_launch_codes_moe.
+bool kq_fp4_moe_supported(int P, int E, int N, int K, int codec);
+size_t kq_fp4_moe_workspace_bytes(int P, int E, int rows, int K);
+int kq_launch_fp4_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
+                      const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
+                      int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, KqOutMap om,
+                      hipStream_t s);
 // Helpers of the slot-mixing ops: idx [T][S-1] -> idx2 [T][S] (last slot = expert 0), and
 // out[t][n] = T(sum_s scores[t][s] * yf[t][s][n]).
 int kq_launch_pad_idx(const uint32_t* idx, uint32_t* idx2, int T, int S, hipStream_t s);

@@ -1,0 +1,382 @@
+// Batched MoE on mxfp4 stacks with gfx950's block-scaled matrix instruction.
+//
+// v_mfma_scale_f32_16x16x128_f8f6f4 multiplies a 16 x 128 tile by a 128 x 16 tile whose elements are 4-, 6- or 8-bit
+// floats and applies one e8m0 (power-of-two) scale per operand row and 32 elements: exactly the mxfp4 wire block, a
+// scale byte and 32 e2m1 codes.  The weights therefore go from memory into the B operand as they are stored, no
+// decode at all: lane (n, kb) of a 16-column tile loads block 4 s + kb of weight row n, its 16 code bytes as the
+// operand and its scale byte as the scale.  (The reference's weight is 2^(e - 128) * (2 * e2m1), the instruction's
+// 2^(e - 127) * e2m1: the same number; scale byte 255, which the instruction reads as NaN, is not a valid e8m0 scale.)
+//
+// Activations: a bf16 value has 8 significant bits, an e4m3 value 4, so x = hi + lo with two e4m3 terms that share
+// a power-of-two scale per 32 values, those of a wire block (f16 inputs: three terms), written once per activation row by a prepass, and an
+// MFMA per term.  Products are exact and summed in f32 by the matrix core.  A value more than 2^13 below the largest
+// of its 32-group loses bits (an absolute error below 2^-16 of that largest value).
+//
+// Operand layout of the instruction (measured): B lane (n, kb) holds k = 32 kb .. 32 kb + 31 of column n, code i in
+// nibble i; A lane (m, a) holds k = 16 a .. 16 a + 15 in bytes 0 .. 15 and k = 64 + 16 a .. + 15 in bytes 16 .. 31 of
+// row m; the scale register (byte picked by op_sel) of lane (row, kb) applies to k = 32 kb .. 32 kb + 31 of that row,
+// for A as for B (for A that is not the lane holding those values); D lane l holds column l % 16, rows 4 (l / 16) .. + 3.  A wire block keeps weight j in the low and weight j + 16 in the high nibble
+// of byte j, so code i of a block is weight i / 2 (+ 16 for odd i): the prepass stores the activations in that order.
+//
+// Kernel: pairs sorted by expert into segments (the sort of kq_moe.hip); a workgroup of four waves takes one m-tile
+// (16 pairs) of a segment and 128 weight rows (fused gate / up: 64 + the same 64 of the up matrix).  The waves split
+// K (steps of 128 dealt round-robin): every wave streams all eight column tiles of its steps straight from global
+// memory into registers (aligned dwords around each 17-byte block, the codes realigned with byte shifts), one step
+// ahead, and the four partial sums meet in LDS.  No LDS staging, no barrier in the stream, about a dozen vector
+// instructions per 32 weights.
+#include "kq_common.h"
+#include "kq_decode.h"
+#include "kq_epilogue.h"
+
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+
+struct Segment {
+  int expert, start, count, pad;
+};
+
+constexpr int F4_J = 8;          // column tiles (of 16) a wave streams per step
+constexpr int F4_THREADS = 256;  // four waves
+
+template <int DT>
+constexpr int f4_terms() { return DT == KQ_BF16 ? 2 : 3; }
+
+struct F4Args {
+  const uint8_t* xa;   // [rows][nsteps][NT][4][32] e4m3 terms in operand order
+  const uint32_t* xs;  // [rows][nsteps][4]: byte t = e8m0 scale of term t
+  const uint8_t* w;
+  const uint8_t* w2;   // up stack (fused gate / up) or null
+  const uint8_t* w_end;   // one past the last byte of the stacks: no load may reach beyond
+  const uint8_t* w2_end;
+  void* y;
+  const float* bias;   // f32 [E][N] or null
+  const float* bias2;
+  const int* order;
+  const Segment* segs;
+  const int* nseg;
+  int N, K, nsteps, x_div, act;
+  int64_t w_expert_stride;
+  float limit, alpha;
+  KqOutMap om;
+};
+
+__device__ __forceinline__ int in_vgpr(int v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+// ------------------------------------------------------------------ activation prepass
+// One workgroup per activation row; a thread writes the 32 operand bytes of one (step, lane block a): positions
+// 8 (a & 1) .. + 7 and 16 + 8 (a & 1) .. + 7 of wire blocks a / 2 and 2 + a / 2 of the step, interleaved.  The scale
+// belongs to the wire block (32 consecutive activations), so the thread looks at both whole blocks.
+template <int DT>
+__global__ __launch_bounds__(128) void fp4_act_prepass_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ xa,
+                                                              uint32_t* __restrict__ xs, int K, int nsteps) {
+  constexpr int NT = f4_terms<DT>();
+  const int row = blockIdx.x;
+  const uint16_t* xr = x + (size_t)row * K;
+  for (int g = threadIdx.x; g < nsteps * 4; g += 128) {
+    const int s = g >> 2, a = g & 3;
+    uint8_t* out = xa + ((size_t)(row * nsteps + s) * NT) * 128 + a * 32;
+    u32x4 p[NT][2];
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+      const int bw = 2 * half + (a >> 1), base = 128 * s + 32 * bw;
+      u32x4 c[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+      if (base < K) {  // K is a multiple of 32: a wire block is inside or outside as a whole
+#pragma unroll
+        for (int i = 0; i < 4; i++) c[i] = *reinterpret_cast<const u32x4*>(xr + base + 8 * i);
+      }
+      auto val = [&](const u32x4& cc, int u) -> float {
+        const uint32_t h = (cc[u >> 1] >> (16 * (u & 1))) & 0xffff;
+        return DT == KQ_F16 ? kq::h2f((uint16_t)h) : __builtin_bit_cast(float, h << 16);
+      };
+      float amax = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int u = 0; u < 8; u++) amax = fmaxf(amax, fabsf(val(c[i], u)));
+      // the block's largest magnitude lands in [128, 256): below e4m3's 448
+      int eb = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff);
+      if (eb == 0xff) eb = 0xfe;  // inf / nan inputs stay inf / nan through the products
+      int sb = eb - 7;            // e8m0 byte of the first term: 2^(eb - 127 - 7)
+      sb = sb < 1 ? 1 : sb;
+      const float mul = __builtin_bit_cast(float, (uint32_t)(254 - sb) << 23);  // 2^(127 - sb), exact
+      // this lane block's sixteen values of the block: 8 (a & 1) + u and 16 + 8 (a & 1) + u, interleaved
+      float v[16];
+      const u32x4 c0 = (a & 1) ? c[1] : c[0], c1 = (a & 1) ? c[3] : c[2];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        v[2 * u] = val(c0, u) * mul;
+        v[2 * u + 1] = val(c1, u) * mul;
+      }
+      uint32_t sword = 0;
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        int tb = sb - 4 * t;  // every further term sits four bits lower
+        const bool live = tb >= 1;
+        tb = live ? tb : 1;
+        sword |= (uint32_t)tb << (8 * t);
+#pragma unroll
+        for (int q = 0; q < 16; q += 4) {
+          int pk = 0;
+          pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[q], v[q + 1], pk, false);
+          pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[q + 2], v[q + 3], pk, true);
+          if (!live) pk = 0;
+          // what is left, in units of the next term (exact: the remainder of a 4-bit rounding, times 16)
+          v[q] = (v[q] - __builtin_amdgcn_cvt_f32_fp8(pk, 0)) * 16.0f;
+          v[q + 1] = (v[q + 1] - __builtin_amdgcn_cvt_f32_fp8(pk, 1)) * 16.0f;
+          v[q + 2] = (v[q + 2] - __builtin_amdgcn_cvt_f32_fp8(pk, 2)) * 16.0f;
+          v[q + 3] = (v[q + 3] - __builtin_amdgcn_cvt_f32_fp8(pk, 3)) * 16.0f;
+          p[t][half][q >> 2] = (uint32_t)pk;
+        }
+      }
+      if ((a & 1) == 0) xs[(size_t)(row * nsteps + s) * 4 + bw] = sword;
+    }
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      *reinterpret_cast<u32x4*>(out + t * 128) = p[t][0];
+      *reinterpret_cast<u32x4*>(out + t * 128 + 16) = p[t][1];
+    }
+  }
+}
+
+// ------------------------------------------------------------------ grouped kernel
+template <int DT, bool GLU>
+__global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
+  constexpr int NT = f4_terms<DT>(), J = F4_J;
+  constexpr int COLS = GLU ? 64 : 128;  // output columns of a workgroup
+  __shared__ v4f red[4][J][64];
+  const int nseg = *a.nseg;
+  if ((int)blockIdx.y >= nseg) return;
+  const Segment sg = a.segs[blockIdx.y];
+  const int mt = blockIdx.z;  // m-tile of the segment (16 pairs)
+  if (16 * mt >= sg.count) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, kb = lane >> 4;
+  const int N = a.N, nsteps = a.nsteps, nblk = a.K >> 5;
+  const uint32_t row_bytes = (uint32_t)nblk * 17u;
+  const int n0 = blockIdx.x * COLS;
+  const int rows_here = sg.count - 16 * mt < 16 ? sg.count - 16 * mt : 16;
+
+  // weight rows of this lane: tile j covers columns n0 + 16 j .. (fused: tiles 4 .. 7 are the same columns of the up
+  // matrix); columns past N re-read the last one
+  const uint8_t* wrow[J];
+#pragma unroll
+  for (int j = 0; j < J; j++) {
+    int c = n0 + 16 * (GLU ? (j & 3) : j) + r;
+    c = c < N ? c : N - 1;
+    const uint8_t* base = (GLU && j >= 4) ? a.w2 : a.w;
+    wrow[j] = base + (int64_t)sg.expert * a.w_expert_stride + (size_t)c * row_bytes;
+  }
+  // activation row of this lane (rows past the segment re-read its last pair; their results are dropped)
+  const int mrow = r < rows_here ? r : rows_here - 1;
+  const int pair = a.order[sg.start + 16 * mt + mrow];
+  const int xrow = pair / a.x_div;
+  const uint8_t* arow = a.xa + ((size_t)xrow * nsteps * NT) * 128 + kb * 32;
+  const uint32_t* srow = a.xs + (size_t)xrow * nsteps * 4 + kb;
+
+  struct Stage {
+    u32x4 b[J];
+    int sb[J];
+    v8i av[NT];
+    int sa;
+  };
+  auto fetch = [&](Stage& st, int s) {
+    int blk = 4 * s + kb;
+    const bool live = blk < nblk;  // past K: any block of the row with a neutral scale (the activations are zeros)
+    blk = live ? blk : nblk - 1;
+    const uint32_t off = (uint32_t)blk * 17u;
+#pragma unroll
+    for (int j = 0; j < J; j++) {
+      // the 17 bytes of the block (scale, 16 code bytes) sit at any byte offset: five aligned dwords around them,
+      // the codes brought to dword boundaries with byte shifts (a global load wider than a byte wants dword alignment)
+      const uintptr_t ad = reinterpret_cast<uintptr_t>(wrow[j] + off);
+      const uint32_t sh = (uint32_t)ad & 3u;
+      const uint32_t* q = reinterpret_cast<const uint32_t*>(ad - sh);
+      const u32x4 d = *reinterpret_cast<const u32x4_a4*>(q);
+      uint32_t d4;
+      if (reinterpret_cast<const uint8_t*>(q + 5) <= ((GLU && j >= 4) ? a.w2_end : a.w_end)) {
+        d4 = q[4];
+      } else {  // the last block of the stack: the dword would reach past its end
+        d4 = 0;
+        const uint8_t* e = (GLU && j >= 4) ? a.w2_end : a.w_end;
+        for (const uint8_t* b = reinterpret_cast<const uint8_t*>(q + 4); b < e; b++)
+          d4 |= (uint32_t)*b << (8 * (int)(b - reinterpret_cast<const uint8_t*>(q + 4)));
+      }
+      const int sc = (int)((d[0] >> (8 * sh)) & 0xff);
+      st.sb[j] = live ? sc : 127;
+      // codes start at byte sh + 1 of the window: a shift by 1 .. 3 bytes, or (sh = 3) the next dword as it is
+      const bool whole = sh == 3;
+      const uint32_t s1 = (sh + 1) & 3u;
+      const uint32_t dd[5] = {d[0], d[1], d[2], d[3], d4};
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        st.b[j][i] = __builtin_amdgcn_alignbyte(dd[i + 1], whole ? dd[i + 1] : dd[i], s1);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(arow + ((size_t)s * NT + t) * 128);
+      const u32x4 hi = *reinterpret_cast<const u32x4*>(arow + ((size_t)s * NT + t) * 128 + 16);
+      st.av[t] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    }
+    st.sa = (int)srow[(size_t)s * 4];
+  };
+  v4f acc[J];
+#pragma unroll
+  for (int j = 0; j < J; j++) acc[j] = v4f{0, 0, 0, 0};
+  auto multiply = [&](const Stage& st) {
+    const int sa = in_vgpr(st.sa);
+#pragma unroll
+    for (int j = 0; j < J; j++) {
+      const v8i bv = {(int)st.b[j][0], (int)st.b[j][1], (int)st.b[j][2], (int)st.b[j][3], 0, 0, 0, 0};
+      const int sb = in_vgpr(st.sb[j]);
+      acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[0], bv, acc[j], 0, 4, 0, sa, 0, sb);
+      acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[1], bv, acc[j], 0, 4, 1, sa, 0, sb);
+      if constexpr (NT == 3)
+        acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[2], bv, acc[j], 0, 4, 2, sa, 0, sb);
+    }
+  };
+
+  // this wave's steps: wave, wave + 4, ...; two stages in rotation, the next step's loads in flight during a multiply
+  Stage st0, st1;
+  int s = wave;
+  if (s < nsteps) fetch(st0, s);
+  while (s < nsteps) {
+    if (s + 4 < nsteps) fetch(st1, s + 4);
+    multiply(st0);
+    s += 4;
+    if (s >= nsteps) break;
+    if (s + 4 < nsteps) fetch(st0, s + 4);
+    multiply(st1);
+    s += 4;
+  }
+
+  // ---- the four partial sums meet in LDS; wave w finishes tiles 2 w, 2 w + 1 (fused: gate tile w with up tile w)
+#pragma unroll
+  for (int j = 0; j < J; j++) red[wave][j][lane] = acc[j];
+  __syncthreads();
+  const int expert = sg.expert;
+  auto total = [&](int j) {
+    v4f v = red[0][j][lane];
+#pragma unroll
+    for (int wv = 1; wv < 4; wv++) {
+      const v4f o = red[wv][j][lane];
+      v[0] += o[0];
+      v[1] += o[1];
+      v[2] += o[2];
+      v[3] += o[3];
+    }
+    return v;
+  };
+  auto finish = [&](int col, const v4f& g, const v4f& u) {
+    if (col >= N) return;
+    const float gb = a.bias ? a.bias[(size_t)expert * N + col] : 0.f;
+    const float ub = (GLU && a.bias2) ? a.bias2[(size_t)expert * N + col] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int m = 4 * kb + i;
+      if (m < rows_here) {
+        const int p = a.order[sg.start + 16 * mt + m];
+        float v = g[i] + gb;
+        if constexpr (GLU) v = kq::glu_epilogue_fast(a.act, v, u[i] + ub, a.limit, a.alpha);
+        kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, p) * N + col, v);
+      }
+    }
+  };
+  if constexpr (GLU) {
+    finish(n0 + 16 * wave + r, total(wave), total(wave + 4));
+  } else {
+    const v4f none = {0, 0, 0, 0};
+    finish(n0 + 16 * (2 * wave) + r, total(2 * wave), none);
+    finish(n0 + 16 * (2 * wave + 1) + r, total(2 * wave + 1), none);
+  }
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+int f4_steps(int K) { return ((K >> 5) + 3) / 4; }
+
+}  // namespace
+
+int kq_launch_moe_sort(const uint32_t* idx, int P, int E, void* order, void* segs, void* nseg, hipStream_t s);
+
+// mxfp4 stacks, more than 16 pairs: K a multiple of 32 (the block), N a multiple of 8 (the op's own rule)
+bool kq_fp4_moe_supported(int P, int E, int N, int K, int codec) {
+  return codec == KQ_MXFP4 && P > 16 && E > 0 && E <= 4096 && (int64_t)E + P / 32 < 65535 && N > 0 && K >= 32 &&
+         (K & 31) == 0 && (int64_t)N * (K >> 5) * 17 < ((int64_t)1 << 32);
+}
+
+// Workspace: sorted pair list, segment table, segment count, then the prepass outputs for `rows` activation rows
+// (three e4m3 terms at most: 384 bytes and four scale words per row and step of 128).
+size_t kq_fp4_moe_workspace_bytes(int P, int E, int rows, int K) {
+  const size_t rs = (size_t)rows * f4_steps(K);
+  return align256((size_t)P * 4) + align256(((size_t)E + P / 32 + 1) * sizeof(Segment)) + 256 + align256(rs * 384) +
+         align256(rs * 16);
+}
+
+// x: [rows][K] (rows = P / x_div); pair p reads row p / x_div and expert idx[p]; out rows through om.
+int kq_launch_fp4_moe(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* idx, const float* bias,
+                      const float* bias2, void* out, int P, int E, int N, int K, int x_div, int64_t w_expert_stride,
+                      int glu, int act, float limit, float alpha, int codec, int dtype, void* ws, KqOutMap om,
+                      hipStream_t s) {
+  if (!kq_fp4_moe_supported(P, E, N, K, codec) || (reinterpret_cast<uintptr_t>(x) & 15) ||
+      (reinterpret_cast<uintptr_t>(ws) & 255))
+    return KQ_ERR_UNSUPPORTED;
+  uint8_t* p = static_cast<uint8_t*>(ws);
+  int* order = reinterpret_cast<int*>(p);
+  Segment* segs = reinterpret_cast<Segment*>(p + align256((size_t)P * 4));
+  int* nseg = reinterpret_cast<int*>(p + align256((size_t)P * 4) + align256(((size_t)E + P / 32 + 1) * sizeof(Segment)));
+  int rc = kq_launch_moe_sort(idx, P, E, order, segs, nseg, s);
+  if (rc) return rc;
+  x_div = x_div < 1 ? 1 : x_div;
+  const int rows = glu ? P / x_div : P, nsteps = f4_steps(K);
+  const size_t rs = (size_t)rows * nsteps;
+  uint8_t* xa = reinterpret_cast<uint8_t*>(nseg) + 256;
+  uint32_t* xs = reinterpret_cast<uint32_t*>(xa + align256(rs * 384));
+  const uint16_t* xi = static_cast<const uint16_t*>(x);
+  if (dtype == KQ_F16)
+    hipLaunchKernelGGL((fp4_act_prepass_kernel<KQ_F16>), dim3(rows), dim3(128), 0, s, xi, xa, xs, K, nsteps);
+  else
+    hipLaunchKernelGGL((fp4_act_prepass_kernel<KQ_BF16>), dim3(rows), dim3(128), 0, s, xi, xa, xs, K, nsteps);
+  KQ_HIP_CHECK(hipGetLastError());
+  F4Args a{};
+  a.xa = xa;
+  a.xs = xs;
+  a.w = w;
+  a.w2 = w2;
+  a.w_end = w + (int64_t)(E - 1) * w_expert_stride + (size_t)N * (K >> 5) * 17;
+  a.w2_end = w2 ? w2 + (int64_t)(E - 1) * w_expert_stride + (size_t)N * (K >> 5) * 17 : nullptr;
+  a.y = out;
+  a.bias = bias;
+  a.bias2 = bias2;
+  a.order = order;
+  a.segs = segs;
+  a.nseg = nseg;
+  a.N = N;
+  a.K = K;
+  a.nsteps = nsteps;
+  a.x_div = x_div;
+  a.act = act;
+  a.w_expert_stride = w_expert_stride;
+  a.limit = limit;
+  a.alpha = alpha;
+  a.om = om;
+  int maxseg = E + P / 32;  // sum over experts of ceil(c_e / 32) <= E + P / 32
+  if (maxseg > P) maxseg = P;
+  const int cols = glu ? 64 : 128;
+  const dim3 grid((N + cols - 1) / cols, maxseg, 2);  // z: the two m-tiles of a segment of up to 32 pairs
+  if (glu) {
+    if (dtype == KQ_F16) hipLaunchKernelGGL((fp4_grouped_kernel<KQ_F16, true>), grid, dim3(F4_THREADS), 0, s, a);
+    else hipLaunchKernelGGL((fp4_grouped_kernel<KQ_BF16, true>), grid, dim3(F4_THREADS), 0, s, a);
+  } else {
+    if (dtype == KQ_F16) hipLaunchKernelGGL((fp4_grouped_kernel<KQ_F16, false>), grid, dim3(F4_THREADS), 0, s, a);
+    else hipLaunchKernelGGL((fp4_grouped_kernel<KQ_BF16, false>), grid, dim3(F4_THREADS), 0, s, a);
+  }
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}

@@ -271,9 +271,6 @@ struct StArgs {
   const float* bias2;  // the same for the up sums of the fused form
   int64_t w_expert_stride;
   KqOutMap om;
-#ifdef KQ_ST_TS
-  uint64_t* ts;
-#endif
 };
 
 // ------------------------------------------------------------------ q4_k / q5_k unit
@@ -918,13 +915,6 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   constexpr int AS = ST_XU * NAP;  // A register pairs per row group
   constexpr int XL = XU / 2;  // 16-byte activation loads per lane and row: XU units x 256 values
 
-#ifdef KQ_ST_TS
-  uint64_t ts[8];
-  ts[0] = __builtin_amdgcn_s_memrealtime();
-#define ST_TS(i) ts[i] = __builtin_amdgcn_s_memrealtime()
-#else
-#define ST_TS(i)
-#endif
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1054,7 +1044,6 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   issue_next();
   // wait for the activations alone: the first unit stays in flight
   if (inflight) vmwait<U::UPI>(); else vmwait<0>();
-  ST_TS(1);
   SFor<MB * XL>::run([&](auto t) { tie_v(xreg[decltype(t)::value]); });
   tie_v(greg);
   if constexpr (IQ2_COP > 1) SFor<8>::run([&](auto ii) { tie_v2(gq[decltype(ii)::value]); });
@@ -1278,7 +1267,6 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
 
   // The other D - 1 units are queued only now: a wave that queues loads faster than the memory system takes them
   // stalls in the issue, and the activation work above would have waited behind that stall.
-  ST_TS(2);
   SFor<D - 1>::run([&](auto) { issue_next(); });
   float acc_a[R], acc_b[GM == 2 ? R : 1];
   int ct = tile0, cslot = 0;  // tile / slot being consumed
@@ -1299,7 +1287,6 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         else if (younger == 2) vmwait<2 * U::UPI>();
         else if (younger == 1) vmwait<1 * U::UPI>();
         else vmwait<0>();
-        ST_TS(3 + u);
         const uint8_t* slot = wb + cslot * U::SLOT;
         const uint8_t* bl = slot + crow * G::LBPB;
         constexpr int us = u / UPS;  // the wave's superblock this unit belongs to
@@ -1332,12 +1319,6 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
       }
     });
 
-#ifdef KQ_ST_TS
-    lgkm_drain();
-    ST_TS(7);
-    if (lane == 0)
-      for (int i = 0; i < 8; i++) a.ts[((size_t)blockIdx.x * ST_WAVES + wave) * 8 + i] = ts[i];
-#endif
     // ---- cross-wave + cross-half reduction of the tile
     float* red = red_all + (parity * ST_WAVES + wave) * (UPS * R * 64);
 #pragma unroll
