@@ -24,9 +24,12 @@
 // memory into registers (aligned dwords around each 17-byte block, the codes realigned with byte shifts), one step
 // ahead, and the four partial sums meet in LDS.  No LDS staging, no barrier in the stream, about a dozen vector
 // instructions per 32 weights.
+#include <type_traits>
+
 #include "kq_common.h"
 #include "kq_decode.h"
 #include "kq_epilogue.h"
+#include "kq_moe_sort.h"
 
 namespace {
 
@@ -35,11 +38,9 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 
-struct Segment {
-  int expert, start, count, pad;
-};
+using kqsort::Segment;
 
-constexpr int F4_J = 8;          // column tiles (of 16) a wave streams per step
+constexpr int F4_STAGES = 2;     // register stages in rotation: a step's loads are queued one step ahead (deeper: no gain)
 constexpr int F4_THREADS = 256;  // four waves
 
 template <int DT>
@@ -64,22 +65,40 @@ struct F4Args {
   KqOutMap om;
 };
 
+}  // namespace
+namespace kq {
+template <int N>
+struct SForF4 {
+  template <class F>
+  __device__ __forceinline__ static void run(F&& f) {
+    SForF4<N - 1>::run(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+};
+template <>
+struct SForF4<0> {
+  template <class F>
+  __device__ __forceinline__ static void run(F&&) {}
+};
+}  // namespace kq
+namespace {
+
 __device__ __forceinline__ int in_vgpr(int v) {
   asm volatile("" : "+v"(v));
   return v;
 }
 
 // ------------------------------------------------------------------ activation prepass
-// One workgroup per activation row; a thread writes the 32 operand bytes of one (step, lane block a): positions
+// One workgroup per activation row (fp4_prologue_kernel); a thread writes the 32 operand bytes of one (step, lane block a): positions
 // 8 (a & 1) .. + 7 and 16 + 8 (a & 1) .. + 7 of wire blocks a / 2 and 2 + a / 2 of the step, interleaved.  The scale
 // belongs to the wire block (32 consecutive activations), so the thread looks at both whole blocks.
+constexpr int F4_PRO_THREADS = 256;
 template <int DT>
-__global__ __launch_bounds__(128) void fp4_act_prepass_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ xa,
-                                                              uint32_t* __restrict__ xs, int K, int nsteps) {
+__device__ __forceinline__ void fp4_prepass_row(const uint16_t* __restrict__ x, uint8_t* __restrict__ xa,
+                                                uint32_t* __restrict__ xs, int K, int nsteps, int row) {
   constexpr int NT = f4_terms<DT>();
-  const int row = blockIdx.x;
   const uint16_t* xr = x + (size_t)row * K;
-  for (int g = threadIdx.x; g < nsteps * 4; g += 128) {
+  for (int g = threadIdx.x; g < nsteps * 4; g += F4_PRO_THREADS) {
     const int s = g >> 2, a = g & 3;
     uint8_t* out = xa + ((size_t)(row * nsteps + s) * NT) * 128 + a * 32;
     u32x4 p[NT][2];
@@ -145,16 +164,36 @@ __global__ __launch_bounds__(128) void fp4_act_prepass_kernel(const uint16_t* __
   }
 }
 
+// The pair sort and the activation prepass in ONE launch: workgroup 0 sorts the pairs by expert, workgroups 1 .. rows
+// convert one activation row each (neither depends on the other).
+template <int DT>
+__global__ __launch_bounds__(F4_PRO_THREADS) void fp4_prologue_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ xa,
+                                                                      uint32_t* __restrict__ xs, int K, int nsteps,
+                                                                      const uint32_t* __restrict__ idx, int P, int E,
+                                                                      int* __restrict__ order, Segment* __restrict__ segs,
+                                                                      int* __restrict__ nseg_out) {
+  __shared__ int cnt[kqsort::SORT_MAX_E];
+  __shared__ int scan_p[F4_PRO_THREADS], scan_s[F4_PRO_THREADS];
+  if (blockIdx.x == 0)  // the longest workgroup of the launch (a chain of barriers) goes first
+    kqsort::moe_sort_body<F4_PRO_THREADS>(idx, P, E, order, segs, nseg_out, cnt, scan_p, scan_s);
+  else
+    fp4_prepass_row<DT>(x, xa, xs, K, nsteps, blockIdx.x - 1);
+}
+
 // ------------------------------------------------------------------ grouped kernel
-template <int DT, bool GLU>
+// J = column tiles (of 16) a wave streams per step (8 or 4); MT = m-tiles (of 16 pairs) a workgroup multiplies with
+// the same weight registers: 1 (grid z walks the m-tiles of a segment, the weights of a longer segment are read
+// twice) or 2 (segments of up to 32 pairs in one pass, J = 4).
+template <int DT, bool GLU, int J, int MT>
 __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
-  constexpr int NT = f4_terms<DT>(), J = F4_J;
-  constexpr int COLS = GLU ? 64 : 128;  // output columns of a workgroup
-  __shared__ v4f red[4][J][64];
+  constexpr int NT = f4_terms<DT>();
+  constexpr int JH = J / 2;                    // fused: gate tiles 0 .. JH - 1, up tiles JH .. J - 1
+  constexpr int COLS = GLU ? 8 * J : 16 * J;  // output columns of a workgroup
+  __shared__ v4f red[4][MT * J][64];
   const int nseg = *a.nseg;
   if ((int)blockIdx.y >= nseg) return;
   const Segment sg = a.segs[blockIdx.y];
-  const int mt = blockIdx.z;  // m-tile of the segment (16 pairs)
+  const int mt = MT == 1 ? blockIdx.z : 0;  // first m-tile (16 pairs) of this workgroup
   if (16 * mt >= sg.count) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -162,30 +201,34 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
   const int N = a.N, nsteps = a.nsteps, nblk = a.K >> 5;
   const uint32_t row_bytes = (uint32_t)nblk * 17u;
   const int n0 = blockIdx.x * COLS;
-  const int rows_here = sg.count - 16 * mt < 16 ? sg.count - 16 * mt : 16;
+  const int rows_here = sg.count - 16 * mt < 16 * MT ? sg.count - 16 * mt : 16 * MT;
 
   // weight rows of this lane: tile j covers columns n0 + 16 j .. (fused: tiles 4 .. 7 are the same columns of the up
   // matrix); columns past N re-read the last one
   const uint8_t* wrow[J];
 #pragma unroll
   for (int j = 0; j < J; j++) {
-    int c = n0 + 16 * (GLU ? (j & 3) : j) + r;
+    int c = n0 + 16 * (GLU ? (j % JH) : j) + r;
     c = c < N ? c : N - 1;
-    const uint8_t* base = (GLU && j >= 4) ? a.w2 : a.w;
+    const uint8_t* base = (GLU && j >= JH) ? a.w2 : a.w;
     wrow[j] = base + (int64_t)sg.expert * a.w_expert_stride + (size_t)c * row_bytes;
   }
-  // activation row of this lane (rows past the segment re-read its last pair; their results are dropped)
-  const int mrow = r < rows_here ? r : rows_here - 1;
-  const int pair = a.order[sg.start + 16 * mt + mrow];
-  const int xrow = pair / a.x_div;
-  const uint8_t* arow = a.xa + ((size_t)xrow * nsteps * NT) * 128 + kb * 32;
-  const uint32_t* srow = a.xs + (size_t)xrow * nsteps * 4 + kb;
+  // activation rows of this lane (rows past the segment re-read its last pair; their results are dropped)
+  const uint8_t* arow[MT];
+  const uint32_t* srow[MT];
+#pragma unroll
+  for (int m = 0; m < MT; m++) {
+    const int mrow = 16 * m + r < rows_here ? 16 * m + r : rows_here - 1;
+    const int xrow = a.order[sg.start + 16 * mt + mrow] / a.x_div;
+    arow[m] = a.xa + ((size_t)xrow * nsteps * NT) * 128 + kb * 32;
+    srow[m] = a.xs + (size_t)xrow * nsteps * 4 + kb;
+  }
 
   struct Stage {
     u32x4 b[J];
     int sb[J];
-    v8i av[NT];
-    int sa;
+    v8i av[MT][NT];
+    int sa[MT];
   };
   auto fetch = [&](Stage& st, int s) {
     int blk = 4 * s + kb;
@@ -201,11 +244,11 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
       const uint32_t* q = reinterpret_cast<const uint32_t*>(ad - sh);
       const u32x4 d = *reinterpret_cast<const u32x4_a4*>(q);
       uint32_t d4;
-      if (reinterpret_cast<const uint8_t*>(q + 5) <= ((GLU && j >= 4) ? a.w2_end : a.w_end)) {
+      if (reinterpret_cast<const uint8_t*>(q + 5) <= ((GLU && j >= JH) ? a.w2_end : a.w_end)) {
         d4 = q[4];
       } else {  // the last block of the stack: the dword would reach past its end
         d4 = 0;
-        const uint8_t* e = (GLU && j >= 4) ? a.w2_end : a.w_end;
+        const uint8_t* e = (GLU && j >= JH) ? a.w2_end : a.w_end;
         for (const uint8_t* b = reinterpret_cast<const uint8_t*>(q + 4); b < e; b++)
           d4 |= (uint32_t)*b << (8 * (int)(b - reinterpret_cast<const uint8_t*>(q + 4)));
       }
@@ -220,46 +263,62 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
         st.b[j][i] = __builtin_amdgcn_alignbyte(dd[i + 1], whole ? dd[i + 1] : dd[i], s1);
     }
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-      const u32x4 lo = *reinterpret_cast<const u32x4*>(arow + ((size_t)s * NT + t) * 128);
-      const u32x4 hi = *reinterpret_cast<const u32x4*>(arow + ((size_t)s * NT + t) * 128 + 16);
-      st.av[t] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-    }
-    st.sa = (int)srow[(size_t)s * 4];
-  };
-  v4f acc[J];
+    for (int m = 0; m < MT; m++) {
 #pragma unroll
-  for (int j = 0; j < J; j++) acc[j] = v4f{0, 0, 0, 0};
+      for (int t = 0; t < NT; t++) {
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(arow[m] + ((size_t)s * NT + t) * 128);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(arow[m] + ((size_t)s * NT + t) * 128 + 16);
+        st.av[m][t] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      }
+      st.sa[m] = (int)srow[m][(size_t)s * 4];
+    }
+  };
+  v4f acc[MT][J];
+#pragma unroll
+  for (int m = 0; m < MT; m++)
+#pragma unroll
+    for (int j = 0; j < J; j++) acc[m][j] = v4f{0, 0, 0, 0};
   auto multiply = [&](const Stage& st) {
-    const int sa = in_vgpr(st.sa);
 #pragma unroll
     for (int j = 0; j < J; j++) {
       const v8i bv = {(int)st.b[j][0], (int)st.b[j][1], (int)st.b[j][2], (int)st.b[j][3], 0, 0, 0, 0};
       const int sb = in_vgpr(st.sb[j]);
-      acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[0], bv, acc[j], 0, 4, 0, sa, 0, sb);
-      acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[1], bv, acc[j], 0, 4, 1, sa, 0, sb);
-      if constexpr (NT == 3)
-        acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[2], bv, acc[j], 0, 4, 2, sa, 0, sb);
+#pragma unroll
+      for (int m = 0; m < MT; m++) {
+        const int sa = in_vgpr(st.sa[m]);
+        acc[m][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[m][0], bv, acc[m][j], 0, 4, 0, sa, 0, sb);
+        acc[m][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[m][1], bv, acc[m][j], 0, 4, 1, sa, 0, sb);
+        if constexpr (NT == 3)
+          acc[m][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[m][2], bv, acc[m][j], 0, 4, 2, sa, 0, sb);
+      }
     }
   };
 
-  // this wave's steps: wave, wave + 4, ...; two stages in rotation, the next step's loads in flight during a multiply
-  Stage st0, st1;
+  // this wave's steps: wave, wave + 4, ...; F4_STAGES register stages in rotation, the loads of the next
+  // F4_STAGES - 1 steps in flight during a multiply
+  constexpr int S = F4_STAGES;
+  Stage st[S];
   int s = wave;
-  if (s < nsteps) fetch(st0, s);
+  kq::SForF4<S - 1>::run([&](auto ic) {
+    constexpr int i = decltype(ic)::value;
+    if (s + 4 * i < nsteps) fetch(st[i], s + 4 * i);
+  });
   while (s < nsteps) {
-    if (s + 4 < nsteps) fetch(st1, s + 4);
-    multiply(st0);
-    s += 4;
-    if (s >= nsteps) break;
-    if (s + 4 < nsteps) fetch(st0, s + 4);
-    multiply(st1);
-    s += 4;
+    kq::SForF4<S>::run([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      if (s < nsteps) {
+        if (s + 4 * (S - 1) < nsteps) fetch(st[(i + S - 1) % S], s + 4 * (S - 1));
+        multiply(st[i]);
+        s += 4;
+      }
+    });
   }
 
-  // ---- the four partial sums meet in LDS; wave w finishes tiles 2 w, 2 w + 1 (fused: gate tile w with up tile w)
+  // ---- the four partial sums meet in LDS; wave w finishes J / 4 tiles (fused: gate tile w with up tile w)
 #pragma unroll
-  for (int j = 0; j < J; j++) red[wave][j][lane] = acc[j];
+  for (int m = 0; m < MT; m++)
+#pragma unroll
+    for (int j = 0; j < J; j++) red[wave][m * J + j][lane] = acc[m][j];
   __syncthreads();
   const int expert = sg.expert;
   auto total = [&](int j) {
@@ -274,13 +333,13 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
     }
     return v;
   };
-  auto finish = [&](int col, const v4f& g, const v4f& u) {
+  auto finish = [&](int m16, int col, const v4f& g, const v4f& u) {
     if (col >= N) return;
     const float gb = a.bias ? a.bias[(size_t)expert * N + col] : 0.f;
     const float ub = (GLU && a.bias2) ? a.bias2[(size_t)expert * N + col] : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      const int m = 4 * kb + i;
+      const int m = 16 * m16 + 4 * kb + i;
       if (m < rows_here) {
         const int p = a.order[sg.start + 16 * mt + m];
         float v = g[i] + gb;
@@ -289,12 +348,15 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
       }
     }
   };
-  if constexpr (GLU) {
-    finish(n0 + 16 * wave + r, total(wave), total(wave + 4));
-  } else {
-    const v4f none = {0, 0, 0, 0};
-    finish(n0 + 16 * (2 * wave) + r, total(2 * wave), none);
-    finish(n0 + 16 * (2 * wave + 1) + r, total(2 * wave + 1), none);
+#pragma unroll
+  for (int m = 0; m < MT; m++) {
+    if constexpr (GLU) {
+      if (wave < JH) finish(m, n0 + 16 * wave + r, total(m * J + wave), total(m * J + wave + JH));
+    } else {
+      const v4f none = {0, 0, 0, 0};
+#pragma unroll
+      for (int t = 0; t < J / 4; t++) finish(m, n0 + 16 * (J / 4 * wave + t) + r, total(m * J + J / 4 * wave + t), none);
+    }
   }
 }
 
@@ -302,8 +364,6 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 int f4_steps(int K) { return ((K >> 5) + 3) / 4; }
 
 }  // namespace
-
-int kq_launch_moe_sort(const uint32_t* idx, int P, int E, void* order, void* segs, void* nseg, hipStream_t s);
 
 // mxfp4 stacks, more than 16 pairs: K a multiple of 32 (the block), N a multiple of 8 (the op's own rule)
 bool kq_fp4_moe_supported(int P, int E, int N, int K, int codec) {
@@ -331,8 +391,6 @@ int kq_launch_fp4_moe(const void* x, const uint8_t* w, const uint8_t* w2, const 
   int* order = reinterpret_cast<int*>(p);
   Segment* segs = reinterpret_cast<Segment*>(p + align256((size_t)P * 4));
   int* nseg = reinterpret_cast<int*>(p + align256((size_t)P * 4) + align256(((size_t)E + P / 32 + 1) * sizeof(Segment)));
-  int rc = kq_launch_moe_sort(idx, P, E, order, segs, nseg, s);
-  if (rc) return rc;
   x_div = x_div < 1 ? 1 : x_div;
   const int rows = glu ? P / x_div : P, nsteps = f4_steps(K);
   const size_t rs = (size_t)rows * nsteps;
@@ -340,9 +398,11 @@ int kq_launch_fp4_moe(const void* x, const uint8_t* w, const uint8_t* w2, const 
   uint32_t* xs = reinterpret_cast<uint32_t*>(xa + align256(rs * 384));
   const uint16_t* xi = static_cast<const uint16_t*>(x);
   if (dtype == KQ_F16)
-    hipLaunchKernelGGL((fp4_act_prepass_kernel<KQ_F16>), dim3(rows), dim3(128), 0, s, xi, xa, xs, K, nsteps);
+    hipLaunchKernelGGL((fp4_prologue_kernel<KQ_F16>), dim3(rows + 1), dim3(F4_PRO_THREADS), 0, s, xi, xa, xs, K, nsteps, idx, P,
+                       E, order, segs, nseg);
   else
-    hipLaunchKernelGGL((fp4_act_prepass_kernel<KQ_BF16>), dim3(rows), dim3(128), 0, s, xi, xa, xs, K, nsteps);
+    hipLaunchKernelGGL((fp4_prologue_kernel<KQ_BF16>), dim3(rows + 1), dim3(F4_PRO_THREADS), 0, s, xi, xa, xs, K, nsteps, idx,
+                       P, E, order, segs, nseg);
   KQ_HIP_CHECK(hipGetLastError());
   F4Args a{};
   a.xa = xa;
@@ -368,15 +428,22 @@ int kq_launch_fp4_moe(const void* x, const uint8_t* w, const uint8_t* w2, const 
   a.om = om;
   int maxseg = E + P / 32;  // sum over experts of ceil(c_e / 32) <= E + P / 32
   if (maxseg > P) maxseg = P;
-  const int cols = glu ? 64 : 128;
-  const dim3 grid((N + cols - 1) / cols, maxseg, 2);  // z: the two m-tiles of a segment of up to 32 pairs
+  // Shapes: the fused op streams 8 column tiles per wave and step (64 output columns per workgroup), the plain op 4
+  // (64 columns: twice the workgroups of the 8-tile form, 50.7 -> 43.5 us on 32 experts of 2880 x 2880 at 256 pairs);
+  // stacks whose experts see more than 12 pairs on average take both m-tiles of a segment in one pass.
+  const bool two = (int64_t)P > 12 * (int64_t)E;
+#define KQ_F4_LAUNCH(DTV, GLUV, JV, MTV)                                                                         \
+  hipLaunchKernelGGL((fp4_grouped_kernel<DTV, GLUV, JV, MTV>),                                                   \
+                     dim3((N + (GLUV ? 8 * JV : 16 * JV) - 1) / (GLUV ? 8 * JV : 16 * JV), maxseg, MTV == 1 ? 2 : 1), \
+                     dim3(F4_THREADS), 0, s, a)
   if (glu) {
-    if (dtype == KQ_F16) hipLaunchKernelGGL((fp4_grouped_kernel<KQ_F16, true>), grid, dim3(F4_THREADS), 0, s, a);
-    else hipLaunchKernelGGL((fp4_grouped_kernel<KQ_BF16, true>), grid, dim3(F4_THREADS), 0, s, a);
+    if (dtype == KQ_F16) { if (two) KQ_F4_LAUNCH(KQ_F16, true, 4, 2); else KQ_F4_LAUNCH(KQ_F16, true, 8, 1); }
+    else { if (two) KQ_F4_LAUNCH(KQ_BF16, true, 4, 2); else KQ_F4_LAUNCH(KQ_BF16, true, 8, 1); }
   } else {
-    if (dtype == KQ_F16) hipLaunchKernelGGL((fp4_grouped_kernel<KQ_F16, false>), grid, dim3(F4_THREADS), 0, s, a);
-    else hipLaunchKernelGGL((fp4_grouped_kernel<KQ_BF16, false>), grid, dim3(F4_THREADS), 0, s, a);
+    if (dtype == KQ_F16) { if (two) KQ_F4_LAUNCH(KQ_F16, false, 4, 2); else KQ_F4_LAUNCH(KQ_F16, false, 4, 1); }
+    else { if (two) KQ_F4_LAUNCH(KQ_BF16, false, 4, 2); else KQ_F4_LAUNCH(KQ_BF16, false, 4, 1); }
   }
+#undef KQ_F4_LAUNCH
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
 }
