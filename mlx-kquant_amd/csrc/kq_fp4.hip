@@ -430,7 +430,8 @@ int kq_launch_fp4_moe(const void* x, const uint8_t* w, const uint8_t* w2, const 
   if (maxseg > P) maxseg = P;
   // Shapes: the fused op streams 8 column tiles per wave and step (64 output columns per workgroup), the plain op 4
   // (64 columns: twice the workgroups of the 8-tile form, 50.7 -> 43.5 us on 32 experts of 2880 x 2880 at 256 pairs);
-  // stacks whose experts see more than 12 pairs on average take both m-tiles of a segment in one pass.
+  // stacks whose experts see more than 12 pairs on average take both m-tiles of a segment in one pass, on 8 tiles
+  // where the registers hold them (bf16: two activation terms; 1024 pairs: 160 + 83 -> 137 + 79 us), else on 4.
   const bool two = (int64_t)P > 12 * (int64_t)E;
 #define KQ_F4_LAUNCH(DTV, GLUV, JV, MTV)                                                                         \
   hipLaunchKernelGGL((fp4_grouped_kernel<DTV, GLUV, JV, MTV>),                                                   \
@@ -438,10 +439,10 @@ int kq_launch_fp4_moe(const void* x, const uint8_t* w, const uint8_t* w2, const 
                      dim3(F4_THREADS), 0, s, a)
   if (glu) {
     if (dtype == KQ_F16) { if (two) KQ_F4_LAUNCH(KQ_F16, true, 4, 2); else KQ_F4_LAUNCH(KQ_F16, true, 8, 1); }
-    else { if (two) KQ_F4_LAUNCH(KQ_BF16, true, 4, 2); else KQ_F4_LAUNCH(KQ_BF16, true, 8, 1); }
+    else { if (two) KQ_F4_LAUNCH(KQ_BF16, true, 8, 2); else KQ_F4_LAUNCH(KQ_BF16, true, 8, 1); }
   } else {
     if (dtype == KQ_F16) { if (two) KQ_F4_LAUNCH(KQ_F16, false, 4, 2); else KQ_F4_LAUNCH(KQ_F16, false, 4, 1); }
-    else { if (two) KQ_F4_LAUNCH(KQ_BF16, false, 4, 2); else KQ_F4_LAUNCH(KQ_BF16, false, 4, 1); }
+    else { if (two) KQ_F4_LAUNCH(KQ_BF16, false, 8, 2); else KQ_F4_LAUNCH(KQ_BF16, false, 4, 1); }
   }
 #undef KQ_F4_LAUNCH
   KQ_HIP_CHECK(hipGetLastError());
