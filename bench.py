@@ -18,7 +18,7 @@ Extra fields: `sweep` (the decode projections of the q4_k_m recipe at M in {1,2,
 (q4_k / q5_k / q6_k GEMM 8192 -> 28672 at M in {512, 2048}), `moe` (128 experts, top-8, hidden 2048,
 intermediate 768: fused gate/up GLU in q4_k and down in q6_k at 1 and 256 tokens), `lowbit` (M=1
 GEMV 8192 -> 8192 in the low-bit codecs), `moe_decode_lowbit` (1 token, 8 of 128 experts, IQ / fp4 / q8_0 stacks),
-`read_ceiling` (stock read-only reduction and device copy on buffers of the GEMV's sizes, cold),
+`read_ceiling` (stock read-only reduction, stock bf16 GEMV and device copy on buffers of the GEMV's sizes, cold),
 `dequantize` (whole-matrix decode to f16, wire bytes in plus
 2 N K bytes out), `mid_m` (16 ... 64 activation rows on 4096-wide matrices), `no_transpose` (transpose = 0:
 128 gathered entries of (M x 128) . (128 x 512), and dense 4096 x 4096), `roofline` for the dominant kernel and `cpu_baseline`
@@ -38,9 +38,13 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLC_BYTES = 256 << 20
 # HBM bytes one headline launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
-# `bench.py --probe`: (16248.2 KiB x 1.9985 + 28.0 KiB x 1.0), each counter scaled by what it reads for
-# the probe's plain 32256 KiB device copy.  Algorithmic bytes are 33,030,144 (weights) + 28,672 (output).
-HEADLINE_TRAFFIC_BYTES = 33_280_000
+# `bench.py --probe` (KiB per dispatch of the GEMV kernel), each counter scaled by what it reads for the probe's
+# plain 32256 KiB device copy (32256 / the copy's reading).  Algorithmic bytes are 33,030,144 (weights) + 28,672
+# (output).
+HEADLINE_FETCH_KIB, HEADLINE_FETCH_SCALE = 16251.8, 1.9984
+HEADLINE_WRITE_KIB, HEADLINE_WRITE_SCALE = 28.0, 1.0
+HEADLINE_TRAFFIC_BYTES = int(round((HEADLINE_FETCH_KIB * HEADLINE_FETCH_SCALE
+                                    + HEADLINE_WRITE_KIB * HEADLINE_WRITE_SCALE) * 1024, -3))
 KQ_BF16 = 2
 
 
@@ -291,30 +295,43 @@ def cold_copies(torch, base, wbytes):
 def read_ceiling(torch, dev, sizes):
     """What this box's memory system delivers to stock kernels on buffers of the GEMV's sizes, cold (rotating
     over copies that together exceed twice the last-level cache) and timed like the GEMV (HIP-graph replays):
-    a read-only reduction (torch.sum over an int32 view: bytes read) and the runtime's device-to-device copy
-    (bytes read + bytes written).  Stated next to the 8 TB/s peak so that a GEMV rate can be compared with what
-    a plain reader reaches on the same part."""
-    rows = []
+    a read-only reduction (torch.sum over a float32 view: bytes read), the stock bf16 GEMV of the BLAS library on the
+    same bytes taken as a [rows, 4096] bf16 matrix (bytes read), and the runtime's device-to-device copy (bytes read
+    + bytes written).  Stated next to the 8 TB/s peak so that a GEMV rate can be compared with what plain readers
+    reach on the same part."""
+    rows_out = []
+    K = 4096
     for label, nbytes in sizes:
         n32 = nbytes // 4
         ncopies = max(2, (2 * LLC_BYTES + nbytes - 1) // nbytes + 1)
         srcs = [torch.randint(-2 ** 31, 2 ** 31 - 1, (n32,), dtype=torch.int32, device=dev) for _ in range(ncopies)]
-        acc = torch.empty((), dtype=torch.int64, device=dev)
+        acc = torch.empty((), dtype=torch.float32, device=dev)
         dsts = [torch.empty_like(srcs[0]) for _ in range(ncopies)]
+        rows = n32 * 2 // K
+        xv = torch.randn(K, device=dev).to(torch.bfloat16)
+        yv = torch.empty(rows, dtype=torch.bfloat16, device=dev)
 
         def summer(v):
-            return lambda stream=None: torch.sum(v, dim=(0,), dtype=torch.int64, out=acc)
+            return lambda stream=None: torch.sum(v.view(torch.float32), dim=(0,), out=acc)
+
+        def gemv(v):
+            m = v.view(torch.bfloat16)[:rows * K].view(rows, K)
+            return lambda stream=None: torch.mv(m, xv, out=yv)
 
         def copier(v, d):
             return lambda stream=None: d.copy_(v)
 
         ts, _ = time_calls(torch, [summer(v) for v in srcs], 200, 20)
+        tg, _ = time_calls(torch, [gemv(v) for v in srcs], 200, 20)
         tc, _ = time_calls(torch, [copier(v, d) for v, d in zip(srcs, dsts)], 200, 20)
-        rows.append({"buffer": label, "bytes": n32 * 4,
-                     "sum_int32_us": round(ts * 1e3, 2), "sum_int32_read_gbs": round(n32 * 4 / (ts * 1e-3) / 1e9, 1),
-                     "copy_us": round(tc * 1e3, 2), "copy_read_plus_write_gbs": round(2 * n32 * 4 / (tc * 1e-3) / 1e9, 1)})
+        rows_out.append({"buffer": label, "bytes": n32 * 4,
+                         "sum_f32_us": round(ts * 1e3, 2), "sum_f32_read_gbs": round(n32 * 4 / (ts * 1e-3) / 1e9, 1),
+                         "stock_bf16_gemv_us": round(tg * 1e3, 2),
+                         "stock_bf16_gemv_read_gbs": round(rows * K * 2 / (tg * 1e-3) / 1e9, 1),
+                         "copy_us": round(tc * 1e3, 2),
+                         "copy_read_plus_write_gbs": round(2 * n32 * 4 / (tc * 1e-3) / 1e9, 1)})
         del srcs, dsts
-    return rows
+    return rows_out
 
 
 def cpu_baseline(wire_np, codec, K, M, budget_s=12.0):
@@ -573,7 +590,7 @@ def main():
                                 "down_us": round(td * 1e3, 1),
                                 "glu_gbs": round(ne * 2 * mbytes / (tg * 1e-3) / 1e9, 1),
                                 "down_gbs": round(ne * mbytes / (td * 1e-3) / 1e9, 1),
-                                "note": "grouped code-level MFMA kernel (f32 biases, swiglu_clamp)"}
+                                "note": "block-scaled fp4 MFMA kernel, wire blocks undecoded (f32 biases, swiglu_clamp)"}
             del gate, up, down
 
         # ---------------- MoE decode (1 token, 8 of 128 experts of 2048 <-> 768) in the low-bit / fp4 codecs

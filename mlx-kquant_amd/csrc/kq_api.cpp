@@ -1,5 +1,6 @@
 // C ABI of libkq (declared in include/kq.h): argument validation, error reporting, the device copy of the
 // IQ codebooks and routing to the HIP launchers.  Compiled by hipcc as HIP (the codebooks are a __device__ array).
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -244,7 +245,8 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
                            const float* bias, const float* bias2, void* out, int T, int R, int E, int N, int K,
                            int64_t estride, int glu, int act, float limit, float alpha, int codec, int dtype, void* ws,
                            size_t ws_bytes, KqOutMap om, hipStream_t s, int entry_rows = 1);
-static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int E, int N, int K);
+static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int E, int N, int K,
+                            bool stream_takes);
 
 int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_dev, const uint32_t* rhs_idx_dev,
                   void* out_dev, int B, int M, int E, int N, int K, int64_t x_batch_stride,
@@ -272,7 +274,9 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
   // many output rows: gather them into a dense matrix and run the expert-grouped kernels
   int64_t P;
   if (workspace_dev && gather_batched_shape(B, M, E, N, K, transpose, codec, &P) &&
-      !per_entry_route(P, M, false, 0, 0, codec, E, N, K) &&
+      !per_entry_route(P, M, false, 0, 0, codec, E, N, K,
+                       kq_gather_stream_takes(x_dev, w_dev, nullptr, (int)(P > 0x7fffffff ? 0x7fffffff : P), N, K, true,
+                                              x_batch_stride, w_expert_stride_bytes, false, codec)) &&
       !(reinterpret_cast<uintptr_t>(workspace_dev) & 255) && !(reinterpret_cast<uintptr_t>(x_dev) & 15) &&
       !(x_batch_stride & 7)) {
     const size_t need = kq_gather_qmm_workspace_size(B, M, E, N, K, transpose, codec, dtype);
@@ -334,83 +338,83 @@ size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int cod
 }
 
 // Batched MoE path: returns KQ_ERR_UNSUPPORTED (error text untouched) when it does not apply.
-// Up to this many (token, expert) pairs of a q4_k / q5_k / q6_k stack the per-entry streamed kernel is the faster
-// route (128 experts of 2048 <-> 768, top-8, fused gate / up + down: 3 tokens 17.5 + 16.3 against 28.0 + 20.5 us,
-// 6 tokens 25.2 + 27.3 against 28.3 + 27.4, 8 tokens 30.0 + 33.7 against 35.1 + 32.9).
-#ifndef KQ_PER_ENTRY_MAX_PAIRS
-#define KQ_PER_ENTRY_MAX_PAIRS 48
-#endif
-// q2_k / q3_k stacks have no expert-grouped kernel of their own (their batched route is the any-codec kernel), so
-// the per-entry kernel stays ahead much longer (same stacks, fused gate / up + down, us: 64 pairs 21.9 + 20.1
-// against 87.9 + 47.6 for q2_k, 36.0 + 24.6 against 113.9 + 60.3 for q3_k; 256 pairs 67 + 61 against 154 + 76 and
-// 126 + 76 against 200 + 106; 512 pairs 125 + 116 against 156 + 86 and 245 + 144 against 202 + 108).
-#ifndef KQ_PER_ENTRY_MAX_PAIRS_LOW
-#define KQ_PER_ENTRY_MAX_PAIRS_LOW 256
-#endif
-// The legacy / other IQ / fp4 codecs: the code-level per-entry kernel against the code-level grouped kernel (same
-// stacks, us: mxfp4 32 pairs 24.9 + 21.0 against 37.4 + 22.7, 64 pairs 41.2 + 36.1 against 53.8 + 34.1; q4_0 64 pairs
-// 39.2 + 27.7 against 52.6 + 33.4; iq2_xs 48 pairs 33.6 + 29.8 against 40.7 + 26.6, even at 64).  nvfp4's batched
-// route is the any-codec kernel: 64 pairs 68 + 51 against 128 + 71, 128 pairs 127 + 96 against 158 + 96, behind at 256.
-#ifndef KQ_PER_ENTRY_MAX_PAIRS_CODES
-#define KQ_PER_ENTRY_MAX_PAIRS_CODES 48
-#endif
-#ifndef KQ_PER_ENTRY_MAX_PAIRS_NVFP4
-#define KQ_PER_ENTRY_MAX_PAIRS_NVFP4 128
-#endif
-// q8_0: the streamed per-entry kernel against the code-level grouped kernel (same stacks, us: 32 pairs 21.0 + 15.0
-// against 38.8 + 23.2, 64 pairs 38.8 + 28.0 against 55.7 + 36.8, 128 pairs 74.3 + 53.0 against 71.4 + 48.6).
-#ifndef KQ_PER_ENTRY_MAX_PAIRS_Q8
-#define KQ_PER_ENTRY_MAX_PAIRS_Q8 64
-#endif
-// iq4_nl / q4_0 / mxfp4 calls the streamed kernel takes (K a multiple of 256), against the
-// code-level grouped kernel (same stacks, us: mxfp4 32 pairs 20.2 + 16.5 against 37.4 + 22.7, 64 pairs 37.2 + 30.1
-// against 50.1 + 30.5, 96 pairs 54.5 + 43.7 against 58.3 + 37.3; q4_0 64 pairs 33.3 + 28.3 against 48.0 + 25.8).
-// nvfp4 calls the streamed kernel takes, against the any-codec kernel (us: 128 pairs 71.6 + 58.4 entry by entry,
-// 160 pairs 87 + 72 against 187 + 92, 256 pairs 138 + 113 against 213 + 105); the streamed kernel stops at 256 entries.
-#ifndef KQ_PER_ENTRY_MAX_PAIRS_NVFP4_STREAMED
-#define KQ_PER_ENTRY_MAX_PAIRS_NVFP4_STREAMED 256
-#endif
-#ifndef KQ_PER_ENTRY_MAX_PAIRS_NIB
-#define KQ_PER_ENTRY_MAX_PAIRS_NIB 64
-#endif
-#ifndef KQ_PER_ENTRY_MAX_PAIRS_IQ
-#define KQ_PER_ENTRY_MAX_PAIRS_IQ 64
-#endif
+//
+// Entry by entry or grouped.  A call of P (token, expert) pairs can run entry by entry (one grid row per pair, every
+// pair streams its expert's matrix) or sorted by expert (one prologue launch, then every expert's matrix once for all
+// of its pairs).  Entry by entry saves the prologue and the mostly empty 32-row segments; it pays by reading a
+// matrix once per pair instead of once per call.  The crossover was measured per codec family on the reference stack
+// (128 experts of 2048 <-> 768, top-8, fused gate / up + down, us entry by entry against grouped):
+//   q4_k / q5_k / q6_k (streamed kernel against the grouped K-quant kernel): 24 pairs 17.5 + 16.3 against
+//     28.0 + 20.5, 48 pairs 25.2 + 27.3 against 28.3 + 27.4, 64 pairs 30.0 + 33.7 against 35.1 + 32.9      -> 48
+//   q2_k / q3_k (streamed against the any-codec kernel): 64 pairs 21.9 + 20.1 against 87.9 + 47.6 (q2_k), 256 pairs
+//     67 + 61 against 154 + 76 and 126 + 76 against 200 + 106, 512 pairs 125 + 116 against 156 + 86        -> 256
+//   q8_0 (streamed against the code-level grouped kernel): 64 pairs 38.8 + 28.0 against 55.7 + 36.8, 128 pairs
+//     74.3 + 53.0 against 71.4 + 48.6                                                                        -> 64
+//   iq4_nl / q4_0 / mxfp4 with K a multiple of 256 (streamed against code-level grouped): mxfp4 64 pairs 37.2 + 30.1
+//     against 50.1 + 30.5, 96 pairs 54.5 + 43.7 against 58.3 + 37.3; q4_0 64 pairs 33.3 + 28.3 against 48.0 + 25.8 -> 64
+//   iq4_xs / iq3_s / iq2_xxs (streamed against code-level grouped)                                          -> 64
+//   nvfp4 with K a multiple of 256 (streamed against the any-codec kernel): 160 pairs 87 + 72 against 187 + 92,
+//     256 pairs 138 + 113 against 213 + 105; the streamed kernel stops at 256 entries                       -> 256
+//   the same codecs where the streamed kernel does not apply, and the other legacy / IQ codecs (code-level per-entry
+//     kernel against code-level grouped): mxfp4 32 pairs 24.9 + 21.0 against 37.4 + 22.7, 64 pairs 41.2 + 36.1
+//     against 53.8 + 34.1; iq2_xs 48 pairs 33.6 + 29.8 against 40.7 + 26.6                                  -> 48
+//   nvfp4 there (against the any-codec kernel): 64 pairs 68 + 51 against 128 + 71, 128 pairs 127 + 96 against
+//     158 + 96                                                                                               -> 128
+// A family's figure is a crossover on that stack only.  What it stands for is carried to other stacks in three
+// bounds, all of which a call must meet to run entry by entry:
+//   pairs:             P <= the figure (more pairs were not measured to pay on any stack);
+//   pairs per expert:  P / E <= figure / 128 (the saving of the grouped route grows with the pairs that share an
+//                      expert: 32 experts of 3072 x 3072 in mxfp4, 64 pairs, 188 + 81 us entry by entry against
+//                      118 + 68 grouped);
+//   bytes read again:  (P - D(P, E)) x bytes of one expert's matrices <= the same expression on the reference stack
+//                      at the figure, D(P, E) = E (1 - exp(-P / E)) being the distinct experts P uniform pairs hit:
+//                      the bytes a call reads beyond the grouped route's are what it pays for skipping the prologue,
+//                      and larger matrices reach that price with fewer repeated experts.
+struct EntryFamily {
+  int pairs;  // crossover on the reference stack
+};
+static constexpr EntryFamily kEntryKQuant{48}, kEntryLowK{256}, kEntryQ8{64}, kEntryNibStreamed{64}, kEntryIq{64},
+    kEntryNvfp4Streamed{256}, kEntryCodes{48}, kEntryNvfp4Codes{128};
+static constexpr int kEntryRefExperts = 128;
+static constexpr double kEntryRefWeights = 768.0 * 2048.0;  // weights of one matrix of the reference stack
+
+static double distinct_experts(double pairs, double experts) { return experts * (1.0 - std::exp(-pairs / experts)); }
+
+static bool entry_by_entry_pays(EntryFamily f, int64_t P, int E, int N, int K) {
+  if (P > f.pairs) return false;
+  if (P * kEntryRefExperts > (int64_t)f.pairs * E) return false;
+  // bytes per weight and the fused form's second matrix scale both sides alike
+  const double again = ((double)P - distinct_experts((double)P, E)) * (double)N * (double)K;
+  const double again_ref = (f.pairs - distinct_experts(f.pairs, kEntryRefExperts)) * kEntryRefWeights;
+  return again <= again_ref;
+}
+
 // True when a call of P (token, expert) pairs is better served entry by entry than by the sorted, expert-grouped
 // kernels.  entry_rows = activation rows per entry of the caller's per-entry fallback (1 for the MoE ops; gather_qmm's
-// M): the per-entry kernels take one row per entry, the older K-quant ones up to eight.
-// The pair counts above were measured on stacks of 128 experts.  Entry by entry every pair reads its expert's matrix
-// again while the grouped kernels read a matrix once per call, so what decides is how many pairs share an expert:
-// the limits shrink in proportion for shorter stacks (32 experts of 3072 x 3072 in mxfp4, 64 pairs: 188 + 81 us entry
-// by entry against 118 + 68 grouped).
-static int64_t per_entry_limit(int limit, int E) {
-  const int64_t scaled = (int64_t)limit * E / 128;
-  return scaled < limit ? scaled : limit;
-}
-static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int E, int N, int K) {
+// M): the per-entry kernels take one row per entry, the older K-quant ones up to eight.  stream_takes: the streamed
+// gathered kernel accepts the call's shape and alignment; where it does not, the families measured on it keep the
+// grouped route (the older per-entry kernels behind it are 2 - 4 x slower at these pair counts).
+static bool per_entry_route(int64_t P, int entry_rows, bool has_bias, int glu, int act, int codec, int E, int N, int K,
+                            bool stream_takes) {
   if (P <= 16) return false;  // the callers never reach the grouped route with so few pairs
   const bool grouped_codec = codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K;
   const bool low_codec = codec == KQ_Q2_K || codec == KQ_Q3_K;  // their batched route is the any-codec kernel
   const bool iq_codec = codec == KQ_IQ4_XS || codec == KQ_IQ3_S || codec == KQ_IQ2_XXS;
   const bool q8 = codec == KQ_Q8_0;  // per-entry kernel: the streamed one; batched: the code-level grouped kernel
-  const bool streamed_k = !((K >> 8) > (glu ? 16 : 32) || (K & 255));
-  const bool streamed_shape = streamed_k && !(has_bias || (glu && act == KQ_ACT_SWIGLU_CLAMP));
   // iq4_nl / q4_0 / mxfp4 / nvfp4 entries the streamed kernel takes (biases and swiglu_clamp included); the others
   // fall to the code-level rule below
-  if ((codec == KQ_IQ4_NL || codec == KQ_Q4_0 || codec == KQ_MXFP4) && streamed_k && entry_rows == 1 &&
-      P <= per_entry_limit(KQ_PER_ENTRY_MAX_PAIRS_NIB, E))
+  if ((codec == KQ_IQ4_NL || codec == KQ_Q4_0 || codec == KQ_MXFP4) && stream_takes && entry_rows == 1 &&
+      entry_by_entry_pays(kEntryNibStreamed, P, E, N, K))
     return true;
-  if (codec == KQ_NVFP4 && streamed_k && entry_rows == 1 && P <= per_entry_limit(KQ_PER_ENTRY_MAX_PAIRS_NVFP4_STREAMED, E))
+  if (codec == KQ_NVFP4 && stream_takes && entry_rows == 1 && entry_by_entry_pays(kEntryNvfp4Streamed, P, E, N, K))
     return true;
   // the other codecs' per-entry kernel is the code-level one, which takes biases and every activation
   if (!grouped_codec && !low_codec && !iq_codec && !q8)
-    return entry_rows == 1 &&
-           P <= per_entry_limit(codec == KQ_NVFP4 ? KQ_PER_ENTRY_MAX_PAIRS_NVFP4 : KQ_PER_ENTRY_MAX_PAIRS_CODES, E) &&
+    return entry_rows == 1 && entry_by_entry_pays(codec == KQ_NVFP4 ? kEntryNvfp4Codes : kEntryCodes, P, E, N, K) &&
            kq_codes_gather_supported(1, N, K, codec);
-  if (!streamed_shape) return false;
-  if (grouped_codec) return P <= per_entry_limit(KQ_PER_ENTRY_MAX_PAIRS, E) && entry_rows <= 8;
-  return entry_rows == 1 &&
-         P <= per_entry_limit(low_codec ? KQ_PER_ENTRY_MAX_PAIRS_LOW : q8 ? KQ_PER_ENTRY_MAX_PAIRS_Q8 : KQ_PER_ENTRY_MAX_PAIRS_IQ, E);
+  if (!stream_takes || has_bias || (glu && act == KQ_ACT_SWIGLU_CLAMP)) return false;
+  if (grouped_codec) return entry_rows <= 8 && entry_by_entry_pays(kEntryKQuant, P, E, N, K);
+  return entry_rows == 1 && entry_by_entry_pays(low_codec ? kEntryLowK : q8 ? kEntryQ8 : kEntryIq, P, E, N, K);
 }
 
 static int try_moe_grouped(const char* op, const void* x, const void* w, const void* w2, const uint32_t* idx,
@@ -421,7 +425,9 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
   // few entries: the per-entry kernels (the caller tries them next) beat the prologue + grouped-kernel pair
-  if (per_entry_route(P, entry_rows, bias || bias2, glu, act, codec, E, N, K)) return KQ_ERR_UNSUPPORTED;
+  if (per_entry_route(P, entry_rows, bias || bias2, glu, act, codec, E, N, K,
+                      kq_gather_stream_takes(x, w, w2, (int)P, N, K, false, K, estride, false, codec)))
+    return KQ_ERR_UNSUPPORTED;
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
     // mxfp4: the wire blocks go into the block-scaled matrix instruction undecoded (kq_fp4.hip)
     if (kq_fp4_moe_supported((int)P, E, N, K, codec)) {

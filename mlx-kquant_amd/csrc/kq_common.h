@@ -119,6 +119,11 @@ int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, 
                             void* out, int entries, int N, int K, int x_div, int64_t x_row_stride,
                             int64_t w_expert_stride, int act, float limit, float alpha, const float* bias,
                             const float* bias2, int codec, int dtype, int E, KqOutMap om, hipStream_t s);
+// Whether kq_launch_gather_stream takes a call of this shape and alignment (strided_x: rows addressed through lhs
+// with x_row_stride); the most entries it takes.
+bool kq_gather_stream_takes(const void* x, const void* w, const void* w2, int entries, int N, int K, bool strided_x,
+                            int64_t x_row_stride, int64_t w_expert_stride, bool second_bias_without_glu, int codec);
+int kq_gather_stream_max_entries();
 // codecs whose gathered calls the streamed kernel also takes with biases and swiglu_clamp (the fp4 stacks that carry
 // them, and the two codecs that share their unit)
 inline bool kq_stream_full_epilogue(int codec) {

@@ -1623,20 +1623,33 @@ int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N,
 #ifndef KQ_GATHER_STREAM_MAX_ENTRIES
 #define KQ_GATHER_STREAM_MAX_ENTRIES 256
 #endif
+int kq_gather_stream_max_entries() { return KQ_GATHER_STREAM_MAX_ENTRIES; }
+
+// Whether the streamed gathered kernel takes a call of this shape and alignment (the launcher's own test, also asked
+// by the router that chooses between the per-entry and the expert-grouped kernels before either runs).
+bool kq_gather_stream_takes(const void* x, const void* w, const void* w2, int entries, int N, int K, bool strided_x,
+                            int64_t x_row_stride, int64_t w_expert_stride, bool second_bias_without_glu, int codec) {
+  if (!st_codec_ok(codec)) return false;
+  if (entries < 1 || entries > KQ_GATHER_STREAM_MAX_ENTRIES || N < 1 || K < 256 || (K & 255)) return false;
+  const bool glu = w2 != nullptr;
+  if ((K >> 8) > (glu ? 16 : 32) || second_bias_without_glu) return false;
+  if ((int64_t)entries * ((N + ST_ROWS - 1) / ST_ROWS) > 65535 * 16) return false;
+  const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : codec == KQ_MXFP4 ? 0 : 1;
+  if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
+      ((uintptr_t)w_expert_stride & wmask) || (reinterpret_cast<uintptr_t>(x) & 15) || ((K * 2) & 15) ||
+      (strided_x && ((x_row_stride * 2) & 15)))
+    return false;
+  return true;
+}
+
 int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, const uint32_t* lhs, const uint32_t* rhs,
                             void* out, int entries, int N, int K, int x_div, int64_t x_row_stride,
                             int64_t w_expert_stride, int act, float limit, float alpha, const float* bias,
                             const float* bias2, int codec, int dtype, int E, KqOutMap om, hipStream_t s) {
-  if (!st_codec_ok(codec)) return KQ_ERR_UNSUPPORTED;
-  if (entries < 1 || entries > KQ_GATHER_STREAM_MAX_ENTRIES || N < 1 || K < 256 || (K & 255) || !rhs) return KQ_ERR_UNSUPPORTED;
-  const bool glu = w2 != nullptr;
-  if ((K >> 8) > (glu ? 16 : 32) || (!glu && bias2)) return KQ_ERR_UNSUPPORTED;
-  if ((int64_t)entries * ((N + ST_ROWS - 1) / ST_ROWS) > 65535 * 16) return KQ_ERR_UNSUPPORTED;
-  const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : codec == KQ_MXFP4 ? 0 : 1;
-  if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
-      ((uintptr_t)w_expert_stride & wmask) || (reinterpret_cast<uintptr_t>(x) & 15) || ((K * 2) & 15) ||
-      (lhs && ((x_row_stride * 2) & 15)))
+  if (!rhs || !kq_gather_stream_takes(x, w, w2, entries, N, K, lhs != nullptr, x_row_stride, w_expert_stride,
+                                      !w2 && bias2, codec))
     return KQ_ERR_UNSUPPORTED;
+  const bool glu = w2 != nullptr;
   StArgs a{};
   a.x = x;
   a.w = w;

@@ -230,6 +230,50 @@ def test_moe_low_bit_routes_either_side_of_the_entry_threshold(kq, codec, T):
     assert rel_l2(dev_to_bits(got), want, "float16") <= TOL, (codec, T)
 
 
+@pytest.mark.parametrize("T", [4, 16])
+def test_moe_routes_on_32_experts_of_2880_square(kq, T):
+    """A stack unlike the one the entry-by-entry limits were measured on (32 experts of 2880 x 2880 in mxfp4, top-4,
+    biases with swiglu_clamp): 16 pairs run entry by entry, 64 on the expert-grouped kernels; the fused gate / up
+    projection and the biased down projection agree with the oracle on both."""
+    codec, E, N, K, R = "mxfp4", 32, 2880, 2880, 4
+    gate, up = _stack(codec, E, N, K, seed=131), _stack(codec, E, N, K, seed=132)
+    rng = np.random.default_rng(133)
+    idx = np.stack([rng.permutation(E)[:R] for _ in range(T)])
+    gb = (rng.standard_normal((E, N)) * 0.05).astype(np.float32)
+    ub = (rng.standard_normal((E, N)) * 0.05).astype(np.float32)
+    xb, xt = make_x((T, K), "bfloat16", seed=134, scale=0.05)
+    got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act="swiglu_clamp", limit=7.0,
+                               alpha=1.702, gate_bias=torch.from_numpy(gb).cuda(), up_bias=torch.from_numpy(ub).cuda())
+    want = _glu_truth(codec, xb, gate, up, idx, "swiglu_clamp", 7.0, 1.702, gb, ub)
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, T
+    hb, ht = make_x((T, R, K), "bfloat16", seed=135, scale=0.05)
+    got = kq.gather_qmv_kq(ht, wire_to_dev(up), codec, _idx_dev(idx), bias=torch.from_numpy(gb).cuda())
+    assert rel_l2(dev_to_bits(got), O.gather_qmv(hb, up, codec, idx, gb, "bfloat16"), "bfloat16") <= TOL, T
+
+
+@pytest.mark.parametrize("N,K,T", [(1536, 2048, 5), (2048, 2560, 5), (1536, 2048, 10)])
+def test_moe_q4k_routes_by_pairs_per_expert_and_bytes_read_again(kq, N, K, T):
+    """64 experts in q4_k, top-4.  20 pairs of 1536 x 2048 matrices run entry by entry; the same 20 pairs of
+    2048 x 2560 matrices would read more bytes again than the grouped route's prologue costs, and 40 pairs are more
+    pairs per expert than were measured to pay: both go to the expert-grouped kernels.  All agree with the oracle;
+    an activation matrix that starts 2 bytes off a 16-byte boundary (which the streamed and the grouped kernels both
+    decline) still does."""
+    codec, E, R = "q4_k", 64, 4
+    gate, up = _stack(codec, E, N, K, seed=141), _stack(codec, E, N, K, seed=142)
+    rng = np.random.default_rng(143)
+    idx = np.stack([rng.permutation(E)[:R] for _ in range(T)])
+    xb, xt = make_x((T, K), "bfloat16", seed=144, scale=0.03)
+    want = _glu_truth(codec, xb, gate, up, idx, "silu")
+    got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act="silu")
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (N, K, T)
+    off = torch.empty(T * K + 8, dtype=xt.dtype, device=xt.device)
+    shifted = off[1:1 + T * K].view(T, K)
+    shifted.copy_(xt)
+    assert shifted.data_ptr() % 16 == 2
+    got = kq.moe_glu_gather_kq(shifted, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act="silu")
+    assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (N, K, T, "shifted")
+
+
 @pytest.mark.parametrize("codec", ["q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("E,N,K,T,R", [(6, 136, 768, 20, 3), (8, 200, 512, 100, 2), (128, 64, 256, 8, 8),
                                        (5, 72, 4352, 9, 2)])
