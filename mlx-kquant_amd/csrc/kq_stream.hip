@@ -1051,16 +1051,34 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   // ---- activations -> f16 fragments (+ sums) in the wave's LDS, then this lane's A registers
   float xscale = 1.0f, inv = 1.0f;
   if constexpr (DT == KQ_BF16) {
-    float amax = 0.f;
+    // largest magnitude: bf16 magnitudes order like their bit patterns, two per packed integer maximum
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    u16x2 am2 = {0, 0};
+    const uint32_t absmask = opaque_sgpr(0x7fff7fffu);
     SFor<MB * XL>::run([&](auto t) {
       const u32x4 v = xreg[decltype(t)::value];
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] << 16)));
-        amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] & 0xffff0000u)));
+        const uint32_t mag = v[e] & absmask;
+        am2 = __builtin_elementwise_max(am2, __builtin_bit_cast(u16x2, mag));
       }
     });
+    float amax = __builtin_bit_cast(float, (uint32_t)(am2[0] > am2[1] ? am2[0] : am2[1]) << 16);
     amax = wave_max_nonneg(amax);
+    if (((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff) == 0xff) {
+      // an infinity or a NaN among the activations (their patterns order above every finite one): the largest
+      // finite-or-infinite magnitude the floating-point maximum finds, which ignores NaNs
+      amax = 0.f;
+      SFor<MB * XL>::run([&](auto t) {
+        const u32x4 v = xreg[decltype(t)::value];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] << 16)));
+          amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, v[e] & 0xffff0000u)));
+        }
+      });
+      amax = wave_max_nonneg(amax);
+    }
     // bring the largest magnitude into [2^14, 2^15): exact power-of-two scaling
     const uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xff;
     if (eb != 0 && eb != 0xff) {
@@ -1087,15 +1105,21 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
       const int gi = lane + 64 * s, uu = gi >> 5, grp = gi & 31;
       const u32x4 v = xreg[m * XL + s];
       _Float16 h[8];
+      typedef _Float16 f16x2p __attribute__((ext_vector_type(2)));
+      f16x2p hp[4];
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         if constexpr (DT == KQ_BF16) {
-          h[2 * e] = (_Float16)(__builtin_bit_cast(float, v[e] << 16) * inv);
-          h[2 * e + 1] = (_Float16)(__builtin_bit_cast(float, v[e] & 0xffff0000u) * inv);
+          // a bf16 number times a power of two is an f16 number unless it falls below the f16 normals, where the
+          // truncating pair conversion drops bits under 2^-38 of the largest magnitude
+          hp[e] = __builtin_bit_cast(f16x2p, __builtin_amdgcn_cvt_pkrtz(__builtin_bit_cast(float, v[e] << 16) * inv,
+                                                                        __builtin_bit_cast(float, v[e] & 0xffff0000u) * inv));
         } else {
-          h[2 * e] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] & 0xffff));
-          h[2 * e + 1] = __builtin_bit_cast(_Float16, (uint16_t)(v[e] >> 16));
+          const uint32_t word = v[e];  // (a bit cast of the vector element itself reads element 0 every time)
+          hp[e] = __builtin_bit_cast(f16x2p, word);
         }
+        h[2 * e] = hp[e][0];
+        h[2 * e + 1] = hp[e][1];
       }
       constexpr int XORD = st_xord<C>();
       if constexpr (XORD == 0) {  // k0 k2 k1 k3 inside every group of four
@@ -1133,8 +1157,11 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
           *reinterpret_cast<u32x4*>(xs + (ml * ST_XU + uu) * 256 + 16 * (grp >> 1) + (high ? 8 : 0)) = o;
       }
       float sum = 0.f;
+      {
+        const f16x2p ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
-      for (int e = 0; e < 8; e++) sum += (float)h[e];
+        for (int e = 0; e < 4; e++) sum = __builtin_amdgcn_fdot2(hp[e], ones, sum, false);
+      }
       sum += dpp_f<0xB1>(sum);  // lanes l ^ 1: 16 values
       if constexpr (XSG == 8) {
         if ((lane & 1) == 0) xsum[(m * ST_XU + uu) * 16 + (grp >> 1)] = sum;
