@@ -380,6 +380,9 @@ def main():
     ap.add_argument("--probe-moe", type=int, default=None, metavar="TOKENS",
                     help="counter probe for `rocprofv3 --pmc`: 10 launches each of the q4_k GLU op and the q6_k down "
                          "op of the 128-expert top-8 MoE at TOKENS tokens, nothing else")
+    ap.add_argument("--probe-moe-mxfp4", type=int, default=None, metavar="TOKENS",
+                    help="counter probe for `rocprofv3 --pmc`: 10 launches each of the biased swiglu_clamp GLU op and "
+                         "the biased down op of the 32-expert top-4 mxfp4 MoE (2880 x 2880) at TOKENS tokens, nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU.",
@@ -426,6 +429,26 @@ def main():
         print(json.dumps({"probe": "10 GLU + 10 down launches", "tokens": T, "experts_touched_mean": sum(touched) / 10,
                           "glu_bytes_per_expert": 2 * I * kq.bytes_per_row("q4_k", H),
                           "down_bytes_per_expert": H * kq.bytes_per_row("q6_k", I)}))
+        return
+
+    if args.probe_moe_mxfp4:
+        E, H, TOPK, T = 32, 2880, 4, args.probe_moe_mxfp4
+        gate = synth_wire_torch("mxfp4", E * H, H, 21, dev).reshape(E, H, -1)
+        up = synth_wire_torch("mxfp4", E * H, H, 22, dev).reshape(E, H, -1)
+        down = synth_wire_torch("mxfp4", E * H, H, 23, dev).reshape(E, H, -1)
+        gb, ub, db = (torch.randn((E, H), device=dev, generator=gx) * 0.01 for _ in range(3))
+        xt = randx((T, H), 0.5)
+        touched = []
+        for r in range(10):
+            idx = torch.randn((T, E), device=dev, generator=gx).topk(TOPK, dim=-1).indices.to(torch.int32).contiguous()
+            call, h = abi.moe_glu(xt, gate, up, "mxfp4", idx, act=3, limit=7.0, alpha=1.702, gate_bias=gb, up_bias=ub)
+            call()
+            abi.gather_qmv(h, down, "mxfp4", idx, bias=db)()
+            touched.append(int(idx.unique().numel()))
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "10 GLU + 10 down launches", "tokens": T, "experts_touched_mean": sum(touched) / 10,
+                          "glu_bytes_per_expert": 2 * H * kq.bytes_per_row("mxfp4", H),
+                          "down_bytes_per_expert": H * kq.bytes_per_row("mxfp4", H)}))
         return
 
     if args.probe_prefill:

@@ -425,11 +425,13 @@ static int try_moe_grouped(const char* op, const void* x, const void* w, const v
   const int64_t P = (int64_t)T * R;
   if (P > 0x7fffffff) return KQ_ERR_UNSUPPORTED;
   // few entries: the per-entry kernels (the caller tries them next) beat the prologue + grouped-kernel pair
-  if (per_entry_route(P, entry_rows, bias || bias2, glu, act, codec, E, N, K,
-                      kq_gather_stream_takes(x, w, w2, (int)P, N, K, false, K, estride, false, codec)))
-    return KQ_ERR_UNSUPPORTED;
+  const bool stream_takes = kq_gather_stream_takes(x, w, w2, (int)P, N, K, false, K, estride, false, codec);
+  if (per_entry_route(P, entry_rows, bias || bias2, glu, act, codec, E, N, K, stream_takes)) return KQ_ERR_UNSUPPORTED;
   if (!kq_moe_grouped_supported((int)P, E, N, K, codec)) {
-    // mxfp4: the wire blocks go into the block-scaled matrix instruction undecoded (kq_fp4.hip)
+    // mxfp4: the wire blocks go into the block-scaled matrix instruction undecoded (kq_fp4.hip).  The plain op on
+    // stacks whose K ends inside a 256-weight unit stays entry by entry on the streamed kernel up to 11 pairs (32
+    // experts of 2880 x 2880: 8 pairs 14.6 us against 16.6 here, 16 pairs 24.9 against 20.3).
+    if (codec == KQ_MXFP4 && !glu && (K & 255) && P < 12 && entry_rows == 1 && stream_takes) return KQ_ERR_UNSUPPORTED;
     if (kq_fp4_moe_supported((int)P, E, N, K, codec)) {
       const size_t need = kq_fp4_moe_workspace_bytes((int)P, E, glu ? T : (int)P, K);
       if (!ws || ws_bytes < need)

@@ -371,7 +371,10 @@ bool kq_fp4_moe_supported(int P, int E, int N, int K, int codec) {
   // there), the code-level one elsewhere, which this kernel passes at 8 pairs (32 experts of 2880 x 2880, fused +
   // plain op: 4 pairs 16.6 + 11.8 us entry by entry against 18.0 + 13.3 here, 8 pairs 27.1 + 17.5 against 24.8 + 16.6,
   // 16 pairs 49.0 + 29.8 against 34.6 + 20.3).
-  const int min_pairs = (K & 255) ? 8 : 17;
+#ifndef KQ_FP4_MIN_PAIRS_TAIL
+#define KQ_FP4_MIN_PAIRS_TAIL 8
+#endif
+  const int min_pairs = (K & 255) ? KQ_FP4_MIN_PAIRS_TAIL : 17;
   return codec == KQ_MXFP4 && P >= min_pairs && E > 0 && E <= 4096 && (int64_t)E + P / 32 < 65535 && N > 0 && K >= 32 &&
          (K & 31) == 0 && (int64_t)N * (K >> 5) * 17 < ((int64_t)1 << 32);
 }

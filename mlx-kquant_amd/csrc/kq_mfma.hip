@@ -1373,9 +1373,9 @@ bool sk_shape_ok(int M, int K, int codec, const void* x, const void* w, const vo
 }  // namespace
 
 size_t kq_qmm_tuned_workspace_bytes(int M, int N, int K, int codec) {
-  if (M < 1 || M > SK_MAXM || (K & 255) || K == 0) return 0;
+  if (M < 1 || M > SK_MAXM || K == 0) return 0;
   const size_t st = kq_stream_workspace_bytes(M, N, K, codec);  // also covers codecs only the streamed kernel takes
-  if (!sk_codec_ok(codec)) return st;
+  if (!sk_codec_ok(codec) || (K & 255)) return st;
   const SkSplit p = sk_split_plan(N, K);
   const size_t own = p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
   return own > st ? own : st;

@@ -238,6 +238,14 @@ constexpr int st_tbl_bytes() {
   return st_pair_table<C>() ? 32768 : C == KQ_IQ2_XXS ? (4096 + 2048) * st_iq2_copies<C, MB, NW, GM>() :
          st_iq3s_merged<C, MB, NW, GM>() ? 65536 + 4096 : C == KQ_IQ3_S ? 4096 + 4096 : 0;
 }
+// Codecs of 32-weight blocks whose unit is eight blocks copied as they lie: K may end inside a unit (any multiple
+// of 32).  The last unit of a row then holds K % 256 / 32 blocks, T bytes.  Nothing past the row's end is read:
+// pieces that lie inside the T bytes travel as usual; the piece the row ends in (16 ps < T < 16 ps + 16) is fetched
+// from T - 16, so that it ends with the row, and the wave then moves its bytes down to where the unit expects them;
+// pieces that start past the end are fetched from the unit's start (their blocks get a zero scale and zero
+// activations, whatever bytes they hold).
+template <int C>
+constexpr bool st_tail_codec() { return C == KQ_MXFP4 || C == KQ_Q4_0 || C == KQ_IQ4_NL || C == KQ_Q8_0; }
 template <int C>
 struct StUnit {
   using G = StGeom<C>;
@@ -485,7 +493,7 @@ __device__ __forceinline__ void q23k_unit(const uint8_t* __restrict__ bl, int kg
 // 1152 leaves q.  MFMA (ib, q): weights 4 q .. 4 q + 3 of block ib; activations = A pair ib, block q.
 template <int R, int AS>
 __device__ __forceinline__ void q80_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
-                                         float* acc) {
+                                         float* acc, int nvalid) {
   constexpr int RG = (R + 3) / 4;
   typedef _Float16 f16x2v __attribute__((ext_vector_type(2)));
   const uint8_t* p8 = bl + 136 * kg;
@@ -503,7 +511,8 @@ __device__ __forceinline__ void q80_unit(const uint8_t* __restrict__ bl, int kg,
     // byte offset of block ib inside the 136: 34 ib -> dword 8.5 ib
     constexpr int d0 = (34 * ib) / 4;            // dword holding d
     constexpr bool even = (ib & 1) == 0;         // d in the low half of dword d0, quants straddle dwords
-    const float dl = kq::h2f((uint16_t)(even ? (w[d0] & 0xffffu) : (w[d0] >> 16))) * xscale;
+    // blocks past the end of K (the last unit of a row whose K ends inside it): scale 0 on sums of zero activations
+    const float dl = 4 * kg + ib < nvalid ? kq::h2f((uint16_t)(even ? (w[d0] & 0xffffu) : (w[d0] >> 16))) * xscale : 0.f;
     f32x4 p[RG];
 #pragma unroll
     for (int g = 0; g < RG; g++) p[g] = f32x4{0, 0, 0, 0};
@@ -596,7 +605,7 @@ __device__ __forceinline__ float ue4m3_half_fast(uint32_t x) {
 }
 template <int C, int R, int AS>
 __device__ __forceinline__ void nib32_unit(const uint8_t* __restrict__ bl, int kg, float xscale, const u32x2* areg,
-                                           const uint8_t* __restrict__ tbl, float* acc) {
+                                           const uint8_t* __restrict__ tbl, float* acc, int nvalid) {
   constexpr int RG = (R + 3) / 4;
   constexpr bool NV = C == KQ_NVFP4;            // 36-byte blocks of 64: scale bytes 0 .. 3, 8 quant bytes per 16 weights
   constexpr int BB = C == KQ_MXFP4 ? 17 : 18;   // block bytes
@@ -673,6 +682,7 @@ __device__ __forceinline__ void nib32_unit(const uint8_t* __restrict__ bl, int k
       dl = kq::e8m0_half((w[so / 4] >> (8 * (so % 4))) & 0xffu) * xscale;
     else
       dl = kq::h2f((uint16_t)((w[so / 4] >> (8 * (so % 4))) & 0xffffu)) * xscale;
+    dl = 4 * kg + ib < nvalid ? dl : 0.f;  // blocks past the end of K: scale 0 on sums of zero activations
     SFor<R>::run([&](auto rr) {
       constexpr int r = decltype(rr)::value;
       acc[r] = fmaf(dl, p[r / 4][r % 4], acc[r]);
@@ -919,8 +929,13 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, kg = lane >> 5;
-  const int M = a.M, N = a.N, K = a.K, nsb = K >> 8, rpt = a.rpt;
-  const uint32_t row_bytes = (uint32_t)nsb * G::BPB;
+  constexpr bool TAIL = st_tail_codec<C>();
+  // units per row; a tail-capable codec's last one may hold fewer than eight blocks
+  const int M = a.M, N = a.N, K = a.K, nsb = TAIL ? (K + 255) >> 8 : K >> 8, rpt = a.rpt;
+  const uint32_t row_bytes = TAIL ? (uint32_t)(K >> 5) * (G::BPB / 8) : (uint32_t)nsb * G::BPB;
+  const int tail_sb = TAIL && (K & 255) ? K >> 8 : -1;             // the unit K ends in
+  const int tail_blocks = (K & 255) >> 5;                           // its blocks
+  const uint32_t tail_bytes = (uint32_t)tail_blocks * (G::BPB / 8);  // and their bytes
   // gathered: this workgroup's entry and its tile inside the entry's matrix (the tile loop below runs once)
   const int g_entry = GM ? __builtin_amdgcn_readfirstlane((int)blockIdx.x / a.tiles_per_entry) : 0;
   const int g_tile = GM ? (int)blockIdx.x - g_entry * a.tiles_per_entry : 0;
@@ -986,7 +1001,9 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
     int sb = wave + ST_WAVES * uu;
     sb = sb < sbn ? sb : (wave < sbn ? wave : 0);  // spare units re-read a valid superblock
     const int mm = m < M ? m : M - 1;
-    xreg[T] = gload16(x16 + (size_t)mm * K + (size_t)(sb_begin + sb) * 256 + 8 * grp);
+    int k0 = (sb_begin + sb) * 256 + 8 * grp;
+    if constexpr (TAIL) k0 = k0 < K ? k0 : 0;  // past the end of K: any valid address, zeroed once it has landed
+    xreg[T] = gload16(x16 + (size_t)mm * K + k0);
   });
   __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled ahead of these loads
 
@@ -1016,9 +1033,25 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
     const uint8_t* base = ((GM == 2 && (iu & 1)) ? wmat2 : wmat) + (size_t)row0 * row_bytes +
                           (size_t)(sb_begin + wave + ST_WAVES * (iu / UPS)) * G::BPB;
     const uint32_t l0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(wb_lds + islot * U::SLOT));
-    SFor<U::FULL>::run([&](auto t) { constexpr int T = decltype(t)::value; dma16(base, goff[T], l0 + T * 1024); });
-    if constexpr (U::HALF) {
-      if (lane < 32) dma16(base, goff[U::FULL], l0 + U::FULL * 1024);
+    bool tail_unit = false;
+    if constexpr (TAIL) tail_unit = sb_begin + wave + ST_WAVES * (iu / UPS) == tail_sb;
+    if (tail_unit) {
+      SFor<U::FULL + 1>::run([&](auto t) {
+        constexpr int T = decltype(t)::value;
+        if constexpr (T < U::FULL || U::HALF) {
+          const int i = lane + 64 * T;
+          const uint32_t po = st_piece_off<C>(i - (i / G::PP) * G::PP);
+          // whole piece inside the row: as usual; the piece the row ends in: the row's last 16 bytes; past the end:
+          // the unit's first 16 bytes
+          const uint32_t off = po + 16 <= tail_bytes ? goff[T] : goff[T] - po + (po < tail_bytes ? tail_bytes - 16 : 0u);
+          if (T < U::FULL || lane < 32) dma16(base, off, l0 + T * 1024);
+        }
+      });
+    } else {
+      SFor<U::FULL>::run([&](auto t) { constexpr int T = decltype(t)::value; dma16(base, goff[T], l0 + T * 1024); });
+      if constexpr (U::HALF) {
+        if (lane < 32) dma16(base, goff[U::FULL], l0 + U::FULL * 1024);
+      }
     }
     if constexpr (G::SIDE_D) {
       int r = row0 + (lane < rpt ? lane : rpt - 1);
@@ -1045,6 +1078,17 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
   // wait for the activations alone: the first unit stays in flight
   if (inflight) vmwait<U::UPI>(); else vmwait<0>();
   SFor<MB * XL>::run([&](auto t) { tie_v(xreg[decltype(t)::value]); });
+  if constexpr (TAIL) {
+    if (tail_sb >= 0) {  // the activations a short last unit has no weights for
+      SFor<MB * XL>::run([&](auto t) {
+        constexpr int T = decltype(t)::value;
+        constexpr int s = T % XL;
+        const int gi = lane + 64 * s, uu = gi >> 5, grp = gi & 31;
+        const int sb = wave + ST_WAVES * uu;
+        if ((sb_begin + sb) * 256 + 8 * grp >= K && sb < sbn) xreg[T] = u32x4{0, 0, 0, 0};
+      });
+    }
+  }
   tie_v(greg);
   if constexpr (IQ2_COP > 1) SFor<8>::run([&](auto ii) { tie_v2(gq[decltype(ii)::value]); });
 
@@ -1318,17 +1362,43 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
         const uint8_t* bl = slot + crow * G::LBPB;
         constexpr int us = u / UPS;  // the wave's superblock this unit belongs to
         float* acc = (GM == 2 && (u & 1)) ? acc_b : acc_a;
+        const int nvalid = sb_begin + wave + ST_WAVES * us == tail_sb ? tail_blocks : 8;
+        (void)nvalid;
+        if constexpr (TAIL) {
+          if (nvalid != 8) {
+            // the piece the row ends in arrived as the row's last 16 bytes: move them down by the 16 ps + 16 - T bytes
+            // they sit too high (lane n < 32 does LDS row n of the slot, every row once)
+            const uint32_t ps = tail_bytes >> 4, sh = 16 * ps + 16 - tail_bytes;  // sh = 1 .. 15
+            if (lane < 32) {
+              uint8_t* pr = wb + cslot * U::SLOT + lane * G::LBPB + 16 * ps;
+              const u32x4 v = *reinterpret_cast<const u32x4*>(pr);
+              uint32_t e0 = v[0], e1 = v[1], e2 = v[2], e3 = v[3];
+              const uint32_t dq = sh >> 2;  // whole dwords (wave-uniform)
+              if (dq == 1) { e0 = e1; e1 = e2; e2 = e3; e3 = 0; }
+              else if (dq == 2) { e0 = e2; e1 = e3; e2 = 0; e3 = 0; }
+              else if (dq == 3) { e0 = e3; e1 = 0; e2 = 0; e3 = 0; }
+              const uint32_t db = sh & 3;   // then bytes
+              u32x4 o;
+              o[0] = __builtin_amdgcn_alignbyte(e1, e0, db);
+              o[1] = __builtin_amdgcn_alignbyte(e2, e1, db);
+              o[2] = __builtin_amdgcn_alignbyte(e3, e2, db);
+              o[3] = __builtin_amdgcn_alignbyte(0u, e3, db);
+              *reinterpret_cast<u32x4*>(pr) = o;
+            }
+            wave_lds_fence();
+          }
+        }
         if constexpr (C == KQ_Q6_K) {
           const float dx = kq::h2f((uint16_t)*reinterpret_cast<const uint32_t*>(slot + ST_ROWS * G::LBPB + 4 * crow)) * xscale;
           q6k_unit<R, AS>(bl, dx, kg, areg + us * NAP, xsum + us * 16, ST_XU * 16, acc);
         } else if constexpr (C == KQ_Q2_K || C == KQ_Q3_K) {
           q23k_unit<C, R, AS>(bl, kg, xscale, areg + us * NAP, xsum + us * 16, ST_XU * 16, acc);
         } else if constexpr (C == KQ_Q8_0) {
-          q80_unit<R, AS>(bl, kg, xscale, areg + us * NAP, acc);
+          q80_unit<R, AS>(bl, kg, xscale, areg + us * NAP, acc, nvalid);
         } else if constexpr (C == KQ_IQ4_XS) {
           iq4xs_unit<R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc);
         } else if constexpr (C == KQ_IQ4_NL || C == KQ_Q4_0 || C == KQ_MXFP4 || C == KQ_NVFP4) {
-          nib32_unit<C, R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc);
+          nib32_unit<C, R, AS>(bl, kg, xscale, areg + us * NAP, tbl + 4 * (lane & 31), acc, nvalid);
         } else if constexpr (C == KQ_IQ2_XXS) {
           constexpr int COP = st_iq2_copies<C, MB, NW, GM>();
           iq2xxs_unit<R, AS, COP>(bl, kg, xscale, areg + us * NAP, COP > 1 ? tbl + 16 * (lane & 15) : tbl, acc);
@@ -1383,6 +1453,12 @@ __global__ __launch_bounds__(64 * NW, WGS) void stream_gemv_kernel(StArgs a) {
     parity ^= 1;
   }
 }
+
+// K the kernel takes: whole 256-weight units, or, for the codecs of 32-weight blocks copied as they lie, a last unit
+// of one to seven whole blocks behind at least one whole unit.
+bool st_tail_ok(int codec) { return codec == KQ_MXFP4 || codec == KQ_Q4_0 || codec == KQ_IQ4_NL || codec == KQ_Q8_0; }
+bool st_k_ok(int K, int codec) { return K >= 256 && ((K & 255) == 0 || (st_tail_ok(codec) && (K & 31) == 0)); }
+int st_k_units(int K) { return (K + 255) >> 8; }
 
 template <int C, int MB, int D, int ST_XU, int ST_WAVES, int GM = 0>
 constexpr size_t st_lds_bytes() {
@@ -1551,7 +1627,7 @@ int st_launch_gather(StArgs a, int entries, hipStream_t s) {
 
 template <int C, int DT>
 int st_launch_gather_nw(const StArgs& a, int entries, bool glu, hipStream_t s) {
-  const int nsb = a.K >> 8;
+  const int nsb = st_k_units(a.K);
   // gate / up pair: two units per superblock; beyond four superblocks eight waves keep a wave at two to four units
   // (a codec whose eight-wave workgroup does not fit the LDS stays on four waves as far as their units reach)
   if (glu) {
@@ -1576,8 +1652,8 @@ bool st_codec_ok(int codec) {
 // The dense and the gathered launchers can be compiled into separate objects (KQ_STREAM_PART = 1 dense, 2 gathered).
 #if !defined(KQ_STREAM_PART) || KQ_STREAM_PART == 1
 bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const void* w) {
-  if (!st_codec_ok(codec) || M < 1 || M > 8 || N < 1 || K < 256 || (K & 255)) return false;
-  if ((int64_t)N * (K >> 8) * 272 >= (int64_t)1 << 40) return false;
+  if (!st_codec_ok(codec) || M < 1 || M > 8 || N < 1 || !st_k_ok(K, codec)) return false;
+  if ((int64_t)N * st_k_units(K) * 272 >= (int64_t)1 << 40) return false;
   // q4_k / q5_k pieces are fetched 16-byte aligned; iq4_xs blocks are 8-byte multiples, q2_k blocks 4-byte ones, the
   // others 2-byte ones
   const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : codec == KQ_MXFP4 ? 0 : 1;
@@ -1586,16 +1662,21 @@ bool kq_stream_supported(int M, int N, int K, int codec, const void* x, const vo
 }
 
 size_t kq_stream_workspace_bytes(int M, int N, int K, int codec) {
-  if (!st_codec_ok(codec) || M < 1 || M > 8 || (K & 255) || K < 256) return 0;
-  const StSplit p = st_split_plan(M, N, K, codec, st_num_cus());
+  if (!st_codec_ok(codec) || M < 1 || M > 8 || !st_k_ok(K, codec)) return 0;
+  const StSplit p = st_split_plan(M, N, 256 * st_k_units(K), codec, st_num_cus());
   return p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0;
 }
 
 int kq_launch_qmm_stream(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                          size_t ws_bytes, hipStream_t s, const void* bias) {
   if (!kq_stream_supported(M, N, K, codec, x, w)) return KQ_ERR_UNSUPPORTED;
-  const StSplit p = st_split_plan(M, N, K, codec, st_num_cus());
+  const StSplit p = st_split_plan(M, N, 256 * st_k_units(K), codec, st_num_cus());
   if (bias && p.ksplit > 1) return KQ_ERR_UNSUPPORTED;  // the bias joins the sum in the unsplit epilogue only
+  // three or more rows of a table-decoded 4-bit codec whose K range has to be cut (few row tiles): the code-level
+  // kernel needs no reduction launch and is ahead (mxfp4 3072 -> 2880: 4 rows 7.8 us against 10.4 here, 8 rows 9.1
+  // against 11.3; 2880 -> 5760: 4 rows 8.5 against 12.0; q4_0 4128 -> 11008: 15.9 against 17.4)
+  if (p.ksplit > 1 && M >= 3 && !bias && (codec == KQ_MXFP4 || codec == KQ_Q4_0 || codec == KQ_IQ4_NL))
+    return KQ_ERR_UNSUPPORTED;
   if (p.ksplit > 1 && (!ws || ws_bytes < (size_t)p.ksplit * M * N * sizeof(float) || (reinterpret_cast<uintptr_t>(ws) & 3)))
     return KQ_ERR_UNSUPPORTED;  // the caller falls through to the kernels that can run unsplit
   StArgs a{};
@@ -1657,9 +1738,13 @@ int kq_gather_stream_max_entries() { return KQ_GATHER_STREAM_MAX_ENTRIES; }
 bool kq_gather_stream_takes(const void* x, const void* w, const void* w2, int entries, int N, int K, bool strided_x,
                             int64_t x_row_stride, int64_t w_expert_stride, bool second_bias_without_glu, int codec) {
   if (!st_codec_ok(codec)) return false;
-  if (entries < 1 || entries > KQ_GATHER_STREAM_MAX_ENTRIES || N < 1 || K < 256 || (K & 255)) return false;
+  if (entries < 1 || entries > KQ_GATHER_STREAM_MAX_ENTRIES || N < 1 || !st_k_ok(K, codec)) return false;
   const bool glu = w2 != nullptr;
-  if ((K >> 8) > (glu ? 16 : 32) || second_bias_without_glu) return false;
+  if (st_k_units(K) > (glu ? 16 : 32) || second_bias_without_glu) return false;
+  // the fused gate / up form on stacks whose K ends inside a unit stays on the code-level kernels, which are ahead
+  // there (32 experts of 2880 x 2880 in mxfp4: 4 pairs 16.4 us against 18.3 here, whose 360 eight-wave workgroups
+  // take two rounds of one per CU; 8 pairs 24.6 on the block-scaled kernel against 26.7)
+  if (glu && (K & 255)) return false;
   if ((int64_t)entries * ((N + ST_ROWS - 1) / ST_ROWS) > 65535 * 16) return false;
   const uintptr_t wmask = codec == KQ_Q4_K || codec == KQ_Q5_K ? 15 : codec == KQ_IQ4_XS ? 7 : codec == KQ_Q2_K ? 3 : codec == KQ_MXFP4 ? 0 : 1;
   if ((reinterpret_cast<uintptr_t>(w) & wmask) || (reinterpret_cast<uintptr_t>(w2) & wmask) ||
@@ -1689,7 +1774,7 @@ int kq_launch_gather_stream(const void* x, const uint8_t* w, const uint8_t* w2, 
   a.N = N;
   a.K = K;
   a.ksplit = 1;
-  a.sb_per_split = K >> 8;
+  a.sb_per_split = st_k_units(K);
   a.x_div = x_div < 1 ? 1 : x_div;
   a.E = E;
   a.act = act;

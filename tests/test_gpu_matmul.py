@@ -142,6 +142,43 @@ def test_qmm_streamed_kernel_shapes(kq, codec, dtype):
         assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype, M, N, K)
 
 
+@pytest.mark.parametrize("codec", ["mxfp4", "q4_0", "iq4_nl", "q8_0"])
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+def test_qmm_streamed_kernel_k_ends_inside_a_unit(kq, codec, dtype):
+    """The codecs of 32-weight blocks run on the streamed kernel for any K that is a multiple of 32 from 256 up: the
+    last 256-weight unit of a row then holds one to seven blocks (K = 2880: 11 units and 2 blocks).  One to eight
+    rows, ragged row tiles, a K range cut over grid z (33 units), the whole 2880 x 2880 matrix."""
+    for M, N, K in ((1, 100, 288), (3, 64, 2880), (8, 37, 480), (2, 200, 8192 + 96), (1, 2880, 2880), (5, 40, 4096 + 32),
+                    (4, 33, 256 + 224)):
+        wire = _wire(codec, N, K, seed=71)
+        xb, xt = make_x((M, K), dtype, seed=72)
+        got = kq.quantized_matmul(xt, wire_to_dev(wire), None, codec)
+        want = O.qmm(xb, wire, codec, True, dtype)
+        assert tuple(got.shape) == (M, N)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (codec, dtype, M, N, K)
+
+
+@pytest.mark.parametrize("codec", ["mxfp4", "q4_0", "q8_0"])
+def test_qmm_k_tail_uses_nothing_past_the_weights(kq, codec):
+    """A short last unit is fetched in 16-byte pieces none of which reaches past its row: a matrix that ends exactly
+    on a page boundary (as 32 x 2880 x 2880 mxfp4 stacks do) or a few bytes before one, with 0xff bytes (NaN scales)
+    around it, gives the oracle's result."""
+    N, K, M = 70, 2880, 2
+    wire = _wire(codec, N, K, seed=73)
+    nbytes = wire.size
+    xb, xt = make_x((M, K), "bfloat16", seed=74)
+    want = O.qmm(xb, wire, codec, True, "bfloat16")
+    buf = torch.full((nbytes + 2 * 4096,), 0xff, dtype=torch.uint8, device="cuda:0")
+    for end_in_page in (2048, 4090, 0):
+        off = (end_in_page - (buf.data_ptr() + nbytes)) % 4096
+        view = buf[off:off + nbytes].view(N, -1)
+        view.copy_(wire_to_dev(wire))
+        assert (view.data_ptr() + nbytes) % 4096 == end_in_page
+        got = kq.quantized_matmul(xt, view, None, codec)
+        assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL, (codec, end_in_page)
+        buf.fill_(0xff)
+
+
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
 @pytest.mark.parametrize("N,K", [(264, 512), (4096, 4096), (1000, 8192), (33, 256), (97, 320), (20000, 1024)])
 def test_qmv_bias_fused_decode(kq, N, K, dtype):

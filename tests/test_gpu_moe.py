@@ -230,6 +230,35 @@ def test_moe_low_bit_routes_either_side_of_the_entry_threshold(kq, codec, T):
     assert rel_l2(dev_to_bits(got), want, "float16") <= TOL, (codec, T)
 
 
+@pytest.mark.parametrize("codec", ["mxfp4", "q4_0", "q8_0", "iq4_nl"])
+@pytest.mark.parametrize("E,N,K,T,R", [(6, 136, 288, 1, 4), (5, 72, 2880, 3, 2), (130, 40, 480, 4, 4)])
+def test_moe_decode_k_ends_inside_a_unit(kq, codec, E, N, K, T, R):
+    """MoE decode (a few pairs, entry by entry on the streamed kernel) on stacks whose K is not a multiple of 256:
+    fused gate / up and the down form, both activation dtypes; mxfp4 also with biases and swiglu_clamp."""
+    gate, up = _stack(codec, E, N, K, seed=151), _stack(codec, E, N, K, seed=152)
+    rng = np.random.default_rng(153)
+    idx = np.stack([rng.permutation(E)[:R] for _ in range(T)])
+    for dtype in ("bfloat16", "float16"):
+        xb, xt = make_x((T, K), dtype, seed=154, scale=0.05)
+        got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act="silu")
+        assert rel_l2(dev_to_bits(got), _glu_truth(codec, xb, gate, up, idx, "silu", dtype=dtype), dtype) <= TOL, (codec, dtype)
+        hb, ht = make_x((T, R, K), dtype, seed=155, scale=0.05)
+        got = kq.gather_qmv_kq(ht, wire_to_dev(up), codec, _idx_dev(idx))
+        assert rel_l2(dev_to_bits(got), O.gather_qmv(hb, up, codec, idx, None, dtype), dtype) <= TOL, (codec, dtype)
+    if codec == "mxfp4":
+        gb = (rng.standard_normal((E, N)) * 0.05).astype(np.float32)
+        ub = (rng.standard_normal((E, N)) * 0.05).astype(np.float32)
+        xb, xt = make_x((T, K), "bfloat16", seed=156, scale=0.05)
+        got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act="swiglu_clamp",
+                                   limit=7.0, alpha=1.702, gate_bias=torch.from_numpy(gb).cuda(),
+                                   up_bias=torch.from_numpy(ub).cuda())
+        want = _glu_truth(codec, xb, gate, up, idx, "swiglu_clamp", 7.0, 1.702, gb, ub)
+        assert rel_l2(dev_to_bits(got), want, "bfloat16") <= TOL
+        hb, ht = make_x((T, R, K), "bfloat16", seed=157, scale=0.05)
+        got = kq.gather_qmv_kq(ht, wire_to_dev(up), codec, _idx_dev(idx), bias=torch.from_numpy(gb).cuda())
+        assert rel_l2(dev_to_bits(got), O.gather_qmv(hb, up, codec, idx, gb, "bfloat16"), "bfloat16") <= TOL
+
+
 @pytest.mark.parametrize("T", [4, 16])
 def test_moe_routes_on_32_experts_of_2880_square(kq, T):
     """A stack unlike the one the entry-by-entry limits were measured on (32 experts of 2880 x 2880 in mxfp4, top-4,
