@@ -41,7 +41,7 @@ LLC_BYTES = 256 << 20
 # `bench.py --probe` (KiB per dispatch of the GEMV kernel), each counter scaled by what it reads for the probe's
 # plain 32256 KiB device copy (32256 / the copy's reading).  Algorithmic bytes are 33,030,144 (weights) + 28,672
 # (output).
-HEADLINE_FETCH_KIB, HEADLINE_FETCH_SCALE = 16251.8, 1.9984
+HEADLINE_FETCH_KIB, HEADLINE_FETCH_SCALE = 16254.3, 1.9984
 HEADLINE_WRITE_KIB, HEADLINE_WRITE_SCALE = 28.0, 1.0
 HEADLINE_TRAFFIC_BYTES = int(round((HEADLINE_FETCH_KIB * HEADLINE_FETCH_SCALE
                                     + HEADLINE_WRITE_KIB * HEADLINE_WRITE_SCALE) * 1024, -3))
@@ -365,7 +365,7 @@ def main():
                     help="prefill section: force a tile shape of the prefill GEMM (kq_set_gemm_tile_rows)")
     ap.add_argument("--only", default=None, metavar="SECTIONS",
                     help="comma-separated extra sections to run (sweep, prefill, moe, moe_mxfp4, moe_decode_lowbit, "
-                         "lowbit, dequantize, mid_m, no_transpose); default all")
+                         "lowbit, large_gemv, dequantize, mid_m, no_transpose); default all")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for `rocprofv3 --pmc`: one device copy of the headline matrix (known bytes) "
                          "followed by 20 cold launches of the headline GEMV, nothing else")
@@ -655,6 +655,22 @@ def main():
                                "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
                 del cps, wq
             out["lowbit"] = lowbit
+
+        # ---------------- long matrices (128256 x 4096, the lm_head shape), M = 1: the launch overheads of the 20 - 70 MB
+        # shapes above amortised, to set beside `read_ceiling` (random structurally valid wire)
+        if want("large_gemv"):
+            large = []
+            n, k = 128256, 4096
+            for c in ("q8_0", "q4_k", "q5_k", "iq4_xs", "q6_k", "q2_k", "q3_k"):
+                wb = n * kq.bytes_per_row(c, k)
+                ncopies = max(2, (2 * LLC_BYTES + wb - 1) // wb + 1)
+                cps = [synth_wire_torch(c, n, k, 31 + i, dev) for i in range(ncopies)]
+                t, _ = time_calls(torch, [abi.qmm(x.new_ones((1, k)), w, c, n, k) for w in cps], 60, 10)
+                large.append({"codec": c, "N": n, "K": k, "M": 1, "us": round(t * 1e3, 2),
+                              "cold_gbs": round(wb / (t * 1e-3) / 1e9, 1),
+                              "pct_hbm_peak": round(100 * wb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)})
+                del cps
+            out["large_gemv"] = large
 
         # ---------------- dequantize to f16 (random structurally valid wire): bytes = wire in + 2 N K out
         if want("dequantize"):
