@@ -109,8 +109,10 @@ int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void
 /* Tuning hook without a counterpart in the reference: workgroup tile of the prefill GEMM.  64 = 64
  * activation rows x 128 weight rows, 128 = 128 x 128, 256 = 64 x 256 on eight waves with two LDS stages
  * (q4_k only; other codecs fall back to automatic), 512 = 128 x 256 on eight waves with 128-row wave tiles and
- * direct-to-LDS loads (q2_k / q3_k / q4_k / q5_k / iq4_xs; 513 = the same kernel as 128 x 128 on four waves);
- * anything else restores the automatic choice.
+ * direct-to-LDS loads (q2_k / q3_k / q4_k / q5_k / iq4_xs; 513 = the same kernel as 128 x 128 on four waves),
+ * 1024 = 256 x 256 on eight waves with 256-row wave tiles on one accumulator set (q4_k / q5_k) for every column
+ * tile; anything else restores the automatic choice (q4_k / q5_k with 256 rows or more: the 256 x 256 kernel on the
+ * column tiles that fill whole rounds of one workgroup per CU, the 128 x 256 kernel on the rest).
  * Process-wide, not thread-safe. */
 void kq_set_gemm_tile_rows(int rows);
 /* Tuning hook without a counterpart in the reference: which skinny-M kernel dense calls use.
@@ -140,11 +142,13 @@ int kq_gather_qmm(const void* x_dev, const void* w_dev, const uint32_t* lhs_idx_
                   int codec, int dtype, void* workspace_dev, size_t workspace_bytes, void* stream);
 
 /* Device workspace (bytes, 256-byte aligned, may be 0) of the two MoE ops below: `glu` != 0 for
- * kq_moe_glu_gather, 0 for kq_gather_qmv.  The batched path (more than 16 (token, expert) pairs; more than 48
- * for q4_k / q5_k / q6_k and the legacy / fp4 / other IQ stacks, 64 for iq4_xs / iq3_s / iq2_xxs / q8_0 and for
- * iq4_nl / q4_0 / mxfp4 with K a multiple of 256,
- * 256 for q2_k / q3_k / nvfp4; for stacks of fewer than 128 experts these limits shrink in proportion, E / 128)
- * sorts the pairs by expert and keeps f16 activations there.  The reference allocates its own
+ * kq_moe_glu_gather, 0 for kq_gather_qmv.  The batched path sorts the pairs by expert and keeps converted
+ * activations there.  It takes calls of more than 16 (token, expert) pairs unless the per-entry kernels are ahead,
+ * which a codec family's measured figure decides (48 pairs for q4_k / q5_k / q6_k and the legacy / fp4 / other IQ
+ * stacks, 64 for iq4_xs / iq3_s / iq2_xxs / q8_0 / iq4_nl / q4_0 / mxfp4 on the streamed kernel, 256 for q2_k / q3_k /
+ * nvfp4), carried to the call's stack as three bounds: that many pairs, that many pairs per 128 experts, and no more
+ * bytes read again than on the stack the figure was measured on (128 experts of 2048 x 768); mxfp4 stacks go to the
+ * block-scaled kernel from 8 pairs where K is no multiple of 256.  The reference allocates its own
  * temporaries inside eval_gpu (src/kquant_moe_glu.cpp:277-382); here the caller owns them. */
 size_t kq_moe_workspace_size(int T, int R, int E, int N, int K, int glu, int codec, int dtype);
 
