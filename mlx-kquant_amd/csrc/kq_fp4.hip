@@ -40,6 +40,13 @@ typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 
 using kqsort::Segment;
 
+// A pointer into device memory as such: the loads through it are global loads, not flat ones (a flat load also
+// counts in the LDS counter, so a wait for an LDS result would wait for the prefetched step as well).
+template <class T>
+__device__ __forceinline__ const __attribute__((address_space(1))) T* in_global(const T* p) {
+  return (const __attribute__((address_space(1))) T*)(uintptr_t)p;
+}
+
 constexpr int F4_STAGES = 2;     // register stages in rotation: a step's loads are queued one step ahead (deeper: no gain)
 constexpr int F4_THREADS = 256;  // four waves
 
@@ -197,7 +204,15 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
   if (16 * mt >= sg.count) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 15, kb = lane >> 4;
+  const int r = lane & 15, kb = lane >> 4;  // this lane's place in the operands: row / column r, block kb of the step
+  // Its place in the loads.  With one m-tile the loads go in row order: four neighbouring lanes take the four blocks
+  // of one row (68 contiguous bytes of weights, 64 of an activation term), so sixteen lanes touch 4 rows instead of
+  // 16, and the loaded registers change lanes once (operand lane 16 p + 4 x + y reads what lane 16 x + 4 y + p
+  // loaded).  With two m-tiles on the same weight registers the exchanged copies do not fit the register file and
+  // the loads stay in operand order.
+  constexpr bool COAL = MT == 1;
+  const int rl = COAL ? lane >> 2 : r, kbl = COAL ? lane & 3 : kb;
+  const int from_lane = 4 * (16 * ((lane >> 2) & 3) + 4 * (lane & 3) + (lane >> 4));
   const int N = a.N, nsteps = a.nsteps, nblk = a.K >> 5;
   const uint32_t row_bytes = (uint32_t)nblk * 17u;
   const int n0 = blockIdx.x * COLS;
@@ -208,7 +223,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
   const uint8_t* wrow[J];
 #pragma unroll
   for (int j = 0; j < J; j++) {
-    int c = n0 + 16 * (GLU ? (j % JH) : j) + r;
+    int c = n0 + 16 * (GLU ? (j % JH) : j) + rl;
     c = c < N ? c : N - 1;
     const uint8_t* base = (GLU && j >= JH) ? a.w2 : a.w;
     wrow[j] = base + (int64_t)sg.expert * a.w_expert_stride + (size_t)c * row_bytes;
@@ -218,10 +233,10 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
   const uint32_t* srow[MT];
 #pragma unroll
   for (int m = 0; m < MT; m++) {
-    const int mrow = 16 * m + r < rows_here ? 16 * m + r : rows_here - 1;
-    const int xrow = a.order[sg.start + 16 * mt + mrow] / a.x_div;
-    arow[m] = a.xa + ((size_t)xrow * nsteps * NT) * 128 + kb * 32;
-    srow[m] = a.xs + (size_t)xrow * nsteps * 4 + kb;
+    const int mrow = 16 * m + rl < rows_here ? 16 * m + rl : rows_here - 1;
+    const int xrow = in_global(a.order)[sg.start + 16 * mt + mrow] / a.x_div;
+    arow[m] = a.xa + ((size_t)xrow * nsteps * NT) * 128 + kbl * 32;
+    srow[m] = a.xs + (size_t)xrow * nsteps * 4 + kbl;
   }
 
   struct Stage {
@@ -231,27 +246,26 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
     int sa[MT];
   };
   auto fetch = [&](Stage& st, int s) {
-    int blk = 4 * s + kb;
+    int blk = 4 * s + kbl;
     const bool live = blk < nblk;  // past K: any block of the row with a neutral scale (the activations are zeros)
     blk = live ? blk : nblk - 1;
     const uint32_t off = (uint32_t)blk * 17u;
 #pragma unroll
     for (int j = 0; j < J; j++) {
       // the 17 bytes of the block (scale, 16 code bytes) sit at any byte offset: five aligned dwords around them,
-      // the codes brought to dword boundaries with byte shifts (a global load wider than a byte wants dword alignment)
+      // the codes brought to dword boundaries with byte shifts
       const uintptr_t ad = reinterpret_cast<uintptr_t>(wrow[j] + off);
       const uint32_t sh = (uint32_t)ad & 3u;
       const uint32_t* q = reinterpret_cast<const uint32_t*>(ad - sh);
-      const u32x4 d = *reinterpret_cast<const u32x4_a4*>(q);
-      uint32_t d4;
-      if (reinterpret_cast<const uint8_t*>(q + 5) <= ((GLU && j >= JH) ? a.w2_end : a.w_end)) {
-        d4 = q[4];
-      } else {  // the last block of the stack: the dword would reach past its end
-        d4 = 0;
-        const uint8_t* e = (GLU && j >= JH) ? a.w2_end : a.w_end;
-        for (const uint8_t* b = reinterpret_cast<const uint8_t*>(q + 4); b < e; b++)
-          d4 |= (uint32_t)*b << (8 * (int)(b - reinterpret_cast<const uint8_t*>(q + 4)));
-      }
+      const u32x4 d = *(const __attribute__((address_space(1))) u32x4_a4*)(uintptr_t)q;  // dword-aligned, no more
+      // the fifth dword; for the last block of the stack it would reach past the end: fetched that many bytes earlier
+      // and shifted back (the bytes past the end are not part of the block)
+      const uint8_t* wend = (GLU && j >= JH) ? a.w2_end : a.w_end;
+      const int64_t over = reinterpret_cast<const uint8_t*>(q + 5) - wend;
+      const uint32_t back = over > 0 ? (uint32_t)over : 0u;
+      typedef uint32_t u32_a1 __attribute__((aligned(1)));
+      const uint32_t d4 =
+          *(const __attribute__((address_space(1))) u32_a1*)(reinterpret_cast<uintptr_t>(q + 4) - back) >> (8 * back);
       const int sc = (int)((d[0] >> (8 * sh)) & 0xff);
       st.sb[j] = live ? sc : 127;
       // codes start at byte sh + 1 of the window: a shift by 1 .. 3 bytes, or (sh = 3) the next dword as it is
@@ -266,11 +280,11 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
     for (int m = 0; m < MT; m++) {
 #pragma unroll
       for (int t = 0; t < NT; t++) {
-        const u32x4 lo = *reinterpret_cast<const u32x4*>(arow[m] + ((size_t)s * NT + t) * 128);
-        const u32x4 hi = *reinterpret_cast<const u32x4*>(arow[m] + ((size_t)s * NT + t) * 128 + 16);
+        const u32x4 lo = *in_global(reinterpret_cast<const u32x4*>(arow[m] + ((size_t)s * NT + t) * 128));
+        const u32x4 hi = *in_global(reinterpret_cast<const u32x4*>(arow[m] + ((size_t)s * NT + t) * 128 + 16));
         st.av[m][t] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
       }
-      st.sa[m] = (int)srow[m][(size_t)s * 4];
+      st.sa[m] = (int)in_global(srow[m])[(size_t)s * 4];
     }
   };
   v4f acc[MT][J];
@@ -278,18 +292,30 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
   for (int m = 0; m < MT; m++)
 #pragma unroll
     for (int j = 0; j < J; j++) acc[m][j] = v4f{0, 0, 0, 0};
+  auto to_operand_lane = [&](int v) { return COAL ? __builtin_amdgcn_ds_bpermute(from_lane, v) : v; };
   auto multiply = [&](const Stage& st) {
+    v8i av[MT][NT];
+    int sav[MT];
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+#pragma unroll
+      for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) av[m][t][i] = to_operand_lane(st.av[m][t][i]);
+      sav[m] = to_operand_lane(st.sa[m]);
+    }
 #pragma unroll
     for (int j = 0; j < J; j++) {
-      const v8i bv = {(int)st.b[j][0], (int)st.b[j][1], (int)st.b[j][2], (int)st.b[j][3], 0, 0, 0, 0};
-      const int sb = in_vgpr(st.sb[j]);
+      const v8i bv = {to_operand_lane((int)st.b[j][0]), to_operand_lane((int)st.b[j][1]), to_operand_lane((int)st.b[j][2]),
+                      to_operand_lane((int)st.b[j][3]), 0, 0, 0, 0};
+      const int sb = in_vgpr(to_operand_lane(st.sb[j]));
 #pragma unroll
       for (int m = 0; m < MT; m++) {
-        const int sa = in_vgpr(st.sa[m]);
-        acc[m][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[m][0], bv, acc[m][j], 0, 4, 0, sa, 0, sb);
-        acc[m][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[m][1], bv, acc[m][j], 0, 4, 1, sa, 0, sb);
+        const int sa = in_vgpr(sav[m]);
+        acc[m][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av[m][0], bv, acc[m][j], 0, 4, 0, sa, 0, sb);
+        acc[m][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av[m][1], bv, acc[m][j], 0, 4, 1, sa, 0, sb);
         if constexpr (NT == 3)
-          acc[m][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st.av[m][2], bv, acc[m][j], 0, 4, 2, sa, 0, sb);
+          acc[m][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av[m][2], bv, acc[m][j], 0, 4, 2, sa, 0, sb);
       }
     }
   };
@@ -335,13 +361,13 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
   };
   auto finish = [&](int m16, int col, const v4f& g, const v4f& u) {
     if (col >= N) return;
-    const float gb = a.bias ? a.bias[(size_t)expert * N + col] : 0.f;
-    const float ub = (GLU && a.bias2) ? a.bias2[(size_t)expert * N + col] : 0.f;
+    const float gb = a.bias ? in_global(a.bias)[(size_t)expert * N + col] : 0.f;
+    const float ub = (GLU && a.bias2) ? in_global(a.bias2)[(size_t)expert * N + col] : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int m = 16 * m16 + 4 * kb + i;
       if (m < rows_here) {
-        const int p = a.order[sg.start + 16 * mt + m];
+        const int p = in_global(a.order)[sg.start + 16 * mt + m];
         float v = g[i] + gb;
         if constexpr (GLU) v = kq::glu_epilogue_fast(a.act, v, u[i] + ub, a.limit, a.alpha);
         kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, p) * N + col, v);
