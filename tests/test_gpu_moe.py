@@ -280,6 +280,35 @@ def test_moe_routes_on_32_experts_of_2880_square(kq, T):
     assert rel_l2(dev_to_bits(got), O.gather_qmv(hb, up, codec, idx, gb, "bfloat16"), "bfloat16") <= TOL, T
 
 
+@pytest.mark.parametrize("T", [16, 40])
+@pytest.mark.parametrize("off", [1, 2, 3])
+def test_moe_mxfp4_stacks_at_any_byte_offset_use_nothing_past_their_end(kq, off, T):
+    """The block-scaled kernel fetches aligned dwords around every 17-byte block.  Stacks that start at an odd byte
+    offset end inside a dword: the result must not depend on the bytes that follow the stack (two fillings), and
+    equals the result on the same stacks at an aligned address bit for bit (16 tokens: one m-tile per segment, 40:
+    two)."""
+    codec, E, N, K, R = "mxfp4", 4, 64, 288, 2
+    gate, up = _stack(codec, E, N, K, seed=141), _stack(codec, E, N, K, seed=142)
+    rng = np.random.default_rng(143)
+    idx = np.stack([rng.permutation(E)[:R] for _ in range(T)])
+    xb, xt = make_x((T, K), "bfloat16", seed=144, scale=0.05)
+    hb, ht = make_x((T, R, K), "bfloat16", seed=145, scale=0.05)
+    want = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx))
+    want_d = kq.gather_qmv_kq(ht, wire_to_dev(up), codec, _idx_dev(idx))
+    assert rel_l2(dev_to_bits(want), _glu_truth(codec, xb, gate, up, idx, "silu"), "bfloat16") <= TOL
+
+    def placed(stack, fill):
+        buf = torch.full((off + stack.size + 64,), fill, dtype=torch.uint8, device="cuda")
+        buf[off:off + stack.size] = wire_to_dev(stack).reshape(-1)
+        return buf[off:off + stack.size].view(stack.shape)
+
+    for fill in (0x00, 0xFF):
+        got = kq.moe_glu_gather_kq(xt, placed(gate, fill), placed(up, fill), codec, _idx_dev(idx))
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (off, T, fill)
+        got = kq.gather_qmv_kq(ht, placed(up, fill), codec, _idx_dev(idx))
+        assert torch.equal(got.view(torch.int16), want_d.view(torch.int16)), (off, T, fill)
+
+
 @pytest.mark.parametrize("N,K,T", [(1536, 2048, 5), (2048, 2560, 5), (1536, 2048, 10)])
 def test_moe_q4k_routes_by_pairs_per_expert_and_bytes_read_again(kq, N, K, T):
     """64 experts in q4_k, top-4.  20 pairs of 1536 x 2048 matrices run entry by entry; the same 20 pairs of
