@@ -386,6 +386,197 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
   }
 }
 
+// ------------------------------------------------------------------ fused gate / up op, one m-tile, waves split the tiles
+// One m-tile (16 pairs) of a segment and 64 output columns per workgroup, as in the kernel above with MT = 1, but the
+// four waves split the column tiles instead of the K steps: wave v owns columns n0 + 16 v .. + 15 (that tile of the
+// gate and of the up matrix) over all of K, so no partial sums meet at the end.  A wave's loads cover four
+// consecutive steps of its rows at a time (272 contiguous bytes per row), the loads of the next four are issued
+// before the present four are multiplied (two register stages; the loop body holds no branch, so the wait before
+// a multiply is exact), and the loaded registers are used untouched until then (anything computed from them at
+// load time would make the wave wait there).  The activation terms of a step are loaded once per workgroup -- wave v
+// takes step 4 q + v of a group of four -- and shared through LDS in operand order, so they need no lane exchange
+// and cost a fifth of the load instructions they cost when every wave fetches the terms of its own step.
+// (The plain op, one tile per wave, measured slower in this form than with the K steps split: 39.7 us in groups of
+// four steps, 45.6 in groups of eight, against 36.6; it stays on the kernel above.)
+template <int DT>
+__global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) {
+  constexpr int NT = f4_terms<DT>();
+  constexpr bool GLU = true;
+  constexpr int TPW = 2;  // tiles per wave: gate and up
+  constexpr int SPG = 4;  // steps per group: a stage is eight blocks per lane
+  constexpr int SPW = 1;  // steps of activation terms a wave loads per group
+  constexpr int A_STEP = NT * 2048 + 256;  // LDS bytes of a step's terms: [term][half][a][m][16] + scales [kb][m]
+  __shared__ __attribute__((aligned(16))) uint8_t abuf[2][SPG][A_STEP];
+  const int nseg = *in_global(a.nseg);
+  if ((int)blockIdx.y >= nseg) return;
+  const Segment sg = a.segs[blockIdx.y];
+  const int mt = blockIdx.z;
+  if (16 * mt >= sg.count) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, kb = lane >> 4;   // place in the operands
+  const int rl = lane >> 2, kbl = lane & 3;  // place in the loads: four neighbouring lanes take the four blocks of a row
+  const int from_lane = 4 * (16 * ((lane >> 2) & 3) + 4 * (lane & 3) + (lane >> 4));
+  const int N = a.N, nsteps = a.nsteps, nblk = a.K >> 5;
+  const uint32_t row_bytes = (uint32_t)nblk * 17u;
+  const int n0 = blockIdx.x * 64;
+  const int rows_here = sg.count - 16 * mt < 16 ? sg.count - 16 * mt : 16;
+  const int ngroups = (nsteps + SPG - 1) / SPG;
+
+  const uint8_t* wrow[TPW];
+#pragma unroll
+  for (int t = 0; t < TPW; t++) {
+    int c = n0 + 16 * wave + rl;
+    c = c < N ? c : N - 1;  // columns past N re-read the last one (not stored)
+    wrow[t] = (t ? a.w2 : a.w) + (int64_t)sg.expert * a.w_expert_stride + (size_t)c * row_bytes;
+  }
+  uint32_t wlow[TPW];  // low address bits of the rows
+  bool last_row[TPW];  // the row is the last of its stack
+#pragma unroll
+  for (int t = 0; t < TPW; t++) {
+    wlow[t] = (uint32_t)reinterpret_cast<uintptr_t>(wrow[t]) & 3u;
+    last_row[t] = wrow[t] + row_bytes == (t ? a.w2_end : a.w_end);
+  }
+  const int mrow = rl < rows_here ? rl : rows_here - 1;  // rows past the segment re-read its last pair (dropped)
+  const int xrow = in_global(a.order)[sg.start + 16 * mt + mrow] / a.x_div;
+  const uint8_t* arow = a.xa + ((size_t)xrow * nsteps * NT) * 128 + kbl * 32;
+  const uint32_t* srow = a.xs + (size_t)xrow * nsteps * 4 + kbl;
+
+  struct Stage {
+    u32x4 d[TPW][SPG];      // the four aligned dwords at and after a block's first byte
+    uint32_t d4[TPW][SPG];  // the fifth
+    u32x4 lo[SPW][NT], hi[SPW][NT];
+    uint32_t sa[SPW];
+  };
+  // the window of block (tile t, step s) of this lane: address of its first dword, the byte shift, and how many
+  // bytes earlier the fifth dword is fetched (the last block of a stack: the dword would reach past the end)
+  auto window = [&](int t, int s, uint32_t& sh, uint32_t& back, bool& live) {
+    int blk = 4 * s + kbl;
+    live = blk < nblk;  // past K: any block of the row with a neutral scale (the activations are zeros)
+    blk = live ? blk : nblk - 1;
+    const uint32_t off = (uint32_t)blk * 17u;
+    sh = (wlow[t] + off) & 3u;
+    back = (last_row[t] && blk == nblk - 1) ? 3u - sh : 0u;
+    return reinterpret_cast<uintptr_t>(wrow[t]) + off - sh;
+  };
+  auto issue = [&](Stage& st, int q) {  // group q: steps SPG q .. + SPG - 1 (past the last: the last once more, unused)
+#pragma unroll
+    for (int t = 0; t < TPW; t++)
+#pragma unroll
+      for (int g = 0; g < SPG; g++) {
+        int s = SPG * q + g;
+        s = s < nsteps ? s : nsteps - 1;
+        uint32_t sh, back;
+        bool live;
+        const uintptr_t qa = window(t, s, sh, back, live);
+        st.d[t][g] = *(const __attribute__((address_space(1))) u32x4_a4*)qa;  // dword-aligned, no more
+        typedef uint32_t u32_a1 __attribute__((aligned(1)));
+        st.d4[t][g] = *(const __attribute__((address_space(1))) u32_a1*)(qa + 16 - back);
+      }
+#pragma unroll
+    for (int i = 0; i < SPW; i++) {
+      int s = SPG * q + 4 * i + wave;
+      s = s < nsteps ? s : nsteps - 1;
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        st.lo[i][t] = *in_global(reinterpret_cast<const u32x4*>(arow + ((size_t)s * NT + t) * 128));
+        st.hi[i][t] = *in_global(reinterpret_cast<const u32x4*>(arow + ((size_t)s * NT + t) * 128 + 16));
+      }
+      st.sa[i] = in_global(srow)[(size_t)s * 4];
+    }
+  };
+  v4f acc[TPW];
+#pragma unroll
+  for (int t = 0; t < TPW; t++) acc[t] = v4f{0, 0, 0, 0};
+  auto consume = [&](const Stage& st, int q) {
+    // this wave's steps of activation terms into LDS: lane (row rl, block kbl) writes where operand lane
+    // (m = rl, a = kbl) will read
+#pragma unroll
+    for (int i = 0; i < SPW; i++) {
+      uint8_t* ab = abuf[q & 1][4 * i + wave];
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        *reinterpret_cast<u32x4*>(ab + (((t * 2 + 0) * 4 + kbl) * 16 + rl) * 16) = st.lo[i][t];
+        *reinterpret_cast<u32x4*>(ab + (((t * 2 + 1) * 4 + kbl) * 16 + rl) * 16) = st.hi[i][t];
+      }
+      *reinterpret_cast<uint32_t*>(ab + NT * 2048 + (kbl * 16 + rl) * 4) = st.sa[i];
+    }
+    __syncthreads();  // two buffers in turn: a buffer is written again two groups later, past the next barrier
+#pragma unroll
+    for (int g = 0; g < SPG; g++) {
+      const int s = SPG * q + g;
+      if (s < nsteps) {  // uniform
+        const uint8_t* ab = abuf[q & 1][g];
+        v8i av[NT];
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+          const u32x4 l = *reinterpret_cast<const u32x4*>(ab + (((t * 2 + 0) * 4 + kb) * 16 + r) * 16);
+          const u32x4 h = *reinterpret_cast<const u32x4*>(ab + (((t * 2 + 1) * 4 + kb) * 16 + r) * 16);
+          av[t] = v8i{(int)l[0], (int)l[1], (int)l[2], (int)l[3], (int)h[0], (int)h[1], (int)h[2], (int)h[3]};
+        }
+        const int sa = in_vgpr(*reinterpret_cast<const int*>(ab + NT * 2048 + (kb * 16 + r) * 4));
+#pragma unroll
+        for (int t = 0; t < TPW; t++) {
+          uint32_t sh, back;
+          bool live;
+          window(t, s, sh, back, live);
+          const u32x4 d = st.d[t][g];
+          const int sc = live ? (int)((d[0] >> (8 * sh)) & 0xff) : 127;
+          // codes start at byte sh + 1 of the window: a shift by 1 .. 3 bytes, or (sh = 3) the next dword as it is
+          const bool whole = sh == 3;
+          const uint32_t s1 = (sh + 1) & 3u;
+          const uint32_t dd[5] = {d[0], d[1], d[2], d[3], st.d4[t][g] >> (8 * back)};
+          v8i bv = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+          for (int i = 0; i < 4; i++)
+            bv[i] = __builtin_amdgcn_ds_bpermute(
+                from_lane, (int)__builtin_amdgcn_alignbyte(dd[i + 1], whole ? dd[i + 1] : dd[i], s1));
+          const int sb = in_vgpr(__builtin_amdgcn_ds_bpermute(from_lane, sc));
+          acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av[0], bv, acc[t], 0, 4, 0, sa, 0, sb);
+          acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av[1], bv, acc[t], 0, 4, 1, sa, 0, sb);
+          if constexpr (NT == 3)
+            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av[2], bv, acc[t], 0, 4, 2, sa, 0, sb);
+        }
+      }
+    }
+  };
+
+  Stage s0, s1;
+  issue(s0, 0);
+  int q = 0;
+  while (q + 2 < ngroups) {  // no branch inside: every wait is for exactly the loads it needs
+    issue(s1, q + 1);
+    consume(s0, q);
+    issue(s0, q + 2);
+    consume(s1, q + 1);
+    q += 2;
+  }
+  if (q + 1 < ngroups) {
+    issue(s1, q + 1);
+    consume(s0, q);
+    consume(s1, q + 1);
+  } else {
+    consume(s0, q);
+  }
+
+  // ---- epilogue: this wave's columns
+  const int col = n0 + 16 * wave + r;
+  if (col < N) {
+    const float gb = a.bias ? in_global(a.bias)[(size_t)sg.expert * N + col] : 0.f;
+    const float ub = (GLU && a.bias2) ? in_global(a.bias2)[(size_t)sg.expert * N + col] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int m = 4 * kb + i;
+      if (m < rows_here) {
+        const int p = in_global(a.order)[sg.start + 16 * mt + m];
+        float v = acc[0][i] + gb;
+        if constexpr (GLU) v = kq::glu_epilogue_fast(a.act, v, acc[TPW - 1][i] + ub, a.limit, a.alpha);
+        kq::store_result<DT>(a.y, a.om, (size_t)kq::out_row(a.om, p) * N + col, v);
+      }
+    }
+  }
+}
+
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 int f4_steps(int K) { return ((K >> 5) + 3) / 4; }
 
@@ -471,13 +662,21 @@ int kq_launch_fp4_moe(const void* x, const uint8_t* w, const uint8_t* w2, const 
   hipLaunchKernelGGL((fp4_grouped_kernel<DTV, GLUV, JV, MTV>),                                                   \
                      dim3((N + (GLUV ? 8 * JV : 16 * JV) - 1) / (GLUV ? 8 * JV : 16 * JV), maxseg, MTV == 1 ? 2 : 1), \
                      dim3(F4_THREADS), 0, s, a)
-  if (glu) {
+#ifndef KQ_F4_TILES
+#define KQ_F4_TILES 1
+#endif
+#define KQ_F4_LAUNCH_TILES(DTV)                                                                               \
+  hipLaunchKernelGGL((fp4_glu_tiles_kernel<DTV>), dim3((N + 63) / 64, maxseg, 2), dim3(F4_THREADS), 0, s, a)
+  if (KQ_F4_TILES && glu && !two) {  // the fused op on one m-tile per pass: the waves split the column tiles
+    if (dtype == KQ_F16) KQ_F4_LAUNCH_TILES(KQ_F16); else KQ_F4_LAUNCH_TILES(KQ_BF16);
+  } else if (glu) {
     if (dtype == KQ_F16) { if (two) KQ_F4_LAUNCH(KQ_F16, true, 4, 2); else KQ_F4_LAUNCH(KQ_F16, true, 8, 1); }
     else { if (two) KQ_F4_LAUNCH(KQ_BF16, true, 8, 2); else KQ_F4_LAUNCH(KQ_BF16, true, 8, 1); }
   } else {
     if (dtype == KQ_F16) { if (two) KQ_F4_LAUNCH(KQ_F16, false, 4, 2); else KQ_F4_LAUNCH(KQ_F16, false, 4, 1); }
     else { if (two) KQ_F4_LAUNCH(KQ_BF16, false, 8, 2); else KQ_F4_LAUNCH(KQ_BF16, false, 4, 1); }
   }
+#undef KQ_F4_LAUNCH_TILES
 #undef KQ_F4_LAUNCH
   KQ_HIP_CHECK(hipGetLastError());
   return KQ_OK;
