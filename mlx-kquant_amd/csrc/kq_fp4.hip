@@ -18,12 +18,14 @@
 // for A as for B (for A that is not the lane holding those values); D lane l holds column l % 16, rows 4 (l / 16) .. + 3.  A wire block keeps weight j in the low and weight j + 16 in the high nibble
 // of byte j, so code i of a block is weight i / 2 (+ 16 for odd i): the prepass stores the activations in that order.
 //
-// Kernel: pairs sorted by expert into segments (the sort of kq_moe.hip); a workgroup of four waves takes one m-tile
-// (16 pairs) of a segment and 128 weight rows (fused gate / up: 64 + the same 64 of the up matrix).  The waves split
-// K (steps of 128 dealt round-robin): every wave streams all eight column tiles of its steps straight from global
-// memory into registers (aligned dwords around each 17-byte block, the codes realigned with byte shifts), one step
-// ahead, and the four partial sums meet in LDS.  No LDS staging, no barrier in the stream, about a dozen vector
-// instructions per 32 weights.
+// Kernels: pairs sorted by expert into segments (the sort of kq_moe_sort.h); a workgroup of four waves takes one
+// m-tile (16 pairs) of a segment and 64 output columns (fused gate / up: 64 weight rows of each matrix).  The weights
+// go straight from global memory into registers (aligned dwords around each 17-byte block, the codes realigned with
+// byte shifts): no LDS staging of weights.  fp4_grouped_kernel: the waves split K (steps of 128 dealt round-robin),
+// every wave streams all column tiles of its steps one step ahead, the four partial sums meet in LDS (the plain op;
+// two m-tiles on the same weight registers).  fp4_glu_tiles_kernel: the waves split the column tiles, a wave reads
+// four consecutive steps of its gate and up tile per load group, one group ahead, and the activation terms of a step
+// are loaded by one wave and shared through LDS (the fused op on one m-tile).
 #include <type_traits>
 
 #include "kq_common.h"
