@@ -524,15 +524,13 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
           window(t, s, sh, back, live);
           const u32x4 d = st.d[t][g];
           const int sc = live ? (int)((d[0] >> (8 * sh)) & 0xff) : 127;
-          // codes start at byte sh + 1 of the window: a shift by 1 .. 3 bytes, or (sh = 3) the next dword as it is
-          const bool whole = sh == 3;
-          const uint32_t s1 = (sh + 1) & 3u;
+          // codes start at byte sh + 1 of the window: bytes sh + 1 .. sh + 4 of each pair of neighbouring dwords
+          const uint32_t sel = 0x03020100u + 0x01010101u * (sh + 1u);
           const uint32_t dd[5] = {d[0], d[1], d[2], d[3], st.d4[t][g] >> (8 * back)};
           v8i bv = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
           for (int i = 0; i < 4; i++)
-            bv[i] = __builtin_amdgcn_ds_bpermute(
-                from_lane, (int)__builtin_amdgcn_alignbyte(dd[i + 1], whole ? dd[i + 1] : dd[i], s1));
+            bv[i] = __builtin_amdgcn_ds_bpermute(from_lane, (int)__builtin_amdgcn_perm(dd[i + 1], dd[i], sel));
           const int sb = in_vgpr(__builtin_amdgcn_ds_bpermute(from_lane, sc));
           acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av[0], bv, acc[t], 0, 4, 0, sa, 0, sb);
           acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av[1], bv, acc[t], 0, 4, 1, sa, 0, sb);
