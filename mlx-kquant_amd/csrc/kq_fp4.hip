@@ -452,16 +452,16 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
   };
   // the window of block (tile t, step s) of this lane: address of its first dword, the byte shift, and how many
   // bytes earlier the fifth dword is fetched (the last block of a stack: the dword would reach past the end)
-  auto window = [&](int t, int s, uint32_t& sh, uint32_t& back, bool& live) {
+  auto window = [&](auto tail_c, int t, int s, uint32_t& sh, uint32_t& back, bool& live) {
     int blk = 4 * s + kbl;
     live = blk < nblk;  // past K: any block of the row with a neutral scale (the activations are zeros)
     blk = live ? blk : nblk - 1;
     const uint32_t off = (uint32_t)blk * 17u;
     sh = (wlow[t] + off) & 3u;
-    back = (last_row[t] && blk == nblk - 1) ? 3u - sh : 0u;
+    back = (decltype(tail_c)::value && last_row[t] && blk == nblk - 1) ? 3u - sh : 0u;
     return reinterpret_cast<uintptr_t>(wrow[t]) + off - sh;
   };
-  auto issue = [&](Stage& st, int q) {  // group q: steps SPG q .. + SPG - 1 (past the last: the last once more, unused)
+  auto issue = [&](auto tail_c, Stage& st, int q) {  // group q: steps SPG q .. + SPG - 1 (past the last: the last once more, unused)
 #pragma unroll
     for (int t = 0; t < TPW; t++)
 #pragma unroll
@@ -470,7 +470,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
         s = s < nsteps ? s : nsteps - 1;
         uint32_t sh, back;
         bool live;
-        const uintptr_t qa = window(t, s, sh, back, live);
+        const uintptr_t qa = window(tail_c, t, s, sh, back, live);
         st.d[t][g] = *(const __attribute__((address_space(1))) u32x4_a4*)qa;  // dword-aligned, no more
         typedef uint32_t u32_a1 __attribute__((aligned(1)));
         st.d4[t][g] = *(const __attribute__((address_space(1))) u32_a1*)(qa + 16 - back);
@@ -490,7 +490,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
   v4f acc[TPW];
 #pragma unroll
   for (int t = 0; t < TPW; t++) acc[t] = v4f{0, 0, 0, 0};
-  auto consume = [&](const Stage& st, int q) {
+  auto consume = [&](auto tail_c, const Stage& st, int q) {
     // this wave's steps of activation terms into LDS: lane (row rl, block kbl) writes where operand lane
     // (m = rl, a = kbl) will read
 #pragma unroll
@@ -521,7 +521,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
         for (int t = 0; t < TPW; t++) {
           uint32_t sh, back;
           bool live;
-          window(t, s, sh, back, live);
+          window(tail_c, t, s, sh, back, live);
           const u32x4 d = st.d[t][g];
           const int sc = live ? (int)((d[0] >> (8 * sh)) & 0xff) : 127;
           // codes start at byte sh + 1 of the window: bytes sh + 1 .. sh + 4 of each pair of neighbouring dwords
@@ -541,23 +541,32 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
     }
   };
 
-  Stage s0, s1;
-  issue(s0, 0);
-  int q = 0;
-  while (q + 2 < ngroups) {  // no branch inside: every wait is for exactly the loads it needs
-    issue(s1, q + 1);
-    consume(s0, q);
-    issue(s0, q + 2);
-    consume(s1, q + 1);
-    q += 2;
-  }
-  if (q + 1 < ngroups) {
-    issue(s1, q + 1);
-    consume(s0, q);
-    consume(s1, q + 1);
-  } else {
-    consume(s0, q);
-  }
+  // The work item that holds the last row of a stack (a uniform condition) runs the form that can fetch a fifth
+  // dword early; every other item the form without that arithmetic.
+  auto stream = [&](auto tail_c) {
+    Stage s0, s1;
+    issue(tail_c, s0, 0);
+    int q = 0;
+    while (q + 2 < ngroups) {  // no branch inside: every wait is for exactly the loads it needs
+      issue(tail_c, s1, q + 1);
+      consume(tail_c, s0, q);
+      issue(tail_c, s0, q + 2);
+      consume(tail_c, s1, q + 1);
+      q += 2;
+    }
+    if (q + 1 < ngroups) {
+      issue(tail_c, s1, q + 1);
+      consume(tail_c, s0, q);
+      consume(tail_c, s1, q + 1);
+    } else {
+      consume(tail_c, s0, q);
+    }
+  };
+  const uint8_t* after_tiles = a.w + (int64_t)sg.expert * a.w_expert_stride + (size_t)N * row_bytes;
+  if (after_tiles == a.w_end && n0 + 64 >= N)
+    stream(std::true_type{});
+  else
+    stream(std::false_type{});
 
   // ---- epilogue: this wave's columns
   const int col = n0 + 16 * wave + r;
