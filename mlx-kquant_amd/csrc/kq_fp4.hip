@@ -425,19 +425,22 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
   const int rows_here = sg.count - 16 * mt < 16 ? sg.count - 16 * mt : 16;
   const int ngroups = (nsteps + SPG - 1) / SPG;
 
-  const uint8_t* wrow[TPW];
-#pragma unroll
-  for (int t = 0; t < TPW; t++) {
+  // A row is addressed as a matrix pointer held in scalar registers plus a 32-bit byte offset per lane (the pointer
+  // is taken four bytes low and the offset four bytes high: a block's window starts up to three bytes before it).
+  const int expert = __builtin_amdgcn_readfirstlane(sg.expert);
+  const uint8_t* wmat[TPW];
+  uint32_t woff, wlow[TPW];  // the lane's row offset in both matrices; low address bits of its rows
+  bool last_row[TPW];        // the row is the last of its stack
+  {
     int c = n0 + 16 * wave + rl;
     c = c < N ? c : N - 1;  // columns past N re-read the last one (not stored)
-    wrow[t] = (t ? a.w2 : a.w) + (int64_t)sg.expert * a.w_expert_stride + (size_t)c * row_bytes;
+    woff = (uint32_t)c * row_bytes + 4u;
   }
-  uint32_t wlow[TPW];  // low address bits of the rows
-  bool last_row[TPW];  // the row is the last of its stack
 #pragma unroll
   for (int t = 0; t < TPW; t++) {
-    wlow[t] = (uint32_t)reinterpret_cast<uintptr_t>(wrow[t]) & 3u;
-    last_row[t] = wrow[t] + row_bytes == (t ? a.w2_end : a.w_end);
+    wmat[t] = (t ? a.w2 : a.w) + (int64_t)expert * a.w_expert_stride - 4;
+    wlow[t] = ((uint32_t)reinterpret_cast<uintptr_t>(wmat[t]) + woff) & 3u;
+    last_row[t] = wmat[t] + woff + row_bytes == (t ? a.w2_end : a.w_end);
   }
   const int mrow = rl < rows_here ? rl : rows_here - 1;  // rows past the segment re-read its last pair (dropped)
   const int xrow = in_global(a.order)[sg.start + 16 * mt + mrow] / a.x_div;
@@ -459,7 +462,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
     const uint32_t off = (uint32_t)blk * 17u;
     sh = (wlow[t] + off) & 3u;
     back = (decltype(tail_c)::value && last_row[t] && blk == nblk - 1) ? 3u - sh : 0u;
-    return reinterpret_cast<uintptr_t>(wrow[t]) + off - sh;
+    return reinterpret_cast<uintptr_t>(wmat[t] + (woff + off - sh));
   };
   auto issue = [&](auto tail_c, Stage& st, int q) {  // group q: steps SPG q .. + SPG - 1 (past the last: the last once more, unused)
 #pragma unroll
@@ -562,7 +565,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
       consume(tail_c, s0, q);
     }
   };
-  const uint8_t* after_tiles = a.w + (int64_t)sg.expert * a.w_expert_stride + (size_t)N * row_bytes;
+  const uint8_t* after_tiles = wmat[0] + 4 + (size_t)N * row_bytes;
   if (after_tiles == a.w_end && n0 + 64 >= N)
     stream(std::true_type{});
   else
@@ -571,8 +574,8 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
   // ---- epilogue: this wave's columns
   const int col = n0 + 16 * wave + r;
   if (col < N) {
-    const float gb = a.bias ? in_global(a.bias)[(size_t)sg.expert * N + col] : 0.f;
-    const float ub = (GLU && a.bias2) ? in_global(a.bias2)[(size_t)sg.expert * N + col] : 0.f;
+    const float gb = a.bias ? in_global(a.bias)[(size_t)expert * N + col] : 0.f;
+    const float ub = (GLU && a.bias2) ? in_global(a.bias2)[(size_t)expert * N + col] : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int m = 4 * kb + i;
@@ -602,7 +605,7 @@ bool kq_fp4_moe_supported(int P, int E, int N, int K, int codec) {
 #endif
   const int min_pairs = (K & 255) ? KQ_FP4_MIN_PAIRS_TAIL : 17;
   return codec == KQ_MXFP4 && P >= min_pairs && E > 0 && E <= 4096 && (int64_t)E + P / 32 < 65535 && N > 0 && K >= 32 &&
-         (K & 31) == 0 && (int64_t)N * (K >> 5) * 17 < ((int64_t)1 << 32);
+         (K & 31) == 0 && (int64_t)N * (K >> 5) * 17 < ((int64_t)1 << 32) - 64;
 }
 
 // Workspace: sorted pair list, segment table, segment count, then the prepass outputs for `rows` activation rows
