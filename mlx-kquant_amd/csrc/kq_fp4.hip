@@ -398,13 +398,12 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
 // load time would make the wave wait there).  The activation terms of a step are loaded once per workgroup -- wave v
 // takes step 4 q + v of a group of four -- and shared through LDS in operand order, so they need no lane exchange
 // and cost a fifth of the load instructions they cost when every wave fetches the terms of its own step.
-// (The plain op, one tile per wave, measured slower in this form than with the K steps split: 39.7 us in groups of
-// four steps, 45.6 in groups of eight, against 36.6; it stays on the kernel above.)
-template <int DT>
+// (GLU = false, the plain op with one tile per wave, measured slower in this form than with the K steps split: 37.3
+// us against 36.6 on 32 experts of 2880 x 2880 at 256 pairs; it stays on the kernel above and is not instantiated.)
+template <int DT, bool GLU = true>
 __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) {
   constexpr int NT = f4_terms<DT>();
-  constexpr bool GLU = true;
-  constexpr int TPW = 2;  // tiles per wave: gate and up
+  constexpr int TPW = GLU ? 2 : 1;  // tiles per wave: gate and up
   constexpr int SPG = 4;  // steps per group: a stage is eight blocks per lane
   constexpr int SPW = 1;  // steps of activation terms a wave loads per group
   constexpr int A_STEP = NT * 2048 + 256;  // LDS bytes of a step's terms: [term][half][a][m][16] + scales [kb][m]
