@@ -49,7 +49,6 @@ __device__ __forceinline__ const __attribute__((address_space(1))) T* in_global(
   return (const __attribute__((address_space(1))) T*)(uintptr_t)p;
 }
 
-constexpr int F4_STAGES = 2;     // register stages in rotation: a step's loads are queued one step ahead (deeper: no gain)
 constexpr int F4_THREADS = 256;  // four waves
 
 template <int DT>
@@ -220,15 +219,24 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
   const int n0 = blockIdx.x * COLS;
   const int rows_here = sg.count - 16 * mt < 16 * MT ? sg.count - 16 * mt : 16 * MT;
 
-  // weight rows of this lane: tile j covers columns n0 + 16 j .. (fused: tiles 4 .. 7 are the same columns of the up
-  // matrix); columns past N re-read the last one
-  const uint8_t* wrow[J];
+  // Weight rows of this lane: tile j covers columns n0 + 16 j .. (fused: tiles JH .. are the same columns of the up
+  // matrix); columns past N re-read the last one.  A row is addressed as a matrix pointer held in scalar registers
+  // plus a 32-bit byte offset per lane (the pointer is taken four bytes low and the offset four bytes high: a
+  // block's window starts up to three bytes before it).
+  const int expert = __builtin_amdgcn_readfirstlane(sg.expert);
+  const uint8_t* wmat[2];
+  wmat[0] = a.w + (int64_t)expert * a.w_expert_stride - 4;
+  wmat[1] = GLU ? a.w2 + (int64_t)expert * a.w_expert_stride - 4 : wmat[0];
+  uint32_t woff[J];
+  uint32_t row_meta = 0;  // bits 2 j, 2 j + 1: low address bits of row j; bit 16 + j: the row is the last of its stack
 #pragma unroll
   for (int j = 0; j < J; j++) {
     int c = n0 + 16 * (GLU ? (j % JH) : j) + rl;
     c = c < N ? c : N - 1;
-    const uint8_t* base = (GLU && j >= JH) ? a.w2 : a.w;
-    wrow[j] = base + (int64_t)sg.expert * a.w_expert_stride + (size_t)c * row_bytes;
+    woff[j] = (uint32_t)c * row_bytes + 4u;
+    const uint8_t* base = wmat[(GLU && j >= JH) ? 1 : 0];
+    row_meta |= (((uint32_t)reinterpret_cast<uintptr_t>(base) + woff[j]) & 3u) << (2 * j);
+    row_meta |= (base + woff[j] + row_bytes == ((GLU && j >= JH) ? a.w2_end : a.w_end) ? 1u : 0u) << (16 + j);
   }
   // activation rows of this lane (rows past the segment re-read its last pair; their results are dropped)
   const uint8_t* arow[MT];
@@ -241,42 +249,36 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
     srow[m] = a.xs + (size_t)xrow * nsteps * 4 + kbl;
   }
 
+  // A stage holds what the loads of a step return, untouched: anything computed from a loaded register at load
+  // time would make the wave wait for the data there.
   struct Stage {
-    u32x4 b[J];
-    int sb[J];
+    u32x4 d[J];      // the four aligned dwords at and after a block's first byte
+    uint32_t d4[J];  // the fifth
     v8i av[MT][NT];
     int sa[MT];
   };
-  auto fetch = [&](Stage& st, int s) {
+  // The 17 bytes of a block (scale, 16 code bytes) sit at any byte offset: five aligned dwords around them, the codes
+  // brought to dword boundaries by one byte permute per dword when the stage is used.  For the last block of a stack
+  // the fifth dword would reach past the end: it is fetched 3 - sh bytes earlier and shifted back (the bytes past
+  // the end are not part of the block); that arithmetic runs only in the work item that holds the stack's last row.
+  auto window = [&](auto tail_c, int j, int s, uint32_t& sh, uint32_t& back, bool& live) {
     int blk = 4 * s + kbl;
-    const bool live = blk < nblk;  // past K: any block of the row with a neutral scale (the activations are zeros)
+    live = blk < nblk;  // past K: any block of the row with a neutral scale (the activations are zeros)
     blk = live ? blk : nblk - 1;
     const uint32_t off = (uint32_t)blk * 17u;
+    sh = (((row_meta >> (2 * j)) & 3u) + off) & 3u;
+    back = (decltype(tail_c)::value && ((row_meta >> (16 + j)) & 1u) && blk == nblk - 1) ? 3u - sh : 0u;
+    return reinterpret_cast<uintptr_t>(wmat[(GLU && j >= JH) ? 1 : 0] + (woff[j] + off - sh));
+  };
+  auto fetch = [&](auto tail_c, Stage& st, int s) {
 #pragma unroll
     for (int j = 0; j < J; j++) {
-      // the 17 bytes of the block (scale, 16 code bytes) sit at any byte offset: five aligned dwords around them,
-      // the codes brought to dword boundaries with byte shifts
-      const uintptr_t ad = reinterpret_cast<uintptr_t>(wrow[j] + off);
-      const uint32_t sh = (uint32_t)ad & 3u;
-      const uint32_t* q = reinterpret_cast<const uint32_t*>(ad - sh);
-      const u32x4 d = *(const __attribute__((address_space(1))) u32x4_a4*)(uintptr_t)q;  // dword-aligned, no more
-      // the fifth dword; for the last block of the stack it would reach past the end: fetched that many bytes earlier
-      // and shifted back (the bytes past the end are not part of the block)
-      const uint8_t* wend = (GLU && j >= JH) ? a.w2_end : a.w_end;
-      const int64_t over = reinterpret_cast<const uint8_t*>(q + 5) - wend;
-      const uint32_t back = over > 0 ? (uint32_t)over : 0u;
+      uint32_t sh, back;
+      bool live;
+      const uintptr_t q = window(tail_c, j, s, sh, back, live);
+      st.d[j] = *(const __attribute__((address_space(1))) u32x4_a4*)q;  // dword-aligned, no more
       typedef uint32_t u32_a1 __attribute__((aligned(1)));
-      const uint32_t d4 =
-          *(const __attribute__((address_space(1))) u32_a1*)(reinterpret_cast<uintptr_t>(q + 4) - back) >> (8 * back);
-      const int sc = (int)((d[0] >> (8 * sh)) & 0xff);
-      st.sb[j] = live ? sc : 127;
-      // codes start at byte sh + 1 of the window: a shift by 1 .. 3 bytes, or (sh = 3) the next dword as it is
-      const bool whole = sh == 3;
-      const uint32_t s1 = (sh + 1) & 3u;
-      const uint32_t dd[5] = {d[0], d[1], d[2], d[3], d4};
-#pragma unroll
-      for (int i = 0; i < 4; i++)
-        st.b[j][i] = __builtin_amdgcn_alignbyte(dd[i + 1], whole ? dd[i + 1] : dd[i], s1);
+      st.d4[j] = *(const __attribute__((address_space(1))) u32_a1*)(q + 16 - back);
     }
 #pragma unroll
     for (int m = 0; m < MT; m++) {
@@ -295,7 +297,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
 #pragma unroll
     for (int j = 0; j < J; j++) acc[m][j] = v4f{0, 0, 0, 0};
   auto to_operand_lane = [&](int v) { return COAL ? __builtin_amdgcn_ds_bpermute(from_lane, v) : v; };
-  auto multiply = [&](const Stage& st) {
+  auto multiply = [&](auto tail_c, const Stage& st, int s) {
     v8i av[MT][NT];
     int sav[MT];
 #pragma unroll
@@ -308,9 +310,18 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
     }
 #pragma unroll
     for (int j = 0; j < J; j++) {
-      const v8i bv = {to_operand_lane((int)st.b[j][0]), to_operand_lane((int)st.b[j][1]), to_operand_lane((int)st.b[j][2]),
-                      to_operand_lane((int)st.b[j][3]), 0, 0, 0, 0};
-      const int sb = in_vgpr(to_operand_lane(st.sb[j]));
+      uint32_t sh, back;
+      bool live;
+      window(tail_c, j, s, sh, back, live);
+      const u32x4 d = st.d[j];
+      const int sc = live ? (int)((d[0] >> (8 * sh)) & 0xff) : 127;
+      // codes start at byte sh + 1 of the window: bytes sh + 1 .. sh + 4 of each pair of neighbouring dwords
+      const uint32_t sel = 0x03020100u + 0x01010101u * (sh + 1u);
+      const uint32_t dd[5] = {d[0], d[1], d[2], d[3], st.d4[j] >> (8 * back)};
+      v8i bv = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 4; i++) bv[i] = to_operand_lane((int)__builtin_amdgcn_perm(dd[i + 1], dd[i], sel));
+      const int sb = in_vgpr(to_operand_lane(sc));
 #pragma unroll
       for (int m = 0; m < MT; m++) {
         const int sa = in_vgpr(sav[m]);
@@ -322,25 +333,35 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
     }
   };
 
-  // this wave's steps: wave, wave + 4, ...; F4_STAGES register stages in rotation, the loads of the next
-  // F4_STAGES - 1 steps in flight during a multiply
-  constexpr int S = F4_STAGES;
-  Stage st[S];
-  int s = wave;
-  kq::SForF4<S - 1>::run([&](auto ic) {
-    constexpr int i = decltype(ic)::value;
-    if (s + 4 * i < nsteps) fetch(st[i], s + 4 * i);
-  });
-  while (s < nsteps) {
-    kq::SForF4<S>::run([&](auto ic) {
-      constexpr int i = decltype(ic)::value;
-      if (s < nsteps) {
-        if (s + 4 * (S - 1) < nsteps) fetch(st[(i + S - 1) % S], s + 4 * (S - 1));
-        multiply(st[i]);
-        s += 4;
-      }
-    });
-  }
+  // This wave's steps: wave, wave + 4, ...: two register stages, the loads of a step issued before the step before
+  // it is multiplied.  The loop body holds no branch, so the wait before a multiply is for exactly the loads it
+  // needs; the work item that holds the last row of a stack (a uniform condition) runs the form with the stack-end
+  // arithmetic, every other item the form without.
+  const int nq = wave < nsteps ? (nsteps - wave + 3) >> 2 : 0;  // steps of this wave
+  auto stream = [&](auto tail_c) {
+    if (nq == 0) return;
+    Stage s0, s1;
+    fetch(tail_c, s0, wave);
+    int q = 0;
+    while (q + 2 < nq) {
+      fetch(tail_c, s1, wave + 4 * (q + 1));
+      multiply(tail_c, s0, wave + 4 * q);
+      fetch(tail_c, s0, wave + 4 * (q + 2));
+      multiply(tail_c, s1, wave + 4 * (q + 1));
+      q += 2;
+    }
+    if (q + 1 < nq) {
+      fetch(tail_c, s1, wave + 4 * (q + 1));
+      multiply(tail_c, s0, wave + 4 * q);
+      multiply(tail_c, s1, wave + 4 * (q + 1));
+    } else {
+      multiply(tail_c, s0, wave + 4 * q);
+    }
+  };
+  if (wmat[0] + 4 + (size_t)N * row_bytes == a.w_end && n0 + COLS >= N)
+    stream(std::true_type{});
+  else
+    stream(std::false_type{});
 
   // ---- the four partial sums meet in LDS; wave w finishes J / 4 tiles (fused: gate tile w with up tile w)
 #pragma unroll
@@ -348,7 +369,6 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
 #pragma unroll
     for (int j = 0; j < J; j++) red[wave][m * J + j][lane] = acc[m][j];
   __syncthreads();
-  const int expert = sg.expert;
   auto total = [&](int j) {
     v4f v = red[0][j][lane];
 #pragma unroll
