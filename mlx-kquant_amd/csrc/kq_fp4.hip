@@ -26,6 +26,7 @@
 // two m-tiles on the same weight registers).  fp4_glu_tiles_kernel: the waves split the column tiles, a wave reads
 // four consecutive steps of its gate and up tile per load group, one group ahead, and the activation terms of a step
 // are loaded by one wave and shared through LDS (the fused op on one m-tile).
+#include <atomic>
 #include <type_traits>
 
 #include "kq_common.h"
@@ -418,14 +419,17 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_grouped_kernel(F4Args a) {
 // load time would make the wave wait there).  The activation terms of a step are loaded once per workgroup -- wave v
 // takes step 4 q + v of a group of four -- and shared through LDS in operand order, so they need no lane exchange
 // and cost a fifth of the load instructions they cost when every wave fetches the terms of its own step.
+// NW = waves per workgroup: four (64 columns), or two (32 columns, every wave loading the terms of two steps of a
+// group) for calls of so few pairs that 64-column groups would leave CUs without a workgroup.
 // (GLU = false, the plain op with one tile per wave, measured slower in this form than with the K steps split: 37.3
 // us against 36.6 on 32 experts of 2880 x 2880 at 256 pairs; it stays on the kernel above and is not instantiated.)
-template <int DT, bool GLU = true>
-__global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) {
+template <int DT, bool GLU = true, int NW = 4>
+__global__ __launch_bounds__(64 * NW, 2) void fp4_glu_tiles_kernel(F4Args a) {
   constexpr int NT = f4_terms<DT>();
   constexpr int TPW = GLU ? 2 : 1;  // tiles per wave: gate and up
   constexpr int SPG = 4;  // steps per group: a stage is eight blocks per lane
-  constexpr int SPW = 1;  // steps of activation terms a wave loads per group
+  constexpr int SPW = 4 / NW;  // steps of activation terms a wave loads per group
+  constexpr int COLS = 16 * NW;  // output columns of a workgroup
   constexpr int A_STEP = NT * 2048 + 256;  // LDS bytes of a step's terms: [term][half][a][m][16] + scales [kb][m]
   __shared__ __attribute__((aligned(16))) uint8_t abuf[2][SPG][A_STEP];
   const int nseg = *in_global(a.nseg);
@@ -440,7 +444,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
   const int from_lane = 4 * (16 * ((lane >> 2) & 3) + 4 * (lane & 3) + (lane >> 4));
   const int N = a.N, nsteps = a.nsteps, nblk = a.K >> 5;
   const uint32_t row_bytes = (uint32_t)nblk * 17u;
-  const int n0 = blockIdx.x * 64;
+  const int n0 = blockIdx.x * COLS;
   const int rows_here = sg.count - 16 * mt < 16 ? sg.count - 16 * mt : 16;
   const int ngroups = (nsteps + SPG - 1) / SPG;
 
@@ -499,7 +503,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
       }
 #pragma unroll
     for (int i = 0; i < SPW; i++) {
-      int s = SPG * q + 4 * i + wave;
+      int s = SPG * q + NW * i + wave;
       s = s < nsteps ? s : nsteps - 1;
 #pragma unroll
       for (int t = 0; t < NT; t++) {
@@ -517,7 +521,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
     // (m = rl, a = kbl) will read
 #pragma unroll
     for (int i = 0; i < SPW; i++) {
-      uint8_t* ab = abuf[q & 1][4 * i + wave];
+      uint8_t* ab = abuf[q & 1][NW * i + wave];
 #pragma unroll
       for (int t = 0; t < NT; t++) {
         *reinterpret_cast<u32x4*>(ab + (((t * 2 + 0) * 4 + kbl) * 16 + rl) * 16) = st.lo[i][t];
@@ -585,7 +589,7 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
     }
   };
   const uint8_t* after_tiles = wmat[0] + 4 + (size_t)N * row_bytes;
-  if (after_tiles == a.w_end && n0 + 64 >= N)
+  if (after_tiles == a.w_end && n0 + COLS >= N)
     stream(std::true_type{});
   else
     stream(std::false_type{});
@@ -609,6 +613,18 @@ __global__ __launch_bounds__(F4_THREADS, 2) void fp4_glu_tiles_kernel(F4Args a) 
 }
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+int f4_num_cus() {
+  // compute units of the current device, looked up once per device
+  static std::atomic<int> cus[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
 int f4_steps(int K) { return ((K >> 5) + 3) / 4; }
 
 }  // namespace
@@ -696,10 +712,15 @@ int kq_launch_fp4_moe(const void* x, const uint8_t* w, const uint8_t* w2, const 
 #ifndef KQ_F4_TILES
 #define KQ_F4_TILES 1
 #endif
-#define KQ_F4_LAUNCH_TILES(DTV)                                                                               \
-  hipLaunchKernelGGL((fp4_glu_tiles_kernel<DTV>), dim3((N + 63) / 64, maxseg, 2), dim3(F4_THREADS), 0, s, a)
+#define KQ_F4_LAUNCH_TILES(DTV, NWV)                                                                            \
+  hipLaunchKernelGGL((fp4_glu_tiles_kernel<DTV, true, NWV>), dim3((N + 16 * NWV - 1) / (16 * NWV), maxseg, 2),   \
+                     dim3(64 * NWV), 0, s, a)
   if (KQ_F4_TILES && glu && !two) {  // the fused op on one m-tile per pass: the waves split the column tiles
-    if (dtype == KQ_F16) KQ_F4_LAUNCH_TILES(KQ_F16); else KQ_F4_LAUNCH_TILES(KQ_BF16);
+    // few pairs: 32-column workgroups of two waves where 64-column groups would leave most CUs one workgroup or none
+    // (32 experts of 2880 x 2880: 8 pairs 25.5 -> 23.1 us; 12 pairs 27.6 -> 29.1 and 16 pairs 33.9 -> 36.2 the other way)
+    const bool narrow = (int64_t)4 * P * ((N + 63) / 64) < (int64_t)7 * f4_num_cus();
+    if (dtype == KQ_F16) { if (narrow) KQ_F4_LAUNCH_TILES(KQ_F16, 2); else KQ_F4_LAUNCH_TILES(KQ_F16, 4); }
+    else { if (narrow) KQ_F4_LAUNCH_TILES(KQ_BF16, 2); else KQ_F4_LAUNCH_TILES(KQ_BF16, 4); }
   } else if (glu) {
     if (dtype == KQ_F16) { if (two) KQ_F4_LAUNCH(KQ_F16, true, 4, 2); else KQ_F4_LAUNCH(KQ_F16, true, 8, 1); }
     else { if (two) KQ_F4_LAUNCH(KQ_BF16, true, 8, 2); else KQ_F4_LAUNCH(KQ_BF16, true, 8, 1); }
