@@ -280,6 +280,31 @@ def test_moe_routes_on_32_experts_of_2880_square(kq, T):
     assert rel_l2(dev_to_bits(got), O.gather_qmv(hb, up, codec, idx, gb, "bfloat16"), "bfloat16") <= TOL, T
 
 
+@pytest.mark.parametrize("E,T,R", [(8, 2, 4), (8, 20, 4), (4, 40, 2)])
+@pytest.mark.parametrize("N,K", [(200, 736), (64, 2880)])
+def test_moe_mxfp4_block_scaled_forms(kq, E, T, R, N, K):
+    """The three forms of the block-scaled kernels on stacks whose K ends inside a step and inside a 256-weight unit
+    (736 = 23 blocks; 2880) and whose last column group is ragged (200 columns): 8 pairs (two-wave workgroups on 32
+    columns), 80 pairs on 8 experts (four waves, one m-tile per pass), 80 pairs on 4 experts (two m-tiles on the same
+    weight registers); fused op with biases and swiglu_clamp and plain op with a bias, both activation dtypes."""
+    codec = "mxfp4"
+    gate, up = _stack(codec, E, N, K, seed=161), _stack(codec, E, N, K, seed=162)
+    rng = np.random.default_rng(163)
+    idx = np.stack([rng.permutation(E)[:R] for _ in range(T)])
+    gb = (rng.standard_normal((E, N)) * 0.05).astype(np.float32)
+    ub = (rng.standard_normal((E, N)) * 0.05).astype(np.float32)
+    for dtype in ("bfloat16", "float16"):
+        xb, xt = make_x((T, K), dtype, seed=164, scale=0.05)
+        got = kq.moe_glu_gather_kq(xt, wire_to_dev(gate), wire_to_dev(up), codec, _idx_dev(idx), act="swiglu_clamp",
+                                   limit=7.0, alpha=1.702, gate_bias=torch.from_numpy(gb).cuda(),
+                                   up_bias=torch.from_numpy(ub).cuda())
+        want = _glu_truth(codec, xb, gate, up, idx, "swiglu_clamp", 7.0, 1.702, gb, ub, dtype=dtype)
+        assert rel_l2(dev_to_bits(got), want, dtype) <= TOL, (E, T, R, N, K, dtype)
+        hb, ht = make_x((T, R, K), dtype, seed=165, scale=0.05)
+        got = kq.gather_qmv_kq(ht, wire_to_dev(up), codec, _idx_dev(idx), bias=torch.from_numpy(gb).cuda())
+        assert rel_l2(dev_to_bits(got), O.gather_qmv(hb, up, codec, idx, gb, dtype), dtype) <= TOL, (E, T, R, N, K, dtype)
+
+
 @pytest.mark.parametrize("T", [16, 40])
 @pytest.mark.parametrize("off", [1, 2, 3])
 def test_moe_mxfp4_stacks_at_any_byte_offset_use_nothing_past_their_end(kq, off, T):
