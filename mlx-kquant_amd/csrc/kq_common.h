@@ -151,7 +151,7 @@ int kq_launch_gemm2(const void* xh, const void* xhl, const float* rs, const uint
 // (mrows >= M prepared rows): column tiles nt0 .. nt0 + ntiles - 1 of 256 weight rows each.
 bool kq_gemm3_supported(int M, int mrows, int N, int K, int codec);
 int kq_launch_gemm3(const void* xh, const void* xhl, const float* rs, const uint8_t* w, void* y, int M, int mrows, int N,
-                    int K, int codec, int dtype, int nt0, int ntiles, hipStream_t s);
+                    int K, int codec, int dtype, int nt0, int ntiles, hipStream_t s, int tile_rows = 256);
 // The same tile kernel for q2_k / q3_k (M >= 256, tiles filling the chip): runs its own activation prepass.
 bool kq_gemm2_low_supported(int M, int N, int K, int codec);
 size_t kq_gemm2_low_workspace_bytes(int M, int K);

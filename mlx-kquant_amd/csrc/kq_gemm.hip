@@ -13,7 +13,7 @@
 // row-per-lane ds_read_b128 fragment fetch free of bank conflicts).
 #include "kq_mma.h"
 
-static int g_gemm_tile = 0;  // kq_set_gemm_tile_rows: 64, 128, 256, 512, 513 or 1024 forces the tile shape, 0 = automatic
+static int g_gemm_tile = 0;  // kq_set_gemm_tile_rows: 64, 128, 256, 512, 513, 1024 or 1025 forces the tile shape, 0 = automatic
 
 namespace {
 
@@ -298,11 +298,43 @@ int launch_gemm(const void* x, const uint8_t* w, void* y, int M, int N, int K, v
       }
     }
   }
+  if constexpr (C == KQ_Q6_K) {
+    // q6_k on the tiles of kq_gemm3.hip (two exact terms per weight: a decoded fragment feeds sixteen MFMAs on 256-row
+    // tiles, eight on 128-row tiles).  One workgroup per CU, so a call costs whole rounds: a round of 256-row tiles
+    // counts 200, a round of 128-row tiles 119 (measured: 0.59 of the taller tile's time), the 64-row kernel 167 per
+    // 256 half-height tiles whatever their number (it runs at 0.6 of the rate and fills the chip with small
+    // workgroups, K cut over the grid when they are few).  Candidates: every column tile on one tile height, or the
+    // column tiles that fill whole rounds at 256 rows and the rest at whichever height is cheaper (2048 x 28672:
+    // 96 + 16 column tiles = 3 rounds + 1 round of half-height tiles).  `1024` forces the 256-row form for every
+    // column tile, `1025` the 128-row form.
+    const int nt256 = (N + 255) / 256, mt256 = (M + 255) / 256, mt128 = (M + 127) / 128;
+    const int64_t cus = gemm_num_cus();
+    if ((tile == 1024 || tile == 1025) && kq_gemm3_supported(M, mpad, N, K, C))
+      return kq_launch_gemm3(xh, xhl, rs, w, y, M, mpad, N, K, C, DT, 0, nt256, s, tile == 1025 ? 128 : 256);
+    if (tile == 0 && M >= 128 && kq_gemm3_supported(M, mpad, N, K, C)) {
+      auto rounds = [&](int64_t wgs) { return (wgs + cus - 1) / cus; };
+      const int64_t c64 = (int64_t)mt128 * nt256 * 167 / cus;
+      const int64_t c128 = rounds((int64_t)mt128 * nt256) * 119;
+      const int64_t full = (int64_t)mt256 * nt256 / cus;      // whole rounds of 256-row tiles
+      const int tall = full > 0 ? (int)(full * cus / mt256) : 0;  // column tiles in them
+      const int rest = nt256 - tall;
+      const int64_t rest256 = rounds((int64_t)mt256 * rest) * 200, rest128 = rounds((int64_t)mt128 * rest) * 119;
+      const int64_t c256 = full * 200 + (rest128 < rest256 ? rest128 : rest256);
+      if (c256 <= c128 && c256 < c64) {
+        if (tall > 0) {
+          const int rc = kq_launch_gemm3(xh, xhl, rs, w, y, M, mpad, N, K, C, DT, 0, tall, s);
+          if (rc != KQ_OK || rest == 0) return rc;
+        }
+        return kq_launch_gemm3(xh, xhl, rs, w, y, M, mpad, N, K, C, DT, tall, rest, s, rest128 < rest256 ? 128 : 256);
+      }
+      if (c128 < c64) return kq_launch_gemm3(xh, xhl, rs, w, y, M, mpad, N, K, C, DT, 0, nt256, s, 128);
+    }
+  }
   if (tile == 512 || tile == 513 || (tile == 0 && M >= 256 && (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 256)) {
     const int rc = kq_launch_gemm2(xh, xhl, rs, w, y, M, N, K, C, DT, tile == 513 ? 1 : 0, s);
     if (rc != KQ_ERR_UNSUPPORTED) return rc;
   }
-  if (tile == 512 || tile == 513 || tile == 1024) tile = 0;
+  if (tile == 512 || tile == 513 || tile == 1024 || tile == 1025) tile = 0;
   if (tile == 256 && C != KQ_Q4_K) tile = 0;
   if (tile == 0) {
     const int64_t wgs = (int64_t)((M + 63) / 64) * ((N + 255) / 256);
@@ -373,5 +405,5 @@ int kq_launch_act_prepass(const void* x, void* xh, void* xhl, float* rs, int M, 
 }
 
 extern "C" void kq_set_gemm_tile_rows(int rows) {
-  g_gemm_tile = (rows == 64 || rows == 128 || rows == 256 || rows == 512 || rows == 513 || rows == 1024) ? rows : 0;
+  g_gemm_tile = (rows == 64 || rows == 128 || rows == 256 || rows == 512 || rows == 513 || rows == 1024 || rows == 1025) ? rows : 0;
 }

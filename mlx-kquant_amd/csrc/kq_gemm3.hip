@@ -322,21 +322,269 @@ int launch_gemm3(const _Float16* xh, const _Float16* xhl, const float* rs, const
   return KQ_OK;
 }
 
+
+// ------------------------------------------------------------------ q6_k
+// Same tile, same activation pipeline.  A q6_k weight sc (q - 32) reaches 4096 and goes in as two exact terms,
+// sc ql and 16 sc (qh - 2), so a decoded fragment feeds sixteen MFMAs.  There is no minimum term: entering a
+// superblock only changes the unit of the running sums.  Two superblock stages of 32 rows do not fit beside the
+// activation stages, so the wire bytes travel by half superblocks (128 weights: 64 bytes of ql, 32 of qh, the
+// scale piece, d) into two slots per wave: half h is consumed in K steps 2 h and 2 h + 1 from registers filled in
+// step 2 h - 1, so its slot takes half h + 2 in step 2 h.
+constexpr int Q6_SLOT_QH = 2048, Q6_SLOT_SC = 3072, Q6_SLOT_D = 3584, Q6_SLOT = 3712;
+constexpr int Q6_W_INSTR = 5;  // load instructions per half: ql 2, qh 1, scales 1, d 1
+template <int MT>
+constexpr int g3_q6_lds_bytes() { return 2 * (32 * MT * G3_KS * 2) + G3_WAVES * 2 * Q6_SLOT; }
+
+// MT = 8: 256 x 256 tiles; MT = 4: 128 x 256 tiles (a decoded fragment feeds eight MFMAs) for the column tiles
+// that do not fill a round of one workgroup per CU.
+template <int DT, int MT>
+__global__ __launch_bounds__(64 * G3_WAVES, 1) void kquant_gemm3_q6k_kernel(const _Float16* __restrict__ xh,
+                                                                           const float* __restrict__ rs,
+                                                                           const uint8_t* __restrict__ w,
+                                                                           uint16_t* __restrict__ y, int M, int mrows,
+                                                                           int N, int K, int mtiles, int nt0) {
+  constexpr int BPB = 210, TM = 32 * MT, A_STAGE = TM * G3_KS * 2, AQ = MT / 2;
+  constexpr int A_OFF = 0, W_OFF = 2 * A_STAGE;
+  constexpr int GPS = G3_KS / 16;   // MFMA groups per step: 4
+  constexpr int SPS = 256 / G3_KS;  // steps per superblock: 4
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, kg = lane >> 5;
+  const int mt = blockIdx.x % mtiles, nt = nt0 + blockIdx.x / mtiles;
+  const int m0 = mt * TM, n0 = nt * G3_BN;
+  const int nsb = K >> 8;
+  const uint32_t row_bytes = (uint32_t)nsb * BPB;
+  const int nrows = N - n0 < G3_BN ? N - n0 : G3_BN;
+  const uint32_t lds0 = lds_addr(smem);
+
+  // ---- load maps (activations as in the kernel above)
+  auto swz = [](int row) { return (row >> 1) & 7; };
+  uint32_t a_voff[AQ];
+#pragma unroll
+  for (int q = 0; q < AQ; q++) {
+    const int r = 8 * (wave + 8 * q) + (lane >> 3);
+    const int gr = m0 + r < mrows ? m0 + r : mrows - 1;
+    a_voff[q] = (uint32_t)gr * (uint32_t)K * 2u + 16u * (uint32_t)((lane & 7) ^ swz(r));
+  }
+  const uint8_t* a_base = reinterpret_cast<const uint8_t*>(xh);
+  // wire: a slot holds, for the wave's 32 rows, 64 bytes of ql (row-major, two load instructions), 32 bytes of qh
+  // (one), the 16 scale bytes (half an instruction) and d (half a 2-byte instruction, zero-extended dwords).  Rows
+  // past N re-read the last row (their columns are not stored).
+  auto wrow = [&](int r) -> uint32_t {
+    r += wave * 32;
+    return (uint32_t)(r < nrows ? r : nrows - 1) * row_bytes;
+  };
+  uint32_t v_ql[2];
+#pragma unroll
+  for (int q = 0; q < 2; q++) v_ql[q] = wrow((64 * q + lane) >> 2) + 16u * (uint32_t)(lane & 3);
+  const uint32_t v_qh = wrow(lane >> 1) + 128u + 16u * (uint32_t)(lane & 1);
+  const uint32_t v_sc = wrow(l32) + 192u;
+  const uint8_t* w_base = w + (size_t)n0 * row_bytes;
+
+  auto issue_a = [&](int step) {
+    const uint8_t* base = a_base + (size_t)step * (G3_KS * 2);
+    const uint32_t l = lds0 + A_OFF + (step & 1) * A_STAGE + wave * 1024;
+#pragma unroll
+    for (int q = 0; q < AQ; q++) dma16(base, a_voff[q], l + q * (G3_WAVES * 1024));
+  };
+  const uint32_t w_lds = lds0 + W_OFF + wave * (2 * Q6_SLOT);
+  auto issue_w = [&](int half) {  // half superblock `half` of this wave's rows -> slot half % 2
+    const uint8_t* base = w_base + (size_t)(half >> 1) * BPB;
+    const uint32_t hf = half & 1, l = w_lds + hf * Q6_SLOT;
+    dma16(base + 64 * hf, v_ql[0], l);
+    dma16(base + 64 * hf, v_ql[1], l + 1024);
+    dma16(base + 32 * hf, v_qh, l + Q6_SLOT_QH);
+    if (lane < 32) {
+      dma16(base, v_sc, l + Q6_SLOT_SC);
+      dma2(base, v_sc + 16u, l + Q6_SLOT_D);
+    }
+  };
+
+  uint32_t a_addr[GPS];
+#pragma unroll
+  for (int g = 0; g < GPS; g++)
+    a_addr[g] = (uint32_t)l32 * 128u + 16u * (uint32_t)((4 * (g >> 1) + 2 * kg + (g & 1)) ^ swz(l32));
+  const uint8_t* slot0 = smem + W_OFF + wave * (2 * Q6_SLOT);
+
+  f32x16 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; t++) acc[t] = f32x16{0};
+
+  const uint32_t magic = opaque_vgpr(0x64006400u);
+  const uint32_t mask_q = opaque_sgpr(0x00f000f0u), mask_h = opaque_sgpr(0x03000300u);
+
+  // ---- this lane's weight row: registers of the half in hand
+  struct Half {
+    uint4 ql[2];      // ql[64 hf + 32 qr + 16 kg ..+15], qr = 0, 1
+    uint4 qh;         // qh[32 hf + 16 kg ..+15]
+    uint32_t scw[2];  // the half's eight int8 scales (zeros when d = 0: the half is fed as zeros)
+  };
+  float r = 1.0f, ratio = 1.0f;  // unit of the running sums; r_old / r_new of the superblock being entered
+  // `first`: the half opens a superblock (its d changes the unit); commit = false leaves r alone (a dry run past K)
+  auto load_half = [&](int hf, bool first, bool commit) -> Half {
+    const uint8_t* sl = slot0 + hf * Q6_SLOT;
+    Half hv;
+    hv.ql[0] = *reinterpret_cast<const uint4*>(sl + l32 * 64 + 16 * kg);
+    hv.ql[1] = *reinterpret_cast<const uint4*>(sl + l32 * 64 + 32 + 16 * kg);
+    hv.qh = *reinterpret_cast<const uint4*>(sl + Q6_SLOT_QH + l32 * 32 + 16 * kg);
+    const uint2 sc = *reinterpret_cast<const uint2*>(sl + Q6_SLOT_SC + l32 * 16 + 8 * hf);
+    const float d = kq::h2f((uint16_t)(*reinterpret_cast<const uint32_t*>(sl + Q6_SLOT_D + l32 * 4) & 0xffff));
+    hv.scw[0] = d != 0.f ? sc.x : 0u;
+    hv.scw[1] = d != 0.f ? sc.y : 0u;
+    if (first) {
+      const float rn = d != 0.f ? d : r;  // a superblock with d = 0 keeps the unit
+      ratio = r * __builtin_amdgcn_rcpf(rn);
+      r = commit ? rn : r;
+    }
+    return hv;
+  };
+
+  // B fragments of MFMA group g of step p of a superblock: sub-block 32 t4 .. + 31 of the half with t4 = g / 2 +
+  // 2 (p % 2) (low nibbles of the ql bytes in the half's first step, high nibbles in its second), K-half s = g % 2
+  auto decode = [&](auto pc, auto gc, const Half& hv, f16x8& blo, f16x8& bhi) {
+    constexpr int p = decltype(pc)::value, g = decltype(gc)::value;
+    constexpr int h = p & 1, qr = g >> 1, s = g & 1, t4 = qr + 2 * h;
+    const uint32_t qw[4] = {hv.ql[qr].x, hv.ql[qr].y, hv.ql[qr].z, hv.ql[qr].w};
+    const uint32_t hw[4] = {hv.qh.x, hv.qh.y, hv.qh.z, hv.qh.w};
+    const int sc = __builtin_amdgcn_sbfe((int)hv.scw[t4 >> 1], 8 * (2 * (t4 & 1) + kg), 8);
+    const float scf = (float)sc;
+    const _Float16 sch = (_Float16)(scf * 0.0625f), ofl = (_Float16)(-64.0f * scf), ofh = (_Float16)(-96.0f * scf);
+    const f16x2 scp = {sch, sch}, oflp = {ofl, ofl}, ofhp = {ofh, ofh};
+    uint32_t fl[4], fh[4];
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+      const uint32_t q = qw[2 * s + e], hq = hw[2 * s + e];
+      const uint32_t qe = h ? q : (q << 4), qo = h ? (q >> 8) : (q >> 4);
+      const uint32_t he = hq << (8 - 2 * t4), ho = t4 ? (hq >> (2 * t4)) : hq;
+      fl[2 * e] = (qe & mask_q) | magic;      // bytes 0, 2 of the word: 1024 + 16 ql
+      fl[2 * e + 1] = (qo & mask_q) | magic;  // bytes 1, 3
+      fh[2 * e] = (he & mask_h) | magic;      // 1024 + 256 qh
+      fh[2 * e + 1] = (ho & mask_h) | magic;
+    }
+    f16x2 bl2[4], bh2[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      // (1024 + 16 ql) sc / 16 - 64 sc = sc ql;  (1024 + 256 qh) sc / 16 - 96 sc = 16 sc (qh - 2)
+      bl2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fl[e]), scp, oflp);
+      bh2[e] = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, fh[e]), scp, ofhp);
+    }
+    blo = f16x8{bl2[0][0], bl2[0][1], bl2[1][0], bl2[1][1], bl2[2][0], bl2[2][1], bl2[3][0], bl2[3][1]};
+    bhi = f16x8{bh2[0][0], bh2[0][1], bh2[1][0], bh2[1][1], bh2[2][0], bh2[2][1], bh2[3][0], bh2[3][1]};
+  };
+
+  // ---- prologue: first loads, registers of half 0, its first fragment
+  const int nhalves = 2 * nsb, nsteps = SPS * nsb;
+  issue_a(0);
+  issue_w(0);
+  issue_w(1);
+  vmwait<Q6_W_INSTR>();  // own wire bytes of half 0 (and everything older) have landed
+  Half cur = load_half(0, true, true);
+  Half nxt = cur;
+  f16x8 blo[2], bhi[2];
+  decode(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, cur, blo[0], bhi[0]);
+
+  // ---- main loop: step s = 4 sb + p.  The activation loads of step s + 1 are queued right after the barrier that
+  // opens step s; half h + 2 follows in the first step of half h and may stay in flight over the next barrier.
+  for (int sb = 0; sb < nsb; sb++) {
+    const bool more = sb + 1 < nsb;
+    StaticFor<SPS>::run([&](auto pc) {
+      constexpr int p = decltype(pc)::value;
+      constexpr int hf = p >> 1;
+      const int step = SPS * sb + p, half = 2 * sb + hf;
+      const uint8_t* a_stage = smem + A_OFF + (p & 1) * A_STAGE;
+      // own loads of this step's activations have landed; a half queued after them may stay in flight
+      if ((p & 1) && half + 2 < nhalves) vmwait<Q6_W_INSTR>(); else vmwait<0>();
+      lds_barrier();
+      if (step + 1 < nsteps) issue_a(step + 1);
+      if (!(p & 1) && half + 2 < nhalves) issue_w(half + 2);
+      f16x8 afr[MT];
+#pragma unroll
+      for (int t = 0; t < MT; t++) afr[t] = *reinterpret_cast<const f16x8*>(a_stage + a_addr[0] + t * 4096);
+      StaticFor<GPS>::run([&](auto gc) {
+        constexpr int g = decltype(gc)::value;
+        // registers of the next half, from its slot (own loads, landed before the barrier that opened this step;
+        // past the end: a harmless re-read)
+        if constexpr ((p & 1) && g == GPS - 2) nxt = load_half(hf ^ 1, p == SPS - 1, more);
+        // B fragments of the next group: of this step, of the half's second step, or of the next half
+        if constexpr (g + 1 < GPS)
+          decode(pc, std::integral_constant<int, g + 1>{}, cur, blo[(g + 1) & 1], bhi[(g + 1) & 1]);
+        else if constexpr (!(p & 1))
+          decode(std::integral_constant<int, p + 1>{}, std::integral_constant<int, 0>{}, cur, blo[0], bhi[0]);
+        else
+          decode(std::integral_constant<int, (p + 1) % SPS>{}, std::integral_constant<int, 0>{}, nxt, blo[0], bhi[0]);
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[t], blo[g & 1], acc[t], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[t], bhi[g & 1], acc[t], 0, 0, 0);
+          if constexpr (g + 1 < GPS) afr[t] = *reinterpret_cast<const f16x8*>(a_stage + a_addr[g + 1] + t * 4096);
+        }
+      });
+      if constexpr (p & 1) cur = nxt;
+      if constexpr (p == SPS - 1) {
+        if (more) {  // the running sums change unit
+#pragma unroll
+          for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[t][i] *= ratio;
+        }
+      }
+    });
+  }
+
+  const int n = n0 + wave * 32 + l32;
+#pragma unroll
+  for (int t = 0; t < MT; t++) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int m = m0 + t * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
+      if (m < M && n < N) {
+        const float v = acc[t][i] * r * rs[m];
+        y[(size_t)m * N + n] = DT == KQ_F16 ? kq::f2f16(v) : kq::f2bf16(v);
+      }
+    }
+  }
+}
+
+template <int DT, int MT>
+int launch_gemm3_q6k(const _Float16* xh, const float* rs, const uint8_t* w, void* y, int M, int mrows, int N, int K,
+                     int nt0, int ntiles, hipStream_t s) {
+  const int mtiles = (M + 32 * MT - 1) / (32 * MT);
+  constexpr int lds = g3_q6_lds_bytes<MT>();
+  static_assert(lds <= 160 * 1024, "tile does not fit the LDS of a CU");
+  auto kern = kquant_gemm3_q6k_kernel<DT, MT>;
+  KQ_SET_MAX_LDS_ONCE((kern), lds);
+  hipLaunchKernelGGL(kern, dim3(mtiles * ntiles), dim3(64 * G3_WAVES), lds, s, xh, rs, w, static_cast<uint16_t*>(y), M,
+                     mrows, N, K, mtiles, nt0);
+  KQ_HIP_CHECK(hipGetLastError());
+  return KQ_OK;
+}
+
 }  // namespace
 
 bool kq_gemm3_supported(int M, int mrows, int N, int K, int codec) {
-  return (codec == KQ_Q4_K || codec == KQ_Q5_K) && M >= 64 && mrows >= M && K >= 256 && (K & 255) == 0 && N > 0 &&
-         (int64_t)256 * (K >> 8) * 176 < ((int64_t)1 << 32) && (int64_t)mrows * K * 2 < ((int64_t)1 << 32);
+  return (codec == KQ_Q4_K || codec == KQ_Q5_K || codec == KQ_Q6_K) && M >= 64 && mrows >= M && K >= 256 && (K & 255) == 0 &&
+         N > 0 && (int64_t)256 * (K >> 8) * 210 < ((int64_t)1 << 32) && (int64_t)mrows * K * 2 < ((int64_t)1 << 32);
 }
 
 // Column tiles nt0 .. nt0 + ntiles - 1 (256 weight rows each) of y = x . W^T; xh / xhl / rs: outputs of the
-// activation prepass with mrows >= M prepared rows.
+// activation prepass with mrows >= M prepared rows (q6_k has no minimum term and reads no xhl; tile_rows = 128
+// selects its 128-row form, any other value the 256-row tiles).
 int kq_launch_gemm3(const void* xh, const void* xhl, const float* rs, const uint8_t* w, void* y, int M, int mrows, int N,
-                    int K, int codec, int dtype, int nt0, int ntiles, hipStream_t s) {
+                    int K, int codec, int dtype, int nt0, int ntiles, hipStream_t s, int tile_rows) {
   if (!kq_gemm3_supported(M, mrows, N, K, codec)) return KQ_ERR_UNSUPPORTED;
   if (ntiles <= 0) return KQ_OK;
   const _Float16* a = static_cast<const _Float16*>(xh);
   const _Float16* h = static_cast<const _Float16*>(xhl);
+  if (codec == KQ_Q6_K) {
+    if (tile_rows == 128)
+      return dtype == KQ_F16 ? launch_gemm3_q6k<KQ_F16, 4>(a, rs, w, y, M, mrows, N, K, nt0, ntiles, s)
+                             : launch_gemm3_q6k<KQ_BF16, 4>(a, rs, w, y, M, mrows, N, K, nt0, ntiles, s);
+    return dtype == KQ_F16 ? launch_gemm3_q6k<KQ_F16, 8>(a, rs, w, y, M, mrows, N, K, nt0, ntiles, s)
+                           : launch_gemm3_q6k<KQ_BF16, 8>(a, rs, w, y, M, mrows, N, K, nt0, ntiles, s);
+  }
   if (codec == KQ_Q4_K)
     return dtype == KQ_F16 ? launch_gemm3<KQ_Q4_K, KQ_F16>(a, h, rs, w, y, M, mrows, N, K, nt0, ntiles, s)
                            : launch_gemm3<KQ_Q4_K, KQ_BF16>(a, h, rs, w, y, M, mrows, N, K, nt0, ntiles, s);

@@ -65,6 +65,13 @@ def test_config3_prefill_8192_to_28672(kq, codec, M):
     _check_matmul(kq, codec, M, 28672, 8192, "bfloat16", 74, 48)
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 28672, 8192), (512, 28672, 8192), (1024, 8192, 8192), (1024, 4096, 14336)])
+def test_prefill_q6k_tile_choice(kq, M, N, K):
+    """q6_k prefill through the automatic tile choice: whole rounds of 256-row tiles plus a round of 128-row tiles,
+    256-row tiles alone, 128-row tiles alone, and the 64-row kernel for a matrix of few tiles."""
+    _check_matmul(kq, "q6_k", M, N, K, "bfloat16", 90, 48)
+
+
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
 @pytest.mark.parametrize("codec", ["q2_k", "q3_k", "iq4_xs"])
 @pytest.mark.parametrize("M,N,K", [(2048, 28672, 8192), (300, 16400, 512), (256, 32768, 256)])

@@ -377,6 +377,37 @@ def test_qmm_prefill_gemm_128x256_tiles(kq, codec):
         lib.kq_set_gemm_tile_rows(0)
 
 
+def test_qmm_prefill_q6k_tall_tiles(kq):
+    """q6_k on the 256-row and 128-row tiles of the unit-chain kernel (kq_set_gemm_tile_rows(1024 / 1025); two exact
+    terms per weight, wire bytes by half superblocks): one, two, four and nine superblocks of K, ragged M and N tiles,
+    fewer rows than a tile, both activation dtypes, and the automatic choice; then a matrix whose blocks hold d = 0,
+    negative d and the extreme scales -128 / 127 (products of 4096 that one f16 term could not hold)."""
+    lib = kq._load()
+    try:
+        for rows in (1024, 1025, 0):
+            lib.kq_set_gemm_tile_rows(rows)
+            for M, N, K, dtype in ((64, 40, 256, "bfloat16"), (130, 257, 512, "float16"), (300, 520, 2304, "bfloat16"),
+                                   (256, 256, 1024, "bfloat16"), (513, 700, 1024, "float16")):
+                wire = _wire("q6_k", N, K, seed=66)
+                xb, xt = make_x((M, K), dtype, seed=67)
+                got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, "q6_k"))
+                want = O.qmm(xb, wire, "q6_k", True, dtype)
+                assert rel_l2(got, want, dtype) <= TOL, (rows, M, N, K, dtype)
+            M, N, K = 270, 300, 1024
+            wire = _wire("q6_k", N, K, seed=68).copy()
+            blocks = wire.reshape(N, K // 256, 210)
+            blocks[::3, ::2, 208:210] = 0          # d = 0: the block keeps the unit of the running sums
+            blocks[1::3, :, 209] |= 0x80           # negative d
+            blocks[:, 1::2, 192:208] = np.tile(np.array([0x80, 0x7f], np.uint8), 8)
+            blocks[:, 1::2, 0:192:7] = 0x00        # q = 0 -> (q - 32) = -32 against scale -128
+            xb, xt = make_x((M, K), "bfloat16", seed=69)
+            got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, "q6_k"))
+            want = O.qmm(xb, wire, "q6_k", True, "bfloat16")
+            assert rel_l2(got, want, "bfloat16") <= TOL, (rows, "special blocks")
+    finally:
+        lib.kq_set_gemm_tile_rows(0)
+
+
 @pytest.mark.parametrize("codec", ["q4_k", "q5_k"])
 def test_qmm_prefill_gemm_256x256_tiles(kq, codec):
     """The 256-row kernel (kq_set_gemm_tile_rows(1024): running sums kept in units of the current superblock scale):
