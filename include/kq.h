@@ -110,9 +110,11 @@ int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void
  * activation rows x 128 weight rows, 128 = 128 x 128, 256 = 64 x 256 on eight waves with two LDS stages
  * (q4_k only; other codecs fall back to automatic), 512 = 128 x 256 on eight waves with 128-row wave tiles and
  * direct-to-LDS loads (q2_k / q3_k / q4_k / q5_k / iq4_xs; 513 = the same kernel as 128 x 128 on four waves),
- * 1024 = 256 x 256 on eight waves with 256-row wave tiles on one accumulator set (q4_k / q5_k) for every column
- * tile; anything else restores the automatic choice (q4_k / q5_k with 256 rows or more: the 256 x 256 kernel on the
- * column tiles that fill whole rounds of one workgroup per CU, the 128 x 256 kernel on the rest).
+ * 1024 = 256 x 256 on eight waves with 256-row wave tiles on one accumulator set (q4_k / q5_k / q6_k) for every
+ * column tile, 1025 = the 128 x 256 form of that kernel (q6_k only; other codecs fall back to automatic);
+ * anything else restores the automatic choice (q4_k / q5_k / q6_k with 256 rows or more: the 256 x 256 kernel on the
+ * column tiles that fill whole rounds of one workgroup per CU, a 128 x 256 kernel on the rest; q6_k matrices of
+ * few tiles stay on the 64-row kernel).
  * Process-wide, not thread-safe. */
 void kq_set_gemm_tile_rows(int rows);
 /* Tuning hook without a counterpart in the reference: which skinny-M kernel dense calls use.
