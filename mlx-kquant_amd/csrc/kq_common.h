@@ -152,6 +152,13 @@ int kq_launch_gemm2(const void* xh, const void* xhl, const float* rs, const uint
 bool kq_gemm3_supported(int M, int mrows, int N, int K, int codec);
 int kq_launch_gemm3(const void* xh, const void* xhl, const float* rs, const uint8_t* w, void* y, int M, int mrows, int N,
                     int K, int codec, int dtype, int nt0, int ntiles, hipStream_t s, int tile_rows = 256);
+// 256-row / 128-row wave tiles for the 32-weight-block codecs with an f16 scale (q8_0, q4_0): every weight as two
+// exact f16 terms (kq_gemm3b.hip).  Runs its own activation prepass into ws (kq_gemm3b_workspace_bytes).
+bool kq_gemm3b_supported(int M, int N, int K, int codec);
+size_t kq_gemm3b_workspace_bytes(int M, int K);
+void kq_gemm3b_force_tile(int rows);
+int kq_launch_gemm3b(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                     hipStream_t s);
 // The same tile kernel for q2_k / q3_k (M >= 256, tiles filling the chip): runs its own activation prepass.
 bool kq_gemm2_low_supported(int M, int N, int K, int codec);
 size_t kq_gemm2_low_workspace_bytes(int M, int K);

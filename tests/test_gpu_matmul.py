@@ -377,6 +377,46 @@ def test_qmm_prefill_gemm_128x256_tiles(kq, codec):
         lib.kq_set_gemm_tile_rows(0)
 
 
+@pytest.mark.parametrize("codec", ["q8_0", "q4_0"])
+def test_qmm_prefill_block32_tall_tiles(kq, codec):
+    """q8_0 / q4_0 on the 256-row and 128-row tiles (every weight d q as two exact f16 terms, wire bytes step by step
+    through a ring of four slots): one to forty-five K steps of 64 (prologue only, ring wrap, K = 2880), ragged M and N
+    tiles, both activation dtypes; blocks with d = 0, negative, subnormal and large d and the extreme codes; and the
+    automatic choice on a matrix wide enough to be taken."""
+    lib = kq._load()
+    wpb, bpb = O.geometry(codec)
+    try:
+        for rows in (1024, 1025):
+            lib.kq_set_gemm_tile_rows(rows)
+            for M, N, K, dtype in ((128, 40, 64, "bfloat16"), (130, 257, 192, "float16"), (300, 520, 2880, "bfloat16"),
+                                   (256, 256, 320, "bfloat16"), (513, 700, 1024, "float16")):
+                wire = _wire(codec, N, K, seed=71)
+                xb, xt = make_x((M, K), dtype, seed=72)
+                got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+                want = O.qmm(xb, wire, codec, True, dtype)
+                assert rel_l2(got, want, dtype) <= TOL, (codec, rows, M, N, K, dtype)
+            M, N, K = 140, 300, 512
+            wire = _wire(codec, N, K, seed=73).copy()
+            blocks = wire.reshape(N, K // wpb, bpb)
+            blocks[::5, ::2, 0:2] = 0                                         # d = 0
+            blocks[1::5, :, 1] |= 0x80                                        # negative d
+            blocks[2::5, 1::2, 0:2] = np.array([0x37, 0x00], np.uint8)        # subnormal d (55 x 2^-24)
+            blocks[3::5, ::3, 0:2] = np.frombuffer(np.float16(200.0).tobytes(), np.uint8)
+            blocks[:, 1::4, 2:bpb:3] = 0x80 if codec == "q8_0" else 0x0f      # q = -128 / nibbles 15 and 0
+            xb, xt = make_x((M, K), "bfloat16", seed=74)
+            got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+            want = O.qmm(xb, wire, codec, True, "bfloat16")
+            assert rel_l2(got, want, "bfloat16") <= TOL, (codec, rows, "special blocks")
+        lib.kq_set_gemm_tile_rows(0)
+        M, N, K = 256, 24600, 128
+        wire = _wire(codec, N, K, seed=75)
+        xb, xt = make_x((M, K), "float16", seed=76)
+        got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+        assert rel_l2(got, O.qmm(xb, wire, codec, True, "float16"), "float16") <= TOL, (codec, "automatic")
+    finally:
+        lib.kq_set_gemm_tile_rows(0)
+
+
 def test_qmm_prefill_q6k_tall_tiles(kq):
     """q6_k on the 256-row and 128-row tiles of the unit-chain kernel (kq_set_gemm_tile_rows(1024 / 1025); two exact
     terms per weight, wire bytes by half superblocks): one, two, four and nine superblocks of K, ragged M and N tiles,
