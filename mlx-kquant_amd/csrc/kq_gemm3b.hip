@@ -1,4 +1,4 @@
-// Prefill GEMM for the 32-weight-block codecs whose weight is (f16 scale) x (small integer): q8_0, q4_0.
+// Prefill GEMM for the 32-weight-block codecs whose weight is (f16 scale) x (small integer): q8_0, q4_0, iq4_nl.
 // y[M,N] = x[M,K] . W^T on the f16 matrix cores, 256-row (or 128-row) wave tiles, exact in the weights.
 //
 // A block's scale d is not an integer, so the exact-integer operands of the K-quant kernels do not apply, and a
@@ -36,6 +36,10 @@ struct B32<KQ_Q8_0> {
 template <>
 struct B32<KQ_Q4_0> {
   static constexpr int BPB = 18, QB = 16;
+};
+template <>
+struct B32<KQ_IQ4_NL> {
+  static constexpr int BPB = 18, QB = 16;  // as q4_0, the nibble indexing a table of sixteen int8 values
 };
 
 template <int C>
@@ -181,11 +185,16 @@ __global__ __launch_bounds__(64 * B3_WAVES, 1) void block32_gemm3_kernel(const _
   for (int t = 0; t < MT; t++) acc[t] = f32x16{0};
 
   const uint32_t magic = opaque_vgpr(0x64006400u);
-  const uint32_t mask_b = opaque_sgpr(C == KQ_Q8_0 ? 0x00ff00ffu : 0x000f000fu);
+  const uint32_t mask_b = opaque_sgpr(C == KQ_Q4_0 ? 0x000f000fu : 0x00ff00ffu);
+  // iq4_nl: the sixteen table values + 128 as bytes (entries 0 - 3, 4 - 7, 8 - 11, 12 - 15), looked up four at a time
+  // with byte permutes: low three bits select inside each half, the fourth bit selects the half
+  const uint32_t kv0 = opaque_sgpr(0x3f2d1801u), kv1 = opaque_sgpr(0x766a5d4fu), kv2 = opaque_sgpr(0xa6998d81u),
+                 kv3 = opaque_sgpr(0xf1d9c5b5u);
+  (void)kv0; (void)kv1; (void)kv2; (void)kv3;
 
   // ---- this lane's weight row: registers of the step in hand
   struct Regs {
-    uint4 q[2];     // q8_0: bytes 16 kg .. + 15 of the block; q4_0: its 16 bytes (this lane takes nibble kg)
+    uint4 q[2];     // q8_0: bytes 16 kg .. + 15 of the block; q4_0 / iq4_nl: its 16 bytes (this lane takes nibble kg)
     uint32_t d[2];  // f16 scale of the block, in both halves of the dword
   };
   auto load_regs = [&](int slot) -> Regs {
@@ -209,13 +218,22 @@ __global__ __launch_bounds__(64 * B3_WAVES, 1) void block32_gemm3_kernel(const _
     constexpr int g = decltype(gc)::value, b = g >> 1, s = g & 1;
     const uint32_t qw[4] = {rg.q[b].x, rg.q[b].y, rg.q[b].z, rg.q[b].w};
     const f16x2 dp = __builtin_bit_cast(f16x2, rg.d[b]);
-    // q8_0: byte ^ 0x80 = q + 128, 0x6400 | that = 1024 + 128 + q; q4_0: 0x6400 | nibble = 1024 + 8 + (n - 8)
-    const f16x2 off = C == KQ_Q8_0 ? f16x2{(_Float16)-1152.0f, (_Float16)-1152.0f} : f16x2{(_Float16)-1032.0f, (_Float16)-1032.0f};
+    // q8_0: byte ^ 0x80 = q + 128, 0x6400 | that = 1024 + 128 + q (iq4_nl: the table holds value + 128);
+    // q4_0: 0x6400 | nibble = 1024 + 8 + (n - 8)
+    const f16x2 off = C == KQ_Q4_0 ? f16x2{(_Float16)-1032.0f, (_Float16)-1032.0f} : f16x2{(_Float16)-1152.0f, (_Float16)-1152.0f};
     f16x2 h2[4], l2[4];
 #pragma unroll
     for (int e = 0; e < 2; e++) {
       uint32_t x = qw[2 * s + e];
-      if constexpr (C == KQ_Q8_0) x ^= 0x80808080u; else x >>= 4 * kg;
+      if constexpr (C == KQ_Q8_0) {
+        x ^= 0x80808080u;
+      } else if constexpr (C == KQ_Q4_0) {
+        x >>= 4 * kg;
+      } else {
+        const uint32_t nib = (x >> (4 * kg)) & 0x0f0f0f0fu, low3 = nib & 0x07070707u;
+        const uint32_t half0 = __builtin_amdgcn_perm(kv1, kv0, low3), half1 = __builtin_amdgcn_perm(kv3, kv2, low3);
+        x = __builtin_amdgcn_perm(half1, half0, ((nib >> 1) & 0x04040404u) | 0x03020100u);
+      }
       const uint32_t fe = (x & mask_b) | magic, fo = ((x >> 8) & mask_b) | magic;  // bytes 0, 2 / bytes 1, 3
       const f16x2 qe = __builtin_bit_cast(f16x2, fe) + off, qo = __builtin_bit_cast(f16x2, fo) + off;
       h2[2 * e] = qe * dp;
@@ -345,7 +363,7 @@ int launch_b3_call(const void* x, const uint8_t* w, void* y, int M, int N, int K
 // Taken for calls of 128 rows or more whose half-height tiles fill three quarters of the CUs; smaller calls stay on
 // the any-codec kernel (small workgroups, K cut over the grid).
 bool kq_gemm3b_supported(int M, int N, int K, int codec) {
-  if (codec != KQ_Q8_0 && codec != KQ_Q4_0) return false;
+  if (codec != KQ_Q8_0 && codec != KQ_Q4_0 && codec != KQ_IQ4_NL) return false;
   if (M < 128 || N <= 0 || K < 64 || (K & 63)) return false;
   const int64_t row_bytes = (int64_t)(K >> 5) * (codec == KQ_Q8_0 ? 34 : 18);
   if (256 * row_bytes >= ((int64_t)1 << 32) || (int64_t)M * K * 2 >= ((int64_t)1 << 32)) return false;
@@ -366,6 +384,9 @@ int kq_launch_gemm3b(const void* x, const uint8_t* w, void* y, int M, int N, int
   if (codec == KQ_Q8_0)
     return dtype == KQ_F16 ? launch_b3_call<KQ_Q8_0, KQ_F16>(x, w, y, M, N, K, ws, force, s)
                            : launch_b3_call<KQ_Q8_0, KQ_BF16>(x, w, y, M, N, K, ws, force, s);
+  if (codec == KQ_IQ4_NL)
+    return dtype == KQ_F16 ? launch_b3_call<KQ_IQ4_NL, KQ_F16>(x, w, y, M, N, K, ws, force, s)
+                           : launch_b3_call<KQ_IQ4_NL, KQ_BF16>(x, w, y, M, N, K, ws, force, s);
   return dtype == KQ_F16 ? launch_b3_call<KQ_Q4_0, KQ_F16>(x, w, y, M, N, K, ws, force, s)
                          : launch_b3_call<KQ_Q4_0, KQ_BF16>(x, w, y, M, N, K, ws, force, s);
 }
