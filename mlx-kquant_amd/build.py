@@ -28,6 +28,7 @@ SOURCES = [
     ("kq_gemm2.hip", ["-Wno-inline-asm"]),
     ("kq_gemm3.hip", ["-Wno-inline-asm"]),
     ("kq_gemm3b.hip", ["-Wno-inline-asm"]),
+    ("kq_gemm3f.hip", ["-Wno-inline-asm"]),
     ("kq_moe.hip", []),
     ("kq_anymma.hip", ["-ffp-contract=off"]),
     # one source, three objects: its kernel families are instantiated in parallel

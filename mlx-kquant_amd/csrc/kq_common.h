@@ -159,6 +159,13 @@ size_t kq_gemm3b_workspace_bytes(int M, int K);
 void kq_gemm3b_force_tile(int rows);
 int kq_launch_gemm3b(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                      hipStream_t s);
+// The same tiles for the fp4 codecs (mxfp4, nvfp4): one exact f16 term per weight, converted from the wire nibbles by
+// the hardware's fp4 -> f16 instruction (kq_gemm3f.hip).  Runs its own activation prepass into ws.
+bool kq_gemm3f_supported(int M, int N, int K, int codec);
+size_t kq_gemm3f_workspace_bytes(int M, int K);
+void kq_gemm3f_force_tile(int rows);
+int kq_launch_gemm3f(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                     hipStream_t s);
 // The same tile kernel for q2_k / q3_k (M >= 256, tiles filling the chip): runs its own activation prepass.
 bool kq_gemm2_low_supported(int M, int N, int K, int codec);
 size_t kq_gemm2_low_workspace_bytes(int M, int K);

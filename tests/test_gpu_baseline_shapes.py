@@ -65,6 +65,14 @@ def test_config3_prefill_8192_to_28672(kq, codec, M):
     _check_matmul(kq, codec, M, 28672, 8192, "bfloat16", 74, 48)
 
 
+@pytest.mark.parametrize("codec", ["mxfp4", "nvfp4"])
+@pytest.mark.parametrize("M,N,K,dtype", [(2048, 28672, 8192, "bfloat16"), (512, 28672, 2880, "float16")])
+def test_prefill_fp4_tile_choice(kq, codec, M, N, K, dtype):
+    """mxfp4 / nvfp4 prefill through the automatic tile choice of the single-term kernel (nvfp4 blocks hold 64
+    weights: K = 2880 is 45 of them)."""
+    _check_matmul(kq, codec, M, N, K, dtype, 94, 48)
+
+
 @pytest.mark.parametrize("codec", ["q8_0", "q4_0", "iq4_nl"])
 @pytest.mark.parametrize("M,N,K", [(2048, 28672, 8192), (512, 28672, 2880), (1024, 8192, 8192)])
 def test_prefill_block32_tile_choice(kq, codec, M, N, K):

@@ -377,6 +377,56 @@ def test_qmm_prefill_gemm_128x256_tiles(kq, codec):
         lib.kq_set_gemm_tile_rows(0)
 
 
+@pytest.mark.parametrize("codec", ["mxfp4", "nvfp4"])
+def test_qmm_prefill_fp4_tall_tiles(kq, codec):
+    """mxfp4 / nvfp4 on the 256-row and 128-row tiles (one exact f16 term per weight out of the hardware's fp4 -> f16
+    conversion): one to forty-five K steps of 64, ragged M and N tiles, both activation dtypes; then scale edge cases —
+    mxfp4 rows whose block exponents jump by tens of binades from step to step (the per-column exponent offset
+    moves and the running sums are rescaled), exponents 0 / 1 / 2, and nvfp4 scale bytes 0x00, 0x7f (both decode to
+    0), 0x80, 0xff and the subnormal scales 0x01 ... 0x07; and the automatic choice on a wide matrix."""
+    lib = kq._load()
+    wpb, bpb = O.geometry(codec)
+    try:
+        for rows in (1024, 1025):
+            lib.kq_set_gemm_tile_rows(rows)
+            for M, N, K, dtype in ((128, 40, 64, "bfloat16"), (130, 257, 192, "float16"), (300, 520, 2880, "bfloat16"),
+                                   (256, 256, 320, "bfloat16"), (513, 700, 1024, "float16")):
+                wire = _wire(codec, N, K, seed=81)
+                xb, xt = make_x((M, K), dtype, seed=82)
+                got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+                want = O.qmm(xb, wire, codec, True, dtype)
+                assert rel_l2(got, want, dtype) <= TOL, (codec, rows, M, N, K, dtype)
+            M, N, K = 140, 300, 768
+            wire = _wire(codec, N, K, seed=83).copy()
+            blocks = wire.reshape(N, K // wpb, bpb)
+            if codec == "mxfp4":
+                jumps = np.array([120, 122, 180, 170, 60, 75, 131, 104, 140, 150, 20, 1, 0, 2, 200, 190, 127, 127,
+                                  90, 117, 118, 91, 127, 100], np.uint8)
+                blocks[0::4, :, 0] = jumps[:K // wpb]
+                blocks[1::4, :, 0] = np.array([0, 1, 2, 1] * (K // wpb // 4), np.uint8)
+                blocks[2::4, ::3, 1:] = 0                                  # blocks of zero codes
+            else:
+                edge = np.array([0x00, 0x7f, 0x80, 0xff, 0x01, 0x02, 0x03, 0x04, 0x05, 0x06, 0x07, 0x08, 0x7e, 0x38,
+                                 0x40, 0x0f], np.uint8)
+                for r in range(0, N, 3):
+                    blocks[r, :, 0:4] = np.resize(np.roll(edge, r), (K // wpb, 4))
+            xb, xt = make_x((M, K), "bfloat16", seed=84)
+            got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+            want = O.qmm(xb, wire, codec, True, "bfloat16")
+            assert rel_l2(got, want, "bfloat16") <= TOL, (codec, rows, "scale edge cases")
+            # row by row as well: a row of tiny weights must not hide behind the large ones
+            per_row = [rel_l2(got[:, r:r + 1], want[:, r:r + 1], "bfloat16") for r in range(0, N, 7)]
+            assert max(per_row) <= TOL, (codec, rows, "scale edge cases, per weight row", max(per_row))
+        lib.kq_set_gemm_tile_rows(0)
+        M, N, K = 256, 24600, 128
+        wire = _wire(codec, N, K, seed=85)
+        xb, xt = make_x((M, K), "float16", seed=86)
+        got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+        assert rel_l2(got, O.qmm(xb, wire, codec, True, "float16"), "float16") <= TOL, (codec, "automatic")
+    finally:
+        lib.kq_set_gemm_tile_rows(0)
+
+
 @pytest.mark.parametrize("codec", ["q8_0", "q4_0", "iq4_nl"])
 def test_qmm_prefill_block32_tall_tiles(kq, codec):
     """q8_0 / q4_0 / iq4_nl on the 256-row and 128-row tiles (every weight d q as two exact f16 terms, wire bytes step by step
