@@ -1,4 +1,5 @@
-// Prefill GEMM for the 32-weight-block codecs whose weight is (f16 scale) x (small integer): q8_0, q4_0, iq4_nl.
+// Prefill GEMM for the 32-weight-block codecs whose weight is (f16 scale) x (small integer) [+ f16 minimum]: q8_0,
+// q4_0, iq4_nl, q5_0, q4_1, q5_1.
 // y[M,N] = x[M,K] . W^T on the f16 matrix cores, 256-row (or 128-row) wave tiles, exact in the weights.
 //
 // A block's scale d is not an integer, so the exact-integer operands of the K-quant kernels do not apply, and a
@@ -9,6 +10,8 @@
 // products of f16 numbers are exact in the f32 accumulator, so results differ from f32 arithmetic on the decoded
 // weights by summation order only.  (|d q| beyond the f16 range, 65504, is not representable this way; no quantizer
 // emits such scales.)  No per-block fold, no unit chain: 20 vector instructions decode eight weights for sixteen MFMAs.
+// q4_1 / q5_1 add the block minimum m, an f16 number, as a third term on a third MFMA (the reference rounds d q + m
+// to f32 once; the three-term sum is exact, the difference at most 2^-24 of the weight).
 //
 // Workgroup = 8 waves = 256 (MT = 8) or 128 (MT = 4) activation rows x 256 weight rows, one per CU, two waves per
 // SIMD.  K advances in steps of 64 (two blocks): two activation stages filled by the whole workgroup with
@@ -41,15 +44,33 @@ template <>
 struct B32<KQ_IQ4_NL> {
   static constexpr int BPB = 18, QB = 16;  // as q4_0, the nibble indexing a table of sixteen int8 values
 };
+template <>
+struct B32<KQ_Q4_1> {
+  static constexpr int BPB = 20, QB = 16;  // d, m, 16 quant bytes
+};
+template <>
+struct B32<KQ_Q5_0> {
+  static constexpr int BPB = 22, QB = 16;  // d, 32 fifth bits, 16 quant bytes
+};
+template <>
+struct B32<KQ_Q5_1> {
+  static constexpr int BPB = 24, QB = 16;  // d, m, 32 fifth bits, 16 quant bytes
+};
 
 template <int C>
 struct B3Geom : B32<C> {
   static constexpr int QP = 2 * B32<C>::QB / 16;   // 16-byte quant pieces per row and step
   static constexpr int Q_INSTR = 32 * QP / 64;     // load instructions for them
   static constexpr int SLOT_Q = 32 * 16 * QP;      // quant bytes of a slot (row-major, 16 QP bytes per row)
-  static constexpr int SLOT = SLOT_Q + 256;        // + the scales: 32 rows x 2 blocks as zero-extended dwords
+  // what stands in front of the quant bytes: a 2-byte scale (one 2-byte load per row and block, parked as a
+  // zero-extended dword), or more (minimum, fifth bits): then the block's first 16 bytes travel as a piece
+  static constexpr int HEAD = B32<C>::BPB - B32<C>::QB;
+  static constexpr bool HEAD16 = HEAD > 2;
+  static constexpr int SLOT = SLOT_Q + (HEAD16 ? 1024 : 256);
   static constexpr int W_INSTR = Q_INSTR + 1;
   static constexpr int STEP_BYTES = 2 * B32<C>::BPB;
+  static constexpr bool MIN = C == KQ_Q4_1 || C == KQ_Q5_1;   // weight = d q + m
+  static constexpr bool FIVE = C == KQ_Q5_0 || C == KQ_Q5_1;  // a fifth bit per weight
 };
 
 template <int C, int MT>
@@ -152,7 +173,7 @@ __global__ __launch_bounds__(64 * B3_WAVES, 1) void block32_gemm3_kernel(const _
 #pragma unroll
   for (int q = 0; q < G::Q_INSTR; q++) {
     const int i = 64 * q + lane, p = i % G::QP;
-    v_q[q] = wrow(i / G::QP) + (uint32_t)(G::BPB * (p / (G::QB / 16)) + 2 + 16 * (p % (G::QB / 16)));
+    v_q[q] = wrow(i / G::QP) + (uint32_t)(G::BPB * (p / (G::QB / 16)) + G::HEAD + 16 * (p % (G::QB / 16)));
   }
   const uint32_t v_d = wrow(lane >> 1) + (uint32_t)(G::BPB * (lane & 1));
   const uint8_t* w_base = w + (size_t)n0 * row_bytes;
@@ -169,7 +190,10 @@ __global__ __launch_bounds__(64 * B3_WAVES, 1) void block32_gemm3_kernel(const _
     const uint32_t l = w_lds + (step & (B3_SLOTS - 1)) * G::SLOT;
 #pragma unroll
     for (int q = 0; q < G::Q_INSTR; q++) dma16(base, v_q[q], l + q * 1024);
-    dma2(base, v_d, l + G::SLOT_Q);
+    if constexpr (G::HEAD16)
+      dma16(base, v_d, l + G::SLOT_Q);  // lane -> (row lane / 2, block lane % 2): 16 bytes each
+    else
+      dma2(base, v_d, l + G::SLOT_Q);
   };
 
   // A fragment of m-tile t, group g: lane half kg holds the weights 16 kg + 8 (g % 2) .. + 7 of block g / 2, i.e.
@@ -185,7 +209,7 @@ __global__ __launch_bounds__(64 * B3_WAVES, 1) void block32_gemm3_kernel(const _
   for (int t = 0; t < MT; t++) acc[t] = f32x16{0};
 
   const uint32_t magic = opaque_vgpr(0x64006400u);
-  const uint32_t mask_b = opaque_sgpr(C == KQ_Q4_0 ? 0x000f000fu : 0x00ff00ffu);
+  const uint32_t mask_b = opaque_sgpr(C == KQ_Q4_0 || C == KQ_Q4_1 ? 0x000f000fu : G::FIVE ? 0x001f001fu : 0x00ff00ffu);
   // iq4_nl: the sixteen table values + 128 as bytes (entries 0 - 3, 4 - 7, 8 - 11, 12 - 15), looked up four at a time
   // with byte permutes: low three bits select inside each half, the fourth bit selects the half
   const uint32_t kv0 = opaque_sgpr(0x3f2d1801u), kv1 = opaque_sgpr(0x766a5d4fu), kv2 = opaque_sgpr(0xa6998d81u),
@@ -194,8 +218,10 @@ __global__ __launch_bounds__(64 * B3_WAVES, 1) void block32_gemm3_kernel(const _
 
   // ---- this lane's weight row: registers of the step in hand
   struct Regs {
-    uint4 q[2];     // q8_0: bytes 16 kg .. + 15 of the block; q4_0 / iq4_nl: its 16 bytes (this lane takes nibble kg)
-    uint32_t d[2];  // f16 scale of the block, in both halves of the dword
+    uint4 q[2];      // q8_0: bytes 16 kg .. + 15 of the block; the nibble codecs: its 16 bytes (this lane takes nibble kg)
+    uint32_t d[2];   // f16 scale of the block, in both halves of the dword
+    uint32_t m[2];   // q4_1 / q5_1: f16 minimum of the block, in both halves
+    uint32_t qh[2];  // q5_0 / q5_1: the fifth bits of this lane's sixteen weights (bits 0 .. 15)
   };
   auto load_regs = [&](int slot) -> Regs {
     const uint8_t* sl = slot0 + slot * G::SLOT;
@@ -207,9 +233,22 @@ __global__ __launch_bounds__(64 * B3_WAVES, 1) void block32_gemm3_kernel(const _
       else
         rg.q[b] = *reinterpret_cast<const uint4*>(sl + l32 * 32 + 16 * b);
     }
-    const uint2 dd = *reinterpret_cast<const uint2*>(sl + G::SLOT_Q + l32 * 8);
-    rg.d[0] = dd.x | (dd.x << 16);
-    rg.d[1] = dd.y | (dd.y << 16);
+    if constexpr (G::HEAD16) {
+#pragma unroll
+      for (int b = 0; b < 2; b++) {
+        const uint2 hd = *reinterpret_cast<const uint2*>(sl + G::SLOT_Q + l32 * 32 + 16 * b);  // block bytes 0 .. 7
+        rg.d[b] = (hd.x & 0xffffu) | (hd.x << 16);
+        rg.m[b] = G::MIN ? (hd.x >> 16) | (hd.x & 0xffff0000u) : 0u;
+        // fifth bits: weight j of the block has bit j of the 32-bit field behind d (and m); this lane's are 16 kg ..
+        const uint32_t field = G::MIN ? hd.y : (hd.x >> 16) | (hd.y << 16);
+        rg.qh[b] = G::FIVE ? field >> (16 * kg) : 0u;
+      }
+    } else {
+      const uint2 dd = *reinterpret_cast<const uint2*>(sl + G::SLOT_Q + l32 * 8);
+      rg.d[0] = dd.x | (dd.x << 16);
+      rg.d[1] = dd.y | (dd.y << 16);
+      rg.m[0] = rg.m[1] = rg.qh[0] = rg.qh[1] = 0u;
+    }
     return rg;
   };
 
@@ -219,16 +258,22 @@ __global__ __launch_bounds__(64 * B3_WAVES, 1) void block32_gemm3_kernel(const _
     const uint32_t qw[4] = {rg.q[b].x, rg.q[b].y, rg.q[b].z, rg.q[b].w};
     const f16x2 dp = __builtin_bit_cast(f16x2, rg.d[b]);
     // q8_0: byte ^ 0x80 = q + 128, 0x6400 | that = 1024 + 128 + q (iq4_nl: the table holds value + 128);
-    // q4_0: 0x6400 | nibble = 1024 + 8 + (n - 8)
-    const f16x2 off = C == KQ_Q4_0 ? f16x2{(_Float16)-1032.0f, (_Float16)-1032.0f} : f16x2{(_Float16)-1152.0f, (_Float16)-1152.0f};
+    // q4_0: 0x6400 | nibble = 1024 + 8 + (n - 8); q5_0: 1024 + 16 + (q - 16); q4_1 / q5_1: 1024 + q
+    constexpr float OFF = C == KQ_Q4_0 ? -1032.0f : C == KQ_Q5_0 ? -1040.0f : G::MIN ? -1024.0f : -1152.0f;
+    const f16x2 off = {(_Float16)OFF, (_Float16)OFF};
     f16x2 h2[4], l2[4];
 #pragma unroll
     for (int e = 0; e < 2; e++) {
       uint32_t x = qw[2 * s + e];
       if constexpr (C == KQ_Q8_0) {
         x ^= 0x80808080u;
-      } else if constexpr (C == KQ_Q4_0) {
+      } else if constexpr (C == KQ_Q4_0 || C == KQ_Q4_1) {
         x >>= 4 * kg;
+      } else if constexpr (G::FIVE) {
+        // the four fifth bits of these four weights, one into bit 4 of each byte
+        const uint32_t four = (rg.qh[b] >> (8 * s + 4 * e)) & 0xfu;
+        const uint32_t spread = (four * 0x00204081u) & 0x01010101u;
+        x = ((x >> (4 * kg)) & 0x0f0f0f0fu) | (spread << 4);
       } else {
         const uint32_t nib = (x >> (4 * kg)) & 0x0f0f0f0fu, low3 = nib & 0x07070707u;
         const uint32_t half0 = __builtin_amdgcn_perm(kv1, kv0, low3), half1 = __builtin_amdgcn_perm(kv3, kv2, low3);
@@ -278,6 +323,12 @@ __global__ __launch_bounds__(64 * B3_WAVES, 1) void block32_gemm3_kernel(const _
         decode(std::integral_constant<int, 0>{}, nxt, bhi[0], blo[0]);
 #pragma unroll
       for (int t = 0; t < MT; t++) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[t], bhi[g & 1], acc[t], 0, 0, 0);
+      if constexpr (G::MIN) {  // third term: the block minimum against the same activations
+        const f16x2 mp = __builtin_bit_cast(f16x2, cur.m[g >> 1]);
+        const f16x8 bm = {mp[0], mp[1], mp[0], mp[1], mp[0], mp[1], mp[0], mp[1]};
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[t], bm, acc[t], 0, 0, 0);
+      }
 #pragma unroll
       for (int t = 0; t < MT; t++) {
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[t], blo[g & 1], acc[t], 0, 0, 0);
@@ -363,9 +414,10 @@ int launch_b3_call(const void* x, const uint8_t* w, void* y, int M, int N, int K
 // Taken for calls of 128 rows or more whose half-height tiles fill three quarters of the CUs; smaller calls stay on
 // the any-codec kernel (small workgroups, K cut over the grid).
 bool kq_gemm3b_supported(int M, int N, int K, int codec) {
-  if (codec != KQ_Q8_0 && codec != KQ_Q4_0 && codec != KQ_IQ4_NL) return false;
+  if (codec != KQ_Q8_0 && codec != KQ_Q4_0 && codec != KQ_IQ4_NL && codec != KQ_Q4_1 && codec != KQ_Q5_0 && codec != KQ_Q5_1)
+    return false;
   if (M < 128 || N <= 0 || K < 64 || (K & 63)) return false;
-  const int64_t row_bytes = (int64_t)(K >> 5) * (codec == KQ_Q8_0 ? 34 : 18);
+  const int64_t row_bytes = (int64_t)(K >> 5) * 34;  // the largest block of the six
   if (256 * row_bytes >= ((int64_t)1 << 32) || (int64_t)M * K * 2 >= ((int64_t)1 << 32)) return false;
   if (g_b3_force > 0) return true;  // a forced tile height takes every shape (tests reach the kernel on small matrices)
   return 4 * (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 3 * (int64_t)b3_num_cus();
@@ -387,6 +439,15 @@ int kq_launch_gemm3b(const void* x, const uint8_t* w, void* y, int M, int N, int
   if (codec == KQ_IQ4_NL)
     return dtype == KQ_F16 ? launch_b3_call<KQ_IQ4_NL, KQ_F16>(x, w, y, M, N, K, ws, force, s)
                            : launch_b3_call<KQ_IQ4_NL, KQ_BF16>(x, w, y, M, N, K, ws, force, s);
+  if (codec == KQ_Q4_1)
+    return dtype == KQ_F16 ? launch_b3_call<KQ_Q4_1, KQ_F16>(x, w, y, M, N, K, ws, force, s)
+                           : launch_b3_call<KQ_Q4_1, KQ_BF16>(x, w, y, M, N, K, ws, force, s);
+  if (codec == KQ_Q5_0)
+    return dtype == KQ_F16 ? launch_b3_call<KQ_Q5_0, KQ_F16>(x, w, y, M, N, K, ws, force, s)
+                           : launch_b3_call<KQ_Q5_0, KQ_BF16>(x, w, y, M, N, K, ws, force, s);
+  if (codec == KQ_Q5_1)
+    return dtype == KQ_F16 ? launch_b3_call<KQ_Q5_1, KQ_F16>(x, w, y, M, N, K, ws, force, s)
+                           : launch_b3_call<KQ_Q5_1, KQ_BF16>(x, w, y, M, N, K, ws, force, s);
   return dtype == KQ_F16 ? launch_b3_call<KQ_Q4_0, KQ_F16>(x, w, y, M, N, K, ws, force, s)
                          : launch_b3_call<KQ_Q4_0, KQ_BF16>(x, w, y, M, N, K, ws, force, s);
 }

@@ -73,10 +73,10 @@ def test_prefill_fp4_tile_choice(kq, codec, M, N, K, dtype):
     _check_matmul(kq, codec, M, N, K, dtype, 94, 48)
 
 
-@pytest.mark.parametrize("codec", ["q8_0", "q4_0", "iq4_nl"])
+@pytest.mark.parametrize("codec", ["q8_0", "q4_0", "iq4_nl", "q4_1", "q5_0", "q5_1"])
 @pytest.mark.parametrize("M,N,K", [(2048, 28672, 8192), (512, 28672, 2880), (1024, 8192, 8192)])
 def test_prefill_block32_tile_choice(kq, codec, M, N, K):
-    """q8_0 / q4_0 / iq4_nl prefill through the automatic tile choice of the two-term kernel: whole rounds of 256-row tiles
+    """q8_0 / q4_0 / iq4_nl / q5_0 / q4_1 / q5_1 prefill through the automatic tile choice of the two-term kernel: whole rounds of 256-row tiles
     plus a round of 128-row tiles, 256-row tiles alone (K = 2880: 45 steps), 128-row tiles alone."""
     _check_matmul(kq, codec, M, N, K, "bfloat16", 92, 48)
 

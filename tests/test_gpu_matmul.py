@@ -427,9 +427,10 @@ def test_qmm_prefill_fp4_tall_tiles(kq, codec):
         lib.kq_set_gemm_tile_rows(0)
 
 
-@pytest.mark.parametrize("codec", ["q8_0", "q4_0", "iq4_nl"])
+@pytest.mark.parametrize("codec", ["q8_0", "q4_0", "iq4_nl", "q4_1", "q5_0", "q5_1"])
 def test_qmm_prefill_block32_tall_tiles(kq, codec):
-    """q8_0 / q4_0 / iq4_nl on the 256-row and 128-row tiles (every weight d q as two exact f16 terms, wire bytes step by step
+    """q8_0 / q4_0 / iq4_nl / q5_0 / q4_1 / q5_1 on the 256-row and 128-row tiles (every weight d q as two exact f16 terms,
+    the block minimum of q4_1 / q5_1 as a third, wire bytes step by step
     through a ring of four slots): one to forty-five K steps of 64 (prologue only, ring wrap, K = 2880), ragged M and N
     tiles, both activation dtypes; blocks with d = 0, negative, subnormal and large d and the extreme codes; and the
     automatic choice on a matrix wide enough to be taken."""
