@@ -324,6 +324,7 @@ int launch_gemm3(const _Float16* xh, const _Float16* xhl, const float* rs, const
 
 
 // ------------------------------------------------------------------ q6_k
+// (block layout as the reference decodes it: src/kquant_cpu_decode.cpp:237-280)
 // Same tile, same activation pipeline.  A q6_k weight sc (q - 32) reaches 4096 and goes in as two exact terms,
 // sc ql and 16 sc (qh - 2), so a decoded fragment feeds sixteen MFMAs.  There is no minimum term: entering a
 // superblock only changes the unit of the running sums.  Two superblock stages of 32 rows do not fit beside the

@@ -20,6 +20,9 @@
 // 2-byte loads) and needs no barrier for them: step s + 3 is queued in step s, registers of step s + 1 are read in
 // step s.  Activations come from a prepass of their own (f16 scaled per row by a power of two, k permuted inside
 // 8-groups to match the byte order of the decode).
+// Block layouts as the reference decodes them: src/kquant_cpu_decode.cpp:49-63 (q8_0), :65-82 (q4_0), :84-102 (q4_1),
+// :104-128 (q5_0), :130-153 (q5_1), :382-397 (iq4_nl); the M > 8 matmul this serves: src/kquant_cpu_decode.cpp:1209-1359,
+// tile policy of the reference's own matrix path: src/kquant_matmul.cpp:77-134, 313-451.
 #include "kq_dma.h"
 #include "kq_mma.h"
 

@@ -19,6 +19,9 @@
 // Workgroup, activation stages and the wave-private ring of four wire slots as in kq_gemm3b.hip; a K step (64
 // weights: one nvfp4 block of 36 bytes, two mxfp4 blocks of 17) travels as three 16-byte pieces per row, the last
 // one ending on the step's last byte (rows are 2-byte aligned whenever K is a multiple of 64).
+// Block layouts and scale decoding as in the reference: src/kquant_cpu_decode.cpp:403-418 (mxfp4), :420-438 (nvfp4),
+// src/kquant_fp_tables.h:21-41 (e8m0 / unsigned e4m3 scales); the M > 8 matmul this serves:
+// src/kquant_cpu_decode.cpp:1209-1359, tile policy of the reference's own matrix path: src/kquant_matmul.cpp:77-134.
 #include "kq_dma.h"
 #include "kq_mma.h"
 
