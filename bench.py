@@ -15,7 +15,7 @@ at least 100 launches), captured once into a HIP graph and replayed, so the host
 enter the figure; `us_per_launch` = step time / `launches_per_step`.
 
 Extra fields: `sweep` (the decode projections of the q4_k_m recipe at M in {1,2,4,8}), `prefill`
-(q4_k / q5_k / q6_k / q2_k / q3_k / iq4_xs / q8_0 / q4_0 / mxfp4 / nvfp4 GEMM 8192 -> 28672 at M in {512, 2048}), `moe` (128 experts, top-8, hidden 2048,
+(q4_k / q5_k / q6_k / q2_k / q3_k / iq4_xs / q8_0 / q4_0 / mxfp4 / nvfp4 / iq3_s / iq2_xxs GEMM 8192 -> 28672 at M in {512, 2048}), `moe` (128 experts, top-8, hidden 2048,
 intermediate 768: fused gate/up GLU in q4_k and down in q6_k at 1 and 256 tokens), `lowbit` (M=1
 GEMV 8192 -> 8192 in the low-bit codecs), `moe_decode_lowbit` (1 token, 8 of 128 experts, IQ / fp4 / q8_0 stacks),
 `read_ceiling` (stock read-only reduction, stock bf16 GEMV and device copy on buffers of the GEMV's sizes, cold),
@@ -571,12 +571,16 @@ def main():
         if want("prefill"):
             prefill = []
             abi.lib.kq_set_gemm_tile_rows(args.gemm_tile)
-            for c in ("q4_k", "q5_k", "q6_k", "q2_k", "q3_k", "iq4_xs", "q8_0", "q4_0", "mxfp4", "nvfp4"):
+            for c in ("q4_k", "q5_k", "q6_k", "q2_k", "q3_k", "iq4_xs", "q8_0", "q4_0", "mxfp4", "nvfp4", "iq3_s", "iq2_xxs"):
                 n, k = 28672, 8192
-                # q4_k / q5_k / q6_k / q8_0 / q4_0 / mxfp4 / nvfp4: 256-row tiles for the whole rounds, 128-row tiles
-                # for the rest; q2_k / q3_k / iq4_xs: 128 x 256 tiles
-                # the fp4 codecs have no encoder (the reference has none either): structurally valid random wire
-                wq = synth_wire_torch(c, n, k, 5, dev) if c in ("mxfp4", "nvfp4") else quantized_weights(kq, torch, c, n, k, 5, dev)
+                # q4_k / q5_k / q6_k / q8_0 / q4_0 / mxfp4 / nvfp4 / iq3_s / iq2_xxs: 256-row tiles for the whole rounds,
+                # 128-row tiles for the rest; q2_k / q3_k / iq4_xs: 128 x 256 tiles
+                # the fp4 codecs have no encoder (the reference has none either): structurally valid random wire;
+                # the codebook encoders search for ~1 us per weight on the host: 512 unique rows, tiled
+                if c in ("mxfp4", "nvfp4"):
+                    wq = synth_wire_torch(c, n, k, 5, dev)
+                else:
+                    wq = quantized_weights(kq, torch, c, n, k, 5, dev, unique_rows=512 if c in ("iq3_s", "iq2_xxs") else None)
                 for m in (512, 2048):
                     # the device idles while the host encodes the weights: about 30 ms of launches bring it back
                     # to its steady clock before the timed ones (the first shape timed read 6 - 15 % low without)

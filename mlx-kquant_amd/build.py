@@ -29,6 +29,7 @@ SOURCES = [
     ("kq_gemm3.hip", ["-Wno-inline-asm"]),
     ("kq_gemm3b.hip", ["-Wno-inline-asm"]),
     ("kq_gemm3f.hip", ["-Wno-inline-asm"]),
+    ("kq_gemm3i.hip", ["-Wno-inline-asm", "-ffp-contract=off"]),
     ("kq_moe.hip", []),
     ("kq_anymma.hip", ["-ffp-contract=off"]),
     # one source, three objects: its kernel families are instantiated in parallel

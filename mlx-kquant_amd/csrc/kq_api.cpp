@@ -128,6 +128,7 @@ size_t kq_qmm_workspace_size(int M, int N, int K, int transpose, int codec, int 
   if (kq_gemm2_low_supported(M, N, K, codec) && kq_gemm2_low_workspace_bytes(M, K) > any) any = kq_gemm2_low_workspace_bytes(M, K);
   if (kq_gemm3b_supported(M, N, K, codec) && kq_gemm3b_workspace_bytes(M, K) > any) any = kq_gemm3b_workspace_bytes(M, K);
   if (kq_gemm3f_supported(M, N, K, codec) && kq_gemm3f_workspace_bytes(M, K) > any) any = kq_gemm3f_workspace_bytes(M, K);
+  if (kq_gemm3i_supported(M, N, K, codec) && kq_gemm3i_workspace_bytes(M, K) > any) any = kq_gemm3i_workspace_bytes(M, K);
   return tuned > any ? tuned : any;
 }
 
@@ -171,6 +172,10 @@ int kq_qmm(const void* x_dev, const void* w_dev, void* y_dev, int M, int N, int 
   if (kq_gemm3f_supported(M, N, K, codec) && workspace_dev && workspace_bytes >= kq_gemm3f_workspace_bytes(M, K)) {
     const int rcf = kq_launch_gemm3f(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev, s);
     if (rcf != KQ_ERR_UNSUPPORTED) return rcf;
+  }
+  if (kq_gemm3i_supported(M, N, K, codec) && workspace_dev && workspace_bytes >= kq_gemm3i_workspace_bytes(M, K)) {
+    const int rci = kq_launch_gemm3i(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype, workspace_dev, s);
+    if (rci != KQ_ERR_UNSUPPORTED) return rci;
   }
   if (M > 8) {
     const int rca = kq_launch_anymma_dense(x_dev, static_cast<const uint8_t*>(w_dev), y_dev, M, N, K, codec, dtype,

@@ -166,6 +166,14 @@ size_t kq_gemm3f_workspace_bytes(int M, int K);
 void kq_gemm3f_force_tile(int rows);
 int kq_launch_gemm3f(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
                      hipStream_t s);
+// The same tiles for the codebook codecs (iq2_xxs, iq2_xs, iq2_s, iq3_xxs, iq3_s, iq1_s, iq1_m): one exact f16 term per
+// weight (the reference-order decoder with d = 1), d in the unit of the running sums (kq_gemm3i.hip).  Runs its own
+// activation prepass into ws.
+bool kq_gemm3i_supported(int M, int N, int K, int codec);
+size_t kq_gemm3i_workspace_bytes(int M, int K);
+void kq_gemm3i_force_tile(int rows);
+int kq_launch_gemm3i(const void* x, const uint8_t* w, void* y, int M, int N, int K, int codec, int dtype, void* ws,
+                     hipStream_t s);
 // The same tile kernel for q2_k / q3_k (M >= 256, tiles filling the chip): runs its own activation prepass.
 bool kq_gemm2_low_supported(int M, int N, int K, int codec);
 size_t kq_gemm2_low_workspace_bytes(int M, int K);

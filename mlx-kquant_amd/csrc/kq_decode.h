@@ -62,7 +62,9 @@ __device__ __forceinline__ void q4k_scale_min(const uint8_t* s, int j, int& sc, 
   }
 }
 
-template <int C>
+// UNIT: the IQ codecs' weights with the superblock scale d taken as 1 (the caller applies d; every such value is an
+// integer multiple of 1/8 below 2048 / 4, i.e. an f16 number)
+template <int C, bool UNIT = false>
 __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, const uint8_t* __restrict__ grids,
                                         float* __restrict__ o) {
   if constexpr (C == KQ_Q8_0) {  // :49-63
@@ -161,7 +163,7 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     const uint8_t* q = b + 8 + 16 * ib + 8 * (r & 1);
     for (int t = 0; t < 8; t++) o[t] = dl * kv_iq4nl((r < 2) ? (q[t] & 15) : (q[t] >> 4));
   } else if constexpr (C == KQ_IQ3_XXS) {  // :467-500
-    float d = ldh(b);
+    float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     uint32_t aux = ld32(b + 66 + 4 * ib);
     float db = d * (0.5f + (float)(aux >> 28)) * 0.5f;
@@ -173,7 +175,7 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
       o[j + 4] = db * (float)g2[j] * sgn(s, j + 4);
     }
   } else if constexpr (C == KQ_IQ3_S) {  // :502-551
-    float d = ldh(b);
+    float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     int nib = (ib & 1) ? (b[106 + (ib >> 1)] >> 4) : (b[106 + (ib >> 1)] & 15);
     float db = d * (float)(1 + 2 * nib);
@@ -188,7 +190,7 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
       o[j + 4] = db * (float)g2[j] * sgn(s, j + 4);
     }
   } else if constexpr (C == KQ_IQ2_XXS) {  // :556-584
-    float d = ldh(b);
+    float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     uint32_t a1 = ld32(b + 2 + 8 * ib + 4);
     float db = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
@@ -196,7 +198,7 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     uint32_t s = ksigns(a1 >> (7 * l));
     for (int j = 0; j < 8; j++) o[j] = db * (float)gr[j] * sgn(s, j);
   } else if constexpr (C == KQ_IQ2_XS) {  // :586-617
-    float d = ldh(b);
+    float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     uint32_t scb = b[66 + ib];
     float dl = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
@@ -205,7 +207,7 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     uint32_t s = ksigns(q >> 9);
     for (int j = 0; j < 8; j++) o[j] = dl * (float)gr[j] * sgn(s, j);
   } else if constexpr (C == KQ_IQ2_S) {  // :619-650
-    float d = ldh(b);
+    float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     uint32_t scb = b[74 + ib];
     float dl = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
@@ -214,7 +216,7 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     uint32_t s = b[34 + 4 * ib + l];
     for (int j = 0; j < 8; j++) o[j] = dl * (float)gr[j] * sgn(s, j);
   } else if constexpr (C == KQ_IQ1_S) {  // :658-685
-    float d = ldh(b);
+    float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     uint32_t qh = ld16(b + 34 + 2 * ib);
     float dl = d * (float)(2 * (int)((qh >> 12) & 7) + 1);
@@ -225,7 +227,7 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     int ib = g >> 2, l = g & 3;
     uint32_t s0 = ld16(b + 48), s1 = ld16(b + 50), s2 = ld16(b + 52), s3 = ld16(b + 54);
     uint16_t du = (uint16_t)((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u));
-    float d = h2f(du);
+    float d = UNIT ? 1.0f : h2f(du);
     uint32_t scw = ld16(b + 48 + 2 * (ib >> 1));
     int sc3 = (scw >> (6 * (ib & 1) + 3 * (l >> 1))) & 7;
     float dl = d * (float)(2 * sc3 + 1);
@@ -234,6 +236,17 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     float delta = (nib & 8) ? -0.125f : 0.125f;
     const uint8_t* gr = grids + KQ_GRID_IQ1S + 8 * (b[4 * ib + l] | ((nib & 7) << 8));
     for (int j = 0; j < 8; j++) o[j] = dl * ((float)(int8_t)gr[j] + delta);
+  }
+}
+
+// superblock scale d of an IQ block (iq1_m keeps it in the top nibbles of its four scale words)
+template <int C>
+__device__ __forceinline__ float iq_block_d(const uint8_t* __restrict__ b) {
+  if constexpr (C == KQ_IQ1_M) {
+    const uint32_t s0 = ld16(b + 48), s1 = ld16(b + 50), s2 = ld16(b + 52), s3 = ld16(b + 54);
+    return h2f((uint16_t)((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u)));
+  } else {
+    return ldh(b);
   }
 }
 

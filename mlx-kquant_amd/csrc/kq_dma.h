@@ -20,6 +20,11 @@ __device__ __forceinline__ void dma16(const uint8_t* sbase, uint32_t voff, uint3
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(sbase)
                : "memory", "m0");
 }
+// 4-byte form: LDS address of lane l = lds + 4 l
+__device__ __forceinline__ void dma4(const uint8_t* sbase, uint32_t voff, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds), "v"(voff), "s"(sbase)
+               : "memory", "m0");
+}
 __device__ __forceinline__ void dma2(const uint8_t* sbase, uint32_t voff, uint32_t lds) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2" ::"s"(lds), "v"(voff), "s"(sbase)
                : "memory", "m0");

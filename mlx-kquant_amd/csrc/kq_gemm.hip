@@ -407,5 +407,6 @@ int kq_launch_act_prepass(const void* x, void* xh, void* xhl, float* rs, int M, 
 extern "C" void kq_set_gemm_tile_rows(int rows) {
   kq_gemm3b_force_tile(rows);
   kq_gemm3f_force_tile(rows);
+  kq_gemm3i_force_tile(rows);
   g_gemm_tile = (rows == 64 || rows == 128 || rows == 256 || rows == 512 || rows == 513 || rows == 1024 || rows == 1025) ? rows : 0;
 }

@@ -65,6 +65,12 @@ def test_config3_prefill_8192_to_28672(kq, codec, M):
     _check_matmul(kq, codec, M, 28672, 8192, "bfloat16", 74, 48)
 
 
+@pytest.mark.parametrize("codec", ["iq2_xxs", "iq3_s", "iq1_s"])
+def test_prefill_iq_tile_choice(kq, codec):
+    """Codebook codecs at the prefill benchmark shape through the automatic tile choice of their tall-tile kernel."""
+    _check_matmul(kq, codec, 2048, 28672, 8192, "bfloat16", 96, 48)
+
+
 @pytest.mark.parametrize("codec", ["mxfp4", "nvfp4"])
 @pytest.mark.parametrize("M,N,K,dtype", [(2048, 28672, 8192, "bfloat16"), (512, 28672, 2880, "float16")])
 def test_prefill_fp4_tile_choice(kq, codec, M, N, K, dtype):

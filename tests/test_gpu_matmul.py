@@ -377,6 +377,45 @@ def test_qmm_prefill_gemm_128x256_tiles(kq, codec):
         lib.kq_set_gemm_tile_rows(0)
 
 
+@pytest.mark.parametrize("codec", ["iq2_xxs", "iq2_xs", "iq2_s", "iq3_xxs", "iq3_s", "iq1_s", "iq1_m"])
+def test_qmm_prefill_iq_tall_tiles(kq, codec):
+    """The codebook codecs on the 256-row and 128-row tiles (the reference-order decoder with d = 1 as one exact f16
+    term, d in the unit of the running sums, codebook in LDS, wire bytes by 4-byte direct-to-LDS loads): one to nine
+    superblocks of K, ragged M and N tiles (the matrix's last row sits in every one of these calls: its last dword is
+    loaded two bytes early and shifted), both activation dtypes; superblocks with d = 0 and negative d; and the
+    automatic choice on a matrix wide enough to be taken."""
+    lib = kq._load()
+    wpb, bpb = O.geometry(codec)
+    try:
+        for rows in (1024, 1025):
+            lib.kq_set_gemm_tile_rows(rows)
+            for M, N, K, dtype in ((128, 40, 256, "bfloat16"), (130, 257, 512, "float16"), (300, 520, 2304, "bfloat16"),
+                                   (513, 700, 1024, "float16")):
+                wire = _wire(codec, N, K, seed=91)
+                xb, xt = make_x((M, K), dtype, seed=92)
+                got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+                want = O.qmm(xb, wire, codec, True, dtype)
+                assert rel_l2(got, want, dtype) <= TOL, (codec, rows, M, N, K, dtype)
+            if codec != "iq1_m":  # iq1_m keeps d in the top nibbles of its scale words
+                M, N, K = 140, 300, 1536
+                wire = _wire(codec, N, K, seed=93).copy()
+                blocks = wire.reshape(N, K // wpb, bpb)
+                blocks[::3, ::2, 0:2] = 0      # d = 0: the superblock keeps the unit of the running sums
+                blocks[1::3, :, 1] |= 0x80     # negative d
+                xb, xt = make_x((M, K), "bfloat16", seed=94)
+                got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+                want = O.qmm(xb, wire, codec, True, "bfloat16")
+                assert rel_l2(got, want, "bfloat16") <= TOL, (codec, rows, "special blocks")
+        lib.kq_set_gemm_tile_rows(0)
+        M, N, K = 256, 24600, 256
+        wire = _wire(codec, N, K, seed=95)
+        xb, xt = make_x((M, K), "float16", seed=96)
+        got = dev_to_bits(kq.quantized_matmul(xt, wire_to_dev(wire), None, codec))
+        assert rel_l2(got, O.qmm(xb, wire, codec, True, "float16"), "float16") <= TOL, (codec, "automatic")
+    finally:
+        lib.kq_set_gemm_tile_rows(0)
+
+
 @pytest.mark.parametrize("codec", ["mxfp4", "nvfp4"])
 def test_qmm_prefill_fp4_tall_tiles(kq, codec):
     """mxfp4 / nvfp4 on the 256-row and 128-row tiles (one exact f16 term per weight out of the hardware's fp4 -> f16
