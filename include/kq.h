@@ -112,7 +112,7 @@ int kq_qmv_bias(const void* x_dev, const void* w_dev, const void* bias_dev, void
  * direct-to-LDS loads (q2_k / q3_k / q4_k / q5_k / iq4_xs; 513 = the same kernel as 128 x 128 on four waves),
  * 1024 = 256 x 256 on eight waves with 256-row wave tiles on one accumulator set (q4_k / q5_k / q6_k) for every
  * column tile, 1025 = the 128 x 256 form of that kernel (q6_k only; other codecs fall back to automatic); for
- * q8_0 / q4_0 / q4_1 / q5_0 / q5_1 / iq4_nl / mxfp4 / nvfp4, 1024 / 1025 force the 256- / 128-row form of their tall-tile kernels on any
+ * q8_0 / q4_0 / q4_1 / q5_0 / q5_1 / iq4_nl / mxfp4 / nvfp4 and the codebook codecs (iq1 / iq2 / iq3), 1024 / 1025 force the 256- / 128-row form of their tall-tile kernels on any
  * shape of 128 rows or more and 64 keeps them on the any-codec kernel;
  * anything else restores the automatic choice (q4_k / q5_k / q6_k with 256 rows or more: the 256 x 256 kernel on the
  * column tiles that fill whole rounds of one workgroup per CU, a 128 x 256 kernel on the rest; q6_k matrices of
