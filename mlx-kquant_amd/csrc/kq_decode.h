@@ -62,6 +62,13 @@ __device__ __forceinline__ void q4k_scale_min(const uint8_t* s, int j, int& sc, 
   }
 }
 
+// A codebook entry read as whole words (the codebook blob is 16-byte aligned wherever it lies, its tables start on
+// multiples of 1024 and their entries are 4 or 8 bytes long) and byte j of it.
+__device__ __forceinline__ uint32_t grid4(const uint8_t* p) { return *reinterpret_cast<const uint32_t*>(p); }
+__device__ __forceinline__ uint2 grid8(const uint8_t* p) { return *reinterpret_cast<const uint2*>(p); }
+__device__ __forceinline__ uint32_t byte_of(uint32_t w, int j) { return (w >> (8 * j)) & 0xffu; }
+__device__ __forceinline__ uint32_t byte_of(uint2 w, int j) { return byte_of(j < 4 ? w.x : w.y, j & 3); }
+
 // UNIT: the IQ codecs' weights with the superblock scale d taken as 1 (the caller applies d; every such value is an
 // integer multiple of 1/8 below 2048 / 4, i.e. an f16 number)
 template <int C, bool UNIT = false>
@@ -168,11 +175,11 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     uint32_t aux = ld32(b + 66 + 4 * ib);
     float db = d * (0.5f + (float)(aux >> 28)) * 0.5f;
     uint32_t s = ksigns(aux >> (7 * l));
-    const uint8_t* g1 = grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l];
-    const uint8_t* g2 = grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l + 1];
+    const uint32_t g1 = grid4(grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l]);
+    const uint32_t g2 = grid4(grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l + 1]);
     for (int j = 0; j < 4; j++) {
-      o[j] = db * (float)g1[j] * sgn(s, j);
-      o[j + 4] = db * (float)g2[j] * sgn(s, j + 4);
+      o[j] = db * (float)byte_of(g1, j) * sgn(s, j);
+      o[j + 4] = db * (float)byte_of(g2, j) * sgn(s, j + 4);
     }
   } else if constexpr (C == KQ_IQ3_S) {  // :502-551
     float d = UNIT ? 1.0f : ldh(b);
@@ -183,46 +190,46 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     uint32_t i1 = b[2 + 8 * ib + 2 * l] | ((h << (8 - 2 * l)) & 256u);
     uint32_t i2 = b[2 + 8 * ib + 2 * l + 1] | ((h << (7 - 2 * l)) & 256u);
     uint32_t s = b[74 + 4 * ib + l];
-    const uint8_t* g1 = grids + KQ_GRID_IQ3S + 4 * i1;
-    const uint8_t* g2 = grids + KQ_GRID_IQ3S + 4 * i2;
+    const uint32_t g1 = grid4(grids + KQ_GRID_IQ3S + 4 * i1);
+    const uint32_t g2 = grid4(grids + KQ_GRID_IQ3S + 4 * i2);
     for (int j = 0; j < 4; j++) {
-      o[j] = db * (float)g1[j] * sgn(s, j);
-      o[j + 4] = db * (float)g2[j] * sgn(s, j + 4);
+      o[j] = db * (float)byte_of(g1, j) * sgn(s, j);
+      o[j + 4] = db * (float)byte_of(g2, j) * sgn(s, j + 4);
     }
   } else if constexpr (C == KQ_IQ2_XXS) {  // :556-584
     float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     uint32_t a1 = ld32(b + 2 + 8 * ib + 4);
     float db = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
-    const uint8_t* gr = grids + KQ_GRID_IQ2XXS + 8 * b[2 + 8 * ib + l];
+    const uint2 gr = grid8(grids + KQ_GRID_IQ2XXS + 8 * b[2 + 8 * ib + l]);
     uint32_t s = ksigns(a1 >> (7 * l));
-    for (int j = 0; j < 8; j++) o[j] = db * (float)gr[j] * sgn(s, j);
+    for (int j = 0; j < 8; j++) o[j] = db * (float)byte_of(gr, j) * sgn(s, j);
   } else if constexpr (C == KQ_IQ2_XS) {  // :586-617
     float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     uint32_t scb = b[66 + ib];
     float dl = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
     uint32_t q = ld16(b + 2 + 2 * (4 * ib + l));
-    const uint8_t* gr = grids + KQ_GRID_IQ2XS + 8 * (q & 511u);
+    const uint2 gr = grid8(grids + KQ_GRID_IQ2XS + 8 * (q & 511u));
     uint32_t s = ksigns(q >> 9);
-    for (int j = 0; j < 8; j++) o[j] = dl * (float)gr[j] * sgn(s, j);
+    for (int j = 0; j < 8; j++) o[j] = dl * (float)byte_of(gr, j) * sgn(s, j);
   } else if constexpr (C == KQ_IQ2_S) {  // :619-650
     float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     uint32_t scb = b[74 + ib];
     float dl = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
     uint32_t gi = b[2 + 4 * ib + l] | (((uint32_t)b[66 + ib] << (8 - 2 * l)) & 0x300u);
-    const uint8_t* gr = grids + KQ_GRID_IQ2S + 8 * gi;
+    const uint2 gr = grid8(grids + KQ_GRID_IQ2S + 8 * gi);
     uint32_t s = b[34 + 4 * ib + l];
-    for (int j = 0; j < 8; j++) o[j] = dl * (float)gr[j] * sgn(s, j);
+    for (int j = 0; j < 8; j++) o[j] = dl * (float)byte_of(gr, j) * sgn(s, j);
   } else if constexpr (C == KQ_IQ1_S) {  // :658-685
     float d = UNIT ? 1.0f : ldh(b);
     int ib = g >> 2, l = g & 3;
     uint32_t qh = ld16(b + 34 + 2 * ib);
     float dl = d * (float)(2 * (int)((qh >> 12) & 7) + 1);
     float delta = (qh & 0x8000u) ? -0.125f : 0.125f;
-    const uint8_t* gr = grids + KQ_GRID_IQ1S + 8 * (b[2 + 4 * ib + l] | (((qh >> (3 * l)) & 7) << 8));
-    for (int j = 0; j < 8; j++) o[j] = dl * ((float)(int8_t)gr[j] + delta);
+    const uint2 gr = grid8(grids + KQ_GRID_IQ1S + 8 * (b[2 + 4 * ib + l] | (((qh >> (3 * l)) & 7) << 8)));
+    for (int j = 0; j < 8; j++) o[j] = dl * ((float)(int8_t)byte_of(gr, j) + delta);
   } else if constexpr (C == KQ_IQ1_M) {  // :687-735
     int ib = g >> 2, l = g & 3;
     uint32_t s0 = ld16(b + 48), s1 = ld16(b + 50), s2 = ld16(b + 52), s3 = ld16(b + 54);
@@ -234,8 +241,8 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     uint32_t hb = b[32 + 2 * ib + (l >> 1)];
     uint32_t nib = (l & 1) ? (hb >> 4) : (hb & 15);
     float delta = (nib & 8) ? -0.125f : 0.125f;
-    const uint8_t* gr = grids + KQ_GRID_IQ1S + 8 * (b[4 * ib + l] | ((nib & 7) << 8));
-    for (int j = 0; j < 8; j++) o[j] = dl * ((float)(int8_t)gr[j] + delta);
+    const uint2 gr = grid8(grids + KQ_GRID_IQ1S + 8 * (b[4 * ib + l] | ((nib & 7) << 8)));
+    for (int j = 0; j < 8; j++) o[j] = dl * ((float)(int8_t)byte_of(gr, j) + delta);
   }
 }
 
