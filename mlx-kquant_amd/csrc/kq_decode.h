@@ -69,6 +69,93 @@ __device__ __forceinline__ uint2 grid8(const uint8_t* p) { return *reinterpret_c
 __device__ __forceinline__ uint32_t byte_of(uint32_t w, int j) { return (w >> (8 * j)) & 0xffu; }
 __device__ __forceinline__ uint32_t byte_of(uint2 w, int j) { return byte_of(j < 4 ? w.x : w.y, j & 3); }
 
+// The codecs whose groups of 8 weights are a codebook entry of 8 magnitudes, 8 sign bits and a scale.
+__host__ __device__ constexpr bool is_sign_grid_codec(int c) {
+  return c == KQ_IQ3_XXS || c == KQ_IQ3_S || c == KQ_IQ2_XXS || c == KQ_IQ2_XS || c == KQ_IQ2_S;
+}
+
+// Group g (weights 8 g .. 8 g + 7) of a block of such a codec: the magnitudes are the bytes of lo (weights 0-3) and hi
+// (4-7), bit j of s is the sign of weight j, db the scale in the reference's order of operations; UNIT takes the
+// superblock scale d as 1.
+template <int C, bool UNIT>
+__device__ __forceinline__ void iq_group(const uint8_t* __restrict__ b, int g, const uint8_t* __restrict__ grids,
+                                         uint32_t& lo, uint32_t& hi, uint32_t& s, float& db) {
+  const float d = UNIT ? 1.0f : ldh(b);
+  const int ib = g >> 2, l = g & 3;
+  if constexpr (C == KQ_IQ3_XXS) {  // :467-500
+    const uint32_t aux = ld32(b + 66 + 4 * ib);
+    db = d * (0.5f + (float)(aux >> 28)) * 0.5f;
+    s = ksigns(aux >> (7 * l));
+    lo = grid4(grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l]);
+    hi = grid4(grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l + 1]);
+  } else if constexpr (C == KQ_IQ3_S) {  // :502-551
+    const int nib = (ib & 1) ? (b[106 + (ib >> 1)] >> 4) : (b[106 + (ib >> 1)] & 15);
+    db = d * (float)(1 + 2 * nib);
+    const uint32_t h = b[66 + ib];
+    const uint32_t i1 = b[2 + 8 * ib + 2 * l] | ((h << (8 - 2 * l)) & 256u);
+    const uint32_t i2 = b[2 + 8 * ib + 2 * l + 1] | ((h << (7 - 2 * l)) & 256u);
+    s = b[74 + 4 * ib + l];
+    lo = grid4(grids + KQ_GRID_IQ3S + 4 * i1);
+    hi = grid4(grids + KQ_GRID_IQ3S + 4 * i2);
+  } else if constexpr (C == KQ_IQ2_XXS) {  // :556-584
+    const uint32_t a1 = ld32(b + 2 + 8 * ib + 4);
+    db = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
+    const uint2 gr = grid8(grids + KQ_GRID_IQ2XXS + 8 * b[2 + 8 * ib + l]);
+    s = ksigns(a1 >> (7 * l));
+    lo = gr.x;
+    hi = gr.y;
+  } else if constexpr (C == KQ_IQ2_XS) {  // :586-617
+    const uint32_t scb = b[66 + ib];
+    db = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
+    const uint32_t q = ld16(b + 2 + 2 * (4 * ib + l));
+    const uint2 gr = grid8(grids + KQ_GRID_IQ2XS + 8 * (q & 511u));
+    s = ksigns(q >> 9);
+    lo = gr.x;
+    hi = gr.y;
+  } else {  // iq2_s :619-650
+    static_assert(C == KQ_IQ2_S, "not a sign-and-grid codec");
+    const uint32_t scb = b[74 + ib];
+    db = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
+    const uint32_t gi = b[2 + 4 * ib + l] | (((uint32_t)b[66 + ib] << (8 - 2 * l)) & 0x300u);
+    const uint2 gr = grid8(grids + KQ_GRID_IQ2S + 8 * gi);
+    s = b[34 + 4 * ib + l];
+    lo = gr.x;
+    hi = gr.y;
+  }
+}
+
+// Group g of a block of the ternary codecs iq1_s / iq1_m: the codebook entry's 8 signed bytes (-1, 0, 1) in lo and hi,
+// the group's scale dl and its shift delta = +-1/8: weight j = dl * (entry[j] + delta).
+template <int C, bool UNIT>
+__device__ __forceinline__ void iq1_group(const uint8_t* __restrict__ b, int g, const uint8_t* __restrict__ grids,
+                                          uint32_t& lo, uint32_t& hi, float& dl, float& delta) {
+  const int ib = g >> 2, l = g & 3;
+  uint2 gr;
+  if constexpr (C == KQ_IQ1_S) {  // :658-685
+    const float d = UNIT ? 1.0f : ldh(b);
+    const uint32_t qh = ld16(b + 34 + 2 * ib);
+    dl = d * (float)(2 * (int)((qh >> 12) & 7) + 1);
+    delta = (qh & 0x8000u) ? -0.125f : 0.125f;
+    gr = grid8(grids + KQ_GRID_IQ1S + 8 * (b[2 + 4 * ib + l] | (((qh >> (3 * l)) & 7) << 8)));
+  } else {  // iq1_m :687-735
+    static_assert(C == KQ_IQ1_M, "not a ternary codec");
+    float d = 1.0f;
+    if constexpr (!UNIT) {
+      const uint32_t s0 = ld16(b + 48), s1 = ld16(b + 50), s2 = ld16(b + 52), s3 = ld16(b + 54);
+      d = h2f((uint16_t)((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u)));
+    }
+    const uint32_t scw = ld16(b + 48 + 2 * (ib >> 1));
+    const int sc3 = (scw >> (6 * (ib & 1) + 3 * (l >> 1))) & 7;
+    dl = d * (float)(2 * sc3 + 1);
+    const uint32_t hb = b[32 + 2 * ib + (l >> 1)];
+    const uint32_t nib = (l & 1) ? (hb >> 4) : (hb & 15);
+    delta = (nib & 8) ? -0.125f : 0.125f;
+    gr = grid8(grids + KQ_GRID_IQ1S + 8 * (b[4 * ib + l] | ((nib & 7) << 8)));
+  }
+  lo = gr.x;
+  hi = gr.y;
+}
+
 // UNIT: the IQ codecs' weights with the superblock scale d taken as 1 (the caller applies d; every such value is an
 // integer multiple of 1/8 below 2048 / 4, i.e. an f16 number)
 template <int C, bool UNIT = false>
@@ -169,80 +256,22 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
     float dl = d * (float)(ls - 32);
     const uint8_t* q = b + 8 + 16 * ib + 8 * (r & 1);
     for (int t = 0; t < 8; t++) o[t] = dl * kv_iq4nl((r < 2) ? (q[t] & 15) : (q[t] >> 4));
-  } else if constexpr (C == KQ_IQ3_XXS) {  // :467-500
-    float d = UNIT ? 1.0f : ldh(b);
-    int ib = g >> 2, l = g & 3;
-    uint32_t aux = ld32(b + 66 + 4 * ib);
-    float db = d * (0.5f + (float)(aux >> 28)) * 0.5f;
-    uint32_t s = ksigns(aux >> (7 * l));
-    const uint32_t g1 = grid4(grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l]);
-    const uint32_t g2 = grid4(grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l + 1]);
+  } else if constexpr (is_sign_grid_codec(C)) {  // iq3_xxs, iq3_s, iq2_xxs, iq2_xs, iq2_s
+    uint32_t lo, hi, s;
+    float db;
+    iq_group<C, UNIT>(b, g, grids, lo, hi, s, db);
     for (int j = 0; j < 4; j++) {
-      o[j] = db * (float)byte_of(g1, j) * sgn(s, j);
-      o[j + 4] = db * (float)byte_of(g2, j) * sgn(s, j + 4);
+      o[j] = db * (float)byte_of(lo, j) * sgn(s, j);
+      o[j + 4] = db * (float)byte_of(hi, j) * sgn(s, j + 4);
     }
-  } else if constexpr (C == KQ_IQ3_S) {  // :502-551
-    float d = UNIT ? 1.0f : ldh(b);
-    int ib = g >> 2, l = g & 3;
-    int nib = (ib & 1) ? (b[106 + (ib >> 1)] >> 4) : (b[106 + (ib >> 1)] & 15);
-    float db = d * (float)(1 + 2 * nib);
-    uint32_t h = b[66 + ib];
-    uint32_t i1 = b[2 + 8 * ib + 2 * l] | ((h << (8 - 2 * l)) & 256u);
-    uint32_t i2 = b[2 + 8 * ib + 2 * l + 1] | ((h << (7 - 2 * l)) & 256u);
-    uint32_t s = b[74 + 4 * ib + l];
-    const uint32_t g1 = grid4(grids + KQ_GRID_IQ3S + 4 * i1);
-    const uint32_t g2 = grid4(grids + KQ_GRID_IQ3S + 4 * i2);
+  } else if constexpr (C == KQ_IQ1_S || C == KQ_IQ1_M) {
+    uint32_t lo, hi;
+    float dl, delta;
+    iq1_group<C, UNIT>(b, g, grids, lo, hi, dl, delta);
     for (int j = 0; j < 4; j++) {
-      o[j] = db * (float)byte_of(g1, j) * sgn(s, j);
-      o[j + 4] = db * (float)byte_of(g2, j) * sgn(s, j + 4);
+      o[j] = dl * ((float)(int8_t)byte_of(lo, j) + delta);
+      o[j + 4] = dl * ((float)(int8_t)byte_of(hi, j) + delta);
     }
-  } else if constexpr (C == KQ_IQ2_XXS) {  // :556-584
-    float d = UNIT ? 1.0f : ldh(b);
-    int ib = g >> 2, l = g & 3;
-    uint32_t a1 = ld32(b + 2 + 8 * ib + 4);
-    float db = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
-    const uint2 gr = grid8(grids + KQ_GRID_IQ2XXS + 8 * b[2 + 8 * ib + l]);
-    uint32_t s = ksigns(a1 >> (7 * l));
-    for (int j = 0; j < 8; j++) o[j] = db * (float)byte_of(gr, j) * sgn(s, j);
-  } else if constexpr (C == KQ_IQ2_XS) {  // :586-617
-    float d = UNIT ? 1.0f : ldh(b);
-    int ib = g >> 2, l = g & 3;
-    uint32_t scb = b[66 + ib];
-    float dl = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
-    uint32_t q = ld16(b + 2 + 2 * (4 * ib + l));
-    const uint2 gr = grid8(grids + KQ_GRID_IQ2XS + 8 * (q & 511u));
-    uint32_t s = ksigns(q >> 9);
-    for (int j = 0; j < 8; j++) o[j] = dl * (float)byte_of(gr, j) * sgn(s, j);
-  } else if constexpr (C == KQ_IQ2_S) {  // :619-650
-    float d = UNIT ? 1.0f : ldh(b);
-    int ib = g >> 2, l = g & 3;
-    uint32_t scb = b[74 + ib];
-    float dl = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
-    uint32_t gi = b[2 + 4 * ib + l] | (((uint32_t)b[66 + ib] << (8 - 2 * l)) & 0x300u);
-    const uint2 gr = grid8(grids + KQ_GRID_IQ2S + 8 * gi);
-    uint32_t s = b[34 + 4 * ib + l];
-    for (int j = 0; j < 8; j++) o[j] = dl * (float)byte_of(gr, j) * sgn(s, j);
-  } else if constexpr (C == KQ_IQ1_S) {  // :658-685
-    float d = UNIT ? 1.0f : ldh(b);
-    int ib = g >> 2, l = g & 3;
-    uint32_t qh = ld16(b + 34 + 2 * ib);
-    float dl = d * (float)(2 * (int)((qh >> 12) & 7) + 1);
-    float delta = (qh & 0x8000u) ? -0.125f : 0.125f;
-    const uint2 gr = grid8(grids + KQ_GRID_IQ1S + 8 * (b[2 + 4 * ib + l] | (((qh >> (3 * l)) & 7) << 8)));
-    for (int j = 0; j < 8; j++) o[j] = dl * ((float)(int8_t)byte_of(gr, j) + delta);
-  } else if constexpr (C == KQ_IQ1_M) {  // :687-735
-    int ib = g >> 2, l = g & 3;
-    uint32_t s0 = ld16(b + 48), s1 = ld16(b + 50), s2 = ld16(b + 52), s3 = ld16(b + 54);
-    uint16_t du = (uint16_t)((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u));
-    float d = UNIT ? 1.0f : h2f(du);
-    uint32_t scw = ld16(b + 48 + 2 * (ib >> 1));
-    int sc3 = (scw >> (6 * (ib & 1) + 3 * (l >> 1))) & 7;
-    float dl = d * (float)(2 * sc3 + 1);
-    uint32_t hb = b[32 + 2 * ib + (l >> 1)];
-    uint32_t nib = (l & 1) ? (hb >> 4) : (hb & 15);
-    float delta = (nib & 8) ? -0.125f : 0.125f;
-    const uint2 gr = grid8(grids + KQ_GRID_IQ1S + 8 * (b[4 * ib + l] | ((nib & 7) << 8)));
-    for (int j = 0; j < 8; j++) o[j] = dl * ((float)(int8_t)byte_of(gr, j) + delta);
   }
 }
 

@@ -2,10 +2,13 @@
 // on the f16 matrix cores, 256-row (or 128-row) wave tiles, ONE exact f16 term per weight.
 //
 // A weight of these codecs is d (f16, one per superblock of 256) times a sub-block factor times a codebook value
-// times a sign; everything but d is an integer multiple of 1/8 below 512 (kq::decode8<C, true>: the reference-order
-// decoder with d taken as 1), i.e. an f16 number.  Those go into the MFMA as they are; d goes into the unit of the
-// running sums exactly as in kq_gemm3.hip: entering a superblock with scale d, S is multiplied by r / d and r becomes
-// d (one multiply per accumulator and superblock; a superblock with d = 0 keeps the unit and feeds zeros).
+// times a sign; everything but d is an integer multiple of 1/8 below 512 (what the reference-order decoder gives with
+// d taken as 1), i.e. an f16 number.  Those go into the MFMA as they are; d goes into the unit of the running sums
+// exactly as in kq_gemm3.hip: entering a superblock with scale d, S is multiplied by r / d and r becomes d (one
+// multiply per accumulator and superblock; a superblock with d = 0 keeps the unit and feeds zeros).  The f16 values
+// are made in packed f16 arithmetic from the block's fields (kq::iq_group / kq::iq1_group, the field readers of the
+// shared decoder): codebook byte m as the f16 number 1024 + m by its bit pattern, one fused (1024 + m) s - 1024 s
+// with the group's scale s, which is exact, signs as XOR masks from a 256-entry table in LDS.
 //
 // Workgroup = 8 waves = 256 (MT = 8) or 128 (MT = 4) activation rows x 256 weight rows, one per CU.  K steps of 64,
 // two activation stages filled by the whole workgroup with direct-to-LDS loads (one barrier per step).  Every wave
@@ -63,7 +66,8 @@ template <int C>
 constexpr int i3_stage() { return 32 * 4 * i3_dpr<C>(); }    // bytes of a wave's stage (32 rows)
 template <int C, int MT>
 constexpr int i3_lds_bytes() {
-  return 2 * (32 * MT * I3_KS * 2) + I3_WAVES * 2 * i3_stage<C>() + I3Geom<C>::TBL_BYTES;
+  return 2 * (32 * MT * I3_KS * 2) + I3_WAVES * 2 * i3_stage<C>() + I3Geom<C>::TBL_BYTES +
+         (kq::is_sign_grid_codec(C) ? 4096 : 0);  // two activation stages, the wire stages, the codebook, the sign masks
 }
 
 // Activations of one row: xh = f16(x 2^-e) in their own order, rs = 2^e (bf16 rows scaled so that the largest
@@ -130,6 +134,7 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
   constexpr bool OVER = (BPB & 3) != 0;                // a block's last dword reaches two bytes past it
   constexpr int TM = 32 * MT, A_STAGE = TM * I3_KS * 2, AQ = MT / 2;
   constexpr int W_OFF = 2 * A_STAGE, T_OFF = W_OFF + I3_WAVES * 2 * STAGE;
+  constexpr int S_OFF = T_OFF + G::TBL_BYTES;  // the sign masks, 4 KiB
   constexpr int GPS = I3_KS / 16;   // MFMA groups per step: 4
   constexpr int SPS = 256 / I3_KS;  // steps per superblock: 4
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -147,6 +152,16 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
   // ---- the codebook into LDS (every wave is past the first barrier before it is read)
   for (int bi = 64 * wave; bi < G::TBL_BYTES / 16; bi += 64 * I3_WAVES)  // 64 pieces of 16 bytes per instruction
     dma16(grids + G::TBL_OFF + (size_t)bi * 16, 16u * (uint32_t)lane, lds0 + T_OFF + (uint32_t)bi * 16);
+
+  // ---- the sign masks of the codecs that keep 8 sign bits per group: entry e, dword i = bit 2 i of e on bit 15, bit
+  // 2 i + 1 on bit 31
+  if constexpr (kq::is_sign_grid_codec(C)) {
+    uint32_t* st = reinterpret_cast<uint32_t*>(smem + S_OFF);
+    for (int i = tid; i < 1024; i += 64 * I3_WAVES) {
+      const uint32_t two = ((uint32_t)i >> 2) >> (2 * (i & 3));
+      st[i] = ((two & 1u) << 15) | ((two & 2u) << 30);
+    }
+  }
 
   // ---- load maps
   // activations: load q covers rows 8 (wave + 8 q) + lane / 8, piece lane % 8 of the step; LDS piece p of row r holds
@@ -231,12 +246,49 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
   };
   // B fragment of group g of step p of superblock sb: weights 64 p + 16 g + 8 kg .. + 7 of this lane's row
   auto decode = [&](int sb, int p, int g, float lv) -> f16x8 {
-    float o[8];
-    kq::decode8<C, true>(w_smem + (sb & 1) * STAGE + l32 * (4 * DPR), 8 * p + 2 * g + kg, tbl, o);
-    const f16x8 b = {(_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3],
-                     (_Float16)o[4], (_Float16)o[5], (_Float16)o[6], (_Float16)o[7]};
-    const u32x4 keep = __builtin_bit_cast(u32x4, b) & (lv != 0.f ? 0xffffffffu : 0u);
-    return __builtin_bit_cast(f16x8, keep);
+    const uint8_t* blk = w_smem + (sb & 1) * STAGE + l32 * (4 * DPR);
+    if constexpr (kq::is_sign_grid_codec(C)) {
+      // magnitude byte m as the f16 1024 + m (bits 0x6400 | m), then (1024 + m) * db - 1024 * db in one fused step:
+      // db has at most 5 significant bits and m * db below 2048 units, so the result is m * db itself; the signs
+      // are the table's masks on the f16 sign bits.  A dead superblock is fed with db = 0.
+      uint32_t lo, hi, sg;
+      float db;
+      kq::iq_group<C, true>(blk, 8 * p + 2 * g + kg, tbl, lo, hi, sg, db);
+      const _Float16 dh = (_Float16)(lv != 0.f ? db : 0.f);
+      const f16x2 mul = {dh, dh}, sub = mul * f16x2{(_Float16)-1024.f, (_Float16)-1024.f};
+      const u32x4 mask = *reinterpret_cast<const u32x4*>(smem + S_OFF + 16 * sg);
+      const uint32_t pair[4] = {__builtin_amdgcn_perm(lo, 0x64646464u, 0x00050004u), __builtin_amdgcn_perm(lo, 0x64646464u, 0x00070006u),
+                                __builtin_amdgcn_perm(hi, 0x64646464u, 0x00050004u), __builtin_amdgcn_perm(hi, 0x64646464u, 0x00070006u)};
+      u32x4 out;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const f16x2 mag = __builtin_bit_cast(f16x2, pair[i]);
+        const f16x2 val = __builtin_elementwise_fma(mag, mul, sub);
+        out[i] = __builtin_bit_cast(uint32_t, val) ^ mask[i];
+      }
+      return __builtin_bit_cast(f16x8, out);
+    } else {
+      // ternary codecs: entry byte e in {-1, 0, 1} as the f16 1152 + e (bits 0x6400 | (e ^ 0x80)), then
+      // (1152 + e) * dl - 1152 * dl = e * dl in one fused step (dl is an odd integer up to 15) and + dl * delta, a
+      // multiple of 1/8 below 17: both exact.  A dead superblock is fed with dl = 0.
+      uint32_t lo, hi;
+      float dl, delta;
+      kq::iq1_group<C, true>(blk, 8 * p + 2 * g + kg, tbl, lo, hi, dl, delta);
+      lo ^= 0x80808080u;
+      hi ^= 0x80808080u;
+      const _Float16 dh = (_Float16)(lv != 0.f ? dl : 0.f), sh = (_Float16)(lv != 0.f ? dl * delta : 0.f);
+      const f16x2 mul = {dh, dh}, sub = mul * f16x2{(_Float16)-1152.f, (_Float16)-1152.f}, shift = {sh, sh};
+      const uint32_t pair[4] = {__builtin_amdgcn_perm(lo, 0x64646464u, 0x00050004u), __builtin_amdgcn_perm(lo, 0x64646464u, 0x00070006u),
+                                __builtin_amdgcn_perm(hi, 0x64646464u, 0x00050004u), __builtin_amdgcn_perm(hi, 0x64646464u, 0x00070006u)};
+      u32x4 out;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const f16x2 mag = __builtin_bit_cast(f16x2, pair[i]);
+        const f16x2 val = __builtin_elementwise_fma(mag, mul, sub) + shift;
+        out[i] = __builtin_bit_cast(uint32_t, val);
+      }
+      return __builtin_bit_cast(f16x8, out);
+    }
   };
 
   // ---- prologue
