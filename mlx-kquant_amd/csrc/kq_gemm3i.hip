@@ -61,9 +61,11 @@ struct I3Geom<KQ_IQ1_M> {
 };
 
 template <int C>
-constexpr int i3_dpr() { return (I3Geom<C>::BPB + 3) / 4; }  // dwords of a block in LDS
+constexpr int i3_dpr() { return (I3Geom<C>::BPB + 3) / 4; }  // dwords that hold a block
 template <int C>
-constexpr int i3_stage() { return 32 * 4 * i3_dpr<C>(); }    // bytes of a wave's stage (32 rows)
+constexpr int i3_dpl() { return i3_dpr<C>() | 1; }           // dwords of a row in LDS: odd, so that the 32 rows' fields lie in 32 banks
+template <int C>
+constexpr int i3_stage() { return 32 * 4 * i3_dpl<C>(); }    // bytes of a wave's stage (32 rows)
 template <int C, int MT>
 constexpr int i3_lds_bytes() {
   return 2 * (32 * MT * I3_KS * 2) + I3_WAVES * 2 * i3_stage<C>() + I3Geom<C>::TBL_BYTES +
@@ -128,8 +130,8 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
                                                                    uint16_t* __restrict__ y, int M, int N, int K,
                                                                    int mtiles, int nt0) {
   using G = I3Geom<C>;
-  constexpr int BPB = G::BPB, DPR = i3_dpr<C>(), STAGE = i3_stage<C>();
-  constexpr int NEL = 32 * DPR, NI = (NEL + 63) / 64;  // dwords of a stage, load instructions for them
+  constexpr int BPB = G::BPB, DPR = i3_dpr<C>(), DPL = i3_dpl<C>(), STAGE = i3_stage<C>();
+  constexpr int NEL = 32 * DPL, NI = (NEL + 63) / 64;  // dwords of a stage, load instructions for them
   constexpr int W_LAST = NEL - 64 * (NI - 1);
   constexpr bool OVER = (BPB & 3) != 0;                // a block's last dword reaches two bytes past it
   constexpr int TM = 32 * MT, A_STAGE = TM * I3_KS * 2, AQ = MT / 2;
@@ -175,7 +177,8 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
     a_voff[q] = (uint32_t)gr * (uint32_t)K * 2u + 16u * (uint32_t)((lane & 7) ^ swz(r));
   }
   const uint8_t* a_base = reinterpret_cast<const uint8_t*>(xh);
-  // wire: dword i = 64 q + lane of a stage -> row i / DPR, dword i % DPR of its block.  Rows past N read the tile's
+  // wire: dword i = 64 q + lane of a stage -> row i / DPL, dword i % DPL of its block (a row's padding dword, where
+  // DPL > DPR, re-reads the block's first dword and is never looked at).  Rows past N read the tile's
   // first row (their columns are not stored) and never a block's last dword.  The last dword of the matrix's last
   // row is read two bytes early (fix = its LDS offset in a stage, shifted down once landed).
   uint32_t w_voff[NI];
@@ -184,8 +187,9 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
   for (int q = 0; q < NI; q++) {
     int i = 64 * q + lane;
     i = i < NEL ? i : NEL - 1;
-    const int r = wave * 32 + i / DPR;
-    int dw = i % DPR;
+    const int r = wave * 32 + i / DPL;
+    int dw = i % DPL;
+    dw = dw < DPR ? dw : 0;
     uint32_t off;
     if (r < nrows) {
       off = (uint32_t)r * row_bytes + 4u * (uint32_t)dw;
@@ -238,7 +242,7 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
   float r = 1.0f, ratio = 1.0f, live = 1.0f, live_n = 1.0f;
   // entering superblock sb (its stage has landed): the unit change it asks for; commit = false leaves r alone
   auto head = [&](int sb, bool commit) {
-    const float d = kq::iq_block_d<C>(w_smem + (sb & 1) * STAGE + l32 * (4 * DPR));
+    const float d = kq::iq_block_d<C>(w_smem + (sb & 1) * STAGE + l32 * (4 * DPL));
     const float rn = d != 0.f ? d : r;  // a superblock with d = 0 keeps the unit and is fed as zeros
     ratio = r * __builtin_amdgcn_rcpf(rn);
     live_n = d != 0.f ? 1.0f : 0.0f;
@@ -246,7 +250,7 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
   };
   // B fragment of group g of step p of superblock sb: weights 64 p + 16 g + 8 kg .. + 7 of this lane's row
   auto decode = [&](int sb, int p, int g, float lv) -> f16x8 {
-    const uint8_t* blk = w_smem + (sb & 1) * STAGE + l32 * (4 * DPR);
+    const uint8_t* blk = w_smem + (sb & 1) * STAGE + l32 * (4 * DPL);
     if constexpr (kq::is_sign_grid_codec(C)) {
       // magnitude byte m as the f16 1024 + m (bits 0x6400 | m), then (1024 + m) * db - 1024 * db in one fused step:
       // db has at most 5 significant bits and m * db below 2048 units, so the result is m * db itself; the signs
