@@ -16,6 +16,17 @@ __device__ __forceinline__ uint32_t ld32(const uint8_t* p) {
   return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
 }
 __device__ __forceinline__ float ldh(const uint8_t* p) { return h2f(ld16(p)); }
+// the same loads where the caller vouches for a 2-byte aligned address (A2), else byte by byte
+template <bool A2>
+__device__ __forceinline__ uint32_t ld16a(const uint8_t* p) {
+  if constexpr (A2) return *reinterpret_cast<const uint16_t*>(p);
+  else return ld16(p);
+}
+template <bool A2>
+__device__ __forceinline__ uint32_t ld32a(const uint8_t* p) {
+  if constexpr (A2) return (uint32_t) * reinterpret_cast<const uint16_t*>(p) | ((uint32_t) * reinterpret_cast<const uint16_t*>(p + 2) << 16);
+  else return ld32(p);
+}
 
 // src/kquant_iq_tables.h:10
 __device__ __forceinline__ float kv_iq4nl(int i) {
@@ -76,29 +87,31 @@ __host__ __device__ constexpr bool is_sign_grid_codec(int c) {
 
 // Group g (weights 8 g .. 8 g + 7) of a block of such a codec: the magnitudes are the bytes of lo (weights 0-3) and hi
 // (4-7), bit j of s is the sign of weight j, db the scale in the reference's order of operations; UNIT takes the
-// superblock scale d as 1.
-template <int C, bool UNIT>
+// superblock scale d as 1, A2 vouches for a 2-byte aligned block.
+template <int C, bool UNIT, bool A2 = false>
 __device__ __forceinline__ void iq_group(const uint8_t* __restrict__ b, int g, const uint8_t* __restrict__ grids,
                                          uint32_t& lo, uint32_t& hi, uint32_t& s, float& db) {
   const float d = UNIT ? 1.0f : ldh(b);
   const int ib = g >> 2, l = g & 3;
   if constexpr (C == KQ_IQ3_XXS) {  // :467-500
-    const uint32_t aux = ld32(b + 66 + 4 * ib);
+    const uint32_t aux = ld32a<A2>(b + 66 + 4 * ib);
     db = d * (0.5f + (float)(aux >> 28)) * 0.5f;
     s = ksigns(aux >> (7 * l));
-    lo = grid4(grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l]);
-    hi = grid4(grids + KQ_GRID_IQ3XXS + 4 * b[2 + 8 * ib + 2 * l + 1]);
+    const uint32_t two = ld16a<A2>(b + 2 + 8 * ib + 2 * l);
+    lo = grid4(grids + KQ_GRID_IQ3XXS + 4 * (two & 255u));
+    hi = grid4(grids + KQ_GRID_IQ3XXS + 4 * (two >> 8));
   } else if constexpr (C == KQ_IQ3_S) {  // :502-551
     const int nib = (ib & 1) ? (b[106 + (ib >> 1)] >> 4) : (b[106 + (ib >> 1)] & 15);
     db = d * (float)(1 + 2 * nib);
     const uint32_t h = b[66 + ib];
-    const uint32_t i1 = b[2 + 8 * ib + 2 * l] | ((h << (8 - 2 * l)) & 256u);
-    const uint32_t i2 = b[2 + 8 * ib + 2 * l + 1] | ((h << (7 - 2 * l)) & 256u);
+    const uint32_t two = ld16a<A2>(b + 2 + 8 * ib + 2 * l);
+    const uint32_t i1 = (two & 255u) | ((h << (8 - 2 * l)) & 256u);
+    const uint32_t i2 = (two >> 8) | ((h << (7 - 2 * l)) & 256u);
     s = b[74 + 4 * ib + l];
     lo = grid4(grids + KQ_GRID_IQ3S + 4 * i1);
     hi = grid4(grids + KQ_GRID_IQ3S + 4 * i2);
   } else if constexpr (C == KQ_IQ2_XXS) {  // :556-584
-    const uint32_t a1 = ld32(b + 2 + 8 * ib + 4);
+    const uint32_t a1 = ld32a<A2>(b + 2 + 8 * ib + 4);
     db = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
     const uint2 gr = grid8(grids + KQ_GRID_IQ2XXS + 8 * b[2 + 8 * ib + l]);
     s = ksigns(a1 >> (7 * l));
@@ -107,7 +120,7 @@ __device__ __forceinline__ void iq_group(const uint8_t* __restrict__ b, int g, c
   } else if constexpr (C == KQ_IQ2_XS) {  // :586-617
     const uint32_t scb = b[66 + ib];
     db = d * (0.5f + (float)((l < 2) ? (scb & 15) : (scb >> 4))) * 0.25f;
-    const uint32_t q = ld16(b + 2 + 2 * (4 * ib + l));
+    const uint32_t q = ld16a<A2>(b + 2 + 2 * (4 * ib + l));
     const uint2 gr = grid8(grids + KQ_GRID_IQ2XS + 8 * (q & 511u));
     s = ksigns(q >> 9);
     lo = gr.x;
@@ -125,15 +138,15 @@ __device__ __forceinline__ void iq_group(const uint8_t* __restrict__ b, int g, c
 }
 
 // Group g of a block of the ternary codecs iq1_s / iq1_m: the codebook entry's 8 signed bytes (-1, 0, 1) in lo and hi,
-// the group's scale dl and its shift delta = +-1/8: weight j = dl * (entry[j] + delta).
-template <int C, bool UNIT>
+// the group's scale dl and its shift delta = +-1/8: weight j = dl * (entry[j] + delta).  A2 as above.
+template <int C, bool UNIT, bool A2 = false>
 __device__ __forceinline__ void iq1_group(const uint8_t* __restrict__ b, int g, const uint8_t* __restrict__ grids,
                                           uint32_t& lo, uint32_t& hi, float& dl, float& delta) {
   const int ib = g >> 2, l = g & 3;
   uint2 gr;
   if constexpr (C == KQ_IQ1_S) {  // :658-685
     const float d = UNIT ? 1.0f : ldh(b);
-    const uint32_t qh = ld16(b + 34 + 2 * ib);
+    const uint32_t qh = ld16a<A2>(b + 34 + 2 * ib);
     dl = d * (float)(2 * (int)((qh >> 12) & 7) + 1);
     delta = (qh & 0x8000u) ? -0.125f : 0.125f;
     gr = grid8(grids + KQ_GRID_IQ1S + 8 * (b[2 + 4 * ib + l] | (((qh >> (3 * l)) & 7) << 8)));
@@ -144,7 +157,7 @@ __device__ __forceinline__ void iq1_group(const uint8_t* __restrict__ b, int g, 
       const uint32_t s0 = ld16(b + 48), s1 = ld16(b + 50), s2 = ld16(b + 52), s3 = ld16(b + 54);
       d = h2f((uint16_t)((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u)));
     }
-    const uint32_t scw = ld16(b + 48 + 2 * (ib >> 1));
+    const uint32_t scw = ld16a<A2>(b + 48 + 2 * (ib >> 1));
     const int sc3 = (scw >> (6 * (ib & 1) + 3 * (l >> 1))) & 7;
     dl = d * (float)(2 * sc3 + 1);
     const uint32_t hb = b[32 + 2 * ib + (l >> 1)];

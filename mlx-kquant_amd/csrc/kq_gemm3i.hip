@@ -257,7 +257,7 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
       // are the table's masks on the f16 sign bits.  A dead superblock is fed with db = 0.
       uint32_t lo, hi, sg;
       float db;
-      kq::iq_group<C, true>(blk, 8 * p + 2 * g + kg, tbl, lo, hi, sg, db);
+      kq::iq_group<C, true, true>(blk, 8 * p + 2 * g + kg, tbl, lo, hi, sg, db);
       const _Float16 dh = (_Float16)(lv != 0.f ? db : 0.f);
       const f16x2 mul = {dh, dh}, sub = mul * f16x2{(_Float16)-1024.f, (_Float16)-1024.f};
       const u32x4 mask = *reinterpret_cast<const u32x4*>(smem + S_OFF + 16 * sg);
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(64 * I3_WAVES, 1) void iq_gemm3_kernel(const _Float
       // multiple of 1/8 below 17: both exact.  A dead superblock is fed with dl = 0.
       uint32_t lo, hi;
       float dl, delta;
-      kq::iq1_group<C, true>(blk, 8 * p + 2 * g + kg, tbl, lo, hi, dl, delta);
+      kq::iq1_group<C, true, true>(blk, 8 * p + 2 * g + kg, tbl, lo, hi, dl, delta);
       lo ^= 0x80808080u;
       hi ^= 0x80808080u;
       const _Float16 dh = (_Float16)(lv != 0.f ? dl : 0.f), sh = (_Float16)(lv != 0.f ? dl * delta : 0.f);
