@@ -87,7 +87,8 @@ __host__ __device__ constexpr bool is_sign_grid_codec(int c) {
 
 // Group g (weights 8 g .. 8 g + 7) of a block of such a codec: the magnitudes are the bytes of lo (weights 0-3) and hi
 // (4-7), bit j of s is the sign of weight j, db the scale in the reference's order of operations; UNIT takes the
-// superblock scale d as 1, A2 vouches for a 2-byte aligned block.
+// superblock scale d as 1 (the caller applies d; db times a magnitude is then an integer multiple of 1/8 below 512,
+// i.e. an f16 number), A2 vouches for a 2-byte aligned block.
 template <int C, bool UNIT, bool A2 = false>
 __device__ __forceinline__ void iq_group(const uint8_t* __restrict__ b, int g, const uint8_t* __restrict__ grids,
                                          uint32_t& lo, uint32_t& hi, uint32_t& s, float& db) {
@@ -169,9 +170,7 @@ __device__ __forceinline__ void iq1_group(const uint8_t* __restrict__ b, int g, 
   hi = gr.y;
 }
 
-// UNIT: the IQ codecs' weights with the superblock scale d taken as 1 (the caller applies d; every such value is an
-// integer multiple of 1/8 below 2048 / 4, i.e. an f16 number)
-template <int C, bool UNIT = false>
+template <int C>
 __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, const uint8_t* __restrict__ grids,
                                         float* __restrict__ o) {
   if constexpr (C == KQ_Q8_0) {  // :49-63
@@ -272,7 +271,7 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
   } else if constexpr (is_sign_grid_codec(C)) {  // iq3_xxs, iq3_s, iq2_xxs, iq2_xs, iq2_s
     uint32_t lo, hi, s;
     float db;
-    iq_group<C, UNIT>(b, g, grids, lo, hi, s, db);
+    iq_group<C, false>(b, g, grids, lo, hi, s, db);
     for (int j = 0; j < 4; j++) {
       o[j] = db * (float)byte_of(lo, j) * sgn(s, j);
       o[j + 4] = db * (float)byte_of(hi, j) * sgn(s, j + 4);
@@ -280,7 +279,7 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ b, int g, co
   } else if constexpr (C == KQ_IQ1_S || C == KQ_IQ1_M) {
     uint32_t lo, hi;
     float dl, delta;
-    iq1_group<C, UNIT>(b, g, grids, lo, hi, dl, delta);
+    iq1_group<C, false>(b, g, grids, lo, hi, dl, delta);
     for (int j = 0; j < 4; j++) {
       o[j] = dl * ((float)(int8_t)byte_of(lo, j) + delta);
       o[j + 4] = dl * ((float)(int8_t)byte_of(hi, j) + delta);
